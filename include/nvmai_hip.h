@@ -1,0 +1,176 @@
+/*
+ * nvmai_hip.h -- C ABI of the MI355X (gfx950) quantized mixture-of-experts hot path.
+ *
+ * Drop-in boundary for NVMAI's operator layer.  Each entry point replaces one
+ * Swift operator wrapper of the reference (sources/NVMAI/Kernels/...) or one
+ * function of its C target (sources/NVMAIKernelsC); the replaced interface is
+ * cited above each declaration.  Conventions, mirroring the reference's
+ * `encode(commandBuffer:...)` wrappers:
+ *   - every pointer is a raw DEVICE pointer unless marked "host"; a Metal
+ *     (buffer, byteOffset) pair becomes pointer + offset computed by the caller;
+ *   - calls only enqueue work on `stream` (a hipStream_t) and never synchronise;
+ *   - status is returned as int: 0 = ok, negative = nvmai_status; nothing aborts;
+ *   - one nvmai_hip_ctx per stream; a ctx is not thread-safe.
+ * Data formats (reference file:line):
+ *   - weights: affine group-64 codes, 4 bit (two per byte, element 2k in the low
+ *     nibble of byte k) or 8 bit, plus one BF16 scale and one BF16 bias per group
+ *     (nvmai_kernels.h:10-21, Quantization.swift:32-38).  Code rows must be
+ *     16-byte aligned.
+ *   - activations: 16-bit, BF16 or FP16 chosen at ctx creation.
+ *   - routing weights, softmax probabilities, KV scale/bias: FP16.
+ */
+#ifndef NVMAI_HIP_H
+#define NVMAI_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct nvmai_hip_ctx nvmai_hip_ctx;
+typedef void* nvmai_stream;   /* hipStream_t */
+
+typedef enum {
+    NVMAI_OK = 0,
+    NVMAI_ERR_INVALID_ARG = -1,   /* shape/size contract violated (reference: precondition) */
+    NVMAI_ERR_UNSUPPORTED = -2,   /* e.g. weight bits not in {4,8} (SharedExpertError.unsupportedWeightBits) */
+    NVMAI_ERR_ALIGNMENT = -3,     /* a pointer or stride is not 16-byte aligned */
+    NVMAI_ERR_SCRATCH = -4,       /* caller scratch too small (SharedExpertError.scratchTooSmall) */
+    NVMAI_ERR_HIP = -5,           /* a HIP runtime call failed */
+    NVMAI_ERR_NO_DEVICE = -6
+} nvmai_status;
+
+enum { NVMAI_ACT_BF16 = 0, NVMAI_ACT_FP16 = 1 };
+
+/* Rows in "router format": kind 4 / 8 = affine codes with BF16 scale/bias per
+ * group of 64; kind 16 = dense BF16 (scales/biases unused); kind 0 = absent. */
+typedef struct {
+    const void* weights;
+    const uint16_t* scales;
+    const uint16_t* biases;
+    int32_t kind;
+} nvmai_rows;
+
+/* Byte offsets of the nine tensors of one expert blob.
+ * Replaces MoEExpertOffsets (MoE.swift:5-29) == ExpertOffsets (moe.metal:141-151). */
+typedef struct {
+    uint32_t gate_w, gate_s, gate_b, up_w, up_s, up_b, down_w, down_s, down_b;
+} nvmai_expert_offsets;
+
+/* Replaces MetalContext (MetalContext.swift) for this path: binds a device,
+ * fixes the activation type, owns the small persistent scratch the reference's
+ * wrappers own (router logits MoE.swift:130-139, split-KV partials
+ * Attention.swift:117-126, sampler stages LogitOutput.swift:244-258). */
+int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** out);
+void nvmai_hip_ctx_destroy(nvmai_hip_ctx* ctx);
+const char* nvmai_hip_status_string(int status);
+
+/* CPUExpertFFN.Offsets(d:f:) (CPUExpertFFN.swift:42-59) for `bits` in {4,8}.
+ * Host-only arithmetic; *stride_bytes receives the blob size. */
+int nvmai_expert_offsets_for(uint32_t d, uint32_t f, uint32_t bits,
+                             nvmai_expert_offsets* out, uint64_t* stride_bytes);
+
+/* Quantization.quantizeInt4Affine / quantizeInt8Affine (Quantization.swift:50-102,
+ * 135-177) for a [rows, n] matrix on the device.  w is FP32 (w_is_bf16 = 0) or
+ * BF16.  Codes, scale bits and bias bits equal the reference's bit for bit. */
+int nvmai_hip_quantize_affine(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* w,
+                              int w_is_bf16, uint32_t rows, uint32_t n, uint32_t bits,
+                              uint8_t* packed, uint16_t* scales, uint16_t* biases);
+
+/* Quantization.dequantizeInt4Affine / Int8 (Quantization.swift:104-119, 179-191):
+ * codes_out (one byte per code) and/or values_out (activations) may be NULL. */
+int nvmai_hip_dequantize_affine(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* packed,
+                                const uint16_t* scales, const uint16_t* biases, uint64_t count,
+                                uint32_t bits, uint8_t* codes_out, void* values_out);
+
+/* DequantInt4GEMV.encode / DequantInt8GEMV.encode / AffineQuantGEMV.encode
+ * (DequantInt4GEMV.swift:66-110, DequantInt8GEMV.swift:50-86, AffineQuant.swift:58)
+ * and, with y_f32 != NULL, nvmai_int4_affine_gemv (nvmai_kernels.h:22-28):
+ * y[t, :] = W x[t, :] for n_tokens inputs.  y (activations) or y_f32 may be NULL. */
+int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
+                          const uint16_t* scales, const uint16_t* biases, uint32_t bits,
+                          const void* x, uint32_t x_stride, uint32_t n_tokens, uint32_t m,
+                          uint32_t n, void* y, float* y_f32, uint32_t y_stride);
+
+/* MoE.encodeRouter (MoE.swift:151-213) and PrefillRouter.encodeBlock
+ * (PrefillRouter.swift:41-95): logits for n_tokens rows of `hidden`, top-k by
+ * (score desc, index asc), softmax over the selected, times per_expert_scale.
+ * eff_scale / per_expert_scale are optional BF16 arrays (NULL = 1.0).
+ * out_idx [n_tokens, top_k] u32, out_w [n_tokens, top_k] FP16;
+ * logits_out optional FP32 [n_tokens, num_experts]. */
+int nvmai_hip_moe_router_topk(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_rows* router,
+                              const void* hidden, uint32_t hidden_stride, uint32_t n_tokens,
+                              const uint16_t* eff_scale, const uint16_t* per_expert_scale,
+                              uint32_t num_experts, uint32_t d, uint32_t top_k,
+                              uint32_t* out_idx, uint16_t* out_w, float* logits_out);
+
+/* MoE.encodeRoutedPersistentPhase1U16Load (MoE.swift:295-339; kernels
+ * moe.metal:642-683, 812-834): acts[slot, :] = silu(gate_slot x) * (up_slot x)
+ * for the top_k blobs in `blobs` (host array of top_k device pointers, the
+ * reference's RoutedBlobs argument buffer).  acts is caller-owned FP32
+ * [top_k, f]. */
+int nvmai_hip_moe_phase1_gate_up_act(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                     const void* const* blobs, const nvmai_expert_offsets* off,
+                                     uint32_t bits, const void* x, float* acts, uint32_t d,
+                                     uint32_t f, uint32_t top_k);
+
+/* MoE.encodeRoutedPersistentPhase1SubsetU16Load (MoE.swift:341-392; kernels
+ * moe.metal:685-727, 836-861): same over active_slots[0..active_count) (device
+ * array); slots >= top_k are skipped, rows of other slots stay untouched. */
+int nvmai_hip_moe_phase1_gate_up_act_subset(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                            const void* const* blobs,
+                                            const nvmai_expert_offsets* off, uint32_t bits,
+                                            const void* x, float* acts, uint32_t d, uint32_t f,
+                                            uint32_t top_k, const uint32_t* active_slots,
+                                            uint32_t active_count);
+
+/* MoE.encodeRoutedPersistentPhase2Reduce (MoE.swift:394-440; kernels
+ * moe.metal:769-810, 863-892): y[d] = residual[d] + sum over slots in slot order
+ * of w[slot] * (down_slot[d, :] . acts[slot, :]).  routing_w is FP16 [top_k];
+ * residual (activations, may be NULL = 0) and y are [d]. */
+int nvmai_hip_moe_phase2_down_reduce(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                     const void* const* blobs, const nvmai_expert_offsets* off,
+                                     uint32_t bits, const float* acts, const uint16_t* routing_w,
+                                     const void* residual, void* y, uint32_t d, uint32_t f,
+                                     uint32_t top_k);
+
+/* SharedExpertRuntime.encode (SharedExpertInt4.swift:100-153) plus the scalar
+ * gate of RealForwardRunner.swift:3884-3900:
+ * y[t, :] = sigmoid(gate . x[t]) * down(silu(gate_proj x[t]) * (up_proj x[t])).
+ * The three projections live in one blob addressed by `off`; shared_gate may be
+ * NULL or kind 0 (no gate). */
+int nvmai_hip_shared_expert(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* blob,
+                            const nvmai_expert_offsets* off, uint32_t bits,
+                            const nvmai_rows* shared_gate, const void* x, uint32_t x_stride,
+                            uint32_t n_tokens, void* y, uint32_t y_stride, uint32_t d, uint32_t f);
+
+/* One MoE layer for a decode batch with every expert resident in HBM
+ * (RealForwardRunner.swift:1900-1920 router, :3866-3912 shared expert, :3914-4297
+ * routed experts, minus the two host round trips and the SSD streaming):
+ * y[t] = sigmoid(g.x[t]) * ffn_shared(x[t]) + sum_slot w[t,slot] * ffn_{idx[t,slot]}(x[t]).
+ * Each distinct routed expert is read once per call. */
+typedef struct {
+    uint32_t d, f, num_experts, top_k, bits;
+    nvmai_rows router;
+    const void* experts_base;        /* expert e at experts_base + e * expert_stride */
+    uint64_t expert_stride;
+    nvmai_expert_offsets offsets;
+    const void* shared_blob;         /* NULL = no shared expert */
+    nvmai_rows shared_gate;          /* kind 0 = ungated */
+    const uint16_t* eff_scale;       /* optional BF16 [d] */
+    const uint16_t* per_expert_scale;/* optional BF16 [num_experts] */
+} nvmai_moe_layer;
+
+/* out_idx [n_tokens, top_k] u32 and out_w FP16 may be NULL; stats (optional,
+ * device u32[2]) receives {work entries, distinct routed experts}. */
+int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_moe_layer* layer,
+                               const void* x, uint32_t x_stride, uint32_t n_tokens, void* y,
+                               uint32_t y_stride, uint32_t* out_idx, uint16_t* out_w,
+                               uint32_t* stats);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NVMAI_HIP_H */

@@ -1,0 +1,99 @@
+"""ctypes view of libnvmai_hip.so (the C ABI declared in include/nvmai_hip.h).
+
+The library is the product; there is no fallback.  If it has not been built the
+import fails loudly.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libnvmai_hip.so")
+
+
+class NvmaiLibraryMissing(ImportError):
+    pass
+
+
+def load():
+    if not os.path.exists(LIB_PATH):
+        raise NvmaiLibraryMissing(
+            "%s is missing: run `python -m nvmai_amd.build` (hipcc, gfx950) first" % LIB_PATH)
+    return C.CDLL(LIB_PATH)
+
+
+lib = load()
+
+vp, u32, u64, i32 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_int32
+
+
+class Rows(C.Structure):
+    """nvmai_rows"""
+    _fields_ = [("weights", vp), ("scales", vp), ("biases", vp), ("kind", i32)]
+
+
+class ExpertOffsets(C.Structure):
+    """nvmai_expert_offsets"""
+    _fields_ = [(n, u32) for n in ("gate_w", "gate_s", "gate_b", "up_w", "up_s", "up_b",
+                                   "down_w", "down_s", "down_b")]
+
+
+class MoeLayer(C.Structure):
+    """nvmai_moe_layer"""
+    _fields_ = [("d", u32), ("f", u32), ("num_experts", u32), ("top_k", u32), ("bits", u32),
+                ("router", Rows), ("experts_base", vp), ("expert_stride", u64),
+                ("offsets", ExpertOffsets), ("shared_blob", vp), ("shared_gate", Rows),
+                ("eff_scale", vp), ("per_expert_scale", vp)]
+
+
+# name -> argtypes (every function returns int unless listed in _OTHER)
+SIGNATURES = {
+    "nvmai_hip_ctx_create": [C.c_int, C.c_int, C.POINTER(vp)],
+    "nvmai_expert_offsets_for": [u32, u32, u32, C.POINTER(ExpertOffsets), C.POINTER(u64)],
+    "nvmai_hip_quantize_affine": [vp, vp, vp, C.c_int, u32, u32, u32, vp, vp, vp],
+    "nvmai_hip_dequantize_affine": [vp, vp, vp, vp, vp, u64, u32, vp, vp],
+    "nvmai_hip_affine_gemv": [vp, vp, vp, vp, vp, u32, vp, u32, u32, u32, u32, vp, vp, u32],
+    "nvmai_hip_moe_router_topk": [vp, vp, C.POINTER(Rows), vp, u32, u32, vp, vp, u32, u32, u32,
+                                  vp, vp, vp],
+    "nvmai_hip_moe_phase1_gate_up_act": [vp, vp, C.POINTER(vp), C.POINTER(ExpertOffsets), u32, vp,
+                                         vp, u32, u32, u32],
+    "nvmai_hip_moe_phase1_gate_up_act_subset": [vp, vp, C.POINTER(vp), C.POINTER(ExpertOffsets),
+                                                u32, vp, vp, u32, u32, u32, vp, u32],
+    "nvmai_hip_moe_phase2_down_reduce": [vp, vp, C.POINTER(vp), C.POINTER(ExpertOffsets), u32, vp,
+                                         vp, vp, vp, u32, u32, u32],
+    "nvmai_hip_shared_expert": [vp, vp, vp, C.POINTER(ExpertOffsets), u32, C.POINTER(Rows), vp,
+                                u32, u32, vp, u32, u32, u32],
+    "nvmai_hip_moe_decode_layer": [vp, vp, C.POINTER(MoeLayer), vp, u32, u32, vp, u32, vp, vp, vp],
+}
+_OTHER = {
+    "nvmai_hip_ctx_destroy": (None, [vp]),
+    "nvmai_hip_status_string": (C.c_char_p, [C.c_int]),
+}
+
+
+def _declare():
+    for name, args in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = args
+    for name, (res, args) in _OTHER.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+
+
+_declare()
+
+STATUS = {0: "ok", -1: "invalid_arg", -2: "unsupported", -3: "alignment", -4: "scratch",
+          -5: "hip", -6: "no_device"}
+
+
+class NvmaiError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        self.name = STATUS.get(status, str(status))
+        super().__init__("%s: %s" % (where, lib.nvmai_hip_status_string(status).decode()))
+
+
+def check(status, where):
+    if status != 0:
+        raise NvmaiError(status, where)

@@ -1,0 +1,55 @@
+// Host-side context shared by every entry-point file.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/nvmai_hip.h"
+
+struct nvmai_hip_ctx {
+    int device;
+    int act;                 // NVMAI_ACT_BF16 / NVMAI_ACT_FP16
+    // Workspace: one device buffer carved by a bump pointer inside each entry
+    // point.  Work on one stream is ordered, so consecutive calls may reuse it.
+    uint8_t* ws;
+    size_t ws_cap;
+    size_t ws_used;
+};
+
+namespace nvmai {
+
+#define NVMAI_HIP_TRY(expr)                         \
+    do {                                            \
+        hipError_t e_ = (expr);                     \
+        if (e_ != hipSuccess) return NVMAI_ERR_HIP; \
+    } while (0)
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Make the workspace at least `bytes` large and reset the bump pointer.  Growing
+// waits for the device (hipFree does) and is meant to happen during warm-up.
+inline int ws_begin(nvmai_hip_ctx* ctx, size_t bytes) {
+    ctx->ws_used = 0;
+    if (bytes <= ctx->ws_cap) return NVMAI_OK;
+    size_t cap = ctx->ws_cap ? ctx->ws_cap : (size_t)1 << 20;
+    while (cap < bytes) cap *= 2;
+    if (ctx->ws) NVMAI_HIP_TRY(hipFree(ctx->ws));
+    ctx->ws = nullptr;
+    ctx->ws_cap = 0;
+    NVMAI_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&ctx->ws), cap));
+    ctx->ws_cap = cap;
+    return NVMAI_OK;
+}
+
+inline size_t ws_round(size_t bytes) { return (bytes + 255) & ~(size_t)255; }
+
+template <typename T>
+inline T* ws_take(nvmai_hip_ctx* ctx, size_t count) {
+    T* p = reinterpret_cast<T*>(ctx->ws + ctx->ws_used);
+    ctx->ws_used += ws_round(count * sizeof(T));
+    return p;
+}
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? NVMAI_OK : NVMAI_ERR_HIP; }
+
+}  // namespace nvmai

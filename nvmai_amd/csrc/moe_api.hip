@@ -1,0 +1,540 @@
+// Entry points of the decode-side MoE path: context, quantizer, affine GEMV,
+// router top-k, routed phase 1 / phase 2, shared expert, fused decode layer.
+#include <new>
+
+#include "ctx.hpp"
+#include "moe_kernels.cuh"
+
+using namespace nvmai;
+
+// ---------------------------------------------------------------------------
+// context
+// ---------------------------------------------------------------------------
+extern "C" int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** out) {
+    if (!out || (act_dtype != NVMAI_ACT_BF16 && act_dtype != NVMAI_ACT_FP16)) return NVMAI_ERR_INVALID_ARG;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) return NVMAI_ERR_NO_DEVICE;
+    if (device < 0 || device >= count) return NVMAI_ERR_INVALID_ARG;
+    NVMAI_HIP_TRY(hipSetDevice(device));
+    nvmai_hip_ctx* ctx = new (std::nothrow) nvmai_hip_ctx();
+    if (!ctx) return NVMAI_ERR_HIP;
+    ctx->device = device;
+    ctx->act = act_dtype;
+    ctx->ws = nullptr;
+    ctx->ws_cap = 0;
+    ctx->ws_used = 0;
+    *out = ctx;
+    return NVMAI_OK;
+}
+
+extern "C" void nvmai_hip_ctx_destroy(nvmai_hip_ctx* ctx) {
+    if (!ctx) return;
+    if (ctx->ws) (void)hipFree(ctx->ws);
+    delete ctx;
+}
+
+extern "C" const char* nvmai_hip_status_string(int status) {
+    switch (status) {
+        case NVMAI_OK: return "ok";
+        case NVMAI_ERR_INVALID_ARG: return "invalid argument";
+        case NVMAI_ERR_UNSUPPORTED: return "unsupported configuration";
+        case NVMAI_ERR_ALIGNMENT: return "pointer or stride not 16-byte aligned";
+        case NVMAI_ERR_SCRATCH: return "scratch too small";
+        case NVMAI_ERR_HIP: return "HIP runtime error";
+        case NVMAI_ERR_NO_DEVICE: return "no HIP device";
+        default: return "unknown status";
+    }
+}
+
+extern "C" int nvmai_expert_offsets_for(uint32_t d, uint32_t f, uint32_t bits,
+                                        nvmai_expert_offsets* out, uint64_t* stride_bytes) {
+    if (!out || d == 0 || f == 0 || d % NVMAI_GROUP || f % NVMAI_GROUP) return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    const uint64_t gate_w = (uint64_t)f * d * bits / 8, gate_meta = (uint64_t)f * (d / NVMAI_GROUP) * 2;
+    const uint64_t down_w = (uint64_t)d * f * bits / 8, down_meta = (uint64_t)d * (f / NVMAI_GROUP) * 2;
+    uint64_t o = 0;
+    if (gate_w * 2 + down_w + 4 * gate_meta + 2 * down_meta > 0xFFFFFFFFull) return NVMAI_ERR_INVALID_ARG;
+    out->gate_w = (uint32_t)o; o += gate_w;
+    out->gate_s = (uint32_t)o; o += gate_meta;
+    out->gate_b = (uint32_t)o; o += gate_meta;
+    out->up_w = (uint32_t)o; o += gate_w;
+    out->up_s = (uint32_t)o; o += gate_meta;
+    out->up_b = (uint32_t)o; o += gate_meta;
+    out->down_w = (uint32_t)o; o += down_w;
+    out->down_s = (uint32_t)o; o += down_meta;
+    out->down_b = (uint32_t)o; o += down_meta;
+    if (stride_bytes) *stride_bytes = o;
+    return NVMAI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// rows-engine dispatch
+// ---------------------------------------------------------------------------
+namespace {
+
+template <int ACT, int BITS, int SEG, int NCH, int MAXTOK, bool DUAL, bool XF32, int RPI, int ITERS>
+void launch_fast(RowsParams& p, uint32_t max_entries, hipStream_t s) {
+    constexpr uint32_t rows_per_block = 4 * (64 / SEG) * RPI * ITERS;
+    p.blocks_per_entry = (p.rows + rows_per_block - 1) / rows_per_block;
+    expert_rows_fast<ACT, BITS, SEG, NCH, MAXTOK, DUAL, XF32, RPI, ITERS>
+        <<<dim3(max_entries * p.blocks_per_entry), dim3(256), 0, s>>>(p);
+}
+
+template <int ACT, int BITS, bool DUAL, bool XF32>
+void launch_rows_t(RowsParams& p, int maxtok, uint32_t max_entries, hipStream_t s) {
+    const uint32_t chunks = p.n * BITS / 128;
+#define NVMAI_FAST(SEG, NCH, RPI, ITERS)                                                        \
+    do {                                                                                        \
+        if (maxtok == 1) launch_fast<ACT, BITS, SEG, NCH, 1, DUAL, XF32, RPI, ITERS>(p, max_entries, s); \
+        else launch_fast<ACT, BITS, SEG, NCH, 4, DUAL, XF32, RPI, ITERS>(p, max_entries, s);    \
+        return;                                                                                 \
+    } while (0)
+    if constexpr (DUAL) {
+        if (chunks == 64) NVMAI_FAST(64, 1, 2, 2);
+        if (chunks == 128) NVMAI_FAST(64, 2, 2, 2);
+    } else {
+        if (chunks == 16) NVMAI_FAST(16, 1, 2, 2);
+        if (chunks == 32) NVMAI_FAST(32, 1, 4, 2);
+        if (chunks == 64) NVMAI_FAST(64, 1, 4, 1);
+        if (chunks == 128) NVMAI_FAST(64, 2, 4, 1);
+    }
+#undef NVMAI_FAST
+    p.blocks_per_entry = (p.rows + 15) / 16;
+    expert_rows_generic<ACT, BITS, DUAL, XF32>
+        <<<dim3(max_entries * p.blocks_per_entry), dim3(256), 0, s>>>(p);
+}
+
+// maxtok: 1 when every entry holds one pair, else MAX_TOK.
+void launch_rows(int act, uint32_t bits, bool dual, bool xf32, RowsParams& p, int maxtok,
+                 uint32_t max_entries, hipStream_t s) {
+    if (max_entries == 0) return;
+    if (xf32 && !dual) {   // inputs are fp32: one instantiation serves both activation types
+        if (bits == 8) launch_rows_t<ACT_BF16, 8, false, true>(p, maxtok, max_entries, s);
+        else launch_rows_t<ACT_BF16, 4, false, true>(p, maxtok, max_entries, s);
+        return;
+    }
+#define NVMAI_ROWS(ACT, BITS)                                                   \
+    do {                                                                        \
+        if (dual) launch_rows_t<ACT, BITS, true, false>(p, maxtok, max_entries, s);   \
+        else launch_rows_t<ACT, BITS, false, false>(p, maxtok, max_entries, s); \
+    } while (0)
+    if (act == ACT_BF16) { if (bits == 8) NVMAI_ROWS(ACT_BF16, 8); else NVMAI_ROWS(ACT_BF16, 4); }
+    else { if (bits == 8) NVMAI_ROWS(ACT_FP16, 8); else NVMAI_ROWS(ACT_FP16, 4); }
+#undef NVMAI_ROWS
+}
+
+int check_shape(uint32_t d, uint32_t f, uint32_t bits) {
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    if (d == 0 || f == 0 || d % NVMAI_GROUP || f % NVMAI_GROUP) return NVMAI_ERR_INVALID_ARG;
+    return NVMAI_OK;
+}
+
+int check_offsets(const nvmai_expert_offsets* o) {
+    if (!o) return NVMAI_ERR_INVALID_ARG;
+    if ((o->gate_w | o->up_w | o->down_w) & 15u) return NVMAI_ERR_ALIGNMENT;
+    if ((o->gate_s | o->gate_b | o->up_s | o->up_b | o->down_s | o->down_b) & 1u) return NVMAI_ERR_ALIGNMENT;
+    return NVMAI_OK;
+}
+
+void set_phase1(RowsParams& p, const nvmai_expert_offsets& o, uint32_t d, uint32_t f) {
+    p.wA = o.gate_w; p.sA = o.gate_s; p.bA = o.gate_b;
+    p.wB = o.up_w; p.sB = o.up_s; p.bB = o.up_b;
+    p.rows = f; p.n = d;
+}
+
+void set_phase2(RowsParams& p, const nvmai_expert_offsets& o, uint32_t d, uint32_t f) {
+    p.wA = o.down_w; p.sA = o.down_s; p.bA = o.down_b;
+    p.wB = p.sB = p.bB = 0;
+    p.rows = d; p.n = f;
+}
+
+void run_router(int act, const RouterParams& rp, hipStream_t s) {
+    const uint32_t rows = rp.num_experts + (rp.gate.kind ? 1u : 0u);
+    dim3 grid((rows + 7) / 8, (rp.tokens + ROUTER_TOK - 1) / ROUTER_TOK);
+    if (act == ACT_BF16) router_logits_kernel<ACT_BF16><<<grid, 256, 0, s>>>(rp);
+    else router_logits_kernel<ACT_FP16><<<grid, 256, 0, s>>>(rp);
+}
+
+int check_rows_desc(const nvmai_rows* r, uint32_t d, bool allow_absent) {
+    if (!r || r->kind == 0) return allow_absent ? NVMAI_OK : NVMAI_ERR_INVALID_ARG;
+    if (r->kind != 4 && r->kind != 8 && r->kind != 16) return NVMAI_ERR_UNSUPPORTED;
+    if (!r->weights || (r->kind != 16 && (!r->scales || !r->biases))) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(r->weights)) return NVMAI_ERR_ALIGNMENT;
+    if (d % NVMAI_GROUP) return NVMAI_ERR_INVALID_ARG;
+    return NVMAI_OK;
+}
+
+RowsDesc to_desc(const nvmai_rows* r) {
+    RowsDesc d{};
+    if (r && r->kind) { d.w = r->weights; d.s = r->scales; d.b = r->biases; d.kind = r->kind; }
+    return d;
+}
+
+void run_combine(int act, const CombineParams& cp, hipStream_t s) {
+    dim3 grid((cp.d + 255) / 256, cp.tokens);
+    if (act == ACT_BF16) combine_kernel<ACT_BF16><<<grid, 256, 0, s>>>(cp);
+    else combine_kernel<ACT_FP16><<<grid, 256, 0, s>>>(cp);
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// quantizer
+// ---------------------------------------------------------------------------
+extern "C" int nvmai_hip_quantize_affine(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* w,
+                                         int w_is_bf16, uint32_t rows, uint32_t n, uint32_t bits,
+                                         uint8_t* packed, uint16_t* scales, uint16_t* biases) {
+    if (!ctx || !w || !packed || !scales || !biases) return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    if (n == 0 || n % NVMAI_GROUP) return NVMAI_ERR_INVALID_ARG;
+    if (rows == 0) return NVMAI_OK;
+    QuantParams q{w, w_is_bf16, rows, n, bits, packed, scales, biases};
+    const uint64_t groups = (uint64_t)rows * (n / NVMAI_GROUP);
+    quantize_affine_kernel<<<dim3((uint32_t)((groups + 3) / 4)), dim3(256), 0, (hipStream_t)stream>>>(q);
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_dequantize_affine(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                           const uint8_t* packed, const uint16_t* scales,
+                                           const uint16_t* biases, uint64_t count, uint32_t bits,
+                                           uint8_t* codes_out, void* values_out) {
+    if (!ctx || !packed) return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    if (values_out && (!scales || !biases)) return NVMAI_ERR_INVALID_ARG;
+    if (count % NVMAI_GROUP) return NVMAI_ERR_INVALID_ARG;
+    if (count == 0) return NVMAI_OK;
+    dim3 grid((uint32_t)((count + 255) / 256));
+    if (ctx->act == ACT_BF16)
+        dequantize_affine_kernel<ACT_BF16><<<grid, 256, 0, (hipStream_t)stream>>>(packed, scales, biases, count, bits, codes_out, values_out);
+    else
+        dequantize_affine_kernel<ACT_FP16><<<grid, 256, 0, (hipStream_t)stream>>>(packed, scales, biases, count, bits, codes_out, values_out);
+    return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// affine GEMV
+// ---------------------------------------------------------------------------
+extern "C" int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
+                                     const uint16_t* scales, const uint16_t* biases, uint32_t bits,
+                                     const void* x, uint32_t x_stride, uint32_t n_tokens,
+                                     uint32_t m, uint32_t n, void* y, float* y_f32,
+                                     uint32_t y_stride) {
+    if (!ctx || !weights || !scales || !biases || !x || (!y && !y_f32)) return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    if (n == 0 || n % NVMAI_GROUP || x_stride < n || y_stride < m) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(weights) || !aligned16(x) || (x_stride % 8)) return NVMAI_ERR_ALIGNMENT;
+    if (m == 0 || n_tokens == 0) return NVMAI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const int maxtok = n_tokens == 1 ? 1 : MAX_TOK;
+    const uint32_t ents = (n_tokens + maxtok - 1) / maxtok;
+    const bool need_tmp = (y != nullptr) || y_stride != m;
+    size_t need = ws_round(ents * sizeof(WorkEntry)) + ws_round(16) + 2 * ws_round(n_tokens * 4u) +
+                  (need_tmp ? ws_round((size_t)n_tokens * m * 4u) : 0);
+    int rc = ws_begin(ctx, need);
+    if (rc) return rc;
+    WorkEntry* entries = ws_take<WorkEntry>(ctx, ents);
+    uint32_t* n_entries = ws_take<uint32_t>(ctx, 4);
+    uint32_t* pair_token = ws_take<uint32_t>(ctx, n_tokens);
+    uint32_t* pair_id = ws_take<uint32_t>(ctx, n_tokens);
+    float* tmp = need_tmp ? ws_take<float>(ctx, (size_t)n_tokens * m) : y_f32;
+    dense_entries_kernel<<<(n_tokens + 255) / 256, 256, 0, s>>>(entries, n_entries, pair_token, pair_id,
+                                                              n_tokens, (uint32_t)maxtok, 0u);
+    RowsParams p{};
+    p.src.slot[0] = weights;
+    p.entries = entries; p.n_entries = n_entries; p.pair_in = pair_token; p.pair_out = pair_id;
+    p.wA = 0;
+    p.sA = reinterpret_cast<const uint8_t*>(scales) - weights;
+    p.bA = reinterpret_cast<const uint8_t*>(biases) - weights;
+    p.x = x; p.x_stride = x_stride; p.out = tmp; p.out_stride = m; p.rows = m; p.n = n;
+    launch_rows(ctx->act, bits, false, false, p, maxtok, ents, s);
+    if (need_tmp) {
+        // copy out with the caller's stride (and convert when asked)
+        for (uint32_t t = 0; t < n_tokens; ++t) {
+            if (y) {
+                uint16_t* dst = (uint16_t*)y + (size_t)t * y_stride;
+                if (ctx->act == ACT_BF16) store_act_kernel<ACT_BF16><<<(m + 255) / 256, 256, 0, s>>>(tmp + (size_t)t * m, dst, m);
+                else store_act_kernel<ACT_FP16><<<(m + 255) / 256, 256, 0, s>>>(tmp + (size_t)t * m, dst, m);
+            }
+            if (y_f32)
+                NVMAI_HIP_TRY(hipMemcpyAsync(y_f32 + (size_t)t * y_stride, tmp + (size_t)t * m,
+                                             (size_t)m * 4, hipMemcpyDeviceToDevice, s));
+        }
+    }
+    return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// router
+// ---------------------------------------------------------------------------
+extern "C" int nvmai_hip_moe_router_topk(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                         const nvmai_rows* router, const void* hidden,
+                                         uint32_t hidden_stride, uint32_t n_tokens,
+                                         const uint16_t* eff_scale, const uint16_t* per_expert_scale,
+                                         uint32_t num_experts, uint32_t d, uint32_t top_k,
+                                         uint32_t* out_idx, uint16_t* out_w, float* logits_out) {
+    if (!ctx || !hidden || !out_idx || !out_w) return NVMAI_ERR_INVALID_ARG;
+    int rc = check_rows_desc(router, d, false);
+    if (rc) return rc;
+    if (num_experts == 0 || num_experts > 64 * TOPK_MAX_PER_LANE) return NVMAI_ERR_INVALID_ARG;
+    if (top_k == 0 || top_k > 64 || top_k > num_experts || hidden_stride < d) return NVMAI_ERR_INVALID_ARG;
+    if (n_tokens == 0) return NVMAI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    float* logits = logits_out;
+    if (!logits) {
+        rc = ws_begin(ctx, ws_round((size_t)n_tokens * num_experts * 4));
+        if (rc) return rc;
+        logits = ws_take<float>(ctx, (size_t)n_tokens * num_experts);
+    }
+    RouterParams rp{};
+    rp.router = to_desc(router);
+    rp.x = hidden; rp.eff_scale = eff_scale; rp.x_stride = hidden_stride; rp.tokens = n_tokens;
+    rp.num_experts = num_experts; rp.d = d; rp.logits = logits; rp.gate_logit = nullptr;
+    run_router(ctx->act, rp, s);
+    SelectParams sp{logits, per_expert_scale, n_tokens, num_experts, top_k, out_idx, out_w};
+    select_topk_kernel<<<(n_tokens + 3) / 4, 256, 0, s>>>(sp);
+    return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// routed phase 1 / phase 2 over the top-k slot blobs of one token
+// ---------------------------------------------------------------------------
+namespace {
+
+int slots_prologue(nvmai_hip_ctx* ctx, const void* const* blobs, const nvmai_expert_offsets* off,
+                   uint32_t bits, uint32_t d, uint32_t f, uint32_t top_k, RowsParams& p) {
+    if (!ctx || !blobs) return NVMAI_ERR_INVALID_ARG;
+    int rc = check_shape(d, f, bits);
+    if (rc) return rc;
+    rc = check_offsets(off);
+    if (rc) return rc;
+    if (top_k == 0 || top_k > 8) return NVMAI_ERR_INVALID_ARG;   // MoE.swift:455-458 requires 8
+    for (uint32_t i = 0; i < top_k; ++i) {
+        if (!blobs[i]) return NVMAI_ERR_INVALID_ARG;
+        if (!aligned16(blobs[i])) return NVMAI_ERR_ALIGNMENT;
+        p.src.slot[i] = (const uint8_t*)blobs[i];
+    }
+    return NVMAI_OK;
+}
+
+}  // namespace
+
+extern "C" int nvmai_hip_moe_phase1_gate_up_act_subset(
+    nvmai_hip_ctx* ctx, nvmai_stream stream, const void* const* blobs,
+    const nvmai_expert_offsets* off, uint32_t bits, const void* x, float* acts, uint32_t d,
+    uint32_t f, uint32_t top_k, const uint32_t* active_slots, uint32_t active_count) {
+    RowsParams p{};
+    int rc = slots_prologue(ctx, blobs, off, bits, d, f, top_k, p);
+    if (rc) return rc;
+    if (!x || !acts || (active_count && !active_slots) || active_count > top_k) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(x) || !aligned16(acts)) return NVMAI_ERR_ALIGNMENT;
+    hipStream_t s = (hipStream_t)stream;
+    rc = ws_begin(ctx, ws_round(8 * sizeof(WorkEntry)) + 3 * ws_round(64));
+    if (rc) return rc;
+    WorkEntry* entries = ws_take<WorkEntry>(ctx, 8);
+    uint32_t* n_entries = ws_take<uint32_t>(ctx, 4);
+    uint32_t* pair_token = ws_take<uint32_t>(ctx, 8);
+    uint32_t* pair_id = ws_take<uint32_t>(ctx, 8);
+    uint32_t count = active_slots ? active_count : top_k;
+    if (active_slots) {
+        subset_entries_kernel<<<1, 64, 0, s>>>(entries, n_entries, pair_token, pair_id, active_slots,
+                                              active_count, top_k);
+    } else {
+        // dense over the slots: entry i -> slot i, input row 0, output row i
+        slot_entries_kernel<<<1, 64, 0, s>>>(entries, n_entries, pair_token, pair_id, top_k, 0);
+    }
+    p.entries = entries; p.n_entries = n_entries; p.pair_in = pair_token; p.pair_out = pair_id;
+    set_phase1(p, *off, d, f);
+    p.x = x; p.x_stride = d; p.out = acts; p.out_stride = f;
+    launch_rows(ctx->act, bits, true, false, p, 1, count, s);
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_moe_phase1_gate_up_act(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                                const void* const* blobs,
+                                                const nvmai_expert_offsets* off, uint32_t bits,
+                                                const void* x, float* acts, uint32_t d, uint32_t f,
+                                                uint32_t top_k) {
+    return nvmai_hip_moe_phase1_gate_up_act_subset(ctx, stream, blobs, off, bits, x, acts, d, f, top_k,
+                                                   nullptr, 0);
+}
+
+extern "C" int nvmai_hip_moe_phase2_down_reduce(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                                const void* const* blobs,
+                                                const nvmai_expert_offsets* off, uint32_t bits,
+                                                const float* acts, const uint16_t* routing_w,
+                                                const void* residual, void* y, uint32_t d, uint32_t f,
+                                                uint32_t top_k) {
+    RowsParams p{};
+    int rc = slots_prologue(ctx, blobs, off, bits, d, f, top_k, p);
+    if (rc) return rc;
+    if (!acts || !routing_w || !y) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(acts)) return NVMAI_ERR_ALIGNMENT;
+    hipStream_t s = (hipStream_t)stream;
+    rc = ws_begin(ctx, ws_round(8 * sizeof(WorkEntry)) + 3 * ws_round(64) + ws_round((size_t)top_k * d * 4));
+    if (rc) return rc;
+    WorkEntry* entries = ws_take<WorkEntry>(ctx, 8);
+    uint32_t* n_entries = ws_take<uint32_t>(ctx, 4);
+    uint32_t* pair_in = ws_take<uint32_t>(ctx, 8);
+    uint32_t* pair_id = ws_take<uint32_t>(ctx, 8);
+    float* partials = ws_take<float>(ctx, (size_t)top_k * d);
+    slot_entries_kernel<<<1, 64, 0, s>>>(entries, n_entries, pair_in, pair_id, top_k, 1);
+    p.entries = entries; p.n_entries = n_entries; p.pair_in = pair_in; p.pair_out = pair_id;
+    set_phase2(p, *off, d, f);
+    p.x = acts; p.x_stride = f; p.out = partials; p.out_stride = d;
+    launch_rows(ctx->act, bits, false, true, p, 1, top_k, s);
+    CombineParams cp{};
+    cp.partials = partials; cp.w = routing_w; cp.residual = residual; cp.gate_logit = nullptr;
+    cp.has_shared = 0; cp.tokens = 1; cp.top_k = top_k; cp.d = d; cp.res_stride = d; cp.y_stride = d;
+    cp.y = y;
+    run_combine(ctx->act, cp, s);
+    return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// shared expert
+// ---------------------------------------------------------------------------
+extern "C" int nvmai_hip_shared_expert(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* blob,
+                                       const nvmai_expert_offsets* off, uint32_t bits,
+                                       const nvmai_rows* shared_gate, const void* x,
+                                       uint32_t x_stride, uint32_t n_tokens, void* y,
+                                       uint32_t y_stride, uint32_t d, uint32_t f) {
+    if (!ctx || !blob || !x || !y) return NVMAI_ERR_INVALID_ARG;
+    int rc = check_shape(d, f, bits);
+    if (rc) return rc;
+    rc = check_offsets(off);
+    if (rc) return rc;
+    rc = check_rows_desc(shared_gate, d, true);
+    if (rc) return rc;
+    if (x_stride < d || y_stride < d) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(blob) || !aligned16(x) || (x_stride % 8)) return NVMAI_ERR_ALIGNMENT;
+    if (n_tokens == 0) return NVMAI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const int maxtok = n_tokens == 1 ? 1 : MAX_TOK;
+    const uint32_t ents = (n_tokens + maxtok - 1) / maxtok;
+    size_t need = ws_round(ents * sizeof(WorkEntry)) + ws_round(16) + 2 * ws_round(n_tokens * 4u) +
+                  ws_round((size_t)n_tokens * f * 4) + ws_round((size_t)n_tokens * d * 4) +
+                  ws_round(n_tokens * 4u) + ws_round(16);
+    rc = ws_begin(ctx, need);
+    if (rc) return rc;
+    WorkEntry* entries = ws_take<WorkEntry>(ctx, ents);
+    uint32_t* n_entries = ws_take<uint32_t>(ctx, 4);
+    uint32_t* pair_token = ws_take<uint32_t>(ctx, n_tokens);
+    uint32_t* pair_id = ws_take<uint32_t>(ctx, n_tokens);
+    float* acts = ws_take<float>(ctx, (size_t)n_tokens * f);
+    float* partials = ws_take<float>(ctx, (size_t)n_tokens * d);
+    float* gate_logit = ws_take<float>(ctx, n_tokens);
+    float* dummy_logits = ws_take<float>(ctx, 4);
+    dense_entries_kernel<<<(n_tokens + 255) / 256, 256, 0, s>>>(entries, n_entries, pair_token, pair_id,
+                                                              n_tokens, (uint32_t)maxtok, 8u);
+    const bool gated = shared_gate && shared_gate->kind;
+    if (gated) {
+        RouterParams rp{};
+        rp.gate = to_desc(shared_gate);
+        rp.x = x; rp.x_stride = x_stride; rp.tokens = n_tokens; rp.num_experts = 0; rp.d = d;
+        rp.logits = dummy_logits; rp.gate_logit = gate_logit;
+        run_router(ctx->act, rp, s);
+    }
+    RowsParams p{};
+    p.src.slot[8] = (const uint8_t*)blob;
+    p.entries = entries; p.n_entries = n_entries; p.pair_in = pair_token; p.pair_out = pair_id;
+    set_phase1(p, *off, d, f);
+    p.x = x; p.x_stride = x_stride; p.out = acts; p.out_stride = f;
+    launch_rows(ctx->act, bits, true, false, p, maxtok, ents, s);
+    RowsParams q = p;
+    set_phase2(q, *off, d, f);
+    q.pair_in = pair_id;
+    q.x = acts; q.x_stride = f; q.out = partials; q.out_stride = d;
+    launch_rows(ctx->act, bits, false, true, q, maxtok, ents, s);
+    CombineParams cp{};
+    cp.partials = partials; cp.w = nullptr; cp.residual = nullptr;
+    cp.gate_logit = gated ? gate_logit : nullptr;
+    cp.has_shared = 1; cp.tokens = n_tokens; cp.top_k = 0; cp.d = d; cp.res_stride = 0;
+    cp.y_stride = y_stride; cp.y = y;
+    run_combine(ctx->act, cp, s);
+    return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// fused decode layer
+// ---------------------------------------------------------------------------
+extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                          const nvmai_moe_layer* L, const void* x, uint32_t x_stride,
+                                          uint32_t n_tokens, void* y, uint32_t y_stride,
+                                          uint32_t* out_idx, uint16_t* out_w, uint32_t* stats) {
+    if (!ctx || !L || !x || !y) return NVMAI_ERR_INVALID_ARG;
+    int rc = check_shape(L->d, L->f, L->bits);
+    if (rc) return rc;
+    rc = check_offsets(&L->offsets);
+    if (rc) return rc;
+    rc = check_rows_desc(&L->router, L->d, false);
+    if (rc) return rc;
+    rc = check_rows_desc(&L->shared_gate, L->d, true);
+    if (rc) return rc;
+    const uint32_t T = n_tokens, K = L->top_k, E = L->num_experts, D = L->d, F = L->f;
+    if (E == 0 || E > 64 * TOPK_MAX_PER_LANE || K == 0 || K > 64 || K > E) return NVMAI_ERR_INVALID_ARG;
+    if (!L->experts_base || x_stride < D || y_stride < D) return NVMAI_ERR_INVALID_ARG;
+    if ((uint64_t)T * K > 4096) return NVMAI_ERR_INVALID_ARG;   // work list is built in LDS
+    if (!aligned16(L->experts_base) || (L->expert_stride & 15u) || !aligned16(x) || (x_stride % 8) ||
+        (L->shared_blob && !aligned16(L->shared_blob)))
+        return NVMAI_ERR_ALIGNMENT;
+    if (T == 0) return NVMAI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const bool has_shared = L->shared_blob != nullptr;
+    const bool gated = has_shared && L->shared_gate.kind != 0;
+    const int maxtok = T == 1 ? 1 : MAX_TOK;
+    const uint32_t pairs = T * K;
+    const uint32_t rows_total = pairs + (has_shared ? T : 0);
+    uint32_t routed_ents = pairs;
+    if (maxtok > 1) routed_ents = pairs < E + pairs / maxtok ? pairs : E + pairs / maxtok;
+    const uint32_t max_entries = routed_ents + (has_shared ? (T + maxtok - 1) / maxtok : 0);
+    size_t need = ws_round((size_t)T * E * 4) + ws_round(T * 4u) + ws_round(pairs * 4u) +
+                  ws_round(pairs * 2u) + ws_round(max_entries * sizeof(WorkEntry)) + ws_round(16) +
+                  2 * ws_round(rows_total * 4u) + ws_round((size_t)rows_total * F * 4) +
+                  ws_round((size_t)rows_total * D * 4);
+    rc = ws_begin(ctx, need);
+    if (rc) return rc;
+    float* logits = ws_take<float>(ctx, (size_t)T * E);
+    float* gate_logit = ws_take<float>(ctx, T);
+    uint32_t* idx = ws_take<uint32_t>(ctx, pairs);
+    uint16_t* wts = ws_take<uint16_t>(ctx, pairs);
+    WorkEntry* entries = ws_take<WorkEntry>(ctx, max_entries);
+    uint32_t* n_entries = ws_take<uint32_t>(ctx, 4);
+    uint32_t* pair_token = ws_take<uint32_t>(ctx, rows_total);
+    uint32_t* pair_id = ws_take<uint32_t>(ctx, rows_total);
+    float* acts = ws_take<float>(ctx, (size_t)rows_total * F);
+    float* partials = ws_take<float>(ctx, (size_t)rows_total * D);
+    if (out_idx) idx = out_idx;
+    if (out_w) wts = out_w;
+
+    RouterParams rp{};
+    rp.router = to_desc(&L->router);
+    if (gated) rp.gate = to_desc(&L->shared_gate);
+    rp.x = x; rp.eff_scale = L->eff_scale; rp.x_stride = x_stride; rp.tokens = T;
+    rp.num_experts = E; rp.d = D; rp.logits = logits; rp.gate_logit = gate_logit;
+    run_router(ctx->act, rp, s);
+    SelectParams sp{logits, L->per_expert_scale, T, E, K, idx, wts};
+    select_topk_kernel<<<(T + 3) / 4, 256, 0, s>>>(sp);
+    GroupParams gp{idx, T, K, E, (uint32_t)maxtok, has_shared ? 1 : 0, entries, n_entries, pair_token, pair_id};
+    group_decode_kernel<<<1, 1024, (pairs + 2048) * 4, s>>>(gp);
+    if (stats) NVMAI_HIP_TRY(hipMemcpyAsync(stats, n_entries, 8, hipMemcpyDeviceToDevice, s));
+
+    RowsParams p{};
+    p.src.pool_base = (const uint8_t*)L->experts_base;
+    p.src.pool_stride = L->expert_stride;
+    p.src.slot[8] = (const uint8_t*)L->shared_blob;
+    p.entries = entries; p.n_entries = n_entries; p.pair_in = pair_token; p.pair_out = pair_id;
+    set_phase1(p, L->offsets, D, F);
+    p.x = x; p.x_stride = x_stride; p.out = acts; p.out_stride = F;
+    launch_rows(ctx->act, L->bits, true, false, p, maxtok, max_entries, s);
+    RowsParams q = p;
+    set_phase2(q, L->offsets, D, F);
+    q.pair_in = pair_id;
+    q.x = acts; q.x_stride = F; q.out = partials; q.out_stride = D;
+    launch_rows(ctx->act, L->bits, false, true, q, maxtok, max_entries, s);
+    CombineParams cp{};
+    cp.partials = partials; cp.w = wts; cp.residual = nullptr; cp.gate_logit = gated ? gate_logit : nullptr;
+    cp.has_shared = has_shared ? 1 : 0; cp.tokens = T; cp.top_k = K; cp.d = D; cp.res_stride = 0;
+    cp.y_stride = y_stride; cp.y = y;
+    run_combine(ctx->act, cp, s);
+    return launch_status();
+}

@@ -1,0 +1,325 @@
+"""GPU parity: quantizer, affine GEMV, router, routed phases, shared expert and the fused
+decode layer, each called through the C ABI and compared with the CPU oracle.
+
+Bars: codes / scale bits / routing indices / router logits bit-exact; fp32 outputs within
+2e-3 and 16-bit outputs within 1e-2 of the oracle, both as max|diff| / max|ref|
+(RelError.swift:5-16)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from gpu_util import act_np, act_tensor, dev, gauss, round_act, say, u16, u32
+
+pytestmark = pytest.mark.gpu
+
+TOL_F32 = 2e-3
+TOL_ACT = 1e-2
+
+
+@pytest.fixture(scope="module")
+def nv():
+    import nvmai_amd
+    return nvmai_amd
+
+
+@pytest.fixture(scope="module", params=[0, 1], ids=["bf16", "fp16"])
+def ctx(request, nv):
+    c = nv.Context(0, request.param)
+    yield c
+    torch.cuda.synchronize()
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def ctx_bf16(nv):
+    c = nv.Context(0, 0)
+    yield c
+    torch.cuda.synchronize()
+    c.close()
+
+
+# ------------------------------------------------------------------ quantizer
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("shape", [(64, 128), (512, 2048), (2048, 512), (3, 2816)])
+def test_quantizer_codes_bit_exact(nv, ctx_bf16, bits, shape):
+    say("quantizer", bits, shape)
+    rng = np.random.default_rng(100 + bits)
+    w = gauss(rng, shape, 0.02)
+    w[0, :64] = 0.42                       # flat group
+    w[1, 64:128] = np.linspace(1, 2, 64)   # positive-only group
+    for as_bf16 in (False, True):
+        wh = O.round_bf16(w) if as_bf16 else w
+        wd = dev(wh).to(torch.bfloat16) if as_bf16 else dev(wh)
+        p, s, b = nv.quantize_affine(ctx_bf16, wd, bits)
+        torch.cuda.synchronize()
+        po, so, bo = O.quantize_affine(wh, bits)
+        assert np.array_equal(p.cpu().numpy(), po)
+        assert np.array_equal(u16(s), so) and np.array_equal(u16(b), bo)
+        codes, vals = nv.dequantize_affine(ctx_bf16, p, s, b, bits)
+        torch.cuda.synchronize()
+        assert np.array_equal(codes.cpu().numpy(), O.unpack_codes(po, bits))
+        want = O.round_bf16(O.dequantize_affine(po, so, bo, shape[1], bits)).reshape(-1)
+        assert np.array_equal(act_np(vals), want)
+
+
+# ------------------------------------------------------------------ GEMV
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,n,tokens", [(64, 128, 1), (512, 2048, 1), (2048, 512, 1), (100, 2816, 3),
+                                        (512, 2048, 7), (2048, 512, 5), (37, 1024, 2), (64, 192, 1)])
+def test_affine_gemv_matches_oracle(nv, ctx, bits, m, n, tokens):
+    say("gemv", ctx.act, bits, m, n, tokens)
+    rng = np.random.default_rng(m * 7 + n + bits)
+    p, s, b = O.quantize_affine(gauss(rng, (m, n), 0.05), bits)
+    x = round_act(gauss(rng, (tokens, n)), ctx.act)
+    want = np.stack([O.affine_gemv(p, s, b, x[t], bits) for t in range(tokens)])
+    pd, sd, bd = dev(p), dev(s.view(np.int16)), dev(b.view(np.int16))
+    y32 = nv.affine_gemv(ctx, pd, sd, bd, bits, act_tensor(x, ctx), m, n, out_f32=True)
+    y16 = nv.affine_gemv(ctx, pd, sd, bd, bits, act_tensor(x, ctx), m, n)
+    torch.cuda.synchronize()
+    assert O.rel_error(y32.cpu().numpy(), want) < TOL_F32
+    assert O.rel_error(act_np(y16), want) < TOL_ACT
+
+
+def test_gemv_bitstream_known_answer(nv, ctx_bf16):
+    # AffineQuantTests.swift:35-56: value=(row*11+col*3)&mask, scale 1, bias 0, x=1 => sum(values)
+    for bits in (4, 8):
+        say("gemv-bitstream", bits)
+        rows, cols = 3, 128
+        mask = (1 << bits) - 1
+        values = np.array([[(r * 11 + c * 3) & mask for c in range(cols)] for r in range(rows)])
+        packed = np.zeros((rows, cols * bits // 8), np.uint8)
+        for r in range(rows):
+            for c in range(cols):
+                packed[r, c * bits // 8] |= (int(values[r, c]) << ((c * bits) % 8)) & 0xFF
+        one = np.full((rows, 2), 0x3F80, np.uint16).view(np.int16)
+        zero = np.zeros((rows, 2), np.int16)
+        x = torch.ones((1, cols), dtype=torch.bfloat16, device="cuda")
+        y = nv.affine_gemv(ctx_bf16, dev(packed), dev(one), dev(zero), bits, x, rows, cols, out_f32=True)
+        torch.cuda.synchronize()
+        assert np.array_equal(y.cpu().numpy()[0], values.sum(1).astype(np.float32))
+
+
+def test_gemv_rejects_bad_arguments(nv, ctx_bf16):
+    say("gemv-errors")
+    w = torch.zeros(64 * 128, dtype=torch.uint8, device="cuda")
+    s = torch.zeros(64 * 2, dtype=torch.int16, device="cuda")
+    x = torch.zeros((1, 128), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(nv.NvmaiError) as e:
+        nv.affine_gemv(ctx_bf16, w, s, s, 6, x, 64, 128)
+    assert e.value.name == "unsupported"
+    with pytest.raises(nv.NvmaiError) as e:
+        nv.affine_gemv(ctx_bf16, w, s, s, 4, x[:, :100], 64, 100)       # n % 64 != 0
+    assert e.value.name == "invalid_arg"
+    with pytest.raises(nv.NvmaiError) as e:
+        nv.affine_gemv(ctx_bf16, w[1:], s, s, 8, x, 8, 128)             # misaligned weights
+    assert e.value.name == "alignment"
+
+
+# ------------------------------------------------------------------ router
+def _router_case(nv, ctx, kind, E, D, tokens, k, rng, eff=None, pes=None, w=None, x=None):
+    if w is None:
+        w = O.round_bf16(gauss(rng, (E, D), 0.02))
+    if x is None:
+        x = round_act(gauss(rng, (tokens, D)), ctx.act)
+    if kind == 16:
+        host = (O.bf16_bits(w), None, None)
+        desc = nv.rows_desc(16, dev(host[0].view(np.int16)))
+    else:
+        host = O.quantize_affine(w, kind)
+        desc = nv.rows_desc(kind, dev(host[0]), dev(host[1].view(np.int16)), dev(host[2].view(np.int16)))
+    effd = None if eff is None else dev(eff.view(np.int16))
+    pesd = None if pes is None else dev(pes.view(np.int16))
+    moe = nv.MoE(ctx)
+    idx, wt, logits = moe.encode_router(desc, act_tensor(x, ctx), E, D, k, effd, pesd, want_logits=True)
+    torch.cuda.synchronize()
+    for t in range(x.shape[0]):
+        lo = O.router_logits(kind, host[0], host[1], host[2], x[t], eff)
+        assert np.array_equal(logits[t].cpu().numpy().view(np.uint32), lo.view(np.uint32)), "logits bits"
+        io, wo = O.router_topk(lo, k, pes)
+        assert np.array_equal(u32(idx[t]), io)
+        assert np.abs(act_np(wt[t]) - O.f16_to_float(wo)).max() < 5e-3     # RouterTopKTests.swift:43
+        assert np.abs(u16(wt[t]).astype(np.int32) - wo.astype(np.int32)).max() <= 1   # fp16 ulp
+    return idx, wt
+
+
+@pytest.mark.parametrize("kind", [16, 8, 4])
+def test_router_indices_and_logits_bit_exact(nv, ctx, kind):
+    rng = np.random.default_rng(kind)
+    for E, D, tokens, k in [(256, 2048, 9, 8), (16, 128, 3, 8), (100, 512, 2, 4), (256, 2048, 1, 8)]:
+        say("router", ctx.act, kind, E, D, tokens, k)
+        _router_case(nv, ctx, kind, E, D, tokens, k, rng)
+    say("router scales", kind)
+    eff = O.bf16_bits(rng.uniform(0.5, 1.5, 128).astype(np.float32) / np.float32(math.sqrt(128)))
+    pes = O.bf16_bits(rng.uniform(0.6, 1.4, 16).astype(np.float32))
+    _router_case(nv, ctx, kind, 16, 128, 4, 8, rng, eff, pes)
+
+
+def test_router_near_tie_and_exact_ties(nv, ctx_bf16):
+    # RouterTopKTests.swift:46-70: gains 0.5 and 0.5*(1+1e-4) must order like the reference
+    say("router near tie")
+    E, D = 16, 128
+    g = O.SplitMix64(0x71E0F4A)
+    pattern = g.uniform_array(D, 0.2, 1.0)
+    hidden = O.round_bf16(g.uniform_array(D, 0.5, 1.5))[None, :]
+    gains = np.array([1.0 - e * 0.05 for e in range(7)] + [0.5, 0.5 * (1 + 1e-4)] +
+                     [0.4 - (e - 9) * 0.02 for e in range(9, E)], np.float32)
+    w = np.stack([pattern * gn for gn in gains]).astype(np.float32)
+    idx, _ = _router_case(nv, ctx_bf16, 8, E, D, 1, 8, None, w=w, x=hidden)
+    assert list(u32(idx[0])[:7]) == list(range(7))
+    say("router exact ties")
+    w = np.tile(O.round_bf16(gauss(np.random.default_rng(1), (1, 256), 0.05)), (64, 1))  # identical rows
+    idx, wt = _router_case(nv, ctx_bf16, 16, 64, 256, 2, 8, np.random.default_rng(2), w=w)
+    assert list(u32(idx[0])) == list(range(8)) and np.all(act_np(wt) == 0.125)
+
+
+# ------------------------------------------------------------------ routed phases
+def _constant_blob(d, f, bits):
+    off = O.expert_offsets(d, f, bits)
+    blob = np.zeros(int(off[9]), np.uint8)
+    bf = lambda v: int(np.float32(v).view(np.uint32)) >> 16
+    for o, count, v in ((off[2], f * d // 64, 1 / 64), (off[5], f * d // 64, 0.5 / 64),
+                        (off[8], d * f // 64, 1 / 64)):
+        blob[int(o):int(o) + 2 * count].view(np.uint16)[:] = bf(v)
+    return blob
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_routed_pipeline_constant_blob_known_answer(nv, ctx, bits):
+    # MoEFusedFFNTests.swift:17-54: x=1, eight experts at weight 0.125 => silu(2) everywhere
+    say("constant blob", ctx.act, bits)
+    d, f, k = 128, 64, 8
+    blobs = [dev(_constant_blob(d, f, bits)) for _ in range(k)]
+    off, _ = nv.expert_offsets(d, f, bits)
+    moe = nv.MoE(ctx, bits)
+    x = torch.ones(d, dtype=ctx.dtype, device="cuda")
+    acts = torch.zeros((k, f), dtype=torch.float32, device="cuda")
+    w = torch.full((k,), 0.125, dtype=torch.float16, device="cuda")
+    res = torch.zeros(d, dtype=ctx.dtype, device="cuda")
+    y = torch.empty(d, dtype=ctx.dtype, device="cuda")
+    moe.encode_routed_phase1(blobs, off, x, acts, d, f, k)
+    moe.encode_routed_phase2_reduce(blobs, off, acts, w, res, y, d, f, k)
+    torch.cuda.synchronize()
+    assert np.abs(act_np(y) - 2.0 / (1.0 + math.exp(-2.0))).max() < 0.01
+
+
+def _random_blobs(rng, d, f, bits, count, std=0.05):
+    mk = lambda r, c: O.round_bf16(gauss(rng, (r, c), std))
+    return np.stack([O.pack_expert(mk(f, d), mk(f, d), mk(d, f), bits) for _ in range(count)])
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("d,f", [(128, 64), (2048, 512), (1024, 256), (192, 128)])
+def test_routed_phases_match_oracle_and_split_equals_full(nv, ctx, bits, d, f):
+    say("routed phases", ctx.act, bits, d, f)
+    rng = np.random.default_rng(d + f + bits)
+    k = 8
+    host = _random_blobs(rng, d, f, bits, k, 0.05 if d < 1024 else 0.02)
+    blobs = [dev(host[i]) for i in range(k)]
+    off, stride = nv.expert_offsets(d, f, bits)
+    assert stride == host.shape[1]
+    x = round_act(gauss(rng, d), ctx.act)
+    rw = O.f16_bits(rng.dirichlet(np.ones(k)).astype(np.float32))
+    residual = round_act(gauss(rng, d, 0.1), ctx.act)
+    want = residual.copy()
+    for i in range(k):
+        O.expert_ffn_accumulate(host[i], bits, x, d, f, float(O.f16_to_float(rw[i])), want)
+    moe = nv.MoE(ctx, bits)
+    xd = act_tensor(x, ctx)
+    acts = torch.zeros((k, f), dtype=torch.float32, device="cuda")
+    y = torch.empty(d, dtype=ctx.dtype, device="cuda")
+    moe.encode_routed_phase1(blobs, off, xd, acts, d, f, k)
+    moe.encode_routed_phase2_reduce(blobs, off, acts, dev(rw.view(np.float16)), act_tensor(residual, ctx), y, d, f, k)
+    torch.cuda.synchronize()
+    assert O.rel_error(act_np(y), want) < TOL_ACT
+    # hit/miss split (MoEFusedFFNTests.swift:195-197): two subset launches == one full launch, bit for bit
+    acts2 = torch.zeros_like(acts)
+    hits = torch.tensor([0, 2, 3, 7], dtype=torch.int32, device="cuda")
+    miss = torch.tensor([1, 4, 5, 6, 99], dtype=torch.int32, device="cuda")[:4]
+    moe.encode_routed_phase1(blobs, off, xd, acts2, d, f, k, active_slots=hits)
+    moe.encode_routed_phase1(blobs, off, xd, acts2, d, f, k, active_slots=miss)
+    torch.cuda.synchronize()
+    assert torch.equal(acts, acts2)
+    # slots >= top_k are skipped
+    acts3 = torch.full_like(acts, 7.0)
+    moe.encode_routed_phase1(blobs, off, xd, acts3, d, f, k,
+                             active_slots=torch.tensor([5, 8, 1000], dtype=torch.int32, device="cuda"))
+    torch.cuda.synchronize()
+    assert torch.equal(acts3[5], acts[5]) and bool((acts3[[0, 1, 2, 3, 4, 6, 7]] == 7.0).all())
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_shared_expert_with_scalar_gate(nv, ctx, bits):
+    rng = np.random.default_rng(bits)
+    for d, f, tokens in [(128, 64, 1), (2048, 512, 1), (2048, 512, 6), (256, 128, 9)]:
+        say("shared expert", ctx.act, bits, d, f, tokens)
+        host = _random_blobs(rng, d, f, bits, 1, 0.03)[0]
+        gate = O.quantize_affine(O.round_bf16(gauss(rng, (1, d), 0.05)), 8)
+        x = round_act(gauss(rng, (tokens, d)), ctx.act)
+        off, _ = nv.expert_offsets(d, f, bits)
+        se = nv.SharedExpertRuntime(ctx, bits)
+        gdesc = nv.rows_desc(8, dev(gate[0]), dev(gate[1].view(np.int16)), dev(gate[2].view(np.int16)))
+        y = se.encode(dev(host), off, act_tensor(x, ctx), d, f, gdesc)
+        y0 = se.encode(dev(host), off, act_tensor(x, ctx), d, f, None)
+        torch.cuda.synchronize()
+        for t in range(tokens):
+            plain = O.expert_ffn_accumulate(host, bits, x[t], d, f, 1.0, np.zeros(d, np.float32))
+            g = O.router_logits(8, gate[0], gate[1], gate[2], x[t])[0]
+            assert O.rel_error(act_np(y0[t]), plain) < TOL_ACT
+            assert O.rel_error(act_np(y[t]), plain / (1 + np.exp(-g))) < TOL_ACT
+    with pytest.raises(nv.NvmaiError) as e:                 # SharedExpertError.unsupportedWeightBits
+        nv.SharedExpertRuntime(ctx, 6)
+    assert e.value.name == "unsupported"
+
+
+# ------------------------------------------------------------------ fused decode layer
+def _layer_case(nv, ctx, rng, d, f, E, k, bits, tokens, router_kind, std):
+    mk = lambda r, c, s_=std: O.round_bf16(gauss(rng, (r, c), s_))
+    # build the pool on the GPU with the (bit-exact) device quantizer, then read it back
+    off, stride = nv.expert_offsets(d, f, bits)
+    pool = torch.empty((E + 1, stride), dtype=torch.uint8, device="cuda")
+    for e in range(E + 1):
+        gw = torch.randn((f, d), device="cuda", dtype=torch.float32).mul_(std).to(torch.bfloat16)
+        uw = torch.randn((f, d), device="cuda", dtype=torch.float32).mul_(std).to(torch.bfloat16)
+        dw = torch.randn((d, f), device="cuda", dtype=torch.float32).mul_(std).to(torch.bfloat16)
+        nv.pack_expert(ctx, gw, uw, dw, bits, pool[e])
+    torch.cuda.synchronize()
+    pool_h = pool.cpu().numpy()
+    rw = mk(E, d, 0.02)
+    if router_kind == 16:
+        rh = (O.bf16_bits(rw), None, None)
+        rdesc = nv.rows_desc(16, dev(rh[0].view(np.int16)))
+    else:
+        rh = O.quantize_affine(rw, router_kind)
+        rdesc = nv.rows_desc(router_kind, dev(rh[0]), dev(rh[1].view(np.int16)), dev(rh[2].view(np.int16)))
+    gh = O.quantize_affine(mk(1, d, 0.05), 8)
+    gdesc = nv.rows_desc(8, dev(gh[0]), dev(gh[1].view(np.int16)), dev(gh[2].view(np.int16)))
+    x = round_act(gauss(rng, (tokens, d)), ctx.act)
+    layer = nv.moe_layer_desc(d, f, E, k, bits, rdesc, pool[:E], pool[E], gdesc)
+    stats = torch.zeros(2, dtype=torch.int32, device="cuda")
+    y, idx, w = nv.MoE(ctx, bits).decode_layer(layer, act_tensor(x, ctx), want_routes=True, stats=stats)
+    torch.cuda.synchronize()
+    io, wo, yo = O.moe_layer_forward(x, d, f, k, bits, (router_kind,) + rh, pool_h[:E], pool_h[E], (8,) + gh)
+    assert np.array_equal(u32(idx), io), "routing indices"
+    assert np.abs(u16(w).astype(np.int32) - wo.astype(np.int32)).max() <= 1
+    assert O.rel_error(act_np(y), yo) < TOL_ACT
+    assert int(stats[1]) == len(np.unique(io))
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_decode_layer_toy_shapes(nv, ctx, bits):
+    rng = np.random.default_rng(40 + bits)
+    for d, f, E, k, tokens, kind in [(128, 64, 16, 8, 1, 8), (128, 64, 16, 8, 5, 16), (256, 128, 32, 4, 11, 4),
+                                     (192, 64, 8, 2, 3, 16)]:
+        say("decode layer toy", ctx.act, bits, d, f, E, k, tokens, kind)
+        _layer_case(nv, ctx, rng, d, f, E, k, bits, tokens, kind, 0.05)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("tokens", [1, 4, 32])
+def test_decode_layer_production_shape(nv, ctx_bf16, bits, tokens):
+    # configs[1]: hidden 2048, 256 experts top-8, intermediate 512, shared expert with sigmoid gate
+    say("decode layer production", bits, tokens)
+    _layer_case(nv, ctx_bf16, np.random.default_rng(tokens + bits), 2048, 512, 256, 8, bits, tokens, 16, 0.02)
