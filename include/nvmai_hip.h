@@ -67,6 +67,21 @@ int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** out);
 void nvmai_hip_ctx_destroy(nvmai_hip_ctx* ctx);
 const char* nvmai_hip_status_string(int status);
 
+/* Per-kernel timing, the counterpart of the reference's NVMAI_KERNEL_STATS roles
+ * (RealForwardRunner.swift:1129-1188): while enabled, each tagged kernel launch is
+ * bracketed by events on its stream.  profile_read waits for the recorded events,
+ * returns the summed milliseconds and launch count of one tag and leaves the
+ * records in place; profile_enable(…, 1) clears them. */
+enum {
+    NVMAI_PROF_ROUTER = 0, NVMAI_PROF_SELECT = 1, NVMAI_PROF_GROUP = 2, NVMAI_PROF_PHASE1 = 3,
+    NVMAI_PROF_PHASE2 = 4, NVMAI_PROF_COMBINE = 5, NVMAI_PROF_KV_QUANT = 6, NVMAI_PROF_ATTN_PARTIAL = 7,
+    NVMAI_PROF_ATTN_COMBINE = 8, NVMAI_PROF_SOFTMAX = 9, NVMAI_PROF_SAMPLE = 10,
+    NVMAI_PROF_PREFILL_GROUP = 11, NVMAI_PROF_PREFILL_GEMM1 = 12, NVMAI_PROF_PREFILL_GEMM2 = 13,
+    NVMAI_PROF_PREFILL_COMBINE = 14, NVMAI_PROF_TAGS = 16
+};
+int nvmai_hip_profile_enable(nvmai_hip_ctx* ctx, int on);
+int nvmai_hip_profile_read(nvmai_hip_ctx* ctx, int tag, double* total_ms, uint32_t* launches);
+
 /* CPUExpertFFN.Offsets(d:f:) (CPUExpertFFN.swift:42-59) for `bits` in {4,8}.
  * Host-only arithmetic; *stride_bytes receives the blob size. */
 int nvmai_expert_offsets_for(uint32_t d, uint32_t f, uint32_t bits,

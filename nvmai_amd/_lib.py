@@ -48,6 +48,8 @@ class MoeLayer(C.Structure):
 # name -> argtypes (every function returns int unless listed in _OTHER)
 SIGNATURES = {
     "nvmai_hip_ctx_create": [C.c_int, C.c_int, C.POINTER(vp)],
+    "nvmai_hip_profile_enable": [vp, C.c_int],
+    "nvmai_hip_profile_read": [vp, C.c_int, C.POINTER(C.c_double), C.POINTER(u32)],
     "nvmai_expert_offsets_for": [u32, u32, u32, C.POINTER(ExpertOffsets), C.POINTER(u64)],
     "nvmai_hip_quantize_affine": [vp, vp, vp, C.c_int, u32, u32, u32, vp, vp, vp],
     "nvmai_hip_dequantize_affine": [vp, vp, vp, vp, vp, u64, u32, vp, vp],

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <vector>
+
 #include "../../include/nvmai_hip.h"
 
 struct nvmai_hip_ctx {
@@ -14,6 +16,11 @@ struct nvmai_hip_ctx {
     uint8_t* ws;
     size_t ws_cap;
     size_t ws_used;
+    // Optional per-kernel timing: event pairs recorded around tagged launches.
+    bool prof_on;
+    struct ProfSpan { int tag; hipEvent_t start, stop; };
+    std::vector<ProfSpan> prof_spans;
+    std::vector<hipEvent_t> prof_free;
 };
 
 namespace nvmai {
@@ -49,6 +56,25 @@ inline T* ws_take(nvmai_hip_ctx* ctx, size_t count) {
     ctx->ws_used += ws_round(count * sizeof(T));
     return p;
 }
+
+// Brackets the launches of one kernel with events while profiling is switched on.
+struct ProfScope {
+    nvmai_hip_ctx* ctx;
+    hipStream_t stream;
+    hipEvent_t stop;
+    ProfScope(nvmai_hip_ctx* c, int tag, hipStream_t s) : ctx(c), stream(s), stop(nullptr) {
+        if (!c->prof_on) return;
+        hipEvent_t ev[2] = {nullptr, nullptr};
+        for (auto& e : ev) {
+            if (!c->prof_free.empty()) { e = c->prof_free.back(); c->prof_free.pop_back(); }
+            else if (hipEventCreate(&e) != hipSuccess) return;
+        }
+        (void)hipEventRecord(ev[0], s);
+        stop = ev[1];
+        c->prof_spans.push_back({tag, ev[0], ev[1]});
+    }
+    ~ProfScope() { if (stop) (void)hipEventRecord(stop, stream); }
+};
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? NVMAI_OK : NVMAI_ERR_HIP; }
 

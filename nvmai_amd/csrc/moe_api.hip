@@ -23,6 +23,7 @@ extern "C" int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** o
     ctx->ws = nullptr;
     ctx->ws_cap = 0;
     ctx->ws_used = 0;
+    ctx->prof_on = false;
     *out = ctx;
     return NVMAI_OK;
 }
@@ -30,7 +31,40 @@ extern "C" int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** o
 extern "C" void nvmai_hip_ctx_destroy(nvmai_hip_ctx* ctx) {
     if (!ctx) return;
     if (ctx->ws) (void)hipFree(ctx->ws);
+    for (auto& sp : ctx->prof_spans) { (void)hipEventDestroy(sp.start); (void)hipEventDestroy(sp.stop); }
+    for (auto& e : ctx->prof_free) (void)hipEventDestroy(e);
     delete ctx;
+}
+
+extern "C" int nvmai_hip_profile_enable(nvmai_hip_ctx* ctx, int on) {
+    if (!ctx) return NVMAI_ERR_INVALID_ARG;
+    if (on) {
+        for (auto& sp : ctx->prof_spans) {
+            NVMAI_HIP_TRY(hipEventSynchronize(sp.stop));
+            ctx->prof_free.push_back(sp.start);
+            ctx->prof_free.push_back(sp.stop);
+        }
+        ctx->prof_spans.clear();
+    }
+    ctx->prof_on = on != 0;
+    return NVMAI_OK;
+}
+
+extern "C" int nvmai_hip_profile_read(nvmai_hip_ctx* ctx, int tag, double* total_ms, uint32_t* launches) {
+    if (!ctx || !total_ms || !launches) return NVMAI_ERR_INVALID_ARG;
+    double total = 0.0;
+    uint32_t n = 0;
+    for (auto& sp : ctx->prof_spans) {
+        if (sp.tag != tag) continue;
+        NVMAI_HIP_TRY(hipEventSynchronize(sp.stop));
+        float ms = 0.0f;
+        NVMAI_HIP_TRY(hipEventElapsedTime(&ms, sp.start, sp.stop));
+        total += ms;
+        ++n;
+    }
+    *total_ms = total;
+    *launches = n;
+    return NVMAI_OK;
 }
 
 extern "C" const char* nvmai_hip_status_string(int status) {
@@ -511,11 +545,11 @@ extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream strea
     if (gated) rp.gate = to_desc(&L->shared_gate);
     rp.x = x; rp.eff_scale = L->eff_scale; rp.x_stride = x_stride; rp.tokens = T;
     rp.num_experts = E; rp.d = D; rp.logits = logits; rp.gate_logit = gate_logit;
-    run_router(ctx->act, rp, s);
+    { ProfScope ps(ctx, NVMAI_PROF_ROUTER, s); run_router(ctx->act, rp, s); }
     SelectParams sp{logits, L->per_expert_scale, T, E, K, idx, wts};
-    select_topk_kernel<<<(T + 3) / 4, 256, 0, s>>>(sp);
+    { ProfScope ps(ctx, NVMAI_PROF_SELECT, s); select_topk_kernel<<<(T + 3) / 4, 256, 0, s>>>(sp); }
     GroupParams gp{idx, T, K, E, (uint32_t)maxtok, has_shared ? 1 : 0, entries, n_entries, pair_token, pair_id};
-    group_decode_kernel<<<1, 1024, (pairs + 2048) * 4, s>>>(gp);
+    { ProfScope ps(ctx, NVMAI_PROF_GROUP, s); group_decode_kernel<<<1, 1024, (pairs + 2048) * 4, s>>>(gp); }
     if (stats) NVMAI_HIP_TRY(hipMemcpyAsync(stats, n_entries, 8, hipMemcpyDeviceToDevice, s));
 
     RowsParams p{};
@@ -525,16 +559,16 @@ extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream strea
     p.entries = entries; p.n_entries = n_entries; p.pair_in = pair_token; p.pair_out = pair_id;
     set_phase1(p, L->offsets, D, F);
     p.x = x; p.x_stride = x_stride; p.out = acts; p.out_stride = F;
-    launch_rows(ctx->act, L->bits, true, false, p, maxtok, max_entries, s);
+    { ProfScope ps(ctx, NVMAI_PROF_PHASE1, s); launch_rows(ctx->act, L->bits, true, false, p, maxtok, max_entries, s); }
     RowsParams q = p;
     set_phase2(q, L->offsets, D, F);
     q.pair_in = pair_id;
     q.x = acts; q.x_stride = F; q.out = partials; q.out_stride = D;
-    launch_rows(ctx->act, L->bits, false, true, q, maxtok, max_entries, s);
+    { ProfScope ps(ctx, NVMAI_PROF_PHASE2, s); launch_rows(ctx->act, L->bits, false, true, q, maxtok, max_entries, s); }
     CombineParams cp{};
     cp.partials = partials; cp.w = wts; cp.residual = nullptr; cp.gate_logit = gated ? gate_logit : nullptr;
     cp.has_shared = has_shared ? 1 : 0; cp.tokens = T; cp.top_k = K; cp.d = D; cp.res_stride = 0;
     cp.y_stride = y_stride; cp.y = y;
-    run_combine(ctx->act, cp, s);
+    { ProfScope ps(ctx, NVMAI_PROF_COMBINE, s); run_combine(ctx->act, cp, s); }
     return launch_status();
 }

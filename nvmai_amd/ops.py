@@ -10,6 +10,9 @@ from . import _lib
 from ._lib import ExpertOffsets, MoeLayer, Rows, check, lib
 
 ACT_BF16, ACT_FP16 = 0, 1
+(PROF_ROUTER, PROF_SELECT, PROF_GROUP, PROF_PHASE1, PROF_PHASE2, PROF_COMBINE, PROF_KV_QUANT,
+ PROF_ATTN_PARTIAL, PROF_ATTN_COMBINE, PROF_SOFTMAX, PROF_SAMPLE, PROF_PREFILL_GROUP,
+ PROF_PREFILL_GEMM1, PROF_PREFILL_GEMM2, PROF_PREFILL_COMBINE) = range(15)
 _ACT_TORCH = {ACT_BF16: torch.bfloat16, ACT_FP16: torch.float16}
 
 
@@ -31,6 +34,15 @@ class Context:
         h = C.c_void_p()
         check(lib.nvmai_hip_ctx_create(device, act, C.byref(h)), "ctx_create")
         self.handle = h
+
+    def profile_enable(self, on=True):
+        check(lib.nvmai_hip_profile_enable(self.handle, int(on)), "profile_enable")
+
+    def profile_read(self, tag):
+        """Summed milliseconds and launch count of one NVMAI_PROF_* tag."""
+        ms, n = C.c_double(), C.c_uint32()
+        check(lib.nvmai_hip_profile_read(self.handle, tag, C.byref(ms), C.byref(n)), "profile_read")
+        return ms.value, n.value
 
     def close(self):
         if self.handle:
