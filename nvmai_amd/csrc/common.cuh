@@ -78,6 +78,33 @@ __device__ __forceinline__ float seg_reduce_sum(float v) {
     return v;
 }
 
+// Wave-wide max / min through the same DPP ladder; lanes a step does not reach
+// keep their own value (bound_ctrl off, old = own value), result broadcast.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_keep(int v) {
+    return __builtin_amdgcn_update_dpp(v, v, CTRL, ROW_MASK, 0xF, false);
+}
+
+__device__ __forceinline__ float wave_max_f32(float v) {
+    v = fmaxf(v, __int_as_float(dpp_keep<0xB1, 0xF>(__float_as_int(v))));
+    v = fmaxf(v, __int_as_float(dpp_keep<0x4E, 0xF>(__float_as_int(v))));
+    v = fmaxf(v, __int_as_float(dpp_keep<0x141, 0xF>(__float_as_int(v))));
+    v = fmaxf(v, __int_as_float(dpp_keep<0x140, 0xF>(__float_as_int(v))));
+    v = fmaxf(v, __int_as_float(dpp_keep<0x142, 0xA>(__float_as_int(v))));
+    v = fmaxf(v, __int_as_float(dpp_keep<0x143, 0xC>(__float_as_int(v))));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+    v = min(v, (uint32_t)dpp_keep<0xB1, 0xF>((int)v));
+    v = min(v, (uint32_t)dpp_keep<0x4E, 0xF>((int)v));
+    v = min(v, (uint32_t)dpp_keep<0x141, 0xF>((int)v));
+    v = min(v, (uint32_t)dpp_keep<0x140, 0xF>((int)v));
+    v = min(v, (uint32_t)dpp_keep<0x142, 0xA>((int)v));
+    v = min(v, (uint32_t)dpp_keep<0x143, 0xC>((int)v));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
 // Lane of a SEG-lane segment that holds seg_reduce_sum's result.
 template <int SEG>
 __device__ __forceinline__ bool seg_result_lane(int lane) {
@@ -140,5 +167,11 @@ __device__ __forceinline__ void unpack_chunk(const uint4& w, float* q) {
 }
 
 __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
+
+// silu through the hardware exp2 and reciprocal (about 1e-6 relative): for kernels
+// whose result is rounded to 16 bits or compared at 1e-3.
+__device__ __forceinline__ float silu_fast(float v) {
+    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v));
+}
 
 }  // namespace nvmai

@@ -16,6 +16,7 @@ struct nvmai_hip_ctx {
     uint8_t* ws;
     size_t ws_cap;
     size_t ws_used;
+    uint32_t* tickets;       // small zero-initialised device array for last-block-done kernels
     // Optional per-kernel timing: event pairs recorded around tagged launches.
     bool prof_on;
     struct ProfSpan { int tag; hipEvent_t start, stop; };

@@ -1,5 +1,6 @@
 // Entry points of the decode-side MoE path: context, quantizer, affine GEMV,
 // router top-k, routed phase 1 / phase 2, shared expert, fused decode layer.
+#include <cstdlib>
 #include <new>
 
 #include "ctx.hpp"
@@ -24,6 +25,12 @@ extern "C" int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** o
     ctx->ws_cap = 0;
     ctx->ws_used = 0;
     ctx->prof_on = false;
+    ctx->tickets = nullptr;
+    if (hipMalloc(reinterpret_cast<void**>(&ctx->tickets), 256) != hipSuccess ||
+        hipMemset(ctx->tickets, 0, 256) != hipSuccess) {
+        delete ctx;
+        return NVMAI_ERR_HIP;
+    }
     *out = ctx;
     return NVMAI_OK;
 }
@@ -31,6 +38,7 @@ extern "C" int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** o
 extern "C" void nvmai_hip_ctx_destroy(nvmai_hip_ctx* ctx) {
     if (!ctx) return;
     if (ctx->ws) (void)hipFree(ctx->ws);
+    if (ctx->tickets) (void)hipFree(ctx->tickets);
     for (auto& sp : ctx->prof_spans) { (void)hipEventDestroy(sp.start); (void)hipEventDestroy(sp.stop); }
     for (auto& e : ctx->prof_free) (void)hipEventDestroy(e);
     delete ctx;
@@ -110,8 +118,9 @@ template <int ACT, int BITS, int SEG, int NCH, int MAXTOK, bool DUAL, bool XF32,
 void launch_fast(RowsParams& p, uint32_t max_entries, hipStream_t s) {
     constexpr uint32_t rows_per_block = 4 * (64 / SEG) * RPI * ITERS;
     p.blocks_per_entry = (p.rows + rows_per_block - 1) / rows_per_block;
+    const size_t lds = rows_fast_lds_bytes(p.n, NCH, SEG);
     expert_rows_fast<ACT, BITS, SEG, NCH, MAXTOK, DUAL, XF32, RPI, ITERS>
-        <<<dim3(max_entries * p.blocks_per_entry), dim3(256), 0, s>>>(p);
+        <<<dim3(max_entries * p.blocks_per_entry), dim3(256), lds, s>>>(p);
 }
 
 template <int ACT, int BITS, bool DUAL, bool XF32>
@@ -123,14 +132,23 @@ void launch_rows_t(RowsParams& p, int maxtok, uint32_t max_entries, hipStream_t 
         else launch_fast<ACT, BITS, SEG, NCH, 4, DUAL, XF32, RPI, ITERS>(p, max_entries, s);    \
         return;                                                                                 \
     } while (0)
+    static const int variant = getenv("NVMAI_ROWS_VARIANT") ? atoi(getenv("NVMAI_ROWS_VARIANT")) : 0;
     if constexpr (DUAL) {
-        if (chunks == 64) NVMAI_FAST(64, 1, 2, 2);
-        if (chunks == 128) NVMAI_FAST(64, 2, 2, 2);
+        if (chunks == 64) NVMAI_FAST(64, 1, 1, 8);
+        if (chunks == 128 && variant % 10 == 1) NVMAI_FAST(32, 4, 1, 8);
+        if (chunks == 128 && variant % 10 == 2) NVMAI_FAST(32, 4, 1, 4);
+        if (chunks == 128 && variant % 10 == 3) NVMAI_FAST(64, 2, 1, 4);
+        if (chunks == 128 && variant % 10 == 4) NVMAI_FAST(64, 2, 1, 16);
+        if (chunks == 128) NVMAI_FAST(64, 2, 1, 8);
     } else {
-        if (chunks == 16) NVMAI_FAST(16, 1, 2, 2);
-        if (chunks == 32) NVMAI_FAST(32, 1, 4, 2);
-        if (chunks == 64) NVMAI_FAST(64, 1, 4, 1);
-        if (chunks == 128) NVMAI_FAST(64, 2, 4, 1);
+        if (chunks == 16) NVMAI_FAST(16, 1, 1, 8);
+        if (chunks == 32 && variant / 10 == 1) NVMAI_FAST(16, 2, 1, 8);
+        if (chunks == 32 && variant / 10 == 2) NVMAI_FAST(16, 2, 2, 4);
+        if (chunks == 32 && variant / 10 == 3) NVMAI_FAST(32, 1, 2, 4);
+        if (chunks == 32 && variant / 10 == 4) NVMAI_FAST(32, 1, 4, 4);
+        if (chunks == 32) NVMAI_FAST(32, 1, 2, 8);
+        if (chunks == 64) NVMAI_FAST(64, 1, 2, 4);
+        if (chunks == 128) NVMAI_FAST(64, 2, 1, 8);
     }
 #undef NVMAI_FAST
     p.blocks_per_entry = (p.rows + 15) / 16;
@@ -182,11 +200,29 @@ void set_phase2(RowsParams& p, const nvmai_expert_offsets& o, uint32_t d, uint32
     p.rows = d; p.n = f;
 }
 
-void run_router(int act, const RouterParams& rp, hipStream_t s) {
+// chunks of 16 bytes per row of d elements in router format `kind`
+uint32_t rows_chunks(int kind, uint32_t d) { return kind == 16 ? d / 8 : (kind == 8 ? d / 16 : d / 32); }
+
+template <int ACT>
+void run_router_t(const RouterParams& rp, uint32_t cpl, dim3 grid, hipStream_t s) {
+    if (cpl <= 1) router_logits_kernel<ACT, 1><<<grid, 256, 0, s>>>(rp);
+    else if (cpl <= 2) router_logits_kernel<ACT, 2><<<grid, 256, 0, s>>>(rp);
+    else if (cpl <= 4) router_logits_kernel<ACT, 4><<<grid, 256, 0, s>>>(rp);
+    else router_logits_kernel<ACT, 8><<<grid, 256, 0, s>>>(rp);
+}
+
+// d <= 2048 dense / 4096 at 8 bit / 8192 at 4 bit (8 chunks per lane).
+int run_router(int act, RouterParams& rp, hipStream_t s) {
+    rp.x_vec = aligned16(rp.x) && (rp.x_stride % 8 == 0);
+    uint32_t chunks = rp.router.kind ? rows_chunks(rp.router.kind, rp.d) : 0;
+    if (rp.gate.kind) chunks = chunks > rows_chunks(rp.gate.kind, rp.d) ? chunks : rows_chunks(rp.gate.kind, rp.d);
+    const uint32_t cpl = (chunks + 31) / 32;
+    if (cpl > 8) return NVMAI_ERR_UNSUPPORTED;
     const uint32_t rows = rp.num_experts + (rp.gate.kind ? 1u : 0u);
     dim3 grid((rows + 7) / 8, (rp.tokens + ROUTER_TOK - 1) / ROUTER_TOK);
-    if (act == ACT_BF16) router_logits_kernel<ACT_BF16><<<grid, 256, 0, s>>>(rp);
-    else router_logits_kernel<ACT_FP16><<<grid, 256, 0, s>>>(rp);
+    if (act == ACT_BF16) run_router_t<ACT_BF16>(rp, cpl, grid, s);
+    else run_router_t<ACT_FP16>(rp, cpl, grid, s);
+    return NVMAI_OK;
 }
 
 int check_rows_desc(const nvmai_rows* r, uint32_t d, bool allow_absent) {
@@ -323,7 +359,8 @@ extern "C" int nvmai_hip_moe_router_topk(nvmai_hip_ctx* ctx, nvmai_stream stream
     rp.router = to_desc(router);
     rp.x = hidden; rp.eff_scale = eff_scale; rp.x_stride = hidden_stride; rp.tokens = n_tokens;
     rp.num_experts = num_experts; rp.d = d; rp.logits = logits; rp.gate_logit = nullptr;
-    run_router(ctx->act, rp, s);
+    rc = run_router(ctx->act, rp, s);
+    if (rc) return rc;
     SelectParams sp{logits, per_expert_scale, n_tokens, num_experts, top_k, out_idx, out_w};
     select_topk_kernel<<<(n_tokens + 3) / 4, 256, 0, s>>>(sp);
     return launch_status();
@@ -466,7 +503,8 @@ extern "C" int nvmai_hip_shared_expert(nvmai_hip_ctx* ctx, nvmai_stream stream, 
         rp.gate = to_desc(shared_gate);
         rp.x = x; rp.x_stride = x_stride; rp.tokens = n_tokens; rp.num_experts = 0; rp.d = d;
         rp.logits = dummy_logits; rp.gate_logit = gate_logit;
-        run_router(ctx->act, rp, s);
+        rc = run_router(ctx->act, rp, s);
+        if (rc) return rc;
     }
     RowsParams p{};
     p.src.slot[8] = (const uint8_t*)blob;
@@ -545,12 +583,15 @@ extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream strea
     if (gated) rp.gate = to_desc(&L->shared_gate);
     rp.x = x; rp.eff_scale = L->eff_scale; rp.x_stride = x_stride; rp.tokens = T;
     rp.num_experts = E; rp.d = D; rp.logits = logits; rp.gate_logit = gate_logit;
-    { ProfScope ps(ctx, NVMAI_PROF_ROUTER, s); run_router(ctx->act, rp, s); }
+    { ProfScope ps(ctx, NVMAI_PROF_ROUTER, s); rc = run_router(ctx->act, rp, s); }
+    if (rc) return rc;
     SelectParams sp{logits, L->per_expert_scale, T, E, K, idx, wts};
-    { ProfScope ps(ctx, NVMAI_PROF_SELECT, s); select_topk_kernel<<<(T + 3) / 4, 256, 0, s>>>(sp); }
-    GroupParams gp{idx, T, K, E, (uint32_t)maxtok, has_shared ? 1 : 0, entries, n_entries, pair_token, pair_id};
-    { ProfScope ps(ctx, NVMAI_PROF_GROUP, s); group_decode_kernel<<<1, 1024, (pairs + 2048) * 4, s>>>(gp); }
-    if (stats) NVMAI_HIP_TRY(hipMemcpyAsync(stats, n_entries, 8, hipMemcpyDeviceToDevice, s));
+    GroupParams gp{sp, (uint32_t)maxtok, has_shared ? 1 : 0, entries, n_entries, stats, pair_token, pair_id,
+                   ctx->tickets};
+    {
+        ProfScope ps(ctx, NVMAI_PROF_GROUP, s);
+        select_group_kernel<<<(T + 3) / 4, 256, (4 * E + 8 + pairs) * 4, s>>>(gp);
+    }
 
     RowsParams p{};
     p.src.pool_base = (const uint8_t*)L->experts_base;

@@ -74,139 +74,285 @@ __device__ __forceinline__ void load_x(const void* x, size_t row_off, uint32_t e
 // ---- fast engine ------------------------------------------------------------
 // A row of n codes is n*BITS/128 chunks of 16 bytes.  SEG lanes share a row
 // (SEG*NCH chunks), so one wave covers 64/SEG rows per load instruction and
-// every load instruction moves 1 KiB of contiguous weights.  Lane inputs are
-// the same columns for every row, so they sit in registers for the whole block.
-// Per chunk the arithmetic is the reference's factoring (nvmai_kernels.h:19-21):
-// acc += scale * sum(q*x) + bias * sum(x), with sum(x) hoisted out of the row
-// loop as int4_affine_gemv.c:41-53 does.
-template <int ACT, int BITS, int SEG, int NCH, int TOK, bool DUAL, bool XF32, int RPI, int ITERS>
-__device__ __forceinline__ void expert_rows_body(const RowsParams& p, const WorkEntry& we, uint32_t rb) {
+// every load instruction moves 1 KiB of contiguous weights.  A block owns a run
+// of rows of one work entry; weight loads are double-buffered in registers, the
+// first batch being issued before the inputs are staged.
+//
+// Arithmetic.  The kernel is fed by HBM only if the VALU work per weight byte is
+// small, so the inner product runs on v_dot2_f32_f16 (two multiply-adds per lane
+// per instruction, fp32 accumulate):
+//   - a code q becomes the fp16 value 1024 + q by OR-ing it under the constant
+//     0x6400 (exact: fp16 has a unit ulp in [1024, 2048)); one byte-permute or
+//     and-or instruction builds two such values;
+//   - each input row is scaled by a power of two so that its largest magnitude
+//     lies in [1024, 2048) and is converted to fp16.  For 16-bit activations the
+//     conversion is exact for everything within 2^-24 of the row maximum, i.e.
+//     to fp32 precision; fp32 inputs (the SwiGLU activations entering the down
+//     projection) are rounded to 11 significant bits, as the reference rounds
+//     them to fp16 in memory (moe.metal:682);
+//   - per chunk sum(q*x) = dot2-sum - 1024*sum(x), then the reference's factoring
+//     (nvmai_kernels.h:19-21): acc += scale * sum(q*x) + bias * sum(x), with
+//     sum(x) hoisted out of the row loop as int4_affine_gemv.c:41-53 does;
+//   - the row result is multiplied by the inverse power of two.
+template <int BITS, int SEG, int NCH, bool DUAL, int RPI>
+struct RowStage {
+    uint4 qa[RPI][NCH], qb[DUAL ? RPI : 1][NCH];
+    uint16_t sa[RPI][NCH], ba[RPI][NCH], sb[DUAL ? RPI : 1][NCH], bb[DUAL ? RPI : 1][NCH];
+};
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), c, false);
+}
+
+// 16 bytes of codes -> packed fp16 pairs (1024 + q).  8 bit: pair m holds the
+// elements (2m, 2m+1).  4 bit: dword d of the chunk yields pairs 4d+j holding the
+// elements (8d+j, 8d+j+4); the staged inputs are packed the same way.
+template <int BITS>
+__device__ __forceinline__ void unpack_pairs(const uint4& w, uint32_t* qp) {
+    const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        if (BITS == 8) {
+            qp[2 * d] = __builtin_amdgcn_perm(ws[d], 0x64646464u, 0x00050004u);
+            qp[2 * d + 1] = __builtin_amdgcn_perm(ws[d], 0x64646464u, 0x00070006u);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) qp[4 * d + j] = ((ws[d] >> (4 * j)) & 0x000F000Fu) | 0x64006400u;
+        }
+    }
+}
+
+__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
+    return (uint32_t)f32_to_f16(lo) | ((uint32_t)f32_to_f16(hi) << 16);
+}
+
+// Eight consecutive scaled inputs -> the four packed pairs of one 16-byte LDS word.
+template <int BITS>
+__device__ __forceinline__ uint4 pack_inputs(const float* v) {
+    if (BITS == 8) return make_uint4(pack_h2(v[0], v[1]), pack_h2(v[2], v[3]), pack_h2(v[4], v[5]), pack_h2(v[6], v[7]));
+    return make_uint4(pack_h2(v[0], v[4]), pack_h2(v[1], v[5]), pack_h2(v[2], v[6]), pack_h2(v[3], v[7]));
+}
+
+template <int ACT, bool XF32>
+__device__ __forceinline__ void load8(const void* x, size_t off, float* v) {
+    if (XF32) {
+        const float4 a = *reinterpret_cast<const float4*>((const float*)x + off);
+        const float4 b = *reinterpret_cast<const float4*>((const float*)x + off + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        const uint4 a = *reinterpret_cast<const uint4*>((const uint16_t*)x + off);
+        act2_to_f32<ACT>(a.x, v[0], v[1]); act2_to_f32<ACT>(a.y, v[2], v[3]);
+        act2_to_f32<ACT>(a.z, v[4], v[5]); act2_to_f32<ACT>(a.w, v[6], v[7]);
+    }
+}
+
+// Power of two that maps amax into [1024, 2048), and its inverse; 1 when amax is
+// zero, denormal-small, infinite or NaN.
+__device__ __forceinline__ void pow2_scale(float amax, float& sc, float& isc) {
+    const uint32_t e = (__float_as_uint(amax) >> 23) & 0xFFu;
+    if (e < 24u || e > 254u) { sc = 1.0f; isc = 1.0f; return; }
+    sc = __uint_as_float((264u - e) << 23);      // 2^(10 - (e - 127))
+    isc = __uint_as_float((e - 10u) << 23);      // 2^((e - 127) - 10)
+}
+
+// TOKS = 1: exactly one input, kept in registers for the whole block.  TOKS = 0:
+// we.pair_count inputs (2..MAX_TOK), walked by a real loop inside each stage so
+// that only one input's columns are live at a time.
+// LDS: [ntok][n/8] uint4 packed inputs | [ntok][NCH*SEG] float chunk sums |
+//      [MAX_TOK*4] float wave maxima | [MAX_TOK] float inverse scales.
+template <int ACT, int BITS, int SEG, int NCH, int TOKS, bool DUAL, bool XF32, int RPI, int ITERS>
+__device__ __forceinline__ void expert_rows_body(const RowsParams& p, const WorkEntry& we, uint32_t rb,
+                                                 uint4* lds) {
     constexpr int EPC = Chunk<BITS>::elems;
+    constexpr int PAIRS = EPC / 2;                // packed pairs per chunk
+    constexpr int H = PAIRS / 4;                  // 16-byte LDS words per chunk
     constexpr int RPL = 64 / SEG;                 // rows per load instruction
     constexpr int ROWS_WAVE = RPL * RPI * ITERS;
+    constexpr int WORDS_TOK = NCH * H * SEG;      // == n / 8
+    static_assert(ITERS % 2 == 0, "ITERS must be even (double buffering)");
+    using Stage = RowStage<BITS, SEG, NCH, DUAL, RPI>;
+    const int ntok = TOKS ? TOKS : (int)we.pair_count;
     const uint8_t* blob = blob_ptr(p.src, we.expert);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int seg_id = lane / SEG, sl = lane % SEG;
     const uint32_t groups = p.n / NVMAI_GROUP;
     const uint32_t row_bytes = p.n * BITS / 8;
-
-    float xr[TOK][NCH][EPC];
-    float xs[TOK][NCH];
-    uint32_t out_row[TOK];
-#pragma unroll
-    for (int t = 0; t < TOK; ++t) {
-        const bool live = (uint32_t)t < we.pair_count;
-        const uint32_t pi = we.pair_start + (live ? t : 0);
-        const size_t in_off = (size_t)p.pair_in[pi] * p.x_stride;
-        out_row[t] = p.pair_out[pi];
-#pragma unroll
-        for (int c = 0; c < NCH; ++c) {
-            load_x<ACT, XF32, EPC>(p.x, in_off, (uint32_t)(sl + c * SEG) * EPC, xr[t][c]);
-            float s = 0.0f;
-#pragma unroll
-            for (int j = 0; j < EPC; ++j) {
-                if (!live) xr[t][c][j] = 0.0f;
-                s += xr[t][c][j];
-            }
-            xs[t][c] = s;
-        }
-    }
-
     const uint8_t* WA = blob + p.wA;
     const uint16_t* SA = reinterpret_cast<const uint16_t*>(blob + p.sA);
     const uint16_t* BA = reinterpret_cast<const uint16_t*>(blob + p.bA);
     const uint8_t* WB = DUAL ? blob + p.wB : nullptr;
     const uint16_t* SB = DUAL ? reinterpret_cast<const uint16_t*>(blob + p.sB) : nullptr;
     const uint16_t* BB = DUAL ? reinterpret_cast<const uint16_t*>(blob + p.bB) : nullptr;
-
     const uint32_t row_base = (rb * 4 + wave) * ROWS_WAVE;
-#pragma unroll 1
-    for (int it = 0; it < ITERS; ++it) {
-        uint4 qa[RPI][NCH], qb[RPI][NCH];
-        uint16_t sa[RPI][NCH], ba[RPI][NCH], sb[RPI][NCH], bb[RPI][NCH];
-        uint32_t rows_i[RPI];
-        // issue every load of this iteration before the first use
+    uint4* xw = lds;
+    float* xs_tab = reinterpret_cast<float*>(lds + MAX_TOK * WORDS_TOK);
+    float* wmax_tab = xs_tab + MAX_TOK * NCH * SEG;
+    float* isc_tab = wmax_tab + MAX_TOK * 4;
+
+    auto load_stage = [&](Stage& st, int it) {
 #pragma unroll
         for (int i = 0; i < RPI; ++i) {
             const uint32_t row = row_base + (it * RPI + i) * RPL + seg_id;
-            rows_i[i] = row;
             const uint32_t r = row < p.rows ? row : p.rows - 1;
 #pragma unroll
             for (int c = 0; c < NCH; ++c) {
                 const uint32_t chunk = sl + c * SEG;
                 const uint32_t g = chunk * EPC / NVMAI_GROUP;
-                qa[i][c] = *reinterpret_cast<const uint4*>(WA + (size_t)r * row_bytes + chunk * 16);
-                sa[i][c] = SA[(size_t)r * groups + g];
-                ba[i][c] = BA[(size_t)r * groups + g];
+                st.qa[i][c] = *reinterpret_cast<const uint4*>(WA + (size_t)r * row_bytes + chunk * 16);
+                st.sa[i][c] = SA[(size_t)r * groups + g];
+                st.ba[i][c] = BA[(size_t)r * groups + g];
                 if (DUAL) {
-                    qb[i][c] = *reinterpret_cast<const uint4*>(WB + (size_t)r * row_bytes + chunk * 16);
-                    sb[i][c] = SB[(size_t)r * groups + g];
-                    bb[i][c] = BB[(size_t)r * groups + g];
+                    st.qb[i][c] = *reinterpret_cast<const uint4*>(WB + (size_t)r * row_bytes + chunk * 16);
+                    st.sb[i][c] = SB[(size_t)r * groups + g];
+                    st.bb[i][c] = BB[(size_t)r * groups + g];
                 }
             }
         }
+    };
+
+    Stage s0, s1;
+    load_stage(s0, 0);                            // both in flight while the inputs are staged
+    load_stage(s1, 1);
+
+    // ---- pass 1: largest magnitude of every input row
+#pragma unroll 1
+    for (int t = 0; t < ntok; ++t) {
+        const size_t in_off = (size_t)p.pair_in[we.pair_start + t] * p.x_stride;
+        float m = 0.0f;
+        for (uint32_t e0 = threadIdx.x * 8; e0 < p.n; e0 += 256 * 8) {
+            float v[8];
+            load8<ACT, XF32>(p.x, in_off + e0, v);
 #pragma unroll
-        for (int i = 0; i < RPI; ++i) {
-            float accA[TOK], accB[TOK];
+            for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[j]));
+        }
+        m = wave_max_f32(m);
+        if (lane == 0) wmax_tab[t * 4 + wave] = m;
+    }
+    __syncthreads();
+    // ---- pass 2: scale, convert, pack
+#pragma unroll 1
+    for (int t = 0; t < ntok; ++t) {
+        const size_t in_off = (size_t)p.pair_in[we.pair_start + t] * p.x_stride;
+        const float amax = fmaxf(fmaxf(wmax_tab[t * 4], wmax_tab[t * 4 + 1]),
+                                 fmaxf(wmax_tab[t * 4 + 2], wmax_tab[t * 4 + 3]));
+        float sc, isc;
+        pow2_scale(amax, sc, isc);
+        if (threadIdx.x == 0) isc_tab[t] = isc;
+        for (uint32_t e0 = threadIdx.x * 8; e0 < p.n; e0 += 256 * 8) {
+            float v[8];
+            load8<ACT, XF32>(p.x, in_off + e0, v);
 #pragma unroll
-            for (int t = 0; t < TOK; ++t) { accA[t] = 0.0f; accB[t] = 0.0f; }
-#pragma unroll
-            for (int c = 0; c < NCH; ++c) {
-                float q[EPC];
-                unpack_chunk<BITS>(qa[i][c], q);
-                const float s = bf16_to_f32(sa[i][c]), b = bf16_to_f32(ba[i][c]);
-#pragma unroll
-                for (int t = 0; t < TOK; ++t) {
-                    float dot = 0.0f;
-#pragma unroll
-                    for (int j = 0; j < EPC; ++j) dot = fmaf(q[j], xr[t][c][j], dot);
-                    accA[t] = fmaf(s, dot, accA[t]);
-                    accA[t] = fmaf(b, xs[t][c], accA[t]);
-                }
-                if (DUAL) {
-                    unpack_chunk<BITS>(qb[i][c], q);
-                    const float s2 = bf16_to_f32(sb[i][c]), b2 = bf16_to_f32(bb[i][c]);
-#pragma unroll
-                    for (int t = 0; t < TOK; ++t) {
-                        float dot = 0.0f;
-#pragma unroll
-                        for (int j = 0; j < EPC; ++j) dot = fmaf(q[j], xr[t][c][j], dot);
-                        accB[t] = fmaf(s2, dot, accB[t]);
-                        accB[t] = fmaf(b2, xs[t][c], accB[t]);
-                    }
-                }
-            }
-            const bool writer = seg_result_lane<SEG>(lane) && rows_i[i] < p.rows;
-#pragma unroll
-            for (int t = 0; t < TOK; ++t) {
-                float a = seg_reduce_sum<SEG>(accA[t]);
-                float v = a;
-                if (DUAL) {
-                    float u = seg_reduce_sum<SEG>(accB[t]);
-                    v = silu(a) * u;      // moe.metal:134-139 (silu branch), CPUExpertFFN.swift:122-124
-                }
-                if (writer && (uint32_t)t < we.pair_count)
-                    p.out[(size_t)out_row[t] * p.out_stride + rows_i[i]] = v;
-            }
+            for (int j = 0; j < 8; ++j) v[j] *= sc;
+            const uint32_t chunk = e0 / EPC, piece = (e0 % EPC) / 8;
+            xw[t * WORDS_TOK + ((chunk / SEG) * H + piece) * SEG + (chunk % SEG)] = pack_inputs<BITS>(v);
         }
     }
+    __syncthreads();
+    // ---- chunk sums of the converted inputs, one thread per (input, chunk)
+    for (int idx = threadIdx.x; idx < ntok * NCH * SEG; idx += 256) {
+        const int t = idx / (NCH * SEG), cs = idx % (NCH * SEG), c = cs / SEG, l = cs % SEG;
+        float sum = 0.0f;
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            const uint4 w = xw[t * WORDS_TOK + (c * H + h) * SEG + l];
+            const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                sum += f16_to_f32((uint16_t)(ws[d] & 0xFFFFu));
+                sum += f16_to_f32((uint16_t)(ws[d] >> 16));
+            }
+        }
+        xs_tab[t * NCH * SEG + c * SEG + l] = sum;
+    }
+    __syncthreads();
+
+    auto compute_stage = [&](const Stage& st, int it) {
+        uint32_t qpa[RPI][NCH][PAIRS], qpb[DUAL ? RPI : 1][NCH][PAIRS];
+#pragma unroll
+        for (int i = 0; i < RPI; ++i)
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                unpack_pairs<BITS>(st.qa[i][c], qpa[i][c]);
+                if (DUAL) unpack_pairs<BITS>(st.qb[i][c], qpb[i][c]);
+            }
+#pragma unroll 1
+        for (int t = 0; t < ntok; ++t) {
+            uint32_t xp[NCH][PAIRS];
+            float xs[NCH];
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+#pragma unroll
+                for (int h = 0; h < H; ++h) {
+                    const uint4 w = xw[t * WORDS_TOK + (c * H + h) * SEG + sl];
+                    xp[c][4 * h] = w.x; xp[c][4 * h + 1] = w.y; xp[c][4 * h + 2] = w.z; xp[c][4 * h + 3] = w.w;
+                }
+                xs[c] = xs_tab[t * NCH * SEG + c * SEG + sl];
+            }
+            const float isc = isc_tab[t];
+            const uint32_t out_row = p.pair_out[we.pair_start + t];
+#pragma unroll
+            for (int i = 0; i < RPI; ++i) {
+                const uint32_t row = row_base + (it * RPI + i) * RPL + seg_id;
+                float accA = 0.0f, accB = 0.0f;
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+                    float dotA = 0.0f, dotB = 0.0f;
+#pragma unroll
+                    for (int m = 0; m < PAIRS; ++m) {
+                        dotA = dot2_acc(qpa[i][c][m], xp[c][m], dotA);
+                        if (DUAL) dotB = dot2_acc(qpb[i][c][m], xp[c][m], dotB);
+                    }
+                    dotA = fmaf(-1024.0f, xs[c], dotA);
+                    accA = fmaf(bf16_to_f32(st.sa[i][c]), dotA, accA);
+                    accA = fmaf(bf16_to_f32(st.ba[i][c]), xs[c], accA);
+                    if (DUAL) {
+                        dotB = fmaf(-1024.0f, xs[c], dotB);
+                        accB = fmaf(bf16_to_f32(st.sb[i][c]), dotB, accB);
+                        accB = fmaf(bf16_to_f32(st.bb[i][c]), xs[c], accB);
+                    }
+                }
+                const float a = seg_reduce_sum<SEG>(accA) * isc;
+                float v = a;
+                if (DUAL) {
+                    const float u = seg_reduce_sum<SEG>(accB) * isc;
+                    v = silu_fast(a) * u; // moe.metal:134-139 (silu branch), CPUExpertFFN.swift:122-124
+                }
+                if (seg_result_lane<SEG>(lane) && row < p.rows)
+                    p.out[(size_t)out_row * p.out_stride + row] = v;
+            }
+        }
+    };
+
+#pragma unroll 1
+    for (int it = 0; it < ITERS; it += 2) {
+        compute_stage(s0, it);
+        if (it + 2 < ITERS) load_stage(s0, it + 2);
+        compute_stage(s1, it + 1);
+        if (it + 3 < ITERS) load_stage(s1, it + 3);
+    }
+}
+
+// Bytes of dynamic LDS the fast engine needs for rows of n codes.
+__host__ __device__ inline size_t rows_fast_lds_bytes(uint32_t n, int nch, int seg) {
+    return (size_t)MAX_TOK * (n / 8) * 16 + (size_t)MAX_TOK * nch * seg * 4 + MAX_TOK * 4 * 4 + MAX_TOK * 4;
 }
 
 // MAXTOK = 1: single-input launches.  MAXTOK = 4: the body is chosen by the
 // entry's pair count (uniform per block), so an expert routed to by one token
-// does not pay for four.
+// does not pay for more.
 template <int ACT, int BITS, int SEG, int NCH, int MAXTOK, bool DUAL, bool XF32, int RPI, int ITERS>
 __global__ __launch_bounds__(256) void expert_rows_fast(RowsParams p) {
+    extern __shared__ uint4 rows_lds[];
     const uint32_t entry = blockIdx.x / p.blocks_per_entry;
     if (entry >= *p.n_entries) return;
     const uint32_t rb = blockIdx.x % p.blocks_per_entry;
     const WorkEntry we = p.entries[entry];
     if (MAXTOK == 1 || we.pair_count == 1)
-        expert_rows_body<ACT, BITS, SEG, NCH, 1, DUAL, XF32, RPI, ITERS>(p, we, rb);
-    else if (we.pair_count == 2)
-        expert_rows_body<ACT, BITS, SEG, NCH, 2, DUAL, XF32, RPI, ITERS>(p, we, rb);
+        expert_rows_body<ACT, BITS, SEG, NCH, 1, DUAL, XF32, RPI, ITERS>(p, we, rb, rows_lds);
     else
-        expert_rows_body<ACT, BITS, SEG, NCH, 4, DUAL, XF32, RPI, ITERS>(p, we, rb);
+        expert_rows_body<ACT, BITS, SEG, NCH, 0, DUAL, XF32, RPI, ITERS>(p, we, rb, rows_lds);
 }
 
 // ---- generic engine -----------------------------------------------------------
@@ -301,78 +447,143 @@ struct RouterParams {
     RowsDesc router;
     RowsDesc gate;                 // optional single row appended after the experts
     const void* x;                 // [tokens, x_stride] activations
+    int x_vec;                     // rows of x (and eff_scale) are 16-byte aligned
     const uint16_t* eff_scale;     // optional bf16 [d]
     uint32_t x_stride, tokens, num_experts, d;
     float* logits;                 // [tokens, num_experts]
     float* gate_logit;             // [tokens]
 };
 
-template <int ACT>
-__device__ __forceinline__ float router_x(const RouterParams& p, size_t row_off, uint32_t e) {
-    float v = act_to_f32<ACT>(((const uint16_t*)p.x)[row_off + e]);
-    if (p.eff_scale) v = __fmul_rn(v, bf16_to_f32(p.eff_scale[e]));
-    return v;
+constexpr int ROUTER_TOK = 4;   // tokens per block in y
+
+// EPC consecutive activations of one row as floats, optionally times the bf16
+// effective scale (one rounding, as moe.metal:200-201 multiplies before use).
+template <int ACT, int EPC>
+__device__ __forceinline__ void router_x_from_raw(const RouterParams& p, const uint4* raw, uint32_t e0, float* xv) {
+#pragma unroll
+    for (int i = 0; i < EPC / 8; ++i) {
+        act2_to_f32<ACT>(raw[i].x, xv[8 * i], xv[8 * i + 1]);
+        act2_to_f32<ACT>(raw[i].y, xv[8 * i + 2], xv[8 * i + 3]);
+        act2_to_f32<ACT>(raw[i].z, xv[8 * i + 4], xv[8 * i + 5]);
+        act2_to_f32<ACT>(raw[i].w, xv[8 * i + 6], xv[8 * i + 7]);
+    }
+    if (p.eff_scale) {
+#pragma unroll
+        for (int j = 0; j < EPC; ++j) xv[j] = __fmul_rn(xv[j], bf16_to_f32(p.eff_scale[e0 + j]));
+    }
 }
 
-template <int ACT>
-__device__ float router_row_dot(const RouterParams& p, const RowsDesc& r, uint32_t row,
-                                size_t x_off, int hl) {
-    float acc = 0.0f;
-    if (r.kind == 16) {
-        const uint32_t chunks = p.d / 8;
-        const uint16_t* wr = (const uint16_t*)r.w + (size_t)row * p.d;
-        for (uint32_t c = hl; c < chunks; c += 32) {
-            uint4 raw = *reinterpret_cast<const uint4*>(wr + c * 8);
-            const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+template <int ACT, int EPC>
+__device__ __forceinline__ void router_load_raw(const RouterParams& p, size_t x_off, uint32_t e0, uint4* raw) {
+    if (p.x_vec) {
+        const uint4* px = reinterpret_cast<const uint4*>((const uint16_t*)p.x + x_off + e0);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                acc = fmaf(__uint_as_float(words[j] << 16), router_x<ACT>(p, x_off, c * 8 + 2 * j), acc);
-                acc = fmaf(__uint_as_float(words[j] & 0xFFFF0000u), router_x<ACT>(p, x_off, c * 8 + 2 * j + 1), acc);
-            }
+        for (int i = 0; i < EPC / 8; ++i) raw[i] = px[i];
+    } else {                       // unaligned rows (e.g. a padded hidden stride): element loads
+        const uint16_t* px = (const uint16_t*)p.x + x_off + e0;
+#pragma unroll
+        for (int i = 0; i < EPC / 8; ++i) {
+            raw[i].x = px[8 * i] | ((uint32_t)px[8 * i + 1] << 16);
+            raw[i].y = px[8 * i + 2] | ((uint32_t)px[8 * i + 3] << 16);
+            raw[i].z = px[8 * i + 4] | ((uint32_t)px[8 * i + 5] << 16);
+            raw[i].w = px[8 * i + 6] | ((uint32_t)px[8 * i + 7] << 16);
         }
-    } else {
-        const int epc = r.kind == 8 ? 16 : 32;
-        const uint32_t chunks = p.d / epc;
-        const uint32_t groups = p.d / NVMAI_GROUP;
-        const uint8_t* wr = (const uint8_t*)r.w + (size_t)row * (p.d * r.kind / 8);
-        for (uint32_t c = hl; c < chunks; c += 32) {
-            const uint4 raw = *reinterpret_cast<const uint4*>(wr + c * 16);
-            const uint32_t g = c * epc / NVMAI_GROUP;
-            const float s = bf16_to_f32(r.s[(size_t)row * groups + g]);
-            const float b = bf16_to_f32(r.b[(size_t)row * groups + g]);
-            float q[32];
-            if (r.kind == 8) unpack_chunk<8>(raw, q); else unpack_chunk<4>(raw, q);
-            float dot = 0.0f, xs = 0.0f;
-            for (int j = 0; j < epc; ++j) {
-                const float xv = router_x<ACT>(p, x_off, c * epc + j);
-                dot = fmaf(q[j], xv, dot);
-                xs = __fadd_rn(xs, xv);
+    }
+}
+
+// One row against up to ROUTER_TOK tokens; hl = lane in the half-wave, CPL =
+// chunks per lane (compile time) so that every load is issued before the first
+// use: a dependent round trip to HBM costs more than the whole arithmetic.
+// Per token the lane accumulates over its chunks in ascending order.
+template <int ACT, int KIND, int CPL>
+__device__ __forceinline__ void router_row_dots(const RouterParams& p, const RowsDesc& r, uint32_t row,
+                                                uint32_t t0, uint32_t nt, int hl, float* acc) {
+    constexpr int EPC = KIND == 16 ? 8 : (KIND == 8 ? 16 : 32);
+    constexpr int XV = EPC / 8;
+    const uint32_t chunks = p.d / EPC;
+    const uint32_t groups = p.d / NVMAI_GROUP;
+    const uint8_t* wr = (const uint8_t*)r.w + (size_t)row * ((size_t)p.d * KIND / 8);
+    uint4 wraw[CPL], xraw[ROUTER_TOK][CPL][XV];
+    uint16_t sraw[CPL], braw[CPL];
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) {
+        const uint32_t c = hl + 32 * i;
+        if (c < chunks) {
+            wraw[i] = *reinterpret_cast<const uint4*>(wr + (size_t)c * 16);
+            if (KIND != 16) {
+                const uint32_t g = c * EPC / NVMAI_GROUP;
+                sraw[i] = r.s[(size_t)row * groups + g];
+                braw[i] = r.b[(size_t)row * groups + g];
             }
-            acc = fmaf(s, dot, acc);
-            acc = fmaf(b, xs, acc);
+#pragma unroll
+            for (int t = 0; t < ROUTER_TOK; ++t)
+                if ((uint32_t)t < nt) router_load_raw<ACT, EPC>(p, (size_t)(t0 + t) * p.x_stride, c * EPC, xraw[t][i]);
         }
     }
 #pragma unroll
-    for (int off = 16; off >= 1; off >>= 1) acc = __fadd_rn(acc, shfl_xor_f(acc, off));
-    return acc;
+    for (int t = 0; t < ROUTER_TOK; ++t) acc[t] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) {
+        const uint32_t c = hl + 32 * i;
+        if (c >= chunks) break;
+        float q[EPC];
+        if (KIND == 16) {
+            act2_to_f32<ACT_BF16>(wraw[i].x, q[0], q[1]); act2_to_f32<ACT_BF16>(wraw[i].y, q[2], q[3]);
+            act2_to_f32<ACT_BF16>(wraw[i].z, q[4], q[5]); act2_to_f32<ACT_BF16>(wraw[i].w, q[6], q[7]);
+        } else {
+            unpack_chunk<KIND == 16 ? 8 : KIND>(wraw[i], q);
+        }
+#pragma unroll
+        for (int t = 0; t < ROUTER_TOK; ++t) {
+            if ((uint32_t)t >= nt) break;
+            float xv[EPC];
+            router_x_from_raw<ACT, EPC>(p, xraw[t][i], c * EPC, xv);
+            if (KIND == 16) {
+#pragma unroll
+                for (int j = 0; j < EPC; ++j) acc[t] = fmaf(q[j], xv[j], acc[t]);
+            } else {
+                float dot = 0.0f, xs = 0.0f;
+#pragma unroll
+                for (int j = 0; j < EPC; ++j) {
+                    dot = fmaf(q[j], xv[j], dot);
+                    xs = __fadd_rn(xs, xv[j]);
+                }
+                acc[t] = fmaf(bf16_to_f32(sraw[i]), dot, acc[t]);
+                acc[t] = fmaf(bf16_to_f32(braw[i]), xs, acc[t]);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < ROUTER_TOK; ++t)
+#pragma unroll
+        for (int off = 16; off >= 1; off >>= 1) acc[t] = __fadd_rn(acc[t], shfl_xor_f(acc[t], off));
 }
 
-constexpr int ROUTER_TOK = 4;   // tokens per block in y
+template <int ACT, int CPL>
+__device__ __forceinline__ void router_row_any(const RouterParams& p, const RowsDesc& r, uint32_t row,
+                                               uint32_t t0, uint32_t nt, int hl, float* acc) {
+    if (r.kind == 16) router_row_dots<ACT, 16, CPL>(p, r, row, t0, nt, hl, acc);
+    else if (r.kind == 8) router_row_dots<ACT, 8, CPL>(p, r, row, t0, nt, hl, acc);
+    else router_row_dots<ACT, 4, CPL>(p, r, row, t0, nt, hl, acc);
+}
 
-template <int ACT>
+// Largest chunk count per lane over the router and gate rows must be <= CPL.
+template <int ACT, int CPL>
 __global__ __launch_bounds__(256) void router_logits_kernel(RouterParams p) {
     const int hw = threadIdx.x >> 5, hl = threadIdx.x & 31;
     const uint32_t row = blockIdx.x * 8 + hw;
     const uint32_t total_rows = p.num_experts + (p.gate.kind ? 1u : 0u);
     if (row >= total_rows) return;                   // uniform per half-wave
     const bool is_gate = row >= p.num_experts;
-    for (uint32_t t = blockIdx.y * ROUTER_TOK; t < min(p.tokens, (blockIdx.y + 1) * ROUTER_TOK); ++t) {
-        const size_t x_off = (size_t)t * p.x_stride;
-        float v = is_gate ? router_row_dot<ACT>(p, p.gate, 0, x_off, hl)
-                          : router_row_dot<ACT>(p, p.router, row, x_off, hl);
-        if (hl == 0) {
-            if (is_gate) p.gate_logit[t] = v;
-            else p.logits[(size_t)t * p.num_experts + row] = v;
+    const uint32_t t0 = blockIdx.y * ROUTER_TOK;
+    const uint32_t nt = min((uint32_t)ROUTER_TOK, p.tokens - t0);
+    float acc[ROUTER_TOK];
+    if (is_gate) router_row_any<ACT, CPL>(p, p.gate, 0, t0, nt, hl, acc);
+    else router_row_any<ACT, CPL>(p, p.router, row, t0, nt, hl, acc);
+    if (hl == 0) {
+        for (uint32_t t = 0; t < nt; ++t) {
+            if (is_gate) p.gate_logit[t0 + t] = acc[t];
+            else p.logits[(size_t)(t0 + t) * p.num_experts + row] = acc[t];
         }
     }
 }
@@ -414,12 +625,10 @@ __device__ void select_topk_wave(const SelectParams& p, uint32_t t, int lane) {
             const uint32_t e = lane + 64 * j;
             if (!taken[j] && (bi == 0xFFFFFFFFu || better(val[j], e, bv, bi))) { bv = val[j]; bi = e; }
         }
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            const float ov = shfl_xor_f(bv, off);
-            const uint32_t oi = shfl_xor_u(bi, off);
-            if (oi != 0xFFFFFFFFu && (bi == 0xFFFFFFFFu || better(ov, oi, bv, bi))) { bv = ov; bi = oi; }
-        }
+        // wave argmax: highest value, lowest index among equals
+        const float wm = wave_max_f32(bi == 0xFFFFFFFFu ? -INFINITY : bv);
+        bi = wave_min_u32((bi != 0xFFFFFFFFu && bv == wm) ? bi : 0xFFFFFFFFu);
+        bv = wm;
         if (bi == 0xFFFFFFFFu) { bi = 0; bv = -INFINITY; }   // fewer candidates than k
 #pragma unroll
         for (int j = 0; j < TOPK_MAX_PER_LANE; ++j)
@@ -444,92 +653,95 @@ __global__ __launch_bounds__(256) void select_topk_kernel(SelectParams p) {
 }
 
 // ---- decode work list --------------------------------------------------------------
-// Groups the (token, slot) pairs of a small decode batch by expert so that each
-// distinct expert is streamed once, and appends the shared expert over all
-// tokens.  One block; thread e owns expert e.  Pair order inside an expert is
-// (token, slot) ascending, which makes the result deterministic.
+// Top-k for every token of a small decode batch (one wave per token, four per
+// block), then the block that finishes last groups the (token, slot) pairs by
+// expert so that each distinct expert is streamed once, and appends the shared
+// expert over all tokens.  Entries are ordered heaviest first (shared expert, then
+// routed entries by pair count 4, 3, 2, 1) so that the long blocks start early.
+// The order of pairs and entries inside a class comes from LDS atomics and may
+// differ between runs; every pair's arithmetic is independent of it, so the
+// results do not.
 struct GroupParams {
-    const uint32_t* idx;       // [tokens, top_k]
-    uint32_t tokens, top_k, num_experts;
+    SelectParams sel;
     uint32_t tok_per_entry;    // 1..MAX_TOK
     int has_shared;
     WorkEntry* entries;
     uint32_t* n_entries;       // [0] = entries, [1] = distinct experts
+    uint32_t* stats;           // optional copy of n_entries[0..1]
     uint32_t* pair_token;      // input row per pair for phase 1
     uint32_t* pair_id;         // act / partial row per pair
+    uint32_t* ticket;          // zero between launches; counts finished blocks
 };
 
-__global__ __launch_bounds__(1024) void group_decode_kernel(GroupParams p) {
+__global__ __launch_bounds__(256) void select_group_kernel(GroupParams p) {
     extern __shared__ uint32_t lds[];
-    uint32_t* s_idx = lds;                                // tokens*top_k
-    uint32_t* s_scan = lds + p.tokens * p.top_k;          // 2 * blockDim
-    const uint32_t tid = threadIdx.x, n_pairs = p.tokens * p.top_k;
-    for (uint32_t i = tid; i < n_pairs; i += blockDim.x) s_idx[i] = p.idx[i];
-    __syncthreads();
-    uint32_t cnt = 0;
-    if (tid < p.num_experts)
-        for (uint32_t i = 0; i < n_pairs; ++i) cnt += (s_idx[i] == tid);
-    const uint32_t ent = (cnt + p.tok_per_entry - 1) / p.tok_per_entry;
-    // inclusive scans of pair counts and entry counts (Hillis-Steele in LDS)
-    uint32_t* sc_pairs = s_scan;
-    uint32_t* sc_ent = s_scan + blockDim.x;
-    sc_pairs[tid] = cnt;
-    sc_ent[tid] = ent;
-    __syncthreads();
-    for (uint32_t off = 1; off < blockDim.x; off <<= 1) {
-        uint32_t a = 0, b = 0;
-        if (tid >= off) { a = sc_pairs[tid - off]; b = sc_ent[tid - off]; }
-        __syncthreads();
-        sc_pairs[tid] += a;
-        sc_ent[tid] += b;
-        __syncthreads();
+    const uint32_t tokens = p.sel.tokens, top_k = p.sel.top_k, E = p.sel.num_experts;
+    const uint32_t n_pairs = tokens * top_k;
+    const uint32_t tid = threadIdx.x;
+    {
+        const uint32_t t = blockIdx.x * 4 + (tid >> 6);
+        if (t < tokens) select_topk_wave(p.sel, t, tid & 63);
     }
-    const uint32_t pair_start = sc_pairs[tid] - cnt, ent_start = sc_ent[tid] - ent;
-    const uint32_t total_ent = sc_ent[blockDim.x - 1];
-    if (cnt) {
-        uint32_t k = 0;
-        for (uint32_t i = 0; i < n_pairs; ++i) {
-            if (s_idx[i] != tid) continue;
-            if (k % p.tok_per_entry == 0) {
-                WorkEntry we;
-                we.expert = tid;
-                we.pair_start = pair_start + k;
-                we.pair_count = min(p.tok_per_entry, cnt - k);
-                we.reserved = 0;
-                p.entries[ent_start + k / p.tok_per_entry] = we;
-            }
-            p.pair_token[pair_start + k] = i / p.top_k;
-            p.pair_id[pair_start + k] = i;
-            ++k;
-        }
-    }
-    // distinct experts = number of threads with cnt > 0
+    __threadfence();                      // this block's indices are visible device-wide
     __syncthreads();
-    sc_pairs[tid] = cnt ? 1u : 0u;
+    if (tid == 0) lds[0] = atomicAdd(p.ticket, 1u);
     __syncthreads();
-    for (uint32_t off = blockDim.x / 2; off > 0; off >>= 1) {
-        if (tid < off) sc_pairs[tid] += sc_pairs[tid + off];
-        __syncthreads();
+    if (lds[0] != gridDim.x - 1) return;  // uniform per block
+    __syncthreads();
+
+    uint32_t* cnt = lds;                  // [E] pairs per expert
+    uint32_t* start = lds + E;            // [E] first pair of the expert
+    uint32_t* slotf = lds + 2 * E;        // [E] first full entry of the expert inside its class
+    uint32_t* slotr = lds + 3 * E;        // [E] remainder entry of the expert inside its class
+    uint32_t* misc = lds + 4 * E;         // [0] pair cursor, [1..4] entries per class, [5] distinct
+    uint32_t* rank = lds + 4 * E + 8;     // [n_pairs] rank of the pair inside its expert
+    const volatile uint32_t* idx = p.sel.out_idx;   // written by other blocks: read past L1
+    for (uint32_t i = tid; i < 4 * E + 8; i += 256) lds[i] = 0;
+    __syncthreads();
+    for (uint32_t i = tid; i < n_pairs; i += 256) rank[i] = atomicAdd(&cnt[idx[i]], 1u);
+    __syncthreads();
+    const uint32_t tpe = p.tok_per_entry;
+    for (uint32_t e = tid; e < E; e += 256) {
+        const uint32_t c = cnt[e];
+        if (!c) continue;
+        start[e] = atomicAdd(&misc[0], c);
+        atomicAdd(&misc[5], 1u);
+        const uint32_t full = c / tpe, rem = c % tpe;
+        if (full) slotf[e] = atomicAdd(&misc[tpe], full);
+        if (rem) slotr[e] = atomicAdd(&misc[rem], 1u);
     }
-    uint32_t shared_ent = 0;
+    __syncthreads();
+    const uint32_t shared_ent = p.has_shared ? (tokens + tpe - 1) / tpe : 0;
+    uint32_t base[MAX_TOK + 1];
+    uint32_t run = shared_ent;
+    for (int c = MAX_TOK; c >= 1; --c) { base[c] = run; run += misc[c]; }
+    const uint32_t total_ent = run;
+    for (uint32_t e = tid; e < E; e += 256) {
+        const uint32_t c = cnt[e];
+        if (!c) continue;
+        const uint32_t full = c / tpe, rem = c % tpe;
+        for (uint32_t j = 0; j < full; ++j)
+            p.entries[base[tpe] + slotf[e] + j] = WorkEntry{e, start[e] + j * tpe, tpe, 0};
+        if (rem) p.entries[base[rem] + slotr[e]] = WorkEntry{e, start[e] + full * tpe, rem, 0};
+    }
+    for (uint32_t i = tid; i < n_pairs; i += 256) {
+        const uint32_t pos = start[idx[i]] + rank[i];
+        p.pair_token[pos] = i / top_k;
+        p.pair_id[pos] = i;
+    }
     if (p.has_shared) {
-        shared_ent = (p.tokens + p.tok_per_entry - 1) / p.tok_per_entry;
-        for (uint32_t j = tid; j < shared_ent; j += blockDim.x) {
-            WorkEntry we;
-            we.expert = NVMAI_SLOT_FLAG | 8u;
-            we.pair_start = n_pairs + j * p.tok_per_entry;
-            we.pair_count = min(p.tok_per_entry, p.tokens - j * p.tok_per_entry);
-            we.reserved = 0;
-            p.entries[total_ent + j] = we;
-        }
-        for (uint32_t t = tid; t < p.tokens; t += blockDim.x) {
+        for (uint32_t j = tid; j < shared_ent; j += 256)
+            p.entries[j] = WorkEntry{NVMAI_SLOT_FLAG | 8u, n_pairs + j * tpe, min(tpe, tokens - j * tpe), 0};
+        for (uint32_t t = tid; t < tokens; t += 256) {
             p.pair_token[n_pairs + t] = t;
             p.pair_id[n_pairs + t] = n_pairs + t;
         }
     }
     if (tid == 0) {
-        p.n_entries[0] = total_ent + shared_ent;
-        p.n_entries[1] = sc_pairs[0];
+        p.n_entries[0] = total_ent;
+        p.n_entries[1] = misc[5];
+        if (p.stats) { p.stats[0] = total_ent; p.stats[1] = misc[5]; }
+        *p.ticket = 0;                    // ready for the next launch
     }
 }
 

@@ -157,6 +157,27 @@ def test_router_indices_and_logits_bit_exact(nv, ctx, kind):
     _router_case(nv, ctx, kind, 16, 128, 4, 8, rng, eff, pes)
 
 
+def test_router_padded_hidden_stride(nv, ctx_bf16):
+    # PrefillRouterTests.swift:33-95: rows of `hidden` are d + 13 apart and the padding is left alone
+    say("router padded stride")
+    E, D, T, k = 16, 128, 3, 8
+    rng = np.random.default_rng(77)
+    stride = D + 13
+    w = O.round_bf16(gauss(rng, (E, D), 0.04) + np.arange(E, dtype=np.float32)[:, None] * np.float32(0.015))
+    host = O.quantize_affine(w, 8)
+    desc = nv.rows_desc(8, dev(host[0]), dev(host[1].view(np.int16)), dev(host[2].view(np.int16)))
+    block = np.full((T, stride), -31.0, np.float32)
+    block[:, :D] = O.round_bf16(rng.uniform(-1, 1, (T, D)).astype(np.float32))
+    hd = dev(block).to(torch.bfloat16)
+    idx, wt = nv.MoE(ctx_bf16).encode_router(desc, hd[:, :D], E, D, k)
+    torch.cuda.synchronize()
+    for t in range(T):
+        io, wo = O.router_topk(O.router_logits(8, host[0], host[1], host[2], block[t, :D]), k)
+        assert np.array_equal(u32(idx[t]), io)
+        assert np.abs(act_np(wt[t]) - O.f16_to_float(wo)).max() < 5e-3
+    assert np.array_equal(act_np(hd)[:, D:], block[:, D:])
+
+
 def test_router_near_tie_and_exact_ties(nv, ctx_bf16):
     # RouterTopKTests.swift:46-70: gains 0.5 and 0.5*(1+1e-4) must order like the reference
     say("router near tie")
