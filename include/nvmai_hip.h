@@ -185,6 +185,86 @@ int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream stream, const nv
                                uint32_t y_stride, uint32_t* out_idx, uint16_t* out_w,
                                uint32_t* stats);
 
+
+/* ---- KV cache -------------------------------------------------------------------------- */
+
+/* KVCacheManager.rowLayout (KVCacheManager.swift:437-446): bytes per token row and bytes of
+ * packed codes for `elements` = num_kv_heads * head_dim values at `bits` in {4, 8, 16}.
+ * Row = codes | FP16 scales[groups] | FP16 biases[groups], groups of 64.  Host arithmetic. */
+int nvmai_kv_row_layout(uint32_t elements, uint32_t bits, uint32_t* stride, uint32_t* value_bytes);
+
+/* KVView (KVCacheManager.swift:19-31) without the Metal buffer: where a layer's K or V rows
+ * live and how they are encoded. */
+typedef struct {
+    void* base;            /* row of position p at base + p * stride */
+    uint32_t stride;
+    uint32_t value_bytes;
+    uint32_t bits;         /* KVCachePrecision raw value: 4, 8 or 16 (RuntimeConfiguration.swift:81-88) */
+    uint32_t group_size;   /* 64 */
+} nvmai_kv_view;
+
+/* KVCacheQuantizer.encode (KVCacheQuantizer.swift:13-50; kernel kv_cache_quantize.metal:7-73):
+ * quantize token_count rows of element_count activations (row t at source + t *
+ * source_stride elements) into destination rows 0..token_count-1. */
+int nvmai_hip_kv_quantize_affine(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* source,
+                                 uint32_t source_stride, const nvmai_kv_view* destination,
+                                 uint32_t token_count, uint32_t element_count);
+
+/* RoPE.encodeNeoxSubdim (RoPE.swift:48; kernel rope.metal:80-102), in place on
+ * data[tokens, heads, head_dim].  positions: optional device array of one position per token;
+ * NULL = every token at `position` (the reference's single-position call). */
+int nvmai_hip_rope_neox_subdim(nvmai_hip_ctx* ctx, nvmai_stream stream, void* data, uint32_t tokens,
+                               uint32_t heads, uint32_t head_dim, uint32_t rotary_dim,
+                               const uint32_t* positions, uint32_t position, float theta);
+
+/* Attention.encodeFull / encodeSWA (Attention.swift:207-239, 170-205; kernels
+ * attention.metal:163-261, 388-429) with a batch dimension: one query token per sequence,
+ * q and out are [batch, num_q_heads, head_dim] activations, sequence b reads rows
+ * [kv_start, seq_len) of k->base + b * kv_batch_stride (same for v).  scale <= 0 selects
+ * 1/sqrt(head_dim) (Attention.defaultScale).  seq_len == kv_start writes zeros. */
+int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
+                               const nvmai_kv_view* k, const nvmai_kv_view* v,
+                               uint64_t kv_batch_stride, void* out, uint32_t batch,
+                               uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                               uint32_t seq_len, uint32_t kv_start, float scale);
+
+/* Attention.splitGeometry (Attention.swift:148-168): the reference's chunking of a KV range,
+ * reported for callers that size scratch the way it does.  Host arithmetic. */
+int nvmai_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len,
+                                   uint32_t kv_start, int prefer_gqa_swa, uint32_t* effective_length,
+                                   uint32_t* num_chunks, uint32_t* chunk_length,
+                                   uint32_t* partial_threadgroups);
+
+/* ---- logits -> token --------------------------------------------------------------------- */
+
+/* LogitSoftcapSoftmaxTiled.encode (LogitOutput.swift:90-141; kernels logit.metal:155-257):
+ * probs[r, :] = softmax(softcap(logits[r, :])) as FP16 for `rows` rows of v activations.
+ * softcap <= 0 disables the cap. */
+int nvmai_hip_softmax_tiled(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* logits,
+                            uint32_t logits_stride, uint16_t* probs, uint32_t probs_stride,
+                            uint32_t rows, uint32_t v, float softcap);
+
+/* SampleTopK64.encode (LogitOutput.swift:267-333; kernels logit.metal:628-758): one token per
+ * row from the top `top_k` (1..64) of FP16 probs with top-p and temperature (> 0); seeds is a
+ * HOST array of one xorshift64* seed per row (rows <= 32).  top64_out (optional, device):
+ * per row the 64 sorted candidates as (float bits, index) u32 pairs. */
+int nvmai_hip_sample_topk64(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint16_t* probs,
+                            uint32_t probs_stride, uint32_t rows, uint32_t v, float temperature,
+                            float top_p, const uint64_t* seeds, uint32_t top_k, uint32_t* out_token,
+                            uint32_t* top64_out);
+
+/* Sample.encode (LogitOutput.swift:157-199; kernel logit.metal:315-585): temperature <= 0 is
+ * greedy argmax (lowest index wins ties); otherwise top_k (0 = none, capped at 256) argmax
+ * passes and the same top-p / temperature / inverse-CDF draw.  The Gumbel shortcut the
+ * reference takes when neither top-k nor top-p is set is not built: that case runs the
+ * truncating path with k = 256, which the reference reaches with top_k = 256. */
+int nvmai_hip_sample(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint16_t* probs,
+                     uint32_t probs_stride, uint32_t rows, uint32_t v, float temperature,
+                     uint32_t top_k, float top_p, const uint64_t* seeds, uint32_t* out_token);
+
+/* Sampler.seedFor (Sampler.swift:304-325): splitmix64(seed + position), 0 mapped away. */
+uint64_t nvmai_sampler_seed_for(uint64_t seed, int64_t position);
+
 #ifdef __cplusplus
 }
 #endif

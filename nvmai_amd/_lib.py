@@ -45,6 +45,11 @@ class MoeLayer(C.Structure):
                 ("eff_scale", vp), ("per_expert_scale", vp)]
 
 
+class KvView(C.Structure):
+    """nvmai_kv_view"""
+    _fields_ = [("base", vp), ("stride", u32), ("value_bytes", u32), ("bits", u32), ("group_size", u32)]
+
+
 # name -> argtypes (every function returns int unless listed in _OTHER)
 SIGNATURES = {
     "nvmai_hip_ctx_create": [C.c_int, C.c_int, C.POINTER(vp)],
@@ -65,10 +70,21 @@ SIGNATURES = {
     "nvmai_hip_shared_expert": [vp, vp, vp, C.POINTER(ExpertOffsets), u32, C.POINTER(Rows), vp,
                                 u32, u32, vp, u32, u32, u32],
     "nvmai_hip_moe_decode_layer": [vp, vp, C.POINTER(MoeLayer), vp, u32, u32, vp, u32, vp, vp, vp],
+    "nvmai_kv_row_layout": [u32, u32, C.POINTER(u32), C.POINTER(u32)],
+    "nvmai_hip_kv_quantize_affine": [vp, vp, vp, u32, C.POINTER(KvView), u32, u32],
+    "nvmai_hip_rope_neox_subdim": [vp, vp, vp, u32, u32, u32, u32, vp, u32, C.c_float],
+    "nvmai_hip_attention_decode": [vp, vp, vp, C.POINTER(KvView), C.POINTER(KvView), u64, vp, u32, u32, u32,
+                                   u32, u32, u32, C.c_float],
+    "nvmai_attention_split_geometry": [u32, u32, u32, u32, C.c_int, C.POINTER(u32), C.POINTER(u32),
+                                       C.POINTER(u32), C.POINTER(u32)],
+    "nvmai_hip_softmax_tiled": [vp, vp, vp, u32, vp, u32, u32, u32, C.c_float],
+    "nvmai_hip_sample_topk64": [vp, vp, vp, u32, u32, u32, C.c_float, C.c_float, C.POINTER(u64), u32, vp, vp],
+    "nvmai_hip_sample": [vp, vp, vp, u32, u32, u32, C.c_float, u32, C.c_float, C.POINTER(u64), vp],
 }
 _OTHER = {
     "nvmai_hip_ctx_destroy": (None, [vp]),
     "nvmai_hip_status_string": (C.c_char_p, [C.c_int]),
+    "nvmai_sampler_seed_for": (u64, [u64, C.c_int64]),
 }
 
 

@@ -1,0 +1,149 @@
+// Entry points: KV row layout, quantize-on-write, partial RoPE, GQA decode attention.
+#include <cmath>
+
+#include "attn_kernels.cuh"
+#include "ctx.hpp"
+
+using namespace nvmai;
+
+extern "C" int nvmai_kv_row_layout(uint32_t elements, uint32_t bits, uint32_t* stride, uint32_t* value_bytes) {
+    if (!stride || !value_bytes || elements == 0) return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8 && bits != 16) return NVMAI_ERR_UNSUPPORTED;
+    if (bits == 16) { *stride = elements * 2; *value_bytes = elements * 2; return NVMAI_OK; }
+    const uint32_t packed = (elements * bits + 7) / 8;
+    const uint32_t aligned = (packed + 1) & ~1u;
+    const uint32_t groups = (elements + 63) / 64;
+    *stride = aligned + groups * 4;
+    *value_bytes = aligned;
+    return NVMAI_OK;
+}
+
+extern "C" int nvmai_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len,
+                                              uint32_t kv_start, int prefer_gqa_swa, uint32_t* effective_length,
+                                              uint32_t* num_chunks, uint32_t* chunk_length,
+                                              uint32_t* partial_threadgroups) {
+    if (!num_kv_heads || num_q_heads % num_kv_heads || !effective_length || !num_chunks || !chunk_length ||
+        !partial_threadgroups)
+        return NVMAI_ERR_INVALID_ARG;
+    const long q_per_kv = num_q_heads / num_kv_heads;
+    const bool use_gqa = prefer_gqa_swa && q_per_kv <= 2;
+    const long eff = (long)seq_len - (long)kv_start, e1 = eff > 1 ? eff : 1;
+    long base = use_gqa ? 8 : 16;                    // Attention.swift:53-54
+    if (e1 < base) base = e1;
+    long nc = base;
+    if (use_gqa) { long alt = base * q_per_kv; if (alt > 64) alt = 64; if (alt > nc) nc = alt; }
+    *effective_length = (uint32_t)eff;
+    *num_chunks = (uint32_t)nc;
+    *chunk_length = (uint32_t)((e1 + nc - 1) / nc);
+    *partial_threadgroups = (uint32_t)((use_gqa ? num_kv_heads : num_q_heads) * nc);
+    return NVMAI_OK;
+}
+
+namespace {
+int check_view(const nvmai_kv_view* v, uint32_t elements) {
+    if (!v || !v->base) return NVMAI_ERR_INVALID_ARG;
+    if (v->bits != 4 && v->bits != 8 && v->bits != 16) return NVMAI_ERR_UNSUPPORTED;
+    if (v->group_size != 64) return NVMAI_ERR_UNSUPPORTED;
+    uint32_t stride = 0, vb = 0;
+    if (nvmai_kv_row_layout(elements, v->bits, &stride, &vb) != NVMAI_OK) return NVMAI_ERR_INVALID_ARG;
+    if (v->value_bytes != vb || v->stride < stride || (v->stride & 1u)) return NVMAI_ERR_INVALID_ARG;
+    return NVMAI_OK;
+}
+}  // namespace
+
+extern "C" int nvmai_hip_kv_quantize_affine(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* source,
+                                            uint32_t source_stride, const nvmai_kv_view* dst,
+                                            uint32_t token_count, uint32_t element_count) {
+    if (!ctx || !source || element_count == 0 || source_stride < element_count) return NVMAI_ERR_INVALID_ARG;
+    int rc = check_view(dst, element_count);
+    if (rc) return rc;
+    if (dst->bits == 16) return NVMAI_ERR_UNSUPPORTED;        // "KV quantizer requires 4-bit or 8-bit destination"
+    if (token_count == 0) return NVMAI_ERR_INVALID_ARG;       // KVCacheQuantizer.swift:22
+    KvFormat f{dst->bits, dst->stride, dst->value_bytes, element_count};
+    const uint64_t waves = (uint64_t)token_count * ((element_count + 63) / 64);
+    dim3 grid((uint32_t)((waves + 3) / 4));
+    ProfScope ps(ctx, NVMAI_PROF_KV_QUANT, (hipStream_t)stream);
+    if (ctx->act == ACT_BF16) kv_quantize_kernel<ACT_BF16><<<grid, 256, 0, (hipStream_t)stream>>>(source, source_stride, (uint8_t*)dst->base, f, token_count);
+    else kv_quantize_kernel<ACT_FP16><<<grid, 256, 0, (hipStream_t)stream>>>(source, source_stride, (uint8_t*)dst->base, f, token_count);
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_rope_neox_subdim(nvmai_hip_ctx* ctx, nvmai_stream stream, void* data, uint32_t tokens,
+                                          uint32_t heads, uint32_t head_dim, uint32_t rotary_dim,
+                                          const uint32_t* positions, uint32_t position, float theta) {
+    if (!ctx || !data || rotary_dim > head_dim || (rotary_dim & 1u) || heads == 0 || head_dim == 0)
+        return NVMAI_ERR_INVALID_ARG;
+    const uint64_t n = (uint64_t)tokens * heads * (rotary_dim / 2);
+    if (n == 0) return NVMAI_OK;
+    dim3 grid((uint32_t)((n + 255) / 256));
+    if (ctx->act == ACT_BF16) rope_neox_subdim_kernel<ACT_BF16><<<grid, 256, 0, (hipStream_t)stream>>>(data, tokens, heads, head_dim, rotary_dim, positions, position, theta);
+    else rope_neox_subdim_kernel<ACT_FP16><<<grid, 256, 0, (hipStream_t)stream>>>(data, tokens, heads, head_dim, rotary_dim, positions, position, theta);
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
+                                          const nvmai_kv_view* k, const nvmai_kv_view* v,
+                                          uint64_t kv_batch_stride, void* out, uint32_t batch,
+                                          uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                          uint32_t seq_len, uint32_t kv_start, float scale) {
+    if (!ctx || !q || !out || batch == 0 || head_dim == 0 || num_kv_heads == 0) return NVMAI_ERR_INVALID_ARG;
+    if (num_q_heads % num_kv_heads) return NVMAI_ERR_INVALID_ARG;      // Attention.swift:221-222
+    if (head_dim > 512) return NVMAI_ERR_INVALID_ARG;                  // Attention.swift:223-224
+    if (kv_start > seq_len) return NVMAI_ERR_INVALID_ARG;
+    const uint32_t elements = num_kv_heads * head_dim;
+    int rc = check_view(k, elements);
+    if (rc) return rc;
+    rc = check_view(v, elements);
+    if (rc) return rc;
+    if (k->bits != v->bits || k->stride != v->stride) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(q)) return NVMAI_ERR_ALIGNMENT;
+    hipStream_t s = (hipStream_t)stream;
+    const uint32_t len = seq_len - kv_start;
+    const uint32_t qpk = num_q_heads / num_kv_heads;
+    const bool fast = head_dim == ATTN_HD && (k->bits == 4 || k->bits == 8) && qpk <= 16 &&
+                      aligned16(k->base) && aligned16(v->base) && (k->stride % 16 == 0) &&
+                      (kv_batch_stride % 16 == 0);
+    // Chunking: enough blocks to fill the device, chunks a multiple of the 32-token step.
+    const uint32_t units = fast ? batch * num_kv_heads : batch * num_q_heads;
+    uint32_t nc = (512 + units - 1) / units;
+    const uint32_t max_nc = (len + 127) / 128 ? (len + 127) / 128 : 1;
+    if (nc > max_nc) nc = max_nc;
+    if (nc < 1) nc = 1;
+    uint32_t chunk_len = ((len > 0 ? len : 1) + nc - 1) / nc;
+    chunk_len = (chunk_len + 31) & ~31u;
+    nc = ((len > 0 ? len : 1) + chunk_len - 1) / chunk_len;
+    const size_t heads_total = (size_t)batch * num_q_heads;
+    rc = ws_begin(ctx, 2 * ws_round(heads_total * nc * 4) + ws_round(heads_total * nc * head_dim * 4));
+    if (rc) return rc;
+    AttnParams p{};
+    p.q = q; p.k = (const uint8_t*)k->base; p.v = (const uint8_t*)v->base; p.kv_batch_stride = kv_batch_stride;
+    p.f = KvFormat{k->bits, k->stride, k->value_bytes, elements};
+    p.head_dim = head_dim; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads; p.batch = batch;
+    p.seq_len = seq_len; p.kv_start = kv_start; p.num_chunks = nc; p.chunk_len = chunk_len;
+    p.scale = scale > 0.0f ? scale : 1.0f / std::sqrt((float)head_dim);
+    p.m_part = ws_take<float>(ctx, heads_total * nc);
+    p.d_part = ws_take<float>(ctx, heads_total * nc);
+    p.o_part = ws_take<float>(ctx, heads_total * nc * head_dim);
+    p.out = out;
+    {
+        ProfScope ps(ctx, NVMAI_PROF_ATTN_PARTIAL, s);
+        if (fast) {
+            const size_t lds = (256 + 3 * (16 * ATTN_HD + 32)) * sizeof(float);
+            dim3 grid(batch * num_kv_heads * nc);
+#define NVMAI_ATTN(ACT, BITS) attn_partial_mfma_kernel<ACT, BITS><<<grid, 256, lds, s>>>(p)
+            if (ctx->act == ACT_BF16) { if (k->bits == 8) NVMAI_ATTN(ACT_BF16, 8); else NVMAI_ATTN(ACT_BF16, 4); }
+            else { if (k->bits == 8) NVMAI_ATTN(ACT_FP16, 8); else NVMAI_ATTN(ACT_FP16, 4); }
+#undef NVMAI_ATTN
+        } else {
+            dim3 grid(batch * num_q_heads * nc);
+            if (ctx->act == ACT_BF16) attn_partial_generic_kernel<ACT_BF16><<<grid, 256, 0, s>>>(p);
+            else attn_partial_generic_kernel<ACT_FP16><<<grid, 256, 0, s>>>(p);
+        }
+    }
+    {
+        ProfScope ps(ctx, NVMAI_PROF_ATTN_COMBINE, s);
+        if (ctx->act == ACT_BF16) attn_combine_kernel<ACT_BF16><<<dim3((uint32_t)heads_total), 256, 0, s>>>(p);
+        else attn_combine_kernel<ACT_FP16><<<dim3((uint32_t)heads_total), 256, 0, s>>>(p);
+    }
+    return launch_status();
+}

@@ -1,0 +1,524 @@
+// KV-cache quantize-on-write, partial RoPE and GQA decode attention over quantized K/V.
+// gfx950, wave64.
+#pragma once
+
+#include "common.cuh"
+
+namespace nvmai {
+
+// ---- KV row layout (KVCacheManager.swift:437-446) -----------------------------------------
+// row = packed codes (value_bytes, even) | fp16 scales[groups] | fp16 biases[groups]
+struct KvFormat {
+    uint32_t bits;         // 4, 8 or 16
+    uint32_t stride;       // bytes per token row
+    uint32_t value_bytes;
+    uint32_t elements;     // num_kv_heads * head_dim
+};
+
+// ---- quantize on write (kv_cache_quantize.metal:7-73) -------------------------------------
+// One wave per (token, group of 64): lane = element.  scale = (max-min)/levels from the
+// unrounded fp32 extremes (0 for a flat group), code = round_half_away(clamp((v-bias)/scale)),
+// stored scale/bias = fp16 of the fp32 values.  Every step is one IEEE operation.
+template <int ACT>
+__global__ __launch_bounds__(256) void kv_quantize_kernel(const void* src, uint32_t src_stride, uint8_t* dst,
+                                                         KvFormat f, uint32_t tokens) {
+    const uint32_t groups = (f.elements + 63) / 64;
+    const uint64_t gid = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (gid >= (uint64_t)tokens * groups) return;
+    const uint32_t token = gid / groups, g = gid % groups;
+    const int lane = threadIdx.x & 63;
+    const uint32_t e = g * 64 + lane;
+    const bool active = e < f.elements;
+    const float v = active ? act_to_f32<ACT>(((const uint16_t*)src)[(size_t)token * src_stride + e]) : 0.0f;
+    float mn = active ? v : INFINITY, mx = active ? v : -INFINITY;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        mn = fminf(mn, shfl_xor_f(mn, off));
+        mx = fmaxf(mx, shfl_xor_f(mx, off));
+    }
+    const float levels = f.bits == 4 ? 15.0f : 255.0f;
+    const float bias = mn;
+    const float scale = mx > mn ? __fdiv_rn(__fsub_rn(mx, mn), levels) : 0.0f;
+    uint8_t* row = dst + (size_t)token * f.stride;
+    if (lane == 0) {
+        reinterpret_cast<uint16_t*>(row + f.value_bytes)[g] = f32_to_f16(scale);
+        reinterpret_cast<uint16_t*>(row + f.value_bytes)[groups + g] = f32_to_f16(bias);
+    }
+    float q = 0.0f;
+    if (scale > 0.0f) q = roundf(fminf(fmaxf(__fdiv_rn(__fsub_rn(v, bias), scale), 0.0f), levels));
+    const uint32_t code = active ? (uint32_t)q : 0u;
+    if (f.bits == 8) {
+        if (active) row[e] = (uint8_t)code;
+    } else {
+        const uint32_t hi = shfl_xor_u(code, 1);     // inactive neighbours contribute 0
+        if (active && (lane & 1) == 0) row[e / 2] = (uint8_t)(code | (hi << 4));
+    }
+}
+
+// ---- partial RoPE (rope.metal:32-50, 80-102) ------------------------------------------------
+// data [tokens, heads, head_dim] in place; pair (i, rot/2 + i), angle = pos * theta^(-2i/rot).
+template <int ACT>
+__global__ void rope_neox_subdim_kernel(void* data, uint32_t tokens, uint32_t heads, uint32_t head_dim,
+                                        uint32_t rotary_dim, const uint32_t* positions, uint32_t position0,
+                                        float theta) {
+    const uint32_t half_rot = rotary_dim / 2;
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (uint64_t)tokens * heads * half_rot) return;
+    const uint32_t pair = i % half_rot;
+    const uint64_t th = i / half_rot;              // token * heads + head
+    const uint32_t token = th / heads;
+    const uint32_t pos = positions ? positions[token] : position0;
+    uint16_t* head = (uint16_t*)data + th * head_dim;
+    const float exponent = __fdiv_rn(-(float)(2u * pair), (float)rotary_dim);
+    const float angle = __fmul_rn((float)pos, powf(theta, exponent));
+    const float c = cosf(angle), s = sinf(angle);
+    const float x0 = act_to_f32<ACT>(head[pair]), x1 = act_to_f32<ACT>(head[half_rot + pair]);
+    head[pair] = f32_to_act<ACT>(__fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s)));
+    head[half_rot + pair] = f32_to_act<ACT>(__fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c)));
+}
+
+// ---- decode attention ------------------------------------------------------------------------
+struct AttnParams {
+    const void* q;             // [batch, num_q_heads, head_dim] activations
+    const uint8_t* k;          // cache of sequence b at k + b * kv_batch_stride
+    const uint8_t* v;
+    uint64_t kv_batch_stride;  // bytes
+    KvFormat f;
+    uint32_t head_dim, num_q_heads, num_kv_heads, batch;
+    uint32_t seq_len, kv_start;
+    uint32_t num_chunks, chunk_len;
+    float scale;
+    float* m_part;             // [batch, num_q_heads, num_chunks]
+    float* d_part;
+    float* o_part;             // [batch, num_q_heads, num_chunks, head_dim]
+    void* out;                 // [batch, num_q_heads, head_dim] activations
+};
+
+__device__ __forceinline__ float kv_load(const uint8_t* row, const KvFormat& f, uint32_t e) {   // attention.metal:89-117
+    if (f.bits == 16) return f16_to_f32(reinterpret_cast<const uint16_t*>(row)[e]);
+    const uint32_t groups = (f.elements + 63) / 64;
+    const uint32_t q = f.bits == 8 ? row[e] : ((e & 1) ? (row[e / 2] >> 4) : (row[e / 2] & 0x0F));
+    const uint16_t* meta = reinterpret_cast<const uint16_t*>(row + f.value_bytes);
+    return fmaf((float)q, f16_to_f32(meta[e / 64]), f16_to_f32(meta[groups + e / 64]));
+}
+
+// Generic split-KV partial (attention.metal:163-261): any head_dim <= 512, any format.
+// One block per (batch, q head, chunk); thread i owns dims i, i+256.
+template <int ACT>
+__global__ __launch_bounds__(256) void attn_partial_generic_kernel(AttnParams p) {
+    __shared__ float red[4];
+    const uint32_t chunk = blockIdx.x % p.num_chunks;
+    const uint32_t head = (blockIdx.x / p.num_chunks) % p.num_q_heads;
+    const uint32_t b = blockIdx.x / (p.num_chunks * p.num_q_heads);
+    const uint32_t kvh = head / (p.num_q_heads / p.num_kv_heads);
+    const uint32_t p0 = p.kv_start + chunk * p.chunk_len, p1 = min(p0 + p.chunk_len, p.seq_len);
+    const uint16_t* qh = (const uint16_t*)p.q + ((size_t)b * p.num_q_heads + head) * p.head_dim;
+    const uint32_t tid = threadIdx.x;
+    float qv[2], o[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int s = 0; s < 2; ++s) qv[s] = tid + 256 * s < p.head_dim ? act_to_f32<ACT>(qh[tid + 256 * s]) : 0.0f;
+    float m = -INFINITY, d = 0.0f;
+    for (uint32_t pos = p0; pos < p1; ++pos) {
+        const uint8_t* kr = p.k + b * p.kv_batch_stride + (size_t)pos * p.f.stride;
+        const uint8_t* vr = p.v + b * p.kv_batch_stride + (size_t)pos * p.f.stride;
+        float part = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+            if (tid + 256 * s < p.head_dim) part = fmaf(qv[s], kv_load(kr, p.f, kvh * p.head_dim + tid + 256 * s), part);
+        part = wave_sum_bcast(part);
+        if ((tid & 63) == 0) red[tid >> 6] = part;
+        __syncthreads();
+        const float sc = (red[0] + red[1] + red[2] + red[3]) * p.scale;
+        __syncthreads();
+        const float mn = fmaxf(m, sc);
+        const float alpha = expf(m - mn), pe = expf(sc - mn);
+        d = d * alpha + pe;
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+            if (tid + 256 * s < p.head_dim)
+                o[s] = o[s] * alpha + pe * kv_load(vr, p.f, kvh * p.head_dim + tid + 256 * s);
+        m = mn;
+    }
+    const size_t base = ((size_t)b * p.num_q_heads + head) * p.num_chunks + chunk;
+    if (tid == 0) { p.m_part[base] = m; p.d_part[base] = d; }
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+        if (tid + 256 * s < p.head_dim) p.o_part[base * p.head_dim + tid + 256 * s] = o[s];
+}
+
+// Combine (attention.metal:388-429): m* = max m_c, D = sum d_c e^(m_c - m*),
+// out = sum o_c e^(m_c - m*) / D; all chunks empty -> zeros.  One block per (batch, q head).
+template <int ACT>
+__global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
+    const size_t bh = blockIdx.x;
+    const float* mr = p.m_part + bh * p.num_chunks;
+    const float* dr = p.d_part + bh * p.num_chunks;
+    const float* orow = p.o_part + bh * p.num_chunks * p.head_dim;
+    uint16_t* out = (uint16_t*)p.out + bh * p.head_dim;
+    float mg = -INFINITY;
+    for (uint32_t c = 0; c < p.num_chunks; ++c) mg = fmaxf(mg, mr[c]);
+    if (mg == -INFINITY) {
+        for (uint32_t i = threadIdx.x; i < p.head_dim; i += 256) out[i] = f32_to_act<ACT>(0.0f);
+        return;
+    }
+    float D = 0.0f;
+    for (uint32_t c = 0; c < p.num_chunks; ++c) D += dr[c] * expf(mr[c] - mg);
+    const float inv = D > 0.0f ? 1.0f / D : 0.0f;
+    for (uint32_t i = threadIdx.x; i < p.head_dim; i += 256) {
+        float acc = 0.0f;
+        for (uint32_t c = 0; c < p.num_chunks; ++c) acc += orow[(size_t)c * p.head_dim + i] * expf(mr[c] - mg);
+        out[i] = f32_to_act<ACT>(acc * inv);
+    }
+}
+
+// ---- MFMA partial for head_dim 256, 4/8-bit K/V, up to 16 q heads per kv head ---------------
+// One block per (batch, kv head, chunk): every q head of the group is served from ONE read of
+// the K/V rows.  Each wave walks 32-token steps of the chunk with its own online-softmax state;
+// the four waves merge through LDS at the end.
+//   S^T[tokens, heads] = K . Q^T   v_mfma_f32_16x16x32_f16, A = codes as fp16 (1024 + c),
+//                                  B = q scaled by a power of two per head and cast to fp16;
+//                                  one accumulator per 64-wide group so that the row's fp16
+//                                  scale and bias are applied exactly:
+//                                  s = sum_g sc_g (acc_g - 1024 qsum_g) + bi_g qsum_g
+//   O[heads, dims]    = P'_g . V   A = p_t * vsc[t, g] as fp16 (one operand per group),
+//                                  B = V codes as fp16 (1024 + c); the bias and the 1024
+//                                  offset are carried in a per-(head, group) correction.
+// Lane roles (l = lane, r = l / 16, i = l % 16):
+//   K operand: token i of the 16-token tile, dims 64g + 16r + 8h .. +8 for MFMA call (g, h)
+//   Q operand: head i, the same dims
+//   S^T accumulators: head i, tokens 4r .. 4r+3 of the tile
+//   P' operand: head i, tokens {4r..4r+3 of tile 0, 4r..4r+3 of tile 1} of the 32-token step
+//   V operand (group g, tile n): dim 64g + 4i + n, the same eight tokens
+//   O accumulators (g, n): dim 64g + 4i + n, heads 4r .. 4r+3
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+
+union H8 { h8_t v; uint32_t u[4]; };
+
+__device__ __forceinline__ f4_t mfma16(const H8& a, const H8& b, f4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.v, b.v, c, 0, 0, 0);
+}
+
+constexpr int ATTN_HD = 256;
+constexpr int ATTN_STEP = 32;
+
+template <int ACT, int BITS>
+__global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
+    // LDS: per wave [16 heads][256 dims] O + [16] m + [16] d for the final merge (waves 1..3),
+    // plus a 64-float scratch per wave for head-indexed broadcasts.
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, r = lane >> 4;
+    float* bc = lds + wave * 64;                                   // broadcast scratch
+    float* merge = lds + 256;                                      // [3][16*256 + 32]
+    const uint32_t chunk = blockIdx.x % p.num_chunks;
+    const uint32_t kvh = (blockIdx.x / p.num_chunks) % p.num_kv_heads;
+    const uint32_t b = blockIdx.x / (p.num_chunks * p.num_kv_heads);
+    const uint32_t qpk = p.num_q_heads / p.num_kv_heads;           // <= 16
+    const uint32_t p0 = p.kv_start + chunk * p.chunk_len, p1 = min(p0 + p.chunk_len, p.seq_len);
+    const uint32_t groups_total = (p.f.elements + 63) / 64;
+    const uint32_t code_off = kvh * ATTN_HD * BITS / 8;            // this head's codes inside a row
+    const uint32_t meta_sc = p.f.value_bytes + 2 * (kvh * 4);      // 4 fp16 scales of this head
+    const uint32_t meta_bi = p.f.value_bytes + 2 * groups_total + 2 * (kvh * 4);
+    const uint8_t* kbase = p.k + b * p.kv_batch_stride;
+    const uint8_t* vbase = p.v + b * p.kv_batch_stride;
+
+    // ---- Q: head i (zero for i >= qpk), scaled to fp16; operands and per-group sums
+    H8 qop[4][2];
+    float qsum[4];
+    float q_unscale;                                               // scale * 2^-k of head i
+    {
+        const bool live = (uint32_t)i < qpk;
+        const uint16_t* qh = (const uint16_t*)p.q + ((size_t)b * p.num_q_heads + kvh * qpk + (live ? i : 0)) * ATTN_HD;
+        float qf[4][2][8];
+        float amax = 0.0f;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint4 raw = *reinterpret_cast<const uint4*>(qh + 64 * g + 16 * r + 8 * h);
+                act2_to_f32<ACT>(raw.x, qf[g][h][0], qf[g][h][1]); act2_to_f32<ACT>(raw.y, qf[g][h][2], qf[g][h][3]);
+                act2_to_f32<ACT>(raw.z, qf[g][h][4], qf[g][h][5]); act2_to_f32<ACT>(raw.w, qf[g][h][6], qf[g][h][7]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (!live) qf[g][h][e] = 0.0f;
+                    amax = fmaxf(amax, fabsf(qf[g][h][e]));
+                }
+            }
+        amax = fmaxf(amax, shfl_xor_f(amax, 16));
+        amax = fmaxf(amax, shfl_xor_f(amax, 32));
+        // power of two mapping amax into [1024, 2048) (1 for zero / non-finite rows)
+        const uint32_t ex = (__float_as_uint(amax) >> 23) & 0xFFu;
+        float sc = 1.0f, isc = 1.0f;
+        if (ex >= 24u && ex <= 254u) { sc = __uint_as_float((264u - ex) << 23); isc = __uint_as_float((ex - 10u) << 23); }
+        q_unscale = p.scale * isc;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float s = 0.0f;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                uint16_t hb[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    hb[e] = f32_to_f16(qf[g][h][e] * sc);
+                    s += f16_to_f32(hb[e]);
+                }
+                if (BITS == 8) {
+                    // K codes unpack in natural byte order: pairs (0,1) (2,3) (4,5) (6,7)
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) qop[g][h].u[w] = hb[2 * w] | ((uint32_t)hb[2 * w + 1] << 16);
+                } else {
+                    // 4-bit codes unpack as pairs (j, j+4) of the dword's eight nibbles
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) qop[g][h].u[w] = hb[w] | ((uint32_t)hb[w + 4] << 16);
+                }
+            }
+            s += shfl_xor_f(s, 16);
+            s += shfl_xor_f(s, 32);
+            qsum[g] = s;                                           // over all 64 dims of group g, head i
+        }
+    }
+
+    f4_t oacc[4][4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int n = 0; n < 4; ++n) oacc[g][n] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY, d_run = 0.0f;                          // head i; d over this lane's tokens only
+    float corr[4] = {0.0f, 0.0f, 0.0f, 0.0f};                       // head i, this lane's tokens only
+
+    for (uint32_t s0 = p0 + wave * ATTN_STEP; s0 < p1; s0 += 4 * ATTN_STEP) {
+        // ---- loads: K codes (token i of each tile), metadata and V codes of this lane's 8 tokens
+        uint32_t kraw[2][4][4];                                     // [tile][group][dwords]; 4-bit uses 2 dwords
+        uint32_t tok[8];                                            // clamped token positions of the P/V slots
+        bool tok_ok[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const uint32_t pos = s0 + (t >> 2) * 16 + 4 * r + (t & 3);
+            tok_ok[t] = pos < p1;
+            tok[t] = tok_ok[t] ? pos : p1 - 1;
+        }
+#pragma unroll
+        for (int tile = 0; tile < 2; ++tile) {
+            const uint32_t pos = min(s0 + tile * 16 + i, p1 - 1);
+            const uint8_t* row = kbase + (size_t)pos * p.f.stride + code_off;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                if (BITS == 8) {
+                    const uint4 w = *reinterpret_cast<const uint4*>(row + 64 * g + 16 * r);
+                    kraw[tile][g][0] = w.x; kraw[tile][g][1] = w.y; kraw[tile][g][2] = w.z; kraw[tile][g][3] = w.w;
+                } else {
+                    const uint2 w = *reinterpret_cast<const uint2*>(row + 32 * g + 8 * r);
+                    kraw[tile][g][0] = w.x; kraw[tile][g][1] = w.y;
+                }
+            }
+        }
+        uint2 ksc[8], kbi[8], vsc[8], vbi[8];                        // 4 fp16 each
+        uint32_t vraw[8][4];                                        // [token slot][group]: 4 codes (8-bit) / 4 nibbles
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const uint8_t* krow = kbase + (size_t)tok[t] * p.f.stride;
+            const uint8_t* vrow = vbase + (size_t)tok[t] * p.f.stride;
+            ksc[t] = *reinterpret_cast<const uint2*>(krow + meta_sc);
+            kbi[t] = *reinterpret_cast<const uint2*>(krow + meta_bi);
+            vsc[t] = *reinterpret_cast<const uint2*>(vrow + meta_sc);
+            vbi[t] = *reinterpret_cast<const uint2*>(vrow + meta_bi);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                if (BITS == 8) vraw[t][g] = *reinterpret_cast<const uint32_t*>(vrow + code_off + 64 * g + 4 * i);
+                else vraw[t][g] = *reinterpret_cast<const uint16_t*>(vrow + code_off + 32 * g + 2 * i);
+            }
+        }
+
+        // ---- S^T = K . Q^T per group, then the exact affine correction
+        float sv[8];                                                // scores of head i at this lane's 8 tokens
+#pragma unroll
+        for (int tile = 0; tile < 2; ++tile) {
+            f4_t sacc[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                sacc[g] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    H8 a;
+                    if (BITS == 8) {
+                        const uint32_t w0 = kraw[tile][g][2 * h], w1 = kraw[tile][g][2 * h + 1];
+                        a.u[0] = __builtin_amdgcn_perm(w0, 0x64646464u, 0x00050004u);
+                        a.u[1] = __builtin_amdgcn_perm(w0, 0x64646464u, 0x00070006u);
+                        a.u[2] = __builtin_amdgcn_perm(w1, 0x64646464u, 0x00050004u);
+                        a.u[3] = __builtin_amdgcn_perm(w1, 0x64646464u, 0x00070006u);
+                    } else {
+                        const uint32_t w = kraw[tile][g][h];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) a.u[j] = ((w >> (4 * j)) & 0x000F000Fu) | 0x64006400u;
+                    }
+                    sacc[g] = mfma16(a, qop[g][h], sacc[g]);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int slot = tile * 4 + t;
+                const uint32_t scw[2] = {ksc[slot].x, ksc[slot].y}, biw[2] = {kbi[slot].x, kbi[slot].y};
+                float acc = 0.0f;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const float sc = f16_to_f32((uint16_t)(scw[g >> 1] >> (16 * (g & 1))));
+                    const float bi = f16_to_f32((uint16_t)(biw[g >> 1] >> (16 * (g & 1))));
+                    acc = fmaf(sc, fmaf(-1024.0f, qsum[g], sacc[g][t]), acc);
+                    acc = fmaf(bi, qsum[g], acc);
+                }
+                sv[slot] = tok_ok[slot] ? acc * q_unscale : -INFINITY;
+            }
+        }
+
+        // ---- online softmax for head i (its tokens are spread over the four lane quarters)
+        float mx = sv[0];
+#pragma unroll
+        for (int t = 1; t < 8; ++t) mx = fmaxf(mx, sv[t]);
+        mx = fmaxf(mx, shfl_xor_f(mx, 16));
+        mx = fmaxf(mx, shfl_xor_f(mx, 32));
+        const float m_new = fmaxf(m_run, mx);                       // finite: the step holds >= 1 valid token
+        const float alpha = expf(m_run - m_new);
+        float pe[8], psum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) { pe[t] = expf(sv[t] - m_new); psum += pe[t]; }
+        d_run = d_run * alpha + psum;
+        m_run = m_new;
+
+        // ---- P'_g = p * vsc_g as fp16; correction terms; rescale O by alpha of its heads
+        H8 pop[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float c = corr[g] * alpha;
+            uint16_t hb[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const uint32_t scw = g < 2 ? vsc[t].x : vsc[t].y, biw = g < 2 ? vbi[t].x : vbi[t].y;
+                const float sc = f16_to_f32((uint16_t)(scw >> (16 * (g & 1))));
+                const float bi = f16_to_f32((uint16_t)(biw >> (16 * (g & 1))));
+                hb[t] = f32_to_f16(pe[t] * sc);
+                c = fmaf(pe[t], bi, c);
+                c = fmaf(-1024.0f, f16_to_f32(hb[t]), c);
+            }
+            corr[g] = c;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) pop[g].u[w] = hb[2 * w] | ((uint32_t)hb[2 * w + 1] << 16);
+        }
+        if (i < 16 && r == 0) bc[i] = alpha;                        // head-indexed broadcast through LDS
+        __builtin_amdgcn_wave_barrier();
+        const float4 al = *reinterpret_cast<const float4*>(bc + 4 * r);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int n = 0; n < 4; ++n) {
+                oacc[g][n][0] *= al.x; oacc[g][n][1] *= al.y; oacc[g][n][2] *= al.z; oacc[g][n][3] *= al.w;
+            }
+
+        // ---- O += P'_g . V   (B operand: dim 64g + 4i + n, this lane's 8 tokens)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int n = 0; n < 4; ++n) {
+                H8 bop;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t a = vraw[2 * w][g], c2 = vraw[2 * w + 1][g];
+                    if (BITS == 8) {
+                        // byte n of two token dwords -> [a.n, 0x64, c2.n, 0x64]
+                        const uint32_t lo = (a >> (8 * n)) & 0xFFu, hi = (c2 >> (8 * n)) & 0xFFu;
+                        bop.u[w] = lo | (hi << 16) | 0x64006400u;
+                    } else {
+                        const uint32_t lo = (a >> (4 * n)) & 0xFu, hi = (c2 >> (4 * n)) & 0xFu;
+                        bop.u[w] = lo | (hi << 16) | 0x64006400u;
+                    }
+                }
+                oacc[g][n] = mfma16(pop[g], bop, oacc[g][n]);
+            }
+    }
+
+    // ---- finish this wave: d and corr over the four quarters, corr folded into O
+    d_run += shfl_xor_f(d_run, 16);
+    d_run += shfl_xor_f(d_run, 32);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        corr[g] += shfl_xor_f(corr[g], 16);
+        corr[g] += shfl_xor_f(corr[g], 32);
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        if (r == 0) bc[i] = corr[g];
+        __builtin_amdgcn_wave_barrier();
+        const float4 cg = *reinterpret_cast<const float4*>(bc + 4 * r);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+            oacc[g][n][0] += cg.x; oacc[g][n][1] += cg.y; oacc[g][n][2] += cg.z; oacc[g][n][3] += cg.w;
+        }
+    }
+
+    // ---- merge the four waves (wave 0 collects), attention.metal:388-429's rule
+    float* mine = merge + (wave - 1) * (16 * ATTN_HD + 32);
+    if (wave > 0) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int n = 0; n < 4; ++n)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) mine[(4 * r + t) * ATTN_HD + 64 * g + 4 * i + n] = oacc[g][n][t];
+        if (r == 0) { mine[16 * ATTN_HD + i] = m_run; mine[16 * ATTN_HD + 16 + i] = d_run; }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float m_all = m_run;
+#pragma unroll
+    for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, merge[w * (16 * ATTN_HD + 32) + 16 * ATTN_HD + i]);
+    // weights e^(m_w - m_all) per head i; broadcast to the O layout (heads 4r..4r+3) through LDS
+    float wgt[4];
+    wgt[0] = m_run == -INFINITY ? 0.0f : expf(m_run - m_all);
+    float d_all = d_run * wgt[0];
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+        const float mw = merge[w * (16 * ATTN_HD + 32) + 16 * ATTN_HD + i];
+        wgt[w + 1] = mw == -INFINITY ? 0.0f : expf(mw - m_all);
+        d_all += merge[w * (16 * ATTN_HD + 32) + 16 * ATTN_HD + 16 + i] * wgt[w + 1];
+    }
+    float4 wq[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        if (r == 0) bc[i] = wgt[w];
+        __builtin_amdgcn_wave_barrier();
+        wq[w] = *reinterpret_cast<const float4*>(bc + 4 * r);
+        __builtin_amdgcn_wave_barrier();
+    }
+    const size_t hbase = (size_t)b * p.num_q_heads + kvh * qpk;
+    if (r == 0 && (uint32_t)i < qpk) {
+        p.m_part[(hbase + i) * p.num_chunks + chunk] = m_all;
+        p.d_part[(hbase + i) * p.num_chunks + chunk] = d_all;
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const uint32_t head = 4 * r + t;
+        if (head >= qpk) continue;
+        const float w0 = t == 0 ? wq[0].x : t == 1 ? wq[0].y : t == 2 ? wq[0].z : wq[0].w;
+        float* dst = p.o_part + ((hbase + head) * p.num_chunks + chunk) * ATTN_HD;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float4 o4;
+            float* o4p = &o4.x;
+#pragma unroll
+            for (int n = 0; n < 4; ++n) {
+                float acc = oacc[g][n][t] * w0;
+#pragma unroll
+                for (int w = 0; w < 3; ++w) {
+                    const float ww = t == 0 ? wq[w + 1].x : t == 1 ? wq[w + 1].y : t == 2 ? wq[w + 1].z : wq[w + 1].w;
+                    acc += merge[w * (16 * ATTN_HD + 32) + head * ATTN_HD + 64 * g + 4 * i + n] * ww;
+                }
+                o4p[n] = acc;
+            }
+            *reinterpret_cast<float4*>(dst + 64 * g + 4 * i) = o4;
+        }
+    }
+}
+
+}  // namespace nvmai

@@ -1,0 +1,75 @@
+// Entry points: tiled softmax over the vocabulary, top-64 and generic samplers.
+#include "ctx.hpp"
+#include "sample_kernels.cuh"
+
+using namespace nvmai;
+
+extern "C" uint64_t nvmai_sampler_seed_for(uint64_t seed, int64_t position) {
+    uint64_t z = seed + (uint64_t)position + 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    return z == 0 ? 0x9E3779B97F4A7C15ull : z;
+}
+
+extern "C" int nvmai_hip_softmax_tiled(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* logits,
+                                       uint32_t logits_stride, uint16_t* probs, uint32_t probs_stride,
+                                       uint32_t rows, uint32_t v, float softcap) {
+    if (!ctx || !logits || !probs || v == 0 || logits_stride < v || probs_stride < v) return NVMAI_ERR_INVALID_ARG;
+    if (rows == 0) return NVMAI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const uint32_t tiles = (v + SOFTMAX_TILE - 1) / SOFTMAX_TILE;
+    int rc = ws_begin(ctx, 2 * ws_round((size_t)rows * tiles * 4));
+    if (rc) return rc;
+    float* tmax = ws_take<float>(ctx, (size_t)rows * tiles);
+    float* tsum = ws_take<float>(ctx, (size_t)rows * tiles);
+    ProfScope ps(ctx, NVMAI_PROF_SOFTMAX, s);
+    dim3 grid(tiles, rows);
+    if (ctx->act == ACT_BF16) {
+        softmax_stage1_kernel<ACT_BF16><<<grid, 256, 0, s>>>(logits, v, logits_stride, softcap, tmax, tsum, tiles);
+        softmax_normalize_kernel<ACT_BF16><<<grid, 256, 0, s>>>(logits, v, logits_stride, softcap, tmax, tsum, tiles, probs, probs_stride);
+    } else {
+        softmax_stage1_kernel<ACT_FP16><<<grid, 256, 0, s>>>(logits, v, logits_stride, softcap, tmax, tsum, tiles);
+        softmax_normalize_kernel<ACT_FP16><<<grid, 256, 0, s>>>(logits, v, logits_stride, softcap, tmax, tsum, tiles, probs, probs_stride);
+    }
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_sample_topk64(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint16_t* probs,
+                                       uint32_t probs_stride, uint32_t rows, uint32_t v, float temperature,
+                                       float top_p, const uint64_t* seeds, uint32_t top_k, uint32_t* out_token,
+                                       uint32_t* top64_out) {
+    if (!ctx || !probs || !seeds || !out_token || probs_stride < v) return NVMAI_ERR_INVALID_ARG;
+    if (v == 0 || v > 262144) return NVMAI_ERR_UNSUPPORTED;      // SampleTopK64Error.unsupportedVocabulary
+    if (!(temperature > 0.0f)) return NVMAI_ERR_INVALID_ARG;     // LogitOutput.swift:280-281
+    if (top_k < 1 || top_k > 64) return NVMAI_ERR_INVALID_ARG;   // LogitOutput.swift:282-283
+    if (rows == 0) return NVMAI_OK;
+    if (rows > SAMPLE_MAX_ROWS) return NVMAI_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const uint32_t g1 = (v + SAMPLE_TILE - 1) / SAMPLE_TILE, c1 = g1 * SAMPLE_KEEP;
+    const uint32_t g2 = (c1 + SAMPLE_TILE - 1) / SAMPLE_TILE, c2 = g2 * SAMPLE_KEEP;
+    int rc = ws_begin(ctx, ws_round((size_t)rows * c1 * 8) + ws_round((size_t)rows * c2 * 8));
+    if (rc) return rc;
+    uint64_t* s1 = ws_take<uint64_t>(ctx, (size_t)rows * c1);
+    uint64_t* s2 = ws_take<uint64_t>(ctx, (size_t)rows * c2);
+    SeedArray sa{};
+    for (uint32_t r = 0; r < rows; ++r) sa.s[r] = seeds[r];
+    ProfScope ps(ctx, NVMAI_PROF_SAMPLE, s);
+    sample_topk64_stage1_kernel<<<dim3(g1, rows), 256, 0, s>>>(probs, v, probs_stride, s1, c1);
+    sample_topk64_reduce_kernel<<<dim3(g2, rows), 256, 0, s>>>(s1, c1, c1, s2, c2);
+    sample_topk64_final_kernel<<<dim3(rows), 256, 0, s>>>(s2, c2, c2, temperature, top_p, sa, top_k, out_token, top64_out);
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_sample(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint16_t* probs,
+                                uint32_t probs_stride, uint32_t rows, uint32_t v, float temperature,
+                                uint32_t top_k, float top_p, const uint64_t* seeds, uint32_t* out_token) {
+    if (!ctx || !probs || !seeds || !out_token || v == 0 || probs_stride < v) return NVMAI_ERR_INVALID_ARG;
+    if (rows == 0) return NVMAI_OK;
+    if (rows > SAMPLE_MAX_ROWS) return NVMAI_ERR_INVALID_ARG;
+    SeedArray sa{};
+    for (uint32_t r = 0; r < rows; ++r) sa.s[r] = seeds[r];
+    ProfScope ps(ctx, NVMAI_PROF_SAMPLE, (hipStream_t)stream);
+    sample_generic_kernel<<<dim3(rows), 256, 0, (hipStream_t)stream>>>(probs, v, probs_stride, temperature, top_k, top_p, sa, out_token);
+    return launch_status();
+}

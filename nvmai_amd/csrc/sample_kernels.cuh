@@ -1,0 +1,261 @@
+// Softmax over the vocabulary and the tiled top-64 / generic samplers.  gfx950, wave64.
+#pragma once
+
+#include "common.cuh"
+
+namespace nvmai {
+
+constexpr int SOFTMAX_TILE = 4096;       // logit.metal:159
+constexpr int SAMPLE_TILE = 1024;        // logit.metal:628-654
+constexpr int SAMPLE_KEEP = 64;
+
+__device__ __forceinline__ float softcap_value(float z, float softcap) {   // logit.metal:42-49
+    return softcap <= 0.0f ? z : softcap * tanhf(z / softcap);
+}
+
+// (max, sum of exp) of two partial states, the empty state being (-inf, 0).
+__device__ __forceinline__ void softmax_merge(float& m, float& d, float m2, float d2) {
+    const float mn = fmaxf(m, m2);
+    const float a = (m == -INFINITY) ? 0.0f : d * expf(m - mn);
+    const float b = (m2 == -INFINITY) ? 0.0f : d2 * expf(m2 - mn);
+    m = mn;
+    d = a + b;
+}
+
+__device__ __forceinline__ void block_softmax_merge(float& m, float& d, float* lds) {
+    // wave butterfly, then the four waves through LDS; every thread ends with the block result
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const float m2 = shfl_xor_f(m, off), d2 = shfl_xor_f(d, off);
+        softmax_merge(m, d, m2, d2);
+    }
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) { lds[2 * wave] = m; lds[2 * wave + 1] = d; }
+    __syncthreads();
+    m = lds[0]; d = lds[1];
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) softmax_merge(m, d, lds[2 * w], lds[2 * w + 1]);
+    __syncthreads();
+}
+
+// Stage 1 (logit.metal:155-200): per 4096-entry tile the running (max, sum exp).
+template <int ACT>
+__global__ __launch_bounds__(256) void softmax_stage1_kernel(const void* logits, uint32_t v, uint32_t row_stride,
+                                                            float softcap, float* tile_max, float* tile_sum,
+                                                            uint32_t tiles) {
+    __shared__ float lds[8];
+    const uint32_t tile = blockIdx.x, row = blockIdx.y;
+    const uint16_t* z = (const uint16_t*)logits + (size_t)row * row_stride;
+    const uint32_t base = tile * SOFTMAX_TILE, end = min(base + SOFTMAX_TILE, v);
+    float m = -INFINITY, d = 0.0f;
+    for (uint32_t i = base + threadIdx.x; i < end; i += 256) {
+        const float x = softcap_value(act_to_f32<ACT>(z[i]), softcap);
+        softmax_merge(m, d, x, 1.0f);
+    }
+    block_softmax_merge(m, d, lds);
+    if (threadIdx.x == 0) { tile_max[(size_t)row * tiles + tile] = m; tile_sum[(size_t)row * tiles + tile] = d; }
+}
+
+// Merge + normalize (logit.metal:202-257): every block folds the tile partials again
+// (a few dozen values), then writes probs = exp(z - max) * (1 / sum) as fp16.
+template <int ACT>
+__global__ __launch_bounds__(256) void softmax_normalize_kernel(const void* logits, uint32_t v, uint32_t row_stride,
+                                                               float softcap, const float* tile_max,
+                                                               const float* tile_sum, uint32_t tiles,
+                                                               uint16_t* probs, uint32_t probs_stride) {
+    __shared__ float lds[8];
+    const uint32_t row = blockIdx.y;
+    float m = -INFINITY, d = 0.0f;
+    for (uint32_t t = threadIdx.x; t < tiles; t += 256)
+        softmax_merge(m, d, tile_max[(size_t)row * tiles + t], tile_sum[(size_t)row * tiles + t]);
+    block_softmax_merge(m, d, lds);
+    const float inv = d > 0.0f ? 1.0f / d : 0.0f;
+    const uint16_t* z = (const uint16_t*)logits + (size_t)row * row_stride;
+    uint16_t* out = probs + (size_t)row * probs_stride;
+    const uint32_t base = blockIdx.x * SOFTMAX_TILE, end = min(base + SOFTMAX_TILE, v);
+    for (uint32_t i = base + threadIdx.x; i < end; i += 256)
+        out[i] = f32_to_f16(expf(softcap_value(act_to_f32<ACT>(z[i]), softcap) - m) * inv);
+}
+
+// ---- sampling ------------------------------------------------------------------------
+constexpr int SAMPLE_MAX_ROWS = 32;
+struct SeedArray { uint64_t s[SAMPLE_MAX_ROWS]; };   // one PRNG seed per row, passed by value
+
+__device__ __forceinline__ uint64_t xorshift64star(uint64_t& s) {        // logit.metal:280-285
+    s ^= s << 13;
+    s ^= s >> 7;
+    s ^= s << 17;
+    return s * 2685821657736338717ull;
+}
+
+__device__ __forceinline__ float uniform01(uint64_t& s) {                // logit.metal:287-292
+    return (float)(uint32_t)(xorshift64star(s) >> 40) * (1.0f / 16777216.0f);
+}
+
+// Total order "better(a, b) = a.v > b.v || (a.v == b.v && a.i < b.i)" (logit.metal:590-594)
+// as one unsigned compare: high word = order-preserving image of the float, low word = ~index.
+__device__ __forceinline__ uint64_t sample_key(float v, uint32_t idx) {
+    uint32_t u = __float_as_uint(v);
+    u ^= (u >> 31) ? 0xFFFFFFFFu : 0x80000000u;
+    return ((uint64_t)u << 32) | (uint32_t)~idx;
+}
+__device__ __forceinline__ float key_value(uint64_t k) {
+    uint32_t u = (uint32_t)(k >> 32);
+    u ^= (u >> 31) ? 0x80000000u : 0xFFFFFFFFu;
+    return __uint_as_float(u);
+}
+__device__ __forceinline__ uint32_t key_index(uint64_t k) { return ~(uint32_t)k; }
+
+// Bitonic sort of 1024 keys in LDS, descending (logit.metal:596-626).
+__device__ __forceinline__ void sort_tile_desc(uint64_t* keys) {
+    for (uint32_t width = 2; width <= SAMPLE_TILE; width <<= 1) {
+        for (uint32_t stride = width >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (uint32_t i = threadIdx.x; i < SAMPLE_TILE; i += 256) {
+                const uint32_t partner = i ^ stride;
+                if (partner <= i) continue;
+                const uint64_t a = keys[i], b = keys[partner];
+                const bool descending = (i & width) == 0;
+                if (descending ? (b > a) : (a > b)) { keys[i] = b; keys[partner] = a; }
+            }
+        }
+    }
+    __syncthreads();
+}
+
+// Stage 1 (logit.metal:628-654): top 64 of each 1024-entry tile of the fp16 probabilities.
+__global__ __launch_bounds__(256) void sample_topk64_stage1_kernel(const uint16_t* probs, uint32_t v,
+                                                                   uint32_t probs_stride, uint64_t* out,
+                                                                   uint32_t out_row_stride) {
+    __shared__ uint64_t keys[SAMPLE_TILE];
+    const uint32_t row = blockIdx.y, base = blockIdx.x * SAMPLE_TILE;
+    const uint16_t* p = probs + (size_t)row * probs_stride;
+    for (uint32_t i = threadIdx.x; i < SAMPLE_TILE; i += 256) {
+        const uint32_t src = base + i;
+        keys[i] = src < v ? sample_key(f16_to_f32(p[src]), src) : sample_key(-INFINITY, 0xFFFFFFFFu);
+    }
+    sort_tile_desc(keys);
+    if (threadIdx.x < SAMPLE_KEEP) out[(size_t)row * out_row_stride + blockIdx.x * SAMPLE_KEEP + threadIdx.x] = keys[threadIdx.x];
+}
+
+// Reduce (logit.metal:656-682): top 64 of each 1024 surviving candidates.
+__global__ __launch_bounds__(256) void sample_topk64_reduce_kernel(const uint64_t* in, uint32_t count,
+                                                                   uint32_t in_row_stride, uint64_t* out,
+                                                                   uint32_t out_row_stride) {
+    __shared__ uint64_t keys[SAMPLE_TILE];
+    const uint32_t row = blockIdx.y, base = blockIdx.x * SAMPLE_TILE;
+    for (uint32_t i = threadIdx.x; i < SAMPLE_TILE; i += 256) {
+        const uint32_t src = base + i;
+        keys[i] = src < count ? in[(size_t)row * in_row_stride + src] : sample_key(-INFINITY, 0xFFFFFFFFu);
+    }
+    sort_tile_desc(keys);
+    if (threadIdx.x < SAMPLE_KEEP) out[(size_t)row * out_row_stride + blockIdx.x * SAMPLE_KEEP + threadIdx.x] = keys[threadIdx.x];
+}
+
+// Selection over the sorted candidates (logit.metal:704-757 == :517-571): cap at k,
+// top-p cut on the cumulative mass, p^(1/T), inverse-CDF draw with xorshift64*.
+__device__ inline uint32_t sample_select(float* val, const uint32_t* idx, uint32_t kept, float temperature,
+                                         float top_p, uint64_t seed, uint32_t fallback) {
+    if (top_p > 0.0f && top_p < 1.0f) {
+        float cum = 0.0f;
+        uint32_t cut = kept;
+        for (uint32_t i = 0; i < kept; ++i) {
+            cum = __fadd_rn(cum, val[i]);
+            if (cum >= top_p) { cut = i + 1; break; }
+        }
+        kept = cut;
+    }
+    const float inv_t = __fdiv_rn(1.0f, temperature);
+    if (temperature != 1.0f)
+        for (uint32_t i = 0; i < kept; ++i) val[i] = powf(val[i], inv_t);
+    float surviving = 0.0f;
+    for (uint32_t i = 0; i < kept; ++i) surviving = __fadd_rn(surviving, val[i]);
+    uint64_t rng = seed;
+    (void)xorshift64star(rng);
+    const float u = __fmul_rn(uniform01(rng), surviving);
+    float run = 0.0f;
+    uint32_t picked = fallback;
+    for (uint32_t i = 0; i < kept; ++i) {
+        run = __fadd_rn(run, val[i]);
+        if (u <= run) { picked = idx[i]; break; }
+    }
+    return picked;
+}
+
+// Final (logit.metal:684-758).  seeds: one per row.  top64 (optional): the 64 sorted
+// candidates per row as (value bits, index) pairs.
+__global__ __launch_bounds__(256) void sample_topk64_final_kernel(const uint64_t* in, uint32_t count,
+                                                                  uint32_t in_row_stride, float temperature,
+                                                                  float top_p, SeedArray seeds,
+                                                                  uint32_t top_k, uint32_t* out_token,
+                                                                  uint32_t* top64) {
+    __shared__ uint64_t keys[SAMPLE_TILE];
+    __shared__ float val[SAMPLE_KEEP];
+    __shared__ uint32_t idx[SAMPLE_KEEP];
+    const uint32_t row = blockIdx.x;
+    for (uint32_t i = threadIdx.x; i < SAMPLE_TILE; i += 256)
+        keys[i] = i < count ? in[(size_t)row * in_row_stride + i] : sample_key(-INFINITY, 0xFFFFFFFFu);
+    sort_tile_desc(keys);
+    if (threadIdx.x < SAMPLE_KEEP) {
+        val[threadIdx.x] = key_value(keys[threadIdx.x]);
+        idx[threadIdx.x] = key_index(keys[threadIdx.x]);
+        if (top64) {
+            top64[((size_t)row * SAMPLE_KEEP + threadIdx.x) * 2] = __float_as_uint(val[threadIdx.x]);
+            top64[((size_t)row * SAMPLE_KEEP + threadIdx.x) * 2 + 1] = idx[threadIdx.x];
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t kept = 0;
+        while (kept < SAMPLE_KEEP && idx[kept] != 0xFFFFFFFFu && isfinite(val[kept])) kept++;
+        kept = min(kept, max(1u, top_k));
+        out_token[row] = sample_select(val, idx, kept, temperature, top_p, seeds.s[row], idx[0]);
+    }
+}
+
+// Generic sampler (logit.metal:315-585): greedy argmax at temperature <= 0, else k argmax
+// passes over the vocabulary (k <= 256), then the same selection.  One block per row.
+__global__ __launch_bounds__(256) void sample_generic_kernel(const uint16_t* probs, uint32_t v,
+                                                             uint32_t probs_stride, float temperature,
+                                                             uint32_t top_k, float top_p, SeedArray seeds,
+                                                             uint32_t* out_token) {
+    __shared__ uint64_t wave_best[4];
+    __shared__ float val[256];
+    __shared__ uint32_t idx[256];
+    const uint32_t row = blockIdx.x;
+    const uint16_t* p = probs + (size_t)row * probs_stride;
+    uint32_t k = temperature <= 0.0f ? 1u : (top_k == 0 ? v : top_k);
+    k = min(min(k, 256u), v);
+    uint64_t prev = ~0ull;               // every later pass takes the best key below the previous one
+    for (uint32_t slot = 0; slot < k; ++slot) {
+        uint64_t best = 0;
+        for (uint32_t i = threadIdx.x; i < v; i += 256) {
+            const float pv = f16_to_f32(p[i]);
+            if (!(pv > -INFINITY)) continue;                 // the kernel's `p > best_v` never takes -inf or NaN
+            const uint64_t key = sample_key(pv, i);
+            if (key < prev && key > best) best = key;
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const uint32_t lo = shfl_xor_u((uint32_t)best, off), hi = shfl_xor_u((uint32_t)(best >> 32), off);
+            const uint64_t o = ((uint64_t)hi << 32) | lo;
+            best = o > best ? o : best;
+        }
+        if ((threadIdx.x & 63) == 0) wave_best[threadIdx.x >> 6] = best;
+        __syncthreads();
+        best = max(max(wave_best[0], wave_best[1]), max(wave_best[2], wave_best[3]));
+        if (threadIdx.x == 0) {
+            val[slot] = best ? key_value(best) : -INFINITY;
+            idx[slot] = best ? key_index(best) : 0xFFFFFFFFu;
+        }
+        prev = best ? best : 0;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        if (temperature <= 0.0f) { out_token[row] = idx[0]; return; }
+        uint32_t kept = 0;
+        while (kept < k && idx[kept] < v && isfinite(val[kept])) kept++;
+        out_token[row] = sample_select(val, idx, kept, temperature, top_p, seeds.s[row], kept > 0 ? idx[0] : 0u);
+    }
+}
+
+}  // namespace nvmai

@@ -7,7 +7,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._lib import ExpertOffsets, MoeLayer, Rows, check, lib
+from ._lib import ExpertOffsets, KvView, MoeLayer, Rows, check, lib
 
 ACT_BF16, ACT_FP16 = 0, 1
 (PROF_ROUTER, PROF_SELECT, PROF_GROUP, PROF_PHASE1, PROF_PHASE2, PROF_COMBINE, PROF_KV_QUANT,
@@ -221,3 +221,157 @@ class SharedExpertRuntime:
                                           gate, _ptr(x2), x2.stride(0), tokens, _ptr(y), y.stride(0), d, f),
               "shared_expert")
         return y
+
+
+# ---------------------------------------------------------------------------------------------
+# KV cache, RoPE, attention
+# ---------------------------------------------------------------------------------------------
+def kv_row_layout(elements, bits):
+    """KVCacheManager.rowLayout (KVCacheManager.swift:437-446) -> (stride, value_bytes)."""
+    s, v = C.c_uint32(), C.c_uint32()
+    check(lib.nvmai_kv_row_layout(elements, bits, C.byref(s), C.byref(v)), "kv_row_layout")
+    return s.value, v.value
+
+
+class KVCache:
+    """One layer's K or V rows for `batch` sequences: the part of KVCacheManager
+    (KVCacheManager.swift) the kernels see.  rows[b, p, :] is the row of position p."""
+
+    def __init__(self, batch, max_context, elements, bits, device="cuda"):
+        self.bits, self.elements = bits, elements
+        self.stride, self.value_bytes = kv_row_layout(elements, bits)
+        self.rows = torch.zeros((batch, max_context, self.stride), dtype=torch.uint8, device=device)
+
+    def view(self, batch_index=0, position=0):
+        """KVView (KVCacheManager.swift:19-31) starting at `position` of one sequence."""
+        v = KvView()
+        v.base = self.rows[batch_index, position].data_ptr()
+        v.stride, v.value_bytes, v.bits, v.group_size = self.stride, self.value_bytes, self.bits, 64
+        return v
+
+    @property
+    def batch_stride(self):
+        return self.rows.stride(0)
+
+
+class KVCacheQuantizer:
+    """Mirror of KVCacheQuantizer (KVCacheQuantizer.swift:6-50)."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+
+    def encode(self, source, source_token_stride_elements, destination, token_count, element_count):
+        check(lib.nvmai_hip_kv_quantize_affine(self.ctx.handle, _stream(), _ptr(source),
+                                               source_token_stride_elements, C.byref(destination), token_count,
+                                               element_count), "kv_quantize_affine")
+
+
+def rope_neox_subdim(ctx, data, rotary_dim, theta, positions=None, position=0):
+    """RoPE.encodeNeoxSubdim (RoPE.swift:48) in place on data[tokens, heads, head_dim]."""
+    tokens, heads, hd = data.shape
+    check(lib.nvmai_hip_rope_neox_subdim(ctx.handle, _stream(), _ptr(data), tokens, heads, hd, rotary_dim,
+                                         _ptr(positions), position, theta), "rope_neox_subdim")
+    return data
+
+
+class Attention:
+    """Mirror of Attention (Attention.swift): decode attention over a KV cache."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+
+    @staticmethod
+    def split_geometry(num_q_heads, num_kv_heads, seq_len, kv_start, prefer_gqa_swa):
+        """Attention.splitGeometry (Attention.swift:148-168)."""
+        vals = [C.c_uint32() for _ in range(4)]
+        check(lib.nvmai_attention_split_geometry(num_q_heads, num_kv_heads, seq_len, kv_start,
+                                                 int(prefer_gqa_swa), *[C.byref(x) for x in vals]),
+              "attention_split_geometry")
+        return tuple(x.value for x in vals)
+
+    def encode_full(self, q, k_cache, v_cache, head_dim, num_q_heads, num_kv_heads, seq_len, scale=None,
+                    kv_start=0, out=None):
+        """Attention.encodeFull (Attention.swift:207-239); q [batch, num_q_heads, head_dim]."""
+        batch = q.shape[0]
+        if out is None:
+            out = torch.empty_like(q)
+        kview, vview = k_cache.view(), v_cache.view()
+        check(lib.nvmai_hip_attention_decode(self.ctx.handle, _stream(), _ptr(q), C.byref(kview), C.byref(vview),
+                                             k_cache.batch_stride, _ptr(out), batch, head_dim, num_q_heads,
+                                             num_kv_heads, seq_len, kv_start, 0.0 if scale is None else scale),
+              "attention_decode")
+        return out
+
+    def encode_swa(self, q, k_cache, v_cache, head_dim, num_q_heads, num_kv_heads, seq_len, window, scale=None):
+        """Attention.encodeSWA (Attention.swift:170-205): the last `window` positions."""
+        return self.encode_full(q, k_cache, v_cache, head_dim, num_q_heads, num_kv_heads, seq_len, scale,
+                                kv_start=seq_len - window if seq_len > window else 0)
+
+
+# ---------------------------------------------------------------------------------------------
+# logits -> token
+# ---------------------------------------------------------------------------------------------
+def sampler_seed_for(seed, position):
+    """Sampler.seedFor (Sampler.swift:304-325)."""
+    return lib.nvmai_sampler_seed_for(seed, position)
+
+
+class LogitSoftcapSoftmaxTiled:
+    """Mirror of LogitSoftcapSoftmaxTiled (LogitOutput.swift:54-141)."""
+
+    def __init__(self, ctx, vocab):
+        if vocab <= 0:
+            raise _lib.NvmaiError(-1, "LogitSoftcapSoftmaxTiled(vocab)")
+        self.ctx, self.vocab = ctx, vocab
+
+    def encode(self, logits, probs=None, softcap=30.0):
+        z = logits.reshape(-1, logits.shape[-1])
+        if z.shape[1] != self.vocab:
+            raise _lib.NvmaiError(-1, "vocab mismatch: built for %d, got %d" % (self.vocab, z.shape[1]))
+        if probs is None:
+            probs = torch.empty(z.shape, dtype=torch.float16, device=z.device)
+        check(lib.nvmai_hip_softmax_tiled(self.ctx.handle, _stream(), _ptr(z), z.stride(0), _ptr(probs),
+                                          probs.stride(0), z.shape[0], self.vocab, softcap), "softmax_tiled")
+        return probs
+
+
+def _seed_array(seeds, rows):
+    seeds = [seeds] * rows if isinstance(seeds, int) else list(seeds)
+    return (C.c_uint64 * rows)(*[s & 0xFFFFFFFFFFFFFFFF for s in seeds])
+
+
+class SampleTopK64:
+    """Mirror of SampleTopK64 (LogitOutput.swift:202-333)."""
+
+    def __init__(self, ctx, vocab):
+        if not 0 < vocab <= 262144:
+            raise _lib.NvmaiError(-2, "SampleTopK64 unsupported vocabulary %d" % vocab)
+        self.ctx, self.vocab = ctx, vocab
+        g1 = (vocab + 1023) // 1024
+        g2 = (g1 * 64 + 1023) // 1024
+        self.scratch_bytes = (g1 * 64 + g2 * 64) * 8        # LogitOutput.swift:236-243
+
+    def encode(self, probs, temperature, top_p, seed, top_k=64, want_top64=False):
+        p = probs.reshape(-1, probs.shape[-1])
+        rows = p.shape[0]
+        out = torch.empty(rows, dtype=torch.int32, device=p.device)
+        top = torch.empty((rows, 64, 2), dtype=torch.int32, device=p.device) if want_top64 else None
+        check(lib.nvmai_hip_sample_topk64(self.ctx.handle, _stream(), _ptr(p), p.stride(0), rows, self.vocab,
+                                          temperature, top_p, _seed_array(seed, rows), top_k, _ptr(out), _ptr(top)),
+              "sample_topk64")
+        return (out, top) if want_top64 else out
+
+
+class Sample:
+    """Mirror of Sample (LogitOutput.swift:152-199): the generic sampler."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+
+    def encode(self, probs, temperature=1.0, top_k=0, top_p=1.0, seed=0):
+        p = probs.reshape(-1, probs.shape[-1])
+        rows = p.shape[0]
+        out = torch.empty(rows, dtype=torch.int32, device=p.device)
+        check(lib.nvmai_hip_sample(self.ctx.handle, _stream(), _ptr(p), p.stride(0), rows, p.shape[1], temperature,
+                                   top_k, top_p, _seed_array(seed, rows), _ptr(out)), "sample")
+        return out

@@ -1,0 +1,202 @@
+"""GPU parity: KV quantize-on-write (codes and fp16 scale/bias bits exact), partial RoPE and GQA
+decode attention over quantized K/V, through the C ABI against the CPU oracle.
+
+Attention bar: 16-bit output within 1e-2 of the oracle's attention over the SAME quantized rows
+(max|diff| / max|ref|, RelError.swift:5-16); and the reference's own bar against unquantized
+attention: 0.02 at 8 bits, 0.20 at 4 bits (KVCacheQuantizedAttentionTests.swift:71)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from gpu_util import act_np, act_tensor, dev, gauss, round_act, say
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def nv():
+    import nvmai_amd
+    return nvmai_amd
+
+
+@pytest.fixture(scope="module", params=[0, 1], ids=["bf16", "fp16"])
+def ctx(request, nv):
+    c = nv.Context(0, request.param)
+    yield c
+    torch.cuda.synchronize()
+    c.close()
+
+
+def test_row_layout_and_geometry_known_answers(nv):
+    # KVCacheQuantizedAttentionTests.swift:76-88, AttentionTests.swift:25-47
+    assert nv.kv_row_layout(512, 16) == (1024, 1024)
+    assert nv.kv_row_layout(512, 8) == (544, 512)
+    assert nv.kv_row_layout(512, 4) == (288, 256)
+    assert nv.Attention.split_geometry(16, 8, 1536, 512, True) == (1024, 16, 64, 128)
+    assert nv.Attention.split_geometry(16, 2, 1536, 0, False) == (1536, 16, 96, 256)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("elements,tokens", [(512, 37), (100, 3), (64, 1), (2048, 5)])
+def test_kv_quantize_codes_bit_exact(nv, ctx, bits, elements, tokens):
+    say("kv quantize", ctx.act, bits, elements, tokens)
+    rng = np.random.default_rng(elements + bits)
+    v = round_act(gauss(rng, (tokens, elements)), ctx.act)
+    v[0, :64] = 0.25                                   # flat group: scale 0, codes 0
+    if tokens > 2:
+        v[2, :] = v[2, 0]
+    src_stride = elements + 24                         # a padded source row, as the QKV stage buffer has
+    src = np.zeros((tokens, src_stride), np.float32)
+    src[:, :elements] = v
+    cache = nv.KVCache(1, tokens + 2, elements, bits)
+    nv.KVCacheQuantizer(ctx).encode(act_tensor(src, ctx), src_stride, cache.view(0, 1), tokens, elements)
+    torch.cuda.synchronize()
+    got = cache.rows[0].cpu().numpy()
+    want = O.kv_quantize(v, bits)
+    assert np.array_equal(got[1:1 + tokens], want)     # codes, fp16 scale bits, fp16 bias bits
+    assert not got[0].any() and not got[-1].any()      # neighbouring rows untouched
+
+
+def test_kv_quantize_rejects_bad_arguments(nv, ctx):
+    say("kv quantize errors")
+    cache = nv.KVCache(1, 4, 512, 16)
+    x = torch.zeros((1, 512), dtype=ctx.dtype, device="cuda")
+    with pytest.raises(nv.NvmaiError) as e:            # "KV quantizer requires 4-bit or 8-bit destination"
+        nv.KVCacheQuantizer(ctx).encode(x, 512, cache.view(), 1, 512)
+    assert e.value.name == "unsupported"
+    cache8 = nv.KVCache(1, 4, 512, 8)
+    with pytest.raises(nv.NvmaiError) as e:            # "source token stride is too small"
+        nv.KVCacheQuantizer(ctx).encode(x, 256, cache8.view(), 1, 512)
+    assert e.value.name == "invalid_arg"
+
+
+def test_rope_matches_oracle(nv, ctx):
+    say("rope", ctx.act)
+    rng = np.random.default_rng(3)
+    x = round_act(gauss(rng, (6, 16, 256)), ctx.act)
+    pos = np.array([0, 1, 17, 4095, 32767, 131071], np.uint32)
+    want = O.rope_neox_subdim(x, 64, pos, 1e7)
+    d = act_tensor(x, ctx)
+    nv.rope_neox_subdim(ctx, d, 64, 1e7, positions=dev(pos.view(np.int32)))
+    torch.cuda.synchronize()
+    got = act_np(d)
+    assert np.array_equal(got[..., 64:], x[..., 64:])                  # pass-through region untouched
+    assert np.array_equal(got[0], x[0])                                # position 0 is the identity
+    assert np.abs(got - round_act(want, ctx.act)).max() <= 2 ** -6     # one 16-bit ulp at |x| < 4
+    assert O.rel_error(got, want) < 1e-2
+    d2 = act_tensor(x[:2], ctx)
+    nv.rope_neox_subdim(ctx, d2, 64, 1e7, position=17)                 # the reference's single-position call
+    torch.cuda.synchronize()
+    want2 = O.rope_neox_subdim(x[:2], 64, np.array([17, 17], np.uint32), 1e7)
+    assert O.rel_error(act_np(d2), want2) < 1e-2
+
+
+def _attention_case(nv, ctx, rng, bits, batch, nq, nkv, hd, seq, kv_start=0, std=1.0, uniform=False):
+    elements = nkv * hd
+    mk = (lambda s: rng.uniform(-0.5, 0.5, s).astype(np.float32)) if uniform else (lambda s: gauss(rng, s, std))
+    q = round_act(mk((batch, nq, hd)), ctx.act)
+    k = round_act(mk((batch, seq, elements)), ctx.act)
+    v = round_act(mk((batch, seq, elements)), ctx.act)
+    kc, vc = nv.KVCache(batch, seq, elements, bits), nv.KVCache(batch, seq, elements, bits)
+    if bits == 16:
+        kc.rows.copy_(dev(k).to(torch.float16).view(torch.uint8).view(batch, seq, -1))
+        vc.rows.copy_(dev(v).to(torch.float16).view(torch.uint8).view(batch, seq, -1))
+    else:
+        quant = nv.KVCacheQuantizer(ctx)
+        for b in range(batch):
+            quant.encode(act_tensor(k[b], ctx), elements, kc.view(b), seq, elements)
+            quant.encode(act_tensor(v[b], ctx), elements, vc.view(b), seq, elements)
+    out = nv.Attention(ctx).encode_full(act_tensor(q, ctx), kc, vc, hd, nq, nkv, seq, scale=None, kv_start=kv_start)
+    torch.cuda.synchronize()
+    got = act_np(out)
+    scale = 1.0 / np.sqrt(hd)
+    for b in range(batch):
+        if bits == 16:
+            k16 = O.f16_to_float(O.f16_bits(k[b]))
+            v16 = O.f16_to_float(O.f16_bits(v[b]))
+            want = O.attention_decode(q[b], k16, v16, 32, nq, nkv, hd, seq, scale, kv_start)
+        else:
+            kq, vq = kc.rows[b].cpu().numpy(), vc.rows[b].cpu().numpy()
+            assert np.array_equal(kq, O.kv_quantize(k[b], bits))       # KV codes bit-exact
+            want = O.attention_decode(q[b], kq, vq, bits, nq, nkv, hd, seq, scale, kv_start)
+        err = O.rel_error(got[b], want)
+        assert err < 1e-2, "batch %d rel %g" % (b, err)
+    return got, q, k, v
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_attention_production_shape(nv, ctx, bits):
+    # configs[3]: 16 query heads, 2 KV heads, head_dim 256; ragged lengths exercise the tails
+    rng = np.random.default_rng(bits)
+    for batch, seq, kv_start in [(1, 8, 0), (1, 1, 0), (2, 33, 0), (1, 127, 0), (1, 128, 0), (3, 1000, 0),
+                                 (1, 4096, 0), (2, 2048, 1024), (1, 300, 299)]:
+        say("attention mfma", ctx.act, bits, batch, seq, kv_start)
+        _attention_case(nv, ctx, rng, bits, batch, 16, 2, 256, seq, kv_start)
+
+
+def test_attention_tracks_unquantized_reference(nv, ctx):
+    # KVCacheQuantizedAttentionTests.swift:7-74: seq 8, uniform(-0.5, 0.5)
+    for bits, tol in ((8, 0.02), (4, 0.20)):
+        say("attention vs unquantized", ctx.act, bits)
+        rng = np.random.default_rng(0x4B56 + bits)
+        got, q, k, v = _attention_case(nv, ctx, rng, bits, 1, 16, 2, 256, 8, uniform=True)
+        want = O.attention_decode(q[0], k[0], v[0], 32, 16, 2, 256, 8, 1 / 16.0)
+        assert O.rel_error(got[0], want) < tol
+
+
+@pytest.mark.parametrize("bits", [16, 8, 4])
+def test_attention_other_shapes_generic_path(nv, ctx, bits):
+    rng = np.random.default_rng(10 + bits)
+    for batch, nq, nkv, hd, seq, kv_start in [(1, 4, 2, 64, 19, 0), (2, 8, 8, 128, 70, 0), (1, 16, 8, 256, 40, 8),
+                                              (1, 2, 1, 512, 9, 0), (1, 4, 4, 96, 5, 0)]:
+        say("attention generic", ctx.act, bits, batch, nq, nkv, hd, seq, kv_start)
+        _attention_case(nv, ctx, rng, bits, batch, nq, nkv, hd, seq, kv_start)
+
+
+def test_attention_empty_range_and_errors(nv, ctx):
+    say("attention empty range")
+    kc, vc = nv.KVCache(1, 8, 512, 8), nv.KVCache(1, 8, 512, 8)
+    q = torch.ones((1, 16, 256), dtype=ctx.dtype, device="cuda")
+    out = nv.Attention(ctx).encode_full(q, kc, vc, 256, 16, 2, 8, kv_start=8)       # attention.metal:410-416
+    torch.cuda.synchronize()
+    assert not act_np(out).any()
+    with pytest.raises(nv.NvmaiError) as e:            # numQHeads must be a multiple of numKVHeads
+        nv.Attention(ctx).encode_full(q, kc, vc, 256, 15, 2, 8)
+    assert e.value.name == "invalid_arg"
+
+
+def test_attention_long_context_properties(nv):
+    # 32K context: too slow for the scalar oracle in full, so (a) one head group against the oracle
+    # and (b) size-independent properties: permuting the KV positions changes nothing, and a cache
+    # whose V rows are all equal returns that row.
+    say("attention 32K")
+    ctx = nv.Context(0, 0)
+    rng = np.random.default_rng(99)
+    nq, nkv, hd, seq, bits = 16, 2, 256, 32768, 8
+    q = O.round_bf16(gauss(rng, (1, nq, hd)))
+    k = torch.randn((seq, nkv * hd), device="cuda").to(torch.bfloat16)
+    v = torch.randn((seq, nkv * hd), device="cuda").to(torch.bfloat16)
+    kc, vc = nv.KVCache(1, seq, nkv * hd, bits), nv.KVCache(1, seq, nkv * hd, bits)
+    quant, attn = nv.KVCacheQuantizer(ctx), nv.Attention(ctx)
+    quant.encode(k, nkv * hd, kc.view(), seq, nkv * hd)
+    quant.encode(v, nkv * hd, vc.view(), seq, nkv * hd)
+    qd = act_tensor(q, ctx)
+    out = attn.encode_full(qd, kc, vc, hd, nq, nkv, seq)
+    perm = torch.randperm(seq, device="cuda")
+    kc2, vc2 = nv.KVCache(1, seq, nkv * hd, bits), nv.KVCache(1, seq, nkv * hd, bits)
+    kc2.rows[0] = kc.rows[0][perm]
+    vc2.rows[0] = vc.rows[0][perm]
+    out2 = attn.encode_full(qd, kc2, vc2, hd, nq, nkv, seq)
+    vc3 = nv.KVCache(1, seq, nkv * hd, bits)
+    vc3.rows[0] = vc.rows[0][:1].expand(seq, -1)
+    out3 = attn.encode_full(qd, kc, vc3, hd, nq, nkv, seq)
+    torch.cuda.synchronize()
+    assert O.rel_error(act_np(out2), act_np(out)) < 1e-2
+    row0 = O.kv_dequant(vc.rows[0][:1].cpu().numpy(), nkv * hd, bits)[0].reshape(nkv, hd)
+    assert np.abs(act_np(out3)[0].reshape(nkv, 8, hd) - row0[:, None, :]).max() < 2e-2
+    want = O.attention_decode(q[0], kc.rows[0].cpu().numpy(), vc.rows[0].cpu().numpy(), bits, nq, nkv, hd, seq,
+                              1 / 16.0)
+    assert O.rel_error(act_np(out)[0], want) < 1e-2
+    torch.cuda.synchronize()
+    ctx.close()

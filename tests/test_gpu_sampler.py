@@ -1,0 +1,131 @@
+"""GPU parity: tiled softmax and the top-64 / generic samplers through the C ABI.
+
+Token ids are integer-class given identical fp16 probabilities: the GPU samplers read the same
+probability buffer as the oracle and must return the same token."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from gpu_util import act_np, act_tensor, dev, gauss, round_act, say, u16, u32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def nv():
+    import nvmai_amd
+    return nvmai_amd
+
+
+@pytest.fixture(scope="module", params=[0, 1], ids=["bf16", "fp16"])
+def ctx(request, nv):
+    c = nv.Context(0, request.param)
+    yield c
+    torch.cuda.synchronize()
+    c.close()
+
+
+def _probs_dev(p_bits):
+    return dev(np.ascontiguousarray(p_bits).view(np.float16))
+
+
+@pytest.mark.parametrize("v", [1003, 4096, 248320])
+def test_softmax_tiled_matches_oracle(nv, ctx, v):
+    say("softmax", ctx.act, v)
+    rng = np.random.default_rng(v)
+    logits = round_act(gauss(rng, (3, v), 4.0), ctx.act)
+    sm = nv.LogitSoftcapSoftmaxTiled(ctx, v)
+    for softcap in (0.0, 30.0):
+        got = u16(sm.encode(act_tensor(logits, ctx), softcap=softcap))
+        torch.cuda.synchronize()
+        for r in range(3):
+            want = O.softmax_f16(logits[r], softcap)
+            assert np.abs(got[r].astype(np.int32) - want.astype(np.int32)).max() <= 2       # fp16 ulps
+            p = O.f16_to_float(got[r]).astype(np.float64)
+            assert abs(p.sum() - 1.0) < 2e-3
+    with pytest.raises(nv.NvmaiError):                       # "vocab mismatch: built for ..."
+        sm.encode(act_tensor(logits[:, :v - 1], ctx))
+
+
+def _lcg_probs(v):
+    i = np.arange(v, dtype=np.uint64)
+    mixed = i * np.uint64(6364136223846793005) + np.uint64(1442695040888963407)
+    p = ((mixed >> np.uint64(40)).astype(np.uint32).astype(np.float32) + np.float32(1)) * np.float32(1.0 / 16777217.0)
+    return O.f16_bits(p)
+
+
+def test_top64_candidates_and_tokens_on_reference_input(nv, ctx):
+    # SampleTopK64Tests.swift:115-130, 168-187: production vocabulary, LCG probabilities
+    say("sampler lcg", ctx.act)
+    v = 262144
+    probs = _lcg_probs(v)
+    pd = _probs_dev(probs)
+    tk = nv.SampleTopK64(ctx, v)
+    assert tk.scratch_bytes == 139264                        # SampleTopK64Tests.swift:117
+    gen = nv.Sample(ctx)
+    tok, top = tk.encode(pd, 1.0, 0.95, 1, 64, want_top64=True)
+    torch.cuda.synchronize()
+    _, idx, val = O.sample_topk64(probs, 1.0, 0.95, 1, 64, want_top64=True)
+    top = top.cpu().numpy().view(np.uint32)[0]
+    assert np.array_equal(top[:, 1], idx) and np.array_equal(top[:, 0], val.view(np.uint32))
+    for k in (1, 2, 7, 20, 33, 63, 64):
+        for t in (0.6, 0.7, 1.0):
+            for seed in (1, 42, 0x123456789ABCDEF0, 2 ** 64 - 1):
+                want = O.sample_topk64(probs, t, 0.95, seed, k)
+                a = int(tk.encode(pd, t, 0.95, seed, k)[0]) & 0xFFFFFFFF
+                assert a == want, (k, t, seed)
+    for k, t, seed in [(1, 0.6, 1), (20, 0.6, 42), (64, 1.0, 7)]:        # generic == tiled, token for token
+        b = int(gen.encode(pd, t, k, 0.95, seed)[0]) & 0xFFFFFFFF
+        assert b == O.sample_generic(probs, t, k, 0.95, seed) == O.sample_topk64(probs, t, 0.95, seed, k)
+
+
+def test_sampler_ties_flat_geometric_and_greedy(nv, ctx):
+    say("sampler small cases", ctx.act)
+    v = 1003
+    tk, gen = nv.SampleTopK64(ctx, v), nv.Sample(ctx)
+    ones = O.f16_bits(np.ones(v, np.float32))
+    flat = O.f16_bits(np.full(v, 1.0 / v, np.float32))
+    geo = np.zeros(v, np.float32)
+    geo[:128] = (0.85 ** np.arange(128)).astype(np.float32)
+    geo = O.f16_bits(geo)
+    for name, probs, ks in (("ones", ones, (64,)), ("flat", flat, (64,)), ("geo", geo, (3, 8, 20, 64))):
+        pd = _probs_dev(probs)
+        for k in ks:
+            rows = 16
+            seeds = [s * 7919 + 1 for s in range(rows)]
+            batch = tk.encode(pd.expand(rows, -1).contiguous(), 1.0, 0.95, seeds, k).cpu().numpy().view(np.uint32)
+            gbatch = gen.encode(pd.expand(rows, -1).contiguous(), 1.0, k, 0.95, seeds).cpu().numpy().view(np.uint32)
+            for r, seed in enumerate(seeds):
+                want = O.sample_topk64(probs, 1.0, 0.95, seed, k)
+                assert batch[r] == want == gbatch[r], (name, k, seed)
+                assert want < 64 and (name != "geo" or want < k)
+    p = np.zeros(512, np.float32)
+    p[[10, 20, 30]] = [0.5, 0.25, 0.25]
+    pd = _probs_dev(O.f16_bits(p))
+    assert int(gen.encode(pd, 0.0, 20, 0.95, 1)[0]) == 10                  # greedy argmax
+    tie = np.zeros(512, np.float32)
+    tie[[40, 7, 300]] = 0.3
+    assert int(gen.encode(_probs_dev(O.f16_bits(tie)), 0.0)[0]) == 7       # lowest index wins a tie
+    with pytest.raises(nv.NvmaiError):                                     # temperature must be > 0
+        nv.SampleTopK64(ctx, 512).encode(pd, 0.0, 0.95, 1, 20)
+    with pytest.raises(nv.NvmaiError):                                     # k in 1...64
+        nv.SampleTopK64(ctx, 512).encode(pd, 1.0, 0.95, 1, 65)
+    with pytest.raises(nv.NvmaiError):                                     # unsupportedVocabulary
+        nv.SampleTopK64(ctx, 262145)
+
+
+def test_softmax_then_sampler_pipeline(nv, ctx):
+    # configs[4] tail: logits over 248,320 entries -> softmax -> top-k 20, top-p 0.95, T 0.6, fixed seed
+    say("softmax+sampler pipeline", ctx.act)
+    v = 248320
+    rng = np.random.default_rng(5)
+    logits = round_act(gauss(rng, (2, v), 3.0), ctx.act)
+    probs = nv.LogitSoftcapSoftmaxTiled(ctx, v).encode(act_tensor(logits, ctx), softcap=0.0)
+    seeds = [nv.sampler_seed_for(1234, pos) for pos in (0, 1)]
+    assert seeds == [O.seed_for(1234, 0), O.seed_for(1234, 1)]
+    tok = nv.SampleTopK64(ctx, v).encode(probs, 0.6, 0.95, seeds, 20).cpu().numpy().view(np.uint32)
+    torch.cuda.synchronize()
+    ph = u16(probs)
+    for r in range(2):
+        assert tok[r] == O.sample_topk64(ph[r], 0.6, 0.95, seeds[r], 20)
