@@ -186,6 +186,90 @@ int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream stream, const nv
                                uint32_t* stats);
 
 
+/* ---- prefill: permutation by expert and grouped expert GEMM ------------------------------- */
+
+/* PrefillTokenExpertPair (PrefillRouter.swift:5-28 == prefill.metal:220-225): 16 bytes;
+ * weight_bits holds the FP16 routing weight in its low 16 bits. */
+typedef struct { uint32_t token, expert, rank, weight_bits; } nvmai_prefill_pair;
+/* PrefillMoEGroup / PrefillMoETile (PrefillMoEGrouping.swift:4-29). */
+typedef struct { uint32_t expert, pair_start, pair_count; } nvmai_prefill_group;
+typedef struct { uint32_t group_start, group_count, pair_start, pair_count; } nvmai_prefill_tile;
+
+/* PrefillMoEGroupingError (PrefillMoEGrouping.swift:52-89), numbered in declaration order. */
+typedef enum {
+    NVMAI_GROUPING_OK = 0, NVMAI_GROUPING_INVALID_QUERY_COUNT = 1, NVMAI_GROUPING_INVALID_TOP_K = 2,
+    NVMAI_GROUPING_INVALID_NUM_EXPERTS = 3, NVMAI_GROUPING_INVALID_TILE_EXPERT_COUNT = 4,
+    NVMAI_GROUPING_PAIR_COUNT_MISMATCH = 5, NVMAI_GROUPING_TOKEN_OUT_OF_RANGE = 6,
+    NVMAI_GROUPING_RANK_OUT_OF_RANGE = 7, NVMAI_GROUPING_EXPERT_OUT_OF_RANGE = 8,
+    NVMAI_GROUPING_DUPLICATE_TOKEN_RANK = 9, NVMAI_GROUPING_SORT_KEY_COUNT_MISMATCH = 10
+} nvmai_grouping_error;
+
+/* PrefillMoEGroupedRoutes (PrefillMoEGrouping.swift:31-50) as caller-owned DEVICE arrays:
+ * sorted_pairs [n_pairs]; expert_offsets / expert_counts [num_experts] (offset 0xFFFFFFFF for
+ * an expert without pairs); groups and tiles [num_experts] of which info[0] / info[1] are
+ * filled.  info is u32[8]: {groups, tiles, nvmai_grouping_error found on the device (6..9 or
+ * 0), index of the first failing pair, largest group, 0, 0, 0}. */
+typedef struct {
+    nvmai_prefill_pair* sorted_pairs;
+    uint32_t* expert_offsets;
+    uint32_t* expert_counts;
+    nvmai_prefill_group* groups;
+    nvmai_prefill_tile* tiles;
+    uint32_t* info;
+} nvmai_prefill_grouping;
+
+/* The argument checks groupTokenExpertPairs makes before it looks at a pair
+ * (PrefillMoEGrouping.swift:99-119); host only.  Returns a nvmai_grouping_error. */
+int nvmai_prefill_grouping_check(int64_t n_pairs, int64_t query_count, int64_t top_k, int64_t num_experts,
+                                 int64_t tile_expert_count, int has_sort_keys, int64_t n_sort_keys);
+
+/* PrefillRouter.makeTokenExpertPairs (PrefillRouter.swift:97-117): token-major pair records
+ * from the router's idx [tokens, top_k] u32 and w [tokens, top_k] FP16. */
+int nvmai_hip_prefill_make_pairs(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint32_t* idx,
+                                 const uint16_t* w, uint32_t tokens, uint32_t top_k,
+                                 nvmai_prefill_pair* pairs);
+
+/* PrefillMoEGrouping.groupTokenExpertPairs (PrefillMoEGrouping.swift:91-192) on the device:
+ * pairs in any order -> pairs sorted by (sort key of the expert, expert, token, rank), the
+ * per-expert offsets and counts, the groups and the tiles of <= tile_expert_count groups.
+ * sort_keys: optional device u64 [num_experts].  A failing nvmai_prefill_grouping_check
+ * returns NVMAI_ERR_INVALID_ARG; per-pair failures are found on the device and land in
+ * info[2..3] (the arrays are then unspecified but every index in them is in range). */
+int nvmai_hip_prefill_group_pairs(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_prefill_pair* pairs,
+                                  uint64_t n_pairs, uint32_t query_count, uint32_t top_k,
+                                  uint32_t num_experts, uint32_t tile_expert_count,
+                                  const uint64_t* sort_keys, uint64_t n_sort_keys,
+                                  const nvmai_prefill_grouping* out);
+
+/* makeTokenExpertPairs + groupTokenExpertPairs in one step, straight from the router's
+ * idx / w (RealPrefillRunner's use of the two, without the host round trip between). */
+int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint32_t* idx,
+                                   const uint16_t* w, uint32_t query_count, uint32_t top_k,
+                                   uint32_t num_experts, uint32_t tile_expert_count,
+                                   const uint64_t* sort_keys, uint64_t n_sort_keys,
+                                   const nvmai_prefill_grouping* out);
+
+/* PrefillGroupedRoutedMoE.encodeStreamedBatched over every tile
+ * (PrefillGroupedRoutedMoE.swift:413-489; kernels prefill.metal:460-534) with all experts
+ * resident: act[p, :] = silu(gate_e x_token(p)) * (up_e x_token(p)) for sorted pair p, then
+ * route_partials[token*top_k + rank, :] = down_e act[p, :], both rounded to the activation
+ * type.  hidden [query_count, hidden_stride]; act_scratch [n_pairs, f] and route_partials
+ * [n_pairs, d] are caller-owned, 16-bit.  d and f must be multiples of 64. */
+int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* experts_base,
+                                  uint64_t expert_stride, const nvmai_expert_offsets* off, uint32_t bits,
+                                  uint32_t d, uint32_t f, uint32_t num_experts, const void* hidden,
+                                  uint32_t hidden_stride, uint32_t query_count, uint32_t top_k,
+                                  const nvmai_prefill_grouping* grouping, void* act_scratch,
+                                  void* route_partials);
+
+/* PrefillMoE.encodeReduceTokenMajor (PrefillMoE.swift:11-40; prefill.metal:437-458):
+ * h2[t, :] = sum over ranks, in rank order, of fma(w[t, r], route_partials[t*top_k + r, :]). */
+int nvmai_hip_prefill_moe_reduce_token_major(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                             const void* route_partials, const uint16_t* route_weights,
+                                             void* h2, uint32_t h2_stride, uint32_t query_count,
+                                             uint32_t top_k, uint32_t d);
+
+
 /* ---- KV cache -------------------------------------------------------------------------- */
 
 /* KVCacheManager.rowLayout (KVCacheManager.swift:437-446): bytes per token row and bytes of

@@ -50,6 +50,11 @@ class KvView(C.Structure):
     _fields_ = [("base", vp), ("stride", u32), ("value_bytes", u32), ("bits", u32), ("group_size", u32)]
 
 
+class PrefillGrouping(C.Structure):
+    """nvmai_prefill_grouping"""
+    _fields_ = [(n, vp) for n in ("sorted_pairs", "expert_offsets", "expert_counts", "groups", "tiles", "info")]
+
+
 # name -> argtypes (every function returns int unless listed in _OTHER)
 SIGNATURES = {
     "nvmai_hip_ctx_create": [C.c_int, C.c_int, C.POINTER(vp)],
@@ -79,6 +84,13 @@ SIGNATURES = {
                                        C.POINTER(u32), C.POINTER(u32)],
     "nvmai_hip_softmax_tiled": [vp, vp, vp, u32, vp, u32, u32, u32, C.c_float],
     "nvmai_hip_sample_topk64": [vp, vp, vp, u32, u32, u32, C.c_float, C.c_float, C.POINTER(u64), u32, vp, vp],
+    "nvmai_prefill_grouping_check": [C.c_int64] * 5 + [C.c_int, C.c_int64],
+    "nvmai_hip_prefill_make_pairs": [vp, vp, vp, vp, u32, u32, vp],
+    "nvmai_hip_prefill_group_pairs": [vp, vp, vp, u64, u32, u32, u32, u32, vp, u64, C.POINTER(PrefillGrouping)],
+    "nvmai_hip_prefill_group_routes": [vp, vp, vp, vp, u32, u32, u32, u32, vp, u64, C.POINTER(PrefillGrouping)],
+    "nvmai_hip_prefill_grouped_moe": [vp, vp, vp, u64, C.POINTER(ExpertOffsets), u32, u32, u32, u32, vp, u32,
+                                      u32, u32, C.POINTER(PrefillGrouping), vp, vp],
+    "nvmai_hip_prefill_moe_reduce_token_major": [vp, vp, vp, vp, vp, u32, u32, u32, u32],
     "nvmai_hip_sample": [vp, vp, vp, u32, u32, u32, C.c_float, u32, C.c_float, C.POINTER(u64), vp],
 }
 _OTHER = {

@@ -1,0 +1,219 @@
+// Entry points: token-expert pairs, grouping by expert, grouped expert GEMMs, rank-order reduce.
+#include "ctx.hpp"
+#include "prefill_kernels.cuh"
+
+using namespace nvmai;
+
+static_assert(sizeof(nvmai_prefill_pair) == sizeof(PrefillPair) && sizeof(nvmai_prefill_group) == sizeof(PrefillGroup) &&
+                  sizeof(nvmai_prefill_tile) == sizeof(PrefillTile),
+              "C-ABI records and kernel records must agree");
+
+extern "C" int nvmai_prefill_grouping_check(int64_t n_pairs, int64_t query_count, int64_t top_k,
+                                            int64_t num_experts, int64_t tile_expert_count, int has_sort_keys,
+                                            int64_t n_sort_keys) {
+    if (query_count < 0) return NVMAI_GROUPING_INVALID_QUERY_COUNT;
+    if (top_k <= 0) return NVMAI_GROUPING_INVALID_TOP_K;
+    if (num_experts <= 0) return NVMAI_GROUPING_INVALID_NUM_EXPERTS;
+    if (tile_expert_count < 1 || tile_expert_count > 16) return NVMAI_GROUPING_INVALID_TILE_EXPERT_COUNT;
+    if (has_sort_keys && n_sort_keys != num_experts) return NVMAI_GROUPING_SORT_KEY_COUNT_MISMATCH;
+    if (n_pairs != query_count * top_k) return NVMAI_GROUPING_PAIR_COUNT_MISMATCH;
+    return NVMAI_GROUPING_OK;
+}
+
+extern "C" int nvmai_hip_prefill_make_pairs(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint32_t* idx,
+                                            const uint16_t* w, uint32_t tokens, uint32_t top_k,
+                                            nvmai_prefill_pair* pairs) {
+    if (!ctx || !idx || !w || !pairs || top_k == 0) return NVMAI_ERR_INVALID_ARG;
+    const uint64_t n = (uint64_t)tokens * top_k;
+    if (n >= (1u << 28)) return NVMAI_ERR_INVALID_ARG;
+    if (n == 0) return NVMAI_OK;
+    prefill_make_pairs_kernel<<<(uint32_t)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+        idx, w, (uint32_t)n, top_k, reinterpret_cast<PrefillPair*>(pairs));
+    return launch_status();
+}
+
+namespace {
+
+constexpr uint32_t MAX_GROUP_EXPERTS = 4096;   // three u32 arrays of the scan kernel in 48 KB of LDS
+
+int check_grouping(const nvmai_prefill_grouping* g, uint64_t n_pairs) {
+    if (!g || (n_pairs && !g->sorted_pairs) || !g->expert_offsets || !g->expert_counts || !g->groups || !g->tiles || !g->info)
+        return NVMAI_ERR_INVALID_ARG;
+    return NVMAI_OK;
+}
+
+// Shared tail: histogram, scan, scatter over slot-ordered expert ids.
+int group_slots(nvmai_hip_ctx* ctx, hipStream_t s, const uint32_t* slot_expert, const uint32_t* w32,
+                const uint16_t* w16, uint32_t n_pairs, uint32_t top_k, uint32_t num_experts,
+                uint32_t tile_expert_count, const uint64_t* sort_keys, uint32_t* block_hist, uint32_t* words,
+                bool report_range, const nvmai_prefill_grouping* out) {
+    const uint32_t n_blocks = (n_pairs + GROUP_CHUNK - 1) / GROUP_CHUNK;
+    if (n_blocks)
+        prefill_hist_kernel<<<n_blocks, 256, num_experts * 4, s>>>(slot_expert, n_pairs, num_experts, block_hist, words,
+                                                                  report_range);
+    prefill_scan_kernel<<<1, 1024, 3 * num_experts * 4, s>>>(
+        block_hist, n_blocks, num_experts, sort_keys, tile_expert_count, out->expert_offsets, out->expert_counts,
+        reinterpret_cast<PrefillGroup*>(out->groups), reinterpret_cast<PrefillTile*>(out->tiles), words, out->info);
+    if (n_blocks)
+        prefill_scatter_kernel<<<n_blocks, 256, GROUP_CHUNK * 4, s>>>(slot_expert, w32, w16, n_pairs, top_k, num_experts,
+                                                                    block_hist, reinterpret_cast<PrefillPair*>(out->sorted_pairs));
+    return launch_status();
+}
+
+}  // namespace
+
+extern "C" int nvmai_hip_prefill_group_pairs(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                             const nvmai_prefill_pair* pairs, uint64_t n_pairs,
+                                             uint32_t query_count, uint32_t top_k, uint32_t num_experts,
+                                             uint32_t tile_expert_count, const uint64_t* sort_keys,
+                                             uint64_t n_sort_keys, const nvmai_prefill_grouping* out) {
+    if (!ctx || (n_pairs && !pairs)) return NVMAI_ERR_INVALID_ARG;
+    int rc = check_grouping(out, n_pairs);
+    if (rc) return rc;
+    if (nvmai_prefill_grouping_check((int64_t)n_pairs, query_count, top_k, num_experts, tile_expert_count,
+                                     sort_keys != nullptr, (int64_t)n_sort_keys) != NVMAI_GROUPING_OK)
+        return NVMAI_ERR_INVALID_ARG;
+    if (n_pairs >= (1u << 28) || num_experts > MAX_GROUP_EXPERTS) return NVMAI_ERR_UNSUPPORTED;
+    const uint32_t n = (uint32_t)n_pairs, n_blocks = (n + GROUP_CHUNK - 1) / GROUP_CHUNK;
+    rc = ws_begin(ctx, 3 * ws_round((size_t)n * 4) + ws_round((size_t)n_blocks * num_experts * 4) + ws_round(64));
+    if (rc) return rc;
+    uint32_t* first = ws_take<uint32_t>(ctx, n);
+    uint32_t* slot_expert = ws_take<uint32_t>(ctx, n);
+    uint32_t* slot_weight = ws_take<uint32_t>(ctx, n);
+    uint32_t* block_hist = ws_take<uint32_t>(ctx, (size_t)n_blocks * num_experts);
+    uint32_t* words = ws_take<uint32_t>(ctx, 16);
+    hipStream_t s = (hipStream_t)stream;
+    ProfScope prof(ctx, NVMAI_PROF_PREFILL_GROUP, s);
+    const uint32_t grid = n ? (n + 255) / 256 : 1;
+    prefill_init_kernel<<<grid, 256, 0, s>>>(first, n, words);
+    if (n) {
+        prefill_claim_kernel<<<grid, 256, 0, s>>>(reinterpret_cast<const PrefillPair*>(pairs), n, query_count, top_k,
+                                                  num_experts, first, words);
+        prefill_slot_kernel<<<grid, 256, 0, s>>>(reinterpret_cast<const PrefillPair*>(pairs), n, query_count, top_k,
+                                                 num_experts, first, slot_expert, slot_weight, words);
+    }
+    return group_slots(ctx, s, slot_expert, slot_weight, nullptr, n, top_k, num_experts, tile_expert_count, sort_keys,
+                       block_hist, words, false, out);
+}
+
+extern "C" int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint32_t* idx,
+                                              const uint16_t* w, uint32_t query_count, uint32_t top_k,
+                                              uint32_t num_experts, uint32_t tile_expert_count,
+                                              const uint64_t* sort_keys, uint64_t n_sort_keys,
+                                              const nvmai_prefill_grouping* out) {
+    const uint64_t n_pairs = (uint64_t)query_count * top_k;
+    if (!ctx || (n_pairs && (!idx || !w))) return NVMAI_ERR_INVALID_ARG;
+    int rc = check_grouping(out, n_pairs);
+    if (rc) return rc;
+    if (nvmai_prefill_grouping_check((int64_t)n_pairs, query_count, top_k, num_experts, tile_expert_count,
+                                     sort_keys != nullptr, (int64_t)n_sort_keys) != NVMAI_GROUPING_OK)
+        return NVMAI_ERR_INVALID_ARG;
+    if (n_pairs >= (1u << 28) || num_experts > MAX_GROUP_EXPERTS) return NVMAI_ERR_UNSUPPORTED;
+    const uint32_t n = (uint32_t)n_pairs, n_blocks = (n + GROUP_CHUNK - 1) / GROUP_CHUNK;
+    rc = ws_begin(ctx, ws_round((size_t)n_blocks * num_experts * 4) + ws_round(64));
+    if (rc) return rc;
+    uint32_t* block_hist = ws_take<uint32_t>(ctx, (size_t)n_blocks * num_experts);
+    uint32_t* words = ws_take<uint32_t>(ctx, 16);
+    hipStream_t s = (hipStream_t)stream;
+    ProfScope prof(ctx, NVMAI_PROF_PREFILL_GROUP, s);
+    prefill_init_kernel<<<1, 256, 0, s>>>(nullptr, 0, words);
+    return group_slots(ctx, s, idx, nullptr, w, n, top_k, num_experts, tile_expert_count, sort_keys, block_hist, words, true,
+                       out);
+}
+
+namespace {
+
+template <int ACT, int BITS>
+void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t max_mtiles, nvmai_hip_ctx* ctx, hipStream_t s) {
+    const size_t lds = (size_t)4 * GEMM_BM * GEMM_LDK * 2;     // 72 KB: above the 64 KB a launch gets unasked
+    static bool raised = false;
+    if (!raised) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, false>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        raised = true;
+    }
+    {
+        ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM1, s);
+        prefill_gemm_kernel<ACT, BITS, true><<<max_mtiles * g1.n_tiles_n, 256, lds, s>>>(g1);
+    }
+    {
+        ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM2, s);
+        prefill_gemm_kernel<ACT, BITS, false><<<max_mtiles * g2.n_tiles_n, 256, lds, s>>>(g2);
+    }
+}
+
+}  // namespace
+
+extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* experts_base,
+                                             uint64_t expert_stride, const nvmai_expert_offsets* off,
+                                             uint32_t bits, uint32_t d, uint32_t f, uint32_t num_experts,
+                                             const void* hidden, uint32_t hidden_stride, uint32_t query_count,
+                                             uint32_t top_k, const nvmai_prefill_grouping* grouping,
+                                             void* act_scratch, void* route_partials) {
+    if (!ctx || !experts_base || !off || !hidden || !act_scratch || !route_partials) return NVMAI_ERR_INVALID_ARG;
+    int rc = check_grouping(grouping, (uint64_t)query_count * top_k);
+    if (rc) return rc;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    if (d == 0 || f == 0 || d % NVMAI_GROUP || f % NVMAI_GROUP || top_k == 0 || num_experts == 0 ||
+        hidden_stride < d)
+        return NVMAI_ERR_INVALID_ARG;
+    const uint32_t offs[9] = {off->gate_w, off->gate_s, off->gate_b, off->up_w, off->up_s, off->up_b,
+                              off->down_w, off->down_s, off->down_b};
+    for (int i = 0; i < 9; ++i)
+        if (offs[i] % (i % 3 == 0 ? 16 : 2)) return NVMAI_ERR_ALIGNMENT;
+    if (!aligned16(experts_base) || expert_stride % 16 || !aligned16(hidden) || hidden_stride % 8 ||
+        !aligned16(act_scratch) || !aligned16(route_partials))
+        return NVMAI_ERR_ALIGNMENT;
+    const uint64_t n_pairs = (uint64_t)query_count * top_k;
+    if (n_pairs >= (1u << 28)) return NVMAI_ERR_UNSUPPORTED;
+    if (n_pairs == 0) return NVMAI_OK;
+    const uint32_t max_mtiles = (uint32_t)(n_pairs / GEMM_BM) + (num_experts < n_pairs ? num_experts : (uint32_t)n_pairs);
+    rc = ws_begin(ctx, ws_round((size_t)max_mtiles * sizeof(MTile)) + ws_round(64));
+    if (rc) return rc;
+    MTile* mtiles = ws_take<MTile>(ctx, max_mtiles);
+    uint32_t* n_mtiles = ws_take<uint32_t>(ctx, 16);
+    hipStream_t s = (hipStream_t)stream;
+    prefill_mtiles_kernel<<<1, 256, 0, s>>>(reinterpret_cast<const PrefillGroup*>(grouping->groups), grouping->info,
+                                            mtiles, n_mtiles);
+    GemmParams g1{};
+    g1.pool = (const uint8_t*)experts_base; g1.pool_stride = expert_stride;
+    g1.wA = off->gate_w; g1.sA = off->gate_s; g1.bA = off->gate_b;
+    g1.wB = off->up_w; g1.sB = off->up_s; g1.bB = off->up_b;
+    g1.mtiles = mtiles; g1.n_mtiles = n_mtiles;
+    g1.pairs = reinterpret_cast<const PrefillPair*>(grouping->sorted_pairs);
+    g1.x = hidden; g1.x_stride = hidden_stride;
+    g1.out = act_scratch; g1.out_stride = f;
+    g1.K = d; g1.N = f; g1.top_k = top_k; g1.n_tiles_n = (f + 63) / 64;
+    GemmParams g2 = g1;
+    g2.wA = off->down_w; g2.sA = off->down_s; g2.bA = off->down_b;
+    g2.wB = g2.sB = g2.bB = 0;
+    g2.x = act_scratch; g2.x_stride = f;
+    g2.out = route_partials; g2.out_stride = d;
+    g2.K = f; g2.N = d; g2.n_tiles_n = (d + 127) / 128;
+    if (ctx->act == ACT_BF16) {
+        if (bits == 4) launch_gemms<ACT_BF16, 4>(g1, g2, max_mtiles, ctx, s);
+        else launch_gemms<ACT_BF16, 8>(g1, g2, max_mtiles, ctx, s);
+    } else {
+        if (bits == 4) launch_gemms<ACT_FP16, 4>(g1, g2, max_mtiles, ctx, s);
+        else launch_gemms<ACT_FP16, 8>(g1, g2, max_mtiles, ctx, s);
+    }
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_prefill_moe_reduce_token_major(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                                        const void* route_partials, const uint16_t* route_weights,
+                                                        void* h2, uint32_t h2_stride, uint32_t query_count,
+                                                        uint32_t top_k, uint32_t d) {
+    if (!ctx || !route_partials || !route_weights || !h2) return NVMAI_ERR_INVALID_ARG;
+    if (query_count == 0 || top_k == 0 || d == 0 || d % 2 || h2_stride < d || h2_stride % 2) return NVMAI_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    ProfScope prof(ctx, NVMAI_PROF_PREFILL_COMBINE, s);
+    dim3 grid((d / 2 + 255) / 256, query_count);
+    if (ctx->act == ACT_BF16)
+        prefill_reduce_kernel<ACT_BF16><<<grid, 256, 0, s>>>(route_partials, route_weights, h2, query_count, top_k, d, h2_stride);
+    else
+        prefill_reduce_kernel<ACT_FP16><<<grid, 256, 0, s>>>(route_partials, route_weights, h2, query_count, top_k, d, h2_stride);
+    return launch_status();
+}

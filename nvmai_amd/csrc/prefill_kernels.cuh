@@ -1,0 +1,421 @@
+// Prefill side of the MoE path: token-expert pair records, the permutation / histogram by
+// expert, the grouped expert GEMMs (dequant to bf16 tiles in LDS + MFMA) and the rank-order
+// combine.  gfx950, wave64.
+#pragma once
+
+#include "common.cuh"
+
+namespace nvmai {
+
+// PrefillTokenExpertPair (PrefillRouter.swift:5-28): 16 bytes, fields at 0/4/8/12.
+struct PrefillPair { uint32_t token, expert, rank, weight_bits; };
+struct PrefillGroup { uint32_t expert, pair_start, pair_count; };                 // PrefillMoEGroup
+struct PrefillTile { uint32_t group_start, group_count, pair_start, pair_count; }; // PrefillMoETile
+
+constexpr int GROUP_CHUNK = 1024;     // slots per block of the histogram / scatter passes
+
+// Device-side validation failures, numbered like PrefillMoEGroupingError's cases
+// (PrefillMoEGrouping.swift:121-137).  The error word holds min over pairs of (index << 4 | code),
+// i.e. the first failing pair in input order, as the reference's loop reports it.
+enum : uint32_t { GROUP_ERR_TOKEN = 6, GROUP_ERR_RANK = 7, GROUP_ERR_EXPERT = 8, GROUP_ERR_DUP = 9 };
+constexpr uint32_t GROUP_NO_ERR = 0xFFFFFFFFu;
+
+// Workspace words: [0] error word.
+__global__ __launch_bounds__(256) void prefill_init_kernel(uint32_t* first, uint32_t n_pairs, uint32_t* words) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (first && i < n_pairs) first[i] = GROUP_NO_ERR;
+    if (i == 0) words[0] = GROUP_NO_ERR;
+}
+
+// PrefillRouter.makeTokenExpertPairs (PrefillRouter.swift:97-117): token-major records.
+__global__ __launch_bounds__(256) void prefill_make_pairs_kernel(const uint32_t* idx, const uint16_t* w,
+                                                                uint32_t n_pairs, uint32_t top_k,
+                                                                PrefillPair* pairs) {
+    const uint32_t p = blockIdx.x * 256 + threadIdx.x;
+    if (p < n_pairs) pairs[p] = PrefillPair{p / top_k, idx[p], p % top_k, (uint32_t)w[p]};
+}
+
+// ---- pairs in any order -> slots (token * top_k + rank) ------------------------------------
+// A valid input holds every slot exactly once, so sorting by (key, expert, token, rank) is a
+// counting sort by expert over the slots in ascending order.
+__global__ __launch_bounds__(256) void prefill_claim_kernel(const PrefillPair* pairs, uint32_t n_pairs,
+                                                           uint32_t query_count, uint32_t top_k,
+                                                           uint32_t num_experts, uint32_t* first,
+                                                           uint32_t* words) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_pairs) return;
+    const PrefillPair p = pairs[i];
+    uint32_t code = 0;
+    if (p.token >= query_count) code = GROUP_ERR_TOKEN;
+    else if (p.rank >= top_k) code = GROUP_ERR_RANK;
+    else if (p.expert >= num_experts) code = GROUP_ERR_EXPERT;
+    if (code) atomicMin(&words[0], i << 4 | code);
+    else atomicMin(&first[p.token * top_k + p.rank], i);
+}
+
+__global__ __launch_bounds__(256) void prefill_slot_kernel(const PrefillPair* pairs, uint32_t n_pairs,
+                                                          uint32_t query_count, uint32_t top_k,
+                                                          uint32_t num_experts, const uint32_t* first,
+                                                          uint32_t* slot_expert, uint32_t* slot_weight,
+                                                          uint32_t* words) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_pairs) return;
+    const PrefillPair p = pairs[i];
+    if (p.token >= query_count || p.rank >= top_k || p.expert >= num_experts) return;
+    const uint32_t slot = p.token * top_k + p.rank;
+    if (first[slot] == i) { slot_expert[slot] = p.expert; slot_weight[slot] = p.weight_bits; }
+    else atomicMin(&words[0], i << 4 | GROUP_ERR_DUP);       // a later pair of an already seen slot
+}
+
+// ---- pass 1: per-block histogram of expert ids ------------------------------------------
+// An unfilled slot (only after a validation error) may hold anything: ids out of range are
+// skipped here and in the scatter, so every later index stays inside its array.  `report`:
+// the ids come straight from a router and have not been range-checked yet.
+__global__ __launch_bounds__(256) void prefill_hist_kernel(const uint32_t* idx, uint32_t n_pairs,
+                                                          uint32_t num_experts, uint32_t* block_hist,
+                                                          uint32_t* words, bool report) {
+    extern __shared__ uint32_t lds[];
+    for (uint32_t e = threadIdx.x; e < num_experts; e += 256) lds[e] = 0;
+    __syncthreads();
+    const uint32_t base = blockIdx.x * GROUP_CHUNK;
+    for (uint32_t i = threadIdx.x; i < GROUP_CHUNK && base + i < n_pairs; i += 256) {
+        const uint32_t e = idx[base + i];
+        if (e < num_experts) atomicAdd(&lds[e], 1u);
+        else if (report) atomicMin(&words[0], (base + i) << 4 | GROUP_ERR_EXPERT);
+    }
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e < num_experts; e += 256) block_hist[(size_t)blockIdx.x * num_experts + e] = lds[e];
+}
+
+// ---- pass 2: offsets, counts, groups, tiles (PrefillMoEGrouping.swift:151-184) ------------
+// One block.  Experts are laid out in ascending (sort key, expert) order; offsets of empty
+// experts are 0xFFFFFFFF.  block_hist is turned into each block's first slot per expert.
+// info: [0] groups, [1] tiles, [2] error code (0 = none), [3] index of the failing pair,
+// [4] largest group.
+__global__ __launch_bounds__(1024) void prefill_scan_kernel(uint32_t* block_hist, uint32_t n_blocks,
+                                                           uint32_t num_experts, const uint64_t* sort_keys,
+                                                           uint32_t tile_expert_count, uint32_t* offsets,
+                                                           uint32_t* counts, PrefillGroup* groups,
+                                                           PrefillTile* tiles, const uint32_t* words,
+                                                           uint32_t* info) {
+    extern __shared__ uint32_t lds[];
+    uint32_t* cnt = lds;                       // [E]
+    uint32_t* order = lds + num_experts;       // [E] expert at position i of the key order
+    uint32_t* start = lds + 2 * num_experts;   // [E] first pair of the expert
+    for (uint32_t e = threadIdx.x; e < num_experts; e += 1024) {
+        uint32_t total = 0;
+        for (uint32_t b = 0; b < n_blocks; ++b) {
+            const uint32_t c = block_hist[(size_t)b * num_experts + e];
+            block_hist[(size_t)b * num_experts + e] = total;      // exclusive prefix over blocks
+            total += c;
+        }
+        cnt[e] = total;
+        uint32_t pos = e;
+        if (sort_keys) {                                          // rank in (key, expert) order
+            pos = 0;
+            const uint64_t my_key = sort_keys[e];
+            for (uint32_t o = 0; o < num_experts; ++o) {
+                const uint64_t k = sort_keys[o];
+                pos += (k < my_key || (k == my_key && o < e)) ? 1u : 0u;
+            }
+        }
+        order[pos] = e;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {                                       // serial walk over the experts
+        uint32_t run = 0, ng = 0, nt = 0, max_pairs = 0;
+        for (uint32_t i = 0; i < num_experts; ++i) {
+            const uint32_t ex = order[i], c = cnt[ex];
+            start[ex] = run;
+            if (c) {
+                groups[ng++] = PrefillGroup{ex, run, c};
+                max_pairs = max(max_pairs, c);
+            }
+            run += c;
+        }
+        for (uint32_t gs = 0; gs < ng; gs += tile_expert_count) {
+            const uint32_t ge = min(ng, gs + tile_expert_count);
+            const PrefillGroup a = groups[gs], z = groups[ge - 1];
+            tiles[nt++] = PrefillTile{gs, ge - gs, a.pair_start, z.pair_start + z.pair_count - a.pair_start};
+        }
+        const uint32_t err = words[0];
+        info[0] = ng;
+        info[1] = nt;
+        info[2] = err == GROUP_NO_ERR ? 0u : (err & 15u);
+        info[3] = err == GROUP_NO_ERR ? 0u : (err >> 4);
+        info[4] = max_pairs;
+    }
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e < num_experts; e += 1024) {
+        counts[e] = cnt[e];
+        offsets[e] = cnt[e] ? start[e] : 0xFFFFFFFFu;
+        for (uint32_t b = 0; b < n_blocks; ++b) block_hist[(size_t)b * num_experts + e] += start[e];
+    }
+}
+
+// ---- pass 3: stable scatter ---------------------------------------------------------------
+// Slots ascend in (token, rank); inside a block thread e walks the block's slots in order and
+// places those of expert e, which keeps (token, rank) ascending inside every expert: the
+// order PrefillMoEGrouping.swift:140-149 sorts into.
+__global__ __launch_bounds__(256) void prefill_scatter_kernel(const uint32_t* idx, const uint32_t* w32,
+                                                             const uint16_t* w16, uint32_t n_pairs,
+                                                             uint32_t top_k, uint32_t num_experts,
+                                                             const uint32_t* block_base, PrefillPair* sorted) {
+    extern __shared__ uint32_t lds[];     // [GROUP_CHUNK] expert ids of this block
+    const uint32_t base = blockIdx.x * GROUP_CHUNK;
+    const uint32_t n = min((uint32_t)GROUP_CHUNK, n_pairs - base);
+    for (uint32_t i = threadIdx.x; i < n; i += 256) lds[i] = idx[base + i];
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e < num_experts; e += 256) {
+        uint32_t pos = block_base[(size_t)blockIdx.x * num_experts + e];
+        for (uint32_t i = 0; i < n; ++i) {
+            if (lds[i] != e) continue;
+            const uint32_t p = base + i;
+            sorted[pos++] = PrefillPair{p / top_k, e, p % top_k, w32 ? w32[p] : (uint32_t)w16[p]};
+        }
+    }
+}
+
+// ---- M tiles of the grouped GEMM ----------------------------------------------------------
+struct MTile { uint32_t expert, row_start, rows; };
+constexpr int GEMM_BM = 128;
+
+// One block: cuts every group into runs of at most GEMM_BM sorted pairs, largest groups first
+// in four coarse classes so that long experts start early.
+__global__ __launch_bounds__(256) void prefill_mtiles_kernel(const PrefillGroup* groups, const uint32_t* info,
+                                                            MTile* mtiles, uint32_t* n_mtiles) {
+    __shared__ uint32_t cursor;
+    if (threadIdx.x == 0) cursor = 0;
+    __syncthreads();
+    const uint32_t ng = info[2] ? 0u : info[0];               // nothing runs on a grouping that failed
+    for (int cls = 3; cls >= 0; --cls) {
+        for (uint32_t g = threadIdx.x; g < ng; g += 256) {
+            const PrefillGroup gr = groups[g];
+            const uint32_t t = (gr.pair_count + GEMM_BM - 1) / GEMM_BM;
+            const int my = t >= 16 ? 3 : t >= 4 ? 2 : t >= 2 ? 1 : 0;
+            if (my != cls) continue;
+            const uint32_t at = atomicAdd(&cursor, t);
+            for (uint32_t j = 0; j < t; ++j)
+                mtiles[at + j] = MTile{gr.expert, gr.pair_start + j * GEMM_BM, min((uint32_t)GEMM_BM, gr.pair_count - j * GEMM_BM)};
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *n_mtiles = cursor;
+}
+
+// ---- grouped GEMM ---------------------------------------------------------------------------
+// out[m, n] = sum_k X[row(m), k] * W_e[n, k] for the rows of one M tile (<= 128 sorted pairs of
+// one expert) and 128 weight rows: DUAL -> 64 gate rows + the same 64 up rows, epilogue
+// silu(g) * u (prefill.metal:460-501); else 128 down rows (prefill.metal:503-534).
+// Per 64-wide k step (one quantization group) each thread dequantizes half a weight row:
+// w = q * scale + bias in fp32, rounded once to the activation type (the reference dequantizes
+// to fp16, tensorops.metal:29-121), into an LDS tile; the activations go to LDS as they are.
+// v_mfma_f32_16x16x32_{bf16,f16} accumulates in fp32.  Wave (wm, wn) owns rows wm*64..+64 and four
+// 16-column tiles: DUAL gate/up columns wn*32..+32, else columns wn*64..+64.
+typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 hf8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 hf2_t __attribute__((ext_vector_type(2)));
+typedef float fl2_t __attribute__((ext_vector_type(2)));
+typedef float fl4_t __attribute__((ext_vector_type(4)));
+
+struct GemmParams {
+    const uint8_t* pool;
+    uint64_t pool_stride;
+    int64_t wA, sA, bA, wB, sB, bB;     // A: gate or down; B: up
+    const MTile* mtiles;
+    const uint32_t* n_mtiles;
+    const PrefillPair* pairs;           // sorted
+    const void* x;                      // DUAL: hidden rows by token; else act rows by sorted position
+    uint32_t x_stride;
+    void* out;                          // DUAL: act[sorted position, N]; else partials[token*top_k+rank, N]
+    uint32_t out_stride;
+    uint32_t K, N, top_k, n_tiles_n;
+};
+
+constexpr int GEMM_BK = 64;
+constexpr int GEMM_LDK = GEMM_BK + 8;   // padded row: conflict-free 16-byte reads
+
+// Two floats -> two 16-bit activations in one dword, round to nearest even.
+template <int ACT>
+__device__ __forceinline__ uint32_t pack_act2(float lo, float hi) {
+    const fl2_t v = {lo, hi};
+    if (ACT == ACT_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2_t));   // v_cvt_pk_bf16_f32
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, hf2_t));
+}
+
+template <int ACT>
+__device__ __forceinline__ fl4_t mfma_16x16x32(const uint4& a, const uint4& b, fl4_t c) {
+    if (ACT == ACT_BF16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, a), __builtin_bit_cast(bf8_t, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(hf8_t, a), __builtin_bit_cast(hf8_t, b), c, 0, 0, 0);
+}
+
+template <int ACT, int BITS, bool DUAL>
+__global__ __launch_bounds__(256) void prefill_gemm_kernel(GemmParams p) {
+    extern __shared__ uint4 gemm_lds[];
+    uint16_t* lds = reinterpret_cast<uint16_t*>(gemm_lds);
+    // [2][128][LDK] activations, then [2][128][LDK] weights
+    uint16_t* xs = lds;
+    uint16_t* ws = lds + 2 * GEMM_BM * GEMM_LDK;
+    const uint32_t tile_id = blockIdx.x / p.n_tiles_n, nt = blockIdx.x % p.n_tiles_n;
+    if (tile_id >= *p.n_mtiles) return;
+    const MTile mt = p.mtiles[tile_id];
+    const uint8_t* blob = p.pool + (uint64_t)mt.expert * p.pool_stride;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1, li = lane & 15, lq = lane >> 4;
+    const uint32_t groups = p.K / NVMAI_GROUP;
+    const uint32_t n_cols = DUAL ? 64 : 128;              // output columns per block
+    const uint32_t n0 = nt * n_cols;
+
+    // ---- this thread's staging duties: half an activation row and half a weight row
+    const int srow = tid >> 1, shalf = tid & 1;
+    const uint16_t* xrow;
+    {
+        const uint32_t m = (uint32_t)srow < mt.rows ? srow : 0;
+        const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
+        xrow = (const uint16_t*)p.x + (size_t)src * p.x_stride + shalf * 32;
+    }
+    const bool w_is_b = DUAL && srow >= 64;
+    uint32_t wn_row = n0 + (DUAL ? (srow & 63) : srow);
+    if (wn_row >= p.N) wn_row = p.N - 1;
+    const uint8_t* wrow = blob + (w_is_b ? p.wB : p.wA) + (size_t)wn_row * (p.K * BITS / 8) + shalf * (32 * BITS / 8);
+    const uint16_t* srow_p = reinterpret_cast<const uint16_t*>(blob + (w_is_b ? p.sB : p.sA)) + (size_t)wn_row * groups;
+    const uint16_t* brow_p = reinterpret_cast<const uint16_t*>(blob + (w_is_b ? p.bB : p.bA)) + (size_t)wn_row * groups;
+
+    uint4 xreg[4], wreg[BITS == 8 ? 2 : 1];
+    uint16_t sreg, breg;
+    auto load_regs = [&](uint32_t ks) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xreg[j] = *reinterpret_cast<const uint4*>(xrow + ks * GEMM_BK + j * 8);
+        const uint8_t* wp = wrow + (size_t)ks * (GEMM_BK * BITS / 8);
+        wreg[0] = *reinterpret_cast<const uint4*>(wp);
+        if (BITS == 8) wreg[BITS == 8 ? 1 : 0] = *reinterpret_cast<const uint4*>(wp + 16);
+        sreg = srow_p[ks];
+        breg = brow_p[ks];
+    };
+    auto store_regs = [&](int buf) {
+        uint16_t* xd = xs + (buf * GEMM_BM + srow) * GEMM_LDK + shalf * 32;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(xd + j * 8) = xreg[j];
+        uint16_t* wd = ws + (buf * GEMM_BM + srow) * GEMM_LDK + shalf * 32;
+        const float s = bf16_to_f32(sreg), b = bf16_to_f32(breg);
+        if (BITS == 4) {
+            const uint32_t words[4] = {wreg[0].x, wreg[0].y, wreg[0].z, wreg[0].w};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                float q[8];
+                unpack4(words[d], q);
+                uint4 o;
+                o.x = pack_act2<ACT>(fmaf(q[0], s, b), fmaf(q[1], s, b));
+                o.y = pack_act2<ACT>(fmaf(q[2], s, b), fmaf(q[3], s, b));
+                o.z = pack_act2<ACT>(fmaf(q[4], s, b), fmaf(q[5], s, b));
+                o.w = pack_act2<ACT>(fmaf(q[6], s, b), fmaf(q[7], s, b));
+                *reinterpret_cast<uint4*>(wd + d * 8) = o;
+            }
+        } else {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint4 wq = wreg[BITS == 8 ? h : 0];
+                const uint32_t words[4] = {wq.x, wq.y, wq.z, wq.w};
+#pragma unroll
+                for (int d = 0; d < 2; ++d) {
+                    float q[8];
+                    unpack8(words[2 * d], q);
+                    unpack8(words[2 * d + 1], q + 4);
+                    uint4 o;
+                    o.x = pack_act2<ACT>(fmaf(q[0], s, b), fmaf(q[1], s, b));
+                    o.y = pack_act2<ACT>(fmaf(q[2], s, b), fmaf(q[3], s, b));
+                    o.z = pack_act2<ACT>(fmaf(q[4], s, b), fmaf(q[5], s, b));
+                    o.w = pack_act2<ACT>(fmaf(q[6], s, b), fmaf(q[7], s, b));
+                    *reinterpret_cast<uint4*>(wd + h * 16 + d * 8) = o;
+                }
+            }
+        }
+    };
+
+    fl4_t acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[a][j] = fl4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const uint32_t nk = p.K / GEMM_BK;
+    load_regs(0);
+    store_regs(0);
+    __syncthreads();
+    for (uint32_t ks = 0; ks < nk; ++ks) {
+        const int buf = ks & 1;
+        if (ks + 1 < nk) load_regs(ks + 1);
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            uint4 afrag[4], bfrag[4];
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+                afrag[a] = *reinterpret_cast<const uint4*>(xs + (buf * GEMM_BM + wm * 64 + a * 16 + li) * GEMM_LDK + kk * 32 + lq * 8);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int brow = DUAL ? (j >> 1) * 64 + wn * 32 + (j & 1) * 16 + li : wn * 64 + j * 16 + li;
+                bfrag[j] = *reinterpret_cast<const uint4*>(ws + (buf * GEMM_BM + brow) * GEMM_LDK + kk * 32 + lq * 8);
+            }
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[a][j] = mfma_16x16x32<ACT>(afrag[a], bfrag[j], acc[a][j]);
+        }
+        if (ks + 1 < nk) store_regs(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds column li of each tile, rows 4*lq .. 4*lq+3
+    uint16_t* out = (uint16_t*)p.out;
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t m = wm * 64 + a * 16 + lq * 4 + t;
+            if (m >= mt.rows) continue;
+            if (DUAL) {
+                const size_t orow = (size_t)(mt.row_start + m) * p.out_stride;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const uint32_t n = n0 + wn * 32 + j * 16 + li;
+                    if (n < p.N) out[orow + n] = f32_to_act<ACT>(silu_fast(acc[a][j][t]) * acc[a][j + 2][t]);
+                }
+            } else {
+                const PrefillPair pr = p.pairs[mt.row_start + m];
+                const size_t orow = ((size_t)pr.token * p.top_k + pr.rank) * p.out_stride;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t n = n0 + wn * 64 + j * 16 + li;
+                    if (n < p.N) out[orow + n] = f32_to_act<ACT>(acc[a][j][t]);
+                }
+            }
+        }
+}
+
+// ---- combine (prefill.metal:437-458) -------------------------------------------------------
+// h2[t, d] = sum over ranks in rank order of fma(w[t, r], partial[t, r, d], acc).
+template <int ACT>
+__global__ __launch_bounds__(256) void prefill_reduce_kernel(const void* partials, const uint16_t* w, void* h2,
+                                                            uint32_t tokens, uint32_t top_k, uint32_t d,
+                                                            uint32_t h2_stride) {
+    const uint32_t t = blockIdx.y;
+    const uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 2;
+    if (c >= d) return;
+    float a0 = 0.0f, a1 = 0.0f;
+    for (uint32_t r = 0; r < top_k; ++r) {
+        const float wr = f16_to_f32(w[(size_t)t * top_k + r]);
+        const uint32_t v = *reinterpret_cast<const uint32_t*>((const uint16_t*)partials + ((size_t)t * top_k + r) * d + c);
+        float lo, hi;
+        act2_to_f32<ACT>(v, lo, hi);
+        a0 = fmaf(wr, lo, a0);
+        a1 = fmaf(wr, hi, a1);
+    }
+    uint16_t* o = (uint16_t*)h2 + (size_t)t * h2_stride + c;
+    o[0] = f32_to_act<ACT>(a0);
+    if (c + 1 < d) o[1] = f32_to_act<ACT>(a1);
+}
+
+}  // namespace nvmai

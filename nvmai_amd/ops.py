@@ -7,7 +7,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._lib import ExpertOffsets, KvView, MoeLayer, Rows, check, lib
+from ._lib import ExpertOffsets, KvView, MoeLayer, PrefillGrouping, Rows, check, lib
 
 ACT_BF16, ACT_FP16 = 0, 1
 (PROF_ROUTER, PROF_SELECT, PROF_GROUP, PROF_PHASE1, PROF_PHASE2, PROF_COMBINE, PROF_KV_QUANT,
@@ -226,6 +226,156 @@ class SharedExpertRuntime:
 # ---------------------------------------------------------------------------------------------
 # KV cache, RoPE, attention
 # ---------------------------------------------------------------------------------------------
+# ---------------------------------------------------------------- prefill
+GROUPING_ERRORS = {1: "invalidQueryCount", 2: "invalidTopK", 3: "invalidNumExperts",
+                   4: "invalidTileExpertCount", 5: "pairCountMismatch", 6: "tokenOutOfRange",
+                   7: "rankOutOfRange", 8: "expertOutOfRange", 9: "duplicateTokenRank",
+                   10: "expertSortKeyCountMismatch"}
+
+
+class PrefillMoEGroupingError(Exception):
+    """PrefillMoEGroupingError (PrefillMoEGrouping.swift:52-89); `pair_index` is the first
+    failing pair for the per-pair cases."""
+
+    def __init__(self, code, pair_index=None):
+        self.code, self.name, self.pair_index = code, GROUPING_ERRORS.get(code, str(code)), pair_index
+        super().__init__(self.name if pair_index is None else "%s (pair %d)" % (self.name, pair_index))
+
+
+class PrefillRouter:
+    """PrefillRouter (PrefillRouter.swift:30-117): block router and pair records."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+        self._moe = MoE(ctx)
+
+    def encode_block(self, router, hidden, num_experts, d, top_k, effective_scale=None, per_expert_scale=None):
+        """PrefillRouter.encodeBlock (PrefillRouter.swift:41-95): idx u32 and FP16 weights [tokens, top_k]."""
+        return self._moe.encode_router(router, hidden, num_experts, d, top_k, effective_scale, per_expert_scale)
+
+    def make_token_expert_pairs(self, indices, weights):
+        """PrefillRouter.makeTokenExpertPairs (PrefillRouter.swift:97-117): int32 [tokens*top_k, 4]
+        records {token, expert, rank, weight bits}."""
+        tokens, top_k = indices.shape
+        pairs = torch.empty((tokens * top_k, 4), dtype=torch.int32, device=indices.device)
+        check(lib.nvmai_hip_prefill_make_pairs(self.ctx.handle, _stream(), _ptr(indices), _ptr(weights), tokens,
+                                               top_k, _ptr(pairs)), "prefill_make_pairs")
+        return pairs
+
+
+class PrefillMoEGroupedRoutes:
+    """PrefillMoEGroupedRoutes (PrefillMoEGrouping.swift:31-50) held in device memory."""
+
+    def __init__(self, n_pairs, query_count, top_k, num_experts, tile_expert_count, device):
+        i32 = dict(dtype=torch.int32, device=device)
+        self.query_count, self.top_k, self.num_experts = query_count, top_k, num_experts
+        self.tile_expert_count = tile_expert_count
+        self.sorted_pairs = torch.empty((n_pairs, 4), **i32)
+        self.per_expert_offsets = torch.empty(num_experts, **i32)
+        self.per_expert_counts = torch.empty(num_experts, **i32)
+        self.groups_buf = torch.empty((num_experts, 3), **i32)
+        self.tiles_buf = torch.empty((num_experts, 4), **i32)
+        self.info = torch.zeros(8, **i32)
+        self.desc = PrefillGrouping(*(t.data_ptr() for t in (self.sorted_pairs, self.per_expert_offsets,
+                                                             self.per_expert_counts, self.groups_buf,
+                                                             self.tiles_buf, self.info)))
+
+    def validate(self):
+        """Waits for the device and raises what the reference would have thrown."""
+        info = self.info.cpu().tolist()
+        if info[2]:
+            raise PrefillMoEGroupingError(info[2], info[3])
+        return info
+
+    @property
+    def groups(self):
+        return self.groups_buf[: self.validate()[0]]
+
+    @property
+    def tiles(self):
+        return self.tiles_buf[: self.validate()[1]]
+
+
+class PrefillMoEGrouping:
+    """PrefillMoEGrouping (PrefillMoEGrouping.swift:91-192) on the device."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+
+    @staticmethod
+    def _check(n_pairs, query_count, top_k, num_experts, tile_expert_count, sort_keys):
+        code = lib.nvmai_prefill_grouping_check(n_pairs, query_count, top_k, num_experts, tile_expert_count,
+                                                sort_keys is not None, 0 if sort_keys is None else sort_keys.numel())
+        if code:
+            raise PrefillMoEGroupingError(code)
+
+    def group_token_expert_pairs(self, pairs, query_count, top_k, num_experts, tile_expert_count=16,
+                                 expert_sort_keys=None, validate=True):
+        """groupTokenExpertPairs: pairs int32 [n, 4] in any order; expert_sort_keys int64 [num_experts]."""
+        n = pairs.shape[0]
+        self._check(n, query_count, top_k, num_experts, tile_expert_count, expert_sort_keys)
+        out = PrefillMoEGroupedRoutes(n, query_count, top_k, num_experts, tile_expert_count, pairs.device)
+        check(lib.nvmai_hip_prefill_group_pairs(self.ctx.handle, _stream(), _ptr(pairs), n, query_count, top_k,
+                                                num_experts, tile_expert_count, _ptr(expert_sort_keys),
+                                                0 if expert_sort_keys is None else expert_sort_keys.numel(),
+                                                C.byref(out.desc)), "prefill_group_pairs")
+        if validate:
+            out.validate()
+        return out
+
+    def group_routes(self, indices, weights, num_experts, tile_expert_count=16, expert_sort_keys=None,
+                     validate=False):
+        """makeTokenExpertPairs + groupTokenExpertPairs from the router's outputs, no host step."""
+        query_count, top_k = indices.shape
+        self._check(query_count * top_k, query_count, top_k, num_experts, tile_expert_count, expert_sort_keys)
+        out = PrefillMoEGroupedRoutes(query_count * top_k, query_count, top_k, num_experts, tile_expert_count,
+                                      indices.device)
+        check(lib.nvmai_hip_prefill_group_routes(self.ctx.handle, _stream(), _ptr(indices), _ptr(weights),
+                                                 query_count, top_k, num_experts, tile_expert_count,
+                                                 _ptr(expert_sort_keys),
+                                                 0 if expert_sort_keys is None else expert_sort_keys.numel(),
+                                                 C.byref(out.desc)), "prefill_group_routes")
+        if validate:
+            out.validate()
+        return out
+
+
+class PrefillGroupedRoutedMoE:
+    """PrefillGroupedRoutedMoE.encodeStreamedBatched over all tiles (PrefillGroupedRoutedMoE.swift:413-489)
+    with the experts resident: expert e at experts[e] of a [num_experts, stride] uint8 pool."""
+
+    def __init__(self, ctx, bits=4):
+        self.ctx, self.bits = ctx, bits
+
+    def encode(self, experts, offsets, hidden, d, f, routes, act_scratch=None, route_partials=None):
+        n = routes.sorted_pairs.shape[0]
+        if act_scratch is None:
+            act_scratch = torch.empty((n, f), dtype=self.ctx.dtype, device=hidden.device)
+        if route_partials is None:
+            route_partials = torch.empty((n, d), dtype=self.ctx.dtype, device=hidden.device)
+        check(lib.nvmai_hip_prefill_grouped_moe(self.ctx.handle, _stream(), _ptr(experts), experts.stride(0),
+                                                C.byref(offsets), self.bits, d, f, experts.shape[0], _ptr(hidden),
+                                                hidden.stride(0), routes.query_count, routes.top_k,
+                                                C.byref(routes.desc), _ptr(act_scratch), _ptr(route_partials)),
+              "prefill_grouped_moe")
+        return route_partials, act_scratch
+
+
+class PrefillMoE:
+    """PrefillMoE.encodeReduceTokenMajor (PrefillMoE.swift:11-40)."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+
+    def encode_reduce_token_major(self, route_partials, route_weights, query_count, top_k, d, h2=None):
+        if h2 is None:
+            h2 = torch.empty((query_count, d), dtype=self.ctx.dtype, device=route_partials.device)
+        check(lib.nvmai_hip_prefill_moe_reduce_token_major(self.ctx.handle, _stream(), _ptr(route_partials),
+                                                           _ptr(route_weights), _ptr(h2), h2.stride(0), query_count,
+                                                           top_k, d), "prefill_moe_reduce_token_major")
+        return h2
+
+
 def kv_row_layout(elements, bits):
     """KVCacheManager.rowLayout (KVCacheManager.swift:437-446) -> (stride, value_bytes)."""
     s, v = C.c_uint32(), C.c_uint32()

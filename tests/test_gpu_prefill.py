@@ -1,0 +1,281 @@
+"""GPU parity for the prefill side: pair records, permutation / histogram by expert, grouped
+expert GEMMs and the rank-order reduce, called through the C ABI and compared with the CPU
+oracle.
+
+Bars: every grouping array bit-exact (integers); 16-bit outputs within 1e-2 of the oracle as
+max|diff| / max|ref| (RelError.swift:5-16)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from gpu_util import act_np, act_tensor, dev, gauss, say, u32
+
+pytestmark = pytest.mark.gpu
+
+TOL_ACT = 1e-2
+
+
+@pytest.fixture(scope="module")
+def nv():
+    import nvmai_amd
+    return nvmai_amd
+
+
+@pytest.fixture(scope="module", params=[0, 1], ids=["bf16", "fp16"])
+def ctx(request, nv):
+    c = nv.Context(0, request.param)
+    yield c
+    torch.cuda.synchronize()
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def ctx_bf16(nv):
+    c = nv.Context(0, 0)
+    yield c
+    torch.cuda.synchronize()
+    c.close()
+
+
+def _pairs(rows):
+    a = np.zeros(len(rows), O.PAIR_DTYPE)
+    for i, (t, e, r, w) in enumerate(rows):
+        a[i] = (t, e, r, w)
+    return a
+
+
+def _pairs_dev(p):
+    return dev(p.view(np.uint32).reshape(-1, 4).view(np.int32))
+
+
+def _check_routes(routes, want):
+    """Every array of the device grouping against the oracle's dict."""
+    torch.cuda.synchronize()
+    info = routes.validate()
+    got_sorted = u32(routes.sorted_pairs).reshape(-1).view(O.PAIR_DTYPE)
+    assert np.array_equal(got_sorted, want["sorted"])
+    assert np.array_equal(u32(routes.per_expert_offsets), want["offsets"])
+    assert np.array_equal(u32(routes.per_expert_counts), want["counts"])
+    assert info[0] == want["groups"].size and info[1] == want["tiles"].size
+    assert np.array_equal(u32(routes.groups).reshape(-1).view(O.GROUP_DTYPE), want["groups"])
+    assert np.array_equal(u32(routes.tiles).reshape(-1).view(O.TILE_DTYPE), want["tiles"])
+    assert info[4] == (want["counts"].max() if want["counts"].size else 0)
+
+
+# ------------------------------------------------------------------ pairs + grouping
+def test_make_pairs_token_major(nv, ctx_bf16):
+    say("prefill make_pairs")
+    # PrefillRouterTests.swift:12-31
+    w = O.f16_bits(np.array([0.1, 0.2, 0.3, 0.4, 0.5, 0.6], np.float32)).reshape(2, 3)
+    idx = np.array([[3, 1, 2], [4, 0, 5]], np.uint32)
+    got = nv.PrefillRouter(ctx_bf16).make_token_expert_pairs(dev(idx.view(np.int32)), dev(w.view(np.int16)))
+    torch.cuda.synchronize()
+    assert np.array_equal(u32(got).reshape(-1).view(O.PAIR_DTYPE), O.make_pairs(idx, w))
+
+
+def test_grouping_reference_known_answers(nv, ctx_bf16):
+    say("prefill grouping known answers")
+    g = nv.PrefillMoEGrouping(ctx_bf16)
+    # PrefillMoEGroupingTests.swift:5-53, input reversed
+    rows = [(0, 3, 0, 10), (0, 1, 1, 11), (0, 4, 2, 12), (1, 1, 0, 13), (1, 3, 1, 14),
+            (1, 2, 2, 15), (2, 4, 0, 16), (2, 3, 1, 17), (2, 1, 2, 18), (3, 5, 0, 19),
+            (3, 1, 1, 20), (3, 4, 2, 21)]
+    p = _pairs(rows[::-1])
+    r = g.group_token_expert_pairs(_pairs_dev(p), 4, 3, 6, tile_expert_count=2)
+    _check_routes(r, O.group_pairs(p, 4, 3, 6, 2))
+    assert u32(r.per_expert_offsets).tolist() == [0xFFFFFFFF, 0, 4, 5, 8, 11]
+    assert u32(r.tiles).tolist() == [[0, 2, 0, 5], [2, 2, 5, 6], [4, 1, 11, 1]]
+    # :55-82 shuffled input, weight bits travel with their pair
+    tm = [(0, 2, 0, 101), (0, 1, 1, 102), (1, 2, 0, 103), (1, 0, 1, 104), (2, 1, 0, 105), (2, 2, 1, 106)]
+    sh = _pairs([tm[5], tm[1], tm[3], tm[0], tm[4], tm[2]])
+    r = g.group_token_expert_pairs(_pairs_dev(sh), 3, 2, 3, 2)
+    _check_routes(r, O.group_pairs(sh, 3, 2, 3, 2))
+    assert u32(r.sorted_pairs)[:, 3].tolist() == [104, 102, 105, 101, 103, 106]
+    # :84-115 expert sort keys
+    rows = _pairs([(0, 1, 0, 10), (0, 2, 1, 20), (1, 3, 0, 30), (1, 1, 1, 11), (2, 2, 0, 21), (2, 3, 1, 31)])
+    keys = np.array([0, 30, 10, 20], np.uint64)
+    r = g.group_token_expert_pairs(_pairs_dev(rows), 3, 2, 4, 2, expert_sort_keys=dev(keys.view(np.int64)))
+    _check_routes(r, O.group_pairs(rows, 3, 2, 4, 2, sort_keys=keys))
+    assert u32(r.groups)[:, 0].tolist() == [2, 3, 1]
+    # :175-203 pressure case
+    rows = _pairs([(t, (t + r_ * 7) % 74, r_, t * 8 + r_) for t in range(32) for r_ in range(8)])
+    r = g.group_token_expert_pairs(_pairs_dev(rows), 32, 8, 128, 16)
+    _check_routes(r, O.group_pairs(rows, 32, 8, 128, 16))
+
+
+def test_grouping_rejects_invalid_metadata(nv, ctx_bf16):
+    say("prefill grouping errors")
+    # PrefillMoEGroupingTests.swift:117-173
+    g = nv.PrefillMoEGrouping(ctx_bf16)
+    one = _pairs_dev(_pairs([(0, 0, 0, 1)]))
+    cases = [((one, 1, 1, 1, 17), {}, "invalidTileExpertCount"),
+             ((_pairs_dev(_pairs([(0, 2, 0, 1)])), 1, 1, 2, 1), {}, "expertOutOfRange"),
+             ((_pairs_dev(_pairs([(0, 0, 0, 1), (0, 1, 0, 2)])), 1, 2, 2, 1), {}, "duplicateTokenRank"),
+             ((one, 1, 1, 2, 1), dict(expert_sort_keys=dev(np.zeros(1, np.int64))), "expertSortKeyCountMismatch"),
+             ((one, 2, 1, 1, 1), {}, "pairCountMismatch"),
+             ((one, -1, 1, 1, 1), {}, "invalidQueryCount"),
+             ((one, 1, 0, 1, 1), {}, "invalidTopK"),
+             ((one, 1, 1, 0, 1), {}, "invalidNumExperts"),
+             ((_pairs_dev(_pairs([(1, 0, 0, 1)])), 1, 1, 1, 1), {}, "tokenOutOfRange"),
+             ((_pairs_dev(_pairs([(0, 0, 1, 1)])), 1, 1, 1, 1), {}, "rankOutOfRange")]
+    for args, kw, name in cases:
+        with pytest.raises(nv.PrefillMoEGroupingError) as e:
+            g.group_token_expert_pairs(*args, **kw)
+        assert e.value.name == name, name
+    # the first failing pair in input order decides, as in the reference's loop
+    p = _pairs([(0, 0, 0, 1), (0, 1, 1, 2), (1, 9, 0, 3), (0, 1, 1, 4), (7, 0, 1, 5)])
+    with pytest.raises(O.GroupingError) as want:
+        O.group_pairs(np.concatenate([p, p[:1]]), 3, 2, 4, 1)
+    with pytest.raises(nv.PrefillMoEGroupingError) as e:
+        g.group_token_expert_pairs(_pairs_dev(np.concatenate([p, p[:1]])), 3, 2, 4, 1)
+    assert e.value.name == want.value.name == "expertOutOfRange" and e.value.pair_index == 2
+    # empty input is valid and yields nothing
+    r = g.group_token_expert_pairs(torch.empty((0, 4), dtype=torch.int32, device="cuda"), 0, 8, 4, 16)
+    _check_routes(r, O.group_pairs(_pairs([]), 0, 8, 4, 16))
+    # the C ABI itself refuses what the host check refuses
+    st = nv.lib.nvmai_hip_prefill_group_pairs(ctx_bf16.handle, None, one.data_ptr(), 1, 1, 1, 1, 17, None, 0,
+                                              r.desc)
+    assert st == -1
+
+
+def _zipf_routes(rng, tokens, E, k, s=1.1):
+    """k distinct experts per token, expert popularity ~ 1 / rank^s."""
+    p = 1.0 / np.arange(1, E + 1) ** s
+    p /= p.sum()
+    perm = rng.permutation(E)
+    keys = rng.random((tokens, E)) ** (1.0 / p[None, :])      # weighted sampling without replacement
+    idx = perm[np.argsort(-keys, axis=1)[:, :k]].astype(np.uint32)
+    w = rng.random((tokens, k)).astype(np.float32) + 0.05
+    w /= w.sum(axis=1, keepdims=True)
+    return idx, O.f16_bits(w)
+
+
+@pytest.mark.parametrize("tokens,E,k,tile", [(1, 8, 2, 16), (37, 20, 3, 4), (1000, 256, 8, 16), (4096, 256, 8, 16),
+                                             (300, 600, 4, 7)])
+def test_grouping_random_routes_bit_exact(nv, ctx_bf16, tokens, E, k, tile):
+    say("prefill grouping random", tokens, E, k, tile)
+    rng = np.random.default_rng(tokens * 31 + E)
+    idx, w = _zipf_routes(rng, tokens, E, k)
+    pairs = O.make_pairs(idx, w)
+    g = nv.PrefillMoEGrouping(ctx_bf16)
+    want = O.group_pairs(pairs, tokens, k, E, tile)
+    # straight from the router's outputs
+    _check_routes(g.group_routes(dev(idx.view(np.int32)), dev(w.view(np.int16)), E, tile), want)
+    # pair records in shuffled order, with and without sort keys
+    shuffled = pairs[rng.permutation(pairs.size)]
+    _check_routes(g.group_token_expert_pairs(_pairs_dev(shuffled), tokens, k, E, tile), want)
+    keys = rng.integers(0, 5, E).astype(np.uint64)
+    _check_routes(g.group_token_expert_pairs(_pairs_dev(shuffled), tokens, k, E, tile,
+                                             expert_sort_keys=dev(keys.view(np.int64))),
+                  O.group_pairs(pairs, tokens, k, E, tile, sort_keys=keys))
+    # histogram / permutation invariants at any size
+    sp = want["sorted"]
+    assert np.array_equal(want["counts"], np.bincount(idx.reshape(-1), minlength=E))
+    assert np.all(np.diff(sp["expert"].astype(np.int64) * 2**40 + sp["token"].astype(np.int64) * 64 + sp["rank"]) > 0)
+
+
+# ------------------------------------------------------------------ grouped GEMM + reduce
+def _prefill_case(nv, ctx, rng, d, f, E, k, bits, tokens, std=0.05, check_tokens=None):
+    mats = [(gauss(rng, (f, d), std), gauss(rng, (f, d), std), gauss(rng, (d, f), std)) for _ in range(E)]
+    blobs = np.stack([O.pack_expert(*m, bits) for m in mats])
+    x = O.round_bf16(gauss(rng, (tokens, d))) if ctx.act == 0 else O.f16_to_float(O.f16_bits(gauss(rng, (tokens, d))))
+    idx, w = _zipf_routes(rng, tokens, E, k)
+    off, stride = nv.expert_offsets(d, f, bits)
+    assert stride == blobs.shape[1]
+    routes = nv.PrefillMoEGrouping(ctx).group_routes(dev(idx.view(np.int32)), dev(w.view(np.int16)), E)
+    partials, act = nv.PrefillGroupedRoutedMoE(ctx, bits).encode(dev(blobs), off, act_tensor(x, ctx), d, f, routes)
+    h2 = nv.PrefillMoE(ctx).encode_reduce_token_major(partials, dev(w.view(np.int16)), tokens, k, d)
+    torch.cuda.synchronize()
+    routes.validate()
+    sel = np.arange(tokens) if check_tokens is None else check_tokens
+    want = O.prefill_moe(blobs, bits, x[sel], d, f, idx[sel], w[sel])
+    err = O.rel_error(act_np(h2)[sel], want)
+    assert err <= TOL_ACT, err
+    return err
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("d,f,E,k,tokens", [(128, 64, 4, 2, 3), (256, 192, 6, 3, 150), (192, 64, 5, 2, 131)])
+def test_grouped_moe_toy_shapes(nv, ctx, bits, d, f, E, k, tokens):
+    say("prefill grouped moe toy", ctx.act, bits, d, f, E, k, tokens)
+    _prefill_case(nv, ctx, np.random.default_rng(d + f + bits), d, f, E, k, bits, tokens)
+
+
+def test_grouped_moe_synthetic_pool_known_answer(nv, ctx_bf16):
+    say("prefill grouped moe synthetic pool")
+    # PrefillGroupedRoutedMoETests.swift:271-280 closed-form weights (silu activation)
+    d, f, E, T = 128, 64, 4, 3
+
+    def rows(expert, role, r, c):
+        i, j = np.meshgrid(np.arange(r), np.arange(c), indexing="ij")
+        return ((expert + 1) * 1e-3 + (role + 1) * 3e-3 + ((i % 7) - 3) * 4e-4 + ((j % 11) - 5) * 2e-4).astype(np.float32)
+    blobs = np.stack([O.pack_expert(rows(e, 0, f, d), rows(e, 1, f, d), rows(e, 2, d, f), 4) for e in range(E)])
+    hidden = np.array([[(i % 17) - 8 for i in range(d)]] * T, np.float32) * np.float32(0.125)
+    hidden += np.arange(T, dtype=np.float32)[:, None] * np.float32(0.25)
+    idx = np.array([[0, 2], [1, 2], [3, 0]], np.uint32)
+    w = O.f16_bits(np.array([[0.75, 0.25], [0.5, 0.5], [0.625, 0.375]], np.float32))
+    off, _ = nv.expert_offsets(d, f, 4)
+    routes = nv.PrefillMoEGrouping(ctx_bf16).group_routes(dev(idx.view(np.int32)), dev(w.view(np.int16)), E)
+    partials, _ = nv.PrefillGroupedRoutedMoE(ctx_bf16, 4).encode(dev(blobs), off, act_tensor(hidden, ctx_bf16), d, f, routes)
+    h2 = nv.PrefillMoE(ctx_bf16).encode_reduce_token_major(partials, dev(w.view(np.int16)), T, 2, d)
+    torch.cuda.synchronize()
+    assert O.rel_error(act_np(h2), O.prefill_moe(blobs, 4, hidden, d, f, idx, w)) <= TOL_ACT
+
+
+def test_reduce_token_major_rank_order(nv, ctx):
+    say("prefill reduce", ctx.act)
+    rng = np.random.default_rng(5)
+    T, k, d = 33, 8, 130
+    part = act_tensor(gauss(rng, (T * k, d)), ctx)
+    w = O.f16_bits(rng.random((T, k)).astype(np.float32))
+    h2 = nv.PrefillMoE(ctx).encode_reduce_token_major(part, dev(w.view(np.int16)), T, k, d)
+    torch.cuda.synchronize()
+    pf, wf = act_np(part).reshape(T, k, d), O.f16_to_float(w)
+    acc = np.zeros((T, d), np.float32)
+    for r in range(k):                                   # prefill.metal:450-457: fma chain in rank order
+        acc = (wf[:, r, None].astype(np.float64) * pf[:, r].astype(np.float64) + acc.astype(np.float64)).astype(np.float32)
+    want = act_tensor(acc, ctx)
+    assert torch.equal(h2.cpu(), want.cpu())
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_grouped_moe_production_shape(nv, ctx_bf16, bits):
+    say("prefill grouped moe production", bits)
+    # 4096 tokens x top-8 of 256 experts, D 2048, F 512, Zipf routing; the oracle checks a
+    # sample of tokens, the rest is covered by linearity below.
+    d, f, E, k, tokens = 2048, 512, 256, 8, 4096
+    rng = np.random.default_rng(77 + bits)
+    off, stride = nv.expert_offsets(d, f, bits)
+    gen = torch.Generator(device="cuda").manual_seed(5 + bits)
+    pool = torch.empty((E, stride), dtype=torch.uint8, device="cuda")
+    for rows_, n, wo, so, bo in ((f, d, off.gate_w, off.gate_s, off.gate_b), (f, d, off.up_w, off.up_s, off.up_b),
+                                 (d, f, off.down_w, off.down_s, off.down_b)):
+        wmat = torch.empty((E * rows_, n), dtype=torch.bfloat16, device="cuda").normal_(0.0, 0.03, generator=gen)
+        p, s, b = nv.quantize_affine(ctx_bf16, wmat, bits)
+        wb, mb = rows_ * n * bits // 8, rows_ * n // 32
+        pool[:, wo:wo + wb] = p.view(E, wb)
+        pool[:, so:so + mb] = s.view(torch.uint8).view(E, mb)
+        pool[:, bo:bo + mb] = b.view(torch.uint8).view(E, mb)
+        del wmat, p, s, b
+    x = O.round_bf16(gauss(rng, (tokens, d)))
+    idx, w = _zipf_routes(rng, tokens, E, k)
+    xd, idxd, wd = act_tensor(x, ctx_bf16), dev(idx.view(np.int32)), dev(w.view(np.int16))
+    grouping, moe, red = nv.PrefillMoEGrouping(ctx_bf16), nv.PrefillGroupedRoutedMoE(ctx_bf16, bits), nv.PrefillMoE(ctx_bf16)
+    routes = grouping.group_routes(idxd, wd, E)
+    partials, _ = moe.encode(pool, off, xd, d, f, routes)
+    h2 = red.encode_reduce_token_major(partials, wd, tokens, k, d)
+    torch.cuda.synchronize()
+    _check_routes(routes, O.group_pairs(O.make_pairs(idx, w), tokens, k, E, 16))
+    sel = np.sort(rng.choice(tokens, 24, replace=False))
+    blobs = pool.cpu().numpy()
+    want = O.prefill_moe(blobs, bits, x[sel], d, f, idx[sel], w[sel])
+    got = act_np(h2)
+    assert O.rel_error(got[sel], want) <= TOL_ACT
+    assert np.isfinite(got).all()
+    # a token's row does not depend on what else is in the batch: the first 512 tokens alone
+    r2 = grouping.group_routes(idxd[:512].contiguous(), wd[:512].contiguous(), E)
+    p2, _ = moe.encode(pool, off, xd[:512].contiguous(), d, f, r2)
+    h2b = red.encode_reduce_token_major(p2, wd[:512].contiguous(), 512, k, d)
+    torch.cuda.synchronize()
+    assert torch.equal(h2b, h2[:512])
