@@ -30,11 +30,19 @@ def parse():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--batch", type=int, default=32, help="tokens per decode step (1..32)")
-    ap.add_argument("--bits", type=int, default=8, choices=[4, 8])
+    ap.add_argument("--bits", type=int, default=None, choices=[4, 8], help="default 8 (4 for --workload prefill)")
     ap.add_argument("--layers", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--sweep", action="store_true", help="also print batch/bits sweep lines to stderr")
-    return ap.parse_args()
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention"],
+                    help="decode = configs[1] (the headline line); prefill = configs[2] grouped GEMM; "
+                         "attention = configs[3] quantized-KV decode attention")
+    ap.add_argument("--context", type=int, default=32768, help="attention: tokens in the KV cache")
+    ap.add_argument("--tokens", type=int, default=4096, help="prefill: tokens per step")
+    a = ap.parse_args()
+    if a.bits is None:
+        a.bits = 4 if a.workload == "prefill" else 8
+    return a
 
 
 def build_layers(nv, ctx, torch, bits, n_layers, seed=1234):
@@ -140,6 +148,134 @@ def cpu_baseline(layers, stride, bits, batch, torch):
                        % (n, bits, reps, dt, algo / 1e6, bytes_ / 1e6))
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def run_prefill(nv, ctx, torch, a):
+    """configs[2]: 4096 tokens, top-8 of 256 experts with Zipf(1.1) popularity, 4-bit experts.
+    A step = grouping by expert + gate/up SwiGLU GEMM + down GEMM + rank-order reduce."""
+    bits, T = a.bits, a.tokens
+    layers, stride = build_layers(nv, ctx, torch, bits, 1)
+    pool = layers[0]["pool"][:E]
+    off, _ = nv.expert_offsets(D, F, bits)
+    gen = torch.Generator(device="cuda").manual_seed(4242)
+    n_x = 4
+    xs = torch.empty((n_x, T, D), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
+    # router logits = log popularity + Gumbel noise: top-8 then samples experts without
+    # replacement with probability proportional to a Zipf(1.1) law over a random expert order
+    pop = 1.0 / torch.arange(1, E + 1, device="cuda", dtype=torch.float32) ** 1.1
+    pop = pop[torch.randperm(E, device="cuda", generator=gen)]
+    u = torch.rand((n_x, T, E), device="cuda", generator=gen).clamp_(1e-9, 1.0)
+    logits = torch.log(pop)[None, None, :] - torch.log(-torch.log(u))
+    top = torch.topk(logits, K, dim=-1)
+    idx = top.indices.to(torch.int32).contiguous()
+    w = torch.softmax(top.values, dim=-1).to(torch.float16).contiguous()
+    grouping, moe, red = nv.PrefillMoEGrouping(ctx), nv.PrefillGroupedRoutedMoE(ctx, bits), nv.PrefillMoE(ctx)
+    act = torch.empty((T * K, F), dtype=torch.bfloat16, device="cuda")
+    partials = torch.empty((T * K, D), dtype=torch.bfloat16, device="cuda")
+    h2 = torch.empty((T, D), dtype=torch.bfloat16, device="cuda")
+
+    def step(i):
+        j = i % n_x
+        routes = grouping.group_routes(idx[j], w[j], E)
+        moe.encode(pool, off, xs[j], D, F, routes, act, partials)
+        red.encode_reduce_token_major(partials, w[j], T, K, D, h2)
+        return routes
+
+    for i in range(a.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(i)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    ctx.profile_enable(True)
+    for i in range(a.steps):
+        step(i)
+    torch.cuda.synchronize()
+    ctx.profile_enable(False)
+    kern = {}
+    for tag, name in ((nv.PROF_PREFILL_GROUP, "group"), (nv.PROF_PREFILL_GEMM1, "gemm_gate_up"),
+                      (nv.PROF_PREFILL_GEMM2, "gemm_down"), (nv.PROF_PREFILL_COMBINE, "reduce")):
+        ms, n = ctx.profile_read(tag)
+        kern[name] = ms / max(n, 1) * 1e3
+    flops = T * K * 6.0 * D * F
+    g1 = T * K * 4.0 * D * F / (kern["gemm_gate_up"] * 1e-6) / 1e12
+    counts = step(0).per_expert_counts.cpu().numpy()
+    return {
+        "metric": METRIC, "value": round(flops / dt / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u%d codes -> bf16 MFMA, f32 accumulate" % bits, "data": "synthetic",
+        "config": {"workload": "configs[2]: MoE prefill grouped GEMM, %d tokens x hidden 2048, top-8 of 256 experts "
+                               "(Zipf 1.1 popularity), %d-bit group-64 experts, intermediate 512" % (T, bits),
+                   "tokens_per_s": round(T / dt), "largest_expert_pairs": int(counts.max()),
+                   "experts_hit": int((counts > 0).sum()),
+                   "kernel_us": {k: round(v, 2) for k, v in kern.items()}},
+        "roofline": {"kernel": "prefill_gemm_kernel<DUAL> (gate/up + SwiGLU)", "bound": "mfma",
+                     "achieved": round(g1, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(g1 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "flops_per_launch": T * K * 4.0 * D * F, "avg_launch_us": round(kern["gemm_gate_up"], 2)},
+        "cpu_baseline": None,
+    }
+
+
+def run_attention(nv, ctx, torch, a):
+    """configs[3]: 16 query heads, 2 KV heads, head_dim 256, KV quantized on write; a step = one
+    decode attention call over `--context` cached tokens for `--batch` sequences."""
+    bits, B, ctx_len = a.bits, min(a.batch, 8), a.context
+    HQ, HKV, HD = 16, 2, 256
+    gen = torch.Generator(device="cuda").manual_seed(31)
+    n_sets = max(1, min(8, int(1.5e9 // (2 * B * ctx_len * 600))))      # rotate caches past L2 / MALL
+    quant, att = nv.KVCacheQuantizer(ctx), nv.Attention(ctx)
+    caches = []
+    for _ in range(n_sets):
+        kc, vc = nv.KVCache(B, ctx_len, HKV * HD, bits), nv.KVCache(B, ctx_len, HKV * HD, bits)
+        for b in range(B):
+            for start in range(0, ctx_len, 8192):
+                n = min(8192, ctx_len - start)
+                for c in (kc, vc):
+                    src = torch.empty((n, HKV * HD), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
+                    quant.encode(src, HKV * HD, c.view(b, start), n, HKV * HD)
+        caches.append((kc, vc))
+    q = torch.empty((B, HQ, HD), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
+    out = torch.empty_like(q)
+    for i in range(a.warmup):
+        att.encode_full(q, *caches[i % n_sets], HD, HQ, HKV, ctx_len, out=out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        att.encode_full(q, *caches[i % n_sets], HD, HQ, HKV, ctx_len, out=out)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    ctx.profile_enable(True)
+    for i in range(a.steps):
+        att.encode_full(q, *caches[i % n_sets], HD, HQ, HKV, ctx_len, out=out)
+    torch.cuda.synchronize()
+    ctx.profile_enable(False)
+    kern = {}
+    for tag, name in ((nv.PROF_ATTN_PARTIAL, "partial"), (nv.PROF_ATTN_COMBINE, "combine")):
+        ms, n = ctx.profile_read(tag)
+        kern[name] = ms / max(n, 1) * 1e3
+    stride = caches[0][0].stride
+    kv_bytes = 2.0 * B * ctx_len * stride
+    step_b = kv_bytes + 2 * B * HQ * HD * 2
+    part = kv_bytes / (kern["partial"] * 1e-6) / 1e9
+    return {
+        "metric": METRIC, "value": round(step_b / dt / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u%d KV codes, f16 MFMA, f32 softmax" % bits, "data": "synthetic",
+        "config": {"workload": "configs[3]: GQA decode attention, 16 query / 2 KV heads, head_dim 256, %d-bit KV "
+                               "(group 64, fp16 scale/bias), context %d, batch %d" % (bits, ctx_len, B),
+                   "frac_of_hbm_peak": round(step_b / dt / 1e9 / HBM_PEAK_GBPS, 4), "cache_sets_rotated": n_sets,
+                   "kernel_us": {k: round(v, 2) for k, v in kern.items()}},
+        "roofline": {"kernel": "attn_partial_mfma_kernel", "bound": "hbm", "achieved": round(part, 2),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(part / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_launch": kv_bytes, "avg_launch_us": round(kern["partial"], 2)},
+        "cpu_baseline": None,
+    }
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -152,6 +288,10 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     ctx = nv.Context(0, nv.ACT_BF16)
+    if a.workload != "decode":
+        line = run_prefill(nv, ctx, torch, a) if a.workload == "prefill" else run_attention(nv, ctx, torch, a)
+        print(json.dumps(line), flush=True)
+        return
     layers, stride = build_layers(nv, ctx, torch, a.bits, a.layers)
     torch.cuda.synchronize()
     r = run_config(nv, ctx, torch, layers, stride, a.bits, a.batch, a.steps, a.warmup, profile=True)

@@ -112,6 +112,7 @@ extern "C" int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream strea
     uint32_t chunk_len = ((len > 0 ? len : 1) + nc - 1) / nc;
     chunk_len = (chunk_len + 31) & ~31u;
     nc = ((len > 0 ? len : 1) + chunk_len - 1) / chunk_len;
+    if (nc > ATTN_MAX_CHUNKS) return NVMAI_ERR_UNSUPPORTED;      // cannot happen: nc <= 512 by construction
     const size_t heads_total = (size_t)batch * num_q_heads;
     rc = ws_begin(ctx, 2 * ws_round(heads_total * nc * 4) + ws_round(heads_total * nc * head_dim * 4));
     if (rc) return rc;
@@ -142,8 +143,9 @@ extern "C" int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream strea
     }
     {
         ProfScope ps(ctx, NVMAI_PROF_ATTN_COMBINE, s);
-        if (ctx->act == ACT_BF16) attn_combine_kernel<ACT_BF16><<<dim3((uint32_t)heads_total), 256, 0, s>>>(p);
-        else attn_combine_kernel<ACT_FP16><<<dim3((uint32_t)heads_total), 256, 0, s>>>(p);
+        const dim3 cgrid((uint32_t)heads_total, (head_dim + 63) / 64);
+        if (ctx->act == ACT_BF16) attn_combine_kernel<ACT_BF16><<<cgrid, 256, 0, s>>>(p);
+        else attn_combine_kernel<ACT_FP16><<<cgrid, 256, 0, s>>>(p);
     }
     return launch_status();
 }

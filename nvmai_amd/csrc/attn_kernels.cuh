@@ -147,27 +147,52 @@ __global__ __launch_bounds__(256) void attn_partial_generic_kernel(AttnParams p)
 }
 
 // Combine (attention.metal:388-429): m* = max m_c, D = sum d_c e^(m_c - m*),
-// out = sum o_c e^(m_c - m*) / D; all chunks empty -> zeros.  One block per (batch, q head).
+// out = sum o_c e^(m_c - m*) / D; all chunks empty -> zeros.  Grid (batch * q heads,
+// ceil(head_dim / 64)); the four waves of a block split the chunks of 64 output dims.
+constexpr uint32_t ATTN_MAX_CHUNKS = 512;
+
 template <int ACT>
 __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
+    __shared__ float wgt[ATTN_MAX_CHUNKS];
+    __shared__ float red[8];
+    __shared__ float part[4][64];
     const size_t bh = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* mr = p.m_part + bh * p.num_chunks;
     const float* dr = p.d_part + bh * p.num_chunks;
     const float* orow = p.o_part + bh * p.num_chunks * p.head_dim;
-    uint16_t* out = (uint16_t*)p.out + bh * p.head_dim;
-    float mg = -INFINITY;
-    for (uint32_t c = 0; c < p.num_chunks; ++c) mg = fmaxf(mg, mr[c]);
-    if (mg == -INFINITY) {
-        for (uint32_t i = threadIdx.x; i < p.head_dim; i += 256) out[i] = f32_to_act<ACT>(0.0f);
+    const uint32_t dim = blockIdx.y * 64 + lane;
+    float mloc = -INFINITY;
+    for (uint32_t c = threadIdx.x; c < p.num_chunks; c += 256) mloc = fmaxf(mloc, mr[c]);
+    mloc = wave_max_f32(mloc);
+    if (lane == 0) red[wave] = mloc;
+    __syncthreads();
+    const float mg = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    if (mg == -INFINITY) {                                   // uniform over the block
+        if (wave == 0 && dim < p.head_dim) ((uint16_t*)p.out)[bh * p.head_dim + dim] = f32_to_act<ACT>(0.0f);
         return;
     }
-    float D = 0.0f;
-    for (uint32_t c = 0; c < p.num_chunks; ++c) D += dr[c] * expf(mr[c] - mg);
-    const float inv = D > 0.0f ? 1.0f / D : 0.0f;
-    for (uint32_t i = threadIdx.x; i < p.head_dim; i += 256) {
-        float acc = 0.0f;
-        for (uint32_t c = 0; c < p.num_chunks; ++c) acc += orow[(size_t)c * p.head_dim + i] * expf(mr[c] - mg);
-        out[i] = f32_to_act<ACT>(acc * inv);
+    float dloc = 0.0f;
+    for (uint32_t c = threadIdx.x; c < p.num_chunks; c += 256) {
+        const float w = expf(mr[c] - mg);
+        wgt[c] = w;
+        dloc += dr[c] * w;
+    }
+    dloc = wave_sum_bcast(dloc);
+    if (lane == 0) red[4 + wave] = dloc;
+    __syncthreads();
+    const float D = (red[4] + red[5]) + (red[6] + red[7]);
+    float acc = 0.0f;
+    if (dim < p.head_dim) {
+        const float* oc = orow + dim;
+#pragma unroll 8
+        for (uint32_t c = wave; c < p.num_chunks; c += 4) acc += oc[(size_t)c * p.head_dim] * wgt[c];
+    }
+    part[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && dim < p.head_dim) {
+        const float tot = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+        ((uint16_t*)p.out)[bh * p.head_dim + dim] = f32_to_act<ACT>(D > 0.0f ? tot / D : 0.0f);
     }
 }
 

@@ -34,7 +34,8 @@ extern "C" int nvmai_hip_prefill_make_pairs(nvmai_hip_ctx* ctx, nvmai_stream str
 
 namespace {
 
-constexpr uint32_t MAX_GROUP_EXPERTS = 4096;   // three u32 arrays of the scan kernel in 48 KB of LDS
+constexpr uint32_t MAX_GROUP_EXPERTS = 2048;   // five u32 arrays of the scan kernel in 40 KB of LDS
+constexpr int ERR_WORD = 8;                    // index into the context's persistent zeroed words
 
 int check_grouping(const nvmai_prefill_grouping* g, uint64_t n_pairs) {
     if (!g || (n_pairs && !g->sorted_pairs) || !g->expert_offsets || !g->expert_counts || !g->groups || !g->tiles || !g->info)
@@ -45,18 +46,18 @@ int check_grouping(const nvmai_prefill_grouping* g, uint64_t n_pairs) {
 // Shared tail: histogram, scan, scatter over slot-ordered expert ids.
 int group_slots(nvmai_hip_ctx* ctx, hipStream_t s, const uint32_t* slot_expert, const uint32_t* w32,
                 const uint16_t* w16, uint32_t n_pairs, uint32_t top_k, uint32_t num_experts,
-                uint32_t tile_expert_count, const uint64_t* sort_keys, uint32_t* block_hist, uint32_t* words,
-                bool report_range, const nvmai_prefill_grouping* out) {
+                uint32_t tile_expert_count, const uint64_t* sort_keys, uint32_t* block_hist, uint32_t* block_base,
+                uint32_t* words, bool report_range, const nvmai_prefill_grouping* out) {
     const uint32_t n_blocks = (n_pairs + GROUP_CHUNK - 1) / GROUP_CHUNK;
     if (n_blocks)
         prefill_hist_kernel<<<n_blocks, 256, num_experts * 4, s>>>(slot_expert, n_pairs, num_experts, block_hist, words,
                                                                   report_range);
-    prefill_scan_kernel<<<1, 1024, 3 * num_experts * 4, s>>>(
-        block_hist, n_blocks, num_experts, sort_keys, tile_expert_count, out->expert_offsets, out->expert_counts,
+    prefill_scan_kernel<<<1, 1024, (5 * num_experts + 32) * 4, s>>>(
+        block_hist, block_base, n_blocks, num_experts, sort_keys, tile_expert_count, out->expert_offsets, out->expert_counts,
         reinterpret_cast<PrefillGroup*>(out->groups), reinterpret_cast<PrefillTile*>(out->tiles), words, out->info);
     if (n_blocks)
         prefill_scatter_kernel<<<n_blocks, 256, GROUP_CHUNK * 4, s>>>(slot_expert, w32, w16, n_pairs, top_k, num_experts,
-                                                                    block_hist, reinterpret_cast<PrefillPair*>(out->sorted_pairs));
+                                                                    block_base, reinterpret_cast<PrefillPair*>(out->sorted_pairs));
     return launch_status();
 }
 
@@ -75,25 +76,26 @@ extern "C" int nvmai_hip_prefill_group_pairs(nvmai_hip_ctx* ctx, nvmai_stream st
         return NVMAI_ERR_INVALID_ARG;
     if (n_pairs >= (1u << 28) || num_experts > MAX_GROUP_EXPERTS) return NVMAI_ERR_UNSUPPORTED;
     const uint32_t n = (uint32_t)n_pairs, n_blocks = (n + GROUP_CHUNK - 1) / GROUP_CHUNK;
-    rc = ws_begin(ctx, 3 * ws_round((size_t)n * 4) + ws_round((size_t)n_blocks * num_experts * 4) + ws_round(64));
+    rc = ws_begin(ctx, 3 * ws_round((size_t)n * 4) + 2 * ws_round((size_t)n_blocks * num_experts * 4));
     if (rc) return rc;
     uint32_t* first = ws_take<uint32_t>(ctx, n);
     uint32_t* slot_expert = ws_take<uint32_t>(ctx, n);
     uint32_t* slot_weight = ws_take<uint32_t>(ctx, n);
     uint32_t* block_hist = ws_take<uint32_t>(ctx, (size_t)n_blocks * num_experts);
-    uint32_t* words = ws_take<uint32_t>(ctx, 16);
+    uint32_t* block_base = ws_take<uint32_t>(ctx, (size_t)n_blocks * num_experts);
+    uint32_t* words = ctx->tickets + ERR_WORD;
     hipStream_t s = (hipStream_t)stream;
     ProfScope prof(ctx, NVMAI_PROF_PREFILL_GROUP, s);
-    const uint32_t grid = n ? (n + 255) / 256 : 1;
-    prefill_init_kernel<<<grid, 256, 0, s>>>(first, n, words);
+    const uint32_t grid = (n + 255) / 256;
     if (n) {
+        prefill_init_kernel<<<grid, 256, 0, s>>>(first, n);
         prefill_claim_kernel<<<grid, 256, 0, s>>>(reinterpret_cast<const PrefillPair*>(pairs), n, query_count, top_k,
                                                   num_experts, first, words);
         prefill_slot_kernel<<<grid, 256, 0, s>>>(reinterpret_cast<const PrefillPair*>(pairs), n, query_count, top_k,
                                                  num_experts, first, slot_expert, slot_weight, words);
     }
     return group_slots(ctx, s, slot_expert, slot_weight, nullptr, n, top_k, num_experts, tile_expert_count, sort_keys,
-                       block_hist, words, false, out);
+                       block_hist, block_base, words, false, out);
 }
 
 extern "C" int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint32_t* idx,
@@ -110,15 +112,14 @@ extern "C" int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream s
         return NVMAI_ERR_INVALID_ARG;
     if (n_pairs >= (1u << 28) || num_experts > MAX_GROUP_EXPERTS) return NVMAI_ERR_UNSUPPORTED;
     const uint32_t n = (uint32_t)n_pairs, n_blocks = (n + GROUP_CHUNK - 1) / GROUP_CHUNK;
-    rc = ws_begin(ctx, ws_round((size_t)n_blocks * num_experts * 4) + ws_round(64));
+    rc = ws_begin(ctx, 2 * ws_round((size_t)n_blocks * num_experts * 4));
     if (rc) return rc;
     uint32_t* block_hist = ws_take<uint32_t>(ctx, (size_t)n_blocks * num_experts);
-    uint32_t* words = ws_take<uint32_t>(ctx, 16);
+    uint32_t* block_base = ws_take<uint32_t>(ctx, (size_t)n_blocks * num_experts);
     hipStream_t s = (hipStream_t)stream;
     ProfScope prof(ctx, NVMAI_PROF_PREFILL_GROUP, s);
-    prefill_init_kernel<<<1, 256, 0, s>>>(nullptr, 0, words);
-    return group_slots(ctx, s, idx, nullptr, w, n, top_k, num_experts, tile_expert_count, sort_keys, block_hist, words, true,
-                       out);
+    return group_slots(ctx, s, idx, nullptr, w, n, top_k, num_experts, tile_expert_count, sort_keys, block_hist,
+                       block_base, ctx->tickets + ERR_WORD, true, out);
 }
 
 namespace {

@@ -15,16 +15,15 @@ struct PrefillTile { uint32_t group_start, group_count, pair_start, pair_count; 
 constexpr int GROUP_CHUNK = 1024;     // slots per block of the histogram / scatter passes
 
 // Device-side validation failures, numbered like PrefillMoEGroupingError's cases
-// (PrefillMoEGrouping.swift:121-137).  The error word holds min over pairs of (index << 4 | code),
-// i.e. the first failing pair in input order, as the reference's loop reports it.
+// (PrefillMoEGrouping.swift:121-137).  The error word holds max over pairs of ~(index << 4 | code),
+// i.e. the first failing pair in input order, as the reference's loop reports it; 0 = none.
+// It lives in the context's persistent zeroed words and the scan kernel clears it again.
 enum : uint32_t { GROUP_ERR_TOKEN = 6, GROUP_ERR_RANK = 7, GROUP_ERR_EXPERT = 8, GROUP_ERR_DUP = 9 };
-constexpr uint32_t GROUP_NO_ERR = 0xFFFFFFFFu;
+constexpr uint32_t GROUP_UNCLAIMED = 0xFFFFFFFFu;
 
-// Workspace words: [0] error word.
-__global__ __launch_bounds__(256) void prefill_init_kernel(uint32_t* first, uint32_t n_pairs, uint32_t* words) {
+__global__ __launch_bounds__(256) void prefill_init_kernel(uint32_t* first, uint32_t n_pairs) {
     const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-    if (first && i < n_pairs) first[i] = GROUP_NO_ERR;
-    if (i == 0) words[0] = GROUP_NO_ERR;
+    if (i < n_pairs) first[i] = GROUP_UNCLAIMED;
 }
 
 // PrefillRouter.makeTokenExpertPairs (PrefillRouter.swift:97-117): token-major records.
@@ -49,7 +48,7 @@ __global__ __launch_bounds__(256) void prefill_claim_kernel(const PrefillPair* p
     if (p.token >= query_count) code = GROUP_ERR_TOKEN;
     else if (p.rank >= top_k) code = GROUP_ERR_RANK;
     else if (p.expert >= num_experts) code = GROUP_ERR_EXPERT;
-    if (code) atomicMin(&words[0], i << 4 | code);
+    if (code) atomicMax(&words[0], ~(i << 4 | code));
     else atomicMin(&first[p.token * top_k + p.rank], i);
 }
 
@@ -64,7 +63,7 @@ __global__ __launch_bounds__(256) void prefill_slot_kernel(const PrefillPair* pa
     if (p.token >= query_count || p.rank >= top_k || p.expert >= num_experts) return;
     const uint32_t slot = p.token * top_k + p.rank;
     if (first[slot] == i) { slot_expert[slot] = p.expert; slot_weight[slot] = p.weight_bits; }
-    else atomicMin(&words[0], i << 4 | GROUP_ERR_DUP);       // a later pair of an already seen slot
+    else atomicMax(&words[0], ~(i << 4 | GROUP_ERR_DUP));       // a later pair of an already seen slot
 }
 
 // ---- pass 1: per-block histogram of expert ids ------------------------------------------
@@ -81,34 +80,57 @@ __global__ __launch_bounds__(256) void prefill_hist_kernel(const uint32_t* idx, 
     for (uint32_t i = threadIdx.x; i < GROUP_CHUNK && base + i < n_pairs; i += 256) {
         const uint32_t e = idx[base + i];
         if (e < num_experts) atomicAdd(&lds[e], 1u);
-        else if (report) atomicMin(&words[0], (base + i) << 4 | GROUP_ERR_EXPERT);
+        else if (report) atomicMax(&words[0], ~((base + i) << 4 | GROUP_ERR_EXPERT));
     }
     __syncthreads();
     for (uint32_t e = threadIdx.x; e < num_experts; e += 256) block_hist[(size_t)blockIdx.x * num_experts + e] = lds[e];
 }
 
 // ---- pass 2: offsets, counts, groups, tiles (PrefillMoEGrouping.swift:151-184) ------------
+// Exclusive scan over the 1024 threads of the block; `total` is the sum over all of them.
+__device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t* wave_tot, uint32_t& total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t inc = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t t = (uint32_t)__shfl_up((int)inc, off, 64);
+        if (lane >= off) inc += t;
+    }
+    if (lane == 63) wave_tot[wave] = inc;
+    __syncthreads();
+    uint32_t before = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+        const uint32_t t = wave_tot[w];
+        before += w < wave ? t : 0u;
+        tot += t;
+    }
+    __syncthreads();
+    total = tot;
+    return before + inc - v;
+}
+
 // One block.  Experts are laid out in ascending (sort key, expert) order; offsets of empty
-// experts are 0xFFFFFFFF.  block_hist is turned into each block's first slot per expert.
+// experts are 0xFFFFFFFF.  block_base[b][e] = first sorted slot of expert e's pairs of block b.
 // info: [0] groups, [1] tiles, [2] error code (0 = none), [3] index of the failing pair,
-// [4] largest group.
-__global__ __launch_bounds__(1024) void prefill_scan_kernel(uint32_t* block_hist, uint32_t n_blocks,
+// [4] largest group.  The error word is read and cleared for the next call.
+__global__ __launch_bounds__(1024) void prefill_scan_kernel(const uint32_t* __restrict__ block_hist,
+                                                           uint32_t* __restrict__ block_base, uint32_t n_blocks,
                                                            uint32_t num_experts, const uint64_t* sort_keys,
                                                            uint32_t tile_expert_count, uint32_t* offsets,
                                                            uint32_t* counts, PrefillGroup* groups,
-                                                           PrefillTile* tiles, const uint32_t* words,
-                                                           uint32_t* info) {
+                                                           PrefillTile* tiles, uint32_t* err_word, uint32_t* info) {
     extern __shared__ uint32_t lds[];
-    uint32_t* cnt = lds;                       // [E]
+    uint32_t* cnt = lds;                       // [E] pairs of expert e
     uint32_t* order = lds + num_experts;       // [E] expert at position i of the key order
-    uint32_t* start = lds + 2 * num_experts;   // [E] first pair of the expert
+    uint32_t* start = lds + 2 * num_experts;   // [E] first pair of expert e
+    uint32_t* gstart = lds + 3 * num_experts;  // [E] first pair of group g
+    uint32_t* gcount = lds + 4 * num_experts;  // [E] pairs of group g
+    uint32_t* misc = lds + 5 * num_experts;    // [0..15] wave totals, [16] largest group
+    if (threadIdx.x == 0) misc[16] = 0;
     for (uint32_t e = threadIdx.x; e < num_experts; e += 1024) {
         uint32_t total = 0;
-        for (uint32_t b = 0; b < n_blocks; ++b) {
-            const uint32_t c = block_hist[(size_t)b * num_experts + e];
-            block_hist[(size_t)b * num_experts + e] = total;      // exclusive prefix over blocks
-            total += c;
-        }
+        for (uint32_t b = 0; b < n_blocks; ++b) total += block_hist[(size_t)b * num_experts + e];
         cnt[e] = total;
         uint32_t pos = e;
         if (sort_keys) {                                          // rank in (key, expert) order
@@ -122,34 +144,54 @@ __global__ __launch_bounds__(1024) void prefill_scan_kernel(uint32_t* block_hist
         order[pos] = e;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {                                       // serial walk over the experts
-        uint32_t run = 0, ng = 0, nt = 0, max_pairs = 0;
-        for (uint32_t i = 0; i < num_experts; ++i) {
-            const uint32_t ex = order[i], c = cnt[ex];
-            start[ex] = run;
-            if (c) {
-                groups[ng++] = PrefillGroup{ex, run, c};
-                max_pairs = max(max_pairs, c);
-            }
-            run += c;
+    uint32_t pair_carry = 0, group_carry = 0;
+    for (uint32_t base = 0; base < num_experts; base += 1024) {   // uniform trip count
+        const uint32_t i = base + threadIdx.x;
+        const uint32_t ex = i < num_experts ? order[i] : 0u;
+        const uint32_t c = i < num_experts ? cnt[ex] : 0u;
+        uint32_t pair_total, group_total;
+        const uint32_t first = pair_carry + block_excl_scan(c, misc, pair_total);
+        const uint32_t g = group_carry + block_excl_scan(c ? 1u : 0u, misc, group_total);
+        if (i < num_experts) start[ex] = first;
+        if (c) {
+            groups[g] = PrefillGroup{ex, first, c};
+            gstart[g] = first;
+            gcount[g] = c;
+            atomicMax(&misc[16], c);
         }
-        for (uint32_t gs = 0; gs < ng; gs += tile_expert_count) {
-            const uint32_t ge = min(ng, gs + tile_expert_count);
-            const PrefillGroup a = groups[gs], z = groups[ge - 1];
-            tiles[nt++] = PrefillTile{gs, ge - gs, a.pair_start, z.pair_start + z.pair_count - a.pair_start};
-        }
-        const uint32_t err = words[0];
-        info[0] = ng;
-        info[1] = nt;
-        info[2] = err == GROUP_NO_ERR ? 0u : (err & 15u);
-        info[3] = err == GROUP_NO_ERR ? 0u : (err >> 4);
-        info[4] = max_pairs;
+        pair_carry += pair_total;
+        group_carry += group_total;
     }
     __syncthreads();
+    const uint32_t ng = group_carry;
+    const uint32_t nt = (ng + tile_expert_count - 1) / tile_expert_count;
+    for (uint32_t t = threadIdx.x; t < nt; t += 1024) {
+        const uint32_t gs = t * tile_expert_count, ge = min(ng, gs + tile_expert_count);
+        tiles[t] = PrefillTile{gs, ge - gs, gstart[gs], gstart[ge - 1] + gcount[ge - 1] - gstart[gs]};
+    }
+    if (threadIdx.x == 0) {
+        const uint32_t err = *err_word;            // 0 = none, else ~(index << 4 | code)
+        *err_word = 0;
+        info[0] = ng;
+        info[1] = nt;
+        info[2] = err ? (~err & 15u) : 0u;
+        info[3] = err ? (~err >> 4) : 0u;
+        info[4] = misc[16];
+    }
     for (uint32_t e = threadIdx.x; e < num_experts; e += 1024) {
         counts[e] = cnt[e];
         offsets[e] = cnt[e] ? start[e] : 0xFFFFFFFFu;
-        for (uint32_t b = 0; b < n_blocks; ++b) block_hist[(size_t)b * num_experts + e] += start[e];
+        uint32_t run = start[e];
+        for (uint32_t b0 = 0; b0 < n_blocks; b0 += 8) {
+            uint32_t c[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) c[j] = b0 + j < n_blocks ? block_hist[(size_t)(b0 + j) * num_experts + e] : 0u;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                if (b0 + j < n_blocks) block_base[(size_t)(b0 + j) * num_experts + e] = run;
+                run += c[j];
+            }
+        }
     }
 }
 
@@ -235,6 +277,7 @@ struct GemmParams {
 
 constexpr int GEMM_BK = 64;
 constexpr int GEMM_LDK = GEMM_BK + 8;   // padded row: conflict-free 16-byte reads
+constexpr int GEMM_STAGES = 3;
 
 // Two floats -> two 16-bit activations in one dword, round to nearest even.
 template <int ACT>
@@ -283,25 +326,27 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(GemmParams p) {
     const uint16_t* srow_p = reinterpret_cast<const uint16_t*>(blob + (w_is_b ? p.sB : p.sA)) + (size_t)wn_row * groups;
     const uint16_t* brow_p = reinterpret_cast<const uint16_t*>(blob + (w_is_b ? p.bB : p.bA)) + (size_t)wn_row * groups;
 
-    uint4 xreg[4], wreg[BITS == 8 ? 2 : 1];
-    uint16_t sreg, breg;
-    auto load_regs = [&](uint32_t ks) {
+    // Register stages: the global loads of k step ks + GEMM_STAGES are issued while step ks is
+    // multiplied, so that a load has about GEMM_STAGES MFMA phases to arrive.
+    struct Stage { uint4 x[4]; uint4 w[BITS == 8 ? 2 : 1]; uint16_t s, b; };
+    Stage st[GEMM_STAGES];
+    auto load_regs = [&](Stage& g, uint32_t ks) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) xreg[j] = *reinterpret_cast<const uint4*>(xrow + ks * GEMM_BK + j * 8);
+        for (int j = 0; j < 4; ++j) g.x[j] = *reinterpret_cast<const uint4*>(xrow + ks * GEMM_BK + j * 8);
         const uint8_t* wp = wrow + (size_t)ks * (GEMM_BK * BITS / 8);
-        wreg[0] = *reinterpret_cast<const uint4*>(wp);
-        if (BITS == 8) wreg[BITS == 8 ? 1 : 0] = *reinterpret_cast<const uint4*>(wp + 16);
-        sreg = srow_p[ks];
-        breg = brow_p[ks];
+        g.w[0] = *reinterpret_cast<const uint4*>(wp);
+        if (BITS == 8) g.w[BITS == 8 ? 1 : 0] = *reinterpret_cast<const uint4*>(wp + 16);
+        g.s = srow_p[ks];
+        g.b = brow_p[ks];
     };
-    auto store_regs = [&](int buf) {
+    auto store_regs = [&](const Stage& g, int buf) {
         uint16_t* xd = xs + (buf * GEMM_BM + srow) * GEMM_LDK + shalf * 32;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(xd + j * 8) = xreg[j];
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(xd + j * 8) = g.x[j];
         uint16_t* wd = ws + (buf * GEMM_BM + srow) * GEMM_LDK + shalf * 32;
-        const float s = bf16_to_f32(sreg), b = bf16_to_f32(breg);
+        const float s = bf16_to_f32(g.s), b = bf16_to_f32(g.b);
         if (BITS == 4) {
-            const uint32_t words[4] = {wreg[0].x, wreg[0].y, wreg[0].z, wreg[0].w};
+            const uint32_t words[4] = {g.w[0].x, g.w[0].y, g.w[0].z, g.w[0].w};
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
                 float q[8];
@@ -316,7 +361,7 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(GemmParams p) {
         } else {
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const uint4 wq = wreg[BITS == 8 ? h : 0];
+                const uint4 wq = g.w[BITS == 8 ? h : 0];
                 const uint32_t words[4] = {wq.x, wq.y, wq.z, wq.w};
 #pragma unroll
                 for (int d = 0; d < 2; ++d) {
@@ -341,31 +386,39 @@ __global__ __launch_bounds__(256) void prefill_gemm_kernel(GemmParams p) {
         for (int j = 0; j < 4; ++j) acc[a][j] = fl4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     const uint32_t nk = p.K / GEMM_BK;
-    load_regs(0);
-    store_regs(0);
+#pragma unroll
+    for (int j = 0; j < GEMM_STAGES; ++j)
+        if ((uint32_t)j < nk) load_regs(st[j], j);
+    store_regs(st[0], 0);
     __syncthreads();
-    for (uint32_t ks = 0; ks < nk; ++ks) {
-        const int buf = ks & 1;
-        if (ks + 1 < nk) load_regs(ks + 1);
+    for (uint32_t ks0 = 0; ks0 < nk; ks0 += GEMM_STAGES) {
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-            uint4 afrag[4], bfrag[4];
+        for (int j = 0; j < GEMM_STAGES; ++j) {
+            const uint32_t ks = ks0 + j;
+            if (ks >= nk) break;
+            const int buf = ks & 1;
+            // step ks went from st[j] to LDS one iteration ago: st[j] is free again
+            if (ks + GEMM_STAGES < nk) load_regs(st[j], ks + GEMM_STAGES);
 #pragma unroll
-            for (int a = 0; a < 4; ++a)
-                afrag[a] = *reinterpret_cast<const uint4*>(xs + (buf * GEMM_BM + wm * 64 + a * 16 + li) * GEMM_LDK + kk * 32 + lq * 8);
+            for (int kk = 0; kk < 2; ++kk) {
+                uint4 afrag[4], bfrag[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int brow = DUAL ? (j >> 1) * 64 + wn * 32 + (j & 1) * 16 + li : wn * 64 + j * 16 + li;
-                bfrag[j] = *reinterpret_cast<const uint4*>(ws + (buf * GEMM_BM + brow) * GEMM_LDK + kk * 32 + lq * 8);
+                for (int a = 0; a < 4; ++a)
+                    afrag[a] = *reinterpret_cast<const uint4*>(xs + (buf * GEMM_BM + wm * 64 + a * 16 + li) * GEMM_LDK + kk * 32 + lq * 8);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int brow = DUAL ? (t >> 1) * 64 + wn * 32 + (t & 1) * 16 + li : wn * 64 + t * 16 + li;
+                    bfrag[t] = *reinterpret_cast<const uint4*>(ws + (buf * GEMM_BM + brow) * GEMM_LDK + kk * 32 + lq * 8);
+                }
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        acc[a][t] = mfma_16x16x32<ACT>(afrag[a], bfrag[t], acc[a][t]);
             }
-#pragma unroll
-            for (int a = 0; a < 4; ++a)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[a][j] = mfma_16x16x32<ACT>(afrag[a], bfrag[j], acc[a][j]);
+            if (ks + 1 < nk) store_regs(st[(j + 1) % GEMM_STAGES], buf ^ 1);
+            __syncthreads();
         }
-        if (ks + 1 < nk) store_regs(buf ^ 1);
-        __syncthreads();
     }
 
     // ---- epilogue: lane holds column li of each tile, rows 4*lq .. 4*lq+3
