@@ -56,7 +56,7 @@ int group_slots(nvmai_hip_ctx* ctx, hipStream_t s, const uint32_t* slot_expert, 
         block_hist, block_base, n_blocks, num_experts, sort_keys, tile_expert_count, out->expert_offsets, out->expert_counts,
         reinterpret_cast<PrefillGroup*>(out->groups), reinterpret_cast<PrefillTile*>(out->tiles), words, out->info);
     if (n_blocks)
-        prefill_scatter_kernel<<<n_blocks, 256, GROUP_CHUNK * 4, s>>>(slot_expert, w32, w16, n_pairs, top_k, num_experts,
+        prefill_scatter_kernel<<<n_blocks, 256, num_experts * 4, s>>>(slot_expert, w32, w16, n_pairs, top_k, num_experts,
                                                                     block_base, reinterpret_cast<PrefillPair*>(out->sorted_pairs));
     return launch_status();
 }
@@ -125,8 +125,8 @@ extern "C" int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream s
 namespace {
 
 template <int ACT, int BITS>
-void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t max_mtiles, nvmai_hip_ctx* ctx, hipStream_t s) {
-    const size_t lds = (size_t)4 * GEMM_BM * GEMM_LDK * 2;     // 72 KB: above the 64 KB a launch gets unasked
+void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t mtiles8, nvmai_hip_ctx* ctx, hipStream_t s) {
+    const size_t lds = (size_t)2 * GEMM_BM * GEMM_LDK * 2;     // 68 KB: above the 64 KB a launch gets unasked
     static bool raised = false;
     if (!raised) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, true>),
@@ -137,11 +137,11 @@ void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t max_mtile
     }
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM1, s);
-        prefill_gemm_kernel<ACT, BITS, true><<<max_mtiles * g1.n_tiles_n, 256, lds, s>>>(g1);
+        prefill_gemm_kernel<ACT, BITS, true><<<mtiles8 * g1.n_tiles_n, 256, lds, s>>>(g1);
     }
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM2, s);
-        prefill_gemm_kernel<ACT, BITS, false><<<max_mtiles * g2.n_tiles_n, 256, lds, s>>>(g2);
+        prefill_gemm_kernel<ACT, BITS, false><<<mtiles8 * g2.n_tiles_n, 256, lds, s>>>(g2);
     }
 }
 
@@ -194,11 +194,11 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
     g2.out = route_partials; g2.out_stride = d;
     g2.K = f; g2.N = d; g2.n_tiles_n = (d + 127) / 128;
     if (ctx->act == ACT_BF16) {
-        if (bits == 4) launch_gemms<ACT_BF16, 4>(g1, g2, max_mtiles, ctx, s);
-        else launch_gemms<ACT_BF16, 8>(g1, g2, max_mtiles, ctx, s);
+        if (bits == 4) launch_gemms<ACT_BF16, 4>(g1, g2, (max_mtiles + 7) / 8 * 8, ctx, s);
+        else launch_gemms<ACT_BF16, 8>(g1, g2, (max_mtiles + 7) / 8 * 8, ctx, s);
     } else {
-        if (bits == 4) launch_gemms<ACT_FP16, 4>(g1, g2, max_mtiles, ctx, s);
-        else launch_gemms<ACT_FP16, 8>(g1, g2, max_mtiles, ctx, s);
+        if (bits == 4) launch_gemms<ACT_FP16, 4>(g1, g2, (max_mtiles + 7) / 8 * 8, ctx, s);
+        else launch_gemms<ACT_FP16, 8>(g1, g2, (max_mtiles + 7) / 8 * 8, ctx, s);
     }
     return launch_status();
 }

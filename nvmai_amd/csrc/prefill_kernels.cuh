@@ -196,24 +196,45 @@ __global__ __launch_bounds__(1024) void prefill_scan_kernel(const uint32_t* __re
 }
 
 // ---- pass 3: stable scatter ---------------------------------------------------------------
-// Slots ascend in (token, rank); inside a block thread e walks the block's slots in order and
-// places those of expert e, which keeps (token, rank) ascending inside every expert: the
-// order PrefillMoEGrouping.swift:140-149 sorts into.
+// Slots ascend in (token, rank).  A block places its slots 256 at a time; inside a round the
+// four waves take turns, and inside a wave a lane's place among the lanes of the same expert
+// comes from a ballot, so every expert keeps (token, rank) ascending: the order
+// PrefillMoEGrouping.swift:140-149 sorts into.
 __global__ __launch_bounds__(256) void prefill_scatter_kernel(const uint32_t* idx, const uint32_t* w32,
                                                              const uint16_t* w16, uint32_t n_pairs,
                                                              uint32_t top_k, uint32_t num_experts,
                                                              const uint32_t* block_base, PrefillPair* sorted) {
-    extern __shared__ uint32_t lds[];     // [GROUP_CHUNK] expert ids of this block
-    const uint32_t base = blockIdx.x * GROUP_CHUNK;
-    const uint32_t n = min((uint32_t)GROUP_CHUNK, n_pairs - base);
-    for (uint32_t i = threadIdx.x; i < n; i += 256) lds[i] = idx[base + i];
+    extern __shared__ uint32_t next[];    // [E] next free sorted slot of each expert
+    for (uint32_t e = threadIdx.x; e < num_experts; e += 256) next[e] = block_base[(size_t)blockIdx.x * num_experts + e];
     __syncthreads();
-    for (uint32_t e = threadIdx.x; e < num_experts; e += 256) {
-        uint32_t pos = block_base[(size_t)blockIdx.x * num_experts + e];
-        for (uint32_t i = 0; i < n; ++i) {
-            if (lds[i] != e) continue;
-            const uint32_t p = base + i;
-            sorted[pos++] = PrefillPair{p / top_k, e, p % top_k, w32 ? w32[p] : (uint32_t)w16[p]};
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t base = blockIdx.x * GROUP_CHUNK;
+    for (uint32_t r = 0; r < GROUP_CHUNK / 256; ++r) {          // uniform trip count: barriers inside
+        const uint32_t p = base + r * 256 + threadIdx.x;
+        uint32_t e = p < n_pairs ? idx[p] : 0xFFFFFFFFu;
+        const bool valid = e < num_experts;
+        const uint32_t wbits = valid ? (w32 ? w32[p] : (uint32_t)w16[p]) : 0u;
+        uint32_t rank = 0, total = 0;
+        bool leader = false;
+        unsigned long long todo = __ballot(valid);
+        while (todo) {                                           // one turn per distinct expert in the wave
+            const int first = __builtin_ctzll(todo);
+            const uint32_t le = (uint32_t)__builtin_amdgcn_readlane((int)e, first);
+            const unsigned long long m = __ballot(valid && e == le);
+            if (valid && e == le) {
+                rank = (uint32_t)__builtin_popcountll(m & ((1ull << lane) - 1ull));
+                total = (uint32_t)__builtin_popcountll(m);
+                leader = lane == (uint32_t)first;
+            }
+            todo &= ~m;
+        }
+        for (uint32_t w = 0; w < 4; ++w) {
+            if (wave == w && valid) {
+                const uint32_t pos = next[e] + rank;             // every lane reads before the leader adds
+                sorted[pos] = PrefillPair{p / top_k, e, p % top_k, wbits};
+                if (leader) next[e] += total;
+            }
+            __syncthreads();
         }
     }
 }
@@ -247,13 +268,19 @@ __global__ __launch_bounds__(256) void prefill_mtiles_kernel(const PrefillGroup*
 
 // ---- grouped GEMM ---------------------------------------------------------------------------
 // out[m, n] = sum_k X[row(m), k] * W_e[n, k] for the rows of one M tile (<= 128 sorted pairs of
-// one expert) and 128 weight rows: DUAL -> 64 gate rows + the same 64 up rows, epilogue
-// silu(g) * u (prefill.metal:460-501); else 128 down rows (prefill.metal:503-534).
-// Per 64-wide k step (one quantization group) each thread dequantizes half a weight row:
-// w = q * scale + bias in fp32, rounded once to the activation type (the reference dequantizes
-// to fp16, tensorops.metal:29-121), into an LDS tile; the activations go to LDS as they are.
-// v_mfma_f32_16x16x32_{bf16,f16} accumulates in fp32.  Wave (wm, wn) owns rows wm*64..+64 and four
-// 16-column tiles: DUAL gate/up columns wn*32..+32, else columns wn*64..+64.
+// one expert) and GEMM_BN output columns: DUAL -> gate and up rows of the same columns,
+// epilogue silu(g) * u (prefill.metal:460-501); else down rows (prefill.metal:503-534).
+//
+// k runs in super-steps of 128 (two quantization groups).  The activations of a super-step go
+// through a double-buffered LDS tile shared by the four waves.  The weights never touch LDS:
+// wave w owns 16 * GEMM_NT columns of all 128 rows, and lane (i = lane % 16, q = lane / 16)
+// loads the 32 codes W[n_i, k0 + 32q .. +32) of each of its columns in one 16-byte (4 bit) or
+// two (8 bit) loads, so four neighbouring lanes cover 64 or 128 contiguous bytes of a row.
+// It dequantizes them in registers, w = q * scale + bias in fp32 rounded once to the activation
+// type (the reference dequantizes to fp16, tensorops.metal:29-121), straight into the MFMA B
+// operand: MFMA j of the super-step contracts k0 + 32q + 8j .. +8 over q = 0..3, and the A
+// operand is read from LDS with the same k assignment.  v_mfma_f32_16x16x32_{bf16,f16}
+// accumulates in fp32.
 typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 hf8_t __attribute__((ext_vector_type(8)));
@@ -275,9 +302,9 @@ struct GemmParams {
     uint32_t K, N, top_k, n_tiles_n;
 };
 
-constexpr int GEMM_BK = 64;
-constexpr int GEMM_LDK = GEMM_BK + 8;   // padded row: conflict-free 16-byte reads
-constexpr int GEMM_STAGES = 3;
+constexpr int GEMM_SK = 128;            // k per super-step
+constexpr int GEMM_LDK = GEMM_SK + 8;   // padded LDS row: conflict-free 16-byte reads and writes
+constexpr int GEMM_XST = 2;             // activation register stages in flight
 
 // Two floats -> two 16-bit activations in one dword, round to nearest even.
 template <int ACT>
@@ -294,158 +321,199 @@ __device__ __forceinline__ fl4_t mfma_16x16x32(const uint4& a, const uint4& b, f
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(hf8_t, a), __builtin_bit_cast(hf8_t, b), c, 0, 0, 0);
 }
 
+// Eight codes -> eight dequantized 16-bit values in MFMA operand order.
+template <int ACT>
+__device__ __forceinline__ uint4 dequant8(const float* q, float s, float b) {
+    uint4 o;
+    o.x = pack_act2<ACT>(fmaf(q[0], s, b), fmaf(q[1], s, b));
+    o.y = pack_act2<ACT>(fmaf(q[2], s, b), fmaf(q[3], s, b));
+    o.z = pack_act2<ACT>(fmaf(q[4], s, b), fmaf(q[5], s, b));
+    o.w = pack_act2<ACT>(fmaf(q[6], s, b), fmaf(q[7], s, b));
+    return o;
+}
+
 template <int ACT, int BITS, bool DUAL>
-__global__ __launch_bounds__(256) void prefill_gemm_kernel(GemmParams p) {
+__global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
+    constexpr int NT = 2;                               // 16-column tiles per wave
+    constexpr int WQ = BITS == 8 ? 2 : 1;               // 16-byte loads per (column, super-step)
+    constexpr int GEMM_WST = BITS == 8 ? 2 : 4;         // weight register stages in flight (register budget)
     extern __shared__ uint4 gemm_lds[];
-    uint16_t* lds = reinterpret_cast<uint16_t*>(gemm_lds);
-    // [2][128][LDK] activations, then [2][128][LDK] weights
-    uint16_t* xs = lds;
-    uint16_t* ws = lds + 2 * GEMM_BM * GEMM_LDK;
-    const uint32_t tile_id = blockIdx.x / p.n_tiles_n, nt = blockIdx.x % p.n_tiles_n;
+    uint16_t* xs = reinterpret_cast<uint16_t*>(gemm_lds);      // [2][128][LDK]
+    // Blocks are dealt to the eight XCDs round-robin.  The column tiles of one M tile go to one
+    // XCD, back to back, so that its activation rows are fetched into one L2 only; the M tiles
+    // themselves (sorted by size) are dealt over the XCDs in turn, which balances them.
+    const uint32_t on_xcd = blockIdx.x >> 3;
+    const uint32_t tile_id = (on_xcd / p.n_tiles_n) * 8 + (blockIdx.x & 7u), nt = on_xcd % p.n_tiles_n;
     if (tile_id >= *p.n_mtiles) return;
     const MTile mt = p.mtiles[tile_id];
     const uint8_t* blob = p.pool + (uint64_t)mt.expert * p.pool_stride;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1, li = lane & 15, lq = lane >> 4;
+    const int li = lane & 15, lq = lane >> 4;
     const uint32_t groups = p.K / NVMAI_GROUP;
-    const uint32_t n_cols = DUAL ? 64 : 128;              // output columns per block
+    const uint32_t n_cols = DUAL ? 64 : 128;            // output columns per block
     const uint32_t n0 = nt * n_cols;
 
-    // ---- this thread's staging duties: half an activation row and half a weight row
+    // ---- activation staging: thread (row, half) moves 64 elements of a row per super-step
+    // Rows past the end of a short tile are neither loaded nor multiplied: their LDS rows keep
+    // whatever they held, which only reaches accumulator rows that are never stored.
     const int srow = tid >> 1, shalf = tid & 1;
+    const bool x_live = (uint32_t)srow < mt.rows;
+    const int live_mt = (int)((mt.rows + 15) >> 4);     // 16-row tiles that hold any row
     const uint16_t* xrow;
     {
         const uint32_t m = (uint32_t)srow < mt.rows ? srow : 0;
         const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
-        xrow = (const uint16_t*)p.x + (size_t)src * p.x_stride + shalf * 32;
+        xrow = (const uint16_t*)p.x + (size_t)src * p.x_stride + shalf * 64;
     }
-    const bool w_is_b = DUAL && srow >= 64;
-    uint32_t wn_row = n0 + (DUAL ? (srow & 63) : srow);
-    if (wn_row >= p.N) wn_row = p.N - 1;
-    const uint8_t* wrow = blob + (w_is_b ? p.wB : p.wA) + (size_t)wn_row * (p.K * BITS / 8) + shalf * (32 * BITS / 8);
-    const uint16_t* srow_p = reinterpret_cast<const uint16_t*>(blob + (w_is_b ? p.sB : p.sA)) + (size_t)wn_row * groups;
-    const uint16_t* brow_p = reinterpret_cast<const uint16_t*>(blob + (w_is_b ? p.bB : p.bA)) + (size_t)wn_row * groups;
+    // ---- weight columns of this lane: tile t -> DUAL {gate, up} of column n0 + 16 wave + i,
+    //      else column n0 + 32 wave + 16 t + i
+    const uint8_t* wrow[NT];
+    const uint16_t* srow_p[NT];
+    const uint16_t* brow_p[NT];
+    uint32_t col[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        col[t] = DUAL ? n0 + wave * 16 + li : n0 + wave * 32 + t * 16 + li;
+        const uint32_t r = col[t] < p.N ? col[t] : p.N - 1;
+        const bool second = DUAL && t == 1;
+        wrow[t] = blob + (second ? p.wB : p.wA) + (size_t)r * (p.K * BITS / 8) + lq * (32 * BITS / 8);
+        srow_p[t] = reinterpret_cast<const uint16_t*>(blob + (second ? p.sB : p.sA)) + (size_t)r * groups + (lq >> 1);
+        brow_p[t] = reinterpret_cast<const uint16_t*>(blob + (second ? p.bB : p.bA)) + (size_t)r * groups + (lq >> 1);
+    }
 
-    // Register stages: the global loads of k step ks + GEMM_STAGES are issued while step ks is
-    // multiplied, so that a load has about GEMM_STAGES MFMA phases to arrive.
-    struct Stage { uint4 x[4]; uint4 w[BITS == 8 ? 2 : 1]; uint16_t s, b; };
-    Stage st[GEMM_STAGES];
-    auto load_regs = [&](Stage& g, uint32_t ks) {
+    const uint32_t nss = (p.K + GEMM_SK - 1) / GEMM_SK;
+    // A K that is an odd multiple of 64 leaves half of the last super-step empty: lanes whose k
+    // range lies beyond K contribute zeros (zero activations, zero weights).
+    const bool odd_tail = (p.K % GEMM_SK) != 0;
+
+    struct XStage { uint4 v[8]; };
+    struct WStage { uint4 w[NT][WQ]; uint16_t s[NT], b[NT]; };
+    XStage xst[GEMM_XST];
+    WStage wst[GEMM_WST];
+    auto load_x = [&](XStage& g, uint32_t ss) {
+        const bool dead = !x_live || (odd_tail && ss == nss - 1 && shalf == 1);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) g.x[j] = *reinterpret_cast<const uint4*>(xrow + ks * GEMM_BK + j * 8);
-        const uint8_t* wp = wrow + (size_t)ks * (GEMM_BK * BITS / 8);
-        g.w[0] = *reinterpret_cast<const uint4*>(wp);
-        if (BITS == 8) g.w[BITS == 8 ? 1 : 0] = *reinterpret_cast<const uint4*>(wp + 16);
-        g.s = srow_p[ks];
-        g.b = brow_p[ks];
+        for (int j = 0; j < 8; ++j)
+            g.v[j] = dead ? uint4{0, 0, 0, 0} : *reinterpret_cast<const uint4*>(xrow + ss * GEMM_SK + j * 8);
     };
-    auto store_regs = [&](const Stage& g, int buf) {
-        uint16_t* xd = xs + (buf * GEMM_BM + srow) * GEMM_LDK + shalf * 32;
+    auto load_w = [&](WStage& g, uint32_t ss) {
+        const bool dead = odd_tail && ss == nss - 1 && lq >= 2;
+        const uint32_t sse = dead ? 0u : ss;                    // any valid address; the values are dropped
 #pragma unroll
-        for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(xd + j * 8) = g.x[j];
-        uint16_t* wd = ws + (buf * GEMM_BM + srow) * GEMM_LDK + shalf * 32;
-        const float s = bf16_to_f32(g.s), b = bf16_to_f32(g.b);
-        if (BITS == 4) {
-            const uint32_t words[4] = {g.w[0].x, g.w[0].y, g.w[0].z, g.w[0].w};
+        for (int t = 0; t < NT; ++t) {
+            const uint8_t* wp = wrow[t] + (size_t)sse * (GEMM_SK * BITS / 8);
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                float q[8];
-                unpack4(words[d], q);
-                uint4 o;
-                o.x = pack_act2<ACT>(fmaf(q[0], s, b), fmaf(q[1], s, b));
-                o.y = pack_act2<ACT>(fmaf(q[2], s, b), fmaf(q[3], s, b));
-                o.z = pack_act2<ACT>(fmaf(q[4], s, b), fmaf(q[5], s, b));
-                o.w = pack_act2<ACT>(fmaf(q[6], s, b), fmaf(q[7], s, b));
-                *reinterpret_cast<uint4*>(wd + d * 8) = o;
-            }
-        } else {
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const uint4 wq = g.w[BITS == 8 ? h : 0];
-                const uint32_t words[4] = {wq.x, wq.y, wq.z, wq.w};
-#pragma unroll
-                for (int d = 0; d < 2; ++d) {
-                    float q[8];
-                    unpack8(words[2 * d], q);
-                    unpack8(words[2 * d + 1], q + 4);
-                    uint4 o;
-                    o.x = pack_act2<ACT>(fmaf(q[0], s, b), fmaf(q[1], s, b));
-                    o.y = pack_act2<ACT>(fmaf(q[2], s, b), fmaf(q[3], s, b));
-                    o.z = pack_act2<ACT>(fmaf(q[4], s, b), fmaf(q[5], s, b));
-                    o.w = pack_act2<ACT>(fmaf(q[6], s, b), fmaf(q[7], s, b));
-                    *reinterpret_cast<uint4*>(wd + h * 16 + d * 8) = o;
-                }
-            }
+            for (int h = 0; h < WQ; ++h) g.w[t][h] = *reinterpret_cast<const uint4*>(wp + 16 * h);
+            g.s[t] = dead ? (uint16_t)0 : srow_p[t][2 * sse];
+            g.b[t] = dead ? (uint16_t)0 : brow_p[t][2 * sse];
         }
     };
+    auto store_x = [&](const XStage& g, int buf) {
+        if (!x_live) return;
+        uint16_t* xd = xs + (buf * GEMM_BM + srow) * GEMM_LDK + shalf * 64;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) *reinterpret_cast<uint4*>(xd + j * 8) = g.v[j];
+    };
 
-    fl4_t acc[4][4];
+    fl4_t acc[8][NT];
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < 8; ++a)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[a][j] = fl4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int t = 0; t < NT; ++t) acc[a][t] = fl4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-    const uint32_t nk = p.K / GEMM_BK;
 #pragma unroll
-    for (int j = 0; j < GEMM_STAGES; ++j)
-        if ((uint32_t)j < nk) load_regs(st[j], j);
-    store_regs(st[0], 0);
+    for (int j = 0; j < GEMM_WST - 1; ++j)
+        if ((uint32_t)j < nss) load_w(wst[j], j);
+    load_x(xst[0], 0);
+    if (nss > 1) load_x(xst[1], 1);
+    store_x(xst[0], 0);
     __syncthreads();
-    for (uint32_t ks0 = 0; ks0 < nk; ks0 += GEMM_STAGES) {
+    for (uint32_t ss0 = 0; ss0 < nss; ss0 += GEMM_WST) {
 #pragma unroll
-        for (int j = 0; j < GEMM_STAGES; ++j) {
-            const uint32_t ks = ks0 + j;
-            if (ks >= nk) break;
-            const int buf = ks & 1;
-            // step ks went from st[j] to LDS one iteration ago: st[j] is free again
-            if (ks + GEMM_STAGES < nk) load_regs(st[j], ks + GEMM_STAGES);
+        for (int u = 0; u < GEMM_WST; ++u) {
+            const uint32_t ss = ss0 + u;
+            if (ss >= nss) break;
+            const int buf = ss & 1;
+            // xst[u % 2] held super-step ss, which reached LDS one iteration ago
+            if (ss + 2 < nss) load_x(xst[u % GEMM_XST], ss + 2);
+            if (ss + GEMM_WST - 1 < nss) load_w(wst[(u + GEMM_WST - 1) % GEMM_WST], ss + GEMM_WST - 1);
+            const WStage& g = wst[u];
+            float sc[NT], bi[NT];
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) {
-                uint4 afrag[4], bfrag[4];
+            for (int t = 0; t < NT; ++t) { sc[t] = bf16_to_f32(g.s[t]); bi[t] = bf16_to_f32(g.b[t]); }
+            const uint16_t* xa = xs + (buf * GEMM_BM + li) * GEMM_LDK + lq * 32;
 #pragma unroll
-                for (int a = 0; a < 4; ++a)
-                    afrag[a] = *reinterpret_cast<const uint4*>(xs + (buf * GEMM_BM + wm * 64 + a * 16 + li) * GEMM_LDK + kk * 32 + lq * 8);
+            for (int j = 0; j < 4; ++j) {
+                uint4 bfrag[NT];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const int brow = DUAL ? (t >> 1) * 64 + wn * 32 + (t & 1) * 16 + li : wn * 64 + t * 16 + li;
-                    bfrag[t] = *reinterpret_cast<const uint4*>(ws + (buf * GEMM_BM + brow) * GEMM_LDK + kk * 32 + lq * 8);
+                for (int t = 0; t < NT; ++t) {
+                    float q[8];
+                    if (BITS == 4) {
+                        const uint4 w = g.w[t][0];
+                        unpack4(j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w, q);
+                    } else {
+                        const uint4 w = g.w[t][BITS == 8 ? j >> 1 : 0];
+                        unpack8((j & 1) ? w.z : w.x, q);
+                        unpack8((j & 1) ? w.w : w.y, q + 4);
+                    }
+                    bfrag[t] = dequant8<ACT>(q, sc[t], bi[t]);
                 }
 #pragma unroll
-                for (int a = 0; a < 4; ++a)
+                for (int a = 0; a < 8; ++a) {
+                    if (a >= live_mt) break;
+                    const uint4 afrag = *reinterpret_cast<const uint4*>(xa + a * 16 * GEMM_LDK + j * 8);
 #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        acc[a][t] = mfma_16x16x32<ACT>(afrag[a], bfrag[t], acc[a][t]);
+                    for (int t = 0; t < NT; ++t) acc[a][t] = mfma_16x16x32<ACT>(afrag, bfrag[t], acc[a][t]);
+                }
             }
-            if (ks + 1 < nk) store_regs(st[(j + 1) % GEMM_STAGES], buf ^ 1);
+            if (ss + 1 < nss) store_x(xst[(u + 1) % GEMM_XST], buf ^ 1);
             __syncthreads();
         }
     }
 
-    // ---- epilogue: lane holds column li of each tile, rows 4*lq .. 4*lq+3
-    uint16_t* out = (uint16_t*)p.out;
+    // ---- epilogue: lane holds column i of each tile, rows 16 a + 4 q .. +4.  The block's output
+    // tile is rounded to 16 bits into LDS (the activation buffers are free after the last
+    // barrier) and leaves in 16-byte pieces, whole rows of the tile at a time.
+    constexpr int OC = DUAL ? 64 : 128;                 // columns of the block's tile
+    constexpr int LDO = OC + 8;
+    uint16_t* os = xs;
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < 8; ++a) {
+        if (a >= live_mt) break;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const uint32_t m = wm * 64 + a * 16 + lq * 4 + t;
-            if (m >= mt.rows) continue;
+        for (int r = 0; r < 4; ++r) {
+            const int m = a * 16 + lq * 4 + r;
             if (DUAL) {
-                const size_t orow = (size_t)(mt.row_start + m) * p.out_stride;
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const uint32_t n = n0 + wn * 32 + j * 16 + li;
-                    if (n < p.N) out[orow + n] = f32_to_act<ACT>(silu_fast(acc[a][j][t]) * acc[a][j + 2][t]);
-                }
+                os[m * LDO + wave * 16 + li] = f32_to_act<ACT>(silu_fast(acc[a][0][r]) * acc[a][1][r]);
             } else {
-                const PrefillPair pr = p.pairs[mt.row_start + m];
-                const size_t orow = ((size_t)pr.token * p.top_k + pr.rank) * p.out_stride;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t n = n0 + wn * 64 + j * 16 + li;
-                    if (n < p.N) out[orow + n] = f32_to_act<ACT>(acc[a][j][t]);
-                }
+                for (int t = 0; t < NT; ++t) os[m * LDO + wave * 32 + t * 16 + li] = f32_to_act<ACT>(acc[a][t][r]);
             }
         }
+    }
+    __syncthreads();
+    constexpr int PIECES = OC / 8;                      // 16-byte pieces per row
+    constexpr int ROWS_PER_PASS = 256 / PIECES;
+    const int piece = tid % PIECES, prow = tid / PIECES;
+    uint16_t* out = (uint16_t*)p.out;
+    const bool vec_ok = (p.out_stride % 8 == 0) && n0 + OC <= p.N;
+    for (uint32_t m = prow; m < mt.rows; m += ROWS_PER_PASS) {
+        size_t orow;
+        if (DUAL) orow = (size_t)(mt.row_start + m) * p.out_stride;
+        else {
+            const PrefillPair pr = p.pairs[mt.row_start + m];
+            orow = ((size_t)pr.token * p.top_k + pr.rank) * p.out_stride;
+        }
+        const uint4 v = *reinterpret_cast<const uint4*>(os + m * LDO + piece * 8);
+        const uint32_t c0 = n0 + piece * 8;
+        if (vec_ok) *reinterpret_cast<uint4*>(out + orow + c0) = v;
+        else {
+            const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                if (c0 + j < p.N) out[orow + c0 + j] = e[j];
+        }
+    }
 }
 
 // ---- combine (prefill.metal:437-458) -------------------------------------------------------
