@@ -34,9 +34,10 @@ def parse():
     ap.add_argument("--layers", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--sweep", action="store_true", help="also print batch/bits sweep lines to stderr")
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "copy"],
                     help="decode = configs[1] (the headline line); prefill = configs[2] grouped GEMM; "
-                         "attention = configs[3] quantized-KV decode attention")
+                         "attention = configs[3] quantized-KV decode attention; copy = a plain 1 GiB device copy, "
+                         "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated on")
     ap.add_argument("--context", type=int, default=32768, help="attention: tokens in the KV cache")
     ap.add_argument("--tokens", type=int, default=4096, help="prefill: tokens per step")
     a = ap.parse_args()
@@ -150,6 +151,15 @@ def cpu_baseline(layers, stride, bits, batch, torch):
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
+# HBM bytes per launch of the roofline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this file (KiB per dispatch, FETCH_SIZE scaled x2.00 and WRITE_SIZE x1.00 after calibration on
+# `--workload copy`); the summaries live under profiles/.  Keyed by (workload, bits, batch or
+# tokens); other configurations report null.
+MEASURED_TRAFFIC_BYTES = {
+    ("decode", 8, 32): (180700 * 2.00 + 1336 * 1.00) * 1024,
+    ("prefill", 4, 4096): (283800 * 2.00 + 32770 * 1.00) * 1024,
+}
+
 
 def run_prefill(nv, ctx, torch, a):
     """configs[2]: 4096 tokens, top-8 of 256 experts with Zipf(1.1) popularity, 4-bit experts.
@@ -214,7 +224,8 @@ def run_prefill(nv, ctx, torch, a):
                    "kernel_us": {k: round(v, 2) for k, v in kern.items()}},
         "roofline": {"kernel": "prefill_gemm_kernel<DUAL> (gate/up + SwiGLU)", "bound": "mfma",
                      "achieved": round(g1, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(g1 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(g1 / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(("prefill", bits, T)),
                      "flops_per_launch": T * K * 4.0 * D * F, "avg_launch_us": round(kern["gemm_gate_up"], 2)},
         "cpu_baseline": None,
     }
@@ -276,6 +287,25 @@ def run_attention(nv, ctx, torch, a):
     }
 
 
+def run_copy(torch, a):
+    """A plain copy kernel of known size: 1 GiB read + 1 GiB written per launch."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 256)
+    dst = torch.empty_like(src)
+    for _ in range(a.warmup):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    return {"metric": "plain device copy", "value": round(2 * n / dt / 1e9, 2), "unit": "GB/s", "n_gpus": 1,
+            "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "copy: 1 GiB read + 1 GiB written per launch", "bytes_read": n, "bytes_written": n}}
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -289,7 +319,8 @@ def main():
         sys.exit(2)
     ctx = nv.Context(0, nv.ACT_BF16)
     if a.workload != "decode":
-        line = run_prefill(nv, ctx, torch, a) if a.workload == "prefill" else run_attention(nv, ctx, torch, a)
+        line = (run_prefill(nv, ctx, torch, a) if a.workload == "prefill" else
+                run_attention(nv, ctx, torch, a) if a.workload == "attention" else run_copy(torch, a))
         print(json.dumps(line), flush=True)
         return
     layers, stride = build_layers(nv, ctx, torch, a.bits, a.layers)
@@ -309,7 +340,8 @@ def main():
                    "kernel_us": {k: round(v, 2) for k, v in r["kernel_us"].items()}},
         "roofline": {"kernel": "expert_rows_fast (routed + shared gate/up SwiGLU, phase 1)", "bound": "hbm",
                      "achieved": round(r["phase1_gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(r["phase1_gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(r["phase1_gbps"] / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(("decode", a.bits, a.batch)),
                      "bytes_per_launch": round(r["phase1_bytes"]),
                      "avg_launch_us": round(r["kernel_us"]["phase1"], 2)},
     }

@@ -211,10 +211,13 @@ extern "C" int nvmai_hip_prefill_moe_reduce_token_major(nvmai_hip_ctx* ctx, nvma
     if (query_count == 0 || top_k == 0 || d == 0 || d % 2 || h2_stride < d || h2_stride % 2) return NVMAI_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
     ProfScope prof(ctx, NVMAI_PROF_PREFILL_COMBINE, s);
-    dim3 grid((d / 2 + 255) / 256, query_count);
-    if (ctx->act == ACT_BF16)
-        prefill_reduce_kernel<ACT_BF16><<<grid, 256, 0, s>>>(route_partials, route_weights, h2, query_count, top_k, d, h2_stride);
-    else
-        prefill_reduce_kernel<ACT_FP16><<<grid, 256, 0, s>>>(route_partials, route_weights, h2, query_count, top_k, d, h2_stride);
+    const bool vec = d % 8 == 0 && h2_stride % 8 == 0 && aligned16(route_partials) && aligned16(h2);
+    const uint32_t per = vec ? 8 : 2;
+    dim3 grid((d / per + 255) / 256, query_count);
+#define NVMAI_REDUCE(ACT, VEC) \
+    prefill_reduce_kernel<ACT, VEC><<<grid, 256, 0, s>>>(route_partials, route_weights, h2, query_count, top_k, d, h2_stride)
+    if (ctx->act == ACT_BF16) { if (vec) NVMAI_REDUCE(ACT_BF16, 8); else NVMAI_REDUCE(ACT_BF16, 2); }
+    else { if (vec) NVMAI_REDUCE(ACT_FP16, 8); else NVMAI_REDUCE(ACT_FP16, 2); }
+#undef NVMAI_REDUCE
     return launch_status();
 }
