@@ -124,24 +124,24 @@ extern "C" int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream s
 
 namespace {
 
-template <int ACT, int BITS>
+template <int ACT, int BITS, int NT>
 void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t mtiles8, nvmai_hip_ctx* ctx, hipStream_t s) {
     const size_t lds = (size_t)2 * GEMM_BM * GEMM_LDK * 2;     // 68 KB: above the 64 KB a launch gets unasked
     static bool raised = false;
     if (!raised) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, true>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, true, NT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, false>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, false, NT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         raised = true;
     }
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM1, s);
-        prefill_gemm_kernel<ACT, BITS, true><<<mtiles8 * g1.n_tiles_n, 256, lds, s>>>(g1);
+        prefill_gemm_kernel<ACT, BITS, true, NT><<<mtiles8 * g1.n_tiles_n, 256, lds, s>>>(g1);
     }
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM2, s);
-        prefill_gemm_kernel<ACT, BITS, false><<<mtiles8 * g2.n_tiles_n, 256, lds, s>>>(g2);
+        prefill_gemm_kernel<ACT, BITS, false, NT><<<mtiles8 * g2.n_tiles_n, 256, lds, s>>>(g2);
     }
 }
 
@@ -178,6 +178,7 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
     hipStream_t s = (hipStream_t)stream;
     prefill_mtiles_kernel<<<1, 256, 0, s>>>(reinterpret_cast<const PrefillGroup*>(grouping->groups), grouping->info,
                                             mtiles, n_mtiles);
+    const uint32_t nt = bits == 4 ? 4 : 2;        // 16-column tiles per wave: what the register file allows
     GemmParams g1{};
     g1.pool = (const uint8_t*)experts_base; g1.pool_stride = expert_stride;
     g1.wA = off->gate_w; g1.sA = off->gate_s; g1.bA = off->gate_b;
@@ -186,19 +187,20 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
     g1.pairs = reinterpret_cast<const PrefillPair*>(grouping->sorted_pairs);
     g1.x = hidden; g1.x_stride = hidden_stride;
     g1.out = act_scratch; g1.out_stride = f;
-    g1.K = d; g1.N = f; g1.top_k = top_k; g1.n_tiles_n = (f + 63) / 64;
+    g1.K = d; g1.N = f; g1.top_k = top_k; g1.n_tiles_n = (f + 32 * nt - 1) / (32 * nt);
     GemmParams g2 = g1;
     g2.wA = off->down_w; g2.sA = off->down_s; g2.bA = off->down_b;
     g2.wB = g2.sB = g2.bB = 0;
     g2.x = act_scratch; g2.x_stride = f;
     g2.out = route_partials; g2.out_stride = d;
-    g2.K = f; g2.N = d; g2.n_tiles_n = (d + 127) / 128;
+    g2.K = f; g2.N = d; g2.n_tiles_n = (d + 64 * nt - 1) / (64 * nt);
+    const uint32_t mtiles8 = (max_mtiles + 7) / 8 * 8;
     if (ctx->act == ACT_BF16) {
-        if (bits == 4) launch_gemms<ACT_BF16, 4>(g1, g2, (max_mtiles + 7) / 8 * 8, ctx, s);
-        else launch_gemms<ACT_BF16, 8>(g1, g2, (max_mtiles + 7) / 8 * 8, ctx, s);
+        if (bits == 4) launch_gemms<ACT_BF16, 4, 4>(g1, g2, mtiles8, ctx, s);
+        else launch_gemms<ACT_BF16, 8, 2>(g1, g2, mtiles8, ctx, s);
     } else {
-        if (bits == 4) launch_gemms<ACT_FP16, 4>(g1, g2, (max_mtiles + 7) / 8 * 8, ctx, s);
-        else launch_gemms<ACT_FP16, 8>(g1, g2, (max_mtiles + 7) / 8 * 8, ctx, s);
+        if (bits == 4) launch_gemms<ACT_FP16, 4, 4>(g1, g2, mtiles8, ctx, s);
+        else launch_gemms<ACT_FP16, 8, 2>(g1, g2, mtiles8, ctx, s);
     }
     return launch_status();
 }

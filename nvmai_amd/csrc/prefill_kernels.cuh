@@ -273,7 +273,7 @@ __global__ __launch_bounds__(256) void prefill_mtiles_kernel(const PrefillGroup*
 //
 // k runs in super-steps of 128 (two quantization groups).  The activations of a super-step go
 // through a double-buffered LDS tile shared by the four waves.  The weights never touch LDS:
-// wave w owns 16 * GEMM_NT columns of all 128 rows, and lane (i = lane % 16, q = lane / 16)
+// wave w owns 16 * NT columns of all 128 rows, and lane (i = lane % 16, q = lane / 16)
 // loads the 32 codes W[n_i, k0 + 32q .. +32) of each of its columns in one 16-byte (4 bit) or
 // two (8 bit) loads, so four neighbouring lanes cover 64 or 128 contiguous bytes of a row.
 // It dequantizes them in registers, w = q * scale + bias in fp32 rounded once to the activation
@@ -304,7 +304,6 @@ struct GemmParams {
 
 constexpr int GEMM_SK = 128;            // k per super-step
 constexpr int GEMM_LDK = GEMM_SK + 8;   // padded LDS row: conflict-free 16-byte reads and writes
-constexpr int GEMM_XST = 2;             // activation register stages in flight
 
 // Two floats -> two 16-bit activations in one dword, round to nearest even.
 template <int ACT>
@@ -332,11 +331,15 @@ __device__ __forceinline__ uint4 dequant8(const float* q, float s, float b) {
     return o;
 }
 
-template <int ACT, int BITS, bool DUAL>
+// NT = 16-column tiles per wave (2 or 4): the block covers 32 NT gate/up columns (DUAL) or
+// 64 NT down columns.  NT = 4 reads each activation fragment from LDS once for four MFMAs and
+// halves the number of blocks that re-read an M tile's activations.
+template <int ACT, int BITS, bool DUAL, int NT>
 __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
-    constexpr int NT = 2;                               // 16-column tiles per wave
     constexpr int WQ = BITS == 8 ? 2 : 1;               // 16-byte loads per (column, super-step)
-    constexpr int GEMM_WST = BITS == 8 ? 2 : 4;         // weight register stages in flight (register budget)
+    // register stages in flight (register budget: 128 accumulators at NT = 4)
+    constexpr int GEMM_XST = NT == 4 ? 1 : 2;
+    constexpr int GEMM_WST = (NT == 4 || BITS == 8) ? 2 : 4;
     extern __shared__ uint4 gemm_lds[];
     uint16_t* xs = reinterpret_cast<uint16_t*>(gemm_lds);      // [2][128][LDK]
     // Blocks are dealt to the eight XCDs round-robin.  The column tiles of one M tile go to one
@@ -350,7 +353,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 15, lq = lane >> 4;
     const uint32_t groups = p.K / NVMAI_GROUP;
-    const uint32_t n_cols = DUAL ? 64 : 128;            // output columns per block
+    constexpr uint32_t n_cols = DUAL ? 32 * NT : 64 * NT;   // output columns per block
     const uint32_t n0 = nt * n_cols;
 
     // ---- activation staging: thread (row, half) moves 64 elements of a row per super-step
@@ -365,17 +368,17 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
         xrow = (const uint16_t*)p.x + (size_t)src * p.x_stride + shalf * 64;
     }
-    // ---- weight columns of this lane: tile t -> DUAL {gate, up} of column n0 + 16 wave + i,
-    //      else column n0 + 32 wave + 16 t + i
+    // ---- weight columns of this lane: tile t -> DUAL {gate, up}[t & 1] of column
+    //      n0 + 8 NT wave + 16 (t / 2) + i, else column n0 + 16 NT wave + 16 t + i
     const uint8_t* wrow[NT];
     const uint16_t* srow_p[NT];
     const uint16_t* brow_p[NT];
     uint32_t col[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        col[t] = DUAL ? n0 + wave * 16 + li : n0 + wave * 32 + t * 16 + li;
+        col[t] = DUAL ? n0 + wave * (8 * NT) + (t >> 1) * 16 + li : n0 + wave * (16 * NT) + t * 16 + li;
         const uint32_t r = col[t] < p.N ? col[t] : p.N - 1;
-        const bool second = DUAL && t == 1;
+        const bool second = DUAL && (t & 1);
         wrow[t] = blob + (second ? p.wB : p.wA) + (size_t)r * (p.K * BITS / 8) + lq * (32 * BITS / 8);
         srow_p[t] = reinterpret_cast<const uint16_t*>(blob + (second ? p.sB : p.sA)) + (size_t)r * groups + (lq >> 1);
         brow_p[t] = reinterpret_cast<const uint16_t*>(blob + (second ? p.bB : p.bA)) + (size_t)r * groups + (lq >> 1);
@@ -386,15 +389,20 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     // range lies beyond K contribute zeros (zero activations, zero weights).
     const bool odd_tail = (p.K % GEMM_SK) != 0;
 
-    struct XStage { uint4 v[8]; };
+    // NT = 4 has no registers to spare: the activations of the next super-step then travel in
+    // two halves of four 16-byte pieces through one half-sized stage.
+    constexpr bool XSPLIT = NT == 4;
+    constexpr int XP = XSPLIT ? 4 : 8;                  // 16-byte pieces per stage
+    struct XStage { uint4 v[XP]; };
     struct WStage { uint4 w[NT][WQ]; uint16_t s[NT], b[NT]; };
     XStage xst[GEMM_XST];
     WStage wst[GEMM_WST];
-    auto load_x = [&](XStage& g, uint32_t ss) {
+    auto load_x = [&](XStage& g, uint32_t ss, int part) {
         const bool dead = !x_live || (odd_tail && ss == nss - 1 && shalf == 1);
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            g.v[j] = dead ? uint4{0, 0, 0, 0} : *reinterpret_cast<const uint4*>(xrow + ss * GEMM_SK + j * 8);
+        for (int j = 0; j < XP; ++j)
+            g.v[j] = dead ? uint4{0, 0, 0, 0}
+                          : *reinterpret_cast<const uint4*>(xrow + ss * GEMM_SK + (part * XP + j) * 8);
     };
     auto load_w = [&](WStage& g, uint32_t ss) {
         const bool dead = odd_tail && ss == nss - 1 && lq >= 2;
@@ -408,11 +416,11 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
             g.b[t] = dead ? (uint16_t)0 : brow_p[t][2 * sse];
         }
     };
-    auto store_x = [&](const XStage& g, int buf) {
+    auto store_x = [&](const XStage& g, int buf, int part) {
         if (!x_live) return;
-        uint16_t* xd = xs + (buf * GEMM_BM + srow) * GEMM_LDK + shalf * 64;
+        uint16_t* xd = xs + (buf * GEMM_BM + srow) * GEMM_LDK + shalf * 64 + part * XP * 8;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) *reinterpret_cast<uint4*>(xd + j * 8) = g.v[j];
+        for (int j = 0; j < XP; ++j) *reinterpret_cast<uint4*>(xd + j * 8) = g.v[j];
     };
 
     fl4_t acc[8][NT];
@@ -424,9 +432,17 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
 #pragma unroll
     for (int j = 0; j < GEMM_WST - 1; ++j)
         if ((uint32_t)j < nss) load_w(wst[j], j);
-    load_x(xst[0], 0);
-    if (nss > 1) load_x(xst[1], 1);
-    store_x(xst[0], 0);
+    if (XSPLIT) {
+        load_x(xst[0], 0, 0);
+        store_x(xst[0], 0, 0);
+        load_x(xst[0], 0, 1);
+        store_x(xst[0], 0, 1);
+    } else {
+#pragma unroll
+        for (int j = 0; j < GEMM_XST; ++j)
+            if ((uint32_t)j < nss) load_x(xst[j], j, 0);
+        store_x(xst[0], 0, 0);
+    }
     __syncthreads();
     for (uint32_t ss0 = 0; ss0 < nss; ss0 += GEMM_WST) {
 #pragma unroll
@@ -434,8 +450,8 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
             const uint32_t ss = ss0 + u;
             if (ss >= nss) break;
             const int buf = ss & 1;
-            // xst[u % 2] held super-step ss, which reached LDS one iteration ago
-            if (ss + 2 < nss) load_x(xst[u % GEMM_XST], ss + 2);
+            // xst[u % XST] held super-step ss, which reached LDS one iteration ago
+            if (ss + GEMM_XST < nss) load_x(xst[u % GEMM_XST], ss + GEMM_XST, 0);
             if (ss + GEMM_WST - 1 < nss) load_w(wst[(u + GEMM_WST - 1) % GEMM_WST], ss + GEMM_WST - 1);
             const WStage& g = wst[u];
             float sc[NT], bi[NT];
@@ -465,8 +481,12 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
 #pragma unroll
                     for (int t = 0; t < NT; ++t) acc[a][t] = mfma_16x16x32<ACT>(afrag, bfrag[t], acc[a][t]);
                 }
+                if (XSPLIT && j == 1 && ss + 1 < nss) {         // first half lands, second half leaves
+                    store_x(xst[0], buf ^ 1, 0);
+                    load_x(xst[0], ss + 1, 1);
+                }
             }
-            if (ss + 1 < nss) store_x(xst[(u + 1) % GEMM_XST], buf ^ 1);
+            if (ss + 1 < nss) store_x(xst[(u + 1) % GEMM_XST], buf ^ 1, XSPLIT ? 1 : 0);
             __syncthreads();
         }
     }
@@ -474,7 +494,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     // ---- epilogue: lane holds column i of each tile, rows 16 a + 4 q .. +4.  The block's output
     // tile is rounded to 16 bits into LDS (the activation buffers are free after the last
     // barrier) and leaves in 16-byte pieces, whole rows of the tile at a time.
-    constexpr int OC = DUAL ? 64 : 128;                 // columns of the block's tile
+    constexpr int OC = n_cols;                          // columns of the block's tile
     constexpr int LDO = OC + 8;
     uint16_t* os = xs;
 #pragma unroll
@@ -484,10 +504,13 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         for (int r = 0; r < 4; ++r) {
             const int m = a * 16 + lq * 4 + r;
             if (DUAL) {
-                os[m * LDO + wave * 16 + li] = f32_to_act<ACT>(silu_fast(acc[a][0][r]) * acc[a][1][r]);
+#pragma unroll
+                for (int c = 0; c < NT / 2; ++c)
+                    os[m * LDO + wave * (8 * NT) + c * 16 + li] =
+                        f32_to_act<ACT>(silu_fast(acc[a][2 * c][r]) * acc[a][2 * c + 1][r]);
             } else {
 #pragma unroll
-                for (int t = 0; t < NT; ++t) os[m * LDO + wave * 32 + t * 16 + li] = f32_to_act<ACT>(acc[a][t][r]);
+                for (int t = 0; t < NT; ++t) os[m * LDO + wave * (16 * NT) + t * 16 + li] = f32_to_act<ACT>(acc[a][t][r]);
             }
         }
     }
