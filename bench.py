@@ -157,7 +157,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # tokens); other configurations report null.
 MEASURED_TRAFFIC_BYTES = {
     ("decode", 8, 32): (180700 * 2.00 + 1336 * 1.00) * 1024,
-    ("prefill", 4, 4096): (283800 * 2.00 + 32770 * 1.00) * 1024,
+    ("prefill", 4, 4096): (512200 * 2.00 + 32770 * 1.00) * 1024,
+    ("attention", 8, 8, 131072): (596100 * 2.00 + 4385 * 1.00) * 1024,
 }
 
 
@@ -281,7 +282,8 @@ def run_attention(nv, ctx, torch, a):
                    "frac_of_hbm_peak": round(step_b / dt / 1e9 / HBM_PEAK_GBPS, 4), "cache_sets_rotated": n_sets,
                    "kernel_us": {k: round(v, 2) for k, v in kern.items()}},
         "roofline": {"kernel": "attn_partial_mfma_kernel", "bound": "hbm", "achieved": round(part, 2),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(part / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(part / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(("attention", bits, B, ctx_len)),
                      "bytes_per_launch": kv_bytes, "avg_launch_us": round(kern["partial"], 2)},
         "cpu_baseline": None,
     }
