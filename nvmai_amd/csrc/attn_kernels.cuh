@@ -312,17 +312,13 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
     float m_run = -INFINITY, d_run = 0.0f;                          // head i; d over this lane's tokens only
     float corr[4] = {0.0f, 0.0f, 0.0f, 0.0f};                       // head i, this lane's tokens only
 
-    for (uint32_t s0 = p0 + wave * ATTN_STEP; s0 < p1; s0 += 4 * ATTN_STEP) {
-        // ---- loads: K codes (token i of each tile), metadata and V codes of this lane's 8 tokens
-        uint32_t kraw[2][4][4];                                     // [tile][group][dwords]; 4-bit uses 2 dwords
-        uint32_t tok[8];                                            // clamped token positions of the P/V slots
-        bool tok_ok[8];
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const uint32_t pos = s0 + (t >> 2) * 16 + 4 * r + (t & 3);
-            tok_ok[t] = pos < p1;
-            tok[t] = tok_ok[t] ? pos : p1 - 1;
-        }
+    // K side of a step (codes of token i of both tiles, fp16 scale/bias of this lane's 8 token
+    // slots).  It is dead once the scores are out, so the next step's K side is requested right
+    // there and arrives behind the softmax and the P.V products of the current step.
+    uint32_t kraw[2][4][4];                                         // [tile][group][dwords]; 4-bit uses 2 dwords
+    uint2 ksc[8], kbi[8];                                           // 4 fp16 each
+    auto slot_pos = [&](uint32_t s0, int t) { return s0 + (t >> 2) * 16 + 4 * r + (t & 3); };
+    auto load_k = [&](uint32_t s0) {
 #pragma unroll
         for (int tile = 0; tile < 2; ++tile) {
             const uint32_t pos = min(s0 + tile * 16 + i, p1 - 1);
@@ -338,14 +334,31 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
                 }
             }
         }
-        uint2 ksc[8], kbi[8], vsc[8], vbi[8];                        // 4 fp16 each
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const uint8_t* krow = kbase + (size_t)min(slot_pos(s0, t), p1 - 1) * p.f.stride;
+            ksc[t] = *reinterpret_cast<const uint2*>(krow + meta_sc);
+            kbi[t] = *reinterpret_cast<const uint2*>(krow + meta_bi);
+        }
+    };
+    const uint32_t s_first = p0 + wave * ATTN_STEP;
+    if (s_first < p1) load_k(s_first);
+
+    for (uint32_t s0 = s_first; s0 < p1; s0 += 4 * ATTN_STEP) {
+        // ---- loads: V metadata and codes of this lane's 8 tokens
+        uint32_t tok[8];                                            // clamped token positions of the P/V slots
+        bool tok_ok[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const uint32_t pos = slot_pos(s0, t);
+            tok_ok[t] = pos < p1;
+            tok[t] = tok_ok[t] ? pos : p1 - 1;
+        }
+        uint2 vsc[8], vbi[8];                                       // 4 fp16 each
         uint32_t vraw[8][4];                                        // [token slot][group]: 4 codes (8-bit) / 4 nibbles
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            const uint8_t* krow = kbase + (size_t)tok[t] * p.f.stride;
             const uint8_t* vrow = vbase + (size_t)tok[t] * p.f.stride;
-            ksc[t] = *reinterpret_cast<const uint2*>(krow + meta_sc);
-            kbi[t] = *reinterpret_cast<const uint2*>(krow + meta_bi);
             vsc[t] = *reinterpret_cast<const uint2*>(vrow + meta_sc);
             vbi[t] = *reinterpret_cast<const uint2*>(vrow + meta_bi);
 #pragma unroll
@@ -395,6 +408,8 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
                 sv[slot] = tok_ok[slot] ? acc * q_unscale : -INFINITY;
             }
         }
+
+        if (s0 + 4 * ATTN_STEP < p1) load_k(s0 + 4 * ATTN_STEP);      // next step's K side
 
         // ---- online softmax for head i (its tokens are spread over the four lane quarters)
         float mx = sv[0];
