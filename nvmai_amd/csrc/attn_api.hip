@@ -102,7 +102,8 @@ extern "C" int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream strea
     const uint32_t qpk = num_q_heads / num_kv_heads;
     const bool fast = head_dim == ATTN_HD && (k->bits == 4 || k->bits == 8) && qpk <= 16 &&
                       aligned16(k->base) && aligned16(v->base) && (k->stride % 16 == 0) &&
-                      (kv_batch_stride % 16 == 0);
+                      (kv_batch_stride % 16 == 0) &&
+                      (uint64_t)seq_len * k->stride < (1ull << 32);        // 32-bit row offsets in the kernel
     // Chunking: enough blocks to fill the device, chunks a multiple of the 32-token step.
     const uint32_t units = fast ? batch * num_kv_heads : batch * num_q_heads;
     uint32_t nc = (512 + units - 1) / units;

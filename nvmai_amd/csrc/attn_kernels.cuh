@@ -322,7 +322,7 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
 #pragma unroll
         for (int tile = 0; tile < 2; ++tile) {
             const uint32_t pos = min(s0 + tile * 16 + i, p1 - 1);
-            const uint8_t* row = kbase + (size_t)pos * p.f.stride + code_off;
+            const uint8_t* row = kbase + (pos * p.f.stride + code_off);   // 32-bit offset from a uniform base
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 if (BITS == 8) {
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
         }
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            const uint8_t* krow = kbase + (size_t)min(slot_pos(s0, t), p1 - 1) * p.f.stride;
+            const uint8_t* krow = kbase + min(slot_pos(s0, t), p1 - 1) * p.f.stride;
             ksc[t] = *reinterpret_cast<const uint2*>(krow + meta_sc);
             kbi[t] = *reinterpret_cast<const uint2*>(krow + meta_bi);
         }
@@ -358,7 +358,7 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
         uint32_t vraw[8][4];                                        // [token slot][group]: 4 codes (8-bit) / 4 nibbles
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            const uint8_t* vrow = vbase + (size_t)tok[t] * p.f.stride;
+            const uint8_t* vrow = vbase + tok[t] * p.f.stride;
             vsc[t] = *reinterpret_cast<const uint2*>(vrow + meta_sc);
             vbi[t] = *reinterpret_cast<const uint2*>(vrow + meta_bi);
 #pragma unroll
@@ -448,33 +448,39 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
         __builtin_amdgcn_wave_barrier();
         const float4 al = *reinterpret_cast<const float4*>(bc + 4 * r);
         __builtin_amdgcn_wave_barrier();
+        if (__any(alpha != 1.0f)) {                                 // a running maximum moved somewhere in the wave
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
+            for (int g = 0; g < 4; ++g)
 #pragma unroll
-            for (int n = 0; n < 4; ++n) {
-                oacc[g][n][0] *= al.x; oacc[g][n][1] *= al.y; oacc[g][n][2] *= al.z; oacc[g][n][3] *= al.w;
-            }
+                for (int n = 0; n < 4; ++n) {
+                    oacc[g][n][0] *= al.x; oacc[g][n][1] *= al.y; oacc[g][n][2] *= al.z; oacc[g][n][3] *= al.w;
+                }
+        }
 
         // ---- O += P'_g . V   (B operand: dim 64g + 4i + n, this lane's 8 tokens)
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
+        for (int g = 0; g < 4; ++g) {
+            uint32_t pair4[4];                                      // 4-bit: nibbles of two tokens side by side
+            if (BITS == 4) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) pair4[w] = vraw[2 * w][g] | (vraw[2 * w + 1][g] << 16);
+            }
 #pragma unroll
             for (int n = 0; n < 4; ++n) {
                 H8 bop;
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    const uint32_t a = vraw[2 * w][g], c2 = vraw[2 * w + 1][g];
                     if (BITS == 8) {
-                        // byte n of two token dwords -> [a.n, 0x64, c2.n, 0x64]
-                        const uint32_t lo = (a >> (8 * n)) & 0xFFu, hi = (c2 >> (8 * n)) & 0xFFu;
-                        bop.u[w] = lo | (hi << 16) | 0x64006400u;
+                        // byte n of two token dwords -> [a.n, 0, c2.n, 0], then the 0x64 exponent bytes
+                        const uint32_t sel = 0x0C000C00u | (uint32_t)n | ((uint32_t)(4 + n) << 16);
+                        bop.u[w] = __builtin_amdgcn_perm(vraw[2 * w + 1][g], vraw[2 * w][g], sel) | 0x64006400u;
                     } else {
-                        const uint32_t lo = (a >> (4 * n)) & 0xFu, hi = (c2 >> (4 * n)) & 0xFu;
-                        bop.u[w] = lo | (hi << 16) | 0x64006400u;
+                        bop.u[w] = ((pair4[w] >> (4 * n)) & 0x000F000Fu) | 0x64006400u;
                     }
                 }
                 oacc[g][n] = mfma16(pop[g], bop, oacc[g][n]);
             }
+        }
     }
 
     // ---- finish this wave: d and corr over the four quarters, corr folded into O
