@@ -133,6 +133,15 @@ void launch_rows_t(RowsParams& p, int maxtok, uint32_t max_entries, hipStream_t 
         return;                                                                                 \
     } while (0)
     static const int variant = getenv("NVMAI_ROWS_VARIANT") ? atoi(getenv("NVMAI_ROWS_VARIANT")) : 0;
+    // Few entries (a small decode batch): short blocks, so that the launch still covers the device.
+    const bool few = max_entries <= 40;
+    if constexpr (DUAL) {
+        if (few && chunks == 64) NVMAI_FAST(64, 1, 1, 2);
+        if (few && chunks == 128) NVMAI_FAST(64, 2, 1, 2);
+    } else {
+        if (few && chunks == 16) NVMAI_FAST(16, 1, 1, 2);
+        if (few && chunks == 32) NVMAI_FAST(32, 1, 2, 2);
+    }
     if constexpr (DUAL) {
         if (chunks == 64) NVMAI_FAST(64, 1, 1, 8);
         if (chunks == 128 && variant % 10 == 1) NVMAI_FAST(32, 4, 1, 8);

@@ -216,40 +216,82 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
     load_stage(s0, 0);                            // both in flight while the inputs are staged
     load_stage(s1, 1);
 
-    // ---- pass 1: largest magnitude of every input row
-#pragma unroll 1
-    for (int t = 0; t < ntok; ++t) {
-        const size_t in_off = (size_t)p.pair_in[we.pair_start + t] * p.x_stride;
-        float m = 0.0f;
-        for (uint32_t e0 = threadIdx.x * 8; e0 < p.n; e0 += 256 * 8) {
-            float v[8];
-            load8<ACT, XF32>(p.x, in_off + e0, v);
+    if (p.n <= 256 * 8) {
+        // ---- short rows: every thread holds its eight elements of every input, so the inputs
+        // are read once, all loads in flight together, and scaled from registers
+        constexpr int MT = TOKS ? TOKS : MAX_TOK;
+        float v[MT][8], m[MT];
+        const uint32_t e0 = threadIdx.x * 8;
+        const bool live = e0 < p.n;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[j]));
+        for (int t = 0; t < MT; ++t) {
+            if (t >= ntok) break;
+            if (live) load8<ACT, XF32>(p.x, (size_t)p.pair_in[we.pair_start + t] * p.x_stride + e0, v[t]);
         }
-        m = wave_max_f32(m);
-        if (lane == 0) wmax_tab[t * 4 + wave] = m;
-    }
-    __syncthreads();
-    // ---- pass 2: scale, convert, pack
-#pragma unroll 1
-    for (int t = 0; t < ntok; ++t) {
-        const size_t in_off = (size_t)p.pair_in[we.pair_start + t] * p.x_stride;
-        const float amax = fmaxf(fmaxf(wmax_tab[t * 4], wmax_tab[t * 4 + 1]),
-                                 fmaxf(wmax_tab[t * 4 + 2], wmax_tab[t * 4 + 3]));
-        float sc, isc;
-        pow2_scale(amax, sc, isc);
-        if (threadIdx.x == 0) isc_tab[t] = isc;
-        for (uint32_t e0 = threadIdx.x * 8; e0 < p.n; e0 += 256 * 8) {
-            float v[8];
-            load8<ACT, XF32>(p.x, in_off + e0, v);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] *= sc;
-            const uint32_t chunk = e0 / EPC, piece = (e0 % EPC) / 8;
-            xw[t * WORDS_TOK + ((chunk / SEG) * H + piece) * SEG + (chunk % SEG)] = pack_inputs<BITS>(v);
+        for (int t = 0; t < MT; ++t) {
+            if (t >= ntok) break;
+            m[t] = 0.0f;
+            if (live) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) m[t] = fmaxf(m[t], fabsf(v[t][j]));
+            }
+            m[t] = wave_max_f32(m[t]);
+            if (lane == 0) wmax_tab[t * 4 + wave] = m[t];
         }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            if (t >= ntok) break;
+            const float amax = fmaxf(fmaxf(wmax_tab[t * 4], wmax_tab[t * 4 + 1]),
+                                     fmaxf(wmax_tab[t * 4 + 2], wmax_tab[t * 4 + 3]));
+            float sc, isc;
+            pow2_scale(amax, sc, isc);
+            if (threadIdx.x == 0) isc_tab[t] = isc;
+            if (live) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[t][j] *= sc;
+                const uint32_t chunk = e0 / EPC, piece = (e0 % EPC) / 8;
+                xw[t * WORDS_TOK + ((chunk / SEG) * H + piece) * SEG + (chunk % SEG)] = pack_inputs<BITS>(v[t]);
+            }
+        }
+        __syncthreads();
+    } else {
+        // ---- pass 1: largest magnitude of every input row
+    #pragma unroll 1
+        for (int t = 0; t < ntok; ++t) {
+            const size_t in_off = (size_t)p.pair_in[we.pair_start + t] * p.x_stride;
+            float m = 0.0f;
+            for (uint32_t e0 = threadIdx.x * 8; e0 < p.n; e0 += 256 * 8) {
+                float v[8];
+                load8<ACT, XF32>(p.x, in_off + e0, v);
+    #pragma unroll
+                for (int j = 0; j < 8; ++j) m = fmaxf(m, fabsf(v[j]));
+            }
+            m = wave_max_f32(m);
+            if (lane == 0) wmax_tab[t * 4 + wave] = m;
+        }
+        __syncthreads();
+        // ---- pass 2: scale, convert, pack
+    #pragma unroll 1
+        for (int t = 0; t < ntok; ++t) {
+            const size_t in_off = (size_t)p.pair_in[we.pair_start + t] * p.x_stride;
+            const float amax = fmaxf(fmaxf(wmax_tab[t * 4], wmax_tab[t * 4 + 1]),
+                                     fmaxf(wmax_tab[t * 4 + 2], wmax_tab[t * 4 + 3]));
+            float sc, isc;
+            pow2_scale(amax, sc, isc);
+            if (threadIdx.x == 0) isc_tab[t] = isc;
+            for (uint32_t e0 = threadIdx.x * 8; e0 < p.n; e0 += 256 * 8) {
+                float v[8];
+                load8<ACT, XF32>(p.x, in_off + e0, v);
+    #pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] *= sc;
+                const uint32_t chunk = e0 / EPC, piece = (e0 % EPC) / 8;
+                xw[t * WORDS_TOK + ((chunk / SEG) * H + piece) * SEG + (chunk % SEG)] = pack_inputs<BITS>(v);
+            }
+        }
+        __syncthreads();
     }
-    __syncthreads();
     // ---- chunk sums of the converted inputs, one thread per (input, chunk)
     for (int idx = threadIdx.x; idx < ntok * NCH * SEG; idx += 256) {
         const int t = idx / (NCH * SEG), cs = idx % (NCH * SEG), c = cs / SEG, l = cs % SEG;
