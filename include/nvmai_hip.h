@@ -109,6 +109,16 @@ int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t
                           const void* x, uint32_t x_stride, uint32_t n_tokens, uint32_t m,
                           uint32_t n, void* y, float* y_f32, uint32_t y_stride);
 
+/* nvmai_int4_affine_gemv (nvmai_kernels.h:22-28, int4_affine_gemv.c:28-135) with the
+ * reference's own signature: HOST pointers, 4-bit codes, BF16 scale/bias, fp32 x, out written
+ * (not accumulated), n a multiple of 64.  The operands are copied to device 0, the GEMV runs
+ * there and the call returns when `out` is complete.  It allocates and synchronises on every
+ * call: it exists so that CPUExpertFFN's call sites keep linking; the fast path is
+ * nvmai_hip_affine_gemv on resident weights.  A failure is reported on stderr and fills `out`
+ * with NaN. */
+void nvmai_int4_affine_gemv(const uint8_t* weights, const uint16_t* scales, const uint16_t* biases,
+                            const float* x, size_t rows, size_t n, float* out);
+
 /* MoE.encodeRouter (MoE.swift:151-213) and PrefillRouter.encodeBlock
  * (PrefillRouter.swift:41-95): logits for n_tokens rows of `hidden`, top-k by
  * (score desc, index asc), softmax over the selected, times per_expert_scale.

@@ -96,6 +96,7 @@ SIGNATURES = {
 _OTHER = {
     "nvmai_hip_ctx_destroy": (None, [vp]),
     "nvmai_hip_status_string": (C.c_char_p, [C.c_int]),
+    "nvmai_int4_affine_gemv": (None, [vp, vp, vp, vp, C.c_size_t, C.c_size_t, vp]),
     "nvmai_sampler_seed_for": (u64, [u64, C.c_int64]),
 }
 

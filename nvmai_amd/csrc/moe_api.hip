@@ -1,5 +1,6 @@
 // Entry points of the decode-side MoE path: context, quantizer, affine GEMV,
 // router top-k, routed phase 1 / phase 2, shared expert, fused decode layer.
+#include <cstdio>
 #include <cstdlib>
 #include <new>
 
@@ -293,11 +294,13 @@ extern "C" int nvmai_hip_dequantize_affine(nvmai_hip_ctx* ctx, nvmai_stream stre
 // ---------------------------------------------------------------------------
 // affine GEMV
 // ---------------------------------------------------------------------------
-extern "C" int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
-                                     const uint16_t* scales, const uint16_t* biases, uint32_t bits,
-                                     const void* x, uint32_t x_stride, uint32_t n_tokens,
-                                     uint32_t m, uint32_t n, void* y, float* y_f32,
-                                     uint32_t y_stride) {
+namespace {
+// x holds activations of the context's type, or fp32 when x_is_f32 (the reference's CPU kernel
+// takes fp32 inputs, nvmai_kernels.h:22-28).
+int affine_gemv_any(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
+                    const uint16_t* scales, const uint16_t* biases, uint32_t bits, const void* x,
+                    bool x_is_f32, uint32_t x_stride, uint32_t n_tokens, uint32_t m, uint32_t n, void* y,
+                    float* y_f32, uint32_t y_stride) {
     if (!ctx || !weights || !scales || !biases || !x || (!y && !y_f32)) return NVMAI_ERR_INVALID_ARG;
     if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
     if (n == 0 || n % NVMAI_GROUP || x_stride < n || y_stride < m) return NVMAI_ERR_INVALID_ARG;
@@ -325,7 +328,7 @@ extern "C" int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, co
     p.sA = reinterpret_cast<const uint8_t*>(scales) - weights;
     p.bA = reinterpret_cast<const uint8_t*>(biases) - weights;
     p.x = x; p.x_stride = x_stride; p.out = tmp; p.out_stride = m; p.rows = m; p.n = n;
-    launch_rows(ctx->act, bits, false, false, p, maxtok, ents, s);
+    launch_rows(ctx->act, bits, false, x_is_f32, p, maxtok, ents, s);
     if (need_tmp) {
         // copy out with the caller's stride (and convert when asked)
         for (uint32_t t = 0; t < n_tokens; ++t) {
@@ -340,6 +343,54 @@ extern "C" int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, co
         }
     }
     return launch_status();
+}
+}  // namespace
+
+extern "C" int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
+                                     const uint16_t* scales, const uint16_t* biases, uint32_t bits,
+                                     const void* x, uint32_t x_stride, uint32_t n_tokens,
+                                     uint32_t m, uint32_t n, void* y, float* y_f32,
+                                     uint32_t y_stride) {
+    return affine_gemv_any(ctx, stream, weights, scales, biases, bits, x, false, x_stride, n_tokens, m, n, y,
+                           y_f32, y_stride);
+}
+
+// The reference's CPU entry point with its own signature (host pointers, fp32 x, out written,
+// nothing returned): the operands travel to the device, the GEMV runs there, the result
+// travels back, and the call returns when `out` is complete.  A failure cannot be returned,
+// so it is reported on stderr and `out` is filled with NaN: never a silently wrong result.
+extern "C" void nvmai_int4_affine_gemv(const uint8_t* weights, const uint16_t* scales,
+                                       const uint16_t* biases, const float* x, size_t rows, size_t n,
+                                       float* out) {
+    if (rows == 0) return;
+    static nvmai_hip_ctx* host_ctx = nullptr;
+    int rc = NVMAI_OK;
+    if (!host_ctx) rc = nvmai_hip_ctx_create(0, NVMAI_ACT_BF16, &host_ctx);
+    const size_t wb = rows * n / 2, mb = rows * (n / NVMAI_GROUP) * 2;
+    uint8_t* dev = nullptr;
+    // one allocation: weights | scales | biases | x | out, each 256-byte aligned
+    const size_t o_s = ws_round(wb), o_b = o_s + ws_round(mb), o_x = o_b + ws_round(mb), o_y = o_x + ws_round(n * 4);
+    if (rc == NVMAI_OK && (!weights || !scales || !biases || !x || !out || n == 0 || n % NVMAI_GROUP ||
+                           rows > 0xFFFFFFFFull || n > 0xFFFFFFFFull))
+        rc = NVMAI_ERR_INVALID_ARG;
+    if (rc == NVMAI_OK && hipMalloc(reinterpret_cast<void**>(&dev), o_y + rows * 4) != hipSuccess) rc = NVMAI_ERR_HIP;
+    if (rc == NVMAI_OK &&
+        (hipMemcpy(dev, weights, wb, hipMemcpyHostToDevice) != hipSuccess ||
+         hipMemcpy(dev + o_s, scales, mb, hipMemcpyHostToDevice) != hipSuccess ||
+         hipMemcpy(dev + o_b, biases, mb, hipMemcpyHostToDevice) != hipSuccess ||
+         hipMemcpy(dev + o_x, x, n * 4, hipMemcpyHostToDevice) != hipSuccess))
+        rc = NVMAI_ERR_HIP;
+    if (rc == NVMAI_OK)
+        rc = affine_gemv_any(host_ctx, nullptr, dev, reinterpret_cast<const uint16_t*>(dev + o_s),
+                             reinterpret_cast<const uint16_t*>(dev + o_b), 4, dev + o_x, true, (uint32_t)n, 1,
+                             (uint32_t)rows, (uint32_t)n, nullptr, reinterpret_cast<float*>(dev + o_y),
+                             (uint32_t)rows);
+    if (rc == NVMAI_OK && hipMemcpy(out, dev + o_y, rows * 4, hipMemcpyDeviceToHost) != hipSuccess) rc = NVMAI_ERR_HIP;
+    if (dev) (void)hipFree(dev);
+    if (rc != NVMAI_OK) {
+        fprintf(stderr, "nvmai_int4_affine_gemv: %s\n", nvmai_hip_status_string(rc));
+        if (out) for (size_t r = 0; r < rows; ++r) out[r] = __builtin_nanf("");
+    }
 }
 
 // ---------------------------------------------------------------------------

@@ -124,6 +124,19 @@ def affine_gemv(ctx, weights, scales, biases, bits, x, m, n, out_f32=False):
     return yf if out_f32 else y
 
 
+def int4_affine_gemv(weights, scales, biases, x, rows, n):
+    """nvmai_int4_affine_gemv (nvmai_kernels.h:22-28): numpy host arrays in, fp32 numpy out."""
+    import numpy as np
+    w = np.ascontiguousarray(weights, np.uint8)
+    s = np.ascontiguousarray(scales, np.uint16)
+    b = np.ascontiguousarray(biases, np.uint16)
+    xv = np.ascontiguousarray(x, np.float32)
+    out = np.empty(rows, np.float32)
+    lib.nvmai_int4_affine_gemv(w.ctypes.data, s.ctypes.data, b.ctypes.data, xv.ctypes.data, rows, n,
+                               out.ctypes.data)
+    return out
+
+
 class MoE:
     """Mirror of the reference's `MoE` operator class (MoE.swift:31-464): router, routed
     phase 1 / phase 2 over top-k blobs, plus the resident-pool decode layer."""

@@ -102,6 +102,21 @@ def test_gemv_bitstream_known_answer(nv, ctx_bf16):
         assert np.array_equal(y.cpu().numpy()[0], values.sum(1).astype(np.float32))
 
 
+def test_reference_signature_host_gemv(nv, ctx_bf16):
+    say("nvmai_int4_affine_gemv host signature")
+    rng = np.random.default_rng(11)
+    for rows, n in [(512, 2048), (2048, 512), (5, 192)]:
+        w = gauss(rng, (rows, n), 0.02)
+        p, s, b = O.quantize_affine(w, 4)
+        x = gauss(rng, (n,))
+        got = nv.int4_affine_gemv(p, s, b, x, rows, n)
+        want = O.affine_gemv(p, s, b, x, 4)
+        assert O.rel_error(got, want) <= TOL_F32
+    # a contract violation cannot be returned: it must not look like a result
+    bad = nv.int4_affine_gemv(p, s, b, x[:100], 5, 100)
+    assert np.isnan(bad).all()
+
+
 def test_gemv_rejects_bad_arguments(nv, ctx_bf16):
     say("gemv-errors")
     w = torch.zeros(64 * 128, dtype=torch.uint8, device="cuda")
