@@ -214,6 +214,37 @@ def run_prefill(nv, ctx, torch, a):
     flops = T * K * 6.0 * D * F
     g1 = T * K * 4.0 * D * F / (kern["gemm_gate_up"] * 1e-6) / 1e12
     counts = step(0).per_expert_counts.cpu().numpy()
+    # what a plain dense bf16 GEMM of the library that ships with torch reaches on this device
+    A = torch.empty((8192, 8192), dtype=torch.bfloat16, device="cuda").normal_(0, 1, generator=gen)
+    B = torch.empty((8192, 8192), dtype=torch.bfloat16, device="cuda").normal_(0, 1, generator=gen)
+    for _ in range(3):
+        A @ B
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        A @ B
+    torch.cuda.synchronize()
+    dense = 10 * 2.0 * 8192 ** 3 / (time.perf_counter() - t0) / 1e12
+    del A, B
+    cpu = None
+    if not a.no_cpu:
+        import oracle as O
+        n = 4                                           # tokens of the same step on the CPU oracle
+        blobs = pool.cpu().numpy()
+        x0 = xs[0, :n].float().cpu().numpy()
+        i0 = idx[0, :n].cpu().numpy().astype(np.uint32)
+        w0 = w[0, :n].view(torch.int16).cpu().numpy().view(np.uint16)
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            O.prefill_moe(blobs, bits, x0, D, F, i0, w0)
+            reps += 1
+            if time.perf_counter() - t0 > 10.0 or reps >= 20:
+                break
+        dtc = (time.perf_counter() - t0) / reps
+        cpu = dict(value=n * K * 6.0 * D * F / dtc / 1e12, unit="TFLOP/s", cores=1, kind="port",
+                   sample="oracle prefill_moe, %d tokens x top-%d of the same step, %d reps, %.3f s each"
+                          % (n, K, reps, dtc))
     return {
         "metric": METRIC, "value": round(flops / dt / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
@@ -222,13 +253,14 @@ def run_prefill(nv, ctx, torch, a):
                                "(Zipf 1.1 popularity), %d-bit group-64 experts, intermediate 512" % (T, bits),
                    "tokens_per_s": round(T / dt), "largest_expert_pairs": int(counts.max()),
                    "experts_hit": int((counts > 0).sum()),
+                   "dense_bf16_gemm_8192_tflops": round(dense, 1),
                    "kernel_us": {k: round(v, 2) for k, v in kern.items()}},
         "roofline": {"kernel": "prefill_gemm_kernel<DUAL> (gate/up + SwiGLU)", "bound": "mfma",
                      "achieved": round(g1, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(g1 / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(("prefill", bits, T)),
                      "flops_per_launch": T * K * 4.0 * D * F, "avg_launch_us": round(kern["gemm_gate_up"], 2)},
-        "cpu_baseline": None,
+        "cpu_baseline": cpu,
     }
 
 
@@ -270,6 +302,24 @@ def run_attention(nv, ctx, torch, a):
         ms, n = ctx.profile_read(tag)
         kern[name] = ms / max(n, 1) * 1e3
     stride = caches[0][0].stride
+    cpu = None
+    if not a.no_cpu:
+        import oracle as O
+        n = min(ctx_len, 8192)                          # first rows of sequence 0 on the CPU oracle
+        kr = caches[0][0].rows[0, :n].cpu().numpy()
+        vr = caches[0][1].rows[0, :n].cpu().numpy()
+        q0 = q[0].float().cpu().numpy()
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            O.attention_decode(q0, kr, vr, bits, HQ, HKV, HD, n, 1.0 / 16.0)
+            reps += 1
+            if time.perf_counter() - t0 > 10.0 or reps >= 20:
+                break
+        dtc = (time.perf_counter() - t0) / reps
+        cpu = dict(value=2.0 * n * stride / dtc / 1e9, unit="GB/s", cores=1, kind="port",
+                   sample="oracle attention_decode, one sequence, %d cached tokens, %d reps, %.3f s each"
+                          % (n, reps, dtc))
     kv_bytes = 2.0 * B * ctx_len * stride
     step_b = kv_bytes + 2 * B * HQ * HD * 2
     part = kv_bytes / (kern["partial"] * 1e-6) / 1e9
@@ -285,7 +335,7 @@ def run_attention(nv, ctx, torch, a):
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(part / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(("attention", bits, B, ctx_len)),
                      "bytes_per_launch": kv_bytes, "avg_launch_us": round(kern["partial"], 2)},
-        "cpu_baseline": None,
+        "cpu_baseline": cpu,
     }
 
 
