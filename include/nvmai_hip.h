@@ -347,14 +347,17 @@ int nvmai_hip_sample_topk64(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint1
                             float top_p, const uint64_t* seeds, uint32_t top_k, uint32_t* out_token,
                             uint32_t* top64_out);
 
-/* Sample.encode (LogitOutput.swift:157-199; kernel logit.metal:315-585): temperature <= 0 is
- * greedy argmax (lowest index wins ties); otherwise top_k (0 = none, capped at 256) argmax
- * passes and the same top-p / temperature / inverse-CDF draw.  The Gumbel shortcut the
- * reference takes when neither top-k nor top-p is set is not built: that case runs the
- * truncating path with k = 256, which the reference reaches with top_k = 256. */
+/* Sample.encode (LogitOutput.swift:157-199; kernel logit.metal:315-585), the kernel's three
+ * paths: temperature <= 0 is greedy argmax (lowest index wins ties); top_k == 0 with top_p
+ * outside (0, 1) is the Gumbel-max draw argmax(log p / T + g) with g from SplitMix64 of
+ * (seed, position, index) (logit.metal:296-313, 391-429); otherwise top_k (0 = none, capped at
+ * 256) argmax passes and the top-p / temperature / inverse-CDF draw with xorshift64*.
+ * seeds: HOST array, one per row; positions: HOST array, one per row, NULL = 0 (only the
+ * Gumbel path reads it); rows <= 32. */
 int nvmai_hip_sample(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint16_t* probs,
                      uint32_t probs_stride, uint32_t rows, uint32_t v, float temperature,
-                     uint32_t top_k, float top_p, const uint64_t* seeds, uint32_t* out_token);
+                     uint32_t top_k, float top_p, const uint64_t* seeds, const uint32_t* positions,
+                     uint32_t* out_token);
 
 /* Sampler.seedFor (Sampler.swift:304-325): splitmix64(seed + position), 0 mapped away. */
 uint64_t nvmai_sampler_seed_for(uint64_t seed, int64_t position);

@@ -4,6 +4,9 @@
 
 using namespace nvmai;
 
+// first of SAMPLE_MAX_ROWS persistent zeroed words of the context used as per-row block counters
+constexpr int GUMBEL_TICKETS = 16;
+
 extern "C" uint64_t nvmai_sampler_seed_for(uint64_t seed, int64_t position) {
     uint64_t z = seed + (uint64_t)position + 0x9E3779B97F4A7C15ull;
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
@@ -63,13 +66,26 @@ extern "C" int nvmai_hip_sample_topk64(nvmai_hip_ctx* ctx, nvmai_stream stream, 
 
 extern "C" int nvmai_hip_sample(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint16_t* probs,
                                 uint32_t probs_stride, uint32_t rows, uint32_t v, float temperature,
-                                uint32_t top_k, float top_p, const uint64_t* seeds, uint32_t* out_token) {
+                                uint32_t top_k, float top_p, const uint64_t* seeds, const uint32_t* positions,
+                                uint32_t* out_token) {
     if (!ctx || !probs || !seeds || !out_token || v == 0 || probs_stride < v) return NVMAI_ERR_INVALID_ARG;
     if (rows == 0) return NVMAI_OK;
     if (rows > SAMPLE_MAX_ROWS) return NVMAI_ERR_INVALID_ARG;
     SeedArray sa{};
     for (uint32_t r = 0; r < rows; ++r) sa.s[r] = seeds[r];
-    ProfScope ps(ctx, NVMAI_PROF_SAMPLE, (hipStream_t)stream);
-    sample_generic_kernel<<<dim3(rows), 256, 0, (hipStream_t)stream>>>(probs, v, probs_stride, temperature, top_k, top_p, sa, out_token);
+    hipStream_t s = (hipStream_t)stream;
+    ProfScope ps(ctx, NVMAI_PROF_SAMPLE, s);
+    if (temperature > 0.0f && top_k == 0u && (top_p <= 0.0f || top_p >= 1.0f)) {   // logit.metal:391
+        PosArray pa{};
+        for (uint32_t r = 0; r < rows; ++r) pa.p[r] = positions ? positions[r] : 0u;
+        const int rc = ws_begin(ctx, ws_round((size_t)rows * GUMBEL_BLOCKS * 8));
+        if (rc) return rc;
+        uint64_t* block_best = ws_take<uint64_t>(ctx, (size_t)rows * GUMBEL_BLOCKS);
+        sample_gumbel_kernel<<<dim3(GUMBEL_BLOCKS, rows), 256, 0, s>>>(probs, v, probs_stride, temperature, sa, pa,
+                                                                      block_best, ctx->tickets + GUMBEL_TICKETS,
+                                                                      out_token);
+        return launch_status();
+    }
+    sample_generic_kernel<<<dim3(rows), 256, 0, s>>>(probs, v, probs_stride, temperature, top_k, top_p, sa, out_token);
     return launch_status();
 }

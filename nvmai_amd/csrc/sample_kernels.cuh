@@ -258,4 +258,71 @@ __global__ __launch_bounds__(256) void sample_generic_kernel(const uint16_t* pro
     }
 }
 
+// Gumbel-max draw the reference takes when neither top-k nor top-p is set (logit.metal:296-313,
+// 391-429): argmax_i(log(p_i) / T + g_i), g_i = -log(-log(u_i)), u_i from SplitMix64 of
+// (seed, position, i).  Logarithms in double, rounded to float once per step, so that scores
+// are the same bits on every device.  GUMBEL_BLOCKS blocks per row; the last one to finish
+// folds the block winners (highest score, lowest index among equals).
+constexpr int GUMBEL_BLOCKS = 64;
+struct PosArray { uint32_t p[SAMPLE_MAX_ROWS]; };
+
+__device__ __forceinline__ float gumbel_for(uint64_t seed, uint32_t position, uint32_t row) {
+    uint64_t x = seed ^ ((uint64_t)position * 0xD2B74407B1CE6E93ull) ^ (uint64_t)row;
+    x = x + 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    x = x ^ (x >> 31);
+    const float u = __fmul_rn(__fadd_rn((float)(uint32_t)(x >> 40), 0.5f), 1.0f / 16777216.0f);
+    const float inner = (float)log((double)u);
+    return -(float)log((double)(-inner));
+}
+
+__global__ __launch_bounds__(256) void sample_gumbel_kernel(const uint16_t* probs, uint32_t v, uint32_t probs_stride,
+                                                            float temperature, SeedArray seeds, PosArray positions,
+                                                            uint64_t* block_best, uint32_t* tickets,
+                                                            uint32_t* out_token) {
+    __shared__ uint64_t wave_best[4];
+    __shared__ bool last;
+    const uint32_t row = blockIdx.y;
+    const uint16_t* p = probs + (size_t)row * probs_stride;
+    const float inv_t = __fdiv_rn(1.0f, temperature);
+    uint64_t best = 0;                                   // keys of real candidates are never 0
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < v; i += GUMBEL_BLOCKS * 256) {
+        const float pv = f16_to_f32(p[i]);
+        if (!(pv > 0.0f)) continue;
+        const float sc = __fadd_rn(__fmul_rn(inv_t, (float)log((double)pv)), gumbel_for(seeds.s[row], positions.p[row], i));
+        const uint64_t key = sample_key(sc, i);
+        best = key > best ? key : best;
+    }
+    auto fold = [&](uint64_t b) {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const uint32_t lo = shfl_xor_u((uint32_t)b, off), hi = shfl_xor_u((uint32_t)(b >> 32), off);
+            const uint64_t o = ((uint64_t)hi << 32) | lo;
+            b = o > b ? o : b;
+        }
+        return b;
+    };
+    best = fold(best);
+    if ((threadIdx.x & 63) == 0) wave_best[threadIdx.x >> 6] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        best = max(max(wave_best[0], wave_best[1]), max(wave_best[2], wave_best[3]));
+        block_best[(size_t)row * GUMBEL_BLOCKS + blockIdx.x] = best;
+        __threadfence();
+        last = atomicAdd(&tickets[row], 1u) == GUMBEL_BLOCKS - 1;
+    }
+    __syncthreads();
+    if (!last) return;
+    __threadfence();
+    uint64_t b = threadIdx.x < GUMBEL_BLOCKS ? block_best[(size_t)row * GUMBEL_BLOCKS + threadIdx.x] : 0;
+    if (threadIdx.x < 64) {
+        b = fold(b);
+        if (threadIdx.x == 0) {
+            out_token[row] = b ? key_index(b) : 0u;      // nothing eligible: the reference falls back to 0
+            tickets[row] = 0;                            // ready for the next call
+        }
+    }
+}
+
 }  // namespace nvmai

@@ -531,10 +531,14 @@ class Sample:
     def __init__(self, ctx):
         self.ctx = ctx
 
-    def encode(self, probs, temperature=1.0, top_k=0, top_p=1.0, seed=0):
+    def encode(self, probs, temperature=1.0, top_k=0, top_p=1.0, seed=0, position=0):
+        """seed and position: one value or one per row.  Greedy at temperature <= 0, the Gumbel-max
+        draw when top_k == 0 and top_p is outside (0, 1), else the truncating path."""
         p = probs.reshape(-1, probs.shape[-1])
         rows = p.shape[0]
         out = torch.empty(rows, dtype=torch.int32, device=p.device)
+        pos = position if isinstance(position, (list, tuple)) else [position] * rows
         check(lib.nvmai_hip_sample(self.ctx.handle, _stream(), _ptr(p), p.stride(0), rows, p.shape[1], temperature,
-                                   top_k, top_p, _seed_array(seed, rows), _ptr(out)), "sample")
+                                   top_k, top_p, _seed_array(seed, rows), (C.c_uint32 * rows)(*pos), _ptr(out)),
+              "sample")
         return out

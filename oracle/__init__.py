@@ -76,6 +76,9 @@ _sig("orc_uniform01", C.c_float, C.POINTER(C.c_uint64))
 _sig("orc_seed_for", C.c_uint64, C.c_uint64, C.c_int64)
 _sig("orc_sample_generic", C.c_uint32, u16p, size_t, C.c_float, C.c_uint32, C.c_float,
      C.c_uint64)
+_sig("orc_sample_gumbel", C.c_uint32, u16p, size_t, C.c_float, C.c_uint64, C.c_uint32)
+_sig("orc_sample", C.c_uint32, u16p, size_t, C.c_float, C.c_uint32, C.c_float, C.c_uint64, C.c_uint32)
+_sig("orc_gumbel_for", C.c_float, C.c_uint64, C.c_uint32, C.c_uint32)
 _sig("orc_sample_topk64", C.c_uint32, u16p, size_t, C.c_float, C.c_float, C.c_uint64,
      C.c_uint32, C.c_void_p, C.c_void_p)
 _sig("orc_rel_error", C.c_float, f32p, f32p, size_t)
@@ -416,6 +419,21 @@ def softmax_f16(logits, softcap=0.0, tiled=False):
 def sample_generic(probs_f16, temperature, top_k, top_p, seed):
     p = np.ascontiguousarray(probs_f16, np.uint16)
     return lib.orc_sample_generic(p, p.size, temperature, top_k, top_p, seed)
+
+
+def sample_gumbel(probs_f16, temperature, seed, position=0):
+    p = np.ascontiguousarray(probs_f16, np.uint16)
+    return lib.orc_sample_gumbel(p, p.size, temperature, seed, position)
+
+
+def sample(probs_f16, temperature, top_k, top_p, seed, position=0):
+    """The reference kernel's own choice between greedy, Gumbel-max and the truncating path."""
+    p = np.ascontiguousarray(probs_f16, np.uint16)
+    return lib.orc_sample(p, p.size, temperature, top_k, top_p, seed, position)
+
+
+def gumbel_for(seed, position, row):
+    return lib.orc_gumbel_for(seed, position, row)
 
 
 def sample_topk64(probs_f16, temperature, top_p, seed, top_k=64, want_top64=False):

@@ -21,12 +21,17 @@
  *                                                             tests/test_oracle_prefill.py
  *   KV layout / quantizer           strides 1024/544/288; invariants (min->0,
  *       max->levels, flat->0) and brute-force nearest code.  No reference test
- *       holds KV codes, so the codes are pinned by the closed form only.
+ *       holds KV codes, so the codes are pinned by the closed form only
+ *       (PARITY UNPINNED against the reference).
  *   attention / RoPE                float64 textbook attention, split==single,
  *       geometry known answers, rope identity at position 0  tests/test_oracle_attention.py
  *   softmax / sampler               float64 softmax, tiled==single, generic ==
  *       top-64 token-for-token on the reference's LCG input, xorshift64*
  *       textbook values                                      tests/test_oracle_sampler.py
+ *   Gumbel-max sampler              PARITY UNPINNED against the reference (it holds
+ *       no vector and Metal's fast-math log is not reproducible): pinned by the
+ *       published SplitMix64 constant, the closed form of the noise and the
+ *       property that the draw follows p^(1/T)               tests/test_oracle_sampler.py
  *
  * Canonical summation order of the router logits ("half-wave order"):
  *   a row is cut into 16-byte chunks (16 codes at 8 bits, 32 codes at 4 bits,
@@ -881,6 +886,49 @@ uint32_t orc_sample_generic(const uint16_t *probs_f16, size_t v, float temperatu
     uint32_t kept = 0;
     while (kept < count && idx[kept] < v && isfinite(val[kept])) kept++;
     return sample_tail(val, idx, kept, temperature, top_p, seed, kept > 0 ? idx[0] : 0u);
+}
+
+/* Gumbel-max draw the reference takes when neither top-k nor top-p is set
+ * (logit.metal:296-313, 391-429): argmax_i(log(p_i)/T + g_i), g_i = -log(-log(u_i)), u_i from a
+ * counter-based SplitMix64 of (seed, position, i); zero and negative probabilities are skipped;
+ * highest score wins, lowest index among equals; nothing eligible -> token 0.  The logarithms
+ * are taken in double and rounded to float, one rounding per step, so that a restatement on
+ * another device can reproduce the scores bit for bit (Metal's fast-math log cannot be). */
+static uint64_t lmhead_splitmix64(uint64_t x) {               /* logit.metal:296-301 */
+    x = x + 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+float orc_gumbel_for(uint64_t seed, uint32_t position, uint32_t row) {   /* :303-313 */
+    uint64_t key = seed ^ ((uint64_t)position * 0xD2B74407B1CE6E93ull) ^ (uint64_t)row;
+    uint32_t bits = (uint32_t)(lmhead_splitmix64(key) >> 40);
+    float u = ((float)bits + 0.5f) * (1.0f / 16777216.0f);
+    float inner = (float)log((double)u);
+    return -(float)log((double)(-inner));
+}
+
+uint32_t orc_sample_gumbel(const uint16_t *probs_f16, size_t v, float temperature,
+                           uint64_t seed, uint32_t position) {
+    float inv_t = 1.0f / temperature;
+    float best = -INFINITY;
+    uint32_t bi = 0xFFFFFFFFu;
+    for (size_t i = 0; i < v; ++i) {
+        float p = orc_f16_to_float(probs_f16[i]);
+        if (!(p > 0.0f)) continue;
+        float s = inv_t * (float)log((double)p) + orc_gumbel_for(seed, position, (uint32_t)i);
+        if (s > best) { best = s; bi = (uint32_t)i; }
+    }
+    return bi == 0xFFFFFFFFu ? 0u : bi;
+}
+
+/* The kernel's choice of path (logit.metal:340, 391, 431). */
+uint32_t orc_sample(const uint16_t *probs_f16, size_t v, float temperature, uint32_t top_k,
+                    float top_p, uint64_t seed, uint32_t position) {
+    if (temperature > 0.0f && top_k == 0u && (top_p <= 0.0f || top_p >= 1.0f))
+        return orc_sample_gumbel(probs_f16, v, temperature, seed, position);
+    return orc_sample_generic(probs_f16, v, temperature, top_k, top_p, seed);
 }
 
 typedef struct { float v; uint32_t i; } cand;

@@ -184,6 +184,12 @@ uint64_t orc_xorshift64star(uint64_t *s);            /* logit.metal:280-285 */
 float orc_uniform01(uint64_t *s);                    /* logit.metal:287-292 */
 uint64_t orc_seed_for(uint64_t seed, int64_t position); /* Sampler.swift:304-325 */
 /* generic `sample` (logit.metal:315-585): k argmax passes */
+/* Gumbel-max path (logit.metal:296-313, 391-429) and the kernel's choice of path. */
+float orc_gumbel_for(uint64_t seed, uint32_t position, uint32_t row);
+uint32_t orc_sample_gumbel(const uint16_t *probs_f16, size_t v, float temperature,
+                           uint64_t seed, uint32_t position);
+uint32_t orc_sample(const uint16_t *probs_f16, size_t v, float temperature, uint32_t top_k,
+                    float top_p, uint64_t seed, uint32_t position);
 uint32_t orc_sample_generic(const uint16_t *probs_f16, size_t v, float temperature,
                             uint32_t top_k, float top_p, uint64_t seed);
 /* tiled top-64 (logit.metal:590-758): returns token; if top64_idx/val non-NULL

@@ -129,3 +129,28 @@ def test_softmax_then_sampler_pipeline(nv, ctx):
     ph = u16(probs)
     for r in range(2):
         assert tok[r] == O.sample_topk64(ph[r], 0.6, 0.95, seeds[r], 20)
+
+
+def test_gumbel_max_path_matches_oracle(nv, ctx):
+    say("gumbel sampler", ctx.act)
+    # top_k == 0 and top_p outside (0, 1): logit.metal:391-429; scores must be the same bits
+    gen = nv.Sample(ctx)
+    rng = np.random.default_rng(17)
+    for v in (1003, 248320):
+        p = O.softmax_f16(gauss(rng, (v,), 3.0))
+        p[5] = 0                                                   # an ineligible entry
+        pd = _probs_dev(p)
+        for t, top_p in ((1.0, 1.0), (0.6, 0.0), (2.5, 1.5)):
+            for seed, pos in ((1, 0), (42, 17), (0x123456789ABCDEF0, 4095)):
+                got = int(gen.encode(pd, t, 0, top_p, seed, pos)[0]) & 0xFFFFFFFF
+                assert got == O.sample(p, t, 0, top_p, seed, pos), (v, t, seed, pos)
+    # rows with their own seed and position
+    rows = 7
+    seeds, poss = [100 + r for r in range(rows)], [3 * r for r in range(rows)]
+    batch = gen.encode(pd.expand(rows, -1).contiguous(), 0.8, 0, 1.0, seeds, poss).cpu().numpy().view(np.uint32)
+    assert [int(x) for x in batch] == [O.sample_gumbel(p, 0.8, seeds[r], poss[r]) for r in range(rows)]
+    # a second call right after (the per-row block counters must have been reset)
+    again = gen.encode(pd.expand(rows, -1).contiguous(), 0.8, 0, 1.0, seeds, poss).cpu().numpy().view(np.uint32)
+    assert np.array_equal(batch, again)
+    z = np.zeros(512, np.uint16)
+    assert int(gen.encode(_probs_dev(z), 1.0, 0, 1.0, 1, 0)[0]) == 0   # nothing eligible -> token 0

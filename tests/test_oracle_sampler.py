@@ -103,3 +103,55 @@ def test_sampler_distribution_and_greedy():
     assert np.abs(got - w).max() < 0.03
     assert O.sample_generic(pb, 0.0, 20, 0.95, 1) == 10          # greedy argmax
     assert O.sample_topk64(pb, 1.0, 0.4, 77, 20) == 10           # nucleus cut at the first entry
+
+
+def _splitmix_gumbel_u(seed, position, row):
+    """logit.metal:296-313 in Python integers: the 24-bit draw behind one Gumbel value."""
+    m = (1 << 64) - 1
+    x = (seed ^ ((position * 0xD2B74407B1CE6E93) & m) ^ row) & m
+    x = (x + 0x9E3779B97F4A7C15) & m
+    x = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & m
+    x = ((x ^ (x >> 27)) * 0x94D049BB133111EB) & m
+    x = x ^ (x >> 31)
+    return x >> 40
+
+
+def test_gumbel_noise_closed_form_and_path_choice():
+    # the draw: SplitMix64 of (seed ^ position * C ^ row), top 24 bits, (bits + 0.5) / 2^24
+    for seed, pos, row in [(1, 0, 0), (42, 17, 248319), (0x123456789ABCDEF0, 4095, 7), (0, 0, 0)]:
+        bits = _splitmix_gumbel_u(seed, pos, row)
+        u = np.float32(np.float32(bits) + np.float32(0.5)) * np.float32(1.0 / 16777216.0)
+        want = -np.log(-np.log(np.float64(u)))
+        assert abs(O.gumbel_for(seed, pos, row) - want) <= 4e-7 * max(1.0, abs(want))
+    # SplitMix64's first output for state 0 is a published constant
+    assert _splitmix_gumbel_u(0, 0, 0) == 0xE220A8397B1DCDAF >> 40
+    rng = np.random.default_rng(3)
+    p = O.softmax_f16(rng.standard_normal(1003).astype(np.float32) * 2)
+    # the kernel's choice of path (logit.metal:340, 391, 431)
+    assert O.sample(p, 0.0, 0, 1.0, 5, 9) == O.sample_generic(p, 0.0, 0, 1.0, 5)
+    assert O.sample(p, 0.8, 0, 1.0, 5, 9) == O.sample_gumbel(p, 0.8, 5, 9)
+    assert O.sample(p, 0.8, 0, 0.0, 5, 9) == O.sample_gumbel(p, 0.8, 5, 9)
+    assert O.sample(p, 0.8, 20, 1.0, 5, 9) == O.sample_generic(p, 0.8, 20, 1.0, 5)
+    assert O.sample(p, 0.8, 0, 0.9, 5, 9) == O.sample_generic(p, 0.8, 0, 0.9, 5)
+    # position and seed both move the draw; zero probabilities are never chosen
+    draws = {O.sample_gumbel(p, 1.0, 5, pos) for pos in range(64)}
+    assert len(draws) > 8
+    q = np.zeros(1003, np.uint16)
+    assert O.sample_gumbel(q, 1.0, 1, 0) == 0                      # nothing eligible -> token 0
+    q[777] = O.f16_bits(np.array([0.5], np.float32))[0]
+    assert all(O.sample_gumbel(q, 0.7, s, s) == 777 for s in range(20))
+
+
+def test_gumbel_max_samples_p_to_the_one_over_t():
+    # Gumbel-max over log(p)/T is a categorical draw with weights p^(1/T)
+    rng = np.random.default_rng(0)
+    p = O.softmax_f16(rng.standard_normal(600).astype(np.float32) * 2.5)
+    pf = O.f16_to_float(p).astype(np.float64)
+    for T in (1.0, 0.6):
+        w = np.where(pf > 0, pf ** (1.0 / T), 0.0)
+        w /= w.sum()
+        n = 6000
+        cnt = np.bincount([O.sample_gumbel(p, T, 1000 + s, s % 5) for s in range(n)], minlength=600)
+        top = np.argsort(-w)[:6]
+        sigma = np.sqrt(w[top] * (1 - w[top]) / n)
+        assert np.all(np.abs(cnt[top] / n - w[top]) <= 5 * sigma + 1e-3)
