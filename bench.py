@@ -34,9 +34,10 @@ def parse():
     ap.add_argument("--layers", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--sweep", action="store_true", help="also print batch/bits sweep lines to stderr")
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "copy"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "sampler", "copy"],
                     help="decode = configs[1] (the headline line); prefill = configs[2] grouped GEMM; "
-                         "attention = configs[3] quantized-KV decode attention; copy = a plain 1 GiB device copy, "
+                         "attention = configs[3] quantized-KV decode attention; sampler = the end of configs[4]: "
+                         "quantized LM head GEMV over 248,320 rows, tiled softmax, top-k sampler; copy = a plain 1 GiB device copy, "
                          "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated on")
     ap.add_argument("--context", type=int, default=32768, help="attention: tokens in the KV cache")
     ap.add_argument("--tokens", type=int, default=4096, help="prefill: tokens per step")
@@ -339,6 +340,81 @@ def run_attention(nv, ctx, torch, a):
     }
 
 
+def run_sampler(nv, ctx, torch, a):
+    """The end of configs[4]: logits = LM head (4/8-bit affine [248320, 2048]) x hidden, softcap +
+    tiled softmax, tiled top-k sampler (k 20, top-p 0.95, T 0.6, fixed seed) for `--batch` rows."""
+    V, bits, rows = 248320, a.bits, min(a.batch, 32)
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    n_heads = 4                                            # rotate copies of the head past the caches
+    heads = []
+    for _ in range(n_heads):
+        wt = torch.empty((V, D), dtype=torch.bfloat16, device="cuda").normal_(0.0, 0.02, generator=gen)
+        heads.append(nv.quantize_affine(ctx, wt, bits))
+        del wt
+    xs = torch.empty((8, rows, D), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
+    sm, tk = nv.LogitSoftcapSoftmaxTiled(ctx, V), nv.SampleTopK64(ctx, V)
+    probs = torch.empty((rows, V), dtype=torch.float16, device="cuda")
+    seeds = [nv.sampler_seed_for(1234, r) for r in range(rows)]
+
+    qmm = nv.MPPPrefillInt4QMM(ctx, bits)
+    logits_buf = torch.empty((rows, V), dtype=torch.bfloat16, device="cuda")
+
+    def head(i):
+        # a few rows: the GEMV (each weight row read once per group of 4 inputs); more: the
+        # matrix-core product (weights read and dequantized once for all rows)
+        p_, s_, b_ = heads[i % n_heads]
+        if rows <= 4:
+            return nv.affine_gemv(ctx, p_, s_, b_, bits, xs[i % 8], V, D)
+        return qmm.encode(p_, s_, b_, xs[i % 8], V, D, logits_buf)
+
+    def step(i):
+        logits = head(i)
+        sm.encode(logits, probs, softcap=30.0)
+        return tk.encode(probs, 0.6, 0.95, seeds, 20)
+
+    for i in range(a.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(i)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    # the GEMV alone, by events
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    ev[0].record()
+    for i in range(a.steps):
+        head(i)
+    ev[1].record()
+    torch.cuda.synchronize()
+    gemv_us = ev[0].elapsed_time(ev[1]) / a.steps * 1e3
+    ctx.profile_enable(True)
+    for i in range(a.steps):
+        step(i)
+    torch.cuda.synchronize()
+    ctx.profile_enable(False)
+    kern = {"lm_head_gemv": gemv_us}
+    for tag, name in ((nv.PROF_SOFTMAX, "softmax"), (nv.PROF_SAMPLE, "sample_topk64")):
+        ms, n = ctx.profile_read(tag)
+        kern[name] = ms / max(n, 1) * 1e3
+    head_bytes = V * D * bits / 8 + 2 * V * (D // 64) * 2
+    step_bytes_ = head_bytes + rows * (D * 2 + V * 2 * 2 + V * 2)   # x, logits w+r, probs w (+ r by the sampler)
+    gbps = head_bytes / (gemv_us * 1e-6) / 1e9
+    return {
+        "metric": METRIC, "value": round(rows / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u%d codes, f32 accumulate; fp16 probabilities" % bits, "data": "synthetic",
+        "config": {"workload": "end of configs[4]: %d-bit LM head GEMV over 248,320 x 2048, softcap + tiled softmax, "
+                               "tiled top-k sampler (k 20, top-p 0.95, T 0.6), %d rows per step" % (bits, rows),
+                   "step_gbps": round(step_bytes_ / dt / 1e9, 1),
+                   "kernel_us": {k: round(v, 2) for k, v in kern.items()}},
+        "roofline": {"kernel": "LM head: expert_rows GEMV (<= 4 rows) or prefill_gemm_kernel (more)", "bound": "hbm", "achieved": round(gbps, 2),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_launch": head_bytes, "avg_launch_us": round(gemv_us, 2)},
+        "cpu_baseline": None,
+    }
+
+
 def run_copy(torch, a):
     """A plain copy kernel of known size: 1 GiB read + 1 GiB written per launch."""
     n = 1 << 30
@@ -372,7 +448,8 @@ def main():
     ctx = nv.Context(0, nv.ACT_BF16)
     if a.workload != "decode":
         line = (run_prefill(nv, ctx, torch, a) if a.workload == "prefill" else
-                run_attention(nv, ctx, torch, a) if a.workload == "attention" else run_copy(torch, a))
+                run_attention(nv, ctx, torch, a) if a.workload == "attention" else
+                run_sampler(nv, ctx, torch, a) if a.workload == "sampler" else run_copy(torch, a))
         print(json.dumps(line), flush=True)
         return
     layers, stride = build_layers(nv, ctx, torch, a.bits, a.layers)

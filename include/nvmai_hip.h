@@ -272,6 +272,15 @@ int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream stream, const
                                   const nvmai_prefill_grouping* grouping, void* act_scratch,
                                   void* route_partials);
 
+/* MPPPrefillInt4QMM.encode (MPPPrefillInt4QMM.swift:63-128; kernel tensorops.metal:29-121):
+ * the dense prefill product y[m, n] = x[m, k] . W[n, k]^T for m rows of activations against
+ * one affine 4/8-bit matrix (group 64 along k, BF16 scale/bias), on the matrix cores: weights
+ * dequantized once into MFMA operands, fp32 accumulate, y rounded to the activation type.
+ * k must be a multiple of 64; x, y and the code rows 16-byte aligned. */
+int nvmai_hip_affine_qmm(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
+                         const uint16_t* scales, const uint16_t* biases, uint32_t bits, const void* x,
+                         uint32_t x_stride, void* y, uint32_t y_stride, uint32_t m, uint32_t n, uint32_t k);
+
 /* PrefillMoE.encodeReduceTokenMajor (PrefillMoE.swift:11-40; prefill.metal:437-458):
  * h2[t, :] = sum over ranks, in rank order, of fma(w[t, r], route_partials[t*top_k + r, :]). */
 int nvmai_hip_prefill_moe_reduce_token_major(nvmai_hip_ctx* ctx, nvmai_stream stream,

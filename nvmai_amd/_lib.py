@@ -90,6 +90,7 @@ SIGNATURES = {
     "nvmai_hip_prefill_group_routes": [vp, vp, vp, vp, u32, u32, u32, u32, vp, u64, C.POINTER(PrefillGrouping)],
     "nvmai_hip_prefill_grouped_moe": [vp, vp, vp, u64, C.POINTER(ExpertOffsets), u32, u32, u32, u32, vp, u32,
                                       u32, u32, C.POINTER(PrefillGrouping), vp, vp],
+    "nvmai_hip_affine_qmm": [vp, vp, vp, vp, vp, u32, vp, u32, vp, u32, u32, u32, u32],
     "nvmai_hip_prefill_moe_reduce_token_major": [vp, vp, vp, vp, vp, u32, u32, u32, u32],
     "nvmai_hip_sample": [vp, vp, vp, u32, u32, u32, C.c_float, u32, C.c_float, C.POINTER(u64), C.POINTER(u32), vp],
 }

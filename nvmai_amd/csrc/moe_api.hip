@@ -331,16 +331,9 @@ int affine_gemv_any(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weig
     launch_rows(ctx->act, bits, false, x_is_f32, p, maxtok, ents, s);
     if (need_tmp) {
         // copy out with the caller's stride (and convert when asked)
-        for (uint32_t t = 0; t < n_tokens; ++t) {
-            if (y) {
-                uint16_t* dst = (uint16_t*)y + (size_t)t * y_stride;
-                if (ctx->act == ACT_BF16) store_act_kernel<ACT_BF16><<<(m + 255) / 256, 256, 0, s>>>(tmp + (size_t)t * m, dst, m);
-                else store_act_kernel<ACT_FP16><<<(m + 255) / 256, 256, 0, s>>>(tmp + (size_t)t * m, dst, m);
-            }
-            if (y_f32)
-                NVMAI_HIP_TRY(hipMemcpyAsync(y_f32 + (size_t)t * y_stride, tmp + (size_t)t * m,
-                                             (size_t)m * 4, hipMemcpyDeviceToDevice, s));
-        }
+        const dim3 grid((m + 255) / 256, n_tokens);
+        if (ctx->act == ACT_BF16) store_rows_kernel<ACT_BF16><<<grid, 256, 0, s>>>(tmp, y, y_f32, m, y_stride);
+        else store_rows_kernel<ACT_FP16><<<grid, 256, 0, s>>>(tmp, y, y_f32, m, y_stride);
     }
     return launch_status();
 }

@@ -880,11 +880,15 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineParams p) {
     ((uint16_t*)p.y)[(size_t)t * p.y_stride + d] = f32_to_act<ACT>(acc);
 }
 
-// fp32 [rows, n] -> activations, optionally through act = silu(a) * b of two inputs
+// fp32 rows [tokens, m] -> the caller's rows with its own stride: 16-bit activations (y) and /
+// or fp32 (yf).  blockIdx.y = token.
 template <int ACT>
-__global__ void store_act_kernel(const float* a, void* y, uint32_t count) {
-    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < count) ((uint16_t*)y)[i] = f32_to_act<ACT>(a[i]);
+__global__ void store_rows_kernel(const float* a, void* y, float* yf, uint32_t m, uint32_t y_stride) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
+    if (i >= m) return;
+    const float v = a[(size_t)t * m + i];
+    if (y) ((uint16_t*)y)[(size_t)t * y_stride + i] = f32_to_act<ACT>(v);
+    if (yf) yf[(size_t)t * y_stride + i] = v;
 }
 
 // ---- affine group-64 quantizer ---------------------------------------------------------

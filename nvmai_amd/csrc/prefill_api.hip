@@ -124,8 +124,14 @@ extern "C" int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream s
 
 namespace {
 
+// Blocks of a launch over at most max_mtiles M tiles: whole units, dealt over eight XCDs.
+uint32_t gemm_grid(uint32_t max_mtiles, const GemmParams& g) {
+    const uint32_t units = max_mtiles * g.units_per_tile;
+    return (units + 7) / 8 * 8 * GEMM_UNIT;
+}
+
 template <int ACT, int BITS, int NT>
-void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t mtiles8, nvmai_hip_ctx* ctx, hipStream_t s) {
+void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t max_mtiles, nvmai_hip_ctx* ctx, hipStream_t s) {
     const size_t lds = (size_t)2 * GEMM_BM * GEMM_LDK * 2;     // 68 KB: above the 64 KB a launch gets unasked
     static bool raised = false;
     if (!raised) {
@@ -137,11 +143,11 @@ void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t mtiles8, 
     }
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM1, s);
-        prefill_gemm_kernel<ACT, BITS, true, NT><<<mtiles8 * g1.n_tiles_n, 256, lds, s>>>(g1);
+        prefill_gemm_kernel<ACT, BITS, true, NT><<<gemm_grid(max_mtiles, g1), 256, lds, s>>>(g1);
     }
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM2, s);
-        prefill_gemm_kernel<ACT, BITS, false, NT><<<mtiles8 * g2.n_tiles_n, 256, lds, s>>>(g2);
+        prefill_gemm_kernel<ACT, BITS, false, NT><<<gemm_grid(max_mtiles, g2), 256, lds, s>>>(g2);
     }
 }
 
@@ -188,20 +194,72 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
     g1.x = hidden; g1.x_stride = hidden_stride;
     g1.out = act_scratch; g1.out_stride = f;
     g1.K = d; g1.N = f; g1.top_k = top_k; g1.n_tiles_n = (f + 32 * nt - 1) / (32 * nt);
+    g1.units_per_tile = (g1.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
     GemmParams g2 = g1;
     g2.wA = off->down_w; g2.sA = off->down_s; g2.bA = off->down_b;
     g2.wB = g2.sB = g2.bB = 0;
     g2.x = act_scratch; g2.x_stride = f;
     g2.out = route_partials; g2.out_stride = d;
     g2.K = f; g2.N = d; g2.n_tiles_n = (d + 64 * nt - 1) / (64 * nt);
-    const uint32_t mtiles8 = (max_mtiles + 7) / 8 * 8;
+    g2.units_per_tile = (g2.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
     if (ctx->act == ACT_BF16) {
-        if (bits == 4) launch_gemms<ACT_BF16, 4, 4>(g1, g2, mtiles8, ctx, s);
-        else launch_gemms<ACT_BF16, 8, 2>(g1, g2, mtiles8, ctx, s);
+        if (bits == 4) launch_gemms<ACT_BF16, 4, 4>(g1, g2, max_mtiles, ctx, s);
+        else launch_gemms<ACT_BF16, 8, 2>(g1, g2, max_mtiles, ctx, s);
     } else {
-        if (bits == 4) launch_gemms<ACT_FP16, 4, 4>(g1, g2, mtiles8, ctx, s);
-        else launch_gemms<ACT_FP16, 8, 2>(g1, g2, mtiles8, ctx, s);
+        if (bits == 4) launch_gemms<ACT_FP16, 4, 4>(g1, g2, max_mtiles, ctx, s);
+        else launch_gemms<ACT_FP16, 8, 2>(g1, g2, max_mtiles, ctx, s);
     }
+    return launch_status();
+}
+
+namespace {
+template <int ACT, int BITS, int NT>
+void launch_qmm(const GemmParams& g, uint32_t blocks, hipStream_t s) {
+    const size_t lds = (size_t)2 * GEMM_BM * GEMM_LDK * 2;
+    static bool raised = false;
+    if (!raised) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, false, NT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        raised = true;
+    }
+    prefill_gemm_kernel<ACT, BITS, false, NT><<<blocks, 256, lds, s>>>(g);
+}
+}  // namespace
+
+extern "C" int nvmai_hip_affine_qmm(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
+                                    const uint16_t* scales, const uint16_t* biases, uint32_t bits,
+                                    const void* x, uint32_t x_stride, void* y, uint32_t y_stride, uint32_t m,
+                                    uint32_t n, uint32_t k) {
+    if (!ctx || !weights || !scales || !biases || !x || !y) return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    if (n == 0 || k == 0 || k % NVMAI_GROUP || x_stride < k || y_stride < n) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(weights) || !aligned16(x) || x_stride % 8 || !aligned16(y) ||
+        (reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 1u)
+        return NVMAI_ERR_ALIGNMENT;
+    if (m == 0) return NVMAI_OK;
+    if (m >= (1u << 28)) return NVMAI_ERR_UNSUPPORTED;
+    const uint32_t tiles = (m + GEMM_BM - 1) / GEMM_BM;
+    int rc = ws_begin(ctx, ws_round((size_t)tiles * sizeof(MTile)) + ws_round(64) + ws_round((size_t)m * sizeof(PrefillPair)));
+    if (rc) return rc;
+    MTile* mtiles = ws_take<MTile>(ctx, tiles);
+    uint32_t* n_mtiles = ws_take<uint32_t>(ctx, 16);
+    PrefillPair* pairs = ws_take<PrefillPair>(ctx, m);
+    hipStream_t s = (hipStream_t)stream;
+    ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM2, s);
+    qmm_setup_kernel<<<(m + 255) / 256, 256, 0, s>>>(m, mtiles, n_mtiles, pairs);
+    const uint32_t nt = bits == 4 ? 4 : 2;
+    GemmParams g{};
+    g.pool = weights; g.pool_stride = 0;
+    g.wA = 0;
+    g.sA = reinterpret_cast<const uint8_t*>(scales) - weights;
+    g.bA = reinterpret_cast<const uint8_t*>(biases) - weights;
+    g.mtiles = mtiles; g.n_mtiles = n_mtiles; g.pairs = pairs;
+    g.x = x; g.x_stride = x_stride; g.out = y; g.out_stride = y_stride;
+    g.K = k; g.N = n; g.top_k = 1; g.n_tiles_n = (n + 64 * nt - 1) / (64 * nt);
+    g.units_per_tile = (g.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
+    const uint32_t blocks = gemm_grid(tiles, g);
+    if (ctx->act == ACT_BF16) { if (bits == 4) launch_qmm<ACT_BF16, 4, 4>(g, blocks, s); else launch_qmm<ACT_BF16, 8, 2>(g, blocks, s); }
+    else { if (bits == 4) launch_qmm<ACT_FP16, 4, 4>(g, blocks, s); else launch_qmm<ACT_FP16, 8, 2>(g, blocks, s); }
     return launch_status();
 }
 

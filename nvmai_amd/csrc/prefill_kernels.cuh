@@ -300,9 +300,11 @@ struct GemmParams {
     void* out;                          // DUAL: act[sorted position, N]; else partials[token*top_k+rank, N]
     uint32_t out_stride;
     uint32_t K, N, top_k, n_tiles_n;
+    uint32_t units_per_tile;            // ceil(n_tiles_n / GEMM_UNIT)
 };
 
 constexpr int GEMM_SK = 128;            // k per super-step
+constexpr uint32_t GEMM_UNIT = 4;       // column tiles of one M tile that share an XCD
 constexpr int GEMM_LDK = GEMM_SK + 8;   // padded LDS row: conflict-free 16-byte reads and writes
 
 // Two floats -> two 16-bit activations in one dword, round to nearest even.
@@ -342,12 +344,16 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     constexpr int GEMM_WST = (NT == 4 || BITS == 8) ? 2 : 4;
     extern __shared__ uint4 gemm_lds[];
     uint16_t* xs = reinterpret_cast<uint16_t*>(gemm_lds);      // [2][128][LDK]
-    // Blocks are dealt to the eight XCDs round-robin.  The column tiles of one M tile go to one
-    // XCD, back to back, so that its activation rows are fetched into one L2 only; the M tiles
-    // themselves (sorted by size) are dealt over the XCDs in turn, which balances them.
+    // Blocks are dealt to the eight XCDs round-robin.  A unit = up to GEMM_UNIT consecutive column
+    // tiles of one M tile; its blocks run back to back on one XCD, so that the tile's activation
+    // rows are fetched into that L2 once, and the units (M tiles sorted by size, then columns)
+    // are dealt over the XCDs in turn, which balances them whether there are many M tiles (the
+    // grouped product) or one (a dense product with few rows).
     const uint32_t on_xcd = blockIdx.x >> 3;
-    const uint32_t tile_id = (on_xcd / p.n_tiles_n) * 8 + (blockIdx.x & 7u), nt = on_xcd % p.n_tiles_n;
-    if (tile_id >= *p.n_mtiles) return;
+    const uint32_t unit = (on_xcd / GEMM_UNIT) * 8 + (blockIdx.x & 7u);
+    const uint32_t tile_id = unit / p.units_per_tile;
+    const uint32_t nt = (unit % p.units_per_tile) * GEMM_UNIT + on_xcd % GEMM_UNIT;
+    if (tile_id >= *p.n_mtiles || nt >= p.n_tiles_n) return;
     const MTile mt = p.mtiles[tile_id];
     const uint8_t* blob = p.pool + (uint64_t)mt.expert * p.pool_stride;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -537,6 +543,17 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
                 if (c0 + j < p.N) out[orow + c0 + j] = e[j];
         }
     }
+}
+
+// Work list of a dense product y = x . W^T: M tiles of 128 consecutive rows of one "expert" 0,
+// identity pair records (row i -> output row i).
+__global__ __launch_bounds__(256) void qmm_setup_kernel(uint32_t m, MTile* mtiles, uint32_t* n_mtiles,
+                                                       PrefillPair* pairs) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < m) pairs[i] = PrefillPair{i, 0u, 0u, 0u};
+    const uint32_t tiles = (m + GEMM_BM - 1) / GEMM_BM;
+    if (i < tiles) mtiles[i] = MTile{0u, i * GEMM_BM, min((uint32_t)GEMM_BM, m - i * GEMM_BM)};
+    if (i == 0) *n_mtiles = tiles;
 }
 
 // ---- combine (prefill.metal:437-458) -------------------------------------------------------

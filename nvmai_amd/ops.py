@@ -374,6 +374,26 @@ class PrefillGroupedRoutedMoE:
         return route_partials, act_scratch
 
 
+class MPPPrefillInt4QMM:
+    """MPPPrefillInt4QMM.encode (MPPPrefillInt4QMM.swift:63-128): y[m, n] = x[m, k] . W[n, k]^T on the
+    matrix cores for one affine 4/8-bit matrix."""
+    tile_k = 64
+
+    def __init__(self, ctx, weight_bits=4):
+        if weight_bits not in (4, 8):
+            raise _lib.NvmaiError(-2, "MPPPrefillInt4QMM(weight_bits)")
+        self.ctx, self.bits = ctx, weight_bits
+
+    def encode(self, weights, scales, biases, x, n, k, y=None):
+        x2 = x.reshape(-1, x.shape[-1])
+        m = x2.shape[0]
+        if y is None:
+            y = torch.empty((m, n), dtype=self.ctx.dtype, device=x.device)
+        check(lib.nvmai_hip_affine_qmm(self.ctx.handle, _stream(), _ptr(weights), _ptr(scales), _ptr(biases), self.bits,
+                                       _ptr(x2), x2.stride(0), _ptr(y), y.stride(0), m, n, k), "affine_qmm")
+        return y
+
+
 class PrefillMoE:
     """PrefillMoE.encodeReduceTokenMajor (PrefillMoE.swift:11-40)."""
 

@@ -279,3 +279,35 @@ def test_grouped_moe_production_shape(nv, ctx_bf16, bits):
     h2b = red.encode_reduce_token_major(p2, wd[:512].contiguous(), 512, k, d)
     torch.cuda.synchronize()
     assert torch.equal(h2b, h2[:512])
+
+
+# ------------------------------------------------------------------ dense QMM
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (16, 1000, 2048), (130, 384, 192), (300, 2048, 512)])
+def test_dense_qmm_matches_oracle(nv, ctx, bits, m, n, k):
+    say("dense qmm", ctx.act, bits, m, n, k)
+    # MPPPrefillInt4QMMTests.swift:190-201 bars: max-abs <= 0.03, relative <= 1e-3 of an fp16 path
+    # against its own fp16 oracle; here the bar is the 16-bit class, 1e-2 of max|ref|.
+    rng = np.random.default_rng(m * 7 + n + k + bits)
+    w = gauss(rng, (n, k), 0.05)
+    p, s, b = O.quantize_affine(w, bits)
+    xs = gauss(rng, (m, k))
+    x = O.round_bf16(xs) if ctx.act == 0 else O.f16_to_float(O.f16_bits(xs))
+    y = nv.MPPPrefillInt4QMM(ctx, bits).encode(dev(p), dev(s.view(np.int16)), dev(b.view(np.int16)),
+                                               act_tensor(x, ctx), n, k)
+    torch.cuda.synchronize()
+    want = np.stack([O.affine_gemv(p, s, b, x[t], bits) for t in range(m)])
+    assert O.rel_error(act_np(y), want) <= TOL_ACT
+
+
+def test_dense_qmm_rejects_bad_arguments(nv, ctx_bf16):
+    say("dense qmm errors")
+    q = nv.MPPPrefillInt4QMM(ctx_bf16, 4)
+    p = torch.zeros((64, 48), dtype=torch.uint8, device="cuda")
+    s = torch.zeros((64, 1), dtype=torch.int16, device="cuda")
+    x = torch.zeros((4, 96), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(nv.NvmaiError) as e:                       # k not a multiple of 64
+        q.encode(p, s, s, x, 64, 96)
+    assert e.value.name == "invalid_arg"
+    with pytest.raises(nv.NvmaiError):
+        nv.MPPPrefillInt4QMM(ctx_bf16, 3)
