@@ -105,50 +105,97 @@ __device__ __forceinline__ float key_value(uint64_t k) {
 }
 __device__ __forceinline__ uint32_t key_index(uint64_t k) { return ~(uint32_t)k; }
 
-// Bitonic sort of 1024 keys in LDS, descending (logit.metal:596-626).
-__device__ __forceinline__ void sort_tile_desc(uint64_t* keys) {
-    for (uint32_t width = 2; width <= SAMPLE_TILE; width <<= 1) {
-        for (uint32_t stride = width >> 1; stride > 0; stride >>= 1) {
-            __syncthreads();
-            for (uint32_t i = threadIdx.x; i < SAMPLE_TILE; i += 256) {
-                const uint32_t partner = i ^ stride;
-                if (partner <= i) continue;
-                const uint64_t a = keys[i], b = keys[partner];
-                const bool descending = (i & width) == 0;
-                if (descending ? (b > a) : (a > b)) { keys[i] = b; keys[partner] = a; }
+// The reference sorts every 1024-entry tile with a bitonic network in threadgroup memory and
+// keeps the first 64 (logit.metal:596-626).  Only those 64 matter, and the comparator is a total
+// order, so any exact selection gives the same keys in the same order.  Here each wave sorts 256
+// keys held in registers (key i = reg * 64 + lane; strides below 64 are lane exchanges, 64 and
+// 128 are register swaps: no barriers), the four waves' best 64 meet in LDS, and wave 0 sorts
+// those 256 once more.
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask) {
+    const uint32_t lo = shfl_xor_u((uint32_t)v, mask), hi = shfl_xor_u((uint32_t)(v >> 32), mask);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+__device__ __forceinline__ void wave_sort256_desc(uint64_t k[4], int lane) {
+#pragma unroll
+    for (int width = 2; width <= 256; width <<= 1) {
+#pragma unroll
+        for (int stride = width >> 1; stride > 0; stride >>= 1) {
+            if (stride >= 64) {
+                const int rs = stride >> 6;                        // partner register = r ^ rs
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (r & rs) continue;
+                    const bool desc = (((r << 6) | lane) & width) == 0;
+                    const uint64_t a = k[r], b = k[r ^ rs];
+                    const bool swap = desc ? (b > a) : (a > b);
+                    k[r] = swap ? b : a;
+                    k[r ^ rs] = swap ? a : b;
+                }
+            } else {
+                const bool lower = (lane & stride) == 0;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const bool desc = (((r << 6) | lane) & width) == 0;
+                    const uint64_t a = k[r], b = shfl_xor_u64(a, stride);
+                    const bool take_max = desc == lower;
+                    k[r] = take_max ? (a > b ? a : b) : (a > b ? b : a);
+                }
             }
         }
     }
+}
+
+// The best SAMPLE_KEEP of the block's 1024 keys (mine[r] = key r * 256 + thread), descending,
+// returned in lanes 0..63 of wave 0 (`valid` there); `cand` is 256 keys of LDS.
+__device__ __forceinline__ uint64_t tile_top64(uint64_t mine[4], uint64_t* cand, bool& valid) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    wave_sort256_desc(mine, lane);
+    cand[wave * 64 + lane] = mine[0];                             // sorted keys 0..63 of this wave
     __syncthreads();
+    valid = wave == 0;
+    uint64_t k[4] = {0, 0, 0, 0};
+    if (wave == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) k[r] = cand[r * 64 + lane];
+        wave_sort256_desc(k, lane);
+    }
+    return k[0];
 }
 
 // Stage 1 (logit.metal:628-654): top 64 of each 1024-entry tile of the fp16 probabilities.
 __global__ __launch_bounds__(256) void sample_topk64_stage1_kernel(const uint16_t* probs, uint32_t v,
                                                                    uint32_t probs_stride, uint64_t* out,
                                                                    uint32_t out_row_stride) {
-    __shared__ uint64_t keys[SAMPLE_TILE];
+    __shared__ uint64_t cand[256];
     const uint32_t row = blockIdx.y, base = blockIdx.x * SAMPLE_TILE;
     const uint16_t* p = probs + (size_t)row * probs_stride;
-    for (uint32_t i = threadIdx.x; i < SAMPLE_TILE; i += 256) {
-        const uint32_t src = base + i;
-        keys[i] = src < v ? sample_key(f16_to_f32(p[src]), src) : sample_key(-INFINITY, 0xFFFFFFFFu);
+    uint64_t mine[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t src = base + r * 256 + threadIdx.x;
+        mine[r] = src < v ? sample_key(f16_to_f32(p[src]), src) : sample_key(-INFINITY, 0xFFFFFFFFu);
     }
-    sort_tile_desc(keys);
-    if (threadIdx.x < SAMPLE_KEEP) out[(size_t)row * out_row_stride + blockIdx.x * SAMPLE_KEEP + threadIdx.x] = keys[threadIdx.x];
+    bool valid;
+    const uint64_t best = tile_top64(mine, cand, valid);
+    if (valid) out[(size_t)row * out_row_stride + blockIdx.x * SAMPLE_KEEP + threadIdx.x] = best;
 }
 
 // Reduce (logit.metal:656-682): top 64 of each 1024 surviving candidates.
 __global__ __launch_bounds__(256) void sample_topk64_reduce_kernel(const uint64_t* in, uint32_t count,
                                                                    uint32_t in_row_stride, uint64_t* out,
                                                                    uint32_t out_row_stride) {
-    __shared__ uint64_t keys[SAMPLE_TILE];
+    __shared__ uint64_t cand[256];
     const uint32_t row = blockIdx.y, base = blockIdx.x * SAMPLE_TILE;
-    for (uint32_t i = threadIdx.x; i < SAMPLE_TILE; i += 256) {
-        const uint32_t src = base + i;
-        keys[i] = src < count ? in[(size_t)row * in_row_stride + src] : sample_key(-INFINITY, 0xFFFFFFFFu);
+    uint64_t mine[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t src = base + r * 256 + threadIdx.x;
+        mine[r] = src < count ? in[(size_t)row * in_row_stride + src] : sample_key(-INFINITY, 0xFFFFFFFFu);
     }
-    sort_tile_desc(keys);
-    if (threadIdx.x < SAMPLE_KEEP) out[(size_t)row * out_row_stride + blockIdx.x * SAMPLE_KEEP + threadIdx.x] = keys[threadIdx.x];
+    bool valid;
+    const uint64_t best = tile_top64(mine, cand, valid);
+    if (valid) out[(size_t)row * out_row_stride + blockIdx.x * SAMPLE_KEEP + threadIdx.x] = best;
 }
 
 // Selection over the sorted candidates (logit.metal:704-757 == :517-571): cap at k,
@@ -188,27 +235,59 @@ __global__ __launch_bounds__(256) void sample_topk64_final_kernel(const uint64_t
                                                                   float top_p, SeedArray seeds,
                                                                   uint32_t top_k, uint32_t* out_token,
                                                                   uint32_t* top64) {
-    __shared__ uint64_t keys[SAMPLE_TILE];
+    __shared__ uint64_t cand[256];
     __shared__ float val[SAMPLE_KEEP];
     __shared__ uint32_t idx[SAMPLE_KEEP];
     const uint32_t row = blockIdx.x;
-    for (uint32_t i = threadIdx.x; i < SAMPLE_TILE; i += 256)
-        keys[i] = i < count ? in[(size_t)row * in_row_stride + i] : sample_key(-INFINITY, 0xFFFFFFFFu);
-    sort_tile_desc(keys);
-    if (threadIdx.x < SAMPLE_KEEP) {
-        val[threadIdx.x] = key_value(keys[threadIdx.x]);
-        idx[threadIdx.x] = key_index(keys[threadIdx.x]);
+    uint64_t mine[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t i = r * 256 + threadIdx.x;
+        mine[r] = i < count ? in[(size_t)row * in_row_stride + i] : sample_key(-INFINITY, 0xFFFFFFFFu);
+    }
+    bool valid;
+    const uint64_t best = tile_top64(mine, cand, valid);
+    if (valid) {
+        val[threadIdx.x] = key_value(best);
+        idx[threadIdx.x] = key_index(best);
         if (top64) {
             top64[((size_t)row * SAMPLE_KEEP + threadIdx.x) * 2] = __float_as_uint(val[threadIdx.x]);
             top64[((size_t)row * SAMPLE_KEEP + threadIdx.x) * 2 + 1] = idx[threadIdx.x];
         }
     }
     __syncthreads();
+    if (threadIdx.x >= 64) return;
+    // wave 0: the candidates' p^(1/T) in parallel (the same function on other lanes: the same
+    // bits), every running sum by lane 0 in candidate order as the reference's single thread does
+    __shared__ float powed[SAMPLE_KEEP];
+    const float inv_t = __fdiv_rn(1.0f, temperature);
+    powed[threadIdx.x] = temperature != 1.0f ? powf(val[threadIdx.x], inv_t) : val[threadIdx.x];
+    __builtin_amdgcn_wave_barrier();
     if (threadIdx.x == 0) {
         uint32_t kept = 0;
         while (kept < SAMPLE_KEEP && idx[kept] != 0xFFFFFFFFu && isfinite(val[kept])) kept++;
         kept = min(kept, max(1u, top_k));
-        out_token[row] = sample_select(val, idx, kept, temperature, top_p, seeds.s[row], idx[0]);
+        if (top_p > 0.0f && top_p < 1.0f) {
+            float cum = 0.0f;
+            uint32_t cut = kept;
+            for (uint32_t i = 0; i < kept; ++i) {
+                cum = __fadd_rn(cum, val[i]);
+                if (cum >= top_p) { cut = i + 1; break; }
+            }
+            kept = cut;
+        }
+        float surviving = 0.0f;
+        for (uint32_t i = 0; i < kept; ++i) surviving = __fadd_rn(surviving, powed[i]);
+        uint64_t rng = seeds.s[row];
+        (void)xorshift64star(rng);
+        const float u = __fmul_rn(uniform01(rng), surviving);
+        float run = 0.0f;
+        uint32_t picked = idx[0];
+        for (uint32_t i = 0; i < kept; ++i) {
+            run = __fadd_rn(run, powed[i]);
+            if (u <= run) { picked = idx[i]; break; }
+        }
+        out_token[row] = picked;
     }
 }
 
