@@ -16,7 +16,7 @@ struct nvmai_hip_ctx {
     uint8_t* ws;
     size_t ws_cap;
     size_t ws_used;
-    uint32_t* tickets;       // small zero-initialised device array for last-block-done kernels
+    uint32_t* tickets;       // zero-initialised device words for last-block-done kernels (TICKET_WORDS)
     // Optional per-kernel timing: event pairs recorded around tagged launches.
     bool prof_on;
     struct ProfSpan { int tag; hipEvent_t start, stop; };
@@ -25,6 +25,11 @@ struct nvmai_hip_ctx {
 };
 
 namespace nvmai {
+
+// The context's persistent zeroed words: [0] work-list ticket, [8] prefill grouping error word,
+// [16, 48) sampler block counters, [TICKET_GROUPS, TICKET_WORDS) router token-group tickets.
+constexpr uint32_t TICKET_WORDS = 2048;
+constexpr uint32_t TICKET_GROUPS = 64;
 
 #define NVMAI_HIP_TRY(expr)                         \
     do {                                            \

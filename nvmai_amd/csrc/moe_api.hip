@@ -27,8 +27,8 @@ extern "C" int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** o
     ctx->ws_used = 0;
     ctx->prof_on = false;
     ctx->tickets = nullptr;
-    if (hipMalloc(reinterpret_cast<void**>(&ctx->tickets), 256) != hipSuccess ||
-        hipMemset(ctx->tickets, 0, 256) != hipSuccess) {
+    if (hipMalloc(reinterpret_cast<void**>(&ctx->tickets), TICKET_WORDS * 4) != hipSuccess ||
+        hipMemset(ctx->tickets, 0, TICKET_WORDS * 4) != hipSuccess) {
         delete ctx;
         return NVMAI_ERR_HIP;
     }
@@ -215,10 +215,11 @@ uint32_t rows_chunks(int kind, uint32_t d) { return kind == 16 ? d / 8 : (kind =
 
 template <int ACT>
 void run_router_t(const RouterParams& rp, uint32_t cpl, dim3 grid, hipStream_t s) {
-    if (cpl <= 1) router_logits_kernel<ACT, 1><<<grid, 256, 0, s>>>(rp);
-    else if (cpl <= 2) router_logits_kernel<ACT, 2><<<grid, 256, 0, s>>>(rp);
-    else if (cpl <= 4) router_logits_kernel<ACT, 4><<<grid, 256, 0, s>>>(rp);
-    else router_logits_kernel<ACT, 8><<<grid, 256, 0, s>>>(rp);
+    const size_t lds = (size_t)ROUTER_TOK * rp.d * 2;             // the block's token rows
+    if (cpl <= 1) router_logits_kernel<ACT, 1><<<grid, 256, lds, s>>>(rp);
+    else if (cpl <= 2) router_logits_kernel<ACT, 2><<<grid, 256, lds, s>>>(rp);
+    else if (cpl <= 4) router_logits_kernel<ACT, 4><<<grid, 256, lds, s>>>(rp);
+    else router_logits_kernel<ACT, 8><<<grid, 256, lds, s>>>(rp);
 }
 
 // d <= 2048 dense / 4096 at 8 bit / 8192 at 4 bit (8 chunks per lane).
@@ -636,11 +637,14 @@ extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream strea
     if (gated) rp.gate = to_desc(&L->shared_gate);
     rp.x = x; rp.eff_scale = L->eff_scale; rp.x_stride = x_stride; rp.tokens = T;
     rp.num_experts = E; rp.d = D; rp.logits = logits; rp.gate_logit = gate_logit;
-    { ProfScope ps(ctx, NVMAI_PROF_ROUTER, s); rc = run_router(ctx->act, rp, s); }
-    if (rc) return rc;
     SelectParams sp{logits, L->per_expert_scale, T, E, K, idx, wts};
     GroupParams gp{sp, (uint32_t)maxtok, has_shared ? 1 : 0, entries, n_entries, stats, pair_token, pair_id,
                    ctx->tickets};
+    // Two launches on purpose: one that also selects and groups in its last blocks needs a
+    // device-scope release (an L2 write-back on this multi-die part) from every one of its
+    // hundreds of producer blocks, and measured 18 us slower per step.
+    { ProfScope ps(ctx, NVMAI_PROF_ROUTER, s); rc = run_router(ctx->act, rp, s); }
+    if (rc) return rc;
     {
         ProfScope ps(ctx, NVMAI_PROF_GROUP, s);
         select_group_kernel<<<(T + 3) / 4, 256, (4 * E + 8 + pairs) * 4, s>>>(gp);

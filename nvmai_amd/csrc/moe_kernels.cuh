@@ -515,22 +515,22 @@ __device__ __forceinline__ void router_x_from_raw(const RouterParams& p, const u
     }
 }
 
-template <int ACT, int EPC>
-__device__ __forceinline__ void router_load_raw(const RouterParams& p, size_t x_off, uint32_t e0, uint4* raw) {
+// The block's token rows, as stored, into LDS ([nt][d] 16-bit): the eight rows of a block read
+// the same inputs, and reading them from LDS when they are used keeps only the weights in
+// registers.  Ends with a barrier.
+__device__ __forceinline__ void router_stage_x(const RouterParams& p, uint32_t t0, uint32_t nt, uint16_t* xl) {
     if (p.x_vec) {
-        const uint4* px = reinterpret_cast<const uint4*>((const uint16_t*)p.x + x_off + e0);
-#pragma unroll
-        for (int i = 0; i < EPC / 8; ++i) raw[i] = px[i];
-    } else {                       // unaligned rows (e.g. a padded hidden stride): element loads
-        const uint16_t* px = (const uint16_t*)p.x + x_off + e0;
-#pragma unroll
-        for (int i = 0; i < EPC / 8; ++i) {
-            raw[i].x = px[8 * i] | ((uint32_t)px[8 * i + 1] << 16);
-            raw[i].y = px[8 * i + 2] | ((uint32_t)px[8 * i + 3] << 16);
-            raw[i].z = px[8 * i + 4] | ((uint32_t)px[8 * i + 5] << 16);
-            raw[i].w = px[8 * i + 6] | ((uint32_t)px[8 * i + 7] << 16);
+        const uint32_t per_row = p.d / 8;
+        for (uint32_t i = threadIdx.x; i < nt * per_row; i += 256) {
+            const uint32_t t = i / per_row, c = i % per_row;
+            reinterpret_cast<uint4*>(xl)[i] =
+                *reinterpret_cast<const uint4*>((const uint16_t*)p.x + (size_t)(t0 + t) * p.x_stride + c * 8);
         }
+    } else {                       // unaligned rows (e.g. a padded hidden stride): element loads
+        for (uint32_t i = threadIdx.x; i < nt * p.d; i += 256)
+            xl[i] = ((const uint16_t*)p.x)[(size_t)(t0 + i / p.d) * p.x_stride + i % p.d];
     }
+    __syncthreads();
 }
 
 // One row against up to ROUTER_TOK tokens; hl = lane in the half-wave, CPL =
@@ -539,13 +539,13 @@ __device__ __forceinline__ void router_load_raw(const RouterParams& p, size_t x_
 // Per token the lane accumulates over its chunks in ascending order.
 template <int ACT, int KIND, int CPL>
 __device__ __forceinline__ void router_row_dots(const RouterParams& p, const RowsDesc& r, uint32_t row,
-                                                uint32_t t0, uint32_t nt, int hl, float* acc) {
+                                                const uint16_t* xl, uint32_t nt, int hl, float* acc) {
     constexpr int EPC = KIND == 16 ? 8 : (KIND == 8 ? 16 : 32);
     constexpr int XV = EPC / 8;
     const uint32_t chunks = p.d / EPC;
     const uint32_t groups = p.d / NVMAI_GROUP;
     const uint8_t* wr = (const uint8_t*)r.w + (size_t)row * ((size_t)p.d * KIND / 8);
-    uint4 wraw[CPL], xraw[ROUTER_TOK][CPL][XV];
+    uint4 wraw[CPL];
     uint16_t sraw[CPL], braw[CPL];
 #pragma unroll
     for (int i = 0; i < CPL; ++i) {
@@ -557,9 +557,6 @@ __device__ __forceinline__ void router_row_dots(const RouterParams& p, const Row
                 sraw[i] = r.s[(size_t)row * groups + g];
                 braw[i] = r.b[(size_t)row * groups + g];
             }
-#pragma unroll
-            for (int t = 0; t < ROUTER_TOK; ++t)
-                if ((uint32_t)t < nt) router_load_raw<ACT, EPC>(p, (size_t)(t0 + t) * p.x_stride, c * EPC, xraw[t][i]);
         }
     }
 #pragma unroll
@@ -579,7 +576,10 @@ __device__ __forceinline__ void router_row_dots(const RouterParams& p, const Row
         for (int t = 0; t < ROUTER_TOK; ++t) {
             if ((uint32_t)t >= nt) break;
             float xv[EPC];
-            router_x_from_raw<ACT, EPC>(p, xraw[t][i], c * EPC, xv);
+            uint4 xraw[XV];
+#pragma unroll
+            for (int v = 0; v < XV; ++v) xraw[v] = *reinterpret_cast<const uint4*>(xl + (size_t)t * p.d + c * EPC + 8 * v);
+            router_x_from_raw<ACT, EPC>(p, xraw, c * EPC, xv);
             if (KIND == 16) {
 #pragma unroll
                 for (int j = 0; j < EPC; ++j) acc[t] = fmaf(q[j], xv[j], acc[t]);
@@ -603,25 +603,28 @@ __device__ __forceinline__ void router_row_dots(const RouterParams& p, const Row
 
 template <int ACT, int CPL>
 __device__ __forceinline__ void router_row_any(const RouterParams& p, const RowsDesc& r, uint32_t row,
-                                               uint32_t t0, uint32_t nt, int hl, float* acc) {
-    if (r.kind == 16) router_row_dots<ACT, 16, CPL>(p, r, row, t0, nt, hl, acc);
-    else if (r.kind == 8) router_row_dots<ACT, 8, CPL>(p, r, row, t0, nt, hl, acc);
-    else router_row_dots<ACT, 4, CPL>(p, r, row, t0, nt, hl, acc);
+                                               const uint16_t* xl, uint32_t nt, int hl, float* acc) {
+    if (r.kind == 16) router_row_dots<ACT, 16, CPL>(p, r, row, xl, nt, hl, acc);
+    else if (r.kind == 8) router_row_dots<ACT, 8, CPL>(p, r, row, xl, nt, hl, acc);
+    else router_row_dots<ACT, 4, CPL>(p, r, row, xl, nt, hl, acc);
 }
 
 // Largest chunk count per lane over the router and gate rows must be <= CPL.
 template <int ACT, int CPL>
 __global__ __launch_bounds__(256) void router_logits_kernel(RouterParams p) {
+    extern __shared__ uint4 router_lds[];
+    const uint16_t* xl = reinterpret_cast<const uint16_t*>(router_lds);
     const int hw = threadIdx.x >> 5, hl = threadIdx.x & 31;
     const uint32_t row = blockIdx.x * 8 + hw;
     const uint32_t total_rows = p.num_experts + (p.gate.kind ? 1u : 0u);
-    if (row >= total_rows) return;                   // uniform per half-wave
-    const bool is_gate = row >= p.num_experts;
     const uint32_t t0 = blockIdx.y * ROUTER_TOK;
     const uint32_t nt = min((uint32_t)ROUTER_TOK, p.tokens - t0);
+    router_stage_x(p, t0, nt, reinterpret_cast<uint16_t*>(router_lds));
+    if (row >= total_rows) return;                   // uniform per half-wave
+    const bool is_gate = row >= p.num_experts;
     float acc[ROUTER_TOK];
-    if (is_gate) router_row_any<ACT, CPL>(p, p.gate, 0, t0, nt, hl, acc);
-    else router_row_any<ACT, CPL>(p, p.router, row, t0, nt, hl, acc);
+    if (is_gate) router_row_any<ACT, CPL>(p, p.gate, 0, xl, nt, hl, acc);
+    else router_row_any<ACT, CPL>(p, p.router, row, xl, nt, hl, acc);
     if (hl == 0) {
         for (uint32_t t = 0; t < nt; ++t) {
             if (is_gate) p.gate_logit[t0 + t] = acc[t];
@@ -654,7 +657,8 @@ __device__ void select_topk_wave(const SelectParams& p, uint32_t t, int lane) {
 #pragma unroll
     for (int j = 0; j < TOPK_MAX_PER_LANE; ++j) {
         const uint32_t e = lane + 64 * j;
-        val[j] = e < p.num_experts ? p.logits[(size_t)t * p.num_experts + e] : 0.0f;
+        const size_t at = (size_t)t * p.num_experts + e;
+        val[j] = e >= p.num_experts ? 0.0f : p.logits[at];
         taken[j] = e >= p.num_experts;
     }
     float my_score = 0.0f;
@@ -715,22 +719,11 @@ struct GroupParams {
     uint32_t* ticket;          // zero between launches; counts finished blocks
 };
 
-__global__ __launch_bounds__(256) void select_group_kernel(GroupParams p) {
-    extern __shared__ uint32_t lds[];
+// The work list from every token's routed experts; one block, after all indices are written.
+__device__ void build_work_list(const GroupParams& p, uint32_t* lds) {
     const uint32_t tokens = p.sel.tokens, top_k = p.sel.top_k, E = p.sel.num_experts;
     const uint32_t n_pairs = tokens * top_k;
     const uint32_t tid = threadIdx.x;
-    {
-        const uint32_t t = blockIdx.x * 4 + (tid >> 6);
-        if (t < tokens) select_topk_wave(p.sel, t, tid & 63);
-    }
-    __threadfence();                      // this block's indices are visible device-wide
-    __syncthreads();
-    if (tid == 0) lds[0] = atomicAdd(p.ticket, 1u);
-    __syncthreads();
-    if (lds[0] != gridDim.x - 1) return;  // uniform per block
-    __syncthreads();
-
     uint32_t* cnt = lds;                  // [E] pairs per expert
     uint32_t* start = lds + E;            // [E] first pair of the expert
     uint32_t* slotf = lds + 2 * E;        // [E] first full entry of the expert inside its class
@@ -785,6 +778,23 @@ __global__ __launch_bounds__(256) void select_group_kernel(GroupParams p) {
         if (p.stats) { p.stats[0] = total_ent; p.stats[1] = misc[5]; }
         *p.ticket = 0;                    // ready for the next launch
     }
+}
+
+__global__ __launch_bounds__(256) void select_group_kernel(GroupParams p) {
+    extern __shared__ uint32_t lds[];
+    const uint32_t tokens = p.sel.tokens;
+    const uint32_t tid = threadIdx.x;
+    {
+        const uint32_t t = blockIdx.x * 4 + (tid >> 6);
+        if (t < tokens) select_topk_wave(p.sel, t, tid & 63);
+    }
+    __threadfence();                      // this block's indices are visible device-wide
+    __syncthreads();
+    if (tid == 0) lds[0] = atomicAdd(p.ticket, 1u);
+    __syncthreads();
+    if (lds[0] != gridDim.x - 1) return;  // uniform per block
+    __syncthreads();
+    build_work_list(p, lds);
 }
 
 // Dense work list: `count` inputs through the expert in slot `slot`.
