@@ -647,7 +647,8 @@ extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream strea
     if (rc) return rc;
     {
         ProfScope ps(ctx, NVMAI_PROF_GROUP, s);
-        select_group_kernel<<<(T + 3) / 4, 256, (4 * E + 8 + pairs) * 4, s>>>(gp);
+        if (T <= 4) select_group_one_block_kernel<<<1, 256, (4 * E + 8 + pairs) * 4, s>>>(gp);
+        else select_group_kernel<<<(T + 3) / 4, 256, (4 * E + 8 + pairs) * 4, s>>>(gp);
     }
 
     RowsParams p{};

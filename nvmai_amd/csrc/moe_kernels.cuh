@@ -731,12 +731,12 @@ __device__ void build_work_list(const GroupParams& p, uint32_t* lds) {
     uint32_t* misc = lds + 4 * E;         // [0] pair cursor, [1..4] entries per class, [5] distinct
     uint32_t* rank = lds + 4 * E + 8;     // [n_pairs] rank of the pair inside its expert
     const volatile uint32_t* idx = p.sel.out_idx;   // written by other blocks: read past L1
-    for (uint32_t i = tid; i < 4 * E + 8; i += 256) lds[i] = 0;
+    for (uint32_t i = tid; i < 4 * E + 8; i += blockDim.x) lds[i] = 0;
     __syncthreads();
-    for (uint32_t i = tid; i < n_pairs; i += 256) rank[i] = atomicAdd(&cnt[idx[i]], 1u);
+    for (uint32_t i = tid; i < n_pairs; i += blockDim.x) rank[i] = atomicAdd(&cnt[idx[i]], 1u);
     __syncthreads();
     const uint32_t tpe = p.tok_per_entry;
-    for (uint32_t e = tid; e < E; e += 256) {
+    for (uint32_t e = tid; e < E; e += blockDim.x) {
         const uint32_t c = cnt[e];
         if (!c) continue;
         start[e] = atomicAdd(&misc[0], c);
@@ -751,7 +751,7 @@ __device__ void build_work_list(const GroupParams& p, uint32_t* lds) {
     uint32_t run = shared_ent;
     for (int c = MAX_TOK; c >= 1; --c) { base[c] = run; run += misc[c]; }
     const uint32_t total_ent = run;
-    for (uint32_t e = tid; e < E; e += 256) {
+    for (uint32_t e = tid; e < E; e += blockDim.x) {
         const uint32_t c = cnt[e];
         if (!c) continue;
         const uint32_t full = c / tpe, rem = c % tpe;
@@ -759,15 +759,15 @@ __device__ void build_work_list(const GroupParams& p, uint32_t* lds) {
             p.entries[base[tpe] + slotf[e] + j] = WorkEntry{e, start[e] + j * tpe, tpe, 0};
         if (rem) p.entries[base[rem] + slotr[e]] = WorkEntry{e, start[e] + full * tpe, rem, 0};
     }
-    for (uint32_t i = tid; i < n_pairs; i += 256) {
+    for (uint32_t i = tid; i < n_pairs; i += blockDim.x) {
         const uint32_t pos = start[idx[i]] + rank[i];
         p.pair_token[pos] = i / top_k;
         p.pair_id[pos] = i;
     }
     if (p.has_shared) {
-        for (uint32_t j = tid; j < shared_ent; j += 256)
+        for (uint32_t j = tid; j < shared_ent; j += blockDim.x)
             p.entries[j] = WorkEntry{NVMAI_SLOT_FLAG | 8u, n_pairs + j * tpe, min(tpe, tokens - j * tpe), 0};
-        for (uint32_t t = tid; t < tokens; t += 256) {
+        for (uint32_t t = tid; t < tokens; t += blockDim.x) {
             p.pair_token[n_pairs + t] = t;
             p.pair_id[n_pairs + t] = n_pairs + t;
         }
@@ -793,6 +793,17 @@ __global__ __launch_bounds__(256) void select_group_kernel(GroupParams p) {
     if (tid == 0) lds[0] = atomicAdd(p.ticket, 1u);
     __syncthreads();
     if (lds[0] != gridDim.x - 1) return;  // uniform per block
+    __syncthreads();
+    build_work_list(p, lds);
+}
+
+// The same for at most four tokens in ONE block: nothing crosses a block, so the device-scope
+// release of the multi-block kernel (an L2 write-back on this multi-die part) and its ticket
+// are not needed.
+__global__ __launch_bounds__(256) void select_group_one_block_kernel(GroupParams p) {
+    extern __shared__ uint32_t lds[];
+    const uint32_t t = threadIdx.x >> 6;
+    if (t < p.sel.tokens) select_topk_wave(p.sel, t, threadIdx.x & 63);
     __syncthreads();
     build_work_list(p, lds);
 }
