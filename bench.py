@@ -302,6 +302,16 @@ def run_attention(nv, ctx, torch, a):
     for tag, name in ((nv.PROF_ATTN_PARTIAL, "partial"), (nv.PROF_ATTN_COMBINE, "combine")):
         ms, n = ctx.profile_read(tag)
         kern[name] = ms / max(n, 1) * 1e3
+    # quantize-on-write of 8192-token blocks (the prefill-side use), K and V
+    srcq = torch.empty((8192, HKV * HD), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
+    nq = min(8192, ctx_len)
+    ctx.profile_enable(True)
+    for i in range(20):
+        quant.encode(srcq, HKV * HD, caches[0][i % 2].view(0, 0), nq, HKV * HD)
+    torch.cuda.synchronize()
+    ctx.profile_enable(False)
+    ms, n = ctx.profile_read(nv.PROF_KV_QUANT)
+    kern["kv_quantize_%d_tokens" % nq] = ms / max(n, 1) * 1e3
     stride = caches[0][0].stride
     cpu = None
     if not a.no_cpu:
@@ -331,6 +341,8 @@ def run_attention(nv, ctx, torch, a):
         "config": {"workload": "configs[3]: GQA decode attention, 16 query / 2 KV heads, head_dim 256, %d-bit KV "
                                "(group 64, fp16 scale/bias), context %d, batch %d" % (bits, ctx_len, B),
                    "frac_of_hbm_peak": round(step_b / dt / 1e9 / HBM_PEAK_GBPS, 4), "cache_sets_rotated": n_sets,
+                   "kv_quantize_gbps": round(nq * (HKV * HD * 2 + caches[0][0].stride) /
+                                             (kern["kv_quantize_%d_tokens" % nq] * 1e-6) / 1e9, 1),
                    "kernel_us": {k: round(v, 2) for k, v in kern.items()}},
         "roofline": {"kernel": "attn_partial_mfma_kernel", "bound": "hbm", "achieved": round(part, 2),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(part / HBM_PEAK_GBPS, 4),

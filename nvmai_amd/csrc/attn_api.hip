@@ -60,9 +60,21 @@ extern "C" int nvmai_hip_kv_quantize_affine(nvmai_hip_ctx* ctx, nvmai_stream str
     if (dst->bits == 16) return NVMAI_ERR_UNSUPPORTED;        // "KV quantizer requires 4-bit or 8-bit destination"
     if (token_count == 0) return NVMAI_ERR_INVALID_ARG;       // KVCacheQuantizer.swift:22
     KvFormat f{dst->bits, dst->stride, dst->value_bytes, element_count};
+    ProfScope ps(ctx, NVMAI_PROF_KV_QUANT, (hipStream_t)stream);
+    if (element_count % 64 == 0 && aligned16(source) && source_stride % 8 == 0 &&
+        (reinterpret_cast<uintptr_t>(dst->base) & 7u) == 0 && dst->stride % 8 == 0) {
+        const uint64_t threads = (uint64_t)token_count * (element_count / 8);
+        dim3 vgrid((uint32_t)((threads + 255) / 256));
+        hipStream_t s = (hipStream_t)stream;
+#define NVMAI_KVQ(ACT, BITS) \
+    kv_quantize_vec_kernel<ACT, BITS><<<vgrid, 256, 0, s>>>(source, source_stride, (uint8_t*)dst->base, f, token_count)
+        if (ctx->act == ACT_BF16) { if (dst->bits == 8) NVMAI_KVQ(ACT_BF16, 8); else NVMAI_KVQ(ACT_BF16, 4); }
+        else { if (dst->bits == 8) NVMAI_KVQ(ACT_FP16, 8); else NVMAI_KVQ(ACT_FP16, 4); }
+#undef NVMAI_KVQ
+        return launch_status();
+    }
     const uint64_t waves = (uint64_t)token_count * ((element_count + 63) / 64);
     dim3 grid((uint32_t)((waves + 3) / 4));
-    ProfScope ps(ctx, NVMAI_PROF_KV_QUANT, (hipStream_t)stream);
     if (ctx->act == ACT_BF16) kv_quantize_kernel<ACT_BF16><<<grid, 256, 0, (hipStream_t)stream>>>(source, source_stride, (uint8_t*)dst->base, f, token_count);
     else kv_quantize_kernel<ACT_FP16><<<grid, 256, 0, (hipStream_t)stream>>>(source, source_stride, (uint8_t*)dst->base, f, token_count);
     return launch_status();

@@ -55,6 +55,58 @@ __global__ __launch_bounds__(256) void kv_quantize_kernel(const void* src, uint3
     }
 }
 
+// The same arithmetic with eight consecutive elements per lane (one 16-byte load) and eight
+// lanes per group: for rows of whole groups with 16-byte aligned sources.  min / max do not
+// depend on the order of reduction, every other step is per element, so the codes and the fp16
+// scale / bias are the same bits as the one-element-per-lane kernel's.
+template <int ACT, int BITS>
+__global__ __launch_bounds__(256) void kv_quantize_vec_kernel(const void* src, uint32_t src_stride, uint8_t* dst,
+                                                             KvFormat f, uint32_t tokens) {
+    const uint32_t cpt = f.elements / 8;                          // 16-byte chunks per token
+    const uint64_t gid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (uint64_t)tokens * cpt) return;                    // whole groups of 8 lanes drop out together
+    const uint32_t token = gid / cpt, chunk = gid % cpt;
+    const uint4 raw = *reinterpret_cast<const uint4*>((const uint16_t*)src + (size_t)token * src_stride + chunk * 8);
+    float v[8];
+    act2_to_f32<ACT>(raw.x, v[0], v[1]); act2_to_f32<ACT>(raw.y, v[2], v[3]);
+    act2_to_f32<ACT>(raw.z, v[4], v[5]); act2_to_f32<ACT>(raw.w, v[6], v[7]);
+    float mn = v[0], mx = v[0];
+#pragma unroll
+    for (int j = 1; j < 8; ++j) { mn = fminf(mn, v[j]); mx = fmaxf(mx, v[j]); }
+#pragma unroll
+    for (int off = 4; off >= 1; off >>= 1) {
+        mn = fminf(mn, shfl_xor_f(mn, off));
+        mx = fmaxf(mx, shfl_xor_f(mx, off));
+    }
+    constexpr float levels = BITS == 4 ? 15.0f : 255.0f;
+    const float bias = mn;
+    const float scale = mx > mn ? __fdiv_rn(__fsub_rn(mx, mn), levels) : 0.0f;
+    const uint32_t groups = f.elements / 64, g = chunk / 8;
+    uint8_t* row = dst + (size_t)token * f.stride;
+    if ((chunk & 7u) == 0) {
+        reinterpret_cast<uint16_t*>(row + f.value_bytes)[g] = f32_to_f16(scale);
+        reinterpret_cast<uint16_t*>(row + f.value_bytes)[groups + g] = f32_to_f16(bias);
+    }
+    uint32_t code[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        float q = 0.0f;
+        if (scale > 0.0f) q = roundf(fminf(fmaxf(__fdiv_rn(__fsub_rn(v[j], bias), scale), 0.0f), levels));
+        code[j] = (uint32_t)q;
+    }
+    if (BITS == 8) {
+        uint2 o;
+        o.x = code[0] | code[1] << 8 | code[2] << 16 | code[3] << 24;
+        o.y = code[4] | code[5] << 8 | code[6] << 16 | code[7] << 24;
+        *reinterpret_cast<uint2*>(row + chunk * 8) = o;
+    } else {
+        uint32_t o = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o |= code[j] << (4 * j);
+        *reinterpret_cast<uint32_t*>(row + chunk * 4) = o;
+    }
+}
+
 // ---- partial RoPE (rope.metal:32-50, 80-102) ------------------------------------------------
 // data [tokens, heads, head_dim] in place; pair (i, rot/2 + i), angle = pos * theta^(-2i/rot).
 template <int ACT>
