@@ -157,7 +157,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # `--workload copy`); the summaries live under profiles/.  Keyed by (workload, bits, batch or
 # tokens); other configurations report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("decode", 8, 32): (180700 * 2.00 + 1336 * 1.00) * 1024,
+    ("decode", 8, 32): (180900 * 2.00 + 1339 * 1.00) * 1024,
     ("prefill", 4, 4096): (512200 * 2.00 + 32770 * 1.00) * 1024,
     ("attention", 8, 8, 131072): (596100 * 2.00 + 4385 * 1.00) * 1024,
 }
