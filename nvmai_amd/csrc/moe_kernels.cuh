@@ -198,15 +198,18 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
             const uint32_t r = row < p.rows ? row : p.rows - 1;
 #pragma unroll
             for (int c = 0; c < NCH; ++c) {
-                const uint32_t chunk = sl + c * SEG;
+                // a lane's chunks are neighbours (sl * NCH + c): with NCH * EPC <= 64 they share
+                // one quantization group, whose scale and bias are then loaded once
+                const uint32_t chunk = sl * NCH + c;
                 const uint32_t g = chunk * EPC / NVMAI_GROUP;
+                const bool fresh = c == 0 || NCH * EPC > NVMAI_GROUP;
                 st.qa[i][c] = *reinterpret_cast<const uint4*>(WA + (size_t)r * row_bytes + chunk * 16);
-                st.sa[i][c] = SA[(size_t)r * groups + g];
-                st.ba[i][c] = BA[(size_t)r * groups + g];
+                st.sa[i][c] = fresh ? SA[(size_t)r * groups + g] : st.sa[i][0];
+                st.ba[i][c] = fresh ? BA[(size_t)r * groups + g] : st.ba[i][0];
                 if (DUAL) {
                     st.qb[i][c] = *reinterpret_cast<const uint4*>(WB + (size_t)r * row_bytes + chunk * 16);
-                    st.sb[i][c] = SB[(size_t)r * groups + g];
-                    st.bb[i][c] = BB[(size_t)r * groups + g];
+                    st.sb[i][c] = fresh ? SB[(size_t)r * groups + g] : st.sb[i][0];
+                    st.bb[i][c] = fresh ? BB[(size_t)r * groups + g] : st.bb[i][0];
                 }
             }
         }
@@ -252,7 +255,7 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
 #pragma unroll
                 for (int j = 0; j < 8; ++j) v[t][j] *= sc;
                 const uint32_t chunk = e0 / EPC, piece = (e0 % EPC) / 8;
-                xw[t * WORDS_TOK + ((chunk / SEG) * H + piece) * SEG + (chunk % SEG)] = pack_inputs<BITS>(v[t]);
+                xw[t * WORDS_TOK + ((chunk % NCH) * H + piece) * SEG + (chunk / NCH)] = pack_inputs<BITS>(v[t]);
             }
         }
         __syncthreads();
@@ -287,7 +290,7 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
     #pragma unroll
                 for (int j = 0; j < 8; ++j) v[j] *= sc;
                 const uint32_t chunk = e0 / EPC, piece = (e0 % EPC) / 8;
-                xw[t * WORDS_TOK + ((chunk / SEG) * H + piece) * SEG + (chunk % SEG)] = pack_inputs<BITS>(v);
+                xw[t * WORDS_TOK + ((chunk % NCH) * H + piece) * SEG + (chunk / NCH)] = pack_inputs<BITS>(v);
             }
         }
         __syncthreads();
