@@ -370,27 +370,38 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
     uint32_t kraw[2][4][4];                                         // [tile][group][dwords]; 4-bit uses 2 dwords
     uint2 ksc[8], kbi[8];                                           // 4 fp16 each
     auto slot_pos = [&](uint32_t s0, int t) { return s0 + (t >> 2) * 16 + 4 * r + (t & 3); };
+    // Buffer loads: a scalar resource per cache, one 32-bit lane offset per row, the group and
+    // metadata offsets as immediates or scalars -- no 64-bit address arithmetic per load, and
+    // reads past the end of the sequence's rows return zero instead of faulting.
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(kbase), 0, (int)(p.seq_len * p.f.stride), 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(vbase), 0, (int)(p.seq_len * p.f.stride), 0x00020000);
     auto load_k = [&](uint32_t s0) {
 #pragma unroll
         for (int tile = 0; tile < 2; ++tile) {
             const uint32_t pos = min(s0 + tile * 16 + i, p1 - 1);
-            const uint8_t* row = kbase + (pos * p.f.stride + code_off);   // 32-bit offset from a uniform base
+            const uint32_t off = pos * p.f.stride + (BITS == 8 ? 16 : 8) * r;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 if (BITS == 8) {
-                    const uint4 w = *reinterpret_cast<const uint4*>(row + 64 * g + 16 * r);
+                    const u32x4_t w = __builtin_amdgcn_raw_buffer_load_b128(krsrc, off + 64 * g, code_off, 0);
                     kraw[tile][g][0] = w.x; kraw[tile][g][1] = w.y; kraw[tile][g][2] = w.z; kraw[tile][g][3] = w.w;
                 } else {
-                    const uint2 w = *reinterpret_cast<const uint2*>(row + 32 * g + 8 * r);
+                    const u32x2_t w = __builtin_amdgcn_raw_buffer_load_b64(krsrc, off + 32 * g, code_off, 0);
                     kraw[tile][g][0] = w.x; kraw[tile][g][1] = w.y;
                 }
             }
         }
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            const uint8_t* krow = kbase + min(slot_pos(s0, t), p1 - 1) * p.f.stride;
-            ksc[t] = *reinterpret_cast<const uint2*>(krow + meta_sc);
-            kbi[t] = *reinterpret_cast<const uint2*>(krow + meta_bi);
+            const uint32_t off = min(slot_pos(s0, t), p1 - 1) * p.f.stride;
+            const u32x2_t a = __builtin_amdgcn_raw_buffer_load_b64(krsrc, off, meta_sc, 0);
+            const u32x2_t c = __builtin_amdgcn_raw_buffer_load_b64(krsrc, off, meta_bi, 0);
+            ksc[t] = uint2{a.x, a.y};
+            kbi[t] = uint2{c.x, c.y};
         }
     };
     const uint32_t s_first = p0 + wave * ATTN_STEP;
@@ -410,13 +421,16 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
         uint32_t vraw[8][4];                                        // [token slot][group]: 4 codes (8-bit) / 4 nibbles
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            const uint8_t* vrow = vbase + tok[t] * p.f.stride;
-            vsc[t] = *reinterpret_cast<const uint2*>(vrow + meta_sc);
-            vbi[t] = *reinterpret_cast<const uint2*>(vrow + meta_bi);
+            const uint32_t off = tok[t] * p.f.stride;
+            const u32x2_t a = __builtin_amdgcn_raw_buffer_load_b64(vrsrc, off, meta_sc, 0);
+            const u32x2_t c = __builtin_amdgcn_raw_buffer_load_b64(vrsrc, off, meta_bi, 0);
+            vsc[t] = uint2{a.x, a.y};
+            vbi[t] = uint2{c.x, c.y};
+            const uint32_t voff = off + (BITS == 8 ? 4 : 2) * i;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                if (BITS == 8) vraw[t][g] = *reinterpret_cast<const uint32_t*>(vrow + code_off + 64 * g + 4 * i);
-                else vraw[t][g] = *reinterpret_cast<const uint16_t*>(vrow + code_off + 32 * g + 2 * i);
+                if (BITS == 8) vraw[t][g] = __builtin_amdgcn_raw_buffer_load_b32(vrsrc, voff + 64 * g, code_off, 0);
+                else vraw[t][g] = __builtin_amdgcn_raw_buffer_load_b16(vrsrc, voff + 32 * g, code_off, 0);
             }
         }
 

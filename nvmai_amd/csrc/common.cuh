@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 #define NVMAI_GROUP 64
 #define NVMAI_WAVE 64
@@ -135,6 +136,26 @@ __device__ __forceinline__ void unpack8(uint32_t w, float* q) {
     q[1] = (float)((w >> 8) & 0xFFu);
     q[2] = (float)((w >> 16) & 0xFFu);
     q[3] = (float)(w >> 24);
+}
+
+// unpack4 with the two nibble masks kept as they are written: two ANDs and a shift isolate
+// the codes as bytes, and each code is then one byte-to-float conversion.  (Left to itself the
+// compiler folds the masks into one bit-field extract per code, twice the instructions.)
+__device__ __forceinline__ void unpack4_bytes(uint32_t w, float* q) {
+    uint32_t lo = w & 0x0F0F0F0Fu;          // elements 0,2,4,6
+    uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;   // elements 1,3,5,7
+#if defined(__HIP_DEVICE_COMPILE__)          // the host pass parses this body too and knows no "v" registers
+    asm("" : "+v"(lo));
+    asm("" : "+v"(hi));
+#endif
+    q[0] = (float)(lo & 0xFFu);
+    q[1] = (float)(hi & 0xFFu);
+    q[2] = (float)((lo >> 8) & 0xFFu);
+    q[3] = (float)((hi >> 8) & 0xFFu);
+    q[4] = (float)((lo >> 16) & 0xFFu);
+    q[5] = (float)((hi >> 16) & 0xFFu);
+    q[6] = (float)(lo >> 24);
+    q[7] = (float)(hi >> 24);
 }
 
 // 8 codes of one dword at 4 bits -> floats, element j at bits 4j..4j+3

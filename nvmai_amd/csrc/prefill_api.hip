@@ -132,7 +132,7 @@ uint32_t gemm_grid(uint32_t max_mtiles, const GemmParams& g) {
 
 template <int ACT, int BITS, int NT>
 void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t max_mtiles, nvmai_hip_ctx* ctx, hipStream_t s) {
-    const size_t lds = (size_t)2 * GEMM_BM * GEMM_LDK * 2;     // 68 KB: above the 64 KB a launch gets unasked
+    const size_t lds = GEMM_LDS_BYTES;                          // above the 64 KB a launch gets unasked
     static bool raised = false;
     if (!raised) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, true, NT>),
@@ -175,6 +175,10 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
         return NVMAI_ERR_ALIGNMENT;
     const uint64_t n_pairs = (uint64_t)query_count * top_k;
     if (n_pairs >= (1u << 28)) return NVMAI_ERR_UNSUPPORTED;
+    // the GEMM kernel addresses every operand array with 32-bit byte offsets
+    if ((uint64_t)query_count * hidden_stride * 2 > 0xFFFFFFFFull || n_pairs * f * 2 > 0xFFFFFFFFull ||
+        (uint64_t)d * f * bits / 8 > 0xFFFFFFFFull)
+        return NVMAI_ERR_UNSUPPORTED;
     if (n_pairs == 0) return NVMAI_OK;
     const uint32_t max_mtiles = (uint32_t)(n_pairs / GEMM_BM) + (num_experts < n_pairs ? num_experts : (uint32_t)n_pairs);
     rc = ws_begin(ctx, ws_round((size_t)max_mtiles * sizeof(MTile)) + ws_round(64));
@@ -215,7 +219,7 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
 namespace {
 template <int ACT, int BITS, int NT>
 void launch_qmm(const GemmParams& g, uint32_t blocks, hipStream_t s) {
-    const size_t lds = (size_t)2 * GEMM_BM * GEMM_LDK * 2;
+    const size_t lds = GEMM_LDS_BYTES;
     static bool raised = false;
     if (!raised) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, false, NT>),
@@ -238,6 +242,9 @@ extern "C" int nvmai_hip_affine_qmm(nvmai_hip_ctx* ctx, nvmai_stream stream, con
         return NVMAI_ERR_ALIGNMENT;
     if (m == 0) return NVMAI_OK;
     if (m >= (1u << 28)) return NVMAI_ERR_UNSUPPORTED;
+    // the GEMM kernel addresses every operand array with 32-bit byte offsets
+    if ((uint64_t)m * x_stride * 2 > 0xFFFFFFFFull || (uint64_t)n * k * bits / 8 > 0xFFFFFFFFull)
+        return NVMAI_ERR_UNSUPPORTED;
     const uint32_t tiles = (m + GEMM_BM - 1) / GEMM_BM;
     int rc = ws_begin(ctx, ws_round((size_t)tiles * sizeof(MTile)) + ws_round(64) + ws_round((size_t)m * sizeof(PrefillPair)));
     if (rc) return rc;

@@ -336,14 +336,25 @@ __device__ __forceinline__ uint4 dequant8(const float* q, float s, float b) {
 // NT = 16-column tiles per wave (2 or 4): the block covers 32 NT gate/up columns (DUAL) or
 // 64 NT down columns.  NT = 4 reads each activation fragment from LDS once for four MFMAs and
 // halves the number of blocks that re-read an M tile's activations.
+//
+// Activations reach LDS without passing through registers (buffer_load ... lds, 16 bytes per
+// lane): a wave instruction fills 1 KB = four rows of 128 k, so rows are unpadded and the
+// 16-byte chunks of a row are XOR-swizzled instead (chunk c of row r sits in slot c ^ (r & 15)),
+// which the loading lane arranges by choosing which chunk it fetches.  Weight and scale loads
+// are buffer loads as well: one lane offset each, the tile / matrix / super-step part in a
+// scalar, so the loop carries two address registers for the weights instead of twenty-four.
+constexpr uint32_t GEMM_XBUF = GEMM_BM * GEMM_SK * 2;      // bytes of one activation stage
+// Dynamic LDS of a block: two activation stages and 4 KB of weight stage per wave in the main
+// loop, the padded output tile of the epilogue afterwards (at most 128 x 264 x 2 bytes).
+// 80 KB: two blocks share a compute unit's 160 KB.
+constexpr size_t GEMM_LDS_BYTES = 2 * GEMM_XBUF + 4 * 4096;
+
 template <int ACT, int BITS, bool DUAL, int NT>
 __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     constexpr int WQ = BITS == 8 ? 2 : 1;               // 16-byte loads per (column, super-step)
-    // register stages in flight (register budget: 128 accumulators at NT = 4)
-    constexpr int GEMM_XST = NT == 4 ? 1 : 2;
-    constexpr int GEMM_WST = (NT == 4 || BITS == 8) ? 2 : 4;
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
     extern __shared__ uint4 gemm_lds[];
-    uint16_t* xs = reinterpret_cast<uint16_t*>(gemm_lds);      // [2][128][LDK]
+    uint16_t* xs = reinterpret_cast<uint16_t*>(gemm_lds);      // [2][128][128], swizzled
     // Blocks are dealt to the eight XCDs round-robin.  A unit = up to GEMM_UNIT consecutive column
     // tiles of one M tile; its blocks run back to back on one XCD, so that the tile's activation
     // rows are fetched into that L2 once, and the units (M tiles sorted by size, then columns)
@@ -356,77 +367,106 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     if (tile_id >= *p.n_mtiles || nt >= p.n_tiles_n) return;
     const MTile mt = p.mtiles[tile_id];
     const uint8_t* blob = p.pool + (uint64_t)mt.expert * p.pool_stride;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lq = lane >> 4;
     const uint32_t groups = p.K / NVMAI_GROUP;
     constexpr uint32_t n_cols = DUAL ? 32 * NT : 64 * NT;   // output columns per block
     const uint32_t n0 = nt * n_cols;
-
-    // ---- activation staging: thread (row, half) moves 64 elements of a row per super-step
-    // Rows past the end of a short tile are neither loaded nor multiplied: their LDS rows keep
-    // whatever they held, which only reaches accumulator rows that are never stored.
-    const int srow = tid >> 1, shalf = tid & 1;
-    const bool x_live = (uint32_t)srow < mt.rows;
     const int live_mt = (int)((mt.rows + 15) >> 4);     // 16-row tiles that hold any row
-    const uint16_t* xrow;
-    {
-        const uint32_t m = (uint32_t)srow < mt.rows ? srow : 0;
-        const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
-        xrow = (const uint16_t*)p.x + (size_t)src * p.x_stride + shalf * 64;
-    }
-    // ---- weight columns of this lane: tile t -> DUAL {gate, up}[t & 1] of column
-    //      n0 + 8 NT wave + 16 (t / 2) + i, else column n0 + 16 NT wave + 16 t + i
-    const uint8_t* wrow[NT];
-    const uint16_t* srow_p[NT];
-    const uint16_t* brow_p[NT];
-    uint32_t col[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        col[t] = DUAL ? n0 + wave * (8 * NT) + (t >> 1) * 16 + li : n0 + wave * (16 * NT) + t * 16 + li;
-        const uint32_t r = col[t] < p.N ? col[t] : p.N - 1;
-        const bool second = DUAL && (t & 1);
-        wrow[t] = blob + (second ? p.wB : p.wA) + (size_t)r * (p.K * BITS / 8) + lq * (32 * BITS / 8);
-        srow_p[t] = reinterpret_cast<const uint16_t*>(blob + (second ? p.sB : p.sA)) + (size_t)r * groups + (lq >> 1);
-        brow_p[t] = reinterpret_cast<const uint16_t*>(blob + (second ? p.bB : p.bA)) + (size_t)r * groups + (lq >> 1);
-    }
-
     const uint32_t nss = (p.K + GEMM_SK - 1) / GEMM_SK;
     // A K that is an odd multiple of 64 leaves half of the last super-step empty: lanes whose k
     // range lies beyond K contribute zeros (zero activations, zero weights).
     const bool odd_tail = (p.K % GEMM_SK) != 0;
 
-    // NT = 4 has no registers to spare: the activations of the next super-step then travel in
-    // two halves of four 16-byte pieces through one half-sized stage.
-    constexpr bool XSPLIT = NT == 4;
-    constexpr int XP = XSPLIT ? 4 : 8;                  // 16-byte pieces per stage
-    struct XStage { uint4 v[XP]; };
-    struct WStage { uint4 w[NT][WQ]; uint16_t s[NT], b[NT]; };
-    XStage xst[GEMM_XST];
-    WStage wst[GEMM_WST];
-    auto load_x = [&](XStage& g, uint32_t ss, int part) {
-        const bool dead = !x_live || (odd_tail && ss == nss - 1 && shalf == 1);
+    // ---- activations.  A stage holds 128 rows x 128 k as eight 4 KB blocks, one per 16-row
+    // tile: [k quarter: 4][row: 16][position: 4] 16-byte chunks, chunk c of row r in quarter
+    // c / 4 at position (c % 4) ^ (r / 4).  An MFMA fragment read (16 rows, one chunk each) then
+    // touches every bank once, and a load instruction (64 lanes x 16 bytes = one quarter of one
+    // tile) needs only a lane-constant offset: wave w fills tiles 2 w and 2 w + 1, lane l row
+    // l / 4 of the tile, so two address registers serve all eight loads of a super-step.
+    // Tiles past the end of a short M tile are not loaded: their LDS rows keep whatever they
+    // held, which only reaches accumulator rows that are never stored.
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<void*>(p.x), 0, (int)0xFFFFFFFFu, 0x00020000);
+    uint32_t xoff[2];
 #pragma unroll
-        for (int j = 0; j < XP; ++j)
-            g.v[j] = dead ? uint4{0, 0, 0, 0}
-                          : *reinterpret_cast<const uint4*>(xrow + ss * GEMM_SK + (part * XP + j) * 8);
-    };
-    auto load_w = [&](WStage& g, uint32_t ss) {
-        const bool dead = odd_tail && ss == nss - 1 && lq >= 2;
-        const uint32_t sse = dead ? 0u : ss;                    // any valid address; the values are dropped
+    for (int g = 0; g < 2; ++g) {
+        const uint32_t row = (wave * 2 + g) * 16 + (lane >> 2);
+        const uint32_t m = row < mt.rows ? row : 0;     // a dead row of a live tile repeats row 0
+        const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
+        xoff[g] = src * (p.x_stride * 2u) + (uint32_t)((lane & 3) ^ (lane >> 4)) * 16u;
+    }
+    auto load_x = [&](uint32_t ss, int buf) {
+        uint8_t* stage = reinterpret_cast<uint8_t*>(xs) + buf * GEMM_XBUF;
+        const bool tail = odd_tail && ss == nss - 1;    // the second half of this super-step: zeros, not loads
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            const uint8_t* wp = wrow[t] + (size_t)sse * (GEMM_SK * BITS / 8);
+        for (int g = 0; g < 2; ++g) {
+            if ((wave * 2 + g) * 16 >= mt.rows) break;  // wave-uniform
 #pragma unroll
-            for (int h = 0; h < WQ; ++h) g.w[t][h] = *reinterpret_cast<const uint4*>(wp + 16 * h);
-            g.s[t] = dead ? (uint16_t)0 : srow_p[t][2 * sse];
-            g.b[t] = dead ? (uint16_t)0 : brow_p[t][2 * sse];
+            for (int i = 0; i < 4; ++i) {
+                uint8_t* dst = stage + (wave * 2 + g) * 4096 + i * 1024;
+                if (i >= 2 && tail) *reinterpret_cast<uint4*>(dst + lane * 16) = uint4{0, 0, 0, 0};
+                else __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (__attribute__((address_space(3))) void*)dst, 16, xoff[g],
+                                                              ss * (GEMM_SK * 2) + i * 64, 0, 0);
+            }
         }
     };
-    auto store_x = [&](const XStage& g, int buf, int part) {
-        if (!x_live) return;
-        uint16_t* xd = xs + (buf * GEMM_BM + srow) * GEMM_LDK + shalf * 64 + part * XP * 8;
+
+    // ---- weight columns of this lane: tile t -> DUAL {gate, up}[t & 1] of column
+    //      n0 + 8 NT wave + 16 (t / 2) + i, else column n0 + 16 NT wave + 16 t + i.
+    // Columns past N (a last block that sticks out) read zeros; they are never stored.
+    // One resource per array (codes, scales, biases of matrix A and, DUAL, of matrix B), bounded
+    // by the array's size: the arrays of a dense product need not lie in one allocation.
+    const uint32_t row_bytes = p.K * BITS / 8;
+    const uint32_t w_bytes = p.N * row_bytes, sb_bytes = p.N * groups * 2u;
+    auto rsrc_of = [&](int64_t off, uint32_t bytes) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(blob + off), 0, (int)bytes, 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t wrsA = rsrc_of(p.wA, w_bytes), wrsB = rsrc_of(DUAL ? p.wB : p.wA, w_bytes);
+    const __amdgpu_buffer_rsrc_t srsA = rsrc_of(p.sA, sb_bytes), srsB = rsrc_of(DUAL ? p.sB : p.sA, sb_bytes);
+    const __amdgpu_buffer_rsrc_t brsA = rsrc_of(p.bA, sb_bytes), brsB = rsrc_of(DUAL ? p.bB : p.bA, sb_bytes);
+    const uint32_t col0 = DUAL ? n0 + wave * (8 * NT) + li : n0 + wave * (16 * NT) + li;
+    const uint32_t wv = col0 * row_bytes + lq * (32 * BITS / 8);
+    const uint32_t sv = (col0 * groups + (lq >> 1)) * 2u;
+    uint32_t wso[NT], sso[NT];                          // scalar parts: the tile's first column
 #pragma unroll
-        for (int j = 0; j < XP; ++j) *reinterpret_cast<uint4*>(xd + j * 8) = g.v[j];
+    for (int t = 0; t < NT; ++t) {
+        const uint32_t dcol = DUAL ? (t >> 1) * 16 : t * 16;
+        wso[t] = dcol * row_bytes;
+        sso[t] = dcol * groups * 2u;
+    }
+    // The weights of the next super-step wait in a wave-private LDS stage (the lane's own 16
+    // bytes per tile, written by the load itself), so that only the super-step being multiplied
+    // occupies registers; its scales and biases wait in registers.
+    uint8_t* wlds = reinterpret_cast<uint8_t*>(xs) + 2 * GEMM_XBUF + wave * (NT * WQ * 1024);
+    uint4 wcur[NT][WQ];
+    uint16_t ns[NT], nb[NT];
+    auto issue_w = [&](uint32_t ss) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const uint32_t so = wso[t] + ss * (GEMM_SK * BITS / 8);
+#pragma unroll
+            for (int h = 0; h < WQ; ++h)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds((DUAL && (t & 1)) ? wrsB : wrsA, (__attribute__((address_space(3))) void*)(wlds + (t * WQ + h) * 1024),
+                                                         16, wv + 16 * h, so, 0, 0);
+            ns[t] = __builtin_amdgcn_raw_buffer_load_b16((DUAL && (t & 1)) ? srsB : srsA, sv, sso[t] + ss * 4u, 0);
+            nb[t] = __builtin_amdgcn_raw_buffer_load_b16((DUAL && (t & 1)) ? brsB : brsA, sv, sso[t] + ss * 4u, 0);
+        }
+    };
+    // After vmcnt(0): the stage moves into registers, scales and biases become floats.
+    auto take_w = [&](uint32_t ss, float* sc, float* bi) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int h = 0; h < WQ; ++h)
+                wcur[t][h] = *reinterpret_cast<const uint4*>(wlds + (t * WQ + h) * 1024 + lane * 16);
+        const bool dead = odd_tail && ss == nss - 1 && lq >= 2;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            sc[t] = dead ? 0.0f : bf16_to_f32(ns[t]);
+            bi[t] = dead ? 0.0f : bf16_to_f32(nb[t]);
+        }
     };
 
     fl4_t acc[8][NT];
@@ -435,67 +475,80 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[a][t] = fl4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
+    // The main loop is a flat pipeline over MFMA steps (four per super-step): while the matrix
+    // pipe works through step s, the vector pipe dequantizes the operand of step s + 1 into the
+    // other half of bf[], across super-step boundaries too.  MT = 16-row tiles multiplied
+    // (1, 2, 4 or 8, block-uniform): the body holds no branch, so that the LDS reads of the next
+    // row tile and the dequantization interleave with the MFMAs.
+    auto dequant_step = [&](const float* sc, const float* bi, int j, uint4* bfrag) {
 #pragma unroll
-    for (int j = 0; j < GEMM_WST - 1; ++j)
-        if ((uint32_t)j < nss) load_w(wst[j], j);
-    if (XSPLIT) {
-        load_x(xst[0], 0, 0);
-        store_x(xst[0], 0, 0);
-        load_x(xst[0], 0, 1);
-        store_x(xst[0], 0, 1);
-    } else {
-#pragma unroll
-        for (int j = 0; j < GEMM_XST; ++j)
-            if ((uint32_t)j < nss) load_x(xst[j], j, 0);
-        store_x(xst[0], 0, 0);
-    }
-    __syncthreads();
-    for (uint32_t ss0 = 0; ss0 < nss; ss0 += GEMM_WST) {
-#pragma unroll
-        for (int u = 0; u < GEMM_WST; ++u) {
-            const uint32_t ss = ss0 + u;
-            if (ss >= nss) break;
+        for (int t = 0; t < NT; ++t) {
+            float q[8];
+            if (BITS == 4) {
+                const uint4 w = wcur[t][0];
+                unpack4_bytes(j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w, q);
+            } else {
+                const uint4 w = wcur[t][BITS == 8 ? j >> 1 : 0];
+                unpack8((j & 1) ? w.z : w.x, q);
+                unpack8((j & 1) ? w.w : w.y, q + 4);
+            }
+            bfrag[t] = dequant8<ACT>(q, sc[t], bi[t]);
+        }
+    };
+    // LDS byte address of the lane's fragment of row tile 0, MFMA step 0, stage 0; step j: ^ 16 j
+    const uint32_t xa0 = lq * 1024 + li * 64 + (li >> 2) * 16;
+    auto run = [&](auto mtc) {
+        constexpr int MT = decltype(mtc)::value;
+        uint4 bf[2][NT];
+        float sc[NT], bi[NT];
+        load_x(0, 0);
+        issue_w(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0)
+        take_w(0, sc, bi);
+        __builtin_amdgcn_s_waitcnt(0xC07F);                     // lgkmcnt(0): the stage is read before it is refilled
+        if (nss > 1) issue_w(1);
+        dequant_step(sc, bi, 0, bf[0]);
+        __syncthreads();
+        for (uint32_t ss = 0; ss < nss; ++ss) {
             const int buf = ss & 1;
-            // xst[u % XST] held super-step ss, which reached LDS one iteration ago
-            if (ss + GEMM_XST < nss) load_x(xst[u % GEMM_XST], ss + GEMM_XST, 0);
-            if (ss + GEMM_WST - 1 < nss) load_w(wst[(u + GEMM_WST - 1) % GEMM_WST], ss + GEMM_WST - 1);
-            const WStage& g = wst[u];
-            float sc[NT], bi[NT];
-#pragma unroll
-            for (int t = 0; t < NT; ++t) { sc[t] = bf16_to_f32(g.s[t]); bi[t] = bf16_to_f32(g.b[t]); }
-            const uint16_t* xa = xs + (buf * GEMM_BM + li) * GEMM_LDK + lq * 32;
+            if (ss + 1 < nss) load_x(ss + 1, buf ^ 1);
+            const uint8_t* xb = reinterpret_cast<const uint8_t*>(xs) + buf * GEMM_XBUF;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                uint4 bfrag[NT];
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    float q[8];
-                    if (BITS == 4) {
-                        const uint4 w = g.w[t][0];
-                        unpack4(j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w, q);
-                    } else {
-                        const uint4 w = g.w[t][BITS == 8 ? j >> 1 : 0];
-                        unpack8((j & 1) ? w.z : w.x, q);
-                        unpack8((j & 1) ? w.w : w.y, q + 4);
-                    }
-                    bfrag[t] = dequant8<ACT>(q, sc[t], bi[t]);
+                if (j < 3) dequant_step(sc, bi, j + 1, bf[(j + 1) & 1]);
+                else if (ss + 1 < nss) {
+                    // everything in flight has landed: the next activations and weights in LDS,
+                    // the next scales in registers
+                    __builtin_amdgcn_s_waitcnt(0x0F70);
+                    take_w(ss + 1, sc, bi);
+                    __builtin_amdgcn_s_waitcnt(0xC07F);
+                    if (ss + 2 < nss) issue_w(ss + 2);
+                    dequant_step(sc, bi, 0, bf[0]);
                 }
 #pragma unroll
-                for (int a = 0; a < 8; ++a) {
-                    if (a >= live_mt) break;
-                    const uint4 afrag = *reinterpret_cast<const uint4*>(xa + a * 16 * GEMM_LDK + j * 8);
+                for (int a = 0; a < MT; ++a) {
+                    const uint4 afrag = *reinterpret_cast<const uint4*>(xb + (xa0 ^ (16u * j)) + a * 4096);
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) acc[a][t] = mfma_16x16x32<ACT>(afrag, bfrag[t], acc[a][t]);
+                    for (int t = 0; t < NT; ++t) acc[a][t] = mfma_16x16x32<ACT>(afrag, bf[j & 1][t], acc[a][t]);
                 }
-                if (XSPLIT && j == 1 && ss + 1 < nss) {         // first half lands, second half leaves
-                    store_x(xst[0], buf ^ 1, 0);
-                    load_x(xst[0], ss + 1, 1);
+                // Issue order of the step: fragment reads one row tile ahead of their MFMAs, the
+                // next operand's dequantization spread between the MFMAs.
+                constexpr int VPER = (NT * (BITS == 4 ? 23 : 21) + MT - 1) / MT;
+                __builtin_amdgcn_sched_group_barrier(0x100, MT > 1 ? 2 : 1, 0);
+#pragma unroll
+                for (int a = 0; a < MT; ++a) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, VPER, 0);
+                    if (a + 2 < MT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 }
             }
-            if (ss + 1 < nss) store_x(xst[(u + 1) % GEMM_XST], buf ^ 1, XSPLIT ? 1 : 0);
             __syncthreads();
         }
-    }
+    };
+    if (live_mt > 4) run(std::integral_constant<int, 8>{});
+    else if (live_mt > 2) run(std::integral_constant<int, 4>{});
+    else if (live_mt > 1) run(std::integral_constant<int, 2>{});
+    else run(std::integral_constant<int, 1>{});
 
     // ---- epilogue: lane holds column i of each tile, rows 16 a + 4 q .. +4.  The block's output
     // tile is rounded to 16 bits into LDS (the activation buffers are free after the last
