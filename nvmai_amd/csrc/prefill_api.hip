@@ -132,22 +132,13 @@ uint32_t gemm_grid(uint32_t max_mtiles, const GemmParams& g) {
 
 template <int ACT, int BITS, int NT>
 void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t max_mtiles, nvmai_hip_ctx* ctx, hipStream_t s) {
-    const size_t lds = GEMM_LDS_BYTES;                          // above the 64 KB a launch gets unasked
-    static bool raised = false;
-    if (!raised) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, true, NT>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, false, NT>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        raised = true;
-    }
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM1, s);
-        prefill_gemm_kernel<ACT, BITS, true, NT><<<gemm_grid(max_mtiles, g1), 256, lds, s>>>(g1);
+        prefill_gemm_kernel<ACT, BITS, true, NT><<<gemm_grid(max_mtiles, g1), 256, 0, s>>>(g1);
     }
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM2, s);
-        prefill_gemm_kernel<ACT, BITS, false, NT><<<gemm_grid(max_mtiles, g2), 256, lds, s>>>(g2);
+        prefill_gemm_kernel<ACT, BITS, false, NT><<<gemm_grid(max_mtiles, g2), 256, 0, s>>>(g2);
     }
 }
 
@@ -219,14 +210,7 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
 namespace {
 template <int ACT, int BITS, int NT>
 void launch_qmm(const GemmParams& g, uint32_t blocks, hipStream_t s) {
-    const size_t lds = GEMM_LDS_BYTES;
-    static bool raised = false;
-    if (!raised) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_gemm_kernel<ACT, BITS, false, NT>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        raised = true;
-    }
-    prefill_gemm_kernel<ACT, BITS, false, NT><<<blocks, 256, lds, s>>>(g);
+    prefill_gemm_kernel<ACT, BITS, false, NT><<<blocks, 256, 0, s>>>(g);
 }
 }  // namespace
 

@@ -338,23 +338,34 @@ __device__ __forceinline__ uint4 dequant8(const float* q, float s, float b) {
 // halves the number of blocks that re-read an M tile's activations.
 //
 // Activations reach LDS without passing through registers (buffer_load ... lds, 16 bytes per
-// lane): a wave instruction fills 1 KB = four rows of 128 k, so rows are unpadded and the
-// 16-byte chunks of a row are XOR-swizzled instead (chunk c of row r sits in slot c ^ (r & 15)),
-// which the loading lane arranges by choosing which chunk it fetches.  Weight and scale loads
-// are buffer loads as well: one lane offset each, the tile / matrix / super-step part in a
-// scalar, so the loop carries two address registers for the weights instead of twenty-four.
+// lane), the weights of the next super-step likewise.  Weight and scale loads are buffer loads:
+// one lane offset each, the tile / matrix / super-step part in a scalar, so the loop carries two
+// address registers for the weights instead of twenty-four.
+//
+// LDS of a block: two activation stages and 4 KB of weight stage per wave, 80 KB, so that two
+// blocks share a compute unit's 160 KB.  They are three separate arrays on purpose: the
+// compiler makes every LDS read wait for all LDS-bound loads in flight unless it can prove
+// that they touch different memory, and it can for different arrays.  With one buffer the
+// loads of the next stage would be waited for before the first fragment read of this one.
 constexpr uint32_t GEMM_XBUF = GEMM_BM * GEMM_SK * 2;      // bytes of one activation stage
-// Dynamic LDS of a block: two activation stages and 4 KB of weight stage per wave in the main
-// loop, the padded output tile of the epilogue afterwards (at most 128 x 264 x 2 bytes).
-// 80 KB: two blocks share a compute unit's 160 KB.
-constexpr size_t GEMM_LDS_BYTES = 2 * GEMM_XBUF + 4 * 4096;
+
+// Position swizzle of row r (0..15) of a 16-row tile whose rows are 64 bytes apart: the sixteen
+// 16-byte reads of a fragment (one per row, same chunk) fall into sixteen different 16-byte
+// bank groups of a 256-byte LDS line, and each half of them (rows 0..7, 8..15) into eight
+// different groups of a 128-byte line.
+__device__ __forceinline__ uint32_t gemm_row_swizzle(uint32_t r) { return ((r >> 1) & 3u) ^ (r >> 3); }
 
 template <int ACT, int BITS, bool DUAL, int NT>
 __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     constexpr int WQ = BITS == 8 ? 2 : 1;               // 16-byte loads per (column, super-step)
     typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-    extern __shared__ uint4 gemm_lds[];
-    uint16_t* xs = reinterpret_cast<uint16_t*>(gemm_lds);      // [2][128][128], swizzled
+    __shared__ __attribute__((aligned(16))) uint8_t xs0[GEMM_XBUF];
+    __shared__ __attribute__((aligned(16))) uint8_t xs1[GEMM_XBUF];
+    __shared__ __attribute__((aligned(16))) uint8_t ws[4 * 4096];
+    // Arrays that only load instructions write look never-written to the optimizer, which would
+    // then fold every read of them away: a store that never executes keeps them alive (the
+    // entry points reject K = 0).
+    if (p.K == 0) { xs1[threadIdx.x] = 0; ws[threadIdx.x] = 0; }
     // Blocks are dealt to the eight XCDs round-robin.  A unit = up to GEMM_UNIT consecutive column
     // tiles of one M tile; its blocks run back to back on one XCD, so that the tile's activation
     // rows are fetched into that L2 once, and the units (M tiles sorted by size, then columns)
@@ -381,7 +392,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
 
     // ---- activations.  A stage holds 128 rows x 128 k as eight 4 KB blocks, one per 16-row
     // tile: [k quarter: 4][row: 16][position: 4] 16-byte chunks, chunk c of row r in quarter
-    // c / 4 at position (c % 4) ^ (r / 4).  An MFMA fragment read (16 rows, one chunk each) then
+    // c / 4 at position (c % 4) ^ swizzle(r).  An MFMA fragment read (16 rows, one chunk each) then
     // touches every bank once, and a load instruction (64 lanes x 16 bytes = one quarter of one
     // tile) needs only a lane-constant offset: wave w fills tiles 2 w and 2 w + 1, lane l row
     // l / 4 of the tile, so two address registers serve all eight loads of a super-step.
@@ -395,10 +406,9 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         const uint32_t row = (wave * 2 + g) * 16 + (lane >> 2);
         const uint32_t m = row < mt.rows ? row : 0;     // a dead row of a live tile repeats row 0
         const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
-        xoff[g] = src * (p.x_stride * 2u) + (uint32_t)((lane & 3) ^ (lane >> 4)) * 16u;
+        xoff[g] = src * (p.x_stride * 2u) + (uint32_t)((lane & 3) ^ gemm_row_swizzle(lane >> 2)) * 16u;
     }
-    auto load_x = [&](uint32_t ss, int buf) {
-        uint8_t* stage = reinterpret_cast<uint8_t*>(xs) + buf * GEMM_XBUF;
+    auto load_x = [&](uint32_t ss, uint8_t* stage) {
         const bool tail = odd_tail && ss == nss - 1;    // the second half of this super-step: zeros, not loads
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
@@ -439,7 +449,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     // The weights of the next super-step wait in a wave-private LDS stage (the lane's own 16
     // bytes per tile, written by the load itself), so that only the super-step being multiplied
     // occupies registers; its scales and biases wait in registers.
-    uint8_t* wlds = reinterpret_cast<uint8_t*>(xs) + 2 * GEMM_XBUF + wave * (NT * WQ * 1024);
+    uint8_t* wlds = ws + wave * (NT * WQ * 1024);
     uint4 wcur[NT][WQ];
     uint16_t ns[NT], nb[NT];
     auto issue_w = [&](uint32_t ss) {
@@ -496,12 +506,12 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         }
     };
     // LDS byte address of the lane's fragment of row tile 0, MFMA step 0, stage 0; step j: ^ 16 j
-    const uint32_t xa0 = lq * 1024 + li * 64 + (li >> 2) * 16;
+    const uint32_t xa0 = lq * 1024 + li * 64 + gemm_row_swizzle(li) * 16;
     auto run = [&](auto mtc) {
         constexpr int MT = decltype(mtc)::value;
         uint4 bf[2][NT];
         float sc[NT], bi[NT];
-        load_x(0, 0);
+        load_x(0, xs0);
         issue_w(0);
         __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0)
         take_w(0, sc, bi);
@@ -509,10 +519,9 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         if (nss > 1) issue_w(1);
         dequant_step(sc, bi, 0, bf[0]);
         __syncthreads();
-        for (uint32_t ss = 0; ss < nss; ++ss) {
-            const int buf = ss & 1;
-            if (ss + 1 < nss) load_x(ss + 1, buf ^ 1);
-            const uint8_t* xb = reinterpret_cast<const uint8_t*>(xs) + buf * GEMM_XBUF;
+        // one super-step: multiplies stage `cur` while stage `nxt` fills
+        auto superstep = [&](uint32_t ss, const uint8_t* cur, uint8_t* nxt) {
+            if (ss + 1 < nss) load_x(ss + 1, nxt);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if (j < 3) dequant_step(sc, bi, j + 1, bf[(j + 1) & 1]);
@@ -527,7 +536,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
                 }
 #pragma unroll
                 for (int a = 0; a < MT; ++a) {
-                    const uint4 afrag = *reinterpret_cast<const uint4*>(xb + (xa0 ^ (16u * j)) + a * 4096);
+                    const uint4 afrag = *reinterpret_cast<const uint4*>(cur + (xa0 ^ (16u * j)) + a * 4096);
 #pragma unroll
                     for (int t = 0; t < NT; ++t) acc[a][t] = mfma_16x16x32<ACT>(afrag, bf[j & 1][t], acc[a][t]);
                 }
@@ -543,6 +552,10 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
                 }
             }
             __syncthreads();
+        };
+        for (uint32_t ss = 0; ss < nss; ss += 2) {
+            superstep(ss, xs0, xs1);
+            if (ss + 1 < nss) superstep(ss + 1, xs1, xs0);
         }
     };
     if (live_mt > 4) run(std::integral_constant<int, 8>{});
@@ -550,51 +563,59 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     else if (live_mt > 1) run(std::integral_constant<int, 2>{});
     else run(std::integral_constant<int, 1>{});
 
-    // ---- epilogue: lane holds column i of each tile, rows 16 a + 4 q .. +4.  The block's output
-    // tile is rounded to 16 bits into LDS (the activation buffers are free after the last
-    // barrier) and leaves in 16-byte pieces, whole rows of the tile at a time.
+    // ---- epilogue: lane holds column i of each tile, rows 16 a + 4 q .. +4.  The output tile
+    // is rounded to 16 bits into the first activation stage (free after the last barrier), AP
+    // row tiles at a time, and leaves in 16-byte pieces, whole rows of the tile at a time.
     constexpr int OC = n_cols;                          // columns of the block's tile
     constexpr int LDO = OC + 8;
-    uint16_t* os = xs;
-#pragma unroll
-    for (int a = 0; a < 8; ++a) {
-        if (a >= live_mt) break;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int m = a * 16 + lq * 4 + r;
-            if (DUAL) {
-#pragma unroll
-                for (int c = 0; c < NT / 2; ++c)
-                    os[m * LDO + wave * (8 * NT) + c * 16 + li] =
-                        f32_to_act<ACT>(silu_fast(acc[a][2 * c][r]) * acc[a][2 * c + 1][r]);
-            } else {
-#pragma unroll
-                for (int t = 0; t < NT; ++t) os[m * LDO + wave * (16 * NT) + t * 16 + li] = f32_to_act<ACT>(acc[a][t][r]);
-            }
-        }
-    }
-    __syncthreads();
+    constexpr int AP = OC >= 256 ? 2 : OC >= 128 ? 4 : 8;   // 16 AP rows of LDO elements fit in 32 KB
+    static_assert(16 * AP * LDO * 2 <= (int)GEMM_XBUF, "epilogue tile exceeds an activation stage");
+    uint16_t* os = reinterpret_cast<uint16_t*>(xs0);
     constexpr int PIECES = OC / 8;                      // 16-byte pieces per row
     constexpr int ROWS_PER_PASS = 256 / PIECES;
     const int piece = tid % PIECES, prow = tid / PIECES;
     uint16_t* out = (uint16_t*)p.out;
     const bool vec_ok = (p.out_stride % 8 == 0) && n0 + OC <= p.N;
-    for (uint32_t m = prow; m < mt.rows; m += ROWS_PER_PASS) {
-        size_t orow;
-        if (DUAL) orow = (size_t)(mt.row_start + m) * p.out_stride;
-        else {
-            const PrefillPair pr = p.pairs[mt.row_start + m];
-            orow = ((size_t)pr.token * p.top_k + pr.rank) * p.out_stride;
-        }
-        const uint4 v = *reinterpret_cast<const uint4*>(os + m * LDO + piece * 8);
-        const uint32_t c0 = n0 + piece * 8;
-        if (vec_ok) *reinterpret_cast<uint4*>(out + orow + c0) = v;
-        else {
-            const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
-                if (c0 + j < p.N) out[orow + c0 + j] = e[j];
+    for (int a0 = 0; a0 < 8; a0 += AP) {
+        if (a0 >= live_mt) break;                       // block-uniform
+#pragma unroll
+        for (int da = 0; da < AP; ++da) {
+            const int a = a0 + da;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = da * 16 + lq * 4 + r;
+                if (DUAL) {
+#pragma unroll
+                    for (int c = 0; c < NT / 2; ++c)
+                        os[m * LDO + wave * (8 * NT) + c * 16 + li] =
+                            f32_to_act<ACT>(silu_fast(acc[a][2 * c][r]) * acc[a][2 * c + 1][r]);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) os[m * LDO + wave * (16 * NT) + t * 16 + li] = f32_to_act<ACT>(acc[a][t][r]);
+                }
+            }
         }
+        __syncthreads();
+        const uint32_t m_end = min(mt.rows, (uint32_t)(a0 + AP) * 16u);
+        for (uint32_t m = a0 * 16 + prow; m < m_end; m += ROWS_PER_PASS) {
+            size_t orow;
+            if (DUAL) orow = (size_t)(mt.row_start + m) * p.out_stride;
+            else {
+                const PrefillPair pr = p.pairs[mt.row_start + m];
+                orow = ((size_t)pr.token * p.top_k + pr.rank) * p.out_stride;
+            }
+            const uint4 v = *reinterpret_cast<const uint4*>(os + (m - a0 * 16) * LDO + piece * 8);
+            const uint32_t c0 = n0 + piece * 8;
+            if (vec_ok) *reinterpret_cast<uint4*>(out + orow + c0) = v;
+            else {
+                const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (c0 + j < p.N) out[orow + c0 + j] = e[j];
+            }
+        }
+        if (a0 + AP < 8) __syncthreads();
     }
 }
 
