@@ -542,12 +542,17 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
                 }
                 // Issue order of the step: fragment reads one row tile ahead of their MFMAs, the
                 // next operand's dequantization spread between the MFMAs.
-                constexpr int VPER = (NT * (BITS == 4 ? 23 : 21) + MT - 1) / MT;
+                // An MFMA occupies the matrix pipe for four issue slots: three vector
+                // instructions of the same wave fit behind each one.
+                constexpr int VPER = ((BITS == 4 ? 23 : 21) + MT - 1) / MT;    // per MFMA
                 __builtin_amdgcn_sched_group_barrier(0x100, MT > 1 ? 2 : 1, 0);
 #pragma unroll
                 for (int a = 0; a < MT; ++a) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, NT, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, VPER, 0);
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, VPER, 0);
+                    }
                     if (a + 2 < MT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 }
             }
