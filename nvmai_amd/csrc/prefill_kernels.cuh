@@ -355,6 +355,9 @@ constexpr uint32_t GEMM_XBUF = GEMM_BM * GEMM_SK * 2;      // bytes of one activ
 // different groups of a 128-byte line.
 __device__ __forceinline__ uint32_t gemm_row_swizzle(uint32_t r) { return ((r >> 1) & 3u) ^ (r >> 3); }
 
+// s_waitcnt operand: at most n vector-memory loads still in flight, the other counters free.
+constexpr int gemm_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
+
 template <int ACT, int BITS, bool DUAL, int NT>
 __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     constexpr int WQ = BITS == 8 ? 2 : 1;               // 16-byte loads per (column, super-step)
@@ -409,16 +412,27 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         xoff[g] = src * (p.x_stride * 2u) + (uint32_t)((lane & 3) ^ gemm_row_swizzle(lane >> 2)) * 16u;
     }
     auto load_x = [&](uint32_t ss, uint8_t* stage) {
-        const bool tail = odd_tail && ss == nss - 1;    // the second half of this super-step: zeros, not loads
+        if (!(odd_tail && ss == nss - 1)) {
 #pragma unroll
-        for (int g = 0; g < 2; ++g) {
-            if ((wave * 2 + g) * 16 >= mt.rows) break;  // wave-uniform
+            for (int g = 0; g < 2; ++g) {
+                if ((wave * 2 + g) * 16 >= mt.rows) break;  // wave-uniform
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                uint8_t* dst = stage + (wave * 2 + g) * 4096 + i * 1024;
-                if (i >= 2 && tail) *reinterpret_cast<uint4*>(dst + lane * 16) = uint4{0, 0, 0, 0};
-                else __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (__attribute__((address_space(3))) void*)dst, 16, xoff[g],
-                                                              ss * (GEMM_SK * 2) + i * 64, 0, 0);
+                for (int i = 0; i < 4; ++i)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (__attribute__((address_space(3))) void*)(stage + (wave * 2 + g) * 4096 + i * 1024),
+                                                             16, xoff[g], ss * (GEMM_SK * 2) + i * 64, 0, 0);
+            }
+        } else {
+            // the last super-step of an odd K: its second half takes zeros, not loads
+#pragma unroll 1
+            for (int g = 0; g < 2; ++g) {
+                if ((wave * 2 + g) * 16 >= mt.rows) break;
+                uint8_t* dst = stage + (wave * 2 + g) * 4096;
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (__attribute__((address_space(3))) void*)(dst + i * 1024), 16, xoff[g],
+                                                             ss * (GEMM_SK * 2) + i * 64, 0, 0);
+                *reinterpret_cast<uint4*>(dst + 2048 + lane * 16) = uint4{0, 0, 0, 0};
+                *reinterpret_cast<uint4*>(dst + 3072 + lane * 16) = uint4{0, 0, 0, 0};
             }
         }
     };
@@ -434,24 +448,105 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(blob + off), 0, (int)bytes, 0x00020000);
     };
     const __amdgpu_buffer_rsrc_t wrsA = rsrc_of(p.wA, w_bytes), wrsB = rsrc_of(DUAL ? p.wB : p.wA, w_bytes);
-    const __amdgpu_buffer_rsrc_t srsA = rsrc_of(p.sA, sb_bytes), srsB = rsrc_of(DUAL ? p.sB : p.sA, sb_bytes);
-    const __amdgpu_buffer_rsrc_t brsA = rsrc_of(p.bA, sb_bytes), brsB = rsrc_of(DUAL ? p.bB : p.bA, sb_bytes);
     const uint32_t col0 = DUAL ? n0 + wave * (8 * NT) + li : n0 + wave * (16 * NT) + li;
     const uint32_t wv = col0 * row_bytes + lq * (32 * BITS / 8);
-    const uint32_t sv = (col0 * groups + (lq >> 1)) * 2u;
-    uint32_t wso[NT], sso[NT];                          // scalar parts: the tile's first column
+    uint32_t wso[NT];                                   // scalar part: the tile's first column
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        const uint32_t dcol = DUAL ? (t >> 1) * 16 : t * 16;
-        wso[t] = dcol * row_bytes;
-        sso[t] = dcol * groups * 2u;
+    for (int t = 0; t < NT; ++t) wso[t] = (DUAL ? (t >> 1) * 16 : t * 16) * row_bytes;
+
+    // ---- scales and biases.  A lane needs, per super-step and tile, the scale and bias of its
+    // column for the group its k range lies in.  Loaded lane by lane those are 2 NT two-byte
+    // loads per super-step whose 64 lanes hit 64 different cache lines each, and the address
+    // path, not the matrix pipe, sets the pace of the kernel.  Instead lane 16 t + c fetches for
+    // tile t, column c, the scales (and the biases) of CS super-steps at once: one wide load per
+    // array per CS super-steps.  A consumer lane takes its dword (two groups) from the fetching
+    // lane through the cross-lane network and keeps the half of its group.
+    // Rows of scales start on 2-byte boundaries when K / 64 is odd: the load starts at the dword
+    // below and takes one more, and a funnel shift lines the pairs up.
+    const int ld_t = lane >> 4;
+    const bool ld_on = NT == 4 || ld_t < NT;
+    const bool ld_second = DUAL && (ld_t & 1);
+    uint32_t so_lane, bo_lane;
+    {
+        uint32_t c = DUAL ? n0 + wave * (8 * NT) + (ld_t >> 1) * 16 + li : n0 + wave * (16 * NT) + ld_t * 16 + li;
+        c = min(c, p.N - 1) * groups * 2u;
+        so_lane = (DUAL ? (uint32_t)(ld_second ? p.sB : p.sA) : 0u) + c;
+        bo_lane = (DUAL ? (uint32_t)(ld_second ? p.bB : p.bA) : 0u) + c;
     }
+    // DUAL: gate and up arrays are reached from the expert's base (the lane picks the matrix)
+    const uint32_t blob_bytes = (uint32_t)(p.pool_stride < 0xFFFFFFFFull ? p.pool_stride : 0xFFFFFFFFull);
+    const __amdgpu_buffer_rsrc_t s_rs = DUAL ? rsrc_of(0, blob_bytes) : rsrc_of(p.sA, sb_bytes);
+    const __amdgpu_buffer_rsrc_t b_rs = DUAL ? rsrc_of(0, blob_bytes) : rsrc_of(p.bA, sb_bytes);
+    // raw: CS + 1 dwords from the dword at or below the row's chunk
+    auto load_sb = [&](auto csc, uint32_t* rs_, uint32_t* rb_, uint32_t chunk) {
+        constexpr int CS = decltype(csc)::value;
+        if (ld_on) {
+            if (CS == 1) {
+                typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+                const u32x2_t a = __builtin_amdgcn_raw_buffer_load_b64(s_rs, so_lane & ~3u, chunk * 4, 0);
+                const u32x2_t c = __builtin_amdgcn_raw_buffer_load_b64(b_rs, bo_lane & ~3u, chunk * 4, 0);
+                rs_[0] = a.x; rs_[1] = a.y;
+                rb_[0] = c.x; rb_[1] = c.y;
+            } else if (CS == 2) {
+                typedef uint32_t u32x3_t __attribute__((ext_vector_type(3)));
+                const u32x3_t a = __builtin_amdgcn_raw_buffer_load_b96(s_rs, so_lane & ~3u, chunk * (CS * 4), 0);
+                const u32x3_t c = __builtin_amdgcn_raw_buffer_load_b96(b_rs, bo_lane & ~3u, chunk * (CS * 4), 0);
+                rs_[0] = a.x; rs_[1] = a.y; rs_[2] = a.z;
+                rb_[0] = c.x; rb_[1] = c.y; rb_[2] = c.z;
+            } else {
+                const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(s_rs, so_lane & ~3u, chunk * (CS * 4), 0);
+                const u32x4_t c = __builtin_amdgcn_raw_buffer_load_b128(b_rs, bo_lane & ~3u, chunk * (CS * 4), 0);
+                rs_[0] = a.x; rs_[1] = a.y; rs_[2] = a.z; rs_[3] = a.w;
+                rb_[0] = c.x; rb_[1] = c.y; rb_[2] = c.z; rb_[3] = c.w;
+            }
+        }
+    };
+    // raw -> CS dwords, one per super-step of the chunk: (scale of group 2 ss, of group 2 ss + 1)
+    auto align_sb = [&](auto csc, const uint32_t* rs_, const uint32_t* rb_, uint32_t* cs_, uint32_t* cb_) {
+        constexpr int CS = decltype(csc)::value;
+#pragma unroll
+        for (int h = 0; h < CS; ++h) {
+            cs_[h] = __builtin_amdgcn_alignbit(rs_[h + 1], rs_[h], (so_lane & 2u) * 8u);
+            cb_[h] = __builtin_amdgcn_alignbit(rb_[h + 1], rb_[h], (bo_lane & 2u) * 8u);
+        }
+    };
+    // the fetching lanes' dwords of one super-step -> this lane's (scale, bias) per tile, packed:
+    // scale in the high half, bias in the low half.  The cross-lane reads carry the tile in their
+    // immediate offset, so one address register serves all of them.
+    const uint32_t bp_addr = 4u * li;
+    auto scales_from = [&](uint32_t s_dw, uint32_t b_dw, uint32_t ss, uint32_t* sb) {
+        const bool dead = odd_tail && ss == nss - 1 && lq >= 2;
+        uint32_t ds[4], db[4];
+#if defined(__HIP_DEVICE_COMPILE__)
+        if (NT == 4)
+            asm volatile("ds_bpermute_b32 %0, %8, %9\n\tds_bpermute_b32 %1, %8, %9 offset:64\n\t"
+                         "ds_bpermute_b32 %2, %8, %9 offset:128\n\tds_bpermute_b32 %3, %8, %9 offset:192\n\t"
+                         "ds_bpermute_b32 %4, %8, %10\n\tds_bpermute_b32 %5, %8, %10 offset:64\n\t"
+                         "ds_bpermute_b32 %6, %8, %10 offset:128\n\tds_bpermute_b32 %7, %8, %10 offset:192\n\t"
+                         "s_waitcnt lgkmcnt(0)"
+                         : "=&v"(ds[0]), "=&v"(ds[1]), "=&v"(ds[2]), "=&v"(ds[3]), "=&v"(db[0]), "=&v"(db[1]), "=&v"(db[2]), "=&v"(db[3])
+                         : "v"(bp_addr), "v"(s_dw), "v"(b_dw));
+        else
+            asm volatile("ds_bpermute_b32 %0, %4, %5\n\tds_bpermute_b32 %1, %4, %5 offset:64\n\t"
+                         "ds_bpermute_b32 %2, %4, %6\n\tds_bpermute_b32 %3, %4, %6 offset:64\n\t"
+                         "s_waitcnt lgkmcnt(0)"
+                         : "=&v"(ds[0]), "=&v"(ds[1]), "=&v"(db[0]), "=&v"(db[1])
+                         : "v"(bp_addr), "v"(s_dw), "v"(b_dw));
+#endif
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            // the group of this lane's k range is the low (lq < 2) or the high half of each dword
+            const uint32_t pk = (lq >> 1) ? __builtin_amdgcn_perm(ds[t], db[t], 0x07060302u)
+                                          : __builtin_amdgcn_perm(ds[t], db[t], 0x05040100u);
+            sb[t] = dead ? 0u : pk;
+        }
+    };
+
     // The weights of the next super-step wait in a wave-private LDS stage (the lane's own 16
     // bytes per tile, written by the load itself), so that only the super-step being multiplied
-    // occupies registers; its scales and biases wait in registers.
+    // occupies registers.
     uint8_t* wlds = ws + wave * (NT * WQ * 1024);
     uint4 wcur[NT][WQ];
-    uint16_t ns[NT], nb[NT];
     auto issue_w = [&](uint32_t ss) {
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
@@ -460,101 +555,165 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
             for (int h = 0; h < WQ; ++h)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds((DUAL && (t & 1)) ? wrsB : wrsA, (__attribute__((address_space(3))) void*)(wlds + (t * WQ + h) * 1024),
                                                          16, wv + 16 * h, so, 0, 0);
-            ns[t] = __builtin_amdgcn_raw_buffer_load_b16((DUAL && (t & 1)) ? srsB : srsA, sv, sso[t] + ss * 4u, 0);
-            nb[t] = __builtin_amdgcn_raw_buffer_load_b16((DUAL && (t & 1)) ? brsB : brsA, sv, sso[t] + ss * 4u, 0);
         }
     };
-    // After vmcnt(0): the stage moves into registers, scales and biases become floats.
-    auto take_w = [&](uint32_t ss, float* sc, float* bi) {
+    // After vmcnt(0): the stage moves into registers.
+    auto take_w = [&]() {
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
             for (int h = 0; h < WQ; ++h)
                 wcur[t][h] = *reinterpret_cast<const uint4*>(wlds + (t * WQ + h) * 1024 + lane * 16);
-        const bool dead = odd_tail && ss == nss - 1 && lq >= 2;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            sc[t] = dead ? 0.0f : bf16_to_f32(ns[t]);
-            bi[t] = dead ? 0.0f : bf16_to_f32(nb[t]);
-        }
     };
-
-    fl4_t acc[8][NT];
-#pragma unroll
-    for (int a = 0; a < 8; ++a)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[a][t] = fl4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
     // The main loop is a flat pipeline over MFMA steps (four per super-step): while the matrix
     // pipe works through step s, the vector pipe dequantizes the operand of step s + 1 into the
     // other half of bf[], across super-step boundaries too.  MT = 16-row tiles multiplied
     // (1, 2, 4 or 8, block-uniform): the body holds no branch, so that the LDS reads of the next
     // row tile and the dequantization interleave with the MFMAs.
-    auto dequant_step = [&](const float* sc, const float* bi, int j, uint4* bfrag) {
+    auto dequant_step = [&](const uint4 (*w4)[WQ], const uint32_t* sb, int j, uint4* bfrag) {
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             float q[8];
             if (BITS == 4) {
-                const uint4 w = wcur[t][0];
+                const uint4 w = w4[t][0];
                 unpack4_bytes(j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w, q);
             } else {
-                const uint4 w = wcur[t][BITS == 8 ? j >> 1 : 0];
+                const uint4 w = w4[t][BITS == 8 ? j >> 1 : 0];
                 unpack8((j & 1) ? w.z : w.x, q);
                 unpack8((j & 1) ? w.w : w.y, q + 4);
             }
-            bfrag[t] = dequant8<ACT>(q, sc[t], bi[t]);
+            bfrag[t] = dequant8<ACT>(q, __builtin_bit_cast(float, sb[t] & 0xFFFF0000u), __builtin_bit_cast(float, sb[t] << 16));
         }
     };
     // LDS byte address of the lane's fragment of row tile 0, MFMA step 0, stage 0; step j: ^ 16 j
     const uint32_t xa0 = lq * 1024 + li * 64 + gemm_row_swizzle(li) * 16;
-    auto run = [&](auto mtc) {
+    // MFMAs of step j over MT row tiles of stage `cur`, and the issue order of the step: fragment
+    // reads one row tile ahead of their MFMAs, the next operand's dequantization (already in the
+    // instruction stream) spread between the MFMAs.  An MFMA occupies the matrix pipe for four
+    // issue slots: three vector instructions of the same wave fit behind each one.
+    auto mfma_step = [&](auto mtc, fl4_t (*acc)[NT], const uint8_t* cur, int j, const uint4* bfrag) {
         constexpr int MT = decltype(mtc)::value;
+#pragma unroll
+        for (int a = 0; a < MT; ++a) {
+            const uint4 afrag = *reinterpret_cast<const uint4*>(cur + (xa0 ^ (16u * j)) + a * 4096);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[a][t] = mfma_16x16x32<ACT>(afrag, bfrag[t], acc[a][t]);
+        }
+        constexpr int VPER = ((BITS == 4 ? 23 : 21) + MT - 1) / MT;    // per MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, MT > 1 ? 2 : 1, 0);
+#pragma unroll
+        for (int a = 0; a < MT; ++a) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, VPER, 0);
+            }
+            if (a + 2 < MT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    };
+
+    // ---- epilogue: lane holds column i of each tile, rows 16 a + 4 q .. +4.  The output tile
+    // is rounded to 16 bits into the first activation stage (free after the last barrier), AP
+    // row tiles at a time, and leaves in 16-byte pieces, whole rows of the tile at a time.
+    auto epilogue = [&](auto mtc, fl4_t (*acc)[NT]) {
+        constexpr int MT = decltype(mtc)::value;
+        constexpr int OC = n_cols;                          // columns of the block's tile
+        constexpr int LDO = OC + 8;
+        constexpr int AP0 = OC >= 256 ? 2 : OC >= 128 ? 4 : 8;  // 16 AP rows of LDO elements fit in 32 KB
+        constexpr int AP = AP0 < MT ? AP0 : MT;
+        static_assert(16 * AP * LDO * 2 <= (int)GEMM_XBUF, "epilogue tile exceeds an activation stage");
+        uint16_t* os = reinterpret_cast<uint16_t*>(xs0);
+        constexpr int PIECES = OC / 8;                      // 16-byte pieces per row
+        constexpr int ROWS_PER_PASS = 256 / PIECES;
+        const int piece = tid % PIECES, prow = tid / PIECES;
+        uint16_t* out = (uint16_t*)p.out;
+        const bool vec_ok = (p.out_stride % 8 == 0) && n0 + OC <= p.N;
+#pragma unroll
+        for (int a0 = 0; a0 < MT; a0 += AP) {
+            if (a0 >= live_mt) break;                       // block-uniform
+#pragma unroll
+            for (int da = 0; da < AP; ++da) {
+                const int a = a0 + da;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int m = da * 16 + lq * 4 + r;
+                    if (DUAL) {
+#pragma unroll
+                        for (int c = 0; c < NT / 2; ++c)
+                            os[m * LDO + wave * (8 * NT) + c * 16 + li] =
+                                f32_to_act<ACT>(silu_fast(acc[a][2 * c][r]) * acc[a][2 * c + 1][r]);
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < NT; ++t) os[m * LDO + wave * (16 * NT) + t * 16 + li] = f32_to_act<ACT>(acc[a][t][r]);
+                    }
+                }
+            }
+            __syncthreads();
+            const uint32_t m_end = min(mt.rows, (uint32_t)(a0 + AP) * 16u);
+            for (uint32_t m = a0 * 16 + prow; m < m_end; m += ROWS_PER_PASS) {
+                size_t orow;
+                if (DUAL) orow = (size_t)(mt.row_start + m) * p.out_stride;
+                else {
+                    const PrefillPair pr = p.pairs[mt.row_start + m];
+                    orow = ((size_t)pr.token * p.top_k + pr.rank) * p.out_stride;
+                }
+                const uint4 v = *reinterpret_cast<const uint4*>(os + (m - a0 * 16) * LDO + piece * 8);
+                const uint32_t c0 = n0 + piece * 8;
+                if (vec_ok) *reinterpret_cast<uint4*>(out + orow + c0) = v;
+                else {
+                    const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (c0 + j < p.N) out[orow + c0 + j] = e[j];
+                }
+            }
+            if (a0 + AP < MT) __syncthreads();
+        }
+    };
+
+    // ---- 3 to 8 row tiles (MT = 4 or 8): 128 accumulators leave room for one weight stage in
+    // registers; the next one waits in the wave's LDS stage, two activation stages alternate.
+    auto run_full = [&](auto mtc) {
+        constexpr int MT = decltype(mtc)::value;
+        fl4_t acc[MT][NT];
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[a][t] = fl4_t{0.0f, 0.0f, 0.0f, 0.0f};
         uint4 bf[2][NT];
-        float sc[NT], bi[NT];
+        uint32_t sb[NT];
+        const std::integral_constant<int, 1> cs1{};         // scales: fetched per super-step, one ahead
+        uint32_t rs_[2], rb_[2], cs_[1], cb_[1];            // next super-step's as loaded; lined up on use
+        load_sb(cs1, rs_, rb_, 0);
         load_x(0, xs0);
         issue_w(0);
         __builtin_amdgcn_s_waitcnt(0x0F70);                     // vmcnt(0)
-        take_w(0, sc, bi);
-        __builtin_amdgcn_s_waitcnt(0xC07F);                     // lgkmcnt(0): the stage is read before it is refilled
+        align_sb(cs1, rs_, rb_, cs_, cb_);
+        if (nss > 1) load_sb(cs1, rs_, rb_, 1);
+        take_w();
+        scales_from(cs_[0], cb_[0], 0, sb);
         if (nss > 1) issue_w(1);
-        dequant_step(sc, bi, 0, bf[0]);
+        dequant_step(wcur, sb, 0, bf[0]);
         __syncthreads();
         // one super-step: multiplies stage `cur` while stage `nxt` fills
         auto superstep = [&](uint32_t ss, const uint8_t* cur, uint8_t* nxt) {
             if (ss + 1 < nss) load_x(ss + 1, nxt);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                if (j < 3) dequant_step(sc, bi, j + 1, bf[(j + 1) & 1]);
+                if (j < 3) dequant_step(wcur, sb, j + 1, bf[(j + 1) & 1]);
                 else if (ss + 1 < nss) {
                     // everything in flight has landed: the next activations and weights in LDS,
                     // the next scales in registers
                     __builtin_amdgcn_s_waitcnt(0x0F70);
-                    take_w(ss + 1, sc, bi);
-                    __builtin_amdgcn_s_waitcnt(0xC07F);
+                    take_w();
+                    align_sb(cs1, rs_, rb_, cs_, cb_);
+                    if (ss + 2 < nss) load_sb(cs1, rs_, rb_, ss + 2);
+                    scales_from(cs_[0], cb_[0], ss + 1, sb);    // ends with lgkmcnt(0): the stage is read before it is refilled
                     if (ss + 2 < nss) issue_w(ss + 2);
-                    dequant_step(sc, bi, 0, bf[0]);
+                    dequant_step(wcur, sb, 0, bf[0]);
                 }
-#pragma unroll
-                for (int a = 0; a < MT; ++a) {
-                    const uint4 afrag = *reinterpret_cast<const uint4*>(cur + (xa0 ^ (16u * j)) + a * 4096);
-#pragma unroll
-                    for (int t = 0; t < NT; ++t) acc[a][t] = mfma_16x16x32<ACT>(afrag, bf[j & 1][t], acc[a][t]);
-                }
-                // Issue order of the step: fragment reads one row tile ahead of their MFMAs, the
-                // next operand's dequantization spread between the MFMAs.
-                // An MFMA occupies the matrix pipe for four issue slots: three vector
-                // instructions of the same wave fit behind each one.
-                constexpr int VPER = ((BITS == 4 ? 23 : 21) + MT - 1) / MT;    // per MFMA
-                __builtin_amdgcn_sched_group_barrier(0x100, MT > 1 ? 2 : 1, 0);
-#pragma unroll
-                for (int a = 0; a < MT; ++a) {
-#pragma unroll
-                    for (int t = 0; t < NT; ++t) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x002, VPER, 0);
-                    }
-                    if (a + 2 < MT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                }
+                mfma_step(mtc, acc, cur, j, bf[j & 1]);
             }
             __syncthreads();
         };
@@ -562,66 +721,104 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
             superstep(ss, xs0, xs1);
             if (ss + 1 < nss) superstep(ss + 1, xs1, xs0);
         }
+        epilogue(mtc, acc);
     };
-    if (live_mt > 4) run(std::integral_constant<int, 8>{});
-    else if (live_mt > 2) run(std::integral_constant<int, 4>{});
-    else if (live_mt > 1) run(std::integral_constant<int, 2>{});
-    else run(std::integral_constant<int, 1>{});
 
-    // ---- epilogue: lane holds column i of each tile, rows 16 a + 4 q .. +4.  The output tile
-    // is rounded to 16 bits into the first activation stage (free after the last barrier), AP
-    // row tiles at a time, and leaves in 16-byte pieces, whole rows of the tile at a time.
-    constexpr int OC = n_cols;                          // columns of the block's tile
-    constexpr int LDO = OC + 8;
-    constexpr int AP = OC >= 256 ? 2 : OC >= 128 ? 4 : 8;   // 16 AP rows of LDO elements fit in 32 KB
-    static_assert(16 * AP * LDO * 2 <= (int)GEMM_XBUF, "epilogue tile exceeds an activation stage");
-    uint16_t* os = reinterpret_cast<uint16_t*>(xs0);
-    constexpr int PIECES = OC / 8;                      // 16-byte pieces per row
-    constexpr int ROWS_PER_PASS = 256 / PIECES;
-    const int piece = tid % PIECES, prow = tid / PIECES;
-    uint16_t* out = (uint16_t*)p.out;
-    const bool vec_ok = (p.out_stride % 8 == 0) && n0 + OC <= p.N;
+    // ---- short tiles (1 or 2 row tiles).  Little arithmetic per byte of weights: what
+    // counts is how much is in flight.  The few accumulators leave registers for a ring of three
+    // weight stages (loaded two super-steps ahead), and the three LDS arrays serve as a ring of
+    // three activation stages of MT tiles each.  Every wave issues the same MT activation loads
+    // per super-step: instruction q = MT wave + e fills quarter q % 4 of tile q / 4.
+    auto run_short = [&](auto mtc) {
+        constexpr int MT = decltype(mtc)::value;
+        fl4_t acc[MT][NT];
 #pragma unroll
-    for (int a0 = 0; a0 < 8; a0 += AP) {
-        if (a0 >= live_mt) break;                       // block-uniform
+        for (int a = 0; a < MT; ++a)
 #pragma unroll
-        for (int da = 0; da < AP; ++da) {
-            const int a = a0 + da;
+            for (int t = 0; t < NT; ++t) acc[a][t] = fl4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        uint32_t xo;                                        // the lane's row of the wave's tile
+        {
+            const uint32_t row = ((wave * MT) >> 2) * 16 + (lane >> 2);
+            const uint32_t m = row < mt.rows ? row : 0;
+            const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
+            xo = src * (p.x_stride * 2u) + (uint32_t)((lane & 3) ^ gemm_row_swizzle(lane >> 2)) * 16u;
+        }
+        auto load_xs = [&](uint32_t ss, uint8_t* stage) {
+            const bool tail = odd_tail && ss == nss - 1;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int m = da * 16 + lq * 4 + r;
-                if (DUAL) {
+            for (int e = 0; e < MT; ++e) {
+                const uint32_t q = wave * MT + e;
+                uint8_t* dst = stage + (q >> 2) * 4096 + (q & 3) * 1024;
+                if (tail && (q & 3) >= 2) *reinterpret_cast<uint4*>(dst + lane * 16) = uint4{0, 0, 0, 0};
+                else __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (__attribute__((address_space(3))) void*)dst, 16, xo,
+                                                              ss * (GEMM_SK * 2) + (q & 3) * 64, 0, 0);
+            }
+        };
+        struct WReg { uint4 w[NT][WQ]; };
+        WReg wr[3];
+        auto load_wr = [&](WReg& g, uint32_t ss) {
 #pragma unroll
-                    for (int c = 0; c < NT / 2; ++c)
-                        os[m * LDO + wave * (8 * NT) + c * 16 + li] =
-                            f32_to_act<ACT>(silu_fast(acc[a][2 * c][r]) * acc[a][2 * c + 1][r]);
-                } else {
+            for (int t = 0; t < NT; ++t) {
+                const uint32_t so = wso[t] + ss * (GEMM_SK * BITS / 8);
 #pragma unroll
-                    for (int t = 0; t < NT; ++t) os[m * LDO + wave * (16 * NT) + t * 16 + li] = f32_to_act<ACT>(acc[a][t][r]);
+                for (int h = 0; h < WQ; ++h) {
+                    const u32x4_t w = __builtin_amdgcn_raw_buffer_load_b128((DUAL && (t & 1)) ? wrsB : wrsA, wv + 16 * h, so, 0);
+                    g.w[t][h] = uint4{w.x, w.y, w.z, w.w};
                 }
             }
-        }
+        };
+        constexpr int LW = NT * WQ;                         // weight loads of a super-step
+        uint4 bf[2][NT];
+        uint32_t sb[NT];
+        const std::integral_constant<int, 3> cs3{};         // scales: chunks of three super-steps
+        uint32_t rs_[4], rb_[4], cs_[3], cb_[3];            // next chunk as loaded, this chunk lined up
+        load_sb(cs3, rs_, rb_, 0);
+        load_xs(0, xs0);
+        load_wr(wr[0], 0);
+        if (nss > 1) { load_xs(1, xs1); load_wr(wr[1], 1); }
+        align_sb(cs3, rs_, rb_, cs_, cb_);
+        if (nss > 3) load_sb(cs3, rs_, rb_, 1);
+        scales_from(cs_[0], cb_[0], 0, sb);
+        dequant_step(wr[0].w, sb, 0, bf[0]);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
-        const uint32_t m_end = min(mt.rows, (uint32_t)(a0 + AP) * 16u);
-        for (uint32_t m = a0 * 16 + prow; m < m_end; m += ROWS_PER_PASS) {
-            size_t orow;
-            if (DUAL) orow = (size_t)(mt.row_start + m) * p.out_stride;
-            else {
-                const PrefillPair pr = p.pairs[mt.row_start + m];
-                orow = ((size_t)pr.token * p.top_k + pr.rank) * p.out_stride;
-            }
-            const uint4 v = *reinterpret_cast<const uint4*>(os + (m - a0 * 16) * LDO + piece * 8);
-            const uint32_t c0 = n0 + piece * 8;
-            if (vec_ok) *reinterpret_cast<uint4*>(out + orow + c0) = v;
-            else {
-                const uint16_t* e = reinterpret_cast<const uint16_t*>(&v);
+        // one super-step (U = its place in its chunk): multiplies stage `cur` from weights `wc`;
+        // stage `fill` and weights `wf` take what is needed two super-steps on; `wn` are the
+        // weights of the next super-step
+        auto superstep = [&](auto uc, uint32_t ss, const uint8_t* cur, uint8_t* fill, const WReg& wc, const WReg& wn, WReg& wf) {
+            constexpr int U = decltype(uc)::value;
+            if (ss + 2 < nss) { load_xs(ss + 2, fill); load_wr(wf, ss + 2); }
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (c0 + j < p.N) out[orow + c0 + j] = e[j];
+            for (int j = 0; j < 4; ++j) {
+                if (j < 3) dequant_step(wc.w, sb, j + 1, bf[(j + 1) & 1]);
+                else if (ss + 1 < nss) {
+                    if (U == 2) {
+                        align_sb(cs3, rs_, rb_, cs_, cb_);
+                        if (ss + 4 < nss) load_sb(cs3, rs_, rb_, (ss + 4) / 3);
+                    }
+                    scales_from(cs_[(U + 1) % 3], cb_[(U + 1) % 3], ss + 1, sb);
+                    dequant_step(wn.w, sb, 0, bf[0]);
+                }
+                mfma_step(mtc, acc, cur, j, bf[j & 1]);
             }
+            // The next activation stage was requested a super-step ago; at least the MT + LW
+            // requests from the start of this super-step are younger.  Near the end, or where a
+            // stage took zeros instead of loads, fewer were issued and more is waited for.
+            if (ss + 2 < nss && !(odd_tail && ss + 2 == nss - 1)) __builtin_amdgcn_s_waitcnt(gemm_vmcnt(MT + LW));
+            else __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+        };
+        for (uint32_t ss = 0; ss < nss; ss += 3) {
+            superstep(std::integral_constant<int, 0>{}, ss, xs0, ws, wr[0], wr[1], wr[2]);
+            if (ss + 1 < nss) superstep(std::integral_constant<int, 1>{}, ss + 1, xs1, xs0, wr[1], wr[2], wr[0]);
+            if (ss + 2 < nss) superstep(std::integral_constant<int, 2>{}, ss + 2, ws, xs1, wr[2], wr[0], wr[1]);
         }
-        if (a0 + AP < 8) __syncthreads();
-    }
+        epilogue(mtc, acc);
+    };
+    if (live_mt > 4) run_full(std::integral_constant<int, 8>{});
+    else if (live_mt > 2) run_full(std::integral_constant<int, 4>{});
+    else if (live_mt > 1) run_short(std::integral_constant<int, 2>{});
+    else run_short(std::integral_constant<int, 1>{});
 }
 
 // Work list of a dense product y = x . W^T: M tiles of 128 consecutive rows of one "expert" 0,
