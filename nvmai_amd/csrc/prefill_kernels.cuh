@@ -271,16 +271,15 @@ __global__ __launch_bounds__(256) void prefill_mtiles_kernel(const PrefillGroup*
 // one expert) and GEMM_BN output columns: DUAL -> gate and up rows of the same columns,
 // epilogue silu(g) * u (prefill.metal:460-501); else down rows (prefill.metal:503-534).
 //
-// k runs in super-steps of 128 (two quantization groups).  The activations of a super-step go
-// through a double-buffered LDS tile shared by the four waves.  The weights never touch LDS:
-// wave w owns 16 * NT columns of all 128 rows, and lane (i = lane % 16, q = lane / 16)
-// loads the 32 codes W[n_i, k0 + 32q .. +32) of each of its columns in one 16-byte (4 bit) or
-// two (8 bit) loads, so four neighbouring lanes cover 64 or 128 contiguous bytes of a row.
-// It dequantizes them in registers, w = q * scale + bias in fp32 rounded once to the activation
-// type (the reference dequantizes to fp16, tensorops.metal:29-121), straight into the MFMA B
-// operand: MFMA j of the super-step contracts k0 + 32q + 8j .. +8 over q = 0..3, and the A
-// operand is read from LDS with the same k assignment.  v_mfma_f32_16x16x32_{bf16,f16}
-// accumulates in fp32.
+// k runs in super-steps of 128 (two quantization groups).  The activations of a super-step sit
+// in an LDS stage shared by the four waves.  Wave w owns 16 * NT columns of all 128 rows, and
+// lane (i = lane % 16, q = lane / 16) holds the 32 codes W[n_i, k0 + 32q .. +32) of each of its
+// columns, fetched in one 16-byte (4 bit) or two (8 bit) loads, so four neighbouring lanes
+// cover 64 or 128 contiguous bytes of a row.  It dequantizes them in registers,
+// w = q * scale + bias in fp32 rounded once to the activation type (the reference dequantizes
+// to fp16, tensorops.metal:29-121), straight into the MFMA B operand: MFMA j of the super-step
+// contracts k0 + 32q + 8j .. +8 over q = 0..3, and the A operand is read from LDS with the same
+// k assignment.  v_mfma_f32_16x16x32_{bf16,f16} accumulates in fp32.
 typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 hf8_t __attribute__((ext_vector_type(8)));
@@ -305,7 +304,6 @@ struct GemmParams {
 
 constexpr int GEMM_SK = 128;            // k per super-step
 constexpr uint32_t GEMM_UNIT = 4;       // column tiles of one M tile that share an XCD
-constexpr int GEMM_LDK = GEMM_SK + 8;   // padded LDS row: conflict-free 16-byte reads and writes
 
 // Two floats -> two 16-bit activations in one dword, round to nearest even.
 template <int ACT>
