@@ -158,7 +158,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # tokens); other configurations report null.
 MEASURED_TRAFFIC_BYTES = {
     ("decode", 8, 32): (180900 * 2.00 + 1339 * 1.00) * 1024,
-    ("prefill", 4, 4096): (512200 * 2.00 + 32770 * 1.00) * 1024,
+    ("prefill", 4, 4096): (415000 * 2.00 + 36140 * 1.00) * 1024,
     ("attention", 8, 8, 131072): (596100 * 2.00 + 4385 * 1.00) * 1024,
 }
 
