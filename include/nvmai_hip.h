@@ -264,7 +264,9 @@ int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream stream, cons
  * resident: act[p, :] = silu(gate_e x_token(p)) * (up_e x_token(p)) for sorted pair p, then
  * route_partials[token*top_k + rank, :] = down_e act[p, :], both rounded to the activation
  * type.  hidden [query_count, hidden_stride]; act_scratch [n_pairs, f] and route_partials
- * [n_pairs, d] are caller-owned, 16-bit.  d and f must be multiples of 64. */
+ * [n_pairs, d] are caller-owned, 16-bit.  d and f must be multiples of 64.  The kernel addresses
+ * each operand array with 32-bit byte offsets: hidden, act_scratch, an expert's blob and one weight
+ * matrix must each span less than 4 GiB (NVMAI_ERR_UNSUPPORTED otherwise). */
 int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* experts_base,
                                   uint64_t expert_stride, const nvmai_expert_offsets* off, uint32_t bits,
                                   uint32_t d, uint32_t f, uint32_t num_experts, const void* hidden,
@@ -276,7 +278,8 @@ int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream stream, const
  * the dense prefill product y[m, n] = x[m, k] . W[n, k]^T for m rows of activations against
  * one affine 4/8-bit matrix (group 64 along k, BF16 scale/bias), on the matrix cores: weights
  * dequantized once into MFMA operands, fp32 accumulate, y rounded to the activation type.
- * k must be a multiple of 64; x, y and the code rows 16-byte aligned. */
+ * k must be a multiple of 64; x, y and the code rows 16-byte aligned; x and the code matrix each
+ * below 4 GiB (NVMAI_ERR_UNSUPPORTED otherwise). */
 int nvmai_hip_affine_qmm(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
                          const uint16_t* scales, const uint16_t* biases, uint32_t bits, const void* x,
                          uint32_t x_stride, void* y, uint32_t y_stride, uint32_t m, uint32_t n, uint32_t k);
