@@ -300,6 +300,38 @@ def test_dense_qmm_matches_oracle(nv, ctx, bits, m, n, k):
     assert O.rel_error(act_np(y), want) <= TOL_ACT
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m", [16, 17, 33, 48, 65, 128, 129])
+@pytest.mark.parametrize("n,k", [(200, 320), (264, 256)])
+def test_dense_qmm_every_row_tile_count(nv, ctx_bf16, bits, m, n, k):
+    """One, two, three..four and five..eight 16-row tiles take different loop bodies; k = 320 has
+    an odd number of groups (scale rows on 2-byte boundaries, half a super-step at the end) and
+    n = 200 / 264 leave a last column block that sticks out."""
+    say("dense qmm row tiles", bits, m, n, k)
+    rng = np.random.default_rng(m * 13 + n + k + bits)
+    w = gauss(rng, (n, k), 0.05)
+    p, s, b = O.quantize_affine(w, bits)
+    x = O.round_bf16(gauss(rng, (m, k)))
+    y = nv.MPPPrefillInt4QMM(ctx_bf16, bits).encode(dev(p), dev(s.view(np.int16)), dev(b.view(np.int16)),
+                                                    act_tensor(x, ctx_bf16), n, k)
+    torch.cuda.synchronize()
+    want = np.stack([O.affine_gemv(p, s, b, x[t], bits) for t in range(m)])
+    assert O.rel_error(act_np(y), want) <= TOL_ACT
+
+
+def test_gemm_refuses_operands_beyond_32_bit_offsets(nv, ctx_bf16):
+    say("gemm 4 GiB limits")
+    q = nv.MPPPrefillInt4QMM(ctx_bf16, 4)
+    p = torch.zeros((64, 32), dtype=torch.uint8, device="cuda")
+    s = torch.zeros((64, 1), dtype=torch.int16, device="cuda")
+    x = torch.zeros((4, 64), dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros((4, 64), dtype=torch.bfloat16, device="cuda")
+    # 2^26 rows at a stride of 64 elements would put the last row past 4 GiB: refused before any launch
+    rc = nv.lib.nvmai_hip_affine_qmm(ctx_bf16.handle, None, p.data_ptr(), s.data_ptr(), s.data_ptr(), 4,
+                                     x.data_ptr(), 64, y.data_ptr(), 64, 1 << 26, 64, 64)
+    assert rc == -2                                              # NVMAI_ERR_UNSUPPORTED
+
+
 def test_dense_qmm_rejects_bad_arguments(nv, ctx_bf16):
     say("dense qmm errors")
     q = nv.MPPPrefillInt4QMM(ctx_bf16, 4)
