@@ -331,6 +331,47 @@ __device__ __forceinline__ uint4 dequant8(const float* q, float s, float b) {
     return o;
 }
 
+// Eight codes of one dword (4 bit) or of two (8 bit) -> eight dequantized 16-bit values in MFMA
+// operand order, through fp16 "magic" pairs: (code | 0x6400) is the fp16 number 1024 + code, two
+// of them are made by one AND-OR, and the mixed-precision FMA reads either half directly, so
+// no code is converted to float on its own: w = (1024 + q) * s + (b - 1024 s).  The shifted bias
+// is rounded once in fp32 (error below 2^-14 of a quantization step).  mask (0x000F000F or
+// 0x00FF00FF) and magic (0x64006400) arrive in registers: as literals they would split every
+// AND-OR in two, a three-operand instruction takes no literal here.
+template <int ACT, int BITS>
+__device__ __forceinline__ uint4 dequant8_magic(uint32_t w0, uint32_t w1, float s, float b1024, uint32_t mask, uint32_t magic) {
+    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+    uint32_t pr[4];                         // pr[i] = (code lo_i, code hi_i) as fp16 pairs
+    int lo_of[8], half_of[8];               // element e sits in pr[lo_of[e]], half half_of[e]
+    if (BITS == 4) {
+        // dword w0: codes at bits 4e; pair i = (code i, code i + 4)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pr[i] = ((w0 >> (4 * i)) & mask) | magic;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { lo_of[e] = e & 3; half_of[e] = e >> 2; }
+    } else {
+        // bytes of w0 = codes 0..3, of w1 = codes 4..7; pair (0, 2), (1, 3) of each dword
+        pr[0] = (w0 & mask) | magic;
+        pr[1] = ((w0 >> 8) & mask) | magic;
+        pr[2] = (w1 & mask) | magic;
+        pr[3] = ((w1 >> 8) & mask) | magic;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { lo_of[e] = (e >> 2) * 2 + (e & 1); half_of[e] = (e >> 1) & 1; }
+    }
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const h2_t h = __builtin_bit_cast(h2_t, pr[lo_of[e]]);
+        v[e] = __builtin_fmaf((float)(half_of[e] ? h.y : h.x), s, b1024);
+    }
+    uint4 o;
+    o.x = pack_act2<ACT>(v[0], v[1]);
+    o.y = pack_act2<ACT>(v[2], v[3]);
+    o.z = pack_act2<ACT>(v[4], v[5]);
+    o.w = pack_act2<ACT>(v[6], v[7]);
+    return o;
+}
+
 // NT = 16-column tiles per wave (2 or 4): the block covers 32 NT gate/up columns (DUAL) or
 // 64 NT down columns.  NT = 4 reads each activation fragment from LDS once for four MFMAs and
 // halves the number of blocks that re-read an M tile's activations.
@@ -569,19 +610,23 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     // other half of bf[], across super-step boundaries too.  MT = 16-row tiles multiplied
     // (1, 2, 4 or 8, block-uniform): the body holds no branch, so that the LDS reads of the next
     // row tile and the dequantization interleave with the MFMAs.
+    uint32_t dq_mask = BITS == 4 ? 0x000F000Fu : 0x00FF00FFu, dq_magic = 0x64006400u;
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm("" : "+s"(dq_mask));                            // opaque: kept in a scalar / a vector register
+    asm("" : "+v"(dq_magic));
+#endif
     auto dequant_step = [&](const uint4 (*w4)[WQ], const uint32_t* sb, int j, uint4* bfrag) {
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            float q[8];
+            const float sc = __builtin_bit_cast(float, sb[t] & 0xFFFF0000u);
+            const float b1024 = __builtin_fmaf(-1024.0f, sc, __builtin_bit_cast(float, sb[t] << 16));
             if (BITS == 4) {
                 const uint4 w = w4[t][0];
-                unpack4_bytes(j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w, q);
+                bfrag[t] = dequant8_magic<ACT, 4>(j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w, 0u, sc, b1024, dq_mask, dq_magic);
             } else {
-                const uint4 w = w4[t][BITS == 8 ? j >> 1 : 0];
-                unpack8((j & 1) ? w.z : w.x, q);
-                unpack8((j & 1) ? w.w : w.y, q + 4);
+                const uint4 w = w4[t][j >> 1];
+                bfrag[t] = dequant8_magic<ACT, 8>((j & 1) ? w.z : w.x, (j & 1) ? w.w : w.y, sc, b1024, dq_mask, dq_magic);
             }
-            bfrag[t] = dequant8<ACT>(q, __builtin_bit_cast(float, sb[t] & 0xFFFF0000u), __builtin_bit_cast(float, sb[t] << 16));
         }
     };
     // LDS byte address of the lane's fragment of row tile 0, MFMA step 0, stage 0; step j: ^ 16 j
