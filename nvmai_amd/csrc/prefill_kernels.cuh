@@ -672,6 +672,14 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         const int piece = tid % PIECES, prow = tid / PIECES;
         uint16_t* out = (uint16_t*)p.out;
         const bool vec_ok = (p.out_stride % 8 == 0) && n0 + OC <= p.N;
+        // Down projection: a row's destination comes from its pair record.  All of them are
+        // fetched now, in one round trip, into the second activation stage; fetched row by row
+        // inside the store loop each one would be a dependent global load.
+        uint32_t* orow_tab = reinterpret_cast<uint32_t*>(xs1);
+        if (!DUAL && (uint32_t)tid < mt.rows) {
+            const PrefillPair pr = p.pairs[mt.row_start + tid];
+            orow_tab[tid] = pr.token * p.top_k + pr.rank;
+        }
 #pragma unroll
         for (int a0 = 0; a0 < MT; a0 += AP) {
             if (a0 >= live_mt) break;                       // block-uniform
@@ -695,12 +703,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
             __syncthreads();
             const uint32_t m_end = min(mt.rows, (uint32_t)(a0 + AP) * 16u);
             for (uint32_t m = a0 * 16 + prow; m < m_end; m += ROWS_PER_PASS) {
-                size_t orow;
-                if (DUAL) orow = (size_t)(mt.row_start + m) * p.out_stride;
-                else {
-                    const PrefillPair pr = p.pairs[mt.row_start + m];
-                    orow = ((size_t)pr.token * p.top_k + pr.rank) * p.out_stride;
-                }
+                const size_t orow = (size_t)(DUAL ? mt.row_start + m : orow_tab[m]) * p.out_stride;
                 const uint4 v = *reinterpret_cast<const uint4*>(os + (m - a0 * 16) * LDO + piece * 8);
                 const uint32_t c0 = n0 + piece * 8;
                 if (vec_ok) *reinterpret_cast<uint4*>(out + orow + c0) = v;
