@@ -252,14 +252,17 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
 // One block per (batch, kv head, chunk): every q head of the group is served from ONE read of
 // the K/V rows.  Each wave walks 32-token steps of the chunk with its own online-softmax state;
 // the four waves merge through LDS at the end.
-//   S^T[tokens, heads] = K . Q^T   v_mfma_f32_16x16x32_f16, A = codes as fp16 (1024 + c),
+//   S^T[tokens, heads] = K . Q^T   v_mfma_f32_16x16x32_f16, A = the codes themselves, read as
+//                                  fp16 subnormals (c * 2^-24: the matrix cores take them
+//                                  exactly, and a byte-permute with zero bytes makes two),
 //                                  B = q scaled by a power of two per head and cast to fp16;
 //                                  one accumulator per 64-wide group so that the row's fp16
 //                                  scale and bias are applied exactly:
-//                                  s = sum_g sc_g (acc_g - 1024 qsum_g) + bi_g qsum_g
+//                                  s = 2^24 sum_g sc_g acc_g + sum_g bi_g qsum_g
 //   O[heads, dims]    = P'_g . V   A = p_t * vsc[t, g] as fp16 (one operand per group),
-//                                  B = V codes as fp16 (1024 + c); the bias and the 1024
-//                                  offset are carried in a per-(head, group) correction.
+//                                  B = V codes as fp16 subnormals; O carries the factor 2^-24
+//                                  until the wave finishes, the bias goes into a
+//                                  per-(head, group) correction.
 // Lane roles (l = lane, r = l / 16, i = l % 16):
 //   K operand: token i of the 16-token tile, dims 64g + 16r + 8h .. +8 for MFMA call (g, h)
 //   Q operand: head i, the same dims
@@ -447,14 +450,14 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
                     H8 a;
                     if (BITS == 8) {
                         const uint32_t w0 = kraw[tile][g][2 * h], w1 = kraw[tile][g][2 * h + 1];
-                        a.u[0] = __builtin_amdgcn_perm(w0, 0x64646464u, 0x00050004u);
-                        a.u[1] = __builtin_amdgcn_perm(w0, 0x64646464u, 0x00070006u);
-                        a.u[2] = __builtin_amdgcn_perm(w1, 0x64646464u, 0x00050004u);
-                        a.u[3] = __builtin_amdgcn_perm(w1, 0x64646464u, 0x00070006u);
+                        a.u[0] = __builtin_amdgcn_perm(w0, w0, 0x0C050C04u);      // [c0, 0, c1, 0]
+                        a.u[1] = __builtin_amdgcn_perm(w0, w0, 0x0C070C06u);
+                        a.u[2] = __builtin_amdgcn_perm(w1, w1, 0x0C050C04u);
+                        a.u[3] = __builtin_amdgcn_perm(w1, w1, 0x0C070C06u);
                     } else {
                         const uint32_t w = kraw[tile][g][h];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) a.u[j] = ((w >> (4 * j)) & 0x000F000Fu) | 0x64006400u;
+                        for (int j = 0; j < 4; ++j) a.u[j] = (w >> (4 * j)) & 0x000F000Fu;
                     }
                     sacc[g] = mfma16(a, qop[g][h], sacc[g]);
                 }
@@ -463,15 +466,15 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
             for (int t = 0; t < 4; ++t) {
                 const int slot = tile * 4 + t;
                 const uint32_t scw[2] = {ksc[slot].x, ksc[slot].y}, biw[2] = {kbi[slot].x, kbi[slot].y};
-                float acc = 0.0f;
+                float acc_s = 0.0f, acc_b = 0.0f;
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const float sc = f16_to_f32((uint16_t)(scw[g >> 1] >> (16 * (g & 1))));
                     const float bi = f16_to_f32((uint16_t)(biw[g >> 1] >> (16 * (g & 1))));
-                    acc = fmaf(sc, fmaf(-1024.0f, qsum[g], sacc[g][t]), acc);
-                    acc = fmaf(bi, qsum[g], acc);
+                    acc_s = fmaf(sc, sacc[g][t], acc_s);
+                    acc_b = fmaf(bi, qsum[g], acc_b);
                 }
-                sv[slot] = tok_ok[slot] ? acc * q_unscale : -INFINITY;
+                sv[slot] = tok_ok[slot] ? fmaf(acc_s, 16777216.0f, acc_b) * q_unscale : -INFINITY;
             }
         }
 
@@ -504,7 +507,6 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
                 const float bi = f16_to_f32((uint16_t)(biw >> (16 * (g & 1))));
                 hb[t] = f32_to_f16(pe[t] * sc);
                 c = fmaf(pe[t], bi, c);
-                c = fmaf(-1024.0f, f16_to_f32(hb[t]), c);
             }
             corr[g] = c;
 #pragma unroll
@@ -537,11 +539,11 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
                     if (BITS == 8) {
-                        // byte n of two token dwords -> [a.n, 0, c2.n, 0], then the 0x64 exponent bytes
+                        // byte n of two token dwords -> [a.n, 0, c2.n, 0]: two fp16 subnormals
                         const uint32_t sel = 0x0C000C00u | (uint32_t)n | ((uint32_t)(4 + n) << 16);
-                        bop.u[w] = __builtin_amdgcn_perm(vraw[2 * w + 1][g], vraw[2 * w][g], sel) | 0x64006400u;
+                        bop.u[w] = __builtin_amdgcn_perm(vraw[2 * w + 1][g], vraw[2 * w][g], sel);
                     } else {
-                        bop.u[w] = ((pair4[w] >> (4 * n)) & 0x000F000Fu) | 0x64006400u;
+                        bop.u[w] = (pair4[w] >> (4 * n)) & 0x000F000Fu;
                     }
                 }
                 oacc[g][n] = mfma16(pop[g], bop, oacc[g][n]);
@@ -564,8 +566,9 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
         const float4 cg = *reinterpret_cast<const float4*>(bc + 4 * r);
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int n = 0; n < 4; ++n) {
-            oacc[g][n][0] += cg.x; oacc[g][n][1] += cg.y; oacc[g][n][2] += cg.z; oacc[g][n][3] += cg.w;
+        for (int n = 0; n < 4; ++n) {                               // O leaves its 2^-24 here
+            oacc[g][n][0] = fmaf(oacc[g][n][0], 16777216.0f, cg.x); oacc[g][n][1] = fmaf(oacc[g][n][1], 16777216.0f, cg.y);
+            oacc[g][n][2] = fmaf(oacc[g][n][2], 16777216.0f, cg.z); oacc[g][n][3] = fmaf(oacc[g][n][3], 16777216.0f, cg.w);
         }
     }
 
