@@ -142,9 +142,8 @@ extern "C" int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream strea
     {
         ProfScope ps(ctx, NVMAI_PROF_ATTN_PARTIAL, s);
         if (fast) {
-            const size_t lds = (256 + 3 * (16 * ATTN_HD + 32)) * sizeof(float);
             dim3 grid(batch * num_kv_heads * nc);
-#define NVMAI_ATTN(ACT, BITS) attn_partial_mfma_kernel<ACT, BITS><<<grid, 256, lds, s>>>(p)
+#define NVMAI_ATTN(ACT, BITS) attn_partial_mfma_kernel<ACT, BITS><<<grid, 256, 0, s>>>(p)
             if (ctx->act == ACT_BF16) { if (k->bits == 8) NVMAI_ATTN(ACT_BF16, 8); else NVMAI_ATTN(ACT_BF16, 4); }
             else { if (k->bits == 8) NVMAI_ATTN(ACT_FP16, 8); else NVMAI_ATTN(ACT_FP16, 4); }
 #undef NVMAI_ATTN

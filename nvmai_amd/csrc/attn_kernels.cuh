@@ -279,18 +279,39 @@ __device__ __forceinline__ f4_t mfma16(const H8& a, const H8& b, f4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.v, b.v, c, 0, 0, 0);
 }
 
+// s_waitcnt operand: at most n vector-memory loads still in flight, the other counters free.
+constexpr int gemm_like_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
+
 constexpr int ATTN_HD = 256;
 constexpr int ATTN_STEP = 32;
 
 template <int ACT, int BITS>
-__global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
-    // LDS: per wave [16 heads][256 dims] O + [16] m + [16] d for the final merge (waves 1..3),
-    // plus a 64-float scratch per wave for head-indexed broadcasts.
-    extern __shared__ float lds[];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+__global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p) {
+    // LDS.  Every wave owns a K region and a V region, filled by buffer_load ... lds without
+    // touching registers: 32 tokens x the codes of this KV head, the 16-byte chunks of a token
+    // XOR-swizzled by the token, then 16 bytes of (scales, biases) per token.  The K region is
+    // refilled for the next step as soon as the scores are out, the V region at the end of the
+    // step, so each load has half a step to land and one buffer each suffices: 70 KB per block
+    // at 8 bits, two blocks per compute unit.  K and V are separate arrays so that the compiler
+    // can tell a read of one from a load in flight into the other.  After the loop the K array
+    // is the merge area of a two-round tree: [2][16 heads][256 dims] O + [16] m + [16] d.
+    // A 64-float scratch per wave serves head-indexed broadcasts.
+    constexpr uint32_t CODE_ROW = ATTN_HD * BITS / 8;              // bytes of one token's codes (this head)
+    constexpr uint32_t REGION = 32 * CODE_ROW + 512;              // codes | (scales, biases)
+    constexpr uint32_t OFF_META = 32 * CODE_ROW;
+    constexpr uint32_t MERGE_SLOT = 16 * ATTN_HD + 32;            // floats
+    constexpr uint32_t MERGE_BYTES = 2 * MERGE_SLOT * 4;
+    constexpr uint32_t KARRAY = 4 * REGION > MERGE_BYTES ? 4 * REGION : MERGE_BYTES;
+    __shared__ __attribute__((aligned(16))) uint8_t kst[KARRAY];
+    __shared__ __attribute__((aligned(16))) uint8_t vst[4 * REGION];
+    __shared__ float bc_all[256];
+    // vst is written by load instructions only; a store that never runs keeps the optimizer
+    // from treating it as never written (head_dim 0 is rejected by the entry point)
+    if (p.head_dim == 0) vst[threadIdx.x] = 0;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, r = lane >> 4;
-    float* bc = lds + wave * 64;                                   // broadcast scratch
-    float* merge = lds + 256;                                      // [3][16*256 + 32]
+    float* bc = bc_all + wave * 64;                                // broadcast scratch
+    float* merge = reinterpret_cast<float*>(kst);                  // after the loop
     const uint32_t chunk = blockIdx.x % p.num_chunks;
     const uint32_t kvh = (blockIdx.x / p.num_chunks) % p.num_kv_heads;
     const uint32_t b = blockIdx.x / (p.num_chunks * p.num_kv_heads);
@@ -367,75 +388,47 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
     float m_run = -INFINITY, d_run = 0.0f;                          // head i; d over this lane's tokens only
     float corr[4] = {0.0f, 0.0f, 0.0f, 0.0f};                       // head i, this lane's tokens only
 
-    // K side of a step (codes of token i of both tiles, fp16 scale/bias of this lane's 8 token
-    // slots).  It is dead once the scores are out, so the next step's K side is requested right
-    // there and arrives behind the softmax and the P.V products of the current step.
-    uint32_t kraw[2][4][4];                                         // [tile][group][dwords]; 4-bit uses 2 dwords
-    uint2 ksc[8], kbi[8];                                           // 4 fp16 each
-    auto slot_pos = [&](uint32_t s0, int t) { return s0 + (t >> 2) * 16 + 4 * r + (t & 3); };
-    // Buffer loads: a scalar resource per cache, one 32-bit lane offset per row, the group and
-    // metadata offsets as immediates or scalars -- no 64-bit address arithmetic per load, and
-    // reads past the end of the sequence's rows return zero instead of faulting.
-    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    auto slot_tok = [&](int t) { return (uint32_t)((t >> 2) * 16 + 4 * r + (t & 3)); };   // token of slot t inside the step
+    // Buffer loads: a scalar resource per cache, 32-bit offsets; reads past the end of the
+    // sequence's rows return zero instead of faulting (tokens past the chunk are masked anyway).
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t*>(kbase), 0, (int)(p.seq_len * p.f.stride), 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t*>(vbase), 0, (int)(p.seq_len * p.f.stride), 0x00020000);
-    auto load_k = [&](uint32_t s0) {
+    // One load instruction moves 1 KB = the codes of 4 (8 bit) or 8 (4 bit) tokens: lane l takes
+    // chunk (l % LPT) ^ token of token l / LPT, which lands in slot l % LPT of that token.
+    constexpr int LPT = CODE_ROW / 16;                              // lanes (16-byte chunks) per token
+    constexpr int TPI = 64 / LPT;                                   // tokens per instruction
+    const uint32_t d_tok = lane / LPT, d_slot = lane % LPT;
+    const uint32_t d_chunk16 = ((d_slot ^ d_tok) & (LPT - 1)) * 16u;  // 8 bit: ^ 64 (j & 3) per instruction
+    const uint32_t m_part = (lane & 3) < 2 ? meta_sc + 4 * (lane & 3) : meta_bi + 4 * ((lane & 3) - 2);
+    uint8_t* const myk = kst + wave * REGION;
+    uint8_t* const myv = vst + wave * REGION;
+    constexpr int N_LOADS = 32 / TPI + 2;                           // load instructions of one region
+    auto issue_region = [&](uint32_t s0, const __amdgpu_buffer_rsrc_t& rs, uint8_t* st) {
+        const uint32_t row = (s0 + d_tok) * p.f.stride;
 #pragma unroll
-        for (int tile = 0; tile < 2; ++tile) {
-            const uint32_t pos = min(s0 + tile * 16 + i, p1 - 1);
-            const uint32_t off = pos * p.f.stride + (BITS == 8 ? 16 : 8) * r;
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                if (BITS == 8) {
-                    const u32x4_t w = __builtin_amdgcn_raw_buffer_load_b128(krsrc, off + 64 * g, code_off, 0);
-                    kraw[tile][g][0] = w.x; kraw[tile][g][1] = w.y; kraw[tile][g][2] = w.z; kraw[tile][g][3] = w.w;
-                } else {
-                    const u32x2_t w = __builtin_amdgcn_raw_buffer_load_b64(krsrc, off + 32 * g, code_off, 0);
-                    kraw[tile][g][0] = w.x; kraw[tile][g][1] = w.y;
-                }
-            }
+        for (int j = 0; j < 32 / TPI; ++j) {
+            const uint32_t voff = row + (BITS == 8 ? (d_chunk16 ^ (64u * (j & 3))) : d_chunk16);
+            const uint32_t soff = (uint32_t)(j * TPI) * p.f.stride + code_off;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(st + j * 1024), 16, voff, soff, 0, 0);
         }
+        const uint32_t mrow = (s0 + (lane >> 2)) * p.f.stride + m_part;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const uint32_t off = min(slot_pos(s0, t), p1 - 1) * p.f.stride;
-            const u32x2_t a = __builtin_amdgcn_raw_buffer_load_b64(krsrc, off, meta_sc, 0);
-            const u32x2_t c = __builtin_amdgcn_raw_buffer_load_b64(krsrc, off, meta_bi, 0);
-            ksc[t] = uint2{a.x, a.y};
-            kbi[t] = uint2{c.x, c.y};
-        }
+        for (int m = 0; m < 2; ++m)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(st + OFF_META + m * 256), 4, mrow,
+                                                     (uint32_t)(16 * m) * p.f.stride, 0, 0);
     };
     const uint32_t s_first = p0 + wave * ATTN_STEP;
-    if (s_first < p1) load_k(s_first);
+    if (s_first < p1) { issue_region(s_first, krsrc, myk); issue_region(s_first, vrsrc, myv); }
 
     for (uint32_t s0 = s_first; s0 < p1; s0 += 4 * ATTN_STEP) {
-        // ---- loads: V metadata and codes of this lane's 8 tokens
-        uint32_t tok[8];                                            // clamped token positions of the P/V slots
+        const bool more = s0 + 4 * ATTN_STEP < p1;                  // wave-uniform
+        // the K region of this step has landed; only this step's V loads may still be in flight
+        __builtin_amdgcn_s_waitcnt(gemm_like_vmcnt(N_LOADS));
         bool tok_ok[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const uint32_t pos = slot_pos(s0, t);
-            tok_ok[t] = pos < p1;
-            tok[t] = tok_ok[t] ? pos : p1 - 1;
-        }
-        uint2 vsc[8], vbi[8];                                       // 4 fp16 each
-        uint32_t vraw[8][4];                                        // [token slot][group]: 4 codes (8-bit) / 4 nibbles
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const uint32_t off = tok[t] * p.f.stride;
-            const u32x2_t a = __builtin_amdgcn_raw_buffer_load_b64(vrsrc, off, meta_sc, 0);
-            const u32x2_t c = __builtin_amdgcn_raw_buffer_load_b64(vrsrc, off, meta_bi, 0);
-            vsc[t] = uint2{a.x, a.y};
-            vbi[t] = uint2{c.x, c.y};
-            const uint32_t voff = off + (BITS == 8 ? 4 : 2) * i;
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                if (BITS == 8) vraw[t][g] = __builtin_amdgcn_raw_buffer_load_b32(vrsrc, voff + 64 * g, code_off, 0);
-                else vraw[t][g] = __builtin_amdgcn_raw_buffer_load_b16(vrsrc, voff + 32 * g, code_off, 0);
-            }
-        }
+        for (int t = 0; t < 8; ++t) tok_ok[t] = s0 + slot_tok(t) < p1;
 
         // ---- S^T = K . Q^T per group, then the exact affine correction
         float sv[8];                                                // scores of head i at this lane's 8 tokens
@@ -445,17 +438,26 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 sacc[g] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                // codes of token i of the tile, dims 64 g + 16 r .. +16
+                uint32_t kw[4];
+                if (BITS == 8) {
+                    const uint4 w = *reinterpret_cast<const uint4*>(myk + (tile * 16 + i) * CODE_ROW + (((4 * g + r) ^ i) & 15) * 16);
+                    kw[0] = w.x; kw[1] = w.y; kw[2] = w.z; kw[3] = w.w;
+                } else {
+                    const uint2 w = *reinterpret_cast<const uint2*>(myk + (tile * 16 + i) * CODE_ROW + (((2 * g + (r >> 1)) ^ i) & 7) * 16 + (r & 1) * 8);
+                    kw[0] = w.x; kw[1] = w.y;
+                }
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     H8 a;
                     if (BITS == 8) {
-                        const uint32_t w0 = kraw[tile][g][2 * h], w1 = kraw[tile][g][2 * h + 1];
+                        const uint32_t w0 = kw[2 * h], w1 = kw[2 * h + 1];
                         a.u[0] = __builtin_amdgcn_perm(w0, w0, 0x0C050C04u);      // [c0, 0, c1, 0]
                         a.u[1] = __builtin_amdgcn_perm(w0, w0, 0x0C070C06u);
                         a.u[2] = __builtin_amdgcn_perm(w1, w1, 0x0C050C04u);
                         a.u[3] = __builtin_amdgcn_perm(w1, w1, 0x0C070C06u);
                     } else {
-                        const uint32_t w = kraw[tile][g][h];
+                        const uint32_t w = kw[h];
 #pragma unroll
                         for (int j = 0; j < 4; ++j) a.u[j] = (w >> (4 * j)) & 0x000F000Fu;
                     }
@@ -465,7 +467,8 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const int slot = tile * 4 + t;
-                const uint32_t scw[2] = {ksc[slot].x, ksc[slot].y}, biw[2] = {kbi[slot].x, kbi[slot].y};
+                const uint4 km = *reinterpret_cast<const uint4*>(myk + OFF_META + slot_tok(slot) * 16);
+                const uint32_t scw[2] = {km.x, km.y}, biw[2] = {km.z, km.w};
                 float acc_s = 0.0f, acc_b = 0.0f;
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
@@ -478,7 +481,10 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
             }
         }
 
-        if (s0 + 4 * ATTN_STEP < p1) load_k(s0 + 4 * ATTN_STEP);      // next step's K side
+        // the scores are out: the K region takes the next step's rows (every read of it has
+        // returned, the score arithmetic used them)
+        __builtin_amdgcn_s_waitcnt(0xC07F);                         // lgkmcnt(0)
+        if (more) issue_region(s0 + 4 * ATTN_STEP, krsrc, myk);
 
         // ---- online softmax for head i (its tokens are spread over the four lane quarters)
         float mx = sv[0];
@@ -495,6 +501,11 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
         m_run = m_new;
 
         // ---- P'_g = p * vsc_g as fp16; correction terms; rescale O by alpha of its heads
+        // the V region of this step has landed; the K loads just issued may still be in flight
+        if (more) __builtin_amdgcn_s_waitcnt(gemm_like_vmcnt(N_LOADS)); else __builtin_amdgcn_s_waitcnt(0x0F70);
+        uint4 vm[8];                                                // (sc.x, sc.y, bi.x, bi.y) of the 8 token slots
+#pragma unroll
+        for (int t = 0; t < 8; ++t) vm[t] = *reinterpret_cast<const uint4*>(myv + OFF_META + slot_tok(t) * 16);
         H8 pop[4];
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
@@ -502,7 +513,7 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
             uint16_t hb[8];
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                const uint32_t scw = g < 2 ? vsc[t].x : vsc[t].y, biw = g < 2 ? vbi[t].x : vbi[t].y;
+                const uint32_t scw = g < 2 ? vm[t].x : vm[t].y, biw = g < 2 ? vm[t].z : vm[t].w;
                 const float sc = f16_to_f32((uint16_t)(scw >> (16 * (g & 1))));
                 const float bi = f16_to_f32((uint16_t)(biw >> (16 * (g & 1))));
                 hb[t] = f32_to_f16(pe[t] * sc);
@@ -528,10 +539,18 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
         // ---- O += P'_g . V   (B operand: dim 64g + 4i + n, this lane's 8 tokens)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
+            // this lane's 4 dims (64 g + 4 i ..) of its 8 token slots
+            uint32_t vr[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const uint32_t tk = slot_tok(t);
+                if (BITS == 8) vr[t] = *reinterpret_cast<const uint32_t*>(myv + tk * CODE_ROW + (((4 * g + (i >> 2)) ^ tk) & 15) * 16 + (i & 3) * 4);
+                else vr[t] = *reinterpret_cast<const uint16_t*>(myv + tk * CODE_ROW + (((2 * g + (i >> 3)) ^ tk) & 7) * 16 + (i & 7) * 2);
+            }
             uint32_t pair4[4];                                      // 4-bit: nibbles of two tokens side by side
             if (BITS == 4) {
 #pragma unroll
-                for (int w = 0; w < 4; ++w) pair4[w] = vraw[2 * w][g] | (vraw[2 * w + 1][g] << 16);
+                for (int w = 0; w < 4; ++w) pair4[w] = vr[2 * w] | (vr[2 * w + 1] << 16);
             }
 #pragma unroll
             for (int n = 0; n < 4; ++n) {
@@ -541,7 +560,7 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
                     if (BITS == 8) {
                         // byte n of two token dwords -> [a.n, 0, c2.n, 0]: two fp16 subnormals
                         const uint32_t sel = 0x0C000C00u | (uint32_t)n | ((uint32_t)(4 + n) << 16);
-                        bop.u[w] = __builtin_amdgcn_perm(vraw[2 * w + 1][g], vraw[2 * w][g], sel);
+                        bop.u[w] = __builtin_amdgcn_perm(vr[2 * w + 1], vr[2 * w], sel);
                     } else {
                         bop.u[w] = (pair4[w] >> (4 * n)) & 0x000F000Fu;
                     }
@@ -549,6 +568,9 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
                 oacc[g][n] = mfma16(pop[g], bop, oacc[g][n]);
             }
         }
+        // every read of the V region has returned (the MFMAs took them): it takes the next step's rows
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        if (more) issue_region(s0 + 4 * ATTN_STEP, vrsrc, myv);
     }
 
     // ---- finish this wave: d and corr over the four quarters, corr folded into O
@@ -572,65 +594,65 @@ __global__ __launch_bounds__(256) void attn_partial_mfma_kernel(AttnParams p) {
         }
     }
 
-    // ---- merge the four waves (wave 0 collects), attention.metal:388-429's rule
-    float* mine = merge + (wave - 1) * (16 * ATTN_HD + 32);
-    if (wave > 0) {
+    // ---- merge the four waves, attention.metal:388-429's rule, as a tree of pairwise merges
+    // (3 -> 2 and 1 -> 0, then 2 -> 0).  The merge area lies over the K array: every wave must be
+    // through with its loop first.
+    auto put_state = [&](float* slot) {
 #pragma unroll
         for (int g = 0; g < 4; ++g)
 #pragma unroll
             for (int n = 0; n < 4; ++n)
 #pragma unroll
-                for (int t = 0; t < 4; ++t) mine[(4 * r + t) * ATTN_HD + 64 * g + 4 * i + n] = oacc[g][n][t];
-        if (r == 0) { mine[16 * ATTN_HD + i] = m_run; mine[16 * ATTN_HD + 16 + i] = d_run; }
-    }
+                for (int t = 0; t < 4; ++t) slot[(4 * r + t) * ATTN_HD + 64 * g + 4 * i + n] = oacc[g][n][t];
+        if (r == 0) { slot[16 * ATTN_HD + i] = m_run; slot[16 * ATTN_HD + 16 + i] = d_run; }
+    };
+    auto take_state = [&](const float* slot) {
+        const float m_o = slot[16 * ATTN_HD + i], d_o = slot[16 * ATTN_HD + 16 + i];
+        const float m_new = fmaxf(m_run, m_o);
+        const float wa = m_run == -INFINITY ? 0.0f : expf(m_run - m_new);
+        const float wb = m_o == -INFINITY ? 0.0f : expf(m_o - m_new);
+        d_run = d_run * wa + d_o * wb;
+        m_run = m_new;
+        // weights of heads 4r .. 4r+3 (the O layout) through the broadcast scratch
+        if (r == 0) bc[i] = wa;
+        __builtin_amdgcn_wave_barrier();
+        const float4 a4 = *reinterpret_cast<const float4*>(bc + 4 * r);
+        __builtin_amdgcn_wave_barrier();
+        if (r == 0) bc[i] = wb;
+        __builtin_amdgcn_wave_barrier();
+        const float4 b4 = *reinterpret_cast<const float4*>(bc + 4 * r);
+        __builtin_amdgcn_wave_barrier();
+        const float wa4[4] = {a4.x, a4.y, a4.z, a4.w}, wb4[4] = {b4.x, b4.y, b4.z, b4.w};
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int n = 0; n < 4; ++n)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    oacc[g][n][t] = oacc[g][n][t] * wa4[t] + slot[(4 * r + t) * ATTN_HD + 64 * g + 4 * i + n] * wb4[t];
+    };
+    __syncthreads();
+    if (wave & 1) put_state(merge + (wave >> 1) * MERGE_SLOT);
+    __syncthreads();
+    if (!(wave & 1)) take_state(merge + (wave >> 1) * MERGE_SLOT);
+    __syncthreads();
+    if (wave == 2) put_state(merge);
     __syncthreads();
     if (wave != 0) return;
-    float m_all = m_run;
-#pragma unroll
-    for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, merge[w * (16 * ATTN_HD + 32) + 16 * ATTN_HD + i]);
-    // weights e^(m_w - m_all) per head i; broadcast to the O layout (heads 4r..4r+3) through LDS
-    float wgt[4];
-    wgt[0] = m_run == -INFINITY ? 0.0f : expf(m_run - m_all);
-    float d_all = d_run * wgt[0];
-#pragma unroll
-    for (int w = 0; w < 3; ++w) {
-        const float mw = merge[w * (16 * ATTN_HD + 32) + 16 * ATTN_HD + i];
-        wgt[w + 1] = mw == -INFINITY ? 0.0f : expf(mw - m_all);
-        d_all += merge[w * (16 * ATTN_HD + 32) + 16 * ATTN_HD + 16 + i] * wgt[w + 1];
-    }
-    float4 wq[4];
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-        if (r == 0) bc[i] = wgt[w];
-        __builtin_amdgcn_wave_barrier();
-        wq[w] = *reinterpret_cast<const float4*>(bc + 4 * r);
-        __builtin_amdgcn_wave_barrier();
-    }
+    take_state(merge);
     const size_t hbase = (size_t)b * p.num_q_heads + kvh * qpk;
     if (r == 0 && (uint32_t)i < qpk) {
-        p.m_part[(hbase + i) * p.num_chunks + chunk] = m_all;
-        p.d_part[(hbase + i) * p.num_chunks + chunk] = d_all;
+        p.m_part[(hbase + i) * p.num_chunks + chunk] = m_run;
+        p.d_part[(hbase + i) * p.num_chunks + chunk] = d_run;
     }
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         const uint32_t head = 4 * r + t;
         if (head >= qpk) continue;
-        const float w0 = t == 0 ? wq[0].x : t == 1 ? wq[0].y : t == 2 ? wq[0].z : wq[0].w;
         float* dst = p.o_part + ((hbase + head) * p.num_chunks + chunk) * ATTN_HD;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            float4 o4;
-            float* o4p = &o4.x;
-#pragma unroll
-            for (int n = 0; n < 4; ++n) {
-                float acc = oacc[g][n][t] * w0;
-#pragma unroll
-                for (int w = 0; w < 3; ++w) {
-                    const float ww = t == 0 ? wq[w + 1].x : t == 1 ? wq[w + 1].y : t == 2 ? wq[w + 1].z : wq[w + 1].w;
-                    acc += merge[w * (16 * ATTN_HD + 32) + head * ATTN_HD + 64 * g + 4 * i + n] * ww;
-                }
-                o4p[n] = acc;
-            }
+            const float4 o4 = {oacc[g][0][t], oacc[g][1][t], oacc[g][2][t], oacc[g][3][t]};
             *reinterpret_cast<float4*>(dst + 64 * g + 4 * i) = o4;
         }
     }
