@@ -159,7 +159,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 MEASURED_TRAFFIC_BYTES = {
     ("decode", 8, 32): (180900 * 2.00 + 1339 * 1.00) * 1024,
     ("prefill", 4, 4096): (415000 * 2.00 + 36140 * 1.00) * 1024,
-    ("attention", 8, 8, 131072): (596100 * 2.00 + 4385 * 1.00) * 1024,
+    ("attention", 8, 8, 131072): (599800 * 2.00 + 4383 * 1.00) * 1024,
+    ("attention", 4, 8, 131072): (295900 * 2.00 + 4356 * 1.00) * 1024,
 }
 
 
