@@ -133,7 +133,6 @@ void launch_rows_t(RowsParams& p, int maxtok, uint32_t max_entries, hipStream_t 
         else launch_fast<ACT, BITS, SEG, NCH, 4, DUAL, XF32, RPI, ITERS>(p, max_entries, s);    \
         return;                                                                                 \
     } while (0)
-    static const int variant = getenv("NVMAI_ROWS_VARIANT") ? atoi(getenv("NVMAI_ROWS_VARIANT")) : 0;
     // Few entries (a small decode batch): short blocks, so that the launch still covers the device.
     const bool few = max_entries <= 40;
     if constexpr (DUAL) {
@@ -144,19 +143,12 @@ void launch_rows_t(RowsParams& p, int maxtok, uint32_t max_entries, hipStream_t 
         if (few && chunks == 32) NVMAI_FAST(32, 1, 2, 2);
     }
     if constexpr (DUAL) {
-        if (chunks == 64) NVMAI_FAST(64, 1, 1, 8);
-        if (chunks == 128 && variant % 10 == 1) NVMAI_FAST(32, 4, 1, 8);
-        if (chunks == 128 && variant % 10 == 2) NVMAI_FAST(32, 4, 1, 4);
-        if (chunks == 128 && variant % 10 == 3) NVMAI_FAST(64, 2, 1, 4);
-        if (chunks == 128 && variant % 10 == 4) NVMAI_FAST(64, 2, 1, 16);
+        if (chunks == 64) NVMAI_FAST(64, 1, 2, 2);
         if (chunks == 128) NVMAI_FAST(64, 2, 1, 8);
     } else {
-        if (chunks == 16) NVMAI_FAST(16, 1, 1, 8);
-        if (chunks == 32 && variant / 10 == 1) NVMAI_FAST(16, 2, 1, 8);
-        if (chunks == 32 && variant / 10 == 2) NVMAI_FAST(16, 2, 2, 4);
-        if (chunks == 32 && variant / 10 == 3) NVMAI_FAST(32, 1, 2, 4);
-        if (chunks == 32 && variant / 10 == 4) NVMAI_FAST(32, 1, 4, 4);
-        if (chunks == 32) NVMAI_FAST(32, 1, 2, 8);
+        // short rows: everything a wave reads is requested up front, more waves are resident
+        if (chunks == 16) NVMAI_FAST(16, 1, 2, 2);
+        if (chunks == 32) NVMAI_FAST(32, 1, 4, 2);
         if (chunks == 64) NVMAI_FAST(64, 1, 2, 4);
         if (chunks == 128) NVMAI_FAST(64, 2, 1, 8);
     }

@@ -52,6 +52,15 @@ int group_slots(nvmai_hip_ctx* ctx, hipStream_t s, const uint32_t* slot_expert, 
     if (n_blocks)
         prefill_hist_kernel<<<n_blocks, 256, num_experts * 4, s>>>(slot_expert, n_pairs, num_experts, block_hist, words,
                                                                   report_range);
+    if (n_blocks && n_blocks <= FUSED_MAX_BLOCKS && num_experts <= FUSED_MAX_EXPERTS) {
+        uint32_t id_bits = 0;
+        while ((1u << id_bits) < num_experts) ++id_bits;
+        prefill_scan_scatter_kernel<<<n_blocks, 256, (12 * num_experts + 8) * 4, s>>>(
+            slot_expert, w32, w16, n_pairs, top_k, num_experts, id_bits, block_hist, n_blocks, sort_keys, tile_expert_count,
+            out->expert_offsets, out->expert_counts, reinterpret_cast<PrefillGroup*>(out->groups),
+            reinterpret_cast<PrefillTile*>(out->tiles), words, out->info, reinterpret_cast<PrefillPair*>(out->sorted_pairs));
+        return launch_status();
+    }
     prefill_scan_kernel<<<1, 1024, (5 * num_experts + 32) * 4, s>>>(
         block_hist, block_base, n_blocks, num_experts, sort_keys, tile_expert_count, out->expert_offsets, out->expert_counts,
         reinterpret_cast<PrefillGroup*>(out->groups), reinterpret_cast<PrefillTile*>(out->tiles), words, out->info);
@@ -171,7 +180,8 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
         (uint64_t)d * f * bits / 8 > 0xFFFFFFFFull)
         return NVMAI_ERR_UNSUPPORTED;
     if (n_pairs == 0) return NVMAI_OK;
-    const uint32_t max_mtiles = (uint32_t)(n_pairs / GEMM_BM) + (num_experts < n_pairs ? num_experts : (uint32_t)n_pairs);
+    // full tiles + one remainder per expert + the padding of the list's last long and short rows
+    const uint32_t max_mtiles = (uint32_t)(n_pairs / GEMM_BM) + (num_experts < n_pairs ? num_experts : (uint32_t)n_pairs) + 14;
     rc = ws_begin(ctx, ws_round((size_t)max_mtiles * sizeof(MTile)) + ws_round(64));
     if (rc) return rc;
     MTile* mtiles = ws_take<MTile>(ctx, max_mtiles);

@@ -239,31 +239,231 @@ __global__ __launch_bounds__(256) void prefill_scatter_kernel(const uint32_t* id
     }
 }
 
+// ---- passes 2 and 3 in one launch, for inputs whose histogram is small -----------------------
+// Every block repeats the scan over experts for itself (a few thousand additions), so nothing
+// waits for a one-block launch in between: the block's first sorted slot of expert e is the
+// expert's first slot plus the pairs of e in earlier blocks.  Block 0 also writes what the scan
+// pass writes.  Inside a block wave w places slots [256 w, 256 w + 256) of the chunk, 64 at a
+// time; a lane's place among the lanes of the same expert comes from one ballot per bit of the
+// expert id, and per-wave counters carry it from one 64 to the next, so the four waves never
+// wait for each other and every expert keeps (token, rank) ascending.
+constexpr uint32_t FUSED_MAX_EXPERTS = 512, FUSED_MAX_BLOCKS = 64;
+
+// Exclusive scan over the 256 threads of the block; `total` is the sum over all of them.
+__device__ __forceinline__ uint32_t block256_excl_scan(uint32_t v, uint32_t* wave_tot, uint32_t& total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t inc = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t t = (uint32_t)__shfl_up((int)inc, off, 64);
+        if (lane >= off) inc += t;
+    }
+    if (lane == 63) wave_tot[wave] = inc;
+    __syncthreads();
+    uint32_t before = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t t = wave_tot[w];
+        before += w < wave ? t : 0u;
+        tot += t;
+    }
+    __syncthreads();
+    total = tot;
+    return before + inc - v;
+}
+
+__global__ __launch_bounds__(256) void prefill_scan_scatter_kernel(
+    const uint32_t* __restrict__ idx, const uint32_t* __restrict__ w32, const uint16_t* __restrict__ w16,
+    uint32_t n_pairs, uint32_t top_k, uint32_t num_experts, uint32_t id_bits,
+    const uint32_t* __restrict__ block_hist, uint32_t n_blocks, const uint64_t* __restrict__ sort_keys,
+    uint32_t tile_expert_count, uint32_t* offsets, uint32_t* counts, PrefillGroup* groups, PrefillTile* tiles,
+    uint32_t* err_word, uint32_t* info, PrefillPair* sorted) {
+    extern __shared__ uint32_t lds[];
+    const uint32_t E = num_experts;
+    uint32_t* cnt = lds;                 // [E] pairs of expert e
+    uint32_t* before = lds + E;          // [E] of them in earlier blocks
+    uint32_t* order = lds + 2 * E;       // [E] expert at position i of the key order
+    uint32_t* start = lds + 3 * E;       // [E] first pair of expert e
+    uint32_t* gstart = lds + 4 * E;      // [E] first pair of group g
+    uint32_t* gcount = lds + 5 * E;      // [E] pairs of group g
+    uint32_t* wnext = lds + 6 * E;       // [4][E] per wave: pairs of e, then next free slot of e
+    uint32_t* misc = lds + 10 * E;       // [0..3] wave totals, [4] largest group
+    uint64_t* keys = reinterpret_cast<uint64_t*>(lds + 10 * E + 8);   // [E]
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) misc[4] = 0;
+    for (uint32_t e = tid; e < E; e += 256) {
+        uint32_t total = 0, earlier = 0;
+        for (uint32_t b0 = 0; b0 < n_blocks; b0 += 8) {
+            uint32_t c[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) c[j] = b0 + j < n_blocks ? block_hist[(size_t)(b0 + j) * E + e] : 0u;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                total += c[j];
+                earlier += b0 + j < blockIdx.x ? c[j] : 0u;
+            }
+        }
+        cnt[e] = total;
+        before[e] = earlier;
+        if (sort_keys) keys[e] = sort_keys[e];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) wnext[w * E + e] = 0;
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < E; e += 256) {
+        uint32_t pos = e;
+        if (sort_keys) {                                          // rank in (key, expert) order
+            pos = 0;
+            const uint64_t my_key = keys[e];
+            for (uint32_t o = 0; o < E; ++o) {
+                const uint64_t k = keys[o];
+                pos += (k < my_key || (k == my_key && o < e)) ? 1u : 0u;
+            }
+        }
+        order[pos] = e;
+    }
+    __syncthreads();
+    uint32_t pair_carry = 0, group_carry = 0;
+    for (uint32_t base = 0; base < E; base += 256) {              // uniform trip count
+        const uint32_t i = base + tid;
+        const uint32_t ex = i < E ? order[i] : 0u;
+        const uint32_t c = i < E ? cnt[ex] : 0u;
+        uint32_t pair_total, group_total;
+        const uint32_t first = pair_carry + block256_excl_scan(c, misc, pair_total);
+        const uint32_t g = group_carry + block256_excl_scan(c ? 1u : 0u, misc, group_total);
+        if (i < E) start[ex] = first;
+        if (c) {
+            gstart[g] = first;
+            gcount[g] = c;
+            if (blockIdx.x == 0) {
+                groups[g] = PrefillGroup{ex, first, c};
+                atomicMax(&misc[4], c);
+            }
+        }
+        pair_carry += pair_total;
+        group_carry += group_total;
+    }
+    // ---- this block's slots: the lane's four, counted per wave
+    const uint32_t base = blockIdx.x * GROUP_CHUNK + wave * 256 + lane;
+    uint32_t ex[4], wbits[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t p = base + r * 64;
+        ex[r] = p < n_pairs ? idx[p] : 0xFFFFFFFFu;
+        wbits[r] = ex[r] < E ? (w32 ? w32[p] : (uint32_t)w16[p]) : 0u;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+        if (ex[r] < E) atomicAdd(&wnext[wave * E + ex[r]], 1u);
+    __syncthreads();
+    if (blockIdx.x == 0) {                                        // what the scan pass reports
+        const uint32_t ng = group_carry;
+        const uint32_t nt = (ng + tile_expert_count - 1) / tile_expert_count;
+        for (uint32_t t = tid; t < nt; t += 256) {
+            const uint32_t gs = t * tile_expert_count, ge = min(ng, gs + tile_expert_count);
+            tiles[t] = PrefillTile{gs, ge - gs, gstart[gs], gstart[ge - 1] + gcount[ge - 1] - gstart[gs]};
+        }
+        if (tid == 0) {
+            const uint32_t err = *err_word;        // 0 = none, else ~(index << 4 | code)
+            *err_word = 0;
+            info[0] = ng;
+            info[1] = nt;
+            info[2] = err ? (~err & 15u) : 0u;
+            info[3] = err ? (~err >> 4) : 0u;
+            info[4] = misc[4];
+        }
+        for (uint32_t e = tid; e < E; e += 256) {
+            counts[e] = cnt[e];
+            offsets[e] = cnt[e] ? start[e] : 0xFFFFFFFFu;
+        }
+    }
+    for (uint32_t e = tid; e < E; e += 256) {
+        uint32_t run = start[e] + before[e];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t c = wnext[w * E + e];
+            wnext[w * E + e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t e = ex[r];
+        const bool valid = e < E;
+        unsigned long long same = __ballot(valid);
+        for (uint32_t i = 0; i < id_bits; ++i) {
+            const bool bit = (e >> i) & 1u;
+            const unsigned long long b = __ballot(valid && bit);
+            same &= bit ? b : ~b;
+        }
+        if (valid) {
+            const uint32_t rank = (uint32_t)__builtin_popcountll(same & ((1ull << lane) - 1ull));
+            const uint32_t p = base + r * 64;
+            const uint32_t pos = wnext[wave * E + e] + rank;       // every lane reads before the first one adds
+            sorted[pos] = PrefillPair{p / top_k, e, p % top_k, wbits[r]};
+            if (rank == 0) wnext[wave * E + e] += (uint32_t)__builtin_popcountll(same);
+        }
+    }
+}
+
 // ---- M tiles of the grouped GEMM ----------------------------------------------------------
 struct MTile { uint32_t expert, row_start, rows; };
 constexpr int GEMM_BM = 128;
 
-// One block: cuts every group into runs of at most GEMM_BM sorted pairs, largest groups first
-// in four coarse classes so that long experts start early.
+constexpr uint32_t GEMM_SHORT_ROWS = 32;   // M tiles of at most this many rows take the kernel's short body
+
+// One block: cuts every group into runs of at most GEMM_BM sorted pairs and orders the runs for
+// the GEMM grid.  Long tiles are bound by instruction issue, short ones (a whole expert streamed
+// for a few rows) by memory, so the two kinds are interleaved: both then share every compute
+// unit for the whole launch instead of taking it in turns.  The list is made of rows of eight
+// tiles of one kind, because the grid deals consecutive tiles to the eight XCDs, and a kind's
+// rows are spread evenly among the other's (first row long, last row short); rows are padded
+// with empty tiles.  Long tiles keep their groups' order by size (four coarse classes, largest
+// first) so that the experts with the most tiles start early.
+// n_mtiles <= pairs / GEMM_BM + groups + 14.
 __global__ __launch_bounds__(256) void prefill_mtiles_kernel(const PrefillGroup* groups, const uint32_t* info,
                                                             MTile* mtiles, uint32_t* n_mtiles) {
-    __shared__ uint32_t cursor;
-    if (threadIdx.x == 0) cursor = 0;
+    __shared__ uint32_t n_long, n_short, cur_long, cur_short;
+    if (threadIdx.x == 0) { n_long = 0; n_short = 0; cur_long = 0; cur_short = 0; }
     __syncthreads();
     const uint32_t ng = info[2] ? 0u : info[0];               // nothing runs on a grouping that failed
+    uint32_t my_long = 0, my_short = 0;
+    for (uint32_t g = threadIdx.x; g < ng; g += 256) {
+        const uint32_t c = groups[g].pair_count;
+        const uint32_t t = (c + GEMM_BM - 1) / GEMM_BM, last = c - (t - 1) * GEMM_BM;
+        my_long += t - 1 + (last > GEMM_SHORT_ROWS ? 1u : 0u);
+        my_short += last > GEMM_SHORT_ROWS ? 0u : 1u;
+    }
+    if (my_long) atomicAdd(&n_long, my_long);
+    if (my_short) atomicAdd(&n_short, my_short);
+    __syncthreads();
+    const uint32_t L = n_long, S = n_short;
+    const uint32_t lr = (L + 7) / 8, sr = (S + 7) / 8, rows = lr + sr;
+    // position of the i-th long / short tile: row a of lr long rows sits at floor(a * rows / lr),
+    // row b of sr short rows at ceil((b + 1) * rows / sr) - 1; the two sets partition 0..rows-1
+    auto long_at = [&](uint32_t i) { return (uint32_t)((uint64_t)(i / 8) * rows / lr) * 8 + i % 8; };
+    auto short_at = [&](uint32_t j) { return (uint32_t)(((uint64_t)(j / 8 + 1) * rows + sr - 1) / sr - 1) * 8 + j % 8; };
+    for (uint32_t i = L + threadIdx.x; i < lr * 8; i += 256) mtiles[long_at(i)] = MTile{0, 0, 0};
+    for (uint32_t j = S + threadIdx.x; j < sr * 8; j += 256) mtiles[short_at(j)] = MTile{0, 0, 0};
     for (int cls = 3; cls >= 0; --cls) {
         for (uint32_t g = threadIdx.x; g < ng; g += 256) {
             const PrefillGroup gr = groups[g];
             const uint32_t t = (gr.pair_count + GEMM_BM - 1) / GEMM_BM;
             const int my = t >= 16 ? 3 : t >= 4 ? 2 : t >= 2 ? 1 : 0;
             if (my != cls) continue;
-            const uint32_t at = atomicAdd(&cursor, t);
-            for (uint32_t j = 0; j < t; ++j)
-                mtiles[at + j] = MTile{gr.expert, gr.pair_start + j * GEMM_BM, min((uint32_t)GEMM_BM, gr.pair_count - j * GEMM_BM)};
+            const uint32_t last = gr.pair_count - (t - 1) * GEMM_BM;
+            const bool last_long = last > GEMM_SHORT_ROWS;
+            const uint32_t nl = t - 1 + (last_long ? 1u : 0u);
+            const uint32_t at = nl ? atomicAdd(&cur_long, nl) : 0u;
+            for (uint32_t j = 0; j < nl; ++j)
+                mtiles[long_at(at + j)] = MTile{gr.expert, gr.pair_start + j * GEMM_BM, min((uint32_t)GEMM_BM, gr.pair_count - j * GEMM_BM)};
+            if (!last_long)
+                mtiles[short_at(atomicAdd(&cur_short, 1u))] = MTile{gr.expert, gr.pair_start + (t - 1) * GEMM_BM, last};
         }
         __syncthreads();
     }
-    if (threadIdx.x == 0) *n_mtiles = cursor;
+    if (threadIdx.x == 0) *n_mtiles = rows * 8;
 }
 
 // ---- grouped GEMM ---------------------------------------------------------------------------
@@ -419,6 +619,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     const uint32_t nt = (unit % p.units_per_tile) * GEMM_UNIT + on_xcd % GEMM_UNIT;
     if (tile_id >= *p.n_mtiles || nt >= p.n_tiles_n) return;
     const MTile mt = p.mtiles[tile_id];
+    if (mt.rows == 0) return;                           // padding of the tile list
     const uint8_t* blob = p.pool + (uint64_t)mt.expert * p.pool_stride;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
