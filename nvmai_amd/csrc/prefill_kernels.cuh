@@ -424,44 +424,56 @@ constexpr uint32_t GEMM_SHORT_ROWS = 32;   // M tiles of at most this many rows 
 // n_mtiles <= pairs / GEMM_BM + groups + 14.
 __global__ __launch_bounds__(256) void prefill_mtiles_kernel(const PrefillGroup* groups, const uint32_t* info,
                                                             MTile* mtiles, uint32_t* n_mtiles) {
-    __shared__ uint32_t n_long, n_short, cur_long, cur_short;
-    if (threadIdx.x == 0) { n_long = 0; n_short = 0; cur_long = 0; cur_short = 0; }
+    __shared__ uint32_t cls_long[4], cur_long[4], n_short, cur_short;
+    if (threadIdx.x < 4) { cls_long[threadIdx.x] = 0; cur_long[threadIdx.x] = 0; }
+    if (threadIdx.x == 0) { n_short = 0; cur_short = 0; }
     __syncthreads();
     const uint32_t ng = info[2] ? 0u : info[0];               // nothing runs on a grouping that failed
-    uint32_t my_long = 0, my_short = 0;
+    // a group's tiles: t - 1 full ones and a last one of `last` rows; its class by t
+    auto shape = [](const PrefillGroup& gr, uint32_t& t, uint32_t& last, uint32_t& nl, int& cls) {
+        t = (gr.pair_count + GEMM_BM - 1) / GEMM_BM;
+        last = gr.pair_count - (t - 1) * GEMM_BM;
+        nl = t - 1 + (last > GEMM_SHORT_ROWS ? 1u : 0u);
+        cls = t >= 16 ? 3 : t >= 4 ? 2 : t >= 2 ? 1 : 0;
+    };
+    // the first 256 groups (usually all of them) are read once and stay in registers
+    PrefillGroup first_gr{0, 0, 0};
+    if (threadIdx.x < ng) first_gr = groups[threadIdx.x];
     for (uint32_t g = threadIdx.x; g < ng; g += 256) {
-        const uint32_t c = groups[g].pair_count;
-        const uint32_t t = (c + GEMM_BM - 1) / GEMM_BM, last = c - (t - 1) * GEMM_BM;
-        my_long += t - 1 + (last > GEMM_SHORT_ROWS ? 1u : 0u);
-        my_short += last > GEMM_SHORT_ROWS ? 0u : 1u;
+        const PrefillGroup gr = g < 256 ? first_gr : groups[g];
+        uint32_t t, last, nl; int cls;
+        shape(gr, t, last, nl, cls);
+        if (nl) atomicAdd(&cls_long[cls], nl);
+        if (nl != t) atomicAdd(&n_short, 1u);
     }
-    if (my_long) atomicAdd(&n_long, my_long);
-    if (my_short) atomicAdd(&n_short, my_short);
     __syncthreads();
-    const uint32_t L = n_long, S = n_short;
+    const uint32_t base3 = 0, base2 = cls_long[3], base1 = base2 + cls_long[2], base0 = base1 + cls_long[1];
+    const uint32_t L = base0 + cls_long[0], S = n_short;
     const uint32_t lr = (L + 7) / 8, sr = (S + 7) / 8, rows = lr + sr;
     // position of the i-th long / short tile: row a of lr long rows sits at floor(a * rows / lr),
     // row b of sr short rows at ceil((b + 1) * rows / sr) - 1; the two sets partition 0..rows-1
-    auto long_at = [&](uint32_t i) { return (uint32_t)((uint64_t)(i / 8) * rows / lr) * 8 + i % 8; };
-    auto short_at = [&](uint32_t j) { return (uint32_t)(((uint64_t)(j / 8 + 1) * rows + sr - 1) / sr - 1) * 8 + j % 8; };
+    const bool small = rows <= 0xFFFFu;                           // 32-bit products suffice
+    auto long_at = [&](uint32_t i) {
+        const uint32_t a = i / 8;
+        return (small ? a * rows / lr : (uint32_t)((uint64_t)a * rows / lr)) * 8 + i % 8;
+    };
+    auto short_at = [&](uint32_t j) {
+        const uint32_t b1 = j / 8 + 1;
+        return (small ? (b1 * rows + sr - 1) / sr - 1 : (uint32_t)(((uint64_t)b1 * rows + sr - 1) / sr - 1)) * 8 + j % 8;
+    };
     for (uint32_t i = L + threadIdx.x; i < lr * 8; i += 256) mtiles[long_at(i)] = MTile{0, 0, 0};
     for (uint32_t j = S + threadIdx.x; j < sr * 8; j += 256) mtiles[short_at(j)] = MTile{0, 0, 0};
-    for (int cls = 3; cls >= 0; --cls) {
-        for (uint32_t g = threadIdx.x; g < ng; g += 256) {
-            const PrefillGroup gr = groups[g];
-            const uint32_t t = (gr.pair_count + GEMM_BM - 1) / GEMM_BM;
-            const int my = t >= 16 ? 3 : t >= 4 ? 2 : t >= 2 ? 1 : 0;
-            if (my != cls) continue;
-            const uint32_t last = gr.pair_count - (t - 1) * GEMM_BM;
-            const bool last_long = last > GEMM_SHORT_ROWS;
-            const uint32_t nl = t - 1 + (last_long ? 1u : 0u);
-            const uint32_t at = nl ? atomicAdd(&cur_long, nl) : 0u;
+    for (uint32_t g = threadIdx.x; g < ng; g += 256) {
+        const PrefillGroup gr = g < 256 ? first_gr : groups[g];
+        uint32_t t, last, nl; int cls;
+        shape(gr, t, last, nl, cls);
+        if (nl) {
+            const uint32_t at = (cls == 3 ? base3 : cls == 2 ? base2 : cls == 1 ? base1 : base0) + atomicAdd(&cur_long[cls], nl);
             for (uint32_t j = 0; j < nl; ++j)
                 mtiles[long_at(at + j)] = MTile{gr.expert, gr.pair_start + j * GEMM_BM, min((uint32_t)GEMM_BM, gr.pair_count - j * GEMM_BM)};
-            if (!last_long)
-                mtiles[short_at(atomicAdd(&cur_short, 1u))] = MTile{gr.expert, gr.pair_start + (t - 1) * GEMM_BM, last};
         }
-        __syncthreads();
+        if (nl != t)
+            mtiles[short_at(atomicAdd(&cur_short, 1u))] = MTile{gr.expert, gr.pair_start + (t - 1) * GEMM_BM, last};
     }
     if (threadIdx.x == 0) *n_mtiles = rows * 8;
 }

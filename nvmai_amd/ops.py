@@ -288,7 +288,7 @@ class PrefillMoEGroupedRoutes:
         self.per_expert_counts = torch.empty(num_experts, **i32)
         self.groups_buf = torch.empty((num_experts, 3), **i32)
         self.tiles_buf = torch.empty((num_experts, 4), **i32)
-        self.info = torch.zeros(8, **i32)
+        self.info = torch.empty(8, **i32)           # words 0..4 are written by every grouping call
         self.desc = PrefillGrouping(*(t.data_ptr() for t in (self.sorted_pairs, self.per_expert_offsets,
                                                              self.per_expert_counts, self.groups_buf,
                                                              self.tiles_buf, self.info)))
