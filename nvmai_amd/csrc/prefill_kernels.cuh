@@ -1074,10 +1074,136 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         }
         epilogue(mtc, acc);
     };
+    // ---- short tiles whose scales and biases fit the second activation array: rows of scales
+    // that are a multiple of 16 bytes (K a multiple of 512) and at most 16 KB per array for the
+    // block's columns.  Fetched lane by lane the scales arrive 16 bytes from each of 64 rows per
+    // instruction; here each wave fetches the whole rows of its 16 NT columns once, contiguously,
+    // into a table in LDS, and a super-step reads its dword (two groups) per tile from there.
+    // The activations then alternate between the first activation array and the weight stage
+    // array (fetched one super-step ahead); the weights keep their ring of three register stages.
+    auto run_short_tab = [&](auto mtc) {
+        constexpr int MT = decltype(mtc)::value;
+        fl4_t acc[MT][NT];
+#pragma unroll
+        for (int a = 0; a < MT; ++a)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) acc[a][t] = fl4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        const uint32_t g2 = groups * 2u;                    // bytes per row of scales
+        uint8_t* tab_s = xs1;
+        uint8_t* tab_b = xs1 + GEMM_XBUF / 2;
+        {
+            const uint32_t ppr = g2 / 16u, total = NT * 16u * ppr;      // 16-byte pieces per row, per wave
+            for (uint32_t i = 0; i * 64u < total; ++i) {
+                const uint32_t q = i * 64u + lane;
+                const uint32_t row = q / ppr, piece = q % ppr;          // row = 16 t + column of the tile
+                const uint32_t t = row >> 4, c16 = row & 15u;
+                uint32_t c = DUAL ? n0 + wave * (8 * NT) + (t >> 1) * 16 + c16 : n0 + wave * (16 * NT) + t * 16 + c16;
+                c = min(c, p.N - 1) * g2 + piece * 16u;
+                const uint32_t so = (DUAL ? (uint32_t)((t & 1) ? p.sB : p.sA) : 0u) + c;
+                const uint32_t bo = (DUAL ? (uint32_t)((t & 1) ? p.bB : p.bA) : 0u) + c;
+                const uint32_t at = wave * (NT * 16u) * g2 + i * 1024u;
+                if (q < total) {
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(s_rs, (__attribute__((address_space(3))) void*)(tab_s + at), 16, so, 0, 0, 0);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rs, (__attribute__((address_space(3))) void*)(tab_b + at), 16, bo, 0, 0, 0);
+                }
+            }
+        }
+        const uint32_t tb = (wave * (NT * 16u) + li) * g2;  // the lane's column of tile 0 in the tables
+        auto fetch_sb = [&](uint32_t ss, uint32_t* ds, uint32_t* db) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                ds[t] = *reinterpret_cast<const uint32_t*>(tab_s + tb + t * 16u * g2 + ss * 4u);
+                db[t] = *reinterpret_cast<const uint32_t*>(tab_b + tb + t * 16u * g2 + ss * 4u);
+            }
+        };
+        auto pack_sb = [&](const uint32_t* ds, const uint32_t* db, uint32_t* sb) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                sb[t] = (lq >> 1) ? __builtin_amdgcn_perm(ds[t], db[t], 0x07060302u)
+                                  : __builtin_amdgcn_perm(ds[t], db[t], 0x05040100u);
+        };
+        uint32_t xo;                                        // the lane's row of the wave's tile
+        {
+            const uint32_t row = ((wave * MT) >> 2) * 16 + (lane >> 2);
+            const uint32_t m = row < mt.rows ? row : 0;
+            const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
+            xo = src * (p.x_stride * 2u) + (uint32_t)((lane & 3) ^ gemm_row_swizzle(lane >> 2)) * 16u;
+        }
+        auto load_xs = [&](uint32_t ss, uint8_t* stage) {
+#pragma unroll
+            for (int e = 0; e < MT; ++e) {
+                const uint32_t q = wave * MT + e;
+                uint8_t* dst = stage + (q >> 2) * 4096 + (q & 3) * 1024;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (__attribute__((address_space(3))) void*)dst, 16, xo,
+                                                         ss * (GEMM_SK * 2) + (q & 3) * 64, 0, 0);
+            }
+        };
+        struct WReg { uint4 w[NT][WQ]; };
+        WReg wr[3];
+        auto load_wr = [&](WReg& g, uint32_t ss) {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const uint32_t so = wso[t] + ss * (GEMM_SK * BITS / 8);
+#pragma unroll
+                for (int h = 0; h < WQ; ++h) {
+                    const u32x4_t w = __builtin_amdgcn_raw_buffer_load_b128((DUAL && (t & 1)) ? wrsB : wrsA, wv + 16 * h, so, 0);
+                    g.w[t][h] = uint4{w.x, w.y, w.z, w.w};
+                }
+            }
+        };
+        constexpr int LW = NT * WQ;                         // weight loads of a super-step
+        uint4 bf[2][NT];
+        uint32_t sb[NT];
+        load_xs(0, xs0);
+        load_wr(wr[0], 0);
+        if (nss > 1) load_wr(wr[1], 1);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        {
+            uint32_t ds[NT], db[NT];
+            fetch_sb(0, ds, db);
+            pack_sb(ds, db, sb);
+        }
+        dequant_step(wr[0].w, sb, 0, bf[0]);
+        // one super-step: multiplies stage `cur` from weights `wc`; stage `nxt` takes the next
+        // super-step's activations, `wf` the weights needed two super-steps on; `wn` are the
+        // weights of the next super-step
+        auto superstep = [&](uint32_t ss, const uint8_t* cur, uint8_t* nxt, const WReg& wc, const WReg& wn, WReg& wf) {
+            if (ss + 1 < nss) load_xs(ss + 1, nxt);
+            if (ss + 2 < nss) load_wr(wf, ss + 2);
+            uint32_t ds[NT], db[NT];
+            if (ss + 1 < nss) fetch_sb(ss + 1, ds, db);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (j < 3) dequant_step(wc.w, sb, j + 1, bf[(j + 1) & 1]);
+                else if (ss + 1 < nss) {
+                    pack_sb(ds, db, sb);
+                    dequant_step(wn.w, sb, 0, bf[0]);
+                }
+                mfma_step(mtc, acc, cur, j, bf[j & 1]);
+            }
+            // the next activation stage was requested at the top; only the LW weight requests
+            // that followed it may still be under way
+            if (ss + 2 < nss) __builtin_amdgcn_s_waitcnt(gemm_vmcnt(LW));
+            else __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+        };
+        for (uint32_t ss = 0; ss < nss; ss += 6) {
+            superstep(ss, xs0, ws, wr[0], wr[1], wr[2]);
+            if (ss + 1 < nss) superstep(ss + 1, ws, xs0, wr[1], wr[2], wr[0]);
+            if (ss + 2 < nss) superstep(ss + 2, xs0, ws, wr[2], wr[0], wr[1]);
+            if (ss + 3 < nss) superstep(ss + 3, ws, xs0, wr[0], wr[1], wr[2]);
+            if (ss + 4 < nss) superstep(ss + 4, xs0, ws, wr[1], wr[2], wr[0]);
+            if (ss + 5 < nss) superstep(ss + 5, ws, xs0, wr[2], wr[0], wr[1]);
+        }
+        epilogue(mtc, acc);
+    };
+    // K a multiple of 512 has no half super-step at the end either
+    const bool tab_ok = (groups % 8u) == 0 && 64u * NT * groups * 2u <= GEMM_XBUF / 2;
     if (live_mt > 4) run_full(std::integral_constant<int, 8>{});
     else if (live_mt > 2) run_full(std::integral_constant<int, 4>{});
-    else if (live_mt > 1) run_short(std::integral_constant<int, 2>{});
-    else run_short(std::integral_constant<int, 1>{});
+    else if (live_mt > 1) { if (tab_ok) run_short_tab(std::integral_constant<int, 2>{}); else run_short(std::integral_constant<int, 2>{}); }
+    else { if (tab_ok) run_short_tab(std::integral_constant<int, 1>{}); else run_short(std::integral_constant<int, 1>{}); }
 }
 
 // Work list of a dense product y = x . W^T: M tiles of 128 consecutive rows of one "expert" 0,
