@@ -151,8 +151,10 @@ def _zipf_routes(rng, tokens, E, k, s=1.1):
     return idx, O.f16_bits(w)
 
 
+# (300, 600, ..) and (9000, 64, ..) take the three-launch path (more than 512 experts, more than 64
+# histogram blocks), the others the fused scan + scatter launch
 @pytest.mark.parametrize("tokens,E,k,tile", [(1, 8, 2, 16), (37, 20, 3, 4), (1000, 256, 8, 16), (4096, 256, 8, 16),
-                                             (300, 600, 4, 7)])
+                                             (300, 600, 4, 7), (9000, 64, 8, 16), (8100, 512, 8, 16)])
 def test_grouping_random_routes_bit_exact(nv, ctx_bf16, tokens, E, k, tile):
     say("prefill grouping random", tokens, E, k, tile)
     rng = np.random.default_rng(tokens * 31 + E)
