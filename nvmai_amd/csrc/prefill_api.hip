@@ -240,21 +240,15 @@ extern "C" int nvmai_hip_affine_qmm(nvmai_hip_ctx* ctx, nvmai_stream stream, con
     if ((uint64_t)m * x_stride * 2 > 0xFFFFFFFFull || (uint64_t)n * k * bits / 8 > 0xFFFFFFFFull)
         return NVMAI_ERR_UNSUPPORTED;
     const uint32_t tiles = (m + GEMM_BM - 1) / GEMM_BM;
-    int rc = ws_begin(ctx, ws_round((size_t)tiles * sizeof(MTile)) + ws_round(64) + ws_round((size_t)m * sizeof(PrefillPair)));
-    if (rc) return rc;
-    MTile* mtiles = ws_take<MTile>(ctx, tiles);
-    uint32_t* n_mtiles = ws_take<uint32_t>(ctx, 16);
-    PrefillPair* pairs = ws_take<PrefillPair>(ctx, m);
     hipStream_t s = (hipStream_t)stream;
     ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM2, s);
-    qmm_setup_kernel<<<(m + 255) / 256, 256, 0, s>>>(m, mtiles, n_mtiles, pairs);
     const uint32_t nt = bits == 4 ? 4 : 2;
     GemmParams g{};
     g.pool = weights; g.pool_stride = 0;
     g.wA = 0;
     g.sA = reinterpret_cast<const uint8_t*>(scales) - weights;
     g.bA = reinterpret_cast<const uint8_t*>(biases) - weights;
-    g.mtiles = mtiles; g.n_mtiles = n_mtiles; g.pairs = pairs;
+    g.dense_rows = m;                           // the kernel cuts the rows into M tiles itself
     g.x = x; g.x_stride = x_stride; g.out = y; g.out_stride = y_stride;
     g.K = k; g.N = n; g.top_k = 1; g.n_tiles_n = (n + 64 * nt - 1) / (64 * nt);
     g.units_per_tile = (g.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;

@@ -512,6 +512,8 @@ struct GemmParams {
     uint32_t out_stride;
     uint32_t K, N, top_k, n_tiles_n;
     uint32_t units_per_tile;            // ceil(n_tiles_n / GEMM_UNIT)
+    uint32_t dense_rows;                // > 0: a dense product over rows 0..dense_rows-1 of x (row i -> row i of
+                                        // out), M tiles of GEMM_BM consecutive rows; mtiles, n_mtiles, pairs unused
 };
 
 constexpr int GEMM_SK = 128;            // k per super-step
@@ -629,9 +631,15 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     const uint32_t unit = (on_xcd / GEMM_UNIT) * 8 + (blockIdx.x & 7u);
     const uint32_t tile_id = unit / p.units_per_tile;
     const uint32_t nt = (unit % p.units_per_tile) * GEMM_UNIT + on_xcd % GEMM_UNIT;
-    if (tile_id >= *p.n_mtiles || nt >= p.n_tiles_n) return;
-    const MTile mt = p.mtiles[tile_id];
-    if (mt.rows == 0) return;                           // padding of the tile list
+    MTile mt;
+    if (!DUAL && p.dense_rows) {
+        if (tile_id * GEMM_BM >= p.dense_rows || nt >= p.n_tiles_n) return;
+        mt = MTile{0u, tile_id * GEMM_BM, min((uint32_t)GEMM_BM, p.dense_rows - tile_id * GEMM_BM)};
+    } else {
+        if (tile_id >= *p.n_mtiles || nt >= p.n_tiles_n) return;
+        mt = p.mtiles[tile_id];
+        if (mt.rows == 0) return;                       // padding of the tile list
+    }
     const uint8_t* blob = p.pool + (uint64_t)mt.expert * p.pool_stride;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -890,8 +898,11 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         // inside the store loop each one would be a dependent global load.
         uint32_t* orow_tab = reinterpret_cast<uint32_t*>(xs1);
         if (!DUAL && (uint32_t)tid < mt.rows) {
-            const PrefillPair pr = p.pairs[mt.row_start + tid];
-            orow_tab[tid] = pr.token * p.top_k + pr.rank;
+            if (p.dense_rows) orow_tab[tid] = mt.row_start + tid;
+            else {
+                const PrefillPair pr = p.pairs[mt.row_start + tid];
+                orow_tab[tid] = pr.token * p.top_k + pr.rank;
+            }
         }
 #pragma unroll
         for (int a0 = 0; a0 < MT; a0 += AP) {
@@ -1204,17 +1215,6 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     else if (live_mt > 2) run_full(std::integral_constant<int, 4>{});
     else if (live_mt > 1) { if (tab_ok) run_short_tab(std::integral_constant<int, 2>{}); else run_short(std::integral_constant<int, 2>{}); }
     else { if (tab_ok) run_short_tab(std::integral_constant<int, 1>{}); else run_short(std::integral_constant<int, 1>{}); }
-}
-
-// Work list of a dense product y = x . W^T: M tiles of 128 consecutive rows of one "expert" 0,
-// identity pair records (row i -> output row i).
-__global__ __launch_bounds__(256) void qmm_setup_kernel(uint32_t m, MTile* mtiles, uint32_t* n_mtiles,
-                                                       PrefillPair* pairs) {
-    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-    if (i < m) pairs[i] = PrefillPair{i, 0u, 0u, 0u};
-    const uint32_t tiles = (m + GEMM_BM - 1) / GEMM_BM;
-    if (i < tiles) mtiles[i] = MTile{0u, i * GEMM_BM, min((uint32_t)GEMM_BM, m - i * GEMM_BM)};
-    if (i == 0) *n_mtiles = tiles;
 }
 
 // ---- combine (prefill.metal:437-458) -------------------------------------------------------
