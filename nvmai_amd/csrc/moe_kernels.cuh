@@ -106,9 +106,14 @@ __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float c) {
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), c, false);
 }
 
-// 16 bytes of codes -> packed fp16 pairs (1024 + q).  8 bit: pair m holds the
-// elements (2m, 2m+1).  4 bit: dword d of the chunk yields pairs 4d+j holding the
-// elements (8d+j, 8d+j+4); the staged inputs are packed the same way.
+// 16 bytes of codes -> packed fp16 pairs.  8 bit: pair m holds the elements (2m, 2m+1) as
+// 1024 + q.  4 bit: dword d of the chunk yields pairs 4d+j holding the elements (8d+j, 8d+j+4);
+// the staged inputs are packed the same way.  A nibble at bits 0..3 of a half becomes 1024 + q
+// under 0x6400, a nibble at bits 4..7 becomes 64 + q under 0x5400 (the binade whose fourth
+// mantissa bit weighs one), so the odd pairs need no shift of their own: one shift by 8 and four
+// and-or instructions per dword.  The odd pairs' offset of 64 instead of 1024 is taken back with
+// the sum of the inputs at their positions (ODD_PAIR_OFFSET_GAP).
+constexpr float ODD_PAIR_OFFSET_GAP = 1024.0f - 64.0f;
 template <int BITS>
 __device__ __forceinline__ void unpack_pairs(const uint4& w, uint32_t* qp) {
     const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
@@ -118,8 +123,11 @@ __device__ __forceinline__ void unpack_pairs(const uint4& w, uint32_t* qp) {
             qp[2 * d] = __builtin_amdgcn_perm(ws[d], 0x64646464u, 0x00050004u);
             qp[2 * d + 1] = __builtin_amdgcn_perm(ws[d], 0x64646464u, 0x00070006u);
         } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) qp[4 * d + j] = ((ws[d] >> (4 * j)) & 0x000F000Fu) | 0x64006400u;
+            const uint32_t hi = ws[d] >> 8;
+            qp[4 * d] = (ws[d] & 0x000F000Fu) | 0x64006400u;
+            qp[4 * d + 1] = (ws[d] & 0x00F000F0u) | 0x54005400u;
+            qp[4 * d + 2] = (hi & 0x000F000Fu) | 0x64006400u;
+            qp[4 * d + 3] = (hi & 0x00F000F0u) | 0x54005400u;
         }
     }
 }
@@ -160,7 +168,7 @@ __device__ __forceinline__ void pow2_scale(float amax, float& sc, float& isc) {
 // TOKS = 1: exactly one input, kept in registers for the whole block.  TOKS = 0:
 // we.pair_count inputs (2..MAX_TOK), walked by a real loop inside each stage so
 // that only one input's columns are live at a time.
-// LDS: [ntok][n/8] uint4 packed inputs | [ntok][NCH*SEG] float chunk sums |
+// LDS: [ntok][n/8] uint4 packed inputs | [ntok][NCH*SEG][2] float chunk sums (all, odd pairs) |
 //      [MAX_TOK*4] float wave maxima | [MAX_TOK] float inverse scales.
 template <int ACT, int BITS, int SEG, int NCH, int TOKS, bool DUAL, bool XF32, int RPI, int ITERS>
 __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const WorkEntry& we, uint32_t rb,
@@ -188,7 +196,7 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
     const uint32_t row_base = (rb * 4 + wave) * ROWS_WAVE;
     uint4* xw = lds;
     float* xs_tab = reinterpret_cast<float*>(lds + MAX_TOK * WORDS_TOK);
-    float* wmax_tab = xs_tab + MAX_TOK * NCH * SEG;
+    float* wmax_tab = xs_tab + 2 * MAX_TOK * NCH * SEG;
     float* isc_tab = wmax_tab + MAX_TOK * 4;
 
     auto load_stage = [&](Stage& st, int it) {
@@ -298,18 +306,20 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
     // ---- chunk sums of the converted inputs, one thread per (input, chunk)
     for (int idx = threadIdx.x; idx < ntok * NCH * SEG; idx += 256) {
         const int t = idx / (NCH * SEG), cs = idx % (NCH * SEG), c = cs / SEG, l = cs % SEG;
-        float sum = 0.0f;
+        float sum = 0.0f, odd = 0.0f;                 // odd: the pairs 1, 3, 5, ... of the chunk
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             const uint4 w = xw[t * WORDS_TOK + (c * H + h) * SEG + l];
             const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
-                sum += f16_to_f32((uint16_t)(ws[d] & 0xFFFFu));
-                sum += f16_to_f32((uint16_t)(ws[d] >> 16));
+                const float both = f16_to_f32((uint16_t)(ws[d] & 0xFFFFu)) + f16_to_f32((uint16_t)(ws[d] >> 16));
+                sum += both;
+                if (d & 1) odd += both;
             }
         }
-        xs_tab[t * NCH * SEG + c * SEG + l] = sum;
+        xs_tab[(t * NCH * SEG + c * SEG + l) * 2] = sum;
+        xs_tab[(t * NCH * SEG + c * SEG + l) * 2 + 1] = odd;
     }
     __syncthreads();
 
@@ -325,7 +335,7 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
 #pragma unroll 1
         for (int t = 0; t < ntok; ++t) {
             uint32_t xp[NCH][PAIRS];
-            float xs[NCH];
+            float xs[NCH], xo[NCH];
 #pragma unroll
             for (int c = 0; c < NCH; ++c) {
 #pragma unroll
@@ -333,7 +343,9 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
                     const uint4 w = xw[t * WORDS_TOK + (c * H + h) * SEG + sl];
                     xp[c][4 * h] = w.x; xp[c][4 * h + 1] = w.y; xp[c][4 * h + 2] = w.z; xp[c][4 * h + 3] = w.w;
                 }
-                xs[c] = xs_tab[t * NCH * SEG + c * SEG + sl];
+                const float2 two = *reinterpret_cast<const float2*>(&xs_tab[(t * NCH * SEG + c * SEG + sl) * 2]);
+                xs[c] = two.x;
+                xo[c] = two.y;
             }
             const float isc = isc_tab[t];
             const uint32_t out_row = p.pair_out[we.pair_start + t];
@@ -350,10 +362,12 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
                         if (DUAL) dotB = dot2_acc(qpb[i][c][m], xp[c][m], dotB);
                     }
                     dotA = fmaf(-1024.0f, xs[c], dotA);
+                    if (BITS == 4) dotA = fmaf(ODD_PAIR_OFFSET_GAP, xo[c], dotA);
                     accA = fmaf(bf16_to_f32(st.sa[i][c]), dotA, accA);
                     accA = fmaf(bf16_to_f32(st.ba[i][c]), xs[c], accA);
                     if (DUAL) {
                         dotB = fmaf(-1024.0f, xs[c], dotB);
+                        if (BITS == 4) dotB = fmaf(ODD_PAIR_OFFSET_GAP, xo[c], dotB);
                         accB = fmaf(bf16_to_f32(st.sb[i][c]), dotB, accB);
                         accB = fmaf(bf16_to_f32(st.bb[i][c]), xs[c], accB);
                     }
@@ -381,7 +395,7 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
 
 // Bytes of dynamic LDS the fast engine needs for rows of n codes.
 __host__ __device__ inline size_t rows_fast_lds_bytes(uint32_t n, int nch, int seg) {
-    return (size_t)MAX_TOK * (n / 8) * 16 + (size_t)MAX_TOK * nch * seg * 4 + MAX_TOK * 4 * 4 + MAX_TOK * 4;
+    return (size_t)MAX_TOK * (n / 8) * 16 + (size_t)MAX_TOK * nch * seg * 8 + MAX_TOK * 4 * 4 + MAX_TOK * 4;
 }
 
 // MAXTOK = 1: single-input launches.  MAXTOK = 4: the body is chosen by the
