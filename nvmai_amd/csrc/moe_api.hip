@@ -215,8 +215,36 @@ void run_router_t(const RouterParams& rp, uint32_t cpl, dim3 grid, hipStream_t s
 }
 
 // d <= 2048 dense / 4096 at 8 bit / 8192 at 4 bit (8 chunks per lane).
+template <int ACT>
+void run_router_tiled(const RouterParams& rp, const RowsDesc& r, uint32_t n_rows, float* out, uint32_t out_ld,
+                      hipStream_t s) {
+    const size_t lds = (size_t)RT_TOK * rp.d * 2;
+    const uint32_t per_block = 8 * (r.kind == 4 ? 2 : 4);
+    dim3 grid((n_rows + per_block - 1) / per_block, (rp.tokens + RT_TOK - 1) / RT_TOK);
+#define NVMAI_TILED(KIND)                                                                                    \
+    do {                                                                                                     \
+        if (rp.eff_scale) router_logits_tiled_kernel<ACT, KIND, true><<<grid, 256, lds, s>>>(rp, r, n_rows, out, out_ld);  \
+        else router_logits_tiled_kernel<ACT, KIND, false><<<grid, 256, lds, s>>>(rp, r, n_rows, out, out_ld);  \
+    } while (0)
+    if (r.kind == 16) NVMAI_TILED(16);
+    else if (r.kind == 8) NVMAI_TILED(8);
+    else NVMAI_TILED(4);
+#undef NVMAI_TILED
+}
+
 int run_router(int act, RouterParams& rp, hipStream_t s) {
     rp.x_vec = aligned16(rp.x) && (rp.x_stride % 8 == 0);
+    // Many tokens (a prefill block): the register-tiled kernel, same logits bit for bit
+    if (rp.tokens >= 64 && (size_t)RT_TOK * rp.d * 2 <= 65536) {
+        if (act == ACT_BF16) {
+            run_router_tiled<ACT_BF16>(rp, rp.router, rp.num_experts, rp.logits, rp.num_experts, s);
+            if (rp.gate.kind) run_router_tiled<ACT_BF16>(rp, rp.gate, 1, rp.gate_logit, 1, s);
+        } else {
+            run_router_tiled<ACT_FP16>(rp, rp.router, rp.num_experts, rp.logits, rp.num_experts, s);
+            if (rp.gate.kind) run_router_tiled<ACT_FP16>(rp, rp.gate, 1, rp.gate_logit, 1, s);
+        }
+        return NVMAI_OK;
+    }
     uint32_t chunks = rp.router.kind ? rows_chunks(rp.router.kind, rp.d) : 0;
     if (rp.gate.kind) chunks = chunks > rows_chunks(rp.gate.kind, rp.d) ? chunks : rows_chunks(rp.gate.kind, rp.d);
     const uint32_t cpl = (chunks + 31) / 32;

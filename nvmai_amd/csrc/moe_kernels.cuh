@@ -650,6 +650,122 @@ __global__ __launch_bounds__(256) void router_logits_kernel(RouterParams p) {
     }
 }
 
+// ---- router logits for many tokens ---------------------------------------------------------
+// The same sums in the same order as router_logits_kernel, so the logits are the same bits and
+// the routing does not depend on which kernel ran; only the tiling differs.  A half-wave owns R
+// rows against the block's RT_TOK tokens: a chunk of each row is converted to floats once and
+// then used by every token, and a token's chunk once for the R rows, instead of once per
+// (row, token) pair.  The inputs of the block sit in LDS as stored.  One launch per matrix (the
+// router rows, then the single gate row) because their formats may differ.
+constexpr int RT_TOK = 8;
+
+// EFF: the inputs are multiplied by the bf16 effective scale (a compile-time switch: a branch per
+// token in the loop body makes the compiler convert all sixteen tokens' chunks before the first
+// multiply-add, and the accumulators no longer fit beside them).
+template <int ACT, int KIND, bool EFF>
+__global__ __launch_bounds__(256, KIND == 16 ? 4 : 2) void router_logits_tiled_kernel(RouterParams p, RowsDesc r, uint32_t n_rows,
+                                                                  float* out, uint32_t out_ld) {
+    constexpr int EPC = KIND == 16 ? 8 : (KIND == 8 ? 16 : 32);
+    constexpr int XV = EPC / 8;
+    constexpr int R = KIND == 4 ? 2 : 4;             // rows per half-wave: what the register file holds
+    extern __shared__ uint4 router_lds[];
+    const uint16_t* xl = reinterpret_cast<const uint16_t*>(router_lds);
+    const int hw = threadIdx.x >> 5, hl = threadIdx.x & 31;
+    const uint32_t row0 = (blockIdx.x * 8 + hw) * R;
+    const uint32_t t0 = blockIdx.y * RT_TOK;
+    const uint32_t nt = min((uint32_t)RT_TOK, p.tokens - t0);
+    router_stage_x(p, t0, nt, reinterpret_cast<uint16_t*>(router_lds));
+    if (row0 >= n_rows) return;                      // uniform per half-wave
+    const uint32_t chunks = p.d / EPC;
+    const uint32_t groups = p.d / NVMAI_GROUP;
+    const size_t row_bytes = (size_t)p.d * KIND / 8;
+    float acc[R][RT_TOK];
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+        for (int t = 0; t < RT_TOK; ++t) acc[i][t] = 0.0f;
+#pragma unroll 1
+    for (uint32_t c = hl; c < chunks; c += 32) {
+        float q[R][EPC], sc[R], bi[R];
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const uint32_t row = min(row0 + i, n_rows - 1);     // rows past the end repeat the last one, unstored
+            const uint4 w = *reinterpret_cast<const uint4*>((const uint8_t*)r.w + row * row_bytes + (size_t)c * 16);
+            if (KIND == 16) {
+                act2_to_f32<ACT_BF16>(w.x, q[i][0], q[i][1]); act2_to_f32<ACT_BF16>(w.y, q[i][2], q[i][3]);
+                act2_to_f32<ACT_BF16>(w.z, q[i][4], q[i][5]); act2_to_f32<ACT_BF16>(w.w, q[i][6], q[i][7]);
+            } else {
+                unpack_chunk<KIND == 16 ? 8 : KIND>(w, q[i]);
+                const uint32_t g = c * EPC / NVMAI_GROUP;
+                sc[i] = bf16_to_f32(r.s[(size_t)row * groups + g]);
+                bi[i] = bf16_to_f32(r.b[(size_t)row * groups + g]);
+            }
+        }
+        float eff[EFF ? EPC : 1];
+        if (EFF) {
+#pragma unroll
+            for (int j = 0; j < EPC; ++j) eff[j] = bf16_to_f32(p.eff_scale[c * EPC + j]);
+        }
+        // rows of LDS past the block's last token hold whatever they held: their sums are never stored
+        uint4 xnext[XV];
+#pragma unroll
+        for (int v = 0; v < XV; ++v) xnext[v] = *reinterpret_cast<const uint4*>(xl + c * EPC + 8 * v);
+#pragma unroll
+        for (int t = 0; t < RT_TOK; ++t) {
+            float xv[EPC];
+            uint4 xraw[XV];
+#pragma unroll
+            for (int v = 0; v < XV; ++v) xraw[v] = xnext[v];
+            if (t + 1 < RT_TOK) {                        // the next token's chunk is under way during this one's sums
+#pragma unroll
+                for (int v = 0; v < XV; ++v)
+                    xnext[v] = *reinterpret_cast<const uint4*>(xl + (size_t)(t + 1) * p.d + c * EPC + 8 * v);
+            }
+#pragma unroll
+            for (int v = 0; v < XV; ++v) {
+                act2_to_f32<ACT>(xraw[v].x, xv[8 * v], xv[8 * v + 1]);
+                act2_to_f32<ACT>(xraw[v].y, xv[8 * v + 2], xv[8 * v + 3]);
+                act2_to_f32<ACT>(xraw[v].z, xv[8 * v + 4], xv[8 * v + 5]);
+                act2_to_f32<ACT>(xraw[v].w, xv[8 * v + 6], xv[8 * v + 7]);
+            }
+            if (EFF) {                                   // one rounding, as moe.metal:200-201 multiplies before use
+#pragma unroll
+                for (int j = 0; j < EPC; ++j) xv[j] = __fmul_rn(xv[j], eff[j]);
+            }
+            if (KIND == 16) {
+#pragma unroll
+                for (int i = 0; i < R; ++i)
+#pragma unroll
+                    for (int j = 0; j < EPC; ++j) acc[i][t] = fmaf(q[i][j], xv[j], acc[i][t]);
+            } else {
+                float xs = 0.0f;
+#pragma unroll
+                for (int j = 0; j < EPC; ++j) xs = __fadd_rn(xs, xv[j]);
+#pragma unroll
+                for (int i = 0; i < R; ++i) {
+                    float dot = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < EPC; ++j) dot = fmaf(q[i][j], xv[j], dot);
+                    acc[i][t] = fmaf(sc[i], dot, acc[i][t]);
+                    acc[i][t] = fmaf(bi[i], xs, acc[i][t]);
+                }
+            }
+            // one token at a time: without the fence the scheduler fetches every token's chunk up
+            // front and the accumulators no longer fit beside them
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+        for (int t = 0; t < RT_TOK; ++t) {
+#pragma unroll
+            for (int off = 16; off >= 1; off >>= 1) acc[i][t] = __fadd_rn(acc[i][t], shfl_xor_f(acc[i][t], off));
+            if (hl == 0 && (uint32_t)t < nt && row0 + i < n_rows) out[(size_t)(t0 + t) * out_ld + row0 + i] = acc[i][t];
+            if ((t & 3) == 3) __builtin_amdgcn_sched_barrier(0);     // four butterflies in flight, not all 64
+        }
+}
+
 // ---- top-k select + softmax over the selected ------------------------------------
 // One wave per token.  Selection equals a stable sort by (score desc, index asc)
 // (moe.metal:233-285).  Weights: ex_i = exp(s_i - s_0), sum in slot order,

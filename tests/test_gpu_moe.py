@@ -172,6 +172,38 @@ def test_router_indices_and_logits_bit_exact(nv, ctx, kind):
     _router_case(nv, ctx, kind, 16, 128, 4, 8, rng, eff, pes)
 
 
+@pytest.mark.parametrize("kind", [16, 8, 4])
+def test_router_many_tokens_same_bits(nv, ctx, kind):
+    # 64 tokens and more take the register-tiled kernel: same sums in the same order, so the same bits
+    rng = np.random.default_rng(100 + kind)
+    for E, D, tokens, k in [(256, 2048, 150, 8), (100, 512, 70, 4), (20, 192, 64, 8), (33, 2048, 97, 2)]:
+        say("router tiled", ctx.act, kind, E, D, tokens, k)
+        _router_case(nv, ctx, kind, E, D, tokens, k, rng)
+    say("router tiled scales", kind)
+    eff = O.bf16_bits(rng.uniform(0.5, 1.5, 256).astype(np.float32) / np.float32(math.sqrt(256)))
+    pes = O.bf16_bits(rng.uniform(0.6, 1.4, 40).astype(np.float32))
+    _router_case(nv, ctx, kind, 40, 256, 81, 8, rng, eff, pes)
+
+
+def test_router_many_tokens_padded_stride(nv, ctx_bf16):
+    say("router tiled padded stride")
+    E, D, T, k = 48, 256, 75, 8
+    rng = np.random.default_rng(78)
+    stride = D + 13                                   # rows not 16-byte aligned: element loads into LDS
+    w = O.round_bf16(gauss(rng, (E, D), 0.04))
+    host = O.quantize_affine(w, 8)
+    desc = nv.rows_desc(8, dev(host[0]), dev(host[1].view(np.int16)), dev(host[2].view(np.int16)))
+    block = np.full((T, stride), -31.0, np.float32)
+    block[:, :D] = O.round_bf16(rng.uniform(-1, 1, (T, D)).astype(np.float32))
+    hd = dev(block).to(torch.bfloat16)
+    idx, wt, logits = nv.MoE(ctx_bf16).encode_router(desc, hd[:, :D], E, D, k, want_logits=True)
+    torch.cuda.synchronize()
+    for t in range(T):
+        lo = O.router_logits(8, host[0], host[1], host[2], block[t, :D])
+        assert np.array_equal(logits[t].cpu().numpy().view(np.uint32), lo.view(np.uint32))
+        assert np.array_equal(u32(idx[t]), O.router_topk(lo, k)[0])
+
+
 def test_router_padded_hidden_stride(nv, ctx_bf16):
     # PrefillRouterTests.swift:33-95: rows of `hidden` are d + 13 apart and the padding is left alone
     say("router padded stride")
@@ -351,6 +383,13 @@ def test_decode_layer_toy_shapes(nv, ctx, bits):
                                      (192, 64, 8, 2, 3, 16)]:
         say("decode layer toy", ctx.act, bits, d, f, E, k, tokens, kind)
         _layer_case(nv, ctx, rng, d, f, E, k, bits, tokens, kind, 0.05)
+
+
+def test_decode_layer_many_tokens_gate_row(nv, ctx_bf16):
+    # 64 tokens and more: router rows and the shared expert's gate row through the tiled router kernel
+    say("decode layer many tokens")
+    _layer_case(nv, ctx_bf16, np.random.default_rng(5), 256, 128, 32, 4, 8, 90, 16, 0.05)
+    _layer_case(nv, ctx_bf16, np.random.default_rng(6), 128, 64, 16, 8, 4, 70, 8, 0.05)
 
 
 @pytest.mark.parametrize("bits", [8, 4])
