@@ -216,6 +216,18 @@ def run_prefill(nv, ctx, torch, a):
     flops = T * K * 6.0 * D * F
     g1 = T * K * 4.0 * D * F / (kern["gemm_gate_up"] * 1e-6) / 1e12
     counts = step(0).per_expert_counts.cpu().numpy()
+    # the router + top-k that precedes the step in a layer (not part of the step or of `value`:
+    # the step's routes follow the Zipf law above): bf16 router matrix over the same hidden rows
+    rw = torch.empty((E, D), dtype=torch.bfloat16, device="cuda").normal_(0.0, 0.02, generator=gen)
+    rdesc, rmoe = nv.rows_desc(16, rw.view(torch.int16)), nv.MoE(ctx, bits)
+    for _ in range(3):
+        rmoe.encode_router(rdesc, xs[0], E, D, K)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(10):
+        rmoe.encode_router(rdesc, xs[i % n_x], E, D, K)
+    torch.cuda.synchronize()
+    router_us = (time.perf_counter() - t0) / 10 * 1e6
     # what a plain dense bf16 GEMM of the library that ships with torch reaches on this device
     A = torch.empty((8192, 8192), dtype=torch.bfloat16, device="cuda").normal_(0, 1, generator=gen)
     B = torch.empty((8192, 8192), dtype=torch.bfloat16, device="cuda").normal_(0, 1, generator=gen)
@@ -256,7 +268,8 @@ def run_prefill(nv, ctx, torch, a):
                    "tokens_per_s": round(T / dt), "largest_expert_pairs": int(counts.max()),
                    "experts_hit": int((counts > 0).sum()),
                    "dense_bf16_gemm_8192_tflops": round(dense, 1),
-                   "kernel_us": {k: round(v, 2) for k, v in kern.items()}},
+                   "kernel_us": {k: round(v, 2) for k, v in kern.items()},
+                   "router_topk_us_outside_the_step": round(router_us, 1)},
         "roofline": {"kernel": "prefill_gemm_kernel<DUAL> (gate/up + SwiGLU)", "bound": "mfma",
                      "achieved": round(g1, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(g1 / MFMA_BF16_PEAK_TFLOPS, 4),
