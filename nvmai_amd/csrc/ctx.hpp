@@ -82,6 +82,11 @@ struct ProfScope {
     ~ProfScope() { if (stop) (void)hipEventRecord(stop, stream); }
 };
 
+// One expert over all rows through the grouped-GEMM kernels (prefill_api.hip).
+int expert_ffn_dense(nvmai_hip_ctx* ctx, hipStream_t s, const uint8_t* blob, const nvmai_expert_offsets* off,
+                     uint32_t bits, const void* x, uint32_t x_stride, uint32_t tokens, uint32_t d, uint32_t f,
+                     void* act, void* tmp, const float* gate_logit, void* y, uint32_t y_stride);
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? NVMAI_OK : NVMAI_ERR_HIP; }
 
 }  // namespace nvmai

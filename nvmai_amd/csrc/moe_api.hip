@@ -237,10 +237,10 @@ int run_router(int act, RouterParams& rp, hipStream_t s) {
     // Many tokens (a prefill block): the register-tiled kernel, same logits bit for bit
     if (rp.tokens >= 64 && (size_t)RT_TOK * rp.d * 2 <= 65536) {
         if (act == ACT_BF16) {
-            run_router_tiled<ACT_BF16>(rp, rp.router, rp.num_experts, rp.logits, rp.num_experts, s);
+            if (rp.num_experts) run_router_tiled<ACT_BF16>(rp, rp.router, rp.num_experts, rp.logits, rp.num_experts, s);
             if (rp.gate.kind) run_router_tiled<ACT_BF16>(rp, rp.gate, 1, rp.gate_logit, 1, s);
         } else {
-            run_router_tiled<ACT_FP16>(rp, rp.router, rp.num_experts, rp.logits, rp.num_experts, s);
+            if (rp.num_experts) run_router_tiled<ACT_FP16>(rp, rp.router, rp.num_experts, rp.logits, rp.num_experts, s);
             if (rp.gate.kind) run_router_tiled<ACT_FP16>(rp, rp.gate, 1, rp.gate_logit, 1, s);
         }
         return NVMAI_OK;
@@ -554,6 +554,31 @@ extern "C" int nvmai_hip_shared_expert(nvmai_hip_ctx* ctx, nvmai_stream stream, 
     if (!aligned16(blob) || !aligned16(x) || (x_stride % 8)) return NVMAI_ERR_ALIGNMENT;
     if (n_tokens == 0) return NVMAI_OK;
     hipStream_t s = (hipStream_t)stream;
+    // A block of tokens (prefill): the expert's matrices are read once for all of them by the
+    // grouped-GEMM kernels instead of once per four tokens (the reference runs its dense QMM
+    // there, MPPPrefillInt4QMM.swift:18-128).  Operands past the kernels' 32-bit offsets, and
+    // small batches (the two ways cost the same at about 200 tokens), take the row engine below.
+    if (n_tokens >= 192 && (uint64_t)n_tokens * x_stride * 2 <= 0xFFFFFFFFull &&
+        (uint64_t)n_tokens * d * 2 <= 0xFFFFFFFFull && (uint64_t)d * f * bits / 8 <= 0xFFFFFFFFull) {
+        const bool gated_d = shared_gate && shared_gate->kind;
+        rc = ws_begin(ctx, ws_round((size_t)n_tokens * f * 2) + ws_round((size_t)n_tokens * d * 2) +
+                               ws_round(n_tokens * 4u) + ws_round(16));
+        if (rc) return rc;
+        uint16_t* act = ws_take<uint16_t>(ctx, (size_t)n_tokens * f);
+        uint16_t* tmp = ws_take<uint16_t>(ctx, (size_t)n_tokens * d);
+        float* gate_logit = ws_take<float>(ctx, n_tokens);
+        float* dummy_logits = ws_take<float>(ctx, 4);
+        if (gated_d) {
+            RouterParams rp{};
+            rp.gate = to_desc(shared_gate);
+            rp.x = x; rp.x_stride = x_stride; rp.tokens = n_tokens; rp.num_experts = 0; rp.d = d;
+            rp.logits = dummy_logits; rp.gate_logit = gate_logit;
+            rc = run_router(ctx->act, rp, s);
+            if (rc) return rc;
+        }
+        return nvmai::expert_ffn_dense(ctx, s, (const uint8_t*)blob, off, bits, x, x_stride, n_tokens, d, f, act, tmp,
+                                       gated_d ? gate_logit : nullptr, y, y_stride);
+    }
     const int maxtok = n_tokens == 1 ? 1 : MAX_TOK;
     const uint32_t ents = (n_tokens + maxtok - 1) / maxtok;
     size_t need = ws_round(ents * sizeof(WorkEntry)) + ws_round(16) + 2 * ws_round(n_tokens * 4u) +

@@ -153,6 +153,46 @@ void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t max_mtile
 
 }  // namespace
 
+// One expert over every row of x (the shared expert of a prefill block): gate/up + SwiGLU and
+// down through the grouped-GEMM kernels in their dense mode, then the optional scalar gate.
+// x [tokens, x_stride] and y [tokens, y_stride] in the context's activation type; act and tmp
+// are 16-bit scratch [tokens, f] and [tokens, d], 16-byte aligned.
+namespace nvmai {
+int expert_ffn_dense(nvmai_hip_ctx* ctx, hipStream_t s, const uint8_t* blob, const nvmai_expert_offsets* off,
+                     uint32_t bits, const void* x, uint32_t x_stride, uint32_t tokens, uint32_t d, uint32_t f,
+                     void* act, void* tmp, const float* gate_logit, void* y, uint32_t y_stride) {
+    const uint32_t nt = bits == 4 ? 4 : 2;
+    const uint32_t tiles = (tokens + GEMM_BM - 1) / GEMM_BM;
+    GemmParams g1{};
+    g1.pool = blob; g1.pool_stride = 0x7FFFFFFFull;   // bound of the scale resources; the only "expert" is 0
+    g1.wA = off->gate_w; g1.sA = off->gate_s; g1.bA = off->gate_b;
+    g1.wB = off->up_w; g1.sB = off->up_s; g1.bB = off->up_b;
+    g1.dense_rows = tokens;
+    g1.x = x; g1.x_stride = x_stride; g1.out = act; g1.out_stride = f;
+    g1.K = d; g1.N = f; g1.top_k = 1; g1.n_tiles_n = (f + 32 * nt - 1) / (32 * nt);
+    g1.units_per_tile = (g1.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
+    GemmParams g2 = g1;
+    g2.wA = off->down_w; g2.sA = off->down_s; g2.bA = off->down_b;
+    g2.wB = g2.sB = g2.bB = 0;
+    g2.x = act; g2.x_stride = f; g2.out = tmp; g2.out_stride = d;
+    g2.K = f; g2.N = d; g2.n_tiles_n = (d + 64 * nt - 1) / (64 * nt);
+    g2.units_per_tile = (g2.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
+    if (ctx->act == ACT_BF16) {
+        if (bits == 4) launch_gemms<ACT_BF16, 4, 4>(g1, g2, tiles, ctx, s);
+        else launch_gemms<ACT_BF16, 8, 2>(g1, g2, tiles, ctx, s);
+    } else {
+        if (bits == 4) launch_gemms<ACT_FP16, 4, 4>(g1, g2, tiles, ctx, s);
+        else launch_gemms<ACT_FP16, 8, 2>(g1, g2, tiles, ctx, s);
+    }
+    dim3 grid((d + 255) / 256, tokens);
+    if (ctx->act == ACT_BF16)
+        gate_rows_kernel<ACT_BF16><<<grid, 256, 0, s>>>((const uint16_t*)tmp, gate_logit, (uint16_t*)y, tokens, d, y_stride);
+    else
+        gate_rows_kernel<ACT_FP16><<<grid, 256, 0, s>>>((const uint16_t*)tmp, gate_logit, (uint16_t*)y, tokens, d, y_stride);
+    return launch_status();
+}
+}  // namespace nvmai
+
 extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* experts_base,
                                              uint64_t expert_stride, const nvmai_expert_offsets* off,
                                              uint32_t bits, uint32_t d, uint32_t f, uint32_t num_experts,

@@ -513,7 +513,8 @@ struct GemmParams {
     uint32_t K, N, top_k, n_tiles_n;
     uint32_t units_per_tile;            // ceil(n_tiles_n / GEMM_UNIT)
     uint32_t dense_rows;                // > 0: a dense product over rows 0..dense_rows-1 of x (row i -> row i of
-                                        // out), M tiles of GEMM_BM consecutive rows; mtiles, n_mtiles, pairs unused
+                                        // out; DUAL: gate/up + SwiGLU of one expert over all rows), M tiles of
+                                        // GEMM_BM consecutive rows; mtiles, n_mtiles, pairs unused
 };
 
 constexpr int GEMM_SK = 128;            // k per super-step
@@ -632,7 +633,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     const uint32_t tile_id = unit / p.units_per_tile;
     const uint32_t nt = (unit % p.units_per_tile) * GEMM_UNIT + on_xcd % GEMM_UNIT;
     MTile mt;
-    if (!DUAL && p.dense_rows) {
+    if (p.dense_rows) {
         if (tile_id * GEMM_BM >= p.dense_rows || nt >= p.n_tiles_n) return;
         mt = MTile{0u, tile_id * GEMM_BM, min((uint32_t)GEMM_BM, p.dense_rows - tile_id * GEMM_BM)};
     } else {
@@ -668,7 +669,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     for (int g = 0; g < 2; ++g) {
         const uint32_t row = (wave * 2 + g) * 16 + (lane >> 2);
         const uint32_t m = row < mt.rows ? row : 0;     // a dead row of a live tile repeats row 0
-        const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
+        const uint32_t src = (DUAL && !p.dense_rows) ? p.pairs[mt.row_start + m].token : mt.row_start + m;
         xoff[g] = src * (p.x_stride * 2u) + (uint32_t)((lane & 3) ^ gemm_row_swizzle(lane >> 2)) * 16u;
     }
     auto load_x = [&](uint32_t ss, uint8_t* stage) {
@@ -1010,7 +1011,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         {
             const uint32_t row = ((wave * MT) >> 2) * 16 + (lane >> 2);
             const uint32_t m = row < mt.rows ? row : 0;
-            const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
+            const uint32_t src = (DUAL && !p.dense_rows) ? p.pairs[mt.row_start + m].token : mt.row_start + m;
             xo = src * (p.x_stride * 2u) + (uint32_t)((lane & 3) ^ gemm_row_swizzle(lane >> 2)) * 16u;
         }
         auto load_xs = [&](uint32_t ss, uint8_t* stage) {
@@ -1137,7 +1138,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         {
             const uint32_t row = ((wave * MT) >> 2) * 16 + (lane >> 2);
             const uint32_t m = row < mt.rows ? row : 0;
-            const uint32_t src = DUAL ? p.pairs[mt.row_start + m].token : mt.row_start + m;
+            const uint32_t src = (DUAL && !p.dense_rows) ? p.pairs[mt.row_start + m].token : mt.row_start + m;
             xo = src * (p.x_stride * 2u) + (uint32_t)((lane & 3) ^ gemm_row_swizzle(lane >> 2)) * 16u;
         }
         auto load_xs = [&](uint32_t ss, uint8_t* stage) {
@@ -1215,6 +1216,18 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     else if (live_mt > 2) run_full(std::integral_constant<int, 4>{});
     else if (live_mt > 1) { if (tab_ok) run_short_tab(std::integral_constant<int, 2>{}); else run_short(std::integral_constant<int, 2>{}); }
     else { if (tab_ok) run_short_tab(std::integral_constant<int, 1>{}); else run_short(std::integral_constant<int, 1>{}); }
+}
+
+// y[t, :] = rows[t, :] scaled by 1 / (1 + exp(-gate_logit[t])) where a gate is given (the shared
+// expert's scalar gate, utility.metal:61-70), else copied: rows are 16-bit activations [tokens, d].
+template <int ACT>
+__global__ __launch_bounds__(256) void gate_rows_kernel(const uint16_t* rows, const float* gate_logit, uint16_t* y,
+                                                       uint32_t tokens, uint32_t d, uint32_t y_stride) {
+    const uint32_t t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= d) return;
+    float v = act_to_f32<ACT>(rows[(size_t)t * d + c]);
+    if (gate_logit) v = __fdiv_rn(v, __fadd_rn(1.0f, expf(-gate_logit[t])));
+    y[(size_t)t * y_stride + c] = f32_to_act<ACT>(v);
 }
 
 // ---- combine (prefill.metal:437-458) -------------------------------------------------------
