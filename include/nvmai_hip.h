@@ -103,7 +103,9 @@ int nvmai_hip_dequantize_affine(nvmai_hip_ctx* ctx, nvmai_stream stream, const u
 /* DequantInt4GEMV.encode / DequantInt8GEMV.encode / AffineQuantGEMV.encode
  * (DequantInt4GEMV.swift:66-110, DequantInt8GEMV.swift:50-86, AffineQuant.swift:58)
  * and, with y_f32 != NULL, nvmai_int4_affine_gemv (nvmai_kernels.h:22-28):
- * y[t, :] = W x[t, :] for n_tokens inputs.  y (activations) or y_f32 may be NULL. */
+ * y[t, :] = W x[t, :] for n_tokens inputs.  y (activations) or y_f32 may be NULL.
+ * More than four inputs against a matrix of 1024 rows or more, 16-bit outputs only and 16-byte
+ * aligned operands: runs as nvmai_hip_affine_qmm (the matrix is read once for all inputs). */
 int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
                           const uint16_t* scales, const uint16_t* biases, uint32_t bits,
                           const void* x, uint32_t x_stride, uint32_t n_tokens, uint32_t m,

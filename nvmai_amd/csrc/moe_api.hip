@@ -365,6 +365,15 @@ extern "C" int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, co
                                      const void* x, uint32_t x_stride, uint32_t n_tokens,
                                      uint32_t m, uint32_t n, void* y, float* y_f32,
                                      uint32_t y_stride) {
+    // More than four input rows of a large matrix: the row engine would stream the matrix once per
+    // four rows; the matrix-core product reads and dequantizes it once (from five rows on it is
+    // the faster of the two at LM-head sizes).  Only where its preconditions hold and 16-bit
+    // outputs are all that is asked for.
+    if (ctx && n_tokens > 4 && m >= 1024 && y && !y_f32 && weights && scales && biases && x &&
+        (bits == 4 || bits == 8) && n && n % NVMAI_GROUP == 0 && x_stride >= n && y_stride >= m &&
+        aligned16(weights) && aligned16(x) && x_stride % 8 == 0 && aligned16(y) &&
+        (uint64_t)n_tokens * x_stride * 2 <= 0xFFFFFFFFull && (uint64_t)m * n * bits / 8 <= 0xFFFFFFFFull)
+        return nvmai_hip_affine_qmm(ctx, stream, weights, scales, biases, bits, x, x_stride, y, y_stride, n_tokens, m, n);
     return affine_gemv_any(ctx, stream, weights, scales, biases, bits, x, false, x_stride, n_tokens, m, n, y,
                            y_f32, y_stride);
 }
