@@ -277,6 +277,59 @@ void run_combine(int act, const CombineParams& cp, hipStream_t s) {
     else combine_kernel<ACT_FP16><<<grid, 256, 0, s>>>(cp);
 }
 
+// Small decode batches in three launches (router logits; gate/up that selects for itself; down
+// projection + combine) -- for the shapes both kernels are instantiated for.
+constexpr uint32_t FUSED_DECODE_MAX_TOKENS = 2;    // measured: 3-4 tokens are no faster this way
+
+bool fused_decode_ok(uint32_t T, uint32_t K, bool has_shared, uint32_t d, uint32_t f, uint32_t bits) {
+    const uint32_t c1 = d * bits / 128, c2 = f * bits / 128;
+    return T <= FUSED_DECODE_MAX_TOKENS && T * K <= 64 && K + (has_shared ? 1u : 0u) <= 4 * DC_SLOTS_PER_WAVE &&
+           (d * bits) % 128 == 0 && (c1 == 64 || c1 == 128) &&
+           (f * bits) % 128 == 0 && (c2 == 16 || c2 == 32 || c2 == 64);
+}
+
+template <int ACT, int BITS>
+void launch_routed_t(RowsParams& p, const SelectParams& sel, const RoutedStats& rs, uint32_t slots, hipStream_t s) {
+    const uint32_t chunks = p.n * BITS / 128;
+    constexpr uint32_t rows_per_block = 4 * 1 * 1 * 2;       // four waves, SEG 64, RPI 1, ITERS 2
+    p.blocks_per_entry = (p.rows + rows_per_block - 1) / rows_per_block;
+    const dim3 grid(slots * p.blocks_per_entry, sel.tokens);
+    if (chunks == 64)
+        expert_rows_routed<ACT, BITS, 64, 1, 1, 2><<<grid, 256, rows_fast_lds_bytes(p.n, 1, 64), s>>>(p, sel, rs);
+    else
+        expert_rows_routed<ACT, BITS, 64, 2, 1, 2><<<grid, 256, rows_fast_lds_bytes(p.n, 2, 64), s>>>(p, sel, rs);
+}
+
+void launch_routed(int act, uint32_t bits, RowsParams& p, const SelectParams& sel, const RoutedStats& rs,
+                   uint32_t slots, hipStream_t s) {
+    if (act == ACT_BF16) {
+        if (bits == 8) launch_routed_t<ACT_BF16, 8>(p, sel, rs, slots, s);
+        else launch_routed_t<ACT_BF16, 4>(p, sel, rs, slots, s);
+    } else {
+        if (bits == 8) launch_routed_t<ACT_FP16, 8>(p, sel, rs, slots, s);
+        else launch_routed_t<ACT_FP16, 4>(p, sel, rs, slots, s);
+    }
+}
+
+template <int ACT, int BITS>
+void launch_down_combine_t(const DownCombineParams& p, hipStream_t s) {
+    const uint32_t chunks = p.n * BITS / 128;
+    const dim3 grid((p.rows + DC_ROWS - 1) / DC_ROWS, p.tokens);
+    if (chunks == 16) down_combine_kernel<ACT, BITS, 16><<<grid, 256, 0, s>>>(p);
+    else if (chunks == 32) down_combine_kernel<ACT, BITS, 32><<<grid, 256, 0, s>>>(p);
+    else down_combine_kernel<ACT, BITS, 64><<<grid, 256, 0, s>>>(p);
+}
+
+void launch_down_combine(int act, uint32_t bits, const DownCombineParams& p, hipStream_t s) {
+    if (act == ACT_BF16) {
+        if (bits == 8) launch_down_combine_t<ACT_BF16, 8>(p, s);
+        else launch_down_combine_t<ACT_BF16, 4>(p, s);
+    } else {
+        if (bits == 8) launch_down_combine_t<ACT_FP16, 8>(p, s);
+        else launch_down_combine_t<ACT_FP16, 4>(p, s);
+    }
+}
+
 }  // namespace
 
 // ---------------------------------------------------------------------------
@@ -694,6 +747,29 @@ extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream strea
     SelectParams sp{logits, L->per_expert_scale, T, E, K, idx, wts};
     GroupParams gp{sp, (uint32_t)maxtok, has_shared ? 1 : 0, entries, n_entries, stats, pair_token, pair_id,
                    ctx->tickets};
+    if (fused_decode_ok(T, K, has_shared, D, F, L->bits)) {
+        { ProfScope ps(ctx, NVMAI_PROF_ROUTER, s); rc = run_router(ctx->act, rp, s); }
+        if (rc) return rc;
+        RowsParams p{};
+        p.src.pool_base = (const uint8_t*)L->experts_base;
+        p.src.pool_stride = L->expert_stride;
+        p.src.slot[8] = (const uint8_t*)L->shared_blob;
+        set_phase1(p, L->offsets, D, F);
+        p.x = x; p.x_stride = x_stride; p.out = acts; p.out_stride = F;
+        const RoutedStats rs{stats, has_shared ? 1 : 0};
+        {
+            ProfScope ps(ctx, NVMAI_PROF_PHASE1, s);
+            launch_routed(ctx->act, L->bits, p, sp, rs, K + (has_shared ? 1u : 0u), s);
+        }
+        DownCombineParams dc{};
+        dc.src = p.src;
+        dc.wA = L->offsets.down_w; dc.sA = L->offsets.down_s; dc.bA = L->offsets.down_b;
+        dc.acts = acts; dc.idx = idx; dc.w = wts; dc.gate_logit = gated ? gate_logit : nullptr;
+        dc.has_shared = has_shared ? 1 : 0; dc.tokens = T; dc.top_k = K; dc.rows = D; dc.n = F;
+        dc.y_stride = y_stride; dc.y = y;
+        { ProfScope ps(ctx, NVMAI_PROF_PHASE2, s); launch_down_combine(ctx->act, L->bits, dc, s); }
+        return launch_status();
+    }
     // Two launches on purpose: one that also selects and groups in its last blocks needs a
     // device-scope release (an L2 write-back on this multi-die part) from every one of its
     // hundreds of producer blocks, and measured 18 us slower per step.

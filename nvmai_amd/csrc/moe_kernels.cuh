@@ -170,9 +170,15 @@ __device__ __forceinline__ void pow2_scale(float amax, float& sc, float& isc) {
 // that only one input's columns are live at a time.
 // LDS: [ntok][n/8] uint4 packed inputs | [ntok][NCH*SEG][2] float chunk sums (all, odd pairs) |
 //      [MAX_TOK*4] float wave maxima | [MAX_TOK] float inverse scales.
-template <int ACT, int BITS, int SEG, int NCH, int TOKS, bool DUAL, bool XF32, int RPI, int ITERS>
+//
+// DIRECT (one input only): the entry itself names its rows -- input row we.reserved, output row
+// we.pair_start -- and the pair tables are not read (entries made inside the launch that uses them).
+template <int ACT, int BITS, int SEG, int NCH, int TOKS, bool DUAL, bool XF32, int RPI, int ITERS, bool DIRECT = false>
 __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const WorkEntry& we, uint32_t rb,
                                                  uint4* lds) {
+    static_assert(!DIRECT || TOKS == 1, "a direct entry holds one input");
+    auto in_row = [&](int t) -> uint32_t { return DIRECT ? we.reserved : p.pair_in[we.pair_start + t]; };
+    auto out_row_of = [&](int t) -> uint32_t { return DIRECT ? we.pair_start : p.pair_out[we.pair_start + t]; };
     constexpr int EPC = Chunk<BITS>::elems;
     constexpr int PAIRS = EPC / 2;                // packed pairs per chunk
     constexpr int H = PAIRS / 4;                  // 16-byte LDS words per chunk
@@ -237,7 +243,7 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
             if (t >= ntok) break;
-            if (live) load8<ACT, XF32>(p.x, (size_t)p.pair_in[we.pair_start + t] * p.x_stride + e0, v[t]);
+            if (live) load8<ACT, XF32>(p.x, (size_t)in_row(t) * p.x_stride + e0, v[t]);
         }
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
@@ -271,7 +277,7 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
         // ---- pass 1: largest magnitude of every input row
     #pragma unroll 1
         for (int t = 0; t < ntok; ++t) {
-            const size_t in_off = (size_t)p.pair_in[we.pair_start + t] * p.x_stride;
+            const size_t in_off = (size_t)in_row(t) * p.x_stride;
             float m = 0.0f;
             for (uint32_t e0 = threadIdx.x * 8; e0 < p.n; e0 += 256 * 8) {
                 float v[8];
@@ -286,7 +292,7 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
         // ---- pass 2: scale, convert, pack
     #pragma unroll 1
         for (int t = 0; t < ntok; ++t) {
-            const size_t in_off = (size_t)p.pair_in[we.pair_start + t] * p.x_stride;
+            const size_t in_off = (size_t)in_row(t) * p.x_stride;
             const float amax = fmaxf(fmaxf(wmax_tab[t * 4], wmax_tab[t * 4 + 1]),
                                      fmaxf(wmax_tab[t * 4 + 2], wmax_tab[t * 4 + 3]));
             float sc, isc;
@@ -348,7 +354,7 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
                 xo[c] = two.y;
             }
             const float isc = isc_tab[t];
-            const uint32_t out_row = p.pair_out[we.pair_start + t];
+            const uint32_t out_row = out_row_of(t);
 #pragma unroll
             for (int i = 0; i < RPI; ++i) {
                 const uint32_t row = row_base + (it * RPI + i) * RPL + seg_id;
@@ -784,7 +790,9 @@ __device__ __forceinline__ bool better(float v, uint32_t i, float v2, uint32_t i
     return v > v2 || (v == v2 && i < i2);
 }
 
-__device__ void select_topk_wave(const SelectParams& p, uint32_t t, int lane) {
+// Selection for token t by one wave: lane r < top_k ends with the r-th best (score, index).
+__device__ __forceinline__ void select_topk_core(const SelectParams& p, uint32_t t, int lane, float& my_score,
+                                                 uint32_t& my_idx) {
     float val[TOPK_MAX_PER_LANE];
     bool taken[TOPK_MAX_PER_LANE];
 #pragma unroll
@@ -794,8 +802,8 @@ __device__ void select_topk_wave(const SelectParams& p, uint32_t t, int lane) {
         val[j] = e >= p.num_experts ? 0.0f : p.logits[at];
         taken[j] = e >= p.num_experts;
     }
-    float my_score = 0.0f;
-    uint32_t my_idx = 0;
+    my_score = 0.0f;
+    my_idx = 0;
     for (uint32_t round = 0; round < p.top_k; ++round) {
         float bv = -INFINITY;
         uint32_t bi = 0xFFFFFFFFu;
@@ -814,6 +822,12 @@ __device__ void select_topk_wave(const SelectParams& p, uint32_t t, int lane) {
             if ((uint32_t)(lane + 64 * j) == bi) taken[j] = true;
         if ((uint32_t)lane == round) { my_score = bv; my_idx = bi; }
     }
+}
+
+// Softmax over the selected scores (in the lanes below top_k) times the expert's gain; stores
+// index and fp16 weight of token t.
+__device__ __forceinline__ void select_store_routes(const SelectParams& p, uint32_t t, int lane, float my_score,
+                                                    uint32_t my_idx) {
     const float max_s = readlane_f(my_score, 0);
     const float ex = expf(my_score - max_s);
     float sum = 0.0f;
@@ -824,6 +838,13 @@ __device__ void select_topk_wave(const SelectParams& p, uint32_t t, int lane) {
         p.out_idx[(size_t)t * p.top_k + lane] = my_idx;
         p.out_w[(size_t)t * p.top_k + lane] = f32_to_f16(w);
     }
+}
+
+__device__ void select_topk_wave(const SelectParams& p, uint32_t t, int lane) {
+    float my_score;
+    uint32_t my_idx;
+    select_topk_core(p, t, lane, my_score, my_idx);
+    select_store_routes(p, t, lane, my_score, my_idx);
 }
 
 __global__ __launch_bounds__(256) void select_topk_kernel(SelectParams p) {
@@ -1032,6 +1053,170 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineParams p) {
         acc = __fadd_rn(acc, __fmul_rn(w, p.partials[((size_t)t * p.top_k + r) * p.d + d]));
     }
     ((uint16_t*)p.y)[(size_t)t * p.y_stride + d] = f32_to_act<ACT>(acc);
+}
+
+// ---- small decode batches: three launches instead of five ---------------------------------
+// With a handful of tokens the step is bound by its chain of dependent launches, not by bytes.
+// (1) expert_rows_routed: the gate/up launch selects for itself.  Every wave repeats its token's
+// top-k from the logits (256 floats; the same routine as the select kernels, so the same indices)
+// and takes the expert of its block's slot from it; grid.y = token, a block's entry is (token,
+// slot) with slot top_k = the shared expert.  The first block of a token stores the routes.
+// Tokens that share an expert read it once each (from L2 after the first).
+struct RoutedStats {
+    uint32_t* stats;           // optional: [0] = entries, [1] = distinct routed experts of the step
+    int has_shared;
+};
+
+template <int ACT, int BITS, int SEG, int NCH, int RPI, int ITERS>
+__global__ __launch_bounds__(256) void expert_rows_routed(RowsParams p, SelectParams sel, RoutedStats rs) {
+    extern __shared__ uint4 rows_lds[];
+    const uint32_t slot = blockIdx.x / p.blocks_per_entry, rb = blockIdx.x % p.blocks_per_entry;
+    const uint32_t t = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    WorkEntry we;
+    we.pair_count = 1;
+    we.reserved = t;
+    if (slot < sel.top_k) {
+        float score;
+        uint32_t idx;
+        select_topk_core(sel, t, lane, score, idx);
+        if (blockIdx.x == 0 && threadIdx.x < 64) {
+            select_store_routes(sel, t, lane, score, idx);
+        }
+        we.expert = (uint32_t)__builtin_amdgcn_readlane((int)idx, (int)slot);
+        we.pair_start = t * sel.top_k + slot;
+    } else {
+        we.expert = NVMAI_SLOT_FLAG | 8u;
+        we.pair_start = sel.tokens * sel.top_k + t;
+    }
+    expert_rows_body<ACT, BITS, SEG, NCH, 1, true, false, RPI, ITERS, true>(p, we, rb, rows_lds);
+    // The caller's statistics, off the critical path: the first block counts the distinct experts
+    // of the step once its rows are done (at most four tokens, tokens * top_k <= 64 indices).
+    if (rs.stats && blockIdx.x == 0 && t == 0) {
+        const uint32_t n = sel.tokens * sel.top_k;
+        uint32_t distinct = sel.top_k;
+        if (sel.tokens > 1) {
+            __syncthreads();
+            uint32_t* ids = reinterpret_cast<uint32_t*>(rows_lds);
+            const uint32_t wave = threadIdx.x >> 6;
+            if (wave < sel.tokens) {
+                float score;
+                uint32_t idx;
+                select_topk_core(sel, wave, lane, score, idx);
+                if ((uint32_t)lane < sel.top_k) ids[wave * sel.top_k + lane] = idx;
+            }
+            __syncthreads();
+            bool first = (uint32_t)lane < n;
+            for (uint32_t j = 0; j < (uint32_t)lane && (uint32_t)lane < n; ++j) first = first && ids[j] != ids[lane];
+            distinct = (uint32_t)__popcll(__ballot(first));
+        }
+        if (threadIdx.x == 0) {
+            rs.stats[0] = sel.tokens * (sel.top_k + (rs.has_shared ? 1u : 0u));
+            rs.stats[1] = distinct;
+        }
+    }
+}
+
+// (2) down_combine: the down projection of every slot of a token and the weighted sum over the
+// slots in one launch.  A block owns DC_ROWS output rows of one token; its four waves share the
+// slots (wave w: slots w, w + 4, ...), SEG lanes per row with one 16-byte chunk each, every load
+// of a wave issued before the first use.  Plain fp32: dot = fma chain over the chunk in element
+// order, acc = scale * dot + bias * sum(act), DPP sum over the row's lanes.  The slot partials
+// meet in LDS and DC_ROWS threads add them exactly as combine_kernel does (shared expert first,
+// then the routed slots in slot order).
+constexpr int DC_ROWS = 8;
+constexpr int DC_SLOTS_PER_WAVE = 3;        // top_k + shared <= 12
+
+struct DownCombineParams {
+    BlobSource src;
+    int64_t wA, sA, bA;           // down projection inside the blob
+    const float* acts;            // fp32 [tokens * top_k (+ tokens), n]: routed rows, then shared rows
+    const uint32_t* idx;          // [tokens, top_k]
+    const uint16_t* w;            // fp16 [tokens, top_k]
+    const float* gate_logit;      // optional [tokens]
+    int has_shared;
+    uint32_t tokens, top_k, rows, n, y_stride;
+    void* y;
+};
+
+// (Handing a slot's activation row to the lanes through LDS -- one fetch per wave instead of one
+// per row of a load instruction -- was measured slower: 12 us against 9.6 us per launch at one
+// token; the step is a chain of latencies, and the LDS round trip lengthens it.)
+template <int ACT, int BITS, int SEG>
+__global__ __launch_bounds__(256) void down_combine_kernel(DownCombineParams p) {
+    constexpr int EPC = Chunk<BITS>::elems;
+    constexpr int RPL = 64 / SEG;                 // rows per load instruction
+    constexpr int PASSES = DC_ROWS / RPL;
+    __shared__ float part[4 * DC_SLOTS_PER_WAVE][DC_ROWS];
+    const uint32_t t = blockIdx.y, row0 = blockIdx.x * DC_ROWS;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int seg_id = lane / SEG, sl = lane % SEG;
+    const uint32_t n_slots = p.top_k + (p.has_shared ? 1u : 0u);
+    const uint32_t groups = p.n / NVMAI_GROUP, row_bytes = p.n * BITS / 8;
+    const uint32_t g = (uint32_t)sl * EPC / NVMAI_GROUP;
+
+    // what the final sum needs, requested before everything else: lane k holds the weight of slot k
+    const float wk = (uint32_t)lane < p.top_k ? f16_to_f32(p.w[(size_t)t * p.top_k + lane]) : 0.0f;
+    const float gate = p.gate_logit ? p.gate_logit[t] : 0.0f;
+
+    uint4 q[DC_SLOTS_PER_WAVE][PASSES];
+    uint16_t sc[DC_SLOTS_PER_WAVE][PASSES], bi[DC_SLOTS_PER_WAVE][PASSES];
+    float a[DC_SLOTS_PER_WAVE][EPC];
+#pragma unroll
+    for (int j = 0; j < DC_SLOTS_PER_WAVE; ++j) {
+        const uint32_t slot = wave + 4 * j;
+        if (slot >= n_slots) break;               // uniform per wave
+        const bool routed = slot < p.top_k;
+        const uint32_t expert = routed ? p.idx[(size_t)t * p.top_k + slot] : (NVMAI_SLOT_FLAG | 8u);
+        const uint32_t act_row = routed ? t * p.top_k + slot : p.tokens * p.top_k + t;
+        const uint8_t* blob = blob_ptr(p.src, expert);
+        const uint8_t* W = blob + p.wA;
+        const uint16_t* S = reinterpret_cast<const uint16_t*>(blob + p.sA);
+        const uint16_t* B = reinterpret_cast<const uint16_t*>(blob + p.bA);
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) {
+            const uint32_t row = row0 + i * RPL + seg_id;
+            const uint32_t r = row < p.rows ? row : p.rows - 1;
+            q[j][i] = *reinterpret_cast<const uint4*>(W + (size_t)r * row_bytes + sl * 16);
+            sc[j][i] = S[(size_t)r * groups + g];
+            bi[j][i] = B[(size_t)r * groups + g];
+        }
+        load_x<ACT, true, EPC>(p.acts, (size_t)act_row * p.n, (uint32_t)sl * EPC, a[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < DC_SLOTS_PER_WAVE; ++j) {
+        const uint32_t slot = wave + 4 * j;
+        if (slot >= n_slots) break;
+        const float* aj = a[j];
+        float xs = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPC; ++e) xs += aj[e];
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) {
+            float qf[EPC];
+            unpack_chunk<BITS>(q[j][i], qf);
+            float dot = 0.0f;
+#pragma unroll
+            for (int e = 0; e < EPC; ++e) dot = fmaf(qf[e], aj[e], dot);
+            float acc = fmaf(bf16_to_f32(sc[j][i]), dot, bf16_to_f32(bi[j][i]) * xs);
+            acc = seg_reduce_sum<SEG>(acc);
+            if (seg_result_lane<SEG>(lane)) part[slot][i * RPL + seg_id] = acc;
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {              // lanes below DC_ROWS own an output row each; all 64 serve the lane reads
+        const uint32_t r = lane < DC_ROWS ? lane : 0;
+        float acc = 0.0f;
+        if (p.has_shared) {
+            float s = part[p.top_k][r];
+            if (p.gate_logit) s = __fdiv_rn(s, __fadd_rn(1.0f, expf(-gate)));
+            acc = __fadd_rn(acc, s);
+        }
+        for (uint32_t k = 0; k < p.top_k; ++k)
+            acc = __fadd_rn(acc, __fmul_rn(readlane_f(wk, (int)k), part[k][r]));
+        if (lane < DC_ROWS && row0 + r < p.rows)
+            ((uint16_t*)p.y)[(size_t)t * p.y_stride + row0 + r] = f32_to_act<ACT>(acc);
+    }
 }
 
 // fp32 rows [tokens, m] -> the caller's rows with its own stride: 16-bit activations (y) and /

@@ -345,7 +345,7 @@ def test_shared_expert_with_scalar_gate(nv, ctx, bits):
 
 
 # ------------------------------------------------------------------ fused decode layer
-def _layer_case(nv, ctx, rng, d, f, E, k, bits, tokens, router_kind, std):
+def _layer_case(nv, ctx, rng, d, f, E, k, bits, tokens, router_kind, std, shared=True, gated=True):
     mk = lambda r, c, s_=std: O.round_bf16(gauss(rng, (r, c), s_))
     # build the pool on the GPU with the (bit-exact) device quantizer, then read it back
     off, stride = nv.expert_offsets(d, f, bits)
@@ -367,11 +367,13 @@ def _layer_case(nv, ctx, rng, d, f, E, k, bits, tokens, router_kind, std):
     gh = O.quantize_affine(mk(1, d, 0.05), 8)
     gdesc = nv.rows_desc(8, dev(gh[0]), dev(gh[1].view(np.int16)), dev(gh[2].view(np.int16)))
     x = round_act(gauss(rng, (tokens, d)), ctx.act)
-    layer = nv.moe_layer_desc(d, f, E, k, bits, rdesc, pool[:E], pool[E], gdesc)
+    layer = nv.moe_layer_desc(d, f, E, k, bits, rdesc, pool[:E], pool[E] if shared else None,
+                              gdesc if shared and gated else None)
     stats = torch.zeros(2, dtype=torch.int32, device="cuda")
     y, idx, w = nv.MoE(ctx, bits).decode_layer(layer, act_tensor(x, ctx), want_routes=True, stats=stats)
     torch.cuda.synchronize()
-    io, wo, yo = O.moe_layer_forward(x, d, f, k, bits, (router_kind,) + rh, pool_h[:E], pool_h[E], (8,) + gh)
+    io, wo, yo = O.moe_layer_forward(x, d, f, k, bits, (router_kind,) + rh, pool_h[:E],
+                                     pool_h[E] if shared else None, (8,) + gh if shared and gated else None)
     assert np.array_equal(u32(idx), io), "routing indices"
     assert np.abs(u16(w).astype(np.int32) - wo.astype(np.int32)).max() <= 1
     assert O.rel_error(act_np(y), yo) < TOL_ACT
@@ -400,3 +402,18 @@ def test_decode_layer_production_shape(nv, ctx_bf16, bits, tokens):
     # configs[1]: hidden 2048, 256 experts top-8, intermediate 512, shared expert with sigmoid gate
     say("decode layer production", bits, tokens)
     _layer_case(nv, ctx_bf16, np.random.default_rng(tokens + bits), 2048, 512, 256, 8, bits, tokens, 16, 0.02)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_decode_layer_few_tokens_three_launches(nv, ctx, bits):
+    # one to four tokens: gate/up selects for itself, down projection and combine are one launch;
+    # every row-chunk count both kernels are built for, with and without shared expert and gate,
+    # tokens that share experts (few experts), and one shape outside them (the five-launch path)
+    rng = np.random.default_rng(70 + bits)
+    per = 128 // bits                                  # codes per 16-byte chunk
+    for c1, c2, E, k, tokens, shared, gated in [(64, 16, 16, 8, 1, True, True), (128, 32, 12, 11, 4, True, False),
+                                                (64, 64, 8, 2, 3, False, False), (64, 32, 300, 8, 1, True, True),
+                                                (128, 16, 10, 8, 2, True, True), (64, 8, 8, 4, 2, True, True)]:
+        d, f = c1 * per, c2 * per
+        say("decode layer few tokens", ctx.act, bits, d, f, E, k, tokens, shared, gated)
+        _layer_case(nv, ctx, rng, d, f, E, k, bits, tokens, 16 if d <= 2048 else 8, 0.03, shared, gated)
