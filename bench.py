@@ -423,6 +423,25 @@ def run_sampler(nv, ctx, torch, a):
     for tag, name in ((nv.PROF_SOFTMAX, "softmax"), (nv.PROF_SAMPLE, "sample_topk64")):
         ms, n = ctx.profile_read(tag)
         kern[name] = ms / max(n, 1) * 1e3
+    cpu = None
+    if not a.no_cpu:
+        # the same stage on the CPU oracle, one row, one thread: LM head GEMV, softmax, sampler
+        import oracle as O
+        p_, s_, b_ = (t_.cpu().numpy() for t_ in heads[0])
+        x0 = xs[0, 0].float().cpu().numpy()
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            lg = O.affine_gemv(p_, s_.view(np.uint16), b_.view(np.uint16), x0, bits)
+            pr = O.softmax_f16(O.round_bf16(lg), softcap=30.0, tiled=True)
+            O.sample_topk64(pr, 0.6, 0.95, seeds[0], top_k=20)
+            reps += 1
+            if time.perf_counter() - t0 > 10.0 or reps >= 20:
+                break
+        dtc = (time.perf_counter() - t0) / reps
+        cpu = dict(value=1.0 / dtc, unit="tok/s", cores=1, kind="port",
+                   sample="oracle affine_gemv over the %d-bit LM head + softmax_f16 (tiled) + sample_topk64, "
+                          "one row, %d reps, %.3f s each" % (bits, reps, dtc))
     head_bytes = V * D * bits / 8 + 2 * V * (D // 64) * 2
     step_bytes_ = head_bytes + rows * (D * 2 + V * 2 * 2 + V * 2)   # x, logits w+r, probs w (+ r by the sampler)
     gbps = head_bytes / (gemv_us * 1e-6) / 1e9
@@ -437,7 +456,7 @@ def run_sampler(nv, ctx, torch, a):
         "roofline": {"kernel": "LM head: expert_rows GEMV (<= 4 rows) or prefill_gemm_kernel (more)", "bound": "hbm", "achieved": round(gbps, 2),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
                      "bytes_per_launch": head_bytes, "avg_launch_us": round(gemv_us, 2)},
-        "cpu_baseline": None,
+        "cpu_baseline": cpu,
     }
 
 
