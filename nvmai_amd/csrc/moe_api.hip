@@ -177,6 +177,41 @@ void launch_rows(int act, uint32_t bits, bool dual, bool xf32, RowsParams& p, in
 #undef NVMAI_ROWS
 }
 
+// One matrix against dense_count 16-bit input rows in ONE launch (no work-list launch before it,
+// no copy-out after it): the shapes the fast engine has a single-matrix instantiation for.
+// Returns false, having launched nothing, for any other shape.
+template <int ACT, int BITS>
+bool launch_dense_rows_t(RowsParams& p, int maxtok, uint32_t ents, hipStream_t s) {
+    const uint32_t chunks = p.n * BITS / 128;
+    if ((p.n * BITS) % 128) return false;
+#define NVMAI_DENSE(SEG, NCH, RPI, ITERS)                                                          \
+    do {                                                                                           \
+        constexpr uint32_t rows_per_block = 4 * (64 / SEG) * RPI * ITERS;                          \
+        p.blocks_per_entry = (p.rows + rows_per_block - 1) / rows_per_block;                       \
+        const size_t lds = rows_fast_lds_bytes(p.n, NCH, SEG);                                     \
+        const dim3 grid(ents * p.blocks_per_entry);                                                \
+        if (maxtok == 1) expert_rows_fast<ACT, BITS, SEG, NCH, 1, false, false, RPI, ITERS, true><<<grid, 256, lds, s>>>(p); \
+        else expert_rows_fast<ACT, BITS, SEG, NCH, 4, false, false, RPI, ITERS, true><<<grid, 256, lds, s>>>(p);             \
+        return true;                                                                               \
+    } while (0)
+    const bool few = ents <= 40;      // the same block shapes as the work-list launches
+    if (few && chunks == 16) NVMAI_DENSE(16, 1, 1, 2);
+    if (few && chunks == 32) NVMAI_DENSE(32, 1, 2, 2);
+    if (chunks == 16) NVMAI_DENSE(16, 1, 2, 2);
+    if (chunks == 32) NVMAI_DENSE(32, 1, 4, 2);
+    if (chunks == 64) NVMAI_DENSE(64, 1, 2, 4);
+    if (chunks == 128) NVMAI_DENSE(64, 2, 1, 8);
+#undef NVMAI_DENSE
+    return false;
+}
+
+bool launch_dense_rows(int act, uint32_t bits, RowsParams& p, int maxtok, uint32_t ents, hipStream_t s) {
+    if (act == ACT_BF16) return bits == 8 ? launch_dense_rows_t<ACT_BF16, 8>(p, maxtok, ents, s)
+                                          : launch_dense_rows_t<ACT_BF16, 4>(p, maxtok, ents, s);
+    return bits == 8 ? launch_dense_rows_t<ACT_FP16, 8>(p, maxtok, ents, s)
+                     : launch_dense_rows_t<ACT_FP16, 4>(p, maxtok, ents, s);
+}
+
 int check_shape(uint32_t d, uint32_t f, uint32_t bits) {
     if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
     if (d == 0 || f == 0 || d % NVMAI_GROUP || f % NVMAI_GROUP) return NVMAI_ERR_INVALID_ARG;
@@ -383,6 +418,16 @@ int affine_gemv_any(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weig
     hipStream_t s = (hipStream_t)stream;
     const int maxtok = n_tokens == 1 ? 1 : MAX_TOK;
     const uint32_t ents = (n_tokens + maxtok - 1) / maxtok;
+    if (!x_is_f32) {
+        RowsParams p{};
+        p.src.slot[0] = weights;
+        p.sA = reinterpret_cast<const uint8_t*>(scales) - weights;
+        p.bA = reinterpret_cast<const uint8_t*>(biases) - weights;
+        p.x = x; p.x_stride = x_stride; p.rows = m; p.n = n;
+        p.out = y_f32; p.out_stride = y_stride; p.out_act = y; p.out_act_stride = y_stride;
+        p.dense_count = n_tokens;
+        if (launch_dense_rows(ctx->act, bits, p, maxtok, ents, s)) return launch_status();
+    }
     const bool need_tmp = (y != nullptr) || y_stride != m;
     size_t need = ws_round(ents * sizeof(WorkEntry)) + ws_round(16) + 2 * ws_round(n_tokens * 4u) +
                   (need_tmp ? ws_round((size_t)n_tokens * m * 4u) : 0);

@@ -45,6 +45,10 @@ struct RowsParams {
     uint32_t out_stride;
     uint32_t rows, n;            // matrix shape [rows, n]
     uint32_t blocks_per_entry;
+    // dense launches (one matrix against dense_count input rows, no work list in memory):
+    uint32_t dense_count;
+    void* out_act;               // optional 16-bit copy of the result, rows out_act_stride apart;
+    uint32_t out_act_stride;     // `out` may then be null
 };
 
 // ---- input staging ----------------------------------------------------------
@@ -171,14 +175,21 @@ __device__ __forceinline__ void pow2_scale(float amax, float& sc, float& isc) {
 // LDS: [ntok][n/8] uint4 packed inputs | [ntok][NCH*SEG][2] float chunk sums (all, odd pairs) |
 //      [MAX_TOK*4] float wave maxima | [MAX_TOK] float inverse scales.
 //
-// DIRECT (one input only): the entry itself names its rows -- input row we.reserved, output row
-// we.pair_start -- and the pair tables are not read (entries made inside the launch that uses them).
-template <int ACT, int BITS, int SEG, int NCH, int TOKS, bool DUAL, bool XF32, int RPI, int ITERS, bool DIRECT = false>
+// MODE says where an entry's rows are named (entries made inside the launch that uses them read
+// no pair tables).  ROWS_TABLES: p.pair_in / p.pair_out.  ROWS_DIRECT (one input only): input row
+// we.reserved, output row we.pair_start.  ROWS_DENSE: input and output row we.pair_start + t, and
+// the result goes to p.out (fp32) and / or p.out_act (16 bit), whichever is not null.
+constexpr int ROWS_TABLES = 0, ROWS_DIRECT = 1, ROWS_DENSE = 2;
+template <int ACT, int BITS, int SEG, int NCH, int TOKS, bool DUAL, bool XF32, int RPI, int ITERS, int MODE = ROWS_TABLES>
 __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const WorkEntry& we, uint32_t rb,
                                                  uint4* lds) {
-    static_assert(!DIRECT || TOKS == 1, "a direct entry holds one input");
-    auto in_row = [&](int t) -> uint32_t { return DIRECT ? we.reserved : p.pair_in[we.pair_start + t]; };
-    auto out_row_of = [&](int t) -> uint32_t { return DIRECT ? we.pair_start : p.pair_out[we.pair_start + t]; };
+    static_assert(MODE != ROWS_DIRECT || TOKS == 1, "a direct entry holds one input");
+    auto in_row = [&](int t) -> uint32_t {
+        return MODE == ROWS_DIRECT ? we.reserved : MODE == ROWS_DENSE ? we.pair_start + t : p.pair_in[we.pair_start + t];
+    };
+    auto out_row_of = [&](int t) -> uint32_t {
+        return MODE == ROWS_DIRECT ? we.pair_start : MODE == ROWS_DENSE ? we.pair_start + t : p.pair_out[we.pair_start + t];
+    };
     constexpr int EPC = Chunk<BITS>::elems;
     constexpr int PAIRS = EPC / 2;                // packed pairs per chunk
     constexpr int H = PAIRS / 4;                  // 16-byte LDS words per chunk
@@ -384,8 +395,11 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
                     const float u = seg_reduce_sum<SEG>(accB) * isc;
                     v = silu_fast(a) * u; // moe.metal:134-139 (silu branch), CPUExpertFFN.swift:122-124
                 }
-                if (seg_result_lane<SEG>(lane) && row < p.rows)
-                    p.out[(size_t)out_row * p.out_stride + row] = v;
+                if (seg_result_lane<SEG>(lane) && row < p.rows) {
+                    if (MODE != ROWS_DENSE || p.out) p.out[(size_t)out_row * p.out_stride + row] = v;
+                    if (MODE == ROWS_DENSE && p.out_act)
+                        ((uint16_t*)p.out_act)[(size_t)out_row * p.out_act_stride + row] = f32_to_act<ACT>(v);
+                }
             }
         }
     };
@@ -407,17 +421,28 @@ __host__ __device__ inline size_t rows_fast_lds_bytes(uint32_t n, int nch, int s
 // MAXTOK = 1: single-input launches.  MAXTOK = 4: the body is chosen by the
 // entry's pair count (uniform per block), so an expert routed to by one token
 // does not pay for more.
-template <int ACT, int BITS, int SEG, int NCH, int MAXTOK, bool DUAL, bool XF32, int RPI, int ITERS>
+// DENSE: the matrix in blob slot 0 against the input rows 0 .. dense_count - 1, entry e = the
+// rows e * MAXTOK .. (a grid of exactly that many entries; no work list, no pair tables).
+template <int ACT, int BITS, int SEG, int NCH, int MAXTOK, bool DUAL, bool XF32, int RPI, int ITERS, bool DENSE = false>
 __global__ __launch_bounds__(256) void expert_rows_fast(RowsParams p) {
     extern __shared__ uint4 rows_lds[];
     const uint32_t entry = blockIdx.x / p.blocks_per_entry;
-    if (entry >= *p.n_entries) return;
     const uint32_t rb = blockIdx.x % p.blocks_per_entry;
-    const WorkEntry we = p.entries[entry];
+    constexpr int MODE = DENSE ? ROWS_DENSE : ROWS_TABLES;
+    WorkEntry we;
+    if (DENSE) {
+        we.expert = NVMAI_SLOT_FLAG;
+        we.pair_start = entry * MAXTOK;
+        we.pair_count = min((uint32_t)MAXTOK, p.dense_count - entry * MAXTOK);
+        we.reserved = 0;
+    } else {
+        if (entry >= *p.n_entries) return;
+        we = p.entries[entry];
+    }
     if (MAXTOK == 1 || we.pair_count == 1)
-        expert_rows_body<ACT, BITS, SEG, NCH, 1, DUAL, XF32, RPI, ITERS>(p, we, rb, rows_lds);
+        expert_rows_body<ACT, BITS, SEG, NCH, 1, DUAL, XF32, RPI, ITERS, MODE>(p, we, rb, rows_lds);
     else
-        expert_rows_body<ACT, BITS, SEG, NCH, 0, DUAL, XF32, RPI, ITERS>(p, we, rb, rows_lds);
+        expert_rows_body<ACT, BITS, SEG, NCH, 0, DUAL, XF32, RPI, ITERS, MODE>(p, we, rb, rows_lds);
 }
 
 // ---- generic engine -----------------------------------------------------------
@@ -1089,7 +1114,7 @@ __global__ __launch_bounds__(256) void expert_rows_routed(RowsParams p, SelectPa
         we.expert = NVMAI_SLOT_FLAG | 8u;
         we.pair_start = sel.tokens * sel.top_k + t;
     }
-    expert_rows_body<ACT, BITS, SEG, NCH, 1, true, false, RPI, ITERS, true>(p, we, rb, rows_lds);
+    expert_rows_body<ACT, BITS, SEG, NCH, 1, true, false, RPI, ITERS, ROWS_DIRECT>(p, we, rb, rows_lds);
     // The caller's statistics, off the critical path: the first block counts the distinct experts
     // of the step once its rows are done (at most four tokens, tokens * top_k <= 64 indices).
     if (rs.stats && blockIdx.x == 0 && t == 0) {

@@ -111,11 +111,19 @@ def pack_expert(ctx, gate, up, down, bits, blob=None):
     return blob
 
 
-def affine_gemv(ctx, weights, scales, biases, bits, x, m, n, out_f32=False):
+def affine_gemv(ctx, weights, scales, biases, bits, x, m, n, out_f32=False, y=None, y_f32=None):
     """DequantInt4GEMV.encode / DequantInt8GEMV.encode / AffineQuantGEMV.encode:
-    y[t] = W x[t] for x [tokens, n]."""
+    y[t] = W x[t] for x [tokens, n].  y (activation type) and / or y_f32 may be handed in as
+    [tokens, >= m] buffers with one common row stride; both are then written and returned."""
     x2 = x.reshape(-1, x.shape[-1])
     tokens = x2.shape[0]
+    if y is not None or y_f32 is not None:
+        stride = (y if y is not None else y_f32).stride(0)
+        assert y is None or y_f32 is None or y.stride(0) == y_f32.stride(0)
+        check(lib.nvmai_hip_affine_gemv(ctx.handle, _stream(), _ptr(weights), _ptr(scales), _ptr(biases), bits,
+                                        _ptr(x2), x2.stride(0), tokens, m, n, _ptr(y), _ptr(y_f32), stride),
+              "affine_gemv")
+        return y, y_f32
     y = None if out_f32 else torch.empty((tokens, m), dtype=ctx.dtype, device=x.device)
     yf = torch.empty((tokens, m), dtype=torch.float32, device=x.device) if out_f32 else None
     check(lib.nvmai_hip_affine_gemv(ctx.handle, _stream(), _ptr(weights), _ptr(scales), _ptr(biases), bits,

@@ -83,6 +83,28 @@ def test_affine_gemv_matches_oracle(nv, ctx, bits, m, n, tokens):
     assert O.rel_error(act_np(y16), want) < TOL_ACT
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_affine_gemv_both_outputs_padded_stride(nv, ctx, bits):
+    # 16-bit and fp32 results in one call, rows of the outputs further apart than m; shapes with a
+    # single-launch instantiation (any chunk count 16 / 32 / 64 / 128) and one without (n = 192)
+    rng = np.random.default_rng(90 + bits)
+    per = 128 // bits
+    for m, n, tokens in [(70, 16 * per, 1), (130, 32 * per, 3), (64, 64 * per, 4), (33, 128 * per, 9), (40, 192, 2)]:
+        say("gemv padded", ctx.act, bits, m, n, tokens)
+        p, s, b = O.quantize_affine(gauss(rng, (m, n), 0.05), bits)
+        x = round_act(gauss(rng, (tokens, n)), ctx.act)
+        want = np.stack([O.affine_gemv(p, s, b, x[t], bits) for t in range(tokens)])
+        stride = m + 24
+        y = torch.full((tokens, stride), 7.0, dtype=ctx.dtype, device="cuda")
+        yf = torch.full((tokens, stride), 7.0, dtype=torch.float32, device="cuda")
+        nv.affine_gemv(ctx, dev(p), dev(s.view(np.int16)), dev(b.view(np.int16)), bits, act_tensor(x, ctx), m, n,
+                       y=y, y_f32=yf)
+        torch.cuda.synchronize()
+        assert O.rel_error(yf[:, :m].cpu().numpy(), want) < TOL_F32
+        assert O.rel_error(act_np(y[:, :m]), want) < TOL_ACT
+        assert (yf[:, m:] == 7.0).all() and (y[:, m:].float() == 7.0).all()     # padding untouched
+
+
 def test_gemv_bitstream_known_answer(nv, ctx_bf16):
     # AffineQuantTests.swift:35-56: value=(row*11+col*3)&mask, scale 1, bias 0, x=1 => sum(values)
     for bits in (4, 8):
