@@ -414,12 +414,24 @@ def run_sampler(nv, ctx, torch, a):
     ev[1].record()
     torch.cuda.synchronize()
     gemv_us = ev[0].elapsed_time(ev[1]) / a.steps * 1e3
+    # the fused greedy head (RMSNorm + one logit per row + argmax) over the same matrices, by events
+    chain = nv.LMHeadChain(ctx, bits)
+    norm_w = torch.full((D,), 0x3F80, dtype=torch.int16, device="cuda")
+    toks = torch.empty(rows, dtype=torch.int32, device="cuda")
+    for i in range(a.warmup):
+        chain.encode_greedy_decode(xs[i % 8], norm_w, *heads[i % n_heads], D, V, out=toks)
+    ev[0].record()
+    for i in range(a.steps):
+        chain.encode_greedy_decode(xs[i % 8], norm_w, *heads[i % n_heads], D, V, out=toks)
+    ev[1].record()
+    torch.cuda.synchronize()
+    greedy_us = ev[0].elapsed_time(ev[1]) / a.steps * 1e3
     ctx.profile_enable(True)
     for i in range(a.steps):
         step(i)
     torch.cuda.synchronize()
     ctx.profile_enable(False)
-    kern = {"lm_head_gemv": gemv_us}
+    kern = {"lm_head_gemv": gemv_us, "lm_head_greedy_fused": greedy_us}
     for tag, name in ((nv.PROF_SOFTMAX, "softmax"), (nv.PROF_SAMPLE, "sample_topk64")):
         ms, n = ctx.profile_read(tag)
         kern[name] = ms / max(n, 1) * 1e3

@@ -373,6 +373,39 @@ int nvmai_hip_sample(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint16_t* pr
                      uint32_t top_k, float top_p, const uint64_t* seeds, const uint32_t* positions,
                      uint32_t* out_token);
 
+/* ---- the small operators around the MoE block of a decode step ---------------------------- */
+
+/* RMSNorm.encodeBF16W / encodeNoScale / encodeBF16WPerHead / encodeNoScalePerHead
+ * (RMSNorm.swift:52-142; kernels rmsnorm.metal:64-175): out[r] = x[r] * inv_r * weight with
+ * inv_r = 1 / sqrt(mean(x[r]^2) + eps), fp32 arithmetic, 16-bit activations in and out; row r
+ * at x + r * x_stride elements (the per-head kernels: rows = heads, strides = head_dim).
+ * weight: BF16 [d] shared by all rows, NULL = no scale.  out may be x (in place). */
+int nvmai_hip_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* x, uint32_t x_stride,
+                      const uint16_t* weight, void* out, uint32_t out_stride, uint32_t rows,
+                      uint32_t d, float eps);
+
+/* AffineQuantEmbeddingLookup.encode (kernel embed_lookup_int4, dequant_int4.metal:63-91; a block
+ * of tokens: prefill_embed_lookup_affine_block, prefill.metal:59): out[t] = (q * scale + bias) *
+ * out_scale for row token[t] of a 4- or 8-bit affine table [vocab, d]; a token id >= vocab gives
+ * a row of zeros.  token_ids: device array of n_tokens ids, or NULL = the single id `token_id`
+ * for every row (the reference passes the id by value). */
+int nvmai_hip_embed_lookup(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* table,
+                           const uint16_t* scales, const uint16_t* biases, uint32_t bits,
+                           const uint32_t* token_ids, uint32_t token_id, uint32_t n_tokens, void* out,
+                           uint32_t out_stride, uint32_t d, uint32_t vocab, float out_scale);
+
+/* LMHeadChainInt4.encodeGreedyDecode (LMHeadChainInt4.swift:58-130; kernels rmsnorm_bf16w,
+ * lm_head_greedy_int4_rows_chunk_raw, lm_head_greedy_int4_rows_reduce, logit.metal:761-937):
+ * out_tokens[t] = argmax over the rows of a 4- or 8-bit affine LM head [vocab, d] of
+ * W[row] . RMSNorm(hidden[t]), over the finite logits only, ties to the lower index, 0 when no
+ * logit is finite.  norm_weight: BF16 [d], NULL = hidden is used as it is.  Rows of at most
+ * 2048 bytes (d <= 2048 at 8 bit, 4096 at 4 bit). */
+int nvmai_hip_lm_head_greedy(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* hidden,
+                             uint32_t hidden_stride, uint32_t n_tokens, const uint16_t* norm_weight,
+                             const uint8_t* weights, const uint16_t* scales, const uint16_t* biases,
+                             uint32_t bits, uint32_t* out_tokens, uint32_t d, uint32_t vocab,
+                             float rms_eps);
+
 /* Sampler.seedFor (Sampler.swift:304-325): splitmix64(seed + position), 0 mapped away. */
 uint64_t nvmai_sampler_seed_for(uint64_t seed, int64_t position);
 

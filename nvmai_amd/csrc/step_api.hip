@@ -1,0 +1,79 @@
+// Entry points: RMSNorm, affine embedding lookup, fused greedy LM head.
+#include "ctx.hpp"
+#include "step_kernels.cuh"
+
+using namespace nvmai;
+
+extern "C" int nvmai_hip_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* x, uint32_t x_stride,
+                                 const uint16_t* weight, void* out, uint32_t out_stride, uint32_t rows,
+                                 uint32_t d, float eps) {
+    if (!ctx || !x || !out || d == 0 || x_stride < d || out_stride < d) return NVMAI_ERR_INVALID_ARG;
+    if (rows == 0) return NVMAI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((rows + 3) / 4);
+    if (ctx->act == ACT_BF16)
+        rmsnorm_kernel<ACT_BF16><<<grid, 256, 0, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);
+    else
+        rmsnorm_kernel<ACT_FP16><<<grid, 256, 0, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_embed_lookup(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* table,
+                                      const uint16_t* scales, const uint16_t* biases, uint32_t bits,
+                                      const uint32_t* token_ids, uint32_t token_id, uint32_t n_tokens, void* out,
+                                      uint32_t out_stride, uint32_t d, uint32_t vocab, float out_scale) {
+    if (!ctx || !table || !scales || !biases || !out) return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    if (d == 0 || d % NVMAI_GROUP || out_stride < d) return NVMAI_ERR_INVALID_ARG;
+    if (n_tokens == 0) return NVMAI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((d / 8 + 255) / 256, n_tokens);
+    if (ctx->act == ACT_BF16)
+        embed_lookup_kernel<ACT_BF16><<<grid, 256, 0, s>>>(table, scales, biases, bits, token_ids, token_id, (uint16_t*)out, out_stride, d, vocab, out_scale);
+    else
+        embed_lookup_kernel<ACT_FP16><<<grid, 256, 0, s>>>(table, scales, biases, bits, token_ids, token_id, (uint16_t*)out, out_stride, d, vocab, out_scale);
+    return launch_status();
+}
+
+namespace {
+
+template <int ACT, int BITS>
+void launch_lm_head(const LmHeadParams& p, uint32_t cpl, dim3 grid, hipStream_t s) {
+    const size_t lds = ((size_t)p.d + 16) * 4 + (size_t)p.d * 4;   // floats, block results, two 16-bit rows
+    if (cpl <= 1) lm_head_greedy_kernel<ACT, BITS, 1><<<grid, 256, lds, s>>>(p);
+    else if (cpl <= 2) lm_head_greedy_kernel<ACT, BITS, 2><<<grid, 256, lds, s>>>(p);
+    else lm_head_greedy_kernel<ACT, BITS, 4><<<grid, 256, lds, s>>>(p);
+}
+
+}  // namespace
+
+extern "C" int nvmai_hip_lm_head_greedy(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* hidden,
+                                        uint32_t hidden_stride, uint32_t n_tokens, const uint16_t* norm_weight,
+                                        const uint8_t* weights, const uint16_t* scales, const uint16_t* biases,
+                                        uint32_t bits, uint32_t* out_tokens, uint32_t d, uint32_t vocab,
+                                        float rms_eps) {
+    if (!ctx || !hidden || !weights || !scales || !biases || !out_tokens) return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    if (d == 0 || d % NVMAI_GROUP || hidden_stride < d || vocab == 0) return NVMAI_ERR_INVALID_ARG;   // LMHeadChainInt4.swift:76-77
+    const uint32_t chunks = d * bits / 128;        // d is a multiple of 64: whole 16-byte chunks
+    const uint32_t cpl = (chunks + 31) / 32;
+    if (cpl > 4) return NVMAI_ERR_UNSUPPORTED;     // rows of at most 2048 bytes
+    if (!aligned16(weights)) return NVMAI_ERR_ALIGNMENT;
+    if (n_tokens == 0) return NVMAI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const uint32_t n_blocks = (vocab + LMH_ROWS - 1) / LMH_ROWS;
+    int rc = ws_begin(ctx, ws_round((size_t)n_tokens * n_blocks * sizeof(float2)));
+    if (rc) return rc;
+    LmHeadParams p{};
+    p.hidden = (const uint16_t*)hidden; p.hidden_stride = hidden_stride; p.norm_weight = norm_weight;
+    p.weights = weights; p.scales = scales; p.biases = biases; p.d = d; p.vocab = vocab; p.eps = rms_eps;
+    p.summaries = ws_take<float2>(ctx, (size_t)n_tokens * n_blocks);
+    const dim3 grid(n_blocks, n_tokens);
+    if (ctx->act == ACT_BF16) {
+        if (bits == 8) launch_lm_head<ACT_BF16, 8>(p, cpl, grid, s); else launch_lm_head<ACT_BF16, 4>(p, cpl, grid, s);
+    } else {
+        if (bits == 8) launch_lm_head<ACT_FP16, 8>(p, cpl, grid, s); else launch_lm_head<ACT_FP16, 4>(p, cpl, grid, s);
+    }
+    lm_head_reduce_kernel<<<n_tokens, 256, 0, s>>>(p.summaries, n_blocks, out_tokens);
+    return launch_status();
+}

@@ -1,0 +1,261 @@
+// The small operators around the MoE block of a decode step: RMSNorm, affine embedding lookup,
+// and the fused greedy LM head (RMSNorm -> one logit per vocabulary row -> argmax).  gfx950.
+#pragma once
+
+#include "common.cuh"
+
+namespace nvmai {
+
+// ---- RMSNorm -------------------------------------------------------------------------
+// y = x * inv * w, inv = 1 / sqrt(mean(x^2) + eps) (rmsnorm.metal:31-62, 83-87); no weight:
+// y = x * inv (:152-175).  A row may be one head of a [heads, head_dim] vector (:101-148).
+// One wave per row.  The sum of squares has a fixed order so that a CPU run of the same order
+// gives the same bits: lane l runs acc = fma(x, x, acc) over the elements l, l + 64, ...,
+// then an xor butterfly 32, 16, 8, 4, 2, 1; every later step is one IEEE operation.
+__device__ __forceinline__ float rms_wave_sum(float acc) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) acc = __fadd_rn(acc, shfl_xor_f(acc, off));
+    return acc;
+}
+
+__device__ __forceinline__ float rms_inverse(float sum, uint32_t d, float eps) {
+    const float mean = __fdiv_rn(sum, (float)d);
+    return __fdiv_rn(1.0f, sqrtf(__fadd_rn(mean, eps)));     // sqrtf: correctly rounded (the _rn intrinsic is not)
+}
+
+template <int ACT>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* x, uint32_t x_stride, const uint16_t* weight,
+                                                      uint16_t* out, uint32_t out_stride, uint32_t rows, uint32_t d,
+                                                      float eps) {
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;                       // uniform per wave
+    const uint32_t lane = threadIdx.x & 63;
+    const uint16_t* xr = x + (size_t)row * x_stride;
+    float acc = 0.0f;
+    for (uint32_t i = lane; i < d; i += 64) {
+        const float v = act_to_f32<ACT>(xr[i]);
+        acc = fmaf(v, v, acc);
+    }
+    const float inv = rms_inverse(rms_wave_sum(acc), d, eps);
+    uint16_t* o = out + (size_t)row * out_stride;
+    for (uint32_t i = lane; i < d; i += 64) {       // in place is fine: a lane rereads only what it writes
+        float v = __fmul_rn(act_to_f32<ACT>(xr[i]), inv);
+        if (weight) v = __fmul_rn(v, bf16_to_f32(weight[i]));
+        o[i] = f32_to_act<ACT>(v);
+    }
+}
+
+// ---- embedding lookup ------------------------------------------------------------------
+// out[t, i] = ((float(q) * s + b) * out_scale) for row token[t] of a 4- or 8-bit affine table,
+// zeros for a token id at or past vocab (dequant_int4.metal:63-91; a block of tokens:
+// prefill.metal:59).  One thread per eight elements.
+template <int ACT>
+__global__ __launch_bounds__(256) void embed_lookup_kernel(const uint8_t* table, const uint16_t* scales,
+                                                           const uint16_t* biases, uint32_t bits,
+                                                           const uint32_t* token_ids, uint32_t token_id,
+                                                           uint16_t* out, uint32_t out_stride, uint32_t d,
+                                                           uint32_t vocab, float out_scale) {
+    const uint32_t t = blockIdx.y;
+    const uint32_t e0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (e0 >= d) return;
+    const uint32_t tok = token_ids ? token_ids[t] : token_id;
+    uint16_t* o = out + (size_t)t * out_stride + e0;
+    const uint32_t n = min(8u, d - e0);
+    if (tok >= vocab) {
+        for (uint32_t j = 0; j < n; ++j) o[j] = 0;
+        return;
+    }
+    const uint32_t groups = d / NVMAI_GROUP;
+    const uint8_t* row = table + (size_t)tok * ((size_t)d * bits / 8);
+    const float s = bf16_to_f32(scales[(size_t)tok * groups + e0 / NVMAI_GROUP]);
+    const float b = bf16_to_f32(biases[(size_t)tok * groups + e0 / NVMAI_GROUP]);
+    for (uint32_t j = 0; j < n; ++j) {
+        const uint32_t e = e0 + j;
+        const uint32_t q = bits == 8 ? row[e] : ((row[e >> 1] >> ((e & 1u) * 4u)) & 0xFu);
+        o[j] = f32_to_act<ACT>(__fmul_rn(__fadd_rn(__fmul_rn((float)q, s), b), out_scale));
+    }
+}
+
+// ---- greedy LM head ------------------------------------------------------------------------
+// LMHeadChainInt4.encodeGreedyDecode (LMHeadChainInt4.swift:58-130; kernels logit.metal:761-937):
+// token = argmax over the vocabulary rows of W[row] . norm(hidden), finite logits only, ties to
+// the lower index, 0 when no logit is finite.  The RMSNorm is done inside every block (the row
+// is a few KB) and rounded to the activation type as the reference stores it.
+//
+// One half-wave (32 lanes) per vocabulary row, in the same fixed order as the router logits so
+// that the token can be compared with a CPU run of that order: lane l owns the 16-byte chunks
+// l, l + 32, ... of the row; in a chunk dot = fma(q, x, dot) and xs = xs + x run in element
+// order, then acc = fma(s, dot, acc), acc = fma(b, xs, acc); xor butterfly 16, 8, 4, 2, 1.
+// A lane's inputs and their chunk sums do not depend on the row: they are fetched once per block
+// into registers, and the block walks LMH_ROWS rows, the next row's codes in flight while the
+// current one is summed.  Each block leaves (best logit, index) and a second small launch picks
+// the winner.
+constexpr uint32_t LMH_ROWS = 64;                 // rows per block: 8 per half-wave
+constexpr int LMH_STEPS = LMH_ROWS / 8;
+
+struct LmHeadParams {
+    const uint16_t* hidden;       // [tokens, hidden_stride] activations
+    uint32_t hidden_stride;
+    const uint16_t* norm_weight;  // optional bf16 [d]
+    const uint8_t* weights;       // [vocab, d * bits / 8]
+    const uint16_t* scales;       // bf16 [vocab, d / 64]
+    const uint16_t* biases;
+    uint32_t d, vocab;
+    float eps;
+    float2* summaries;            // [tokens, gridDim.x] (best logit, index bits)
+};
+
+template <int ACT, int BITS, int CPL>
+__global__ __launch_bounds__(256) void lm_head_greedy_kernel(LmHeadParams p) {
+    constexpr int EPC = Chunk<BITS>::elems;
+    // LDS: [d] normed inputs as floats | 16 words of block results | [d] hidden row, [d] norm weight (16 bit)
+    extern __shared__ float lmh_lds[];
+    float* xn = lmh_lds;
+    uint16_t* hraw = reinterpret_cast<uint16_t*>(lmh_lds + p.d + 16);
+    uint16_t* wraw = hraw + p.d;
+    const uint32_t t = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
+    const uint16_t* h = p.hidden + (size_t)t * p.hidden_stride;
+
+    const uint32_t hw = tid >> 5, hl = tid & 31;
+    const uint32_t chunks = p.d * BITS / 128, groups = p.d / NVMAI_GROUP, row_bytes = p.d * BITS / 8;
+    const uint32_t row0 = blockIdx.x * LMH_ROWS;
+    const uint32_t row_end = min(row0 + LMH_ROWS, p.vocab);
+    uint4 q[3][CPL];
+    uint16_t sc[3][CPL], bi[3][CPL];
+    auto load_row = [&](int buf, uint32_t row) {
+        row = min(row, p.vocab - 1);
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+            const uint32_t chunk = min(hl + 32 * c, chunks - 1);    // a lane without a chunk loads the last one
+            q[buf][c] = *reinterpret_cast<const uint4*>(p.weights + (size_t)row * row_bytes + chunk * 16);
+            const uint32_t g = chunk * EPC / NVMAI_GROUP;
+            sc[buf][c] = p.scales[(size_t)row * groups + g];
+            bi[buf][c] = p.biases[(size_t)row * groups + g];
+        }
+    };
+    load_row(0, row0 + hw);                       // in flight while the inputs are prepared
+    load_row(1, row0 + hw + 8);
+
+    // The row and the norm weight reach LDS in one round trip (16-byte loads where the row is
+    // aligned); everything after reads LDS.  Read straight from memory, the strided sum below
+    // would be a chain of dependent round trips at the start of every block.
+    const bool vec = ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(p.norm_weight)) & 15u) == 0 &&
+                     p.d % 8 == 0;
+    if (vec) {
+        for (uint32_t i = tid; i < p.d / 8; i += 256) {
+            reinterpret_cast<uint4*>(hraw)[i] = reinterpret_cast<const uint4*>(h)[i];
+            if (p.norm_weight) reinterpret_cast<uint4*>(wraw)[i] = reinterpret_cast<const uint4*>(p.norm_weight)[i];
+        }
+    } else {
+        for (uint32_t i = tid; i < p.d; i += 256) {
+            hraw[i] = h[i];
+            if (p.norm_weight) wraw[i] = p.norm_weight[i];
+        }
+    }
+    __syncthreads();
+    float inv = 1.0f;
+    if (p.norm_weight) {
+        float acc = 0.0f;
+        for (uint32_t i = lane; i < p.d; i += 64) {
+            const float v = act_to_f32<ACT>(hraw[i]);
+            acc = fmaf(v, v, acc);
+        }
+        inv = rms_inverse(rms_wave_sum(acc), p.d, p.eps);     // every wave for itself, the same bits
+    }
+    for (uint32_t i = tid; i < p.d; i += 256) {
+        float v = act_to_f32<ACT>(hraw[i]);
+        if (p.norm_weight)
+            v = act_to_f32<ACT>(f32_to_act<ACT>(__fmul_rn(__fmul_rn(v, inv), bf16_to_f32(wraw[i]))));
+        xn[i] = v;
+    }
+    __syncthreads();
+
+    float xr[CPL][EPC], xs[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+        const uint32_t chunk = hl + 32 * c;
+        xs[c] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPC; ++e) {
+            xr[c][e] = chunk < chunks ? xn[chunk * EPC + e] : 0.0f;
+            xs[c] = __fadd_rn(xs[c], xr[c][e]);
+        }
+    }
+
+    float best_v = -INFINITY;
+    uint32_t best_i = 0xFFFFFFFFu;
+    auto sum_row = [&](int buf, uint32_t row) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+            if (hl + 32 * c < chunks) {
+                float qf[EPC];
+                unpack_chunk<BITS>(q[buf][c], qf);
+                float dot = 0.0f;
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) dot = fmaf(qf[e], xr[c][e], dot);
+                acc = fmaf(bf16_to_f32(sc[buf][c]), dot, acc);
+                acc = fmaf(bf16_to_f32(bi[buf][c]), xs[c], acc);
+            }
+        }
+#pragma unroll
+        for (int off = 16; off >= 1; off >>= 1) acc = __fadd_rn(acc, shfl_xor_f(acc, off));
+        // rows ascend inside a half-wave: a later equal logit never replaces an earlier one
+        if (row < row_end && isfinite(acc) && (best_i == 0xFFFFFFFFu || acc > best_v)) { best_v = acc; best_i = row; }
+    };
+    // Three register buffers: two rows of codes in flight while one is summed.  Every half-wave
+    // takes the same number of steps and every step loads (a row past the end loads the last row
+    // again and is not counted), so the loop unrolls into straight code in which the compiler
+    // can count the loads in flight; with conditional loads it waited for all of them each step.
+#pragma unroll
+    for (int k = 0; k < LMH_STEPS; ++k) {
+        if (k + 2 < LMH_STEPS) load_row((k + 2) % 3, row0 + hw + 8 * (k + 2));
+        sum_row(k % 3, row0 + hw + 8 * k);
+    }
+    float* res_v = lmh_lds + p.d;
+    uint32_t* res_i = reinterpret_cast<uint32_t*>(lmh_lds + p.d + 8);
+    if (hl == 0) { res_v[hw] = best_v; res_i[hw] = best_i; }
+    __syncthreads();
+    if (tid == 0) {
+        float bv = -INFINITY;
+        uint32_t bidx = 0xFFFFFFFFu;
+        for (int k = 0; k < 8; ++k) {             // half-wave k owns rows row0 + k, + 8, ...: compare indices
+            const float v = res_v[k];
+            const uint32_t i = res_i[k];
+            if (i != 0xFFFFFFFFu && (bidx == 0xFFFFFFFFu || v > bv || (v == bv && i < bidx))) { bv = v; bidx = i; }
+        }
+        p.summaries[(size_t)t * gridDim.x + blockIdx.x] = make_float2(bv, __uint_as_float(bidx));
+    }
+}
+
+// The winner among the block results of one token (logit.metal:890-937): one block per token.
+__global__ __launch_bounds__(256) void lm_head_reduce_kernel(const float2* summaries, uint32_t n_blocks,
+                                                             uint32_t* out_tokens) {
+    __shared__ float sv[256];
+    __shared__ uint32_t si[256];
+    const uint32_t t = blockIdx.x, tid = threadIdx.x;
+    float bv = -INFINITY;
+    uint32_t bidx = 0xFFFFFFFFu;
+    for (uint32_t k = tid; k < n_blocks; k += 256) {
+        const float2 s = summaries[(size_t)t * n_blocks + k];
+        const uint32_t i = __float_as_uint(s.y);
+        if (i != 0xFFFFFFFFu && (bidx == 0xFFFFFFFFu || s.x > bv || (s.x == bv && i < bidx))) { bv = s.x; bidx = i; }
+    }
+    sv[tid] = bv;
+    si[tid] = bidx;
+    __syncthreads();
+    for (uint32_t w = 128; w >= 1; w >>= 1) {
+        if (tid < w) {
+            const float v = sv[tid + w];
+            const uint32_t i = si[tid + w];
+            if (i != 0xFFFFFFFFu && (si[tid] == 0xFFFFFFFFu || v > sv[tid] || (v == sv[tid] && i < si[tid]))) {
+                sv[tid] = v;
+                si[tid] = i;
+            }
+        }
+        __syncthreads();
+    }
+    if (tid == 0) out_tokens[t] = si[0] == 0xFFFFFFFFu ? 0u : si[0];
+}
+
+}  // namespace nvmai

@@ -570,3 +570,68 @@ class Sample:
                                    top_k, top_p, _seed_array(seed, rows), (C.c_uint32 * rows)(*pos), _ptr(out)),
               "sample")
         return out
+
+
+class RMSNorm:
+    """Mirror of RMSNorm (RMSNorm.swift:20-142): x [rows, d] (rows = 1, or heads for the per-head
+    calls); weight: BF16 bits as an int16 tensor [d], or None."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+
+    def _run(self, x, weight, out, eps):
+        x2 = x.reshape(-1, x.shape[-1])
+        if out is None:
+            out = torch.empty_like(x2)
+        o2 = out.reshape(-1, out.shape[-1])
+        check(lib.nvmai_hip_rmsnorm(self.ctx.handle, _stream(), _ptr(x2), x2.stride(0), _ptr(weight), _ptr(o2),
+                                    o2.stride(0), x2.shape[0], x2.shape[1], eps), "rmsnorm")
+        return out
+
+    def encode_bf16w(self, x, weight, out=None, eps=1e-6):
+        return self._run(x, weight, out, eps)
+
+    def encode_no_scale(self, x, out=None, eps=1e-6):
+        return self._run(x, None, out, eps)
+
+    encode_bf16w_per_head = encode_bf16w
+    encode_no_scale_per_head = encode_no_scale
+
+
+class AffineQuantEmbeddingLookup:
+    """Mirror of AffineQuantEmbeddingLookup: rows of a 4- or 8-bit affine table as activations."""
+
+    def __init__(self, ctx, weight_bits):
+        if weight_bits not in (4, 8):
+            raise _lib.NvmaiError(-2, "AffineQuantEmbeddingLookup(weightBits=%d)" % weight_bits)
+        self.ctx, self.bits = ctx, weight_bits
+
+    def encode(self, table, scales, biases, token_ids, d, vocab, out_scale=1.0, out=None):
+        """token_ids: an int (one row) or an int32 device tensor [n]."""
+        single = not torch.is_tensor(token_ids)
+        n = 1 if single else token_ids.numel()
+        if out is None:
+            out = torch.empty((n, d), dtype=self.ctx.dtype, device=table.device)
+        check(lib.nvmai_hip_embed_lookup(self.ctx.handle, _stream(), _ptr(table), _ptr(scales), _ptr(biases), self.bits,
+                                         None if single else _ptr(token_ids), int(token_ids) if single else 0, n,
+                                         _ptr(out), out.stride(0), d, vocab, out_scale), "embed_lookup")
+        return out
+
+
+class LMHeadChain:
+    """Mirror of LMHeadChainInt4.encodeGreedyDecode (LMHeadChainInt4.swift:58-130) for 4- and
+    8-bit heads: RMSNorm, one logit per vocabulary row, argmax."""
+
+    def __init__(self, ctx, weight_bits=4):
+        if weight_bits not in (4, 8):
+            raise _lib.NvmaiError(-2, "LMHeadChain(weightBits=%d)" % weight_bits)
+        self.ctx, self.bits = ctx, weight_bits
+
+    def encode_greedy_decode(self, hidden, norm_weight, weights, scales, biases, d, vocab, rms_eps=1e-6, out=None):
+        h = hidden.reshape(-1, hidden.shape[-1])
+        if out is None:
+            out = torch.empty(h.shape[0], dtype=torch.int32, device=h.device)
+        check(lib.nvmai_hip_lm_head_greedy(self.ctx.handle, _stream(), _ptr(h), h.stride(0), h.shape[0],
+                                           _ptr(norm_weight), _ptr(weights), _ptr(scales), _ptr(biases), self.bits,
+                                           _ptr(out), d, vocab, rms_eps), "lm_head_greedy")
+        return out

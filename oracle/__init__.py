@@ -82,6 +82,10 @@ _sig("orc_gumbel_for", C.c_float, C.c_uint64, C.c_uint32, C.c_uint32)
 _sig("orc_sample_topk64", C.c_uint32, u16p, size_t, C.c_float, C.c_float, C.c_uint64,
      C.c_uint32, C.c_void_p, C.c_void_p)
 _sig("orc_rel_error", C.c_float, f32p, f32p, size_t)
+_sig("orc_rmsnorm", None, f32p, size_t, C.c_void_p, size_t, size_t, C.c_float, f32p, size_t)
+_sig("orc_embed_lookup", None, u8p, u16p, u16p, C.c_int, C.c_uint32, size_t, size_t, C.c_float, f32p)
+_sig("orc_lm_head_greedy", C.c_uint32, f32p, C.c_void_p, u8p, u16p, u16p, C.c_int, size_t, size_t,
+     C.c_float, C.c_int, C.c_void_p)
 
 GROUP = 64
 
@@ -449,6 +453,36 @@ def sample_topk64(probs_f16, temperature, top_p, seed, top_k=64, want_top64=Fals
 
 def seed_for(seed, position):
     return lib.orc_seed_for(seed, position)
+
+
+# ---------------------------------------------------------------- rest of the decode step
+def rmsnorm(x, weight_bf16=None, eps=1e-6):
+    """x [rows, d] float32 (contiguous); weight_bf16: uint16 [d] or None.  Returns float32 [rows, d]."""
+    x = np.ascontiguousarray(x, np.float32)
+    x2 = x.reshape(-1, x.shape[-1])
+    out = np.zeros_like(x2)
+    w = None if weight_bf16 is None else np.ascontiguousarray(weight_bf16, np.uint16)
+    lib.orc_rmsnorm(x2, x2.shape[1], _ptr(w), x2.shape[0], x2.shape[1], eps, out, x2.shape[1])
+    return out.reshape(x.shape)
+
+
+def embed_lookup(table, scales, biases, bits, token, out_scale=1.0):
+    vocab, d = table.shape[0], table.shape[1] * 8 // bits
+    out = np.zeros(d, np.float32)
+    lib.orc_embed_lookup(np.ascontiguousarray(table), np.ascontiguousarray(scales, np.uint16),
+                         np.ascontiguousarray(biases, np.uint16), bits, token, vocab, d, out_scale, out)
+    return out
+
+
+def lm_head_greedy(hidden, norm_weight_bf16, weights, scales, biases, bits, eps=1e-6, act=0, want_logits=False):
+    """hidden float32 [d]; returns the token (and the logits [vocab] when asked)."""
+    h = np.ascontiguousarray(hidden, np.float32)
+    vocab, d = weights.shape[0], weights.shape[1] * 8 // bits
+    nw = None if norm_weight_bf16 is None else np.ascontiguousarray(norm_weight_bf16, np.uint16)
+    logits = np.zeros(vocab, np.float32) if want_logits else None
+    tok = lib.orc_lm_head_greedy(h, _ptr(nw), np.ascontiguousarray(weights), np.ascontiguousarray(scales, np.uint16),
+                                 np.ascontiguousarray(biases, np.uint16), bits, d, vocab, eps, act, _ptr(logits))
+    return (tok, logits) if want_logits else tok
 
 
 def rel_error(actual, reference):

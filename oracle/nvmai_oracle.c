@@ -32,6 +32,15 @@
  *       no vector and Metal's fast-math log is not reproducible): pinned by the
  *       published SplitMix64 constant, the closed form of the noise and the
  *       property that the draw follows p^(1/T)               tests/test_oracle_sampler.py
+ *   RMSNorm                         float64 recomputation, the reference tests'
+ *       constant-head known answer (every output 1), per-head isolation
+ *                                                             tests/test_oracle_step.py
+ *   embedding lookup                the reference's bit-stream known answer
+ *       (AffineQuantTests.swift:58-79), out-of-range token -> zeros, equals the
+ *       dequantizer                                           tests/test_oracle_step.py
+ *   greedy LM head                  the reference tests' known answers (target row,
+ *       ties -> lowest index, all-NaN -> 0, strided hidden row), brute-force
+ *       float64 argmax on well-separated rows                 tests/test_oracle_step.py
  *
  * Canonical summation order of the router logits ("half-wave order"):
  *   a row is cut into 16-byte chunks (16 codes at 8 bits, 32 codes at 4 bits,
@@ -757,6 +766,89 @@ void orc_attention_decode(const float *q, const void *k, const void *v, int kv_b
 
 /* ------------------------------------------------------------------------ */
 /* softmax + sampler                                                         */
+/* ------------------------------------------------------------------------ */
+/* rest of the decode step: RMSNorm, embedding lookup, greedy LM head         */
+/* ------------------------------------------------------------------------ */
+
+/* rmsnorm.metal:31-62 (inv = rsqrt(mean(x^2) + eps)), :83-87 (y = x * inv * w, left to right),
+ * :166-170 (no weight); rows = heads for the per-head kernels (:101-148).  The reference sums
+ * with a 256-thread block reduction whose order Metal does not fix; the order stated here is
+ * the one the HIP kernel implements, so that results can be compared bit for bit: 64 virtual
+ * lanes, lane l runs acc = fmaf(x, x, acc) over the elements l, l + 64, ... in ascending
+ * order, the 64 accumulators are summed by an xor butterfly with offsets 32, 16, 8, 4, 2, 1;
+ * mean = sum / d, inv = 1 / sqrtf(mean + eps), every operation rounded once.  weight: BF16
+ * bits or NULL.  out is NOT rounded to the activation type. */
+void orc_rmsnorm(const float *x, size_t x_stride, const uint16_t *weight_bf16, size_t rows,
+                 size_t d, float eps, float *out, size_t out_stride) {
+    for (size_t r = 0; r < rows; ++r) {
+        const float *xr = x + r * x_stride;
+        float lane[64];
+        for (int l = 0; l < 64; ++l) {
+            float acc = 0.0f;
+            for (size_t i = (size_t)l; i < d; i += 64) acc = fmaf(xr[i], xr[i], acc);
+            lane[l] = acc;
+        }
+        for (int off = 32; off >= 1; off >>= 1) {
+            float next[64];
+            for (int l = 0; l < 64; ++l) next[l] = lane[l] + lane[l ^ off];
+            memcpy(lane, next, sizeof(lane));
+        }
+        const float mean = lane[0] / (float)d;
+        const float inv = 1.0f / sqrtf(mean + eps);
+        for (size_t i = 0; i < d; ++i) {
+            float v = xr[i] * inv;
+            if (weight_bf16) v = v * orc_bf16_to_float(weight_bf16[i]);
+            out[r * out_stride + i] = v;
+        }
+    }
+}
+
+/* dequant_int4.metal:63-91 for 4- and 8-bit tables (AffineQuantEmbeddingLookup):
+ * out[i] = (float(q) * s + b) * out_scale, two roundings then the scale; a token id at or
+ * past vocab gives a row of zeros (:77-80).  out is NOT rounded to the activation type. */
+void orc_embed_lookup(const uint8_t *table, const uint16_t *scales, const uint16_t *biases,
+                      int bits, uint32_t token, size_t vocab, size_t d, float out_scale,
+                      float *out) {
+    if (token >= vocab) { for (size_t i = 0; i < d; ++i) out[i] = 0.0f; return; }
+    const size_t groups = d / ORC_GROUP;
+    const uint8_t *row = table + (size_t)token * (d * (size_t)bits / 8);
+    for (size_t i = 0; i < d; ++i) {
+        const float s = orc_bf16_to_float(scales[token * groups + i / ORC_GROUP]);
+        const float b = orc_bf16_to_float(biases[token * groups + i / ORC_GROUP]);
+        const float w = (float)code_at(row, i, bits) * s + b;
+        out[i] = w * out_scale;
+    }
+}
+
+/* LMHeadChainInt4.encodeGreedyDecode (LMHeadChainInt4.swift:58-130): RMSNorm with a BF16
+ * weight (norm_weight NULL: the hidden row is used as it is), the normed row rounded to the
+ * activation type (act 0 = bf16, 1 = fp16; the reference stores it as half), one logit per
+ * vocabulary row, argmax over the FINITE logits with ties to the lower index, 0 when there
+ * is none (logit.metal:855-861, 925-934).  The reference's per-row sum is a 32-lane simd_sum
+ * whose order Metal does not fix; the logits here are taken in the router's canonical
+ * half-wave order (above), which the HIP kernel implements, so the token is reproducible. */
+uint32_t orc_lm_head_greedy(const float *hidden, const uint16_t *norm_weight_bf16,
+                            const uint8_t *weights, const uint16_t *scales,
+                            const uint16_t *biases, int bits, size_t d, size_t vocab,
+                            float eps, int act, float *logits_out) {
+    float *xn = (float *)malloc(d * sizeof(float));
+    if (norm_weight_bf16) orc_rmsnorm(hidden, d, norm_weight_bf16, 1, d, eps, xn, d);
+    else memcpy(xn, hidden, d * sizeof(float));
+    if (act == 0) orc_round_through_bf16(xn, d); else orc_round_through_f16(xn, d);
+    float *logits = logits_out ? logits_out : (float *)malloc(vocab * sizeof(float));
+    orc_router_logits(weights, scales, biases, bits, xn, NULL, vocab, d, logits);
+    float best_v = -INFINITY;
+    uint32_t best_i = 0xFFFFFFFFu;
+    for (size_t r = 0; r < vocab; ++r) {
+        const float z = logits[r];
+        if (!isfinite(z)) continue;
+        if (best_i == 0xFFFFFFFFu || z > best_v) { best_v = z; best_i = (uint32_t)r; }
+    }
+    if (!logits_out) free(logits);
+    free(xn);
+    return best_i == 0xFFFFFFFFu ? 0u : best_i;
+}
+
 /* ------------------------------------------------------------------------ */
 
 static inline float softcap_value(float z, float softcap) {   /* logit.metal:42-49 */

@@ -199,6 +199,17 @@ uint32_t orc_sample_topk64(const uint16_t *probs_f16, size_t v, float temperatur
                            uint32_t *top64_idx, float *top64_val);
 
 /* RelError.swift:5-16 */
+/* ---- rest of the decode step ------------------------------------------- */
+void orc_rmsnorm(const float *x, size_t x_stride, const uint16_t *weight_bf16, size_t rows,
+                 size_t d, float eps, float *out, size_t out_stride);   /* rmsnorm.metal:31-170 */
+void orc_embed_lookup(const uint8_t *table, const uint16_t *scales, const uint16_t *biases,
+                      int bits, uint32_t token, size_t vocab, size_t d, float out_scale,
+                      float *out);                                      /* dequant_int4.metal:63-91 */
+uint32_t orc_lm_head_greedy(const float *hidden, const uint16_t *norm_weight_bf16,
+                            const uint8_t *weights, const uint16_t *scales,
+                            const uint16_t *biases, int bits, size_t d, size_t vocab,
+                            float eps, int act, float *logits_out);     /* logit.metal:761-937 */
+
 float orc_rel_error(const float *actual, const float *reference, size_t n);
 
 #ifdef __cplusplus

@@ -1,0 +1,185 @@
+"""GPU parity: RMSNorm, affine embedding lookup and the fused greedy LM head through the C ABI.
+
+All three are compared bit for bit: the oracle states the summation order the kernels use, every
+other step is one IEEE operation, and the greedy token is an index."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from gpu_util import act_np, act_tensor, dev, gauss, round_act, say, u16, u32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def nv():
+    import nvmai_amd
+    return nvmai_amd
+
+
+@pytest.fixture(scope="module", params=[0, 1], ids=["bf16", "fp16"])
+def ctx(request, nv):
+    c = nv.Context(0, request.param)
+    yield c
+    torch.cuda.synchronize()
+    c.close()
+
+
+def _act_bits(a, act):
+    return O.bf16_bits(a) if act == 0 else O.f16_bits(a)
+
+
+def _bits(t):
+    """The 16-bit patterns of an activation tensor."""
+    return t.detach().contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+# ------------------------------------------------------------------ RMSNorm
+@pytest.mark.parametrize("rows,d", [(1, 256), (1, 2048), (3, 2816), (16, 256), (5, 100), (9, 64)])
+def test_rmsnorm_bit_exact(nv, ctx, rows, d):
+    say("rmsnorm", ctx.act, rows, d)
+    rng = np.random.default_rng(rows * 31 + d)
+    x = round_act(rng.uniform(-1, 1, (rows, d)).astype(np.float32), ctx.act)
+    w = O.bf16_bits(rng.uniform(0.5, 1.5, d).astype(np.float32))
+    rms = nv.RMSNorm(ctx)
+    got_w = _bits(rms.encode_bf16w(act_tensor(x, ctx), dev(w.view(np.int16))))
+    got_n = _bits(rms.encode_no_scale(act_tensor(x, ctx)))
+    torch.cuda.synchronize()
+    assert np.array_equal(got_w, _act_bits(O.rmsnorm(x, w, 1e-6), ctx.act))
+    assert np.array_equal(got_n, _act_bits(O.rmsnorm(x, None, 1e-6), ctx.act))
+    # the reference's bar against an independent formulation (Tolerance.fp16Reduction, RMSNormTests.swift:53)
+    x64 = x.astype(np.float64)
+    want = x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + 1e-6) * O.bf16_to_float(w).astype(np.float64)
+    got_f = act_np(rms.encode_bf16w(act_tensor(x, ctx), dev(w.view(np.int16))))
+    assert np.abs(got_f - want).max() / np.abs(want).max() < 5e-3
+
+
+def test_rmsnorm_per_head_in_place_known_answer(nv, ctx):
+    # RMSNormTests.swift:119-165: head h is the constant h + 1, unit weights, in place -> all ones;
+    # rows further apart than head_dim (a padded stride) leave the padding alone
+    say("rmsnorm per head", ctx.act)
+    heads, hd, stride = 16, 256, 256 + 8
+    buf = torch.full((heads, stride), 5.0, dtype=ctx.dtype, device="cuda")
+    buf[:, :hd] = torch.arange(1, heads + 1, dtype=torch.float32, device="cuda")[:, None].to(ctx.dtype)
+    view = buf[:, :hd]
+    unit = dev(O.bf16_bits(np.ones(hd, np.float32)).view(np.int16))
+    nv.RMSNorm(ctx).encode_bf16w_per_head(view, unit, out=view)
+    torch.cuda.synchronize()
+    out = buf.float().cpu().numpy()
+    assert np.abs(out[:, :hd] - 1.0).max() < 1e-2
+    assert (out[:, hd:] == 5.0).all()
+    assert nv.lib.nvmai_hip_rmsnorm(ctx.handle, None, None, 8, None, None, 8, 1, 8, 1e-6) == -1    # no buffers
+
+
+# ------------------------------------------------------------------ embedding lookup
+@pytest.mark.parametrize("bits", [4, 8])
+def test_embed_lookup_bit_exact_and_known_answer(nv, ctx, bits):
+    say("embed", ctx.act, bits)
+    # AffineQuantTests.swift:58-79: bit-stream table, scale 1, bias 0 -> the values themselves
+    rows, cols = 3, 128
+    mask = (1 << bits) - 1
+    values = np.array([[(r * 11 + c * 3) & mask for c in range(cols)] for r in range(rows)], np.float32)
+    packed = np.zeros((rows, cols * bits // 8), np.uint8)
+    for r in range(rows):
+        for c in range(cols):
+            packed[r, c * bits // 8] |= (int(values[r, c]) << ((c * bits) % 8)) & 0xFF
+    one = dev(np.full((rows, 2), 0x3F80, np.uint16).view(np.int16))
+    zero = dev(np.zeros((rows, 2), np.int16))
+    emb = nv.AffineQuantEmbeddingLookup(ctx, bits)
+    got = act_np(emb.encode(dev(packed), one, zero, 1, cols, rows))
+    torch.cuda.synchronize()
+    assert np.array_equal(got[0], values[1])
+    # random table, a block of token ids with one out of range, output scale, padded rows
+    rng = np.random.default_rng(50 + bits)
+    vocab, d = 37, 2048 + 64
+    p, s, b = O.quantize_affine(gauss(rng, (vocab, d), 0.05), bits)
+    ids = np.array([0, 36, 5, 37, 12, 0xFFFFFFFF, 5], np.uint32)
+    out = torch.full((len(ids), d + 16), 3.0, dtype=ctx.dtype, device="cuda")
+    emb.encode(dev(p), dev(s.view(np.int16)), dev(b.view(np.int16)), dev(ids.view(np.int32)), d, vocab, 45.25, out)
+    torch.cuda.synchronize()
+    got = _bits(out)
+    for t, tok in enumerate(ids):
+        assert np.array_equal(got[t, :d], _act_bits(O.embed_lookup(p, s, b, bits, int(tok), 45.25), ctx.act))
+    assert (out[:, d:].float() == 3.0).all()
+    assert not got[3, :d].any() and not got[5, :d].any()
+    with pytest.raises(nv.NvmaiError) as e:
+        nv.AffineQuantEmbeddingLookup(ctx, 6)
+    assert e.value.name == "unsupported"
+
+
+# ------------------------------------------------------------------ greedy LM head
+def _const_rows(v, d, special, hi, lo, bits=4):
+    w = np.full((v, d), lo, np.float32)
+    for r in special:
+        w[r] = hi
+    return O.quantize_affine(w, bits)
+
+
+def _head_dev(p, s, b):
+    return dev(p), dev(s.view(np.int16)), dev(b.view(np.int16))
+
+
+def test_greedy_head_reference_known_answers(nv, ctx):
+    # LMHeadChainInt4Tests.swift:136-224
+    say("greedy head known answers", ctx.act)
+    d = 64
+    unit = dev(O.bf16_bits(np.ones(d, np.float32)).view(np.int16))
+    chain = nv.LMHeadChain(ctx, 4)
+    hidden = round_act((0.25 + (np.arange(d) % 7) * 0.01).astype(np.float32), ctx.act)
+    for v in (1024, 2048, 4096):
+        p, s, b = _const_rows(v, d, [v - 3], 1.0, -0.5)
+        tok = chain.encode_greedy_decode(act_tensor(hidden[None], ctx), unit, *_head_dev(p, s, b), d, v)
+        assert int(tok[0]) == v - 3
+    hidden = round_act((0.2 + (np.arange(d) % 5) * 0.02).astype(np.float32), ctx.act)
+    p, s, b = _const_rows(1024, d, [17, 311], 1.0, -0.25)
+    tok = chain.encode_greedy_decode(act_tensor(hidden[None], ctx), unit, *_head_dev(p, s, b), d, 1024)
+    assert int(tok[0]) == 17                                    # ties resolve to the lowest index
+    p, s, b = _const_rows(1024, d, [], 0.25, 0.25)
+    nan = torch.full((1, d), float("nan"), dtype=ctx.dtype, device="cuda")
+    tok = chain.encode_greedy_decode(nan, unit, *_head_dev(p, s, b), d, 1024)
+    assert int(tok[0]) == 0                                     # no finite candidate
+    # the selected row of a strided hidden buffer (:195-224)
+    rows = np.stack([(0.25 + (np.arange(d) % 7) * 0.01) if r == 3 else (-0.4 - (np.arange(d) % 5) * 0.01)
+                     for r in range(5)]).astype(np.float32)
+    hbuf = torch.zeros((5, d + 16), dtype=ctx.dtype, device="cuda")
+    hbuf[:, :d] = act_tensor(rows, ctx)
+    p, s, b = _const_rows(1024, d, [777], 1.0, -0.25)
+    tok = chain.encode_greedy_decode(hbuf[3:4, :d], unit, *_head_dev(p, s, b), d, 1024)
+    assert int(tok[0]) == 777
+
+
+@pytest.mark.parametrize("bits,d,v,tokens", [(4, 2048, 5000, 3), (8, 2048, 3001, 2), (4, 4096, 700, 1),
+                                             (8, 1024, 999, 1), (4, 192, 130, 4), (8, 64, 70, 1)])
+def test_greedy_head_token_equals_oracle(nv, ctx, bits, d, v, tokens):
+    # random rows, nothing separated on purpose: near-ties must fall the same way as in the oracle
+    say("greedy head", ctx.act, bits, d, v, tokens)
+    rng = np.random.default_rng(bits * 1000 + d + v)
+    p, s, b = O.quantize_affine(gauss(rng, (v, d), 0.02), bits)
+    p[v // 2] = p[v // 3]; s[v // 2] = s[v // 3]; b[v // 2] = b[v // 3]          # two identical rows
+    hidden = round_act(gauss(rng, (tokens, d)), ctx.act)
+    nw = O.bf16_bits(rng.uniform(0.5, 1.5, d).astype(np.float32))
+    chain = nv.LMHeadChain(ctx, bits)
+    hd = _head_dev(p, s, b)
+    got = u32(chain.encode_greedy_decode(act_tensor(hidden, ctx), dev(nw.view(np.int16)), *hd, d, v))
+    got_raw = u32(chain.encode_greedy_decode(act_tensor(hidden, ctx), None, *hd, d, v))
+    torch.cuda.synchronize()
+    for t in range(tokens):
+        assert got[t] == O.lm_head_greedy(hidden[t], nw, p, s, b, bits, act=ctx.act)
+        assert got_raw[t] == O.lm_head_greedy(hidden[t], None, p, s, b, bits, act=ctx.act)
+
+
+def test_greedy_head_rejects_bad_arguments(nv, ctx):
+    say("greedy head errors", ctx.act)
+    w = torch.zeros(64 * 64, dtype=torch.uint8, device="cuda")
+    s = torch.zeros(64, dtype=torch.int16, device="cuda")
+    h = torch.zeros((1, 128), dtype=ctx.dtype, device="cuda")
+    with pytest.raises(nv.NvmaiError) as e:
+        nv.LMHeadChain(ctx, 4).encode_greedy_decode(h[:, :100], None, w, s, s, 100, 64)     # d % 64 != 0
+    assert e.value.name == "invalid_arg"
+    with pytest.raises(nv.NvmaiError) as e:
+        nv.LMHeadChain(ctx, 8).encode_greedy_decode(h, None, w[1:], s, s, 128, 8)            # misaligned rows
+    assert e.value.name == "alignment"
+    with pytest.raises(nv.NvmaiError) as e:
+        nv.LMHeadChain(ctx, 6)
+    assert e.value.name == "unsupported"
