@@ -384,6 +384,27 @@ int nvmai_hip_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* x, ui
                       const uint16_t* weight, void* out, uint32_t out_stride, uint32_t rows,
                       uint32_t d, float eps);
 
+/* Elementwise (Elementwise.swift:28-121; kernels utility.metal:32-121) and the SwiGLU product of the
+ * shared expert (SharedExpertInt4.swift:61-96, silu_mul_fp16): 16-bit activations, fp32 arithmetic.
+ *   silu_mul:           out[i] = silu(gate[i]) * up[i]
+ *   sigmoid_gate_mul:   out[i] = out[i] * sigmoid(gate[i])          (in place)
+ *   sigmoid_scalar_mul: y[i]   = y[i] * sigmoid(gate[0])            (in place)
+ *   residual_add:       hidden[i] = hidden[i] + delta[i]            (in place)
+ *   split_q_gate:       packed [heads, 2 dim] -> q [heads, dim], gate [heads, dim]
+ *   concat_rows:        lhs, rhs [rows, dim] -> out [rows, 2 dim] */
+int nvmai_hip_silu_mul(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* gate, const void* up,
+                       void* out, uint32_t count);
+int nvmai_hip_sigmoid_gate_mul(nvmai_hip_ctx* ctx, nvmai_stream stream, void* out, const void* gate,
+                               uint32_t count);
+int nvmai_hip_sigmoid_scalar_mul(nvmai_hip_ctx* ctx, nvmai_stream stream, void* y, const void* gate,
+                                 uint32_t count);
+int nvmai_hip_residual_add(nvmai_hip_ctx* ctx, nvmai_stream stream, void* hidden, const void* delta,
+                           uint32_t count);
+int nvmai_hip_split_q_gate(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* packed, void* q,
+                           void* gate, uint32_t heads, uint32_t dim);
+int nvmai_hip_concat_rows(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* lhs, const void* rhs,
+                          void* out, uint32_t rows, uint32_t dim);
+
 /* AffineQuantEmbeddingLookup.encode (kernel embed_lookup_int4, dequant_int4.metal:63-91; a block
  * of tokens: prefill_embed_lookup_affine_block, prefill.metal:59): out[t] = (q * scale + bias) *
  * out_scale for row token[t] of a 4- or 8-bit affine table [vocab, d]; a token id >= vocab gives

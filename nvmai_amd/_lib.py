@@ -92,6 +92,12 @@ SIGNATURES = {
                                       u32, u32, C.POINTER(PrefillGrouping), vp, vp],
     "nvmai_hip_affine_qmm": [vp, vp, vp, vp, vp, u32, vp, u32, vp, u32, u32, u32, u32],
     "nvmai_hip_prefill_moe_reduce_token_major": [vp, vp, vp, vp, vp, u32, u32, u32, u32],
+    "nvmai_hip_silu_mul": [vp, vp, vp, vp, vp, u32],
+    "nvmai_hip_sigmoid_gate_mul": [vp, vp, vp, vp, u32],
+    "nvmai_hip_sigmoid_scalar_mul": [vp, vp, vp, vp, u32],
+    "nvmai_hip_residual_add": [vp, vp, vp, vp, u32],
+    "nvmai_hip_split_q_gate": [vp, vp, vp, vp, vp, u32, u32],
+    "nvmai_hip_concat_rows": [vp, vp, vp, vp, vp, u32, u32],
     "nvmai_hip_rmsnorm": [vp, vp, vp, u32, vp, vp, u32, u32, u32, C.c_float],
     "nvmai_hip_embed_lookup": [vp, vp, vp, vp, vp, u32, vp, u32, u32, vp, u32, u32, u32, C.c_float],
     "nvmai_hip_lm_head_greedy": [vp, vp, vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, u32, C.c_float],

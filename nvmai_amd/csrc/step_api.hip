@@ -1,4 +1,4 @@
-// Entry points: RMSNorm, affine embedding lookup, fused greedy LM head.
+// Entry points: RMSNorm, the elementwise helpers of the layer loop, affine embedding lookup, fused greedy LM head.
 #include "ctx.hpp"
 #include "step_kernels.cuh"
 
@@ -15,6 +15,63 @@ extern "C" int nvmai_hip_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const 
         rmsnorm_kernel<ACT_BF16><<<grid, 256, 0, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);
     else
         rmsnorm_kernel<ACT_FP16><<<grid, 256, 0, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);
+    return launch_status();
+}
+
+namespace {
+
+template <int OP>
+int run_elementwise(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* a, const void* b, void* out, uint32_t count) {
+    if (!ctx || !a || !b || !out) return NVMAI_ERR_INVALID_ARG;
+    if (count == 0) return NVMAI_OK;
+    const dim3 grid((count + 255) / 256);
+    hipStream_t s = (hipStream_t)stream;
+    if (ctx->act == ACT_BF16)
+        elementwise_kernel<ACT_BF16, OP><<<grid, 256, 0, s>>>((const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, count);
+    else
+        elementwise_kernel<ACT_FP16, OP><<<grid, 256, 0, s>>>((const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, count);
+    return launch_status();
+}
+
+}  // namespace
+
+extern "C" int nvmai_hip_silu_mul(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* gate, const void* up,
+                                  void* out, uint32_t count) {
+    return run_elementwise<EW_SILU_MUL>(ctx, stream, gate, up, out, count);
+}
+
+extern "C" int nvmai_hip_sigmoid_gate_mul(nvmai_hip_ctx* ctx, nvmai_stream stream, void* out, const void* gate,
+                                          uint32_t count) {
+    return run_elementwise<EW_SIGMOID_MUL>(ctx, stream, out, gate, out, count);
+}
+
+extern "C" int nvmai_hip_sigmoid_scalar_mul(nvmai_hip_ctx* ctx, nvmai_stream stream, void* y, const void* gate,
+                                            uint32_t count) {
+    return run_elementwise<EW_SIGMOID_SCALAR>(ctx, stream, y, gate, y, count);
+}
+
+extern "C" int nvmai_hip_residual_add(nvmai_hip_ctx* ctx, nvmai_stream stream, void* hidden, const void* delta,
+                                      uint32_t count) {
+    return run_elementwise<EW_ADD>(ctx, stream, hidden, delta, hidden, count);
+}
+
+extern "C" int nvmai_hip_split_q_gate(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* packed, void* q,
+                                      void* gate, uint32_t heads, uint32_t dim) {
+    if (!ctx || !packed || !q || !gate) return NVMAI_ERR_INVALID_ARG;
+    if ((uint64_t)heads * dim > 0x7FFFFFFFull) return NVMAI_ERR_INVALID_ARG;
+    if (heads * dim == 0) return NVMAI_OK;
+    split_join_rows_kernel<false><<<(heads * dim + 255) / 256, 256, 0, (hipStream_t)stream>>>(
+        (uint16_t*)const_cast<void*>(packed), (uint16_t*)q, (uint16_t*)gate, heads, dim);
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_concat_rows(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* lhs, const void* rhs,
+                                     void* out, uint32_t rows, uint32_t dim) {
+    if (!ctx || !lhs || !rhs || !out) return NVMAI_ERR_INVALID_ARG;
+    if ((uint64_t)rows * dim > 0x7FFFFFFFull) return NVMAI_ERR_INVALID_ARG;
+    if (rows * dim == 0) return NVMAI_OK;
+    split_join_rows_kernel<true><<<(rows * dim + 255) / 256, 256, 0, (hipStream_t)stream>>>(
+        (uint16_t*)out, (uint16_t*)const_cast<void*>(lhs), (uint16_t*)const_cast<void*>(rhs), rows, dim);
     return launch_status();
 }
 

@@ -45,6 +45,46 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* x, uint32_
     }
 }
 
+// ---- elementwise helpers of the layer loop (utility.metal) -----------------------------------
+// 16-bit activations in and out, fp32 arithmetic, one rounding at the end.
+enum ElementwiseOp : int {
+    EW_SILU_MUL = 0,        // out = silu(a) * b, silu(g) = g / (1 + exp(-g))   utility.metal:32-45
+    EW_SIGMOID_MUL = 1,     // out = a / (1 + exp(-b[i]))                        :47-58
+    EW_SIGMOID_SCALAR = 2,  // out = a / (1 + exp(-b[0]))                        :60-72
+    EW_ADD = 3              // out = a + b                                       :95-104
+};
+
+template <int ACT, int OP>
+__global__ __launch_bounds__(256) void elementwise_kernel(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                                                          uint32_t count) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= count) return;
+    const float x = act_to_f32<ACT>(a[i]);
+    const float y = act_to_f32<ACT>(b[OP == EW_SIGMOID_SCALAR ? 0 : i]);
+    float r;
+    if (OP == EW_SILU_MUL) r = __fmul_rn(__fdiv_rn(x, __fadd_rn(1.0f, expf(-x))), y);
+    else if (OP == EW_ADD) r = __fadd_rn(x, y);
+    else r = __fdiv_rn(x, __fadd_rn(1.0f, expf(-y)));
+    out[i] = f32_to_act<ACT>(r);
+}
+
+// split (JOIN = false): packed [rows, 2 dim] -> lo [rows, dim], hi [rows, dim]   (split_q_gate_fp16, :75-92)
+// join  (JOIN = true):  lo, hi [rows, dim]   -> packed [rows, 2 dim]             (concat_rows_fp16, :107-121)
+template <bool JOIN>
+__global__ __launch_bounds__(256) void split_join_rows_kernel(uint16_t* packed, uint16_t* lo, uint16_t* hi,
+                                                              uint32_t rows, uint32_t dim) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * dim) return;
+    const uint32_t r = i / dim, c = i % dim;
+    if (JOIN) {
+        packed[(size_t)r * 2 * dim + c] = lo[i];
+        packed[(size_t)r * 2 * dim + dim + c] = hi[i];
+    } else {
+        lo[i] = packed[(size_t)r * 2 * dim + c];
+        hi[i] = packed[(size_t)r * 2 * dim + dim + c];
+    }
+}
+
 // ---- embedding lookup ------------------------------------------------------------------
 // out[t, i] = ((float(q) * s + b) * out_scale) for row token[t] of a 4- or 8-bit affine table,
 // zeros for a token id at or past vocab (dequant_int4.metal:63-91; a block of tokens:

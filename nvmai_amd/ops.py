@@ -635,3 +635,45 @@ class LMHeadChain:
                                            _ptr(norm_weight), _ptr(weights), _ptr(scales), _ptr(biases), self.bits,
                                            _ptr(out), d, vocab, rms_eps), "lm_head_greedy")
         return out
+
+
+class Elementwise:
+    """Mirror of Elementwise (Elementwise.swift:28-121) plus silu_mul_fp16 (utility.metal:32-45)."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+
+    def encode_silu_mul(self, gate, up, out=None):
+        if out is None:
+            out = torch.empty_like(gate)
+        check(lib.nvmai_hip_silu_mul(self.ctx.handle, _stream(), _ptr(gate), _ptr(up), _ptr(out), gate.numel()), "silu_mul")
+        return out
+
+    def encode_sigmoid_gate_mul(self, out, gate):
+        check(lib.nvmai_hip_sigmoid_gate_mul(self.ctx.handle, _stream(), _ptr(out), _ptr(gate), out.numel()),
+              "sigmoid_gate_mul")
+        return out
+
+    def encode_sigmoid_scalar_mul(self, y, gate):
+        check(lib.nvmai_hip_sigmoid_scalar_mul(self.ctx.handle, _stream(), _ptr(y), _ptr(gate), y.numel()),
+              "sigmoid_scalar_mul")
+        return y
+
+    def encode_residual_add(self, hidden, delta):
+        check(lib.nvmai_hip_residual_add(self.ctx.handle, _stream(), _ptr(hidden), _ptr(delta), hidden.numel()),
+              "residual_add")
+        return hidden
+
+    def encode_split_q_gate(self, packed, heads, dim):
+        q = torch.empty((heads, dim), dtype=packed.dtype, device=packed.device)
+        gate = torch.empty_like(q)
+        check(lib.nvmai_hip_split_q_gate(self.ctx.handle, _stream(), _ptr(packed), _ptr(q), _ptr(gate), heads, dim),
+              "split_q_gate")
+        return q, gate
+
+    def encode_concat_rows(self, lhs, rhs):
+        rows, dim = lhs.shape
+        out = torch.empty((rows, 2 * dim), dtype=lhs.dtype, device=lhs.device)
+        check(lib.nvmai_hip_concat_rows(self.ctx.handle, _stream(), _ptr(lhs), _ptr(rhs), _ptr(out), rows, dim),
+              "concat_rows")
+        return out

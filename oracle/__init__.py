@@ -83,6 +83,7 @@ _sig("orc_sample_topk64", C.c_uint32, u16p, size_t, C.c_float, C.c_float, C.c_ui
      C.c_uint32, C.c_void_p, C.c_void_p)
 _sig("orc_rel_error", C.c_float, f32p, f32p, size_t)
 _sig("orc_rmsnorm", None, f32p, size_t, C.c_void_p, size_t, size_t, C.c_float, f32p, size_t)
+_sig("orc_elementwise", None, C.c_int, f32p, f32p, size_t, f32p)
 _sig("orc_embed_lookup", None, u8p, u16p, u16p, C.c_int, C.c_uint32, size_t, size_t, C.c_float, f32p)
 _sig("orc_lm_head_greedy", C.c_uint32, f32p, C.c_void_p, u8p, u16p, u16p, C.c_int, size_t, size_t,
      C.c_float, C.c_int, C.c_void_p)
@@ -464,6 +465,29 @@ def rmsnorm(x, weight_bf16=None, eps=1e-6):
     w = None if weight_bf16 is None else np.ascontiguousarray(weight_bf16, np.uint16)
     lib.orc_rmsnorm(x2, x2.shape[1], _ptr(w), x2.shape[0], x2.shape[1], eps, out, x2.shape[1])
     return out.reshape(x.shape)
+
+
+EW_SILU_MUL, EW_SIGMOID_MUL, EW_SIGMOID_SCALAR, EW_ADD = 0, 1, 2, 3
+
+
+def elementwise(op, a, b):
+    """utility.metal:32-104 on float32 arrays (b: one value for EW_SIGMOID_SCALAR)."""
+    a = np.ascontiguousarray(a, np.float32)
+    b = np.ascontiguousarray(b, np.float32)
+    out = np.zeros_like(a)
+    lib.orc_elementwise(op, a.reshape(-1), b.reshape(-1), a.size, out.reshape(-1))
+    return out
+
+
+def split_q_gate(packed, heads, dim):
+    """utility.metal:75-92: [heads, 2 dim] -> q [heads, dim], gate [heads, dim]."""
+    p = np.asarray(packed).reshape(heads, 2 * dim)
+    return p[:, :dim].copy(), p[:, dim:].copy()
+
+
+def concat_rows(lhs, rhs):
+    """utility.metal:107-121: [rows, dim] + [rows, dim] -> [rows, 2 dim]."""
+    return np.concatenate([np.asarray(lhs), np.asarray(rhs)], axis=1)
 
 
 def embed_lookup(table, scales, biases, bits, token, out_scale=1.0):

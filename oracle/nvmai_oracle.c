@@ -35,6 +35,10 @@
  *   RMSNorm                         float64 recomputation, the reference tests'
  *       constant-head known answer (every output 1), per-head isolation
  *                                                             tests/test_oracle_step.py
+ *   elementwise helpers             PARITY UNPINNED against the reference (it holds no test
+ *       for them): special values (sigmoid(0) = 1/2, silu(0) = 0, saturation) and float64
+ *       recomputation; the add, split and concatenation are fixed by their definition
+ *                                                             tests/test_oracle_step.py
  *   embedding lookup                the reference's bit-stream known answer
  *       (AffineQuantTests.swift:58-79), out-of-range token -> zeros, equals the
  *       dequantizer                                           tests/test_oracle_step.py
@@ -800,6 +804,18 @@ void orc_rmsnorm(const float *x, size_t x_stride, const uint16_t *weight_bf16, s
             if (weight_bf16) v = v * orc_bf16_to_float(weight_bf16[i]);
             out[r * out_stride + i] = v;
         }
+    }
+}
+
+/* utility.metal:32-45, 47-58, 60-72, 95-104: op 0 silu(a) * b, 1 a * sigmoid(b[i]) written as
+ * a / (1 + exp(-b)), 2 the same with b[0], 3 a + b; fp32, each operation rounded once.  out is
+ * NOT rounded to the activation type. */
+void orc_elementwise(int op, const float *a, const float *b, size_t count, float *out) {
+    for (size_t i = 0; i < count; ++i) {
+        const float x = a[i], y = b[op == 2 ? 0 : i];
+        if (op == 0) out[i] = (x / (1.0f + expf(-x))) * y;
+        else if (op == 3) out[i] = x + y;
+        else out[i] = x / (1.0f + expf(-y));
     }
 }
 

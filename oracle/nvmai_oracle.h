@@ -202,6 +202,7 @@ uint32_t orc_sample_topk64(const uint16_t *probs_f16, size_t v, float temperatur
 /* ---- rest of the decode step ------------------------------------------- */
 void orc_rmsnorm(const float *x, size_t x_stride, const uint16_t *weight_bf16, size_t rows,
                  size_t d, float eps, float *out, size_t out_stride);   /* rmsnorm.metal:31-170 */
+void orc_elementwise(int op, const float *a, const float *b, size_t count, float *out); /* utility.metal:32-104 */
 void orc_embed_lookup(const uint8_t *table, const uint16_t *scales, const uint16_t *biases,
                       int bits, uint32_t token, size_t vocab, size_t d, float out_scale,
                       float *out);                                      /* dequant_int4.metal:63-91 */

@@ -183,3 +183,39 @@ def test_greedy_head_rejects_bad_arguments(nv, ctx):
     with pytest.raises(nv.NvmaiError) as e:
         nv.LMHeadChain(ctx, 6)
     assert e.value.name == "unsupported"
+
+
+# ------------------------------------------------------------------ elementwise helpers
+def _ulp16_apart(got_bits, want_bits):
+    """Largest distance in 16-bit patterns (same sign assumed where values are not tiny)."""
+    return np.abs(got_bits.astype(np.int32) - want_bits.astype(np.int32)).max()
+
+
+def test_elementwise_helpers_match_oracle(nv, ctx):
+    say("elementwise", ctx.act)
+    rng = np.random.default_rng(77)
+    n = 5000
+    a = round_act(gauss(rng, (n,), 3.0), ctx.act)
+    b = round_act(gauss(rng, (n,), 3.0), ctx.act)
+    ew = nv.Elementwise(ctx)
+    got = _bits(ew.encode_silu_mul(act_tensor(a, ctx), act_tensor(b, ctx)))
+    # exp comes from two different libraries: at most one 16-bit ulp apart, and within the 1e-2 bar
+    want = O.elementwise(O.EW_SILU_MUL, a, b)
+    assert _ulp16_apart(got, _act_bits(want, ctx.act)) <= 1
+    got = ew.encode_sigmoid_gate_mul(act_tensor(a, ctx), act_tensor(b, ctx))
+    assert _ulp16_apart(_bits(got), _act_bits(O.elementwise(O.EW_SIGMOID_MUL, a, b), ctx.act)) <= 1
+    assert O.rel_error(act_np(got), O.elementwise(O.EW_SIGMOID_MUL, a, b)) < 1e-2
+    got = ew.encode_sigmoid_scalar_mul(act_tensor(a, ctx), act_tensor(b[:1], ctx))
+    assert _ulp16_apart(_bits(got), _act_bits(O.elementwise(O.EW_SIGMOID_SCALAR, a, b), ctx.act)) <= 1
+    # one IEEE addition, one rounding: bit-exact
+    got = ew.encode_residual_add(act_tensor(a, ctx), act_tensor(b, ctx))
+    assert np.array_equal(_bits(got), _act_bits(O.elementwise(O.EW_ADD, a, b), ctx.act))
+    # data movement: bit-exact
+    heads, dim = 16, 256
+    packed = round_act(gauss(rng, (heads, 2 * dim)), ctx.act)
+    q, g = ew.encode_split_q_gate(act_tensor(packed, ctx), heads, dim)
+    wq, wg = O.split_q_gate(packed, heads, dim)
+    assert np.array_equal(act_np(q), wq) and np.array_equal(act_np(g), wg)
+    assert np.array_equal(act_np(ew.encode_concat_rows(q, g)), packed)
+    torch.cuda.synchronize()
+    assert nv.lib.nvmai_hip_silu_mul(ctx.handle, None, None, None, None, 4) == -1

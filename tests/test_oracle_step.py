@@ -123,3 +123,37 @@ def test_greedy_head_matches_float64_argmax_on_separated_rows():
         want2 = deq @ hidden.astype(np.float64)
         assert tok2 == int(np.argmax(want2))
         assert np.abs(logits2 - want2).max() / np.abs(want2).max() < 1e-5
+
+
+# ------------------------------------------------------------------ elementwise helpers
+def test_elementwise_special_values_and_float64():
+    # the reference holds no test for utility.metal's helpers: what the mathematics fixes
+    z = np.zeros(4, np.float32)
+    one = np.ones(4, np.float32)
+    assert np.array_equal(O.elementwise(O.EW_SILU_MUL, z, one), z)                         # silu(0) = 0
+    assert np.array_equal(O.elementwise(O.EW_SIGMOID_MUL, one, z), one * np.float32(0.5))  # sigmoid(0) = 1/2
+    big = np.full(4, 40.0, np.float32)
+    assert np.array_equal(O.elementwise(O.EW_SIGMOID_MUL, one, big), one)                  # saturates to 1
+    assert np.abs(O.elementwise(O.EW_SIGMOID_MUL, one, -big)).max() < 1e-15                # and to 0
+    assert np.array_equal(O.elementwise(O.EW_SILU_MUL, big, one), big)                     # silu(x) -> x
+    rng = np.random.default_rng(8)
+    a = (rng.standard_normal(4096) * 3).astype(np.float32)
+    b = (rng.standard_normal(4096) * 3).astype(np.float32)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    for op, want in [(O.EW_SILU_MUL, a64 / (1 + np.exp(-a64)) * b64), (O.EW_SIGMOID_MUL, a64 / (1 + np.exp(-b64))),
+                     (O.EW_SIGMOID_SCALAR, a64 / (1 + np.exp(-b64[0]))), (O.EW_ADD, a64 + b64)]:
+        got = O.elementwise(op, a, b)
+        assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max()
+    assert np.array_equal(O.elementwise(O.EW_ADD, a, b), a + b)                            # one IEEE addition
+    # sigmoid(-g) = 1 - sigmoid(g)
+    s_pos = O.elementwise(O.EW_SIGMOID_MUL, np.ones_like(b), b)
+    s_neg = O.elementwise(O.EW_SIGMOID_MUL, np.ones_like(b), -b)
+    assert np.abs(s_pos + s_neg - 1.0).max() < 1e-6
+
+
+def test_split_and_concat_are_inverse_layouts():
+    heads, dim = 5, 12
+    packed = np.arange(heads * 2 * dim, dtype=np.float32).reshape(heads, 2 * dim)
+    q, g = O.split_q_gate(packed, heads, dim)
+    assert q[2, 3] == packed[2, 3] and g[2, 3] == packed[2, dim + 3]          # utility.metal:90-91
+    assert np.array_equal(O.concat_rows(q, g), packed)
