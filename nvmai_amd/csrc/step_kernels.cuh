@@ -130,8 +130,9 @@ __global__ __launch_bounds__(256) void embed_lookup_kernel(const uint8_t* table,
 // into registers, and the block walks LMH_ROWS rows, the next row's codes in flight while the
 // current one is summed.  Each block leaves (best logit, index) and a second small launch picks
 // the winner.
-constexpr uint32_t LMH_ROWS = 64;                 // rows per block: 8 per half-wave
+constexpr uint32_t LMH_ROWS = 128;                // rows per block: 16 per half-wave
 constexpr int LMH_STEPS = LMH_ROWS / 8;
+constexpr int LMH_BUFS = 2;                       // register buffers of codes: LMH_BUFS - 1 rows in flight per half-wave
 
 struct LmHeadParams {
     const uint16_t* hidden;       // [tokens, hidden_stride] activations
@@ -145,8 +146,11 @@ struct LmHeadParams {
     float2* summaries;            // [tokens, gridDim.x] (best logit, index bits)
 };
 
+// (at least three blocks per CU where a lane holds 64 inputs: left alone, the scheduler hoists
+// every load of the unrolled loop and takes all 256 registers, which leaves two waves per SIMD to
+// hide each row's butterfly; with 128 inputs per lane three blocks would spill)
 template <int ACT, int BITS, int CPL>
-__global__ __launch_bounds__(256) void lm_head_greedy_kernel(LmHeadParams p) {
+__global__ __launch_bounds__(256, (CPL * (128 / BITS) > 64 ? 2 : 3)) void lm_head_greedy_kernel(LmHeadParams p) {
     constexpr int EPC = Chunk<BITS>::elems;
     // LDS: [d] normed inputs as floats | 16 words of block results | [d] hidden row, [d] norm weight (16 bit)
     extern __shared__ float lmh_lds[];
@@ -160,8 +164,8 @@ __global__ __launch_bounds__(256) void lm_head_greedy_kernel(LmHeadParams p) {
     const uint32_t chunks = p.d * BITS / 128, groups = p.d / NVMAI_GROUP, row_bytes = p.d * BITS / 8;
     const uint32_t row0 = blockIdx.x * LMH_ROWS;
     const uint32_t row_end = min(row0 + LMH_ROWS, p.vocab);
-    uint4 q[3][CPL];
-    uint16_t sc[3][CPL], bi[3][CPL];
+    uint4 q[LMH_BUFS][CPL];
+    uint16_t sc[LMH_BUFS][CPL], bi[LMH_BUFS][CPL];
     auto load_row = [&](int buf, uint32_t row) {
         row = min(row, p.vocab - 1);
 #pragma unroll
@@ -173,8 +177,8 @@ __global__ __launch_bounds__(256) void lm_head_greedy_kernel(LmHeadParams p) {
             bi[buf][c] = p.biases[(size_t)row * groups + g];
         }
     };
-    load_row(0, row0 + hw);                       // in flight while the inputs are prepared
-    load_row(1, row0 + hw + 8);
+#pragma unroll
+    for (int k = 0; k < LMH_BUFS - 1; ++k) load_row(k, row0 + hw + 8 * k);   // in flight while the inputs are prepared
 
     // The row and the norm weight reach LDS in one round trip (16-byte loads where the row is
     // aligned); everything after reads LDS.  Read straight from memory, the strided sum below
@@ -213,13 +217,16 @@ __global__ __launch_bounds__(256) void lm_head_greedy_kernel(LmHeadParams p) {
     float xr[CPL][EPC], xs[CPL];
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
-        const uint32_t chunk = hl + 32 * c;
+        const uint32_t chunk = min(hl + 32 * c, chunks - 1);     // a lane without this chunk: a copy, never used
+        const float4* src = reinterpret_cast<const float4*>(xn + chunk * EPC);
         xs[c] = 0.0f;
 #pragma unroll
-        for (int e = 0; e < EPC; ++e) {
-            xr[c][e] = chunk < chunks ? xn[chunk * EPC + e] : 0.0f;
-            xs[c] = __fadd_rn(xs[c], xr[c][e]);
+        for (int e = 0; e < EPC / 4; ++e) {
+            const float4 v = src[e];
+            xr[c][4 * e] = v.x; xr[c][4 * e + 1] = v.y; xr[c][4 * e + 2] = v.z; xr[c][4 * e + 3] = v.w;
         }
+#pragma unroll
+        for (int e = 0; e < EPC; ++e) xs[c] = __fadd_rn(xs[c], xr[c][e]);
     }
 
     float best_v = -INFINITY;
@@ -228,15 +235,22 @@ __global__ __launch_bounds__(256) void lm_head_greedy_kernel(LmHeadParams p) {
         float acc = 0.0f;
 #pragma unroll
         for (int c = 0; c < CPL; ++c) {
-            if (hl + 32 * c < chunks) {
-                float qf[EPC];
-                unpack_chunk<BITS>(q[buf][c], qf);
-                float dot = 0.0f;
-#pragma unroll
-                for (int e = 0; e < EPC; ++e) dot = fmaf(qf[e], xr[c][e], dot);
-                acc = fmaf(bf16_to_f32(sc[buf][c]), dot, acc);
-                acc = fmaf(bf16_to_f32(bi[buf][c]), xs[c], acc);
+            // every lane does the arithmetic (a lane without this chunk on a copy of the last one)
+            // and keeps its old sum by a select: a branch here would cut the step into pieces
+            // that each wait for their loads
+            float qf[EPC];
+            if (BITS == 8) {
+                unpack_chunk<8>(q[buf][c], qf);
+            } else {
+                unpack4_bytes(q[buf][c].x, qf); unpack4_bytes(q[buf][c].y, qf + 8);
+                unpack4_bytes(q[buf][c].z, qf + 16); unpack4_bytes(q[buf][c].w, qf + 24);
             }
+            float dot = 0.0f;
+#pragma unroll
+            for (int e = 0; e < EPC; ++e) dot = fmaf(qf[e], xr[c][e], dot);
+            float next = fmaf(bf16_to_f32(sc[buf][c]), dot, acc);
+            next = fmaf(bf16_to_f32(bi[buf][c]), xs[c], next);
+            acc = hl + 32 * c < chunks ? next : acc;
         }
 #pragma unroll
         for (int off = 16; off >= 1; off >>= 1) acc = __fadd_rn(acc, shfl_xor_f(acc, off));
@@ -249,8 +263,8 @@ __global__ __launch_bounds__(256) void lm_head_greedy_kernel(LmHeadParams p) {
     // can count the loads in flight; with conditional loads it waited for all of them each step.
 #pragma unroll
     for (int k = 0; k < LMH_STEPS; ++k) {
-        if (k + 2 < LMH_STEPS) load_row((k + 2) % 3, row0 + hw + 8 * (k + 2));
-        sum_row(k % 3, row0 + hw + 8 * k);
+        if (k + LMH_BUFS - 1 < LMH_STEPS) load_row((k + LMH_BUFS - 1) % LMH_BUFS, row0 + hw + 8 * (k + LMH_BUFS - 1));
+        sum_row(k % LMH_BUFS, row0 + hw + 8 * k);
     }
     float* res_v = lmh_lds + p.d;
     uint32_t* res_i = reinterpret_cast<uint32_t*>(lmh_lds + p.d + 8);
