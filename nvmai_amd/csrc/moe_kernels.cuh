@@ -404,7 +404,10 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
         }
     };
 
-#pragma unroll 1
+    // Unrolled on purpose: as a real loop its two conditional loads meet at the back edge, the
+    // compiler can no longer tell how many loads are in flight behind the stage about to be
+    // used, and waits for all of them -- the stage just requested included.
+#pragma unroll
     for (int it = 0; it < ITERS; it += 2) {
         compute_stage(s0, it);
         if (it + 2 < ITERS) load_stage(s0, it + 2);
