@@ -183,7 +183,7 @@ __device__ __forceinline__ void unpack_chunk(const uint4& w, float* q) {
     if (BITS == 8) {
         unpack8(w.x, q); unpack8(w.y, q + 4); unpack8(w.z, q + 8); unpack8(w.w, q + 12);
     } else {
-        unpack4(w.x, q); unpack4(w.y, q + 8); unpack4(w.z, q + 16); unpack4(w.w, q + 24);
+        unpack4_bytes(w.x, q); unpack4_bytes(w.y, q + 8); unpack4_bytes(w.z, q + 16); unpack4_bytes(w.w, q + 24);
     }
 }
 

@@ -239,12 +239,7 @@ __global__ __launch_bounds__(256, (CPL * (128 / BITS) > 64 ? 2 : 3)) void lm_hea
             // and keeps its old sum by a select: a branch here would cut the step into pieces
             // that each wait for their loads
             float qf[EPC];
-            if (BITS == 8) {
-                unpack_chunk<8>(q[buf][c], qf);
-            } else {
-                unpack4_bytes(q[buf][c].x, qf); unpack4_bytes(q[buf][c].y, qf + 8);
-                unpack4_bytes(q[buf][c].z, qf + 16); unpack4_bytes(q[buf][c].w, qf + 24);
-            }
+            unpack_chunk<BITS>(q[buf][c], qf);     // 4 bit: nibbles isolated as bytes, one conversion per code
             float dot = 0.0f;
 #pragma unroll
             for (int e = 0; e < EPC; ++e) dot = fmaf(qf[e], xr[c][e], dot);
