@@ -177,7 +177,9 @@ int nvmai_hip_shared_expert(nvmai_hip_ctx* ctx, nvmai_stream stream, const void*
  * (RealForwardRunner.swift:1900-1920 router, :3866-3912 shared expert, :3914-4297
  * routed experts, minus the two host round trips and the SSD streaming):
  * y[t] = sigmoid(g.x[t]) * ffn_shared(x[t]) + sum_slot w[t,slot] * ffn_{idx[t,slot]}(x[t]).
- * Each distinct routed expert is read once per call. */
+ * Each distinct routed expert is read once per call (with one or two tokens, where the step is
+ * a chain of launches rather than bytes, each token reads its own experts and the call is three
+ * launches instead of five). */
 typedef struct {
     uint32_t d, f, num_experts, top_k, bits;
     nvmai_rows router;
