@@ -359,6 +359,29 @@ void launch_routed(int act, uint32_t bits, RowsParams& p, const SelectParams& se
 }
 
 template <int ACT, int BITS>
+void launch_slots_t(RowsParams& p, const uint32_t* active_slots, uint32_t count, uint32_t top_k, hipStream_t s) {
+    const uint32_t chunks = p.n * BITS / 128;
+    constexpr uint32_t rows_per_block = 4 * 1 * 1 * 2;       // four waves, SEG 64, RPI 1, ITERS 2
+    p.blocks_per_entry = (p.rows + rows_per_block - 1) / rows_per_block;
+    const dim3 grid(count * p.blocks_per_entry);
+    if (chunks == 64)
+        expert_rows_slots<ACT, BITS, 64, 1, 1, 2><<<grid, 256, rows_fast_lds_bytes(p.n, 1, 64), s>>>(p, active_slots, top_k);
+    else
+        expert_rows_slots<ACT, BITS, 64, 2, 1, 2><<<grid, 256, rows_fast_lds_bytes(p.n, 2, 64), s>>>(p, active_slots, top_k);
+}
+
+void launch_slots(int act, uint32_t bits, RowsParams& p, const uint32_t* active_slots, uint32_t count, uint32_t top_k,
+                  hipStream_t s) {
+    if (act == ACT_BF16) {
+        if (bits == 8) launch_slots_t<ACT_BF16, 8>(p, active_slots, count, top_k, s);
+        else launch_slots_t<ACT_BF16, 4>(p, active_slots, count, top_k, s);
+    } else {
+        if (bits == 8) launch_slots_t<ACT_FP16, 8>(p, active_slots, count, top_k, s);
+        else launch_slots_t<ACT_FP16, 4>(p, active_slots, count, top_k, s);
+    }
+}
+
+template <int ACT, int BITS>
 void launch_down_combine_t(const DownCombineParams& p, hipStream_t s) {
     const uint32_t chunks = p.n * BITS / 128;
     const dim3 grid((p.rows + DC_ROWS - 1) / DC_ROWS, p.tokens);
@@ -592,6 +615,17 @@ extern "C" int nvmai_hip_moe_phase1_gate_up_act_subset(
     if (!x || !acts || (active_count && !active_slots) || active_count > top_k) return NVMAI_ERR_INVALID_ARG;
     if (!aligned16(x) || !aligned16(acts)) return NVMAI_ERR_ALIGNMENT;
     hipStream_t s = (hipStream_t)stream;
+    {   // one launch where the row engine has a short-block instantiation: the entries are made in the kernel
+        const uint32_t c1 = d * bits / 128;
+        if ((d * bits) % 128 == 0 && (c1 == 64 || c1 == 128)) {
+            const uint32_t n = active_slots ? active_count : top_k;
+            if (n == 0) return NVMAI_OK;
+            set_phase1(p, *off, d, f);
+            p.x = x; p.x_stride = d; p.out = acts; p.out_stride = f;
+            launch_slots(ctx->act, bits, p, active_slots, n, top_k, s);
+            return launch_status();
+        }
+    }
     rc = ws_begin(ctx, ws_round(8 * sizeof(WorkEntry)) + 3 * ws_round(64));
     if (rc) return rc;
     WorkEntry* entries = ws_take<WorkEntry>(ctx, 8);
@@ -634,6 +668,19 @@ extern "C" int nvmai_hip_moe_phase2_down_reduce(nvmai_hip_ctx* ctx, nvmai_stream
     if (!acts || !routing_w || !y) return NVMAI_ERR_INVALID_ARG;
     if (!aligned16(acts)) return NVMAI_ERR_ALIGNMENT;
     hipStream_t s = (hipStream_t)stream;
+    {   // one launch (down projection of every slot + weighted sum) where that kernel is instantiated
+        const uint32_t c2 = f * bits / 128;
+        if ((f * bits) % 128 == 0 && (c2 == 16 || c2 == 32 || c2 == 64)) {
+            DownCombineParams dc{};
+            dc.src = p.src;
+            dc.wA = off->down_w; dc.sA = off->down_s; dc.bA = off->down_b;
+            dc.acts = acts; dc.idx = nullptr; dc.w = routing_w; dc.residual = residual; dc.res_stride = d;
+            dc.gate_logit = nullptr; dc.has_shared = 0; dc.tokens = 1; dc.top_k = top_k; dc.rows = d; dc.n = f;
+            dc.y_stride = d; dc.y = y;
+            launch_down_combine(ctx->act, bits, dc, s);
+            return launch_status();
+        }
+    }
     rc = ws_begin(ctx, ws_round(8 * sizeof(WorkEntry)) + 3 * ws_round(64) + ws_round((size_t)top_k * d * 4));
     if (rc) return rc;
     WorkEntry* entries = ws_take<WorkEntry>(ctx, 8);

@@ -1145,6 +1145,23 @@ __global__ __launch_bounds__(256) void expert_rows_routed(RowsParams p, SelectPa
     }
 }
 
+// The routed experts of ONE token given as a table of blob pointers (the reference's RoutedBlobs,
+// moe.metal:153-155): entry i = slot i -- or active_slots[i], skipped when it is not below top_k
+// (the hit / miss split, moe.metal:685-727) -- input row 0, output row = slot.  No work list.
+template <int ACT, int BITS, int SEG, int NCH, int RPI, int ITERS>
+__global__ __launch_bounds__(256) void expert_rows_slots(RowsParams p, const uint32_t* active_slots, uint32_t top_k) {
+    extern __shared__ uint4 rows_lds[];
+    const uint32_t entry = blockIdx.x / p.blocks_per_entry, rb = blockIdx.x % p.blocks_per_entry;
+    const uint32_t slot = active_slots ? active_slots[entry] : entry;
+    if (slot >= top_k) return;                    // uniform per block
+    WorkEntry we;
+    we.expert = NVMAI_SLOT_FLAG | slot;
+    we.pair_start = slot;
+    we.pair_count = 1;
+    we.reserved = 0;
+    expert_rows_body<ACT, BITS, SEG, NCH, 1, true, false, RPI, ITERS, ROWS_DIRECT>(p, we, rb, rows_lds);
+}
+
 // (2) down_combine: the down projection of every slot of a token and the weighted sum over the
 // slots in one launch.  A block owns DC_ROWS output rows of one token; its four waves share the
 // slots (wave w: slots w, w + 4, ...), SEG lanes per row with one 16-byte chunk each, every load
@@ -1159,8 +1176,10 @@ struct DownCombineParams {
     BlobSource src;
     int64_t wA, sA, bA;           // down projection inside the blob
     const float* acts;            // fp32 [tokens * top_k (+ tokens), n]: routed rows, then shared rows
-    const uint32_t* idx;          // [tokens, top_k]
+    const uint32_t* idx;          // [tokens, top_k] pool indices; NULL: slot s reads the blob in table slot s
     const uint16_t* w;            // fp16 [tokens, top_k]
+    const void* residual;         // optional activations [tokens, res_stride], added first
+    uint32_t res_stride;
     const float* gate_logit;      // optional [tokens]
     int has_shared;
     uint32_t tokens, top_k, rows, n, y_stride;
@@ -1186,6 +1205,8 @@ __global__ __launch_bounds__(256) void down_combine_kernel(DownCombineParams p) 
     // what the final sum needs, requested before everything else: lane k holds the weight of slot k
     const float wk = (uint32_t)lane < p.top_k ? f16_to_f32(p.w[(size_t)t * p.top_k + lane]) : 0.0f;
     const float gate = p.gate_logit ? p.gate_logit[t] : 0.0f;
+    const float res = p.residual && wave == 0 && lane < DC_ROWS && row0 + lane < p.rows
+                          ? act_to_f32<ACT>(((const uint16_t*)p.residual)[(size_t)t * p.res_stride + row0 + lane]) : 0.0f;
 
     uint4 q[DC_SLOTS_PER_WAVE][PASSES];
     uint16_t sc[DC_SLOTS_PER_WAVE][PASSES], bi[DC_SLOTS_PER_WAVE][PASSES];
@@ -1195,7 +1216,8 @@ __global__ __launch_bounds__(256) void down_combine_kernel(DownCombineParams p) 
         const uint32_t slot = wave + 4 * j;
         if (slot >= n_slots) break;               // uniform per wave
         const bool routed = slot < p.top_k;
-        const uint32_t expert = routed ? p.idx[(size_t)t * p.top_k + slot] : (NVMAI_SLOT_FLAG | 8u);
+        const uint32_t expert = !routed ? (NVMAI_SLOT_FLAG | 8u)
+                                : p.idx ? p.idx[(size_t)t * p.top_k + slot] : (NVMAI_SLOT_FLAG | slot);
         const uint32_t act_row = routed ? t * p.top_k + slot : p.tokens * p.top_k + t;
         const uint8_t* blob = blob_ptr(p.src, expert);
         const uint8_t* W = blob + p.wA;
@@ -1234,7 +1256,7 @@ __global__ __launch_bounds__(256) void down_combine_kernel(DownCombineParams p) 
     __syncthreads();
     if (wave == 0) {              // lanes below DC_ROWS own an output row each; all 64 serve the lane reads
         const uint32_t r = lane < DC_ROWS ? lane : 0;
-        float acc = 0.0f;
+        float acc = res;
         if (p.has_shared) {
             float s = part[p.top_k][r];
             if (p.gate_logit) s = __fdiv_rn(s, __fadd_rn(1.0f, expf(-gate)));
