@@ -217,6 +217,32 @@ bool launch_dense_rows_t(RowsParams& p, int maxtok, uint32_t ents, hipStream_t s
     return false;
 }
 
+// Gate/up + SwiGLU of ONE expert (blob slot 0) over dense_count input rows in one launch, short blocks.
+template <int ACT, int BITS>
+bool launch_dense_dual_t(RowsParams& p, int maxtok, uint32_t ents, hipStream_t s) {
+    const uint32_t chunks = p.n * BITS / 128;
+    if ((p.n * BITS) % 128 || (chunks != 64 && chunks != 128)) return false;
+    constexpr uint32_t rows_per_block = 4 * 1 * 1 * 2;
+    p.blocks_per_entry = (p.rows + rows_per_block - 1) / rows_per_block;
+    const dim3 grid(ents * p.blocks_per_entry);
+#define NVMAI_DUAL(NCH)                                                                                          \
+    do {                                                                                                         \
+        const size_t lds = rows_fast_lds_bytes(p.n, NCH, 64);                                                    \
+        if (maxtok == 1) expert_rows_fast<ACT, BITS, 64, NCH, 1, true, false, 1, 2, true><<<grid, 256, lds, s>>>(p); \
+        else expert_rows_fast<ACT, BITS, 64, NCH, 4, true, false, 1, 2, true><<<grid, 256, lds, s>>>(p);         \
+    } while (0)
+    if (chunks == 64) NVMAI_DUAL(1); else NVMAI_DUAL(2);
+#undef NVMAI_DUAL
+    return true;
+}
+
+bool launch_dense_dual(int act, uint32_t bits, RowsParams& p, int maxtok, uint32_t ents, hipStream_t s) {
+    if (act == ACT_BF16) return bits == 8 ? launch_dense_dual_t<ACT_BF16, 8>(p, maxtok, ents, s)
+                                          : launch_dense_dual_t<ACT_BF16, 4>(p, maxtok, ents, s);
+    return bits == 8 ? launch_dense_dual_t<ACT_FP16, 8>(p, maxtok, ents, s)
+                     : launch_dense_dual_t<ACT_FP16, 4>(p, maxtok, ents, s);
+}
+
 bool launch_dense_rows(int act, uint32_t bits, RowsParams& p, int maxtok, uint32_t ents, hipStream_t s) {
     if (act == ACT_BF16) return bits == 8 ? launch_dense_rows_t<ACT_BF16, 8>(p, maxtok, ents, s)
                                           : launch_dense_rows_t<ACT_BF16, 4>(p, maxtok, ents, s);
@@ -747,6 +773,43 @@ extern "C" int nvmai_hip_shared_expert(nvmai_hip_ctx* ctx, nvmai_stream stream, 
     }
     const int maxtok = n_tokens == 1 ? 1 : MAX_TOK;
     const uint32_t ents = (n_tokens + maxtok - 1) / maxtok;
+    // A handful of tokens: gate logit, gate/up with its entries made in the kernel, and the down
+    // projection with the gate applied in its epilogue -- three launches (two without a gate)
+    // instead of five.  The down kernel reads the matrix once per token, hence the limit.
+    {
+        const uint32_t c1 = d * bits / 128, c2 = f * bits / 128;
+        if (n_tokens <= 4 && (d * bits) % 128 == 0 && (c1 == 64 || c1 == 128) && (f * bits) % 128 == 0 &&
+            (c2 == 16 || c2 == 32 || c2 == 64)) {
+            const bool gated_s = shared_gate && shared_gate->kind;
+            rc = ws_begin(ctx, ws_round((size_t)n_tokens * f * 4) + ws_round(n_tokens * 4u) + ws_round(16));
+            if (rc) return rc;
+            float* acts = ws_take<float>(ctx, (size_t)n_tokens * f);
+            float* gate_logit = ws_take<float>(ctx, n_tokens);
+            float* dummy_logits = ws_take<float>(ctx, 4);
+            if (gated_s) {
+                RouterParams rp{};
+                rp.gate = to_desc(shared_gate);
+                rp.x = x; rp.x_stride = x_stride; rp.tokens = n_tokens; rp.num_experts = 0; rp.d = d;
+                rp.logits = dummy_logits; rp.gate_logit = gate_logit;
+                rc = run_router(ctx->act, rp, s);
+                if (rc) return rc;
+            }
+            RowsParams p{};
+            p.src.slot[0] = (const uint8_t*)blob;
+            set_phase1(p, *off, d, f);
+            p.x = x; p.x_stride = x_stride; p.out = acts; p.out_stride = f; p.dense_count = n_tokens;
+            if (launch_dense_dual(ctx->act, bits, p, maxtok, ents, s)) {
+                DownCombineParams dc{};
+                dc.src.slot[8] = (const uint8_t*)blob;
+                dc.wA = off->down_w; dc.sA = off->down_s; dc.bA = off->down_b;
+                dc.acts = acts; dc.gate_logit = gated_s ? gate_logit : nullptr;
+                dc.has_shared = 1; dc.tokens = n_tokens; dc.top_k = 0; dc.rows = d; dc.n = f;
+                dc.y_stride = y_stride; dc.y = y;
+                launch_down_combine(ctx->act, bits, dc, s);
+                return launch_status();
+            }
+        }
+    }
     size_t need = ws_round(ents * sizeof(WorkEntry)) + ws_round(16) + 2 * ws_round(n_tokens * 4u) +
                   ws_round((size_t)n_tokens * f * 4) + ws_round((size_t)n_tokens * d * 4) +
                   ws_round(n_tokens * 4u) + ws_round(16);
