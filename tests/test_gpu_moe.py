@@ -345,9 +345,8 @@ def test_shared_expert_with_scalar_gate(nv, ctx, bits):
     rng = np.random.default_rng(bits)
     # 192 tokens and more go through the grouped-GEMM kernels in their dense mode
     # (one to four tokens of a shape the row engine has short blocks for: three launches)
-    for d, f, tokens in [(128, 64, 1), (2048, 512, 1), (2048, 512, 3), (1024, 1024, 4), (2048, 512, 6), (256, 128, 9),
-                         (256, 128, 192), (192, 64, 250),
-                         (2048, 512, 200), (512, 192, 300), (256, 128, 130)]:
+    for d, f, tokens in [(128, 64, 1), (2048, 512, 1), (2048, 512, 6), (256, 128, 9), (256, 128, 192), (192, 64, 250),
+                         (2048, 512, 200), (512, 192, 300), (256, 128, 130), (2048, 512, 3), (1024, 1024, 4)]:
         say("shared expert", ctx.act, bits, d, f, tokens)
         host = _random_blobs(rng, d, f, bits, 1, 0.03)[0]
         gate = O.quantize_affine(O.round_bf16(gauss(rng, (1, d), 0.05)), 8)
