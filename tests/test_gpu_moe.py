@@ -440,3 +440,40 @@ def test_decode_layer_few_tokens_three_launches(nv, ctx, bits):
         d, f = c1 * per, c2 * per
         say("decode layer few tokens", ctx.act, bits, d, f, E, k, tokens, shared, gated)
         _layer_case(nv, ctx, rng, d, f, E, k, bits, tokens, 16 if d <= 2048 else 8, 0.03, shared, gated)
+
+
+@pytest.mark.parametrize("tokens", [1, 12])
+def test_decode_layer_replays_from_a_captured_graph(nv, ctx_bf16, tokens):
+    # The calls only enqueue kernels (no allocation after warm-up, no memset nodes), so a caller may
+    # capture a decode step in a HIP graph: every replay, with new inputs in the same buffers and
+    # eager work in between, must equal the eager result bit for bit (three launches at one token,
+    # five with the work list at twelve).
+    say("decode layer graph replay", tokens)
+    ctx, d, f, E, k, bits = ctx_bf16, 1024, 256, 24, 8, 8
+    gen = torch.Generator(device="cuda").manual_seed(5 + tokens)
+    off, stride = nv.expert_offsets(d, f, bits)
+    pool = torch.empty((E + 1, stride), dtype=torch.uint8, device="cuda")
+    for e in range(E + 1):
+        mk = lambda r, c: torch.empty((r, c), device="cuda").normal_(0.0, 0.03, generator=gen).to(torch.bfloat16)
+        nv.pack_expert(ctx, mk(f, d), mk(f, d), mk(d, f), bits, pool[e])
+    router = torch.empty((E, d), device="cuda").normal_(0.0, 0.05, generator=gen).to(torch.bfloat16)
+    layer = nv.moe_layer_desc(d, f, E, k, bits, nv.rows_desc(16, router.view(torch.int16)), pool[:E], pool[E])
+    moe = nv.MoE(ctx, bits)
+    xs = [torch.empty((tokens, d), device="cuda").normal_(0.0, 1.0, generator=gen).to(torch.bfloat16) for _ in range(4)]
+    x_static = xs[0].clone()
+    y_static = torch.empty((tokens, d), dtype=torch.bfloat16, device="cuda")
+    moe.decode_layer(layer, x_static, y_static)                      # warm-up: the workspace is sized here
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            moe.decode_layer(layer, x_static, y_static)
+    torch.cuda.synchronize()
+    for x in xs:
+        want = moe.decode_layer(layer, x).clone()                    # eager, its own output buffer
+        torch.cuda.synchronize()
+        x_static.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_static, want)
