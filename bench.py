@@ -34,10 +34,11 @@ def parse():
     ap.add_argument("--layers", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--sweep", action="store_true", help="also print batch/bits sweep lines to stderr")
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "sampler", "copy"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "sampler", "greedy", "copy"],
                     help="decode = configs[1] (the headline line); prefill = configs[2] grouped GEMM; "
                          "attention = configs[3] quantized-KV decode attention; sampler = the end of configs[4]: "
-                         "quantized LM head GEMV over 248,320 rows, tiled softmax, top-k sampler; copy = a plain 1 GiB device copy, "
+                         "quantized LM head GEMV over 248,320 rows, tiled softmax, top-k sampler; greedy = the fused greedy LM head "
+                         "(RMSNorm + logits in a fixed order + argmax) over the same head; copy = a plain 1 GiB device copy, "
                          "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated on")
     ap.add_argument("--context", type=int, default=32768, help="attention: tokens in the KV cache")
     ap.add_argument("--tokens", type=int, default=4096, help="prefill: tokens per step")
@@ -472,6 +473,76 @@ def run_sampler(nv, ctx, torch, a):
     }
 
 
+def run_greedy(nv, ctx, torch, a):
+    """LMHeadChain.encode_greedy_decode over a 4/8-bit head [248320, 2048]: one token per hidden row."""
+    V, bits, rows = 248320, a.bits, min(a.batch, 4)
+    gen = torch.Generator(device="cuda").manual_seed(78)
+    n_heads = 4                                            # rotate copies of the head past the caches
+    heads = []
+    for _ in range(n_heads):
+        wt = torch.empty((V, D), dtype=torch.bfloat16, device="cuda").normal_(0.0, 0.02, generator=gen)
+        heads.append(nv.quantize_affine(ctx, wt, bits))
+        del wt
+    xs = torch.empty((8, rows, D), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
+    norm_w = torch.empty(D, dtype=torch.bfloat16, device="cuda").uniform_(0.5, 1.5, generator=gen).view(torch.int16)
+    chain = nv.LMHeadChain(ctx, bits)
+    toks = torch.empty(rows, dtype=torch.int32, device="cuda")
+
+    def step(i):
+        chain.encode_greedy_decode(xs[i % 8], norm_w, *heads[i % n_heads], D, V, out=toks)
+
+    for i in range(a.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(i)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]     # the launch stream is torch's current stream
+    ev[0].record()
+    for i in range(a.steps):
+        step(i)
+    ev[1].record()
+    torch.cuda.synchronize()
+    us = ev[0].elapsed_time(ev[1]) / a.steps * 1e3
+    cpu = None
+    if not a.no_cpu:
+        import oracle as O
+        p_, s_, b_ = (t_.cpu().numpy() for t_ in heads[0])
+        h0 = xs[0, 0].float().cpu().numpy()
+        nw = norm_w.cpu().numpy().view(np.uint16)
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            tok = O.lm_head_greedy(h0, nw, p_, s_.view(np.uint16), b_.view(np.uint16), bits, act=0)
+            reps += 1
+            if time.perf_counter() - t0 > 10.0 or reps >= 20:
+                break
+        dtc = (time.perf_counter() - t0) / reps
+        step(0)
+        torch.cuda.synchronize()
+        assert int(toks[0]) == tok, "greedy token differs from the oracle"
+        cpu = dict(value=1.0 / dtc, unit="tok/s", cores=1, kind="port",
+                   sample="oracle lm_head_greedy over the %d-bit head, one row, %d reps, %.3f s each (same token as "
+                          "the GPU)" % (bits, reps, dtc))
+    head_bytes = V * D * bits / 8 + 2 * V * (D // 64) * 2
+    gbps = rows * head_bytes / (us * 1e-6) / 1e9
+    return {
+        "metric": METRIC, "value": round(rows / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u%d codes, f32 fma chain in a fixed order" % bits, "data": "synthetic",
+        "config": {"workload": "end of configs[4], greedy: RMSNorm + %d-bit LM head 248,320 x 2048 + argmax in one "
+                               "call, %d hidden rows per step (the head is read once per row)" % (bits, rows)},
+        "roofline": {"kernel": "lm_head_greedy_kernel (+ its reduce launch)", "bound": "hbm", "achieved": round(gbps, 2),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     # rocprofv3 --pmc FETCH_SIZE: 264,100 KiB x 2.00 (copy-kernel calibration) at 8 bit, one row
+                     "traffic": 264100 * 2.0 * 1024 if (bits == 8 and rows == 1) else None,
+                     "bytes_per_launch": rows * head_bytes, "avg_launch_us": round(us, 2)},
+        "cpu_baseline": cpu,
+    }
+
+
 def run_copy(torch, a):
     """A plain copy kernel of known size: 1 GiB read + 1 GiB written per launch."""
     n = 1 << 30
@@ -506,7 +577,8 @@ def main():
     if a.workload != "decode":
         line = (run_prefill(nv, ctx, torch, a) if a.workload == "prefill" else
                 run_attention(nv, ctx, torch, a) if a.workload == "attention" else
-                run_sampler(nv, ctx, torch, a) if a.workload == "sampler" else run_copy(torch, a))
+                run_sampler(nv, ctx, torch, a) if a.workload == "sampler" else
+                run_greedy(nv, ctx, torch, a) if a.workload == "greedy" else run_copy(torch, a))
         print(json.dumps(line), flush=True)
         return
     layers, stride = build_layers(nv, ctx, torch, a.bits, a.layers)
