@@ -118,8 +118,26 @@ __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float c) {
 // and-or instructions per dword.  The odd pairs' offset of 64 instead of 1024 is taken back with
 // the sum of the inputs at their positions (ODD_PAIR_OFFSET_GAP).
 constexpr float ODD_PAIR_OFFSET_GAP = 1024.0f - 64.0f;
+// The 4-bit masks and exponent patterns arrive in registers (NibbleConsts, made opaque to the
+// compiler once per kernel): written as literals every AND-OR splits into a v_and and a v_or,
+// because the three-operand v_and_or_b32 takes no literal on this target; with the mask in a
+// scalar and the pattern in a vector register it is one instruction.
+struct NibbleConsts {
+    uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
+};
+__device__ __forceinline__ NibbleConsts nibble_consts() {
+    NibbleConsts c{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm("" : "+s"(c.mask_lo));
+    asm("" : "+s"(c.mask_hi));
+    asm("" : "+v"(c.magic_lo));
+    asm("" : "+v"(c.magic_hi));
+#endif
+    return c;
+}
+
 template <int BITS>
-__device__ __forceinline__ void unpack_pairs(const uint4& w, uint32_t* qp) {
+__device__ __forceinline__ void unpack_pairs(const uint4& w, uint32_t* qp, const NibbleConsts& nc) {
     const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
@@ -128,10 +146,10 @@ __device__ __forceinline__ void unpack_pairs(const uint4& w, uint32_t* qp) {
             qp[2 * d + 1] = __builtin_amdgcn_perm(ws[d], 0x64646464u, 0x00070006u);
         } else {
             const uint32_t hi = ws[d] >> 8;
-            qp[4 * d] = (ws[d] & 0x000F000Fu) | 0x64006400u;
-            qp[4 * d + 1] = (ws[d] & 0x00F000F0u) | 0x54005400u;
-            qp[4 * d + 2] = (hi & 0x000F000Fu) | 0x64006400u;
-            qp[4 * d + 3] = (hi & 0x00F000F0u) | 0x54005400u;
+            qp[4 * d] = (ws[d] & nc.mask_lo) | nc.magic_lo;
+            qp[4 * d + 1] = (ws[d] & nc.mask_hi) | nc.magic_hi;
+            qp[4 * d + 2] = (hi & nc.mask_lo) | nc.magic_lo;
+            qp[4 * d + 3] = (hi & nc.mask_hi) | nc.magic_hi;
         }
     }
 }
@@ -199,6 +217,7 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
     static_assert(ITERS % 2 == 0, "ITERS must be even (double buffering)");
     using Stage = RowStage<BITS, SEG, NCH, DUAL, RPI>;
     const int ntok = TOKS ? TOKS : (int)we.pair_count;
+    const NibbleConsts nib = nibble_consts();
     const uint8_t* blob = blob_ptr(p.src, we.expert);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int seg_id = lane / SEG, sl = lane % SEG;
@@ -346,8 +365,8 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
         for (int i = 0; i < RPI; ++i)
 #pragma unroll
             for (int c = 0; c < NCH; ++c) {
-                unpack_pairs<BITS>(st.qa[i][c], qpa[i][c]);
-                if (DUAL) unpack_pairs<BITS>(st.qb[i][c], qpb[i][c]);
+                unpack_pairs<BITS>(st.qa[i][c], qpa[i][c], nib);
+                if (DUAL) unpack_pairs<BITS>(st.qb[i][c], qpb[i][c], nib);
             }
 #pragma unroll 1
         for (int t = 0; t < ntok; ++t) {
