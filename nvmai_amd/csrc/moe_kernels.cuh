@@ -566,7 +566,11 @@ struct RouterParams {
     float* gate_logit;             // [tokens]
 };
 
-constexpr int ROUTER_TOK = 4;   // tokens per block in y
+// Tokens per block in y.  One: the launch is a chain of latencies (stage the row, load eight
+// weight rows, sum, butterfly), so more blocks with less to do each finish sooner than fewer
+// blocks walking several tokens (measured at 32 tokens: 11.7 us with four, 9.0 with two or one;
+// at four tokens 10.4 -> 6.6 us).  The weight rows are re-read per token from L2.
+constexpr int ROUTER_TOK = 1;
 
 // EPC consecutive activations of one row as floats, optionally times the bf16
 // effective scale (one rounding, as moe.metal:200-201 multiplies before use).
