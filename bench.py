@@ -158,7 +158,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # `--workload copy`); the summaries live under profiles/.  Keyed by (workload, bits, batch or
 # tokens); other configurations report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("decode", 8, 32): (180800 * 2.00 + 1241 * 1.00) * 1024,
+    ("decode", 8, 32): (181300 * 2.00 + 1196 * 1.00) * 1024,
     ("prefill", 4, 4096): (377200 * 2.00 + 36140 * 1.00) * 1024,
     ("attention", 8, 8, 131072): (599800 * 2.00 + 4383 * 1.00) * 1024,
     ("attention", 4, 8, 131072): (295900 * 2.00 + 4356 * 1.00) * 1024,
