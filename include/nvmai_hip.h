@@ -11,6 +11,13 @@
  *   - calls only enqueue work on `stream` (a hipStream_t) and never synchronise;
  *   - status is returned as int: 0 = ok, negative = nvmai_status; nothing aborts;
  *   - one nvmai_hip_ctx per stream; a ctx is not thread-safe.
+ *   - workspace and HIP graphs: entry points take their intermediate buffers from a
+ *     workspace the ctx owns.  It grows (hipMalloc) the first time a call needs more
+ *     than any call before it; blocks it has outgrown stay allocated until
+ *     nvmai_hip_ctx_destroy, so a captured graph stays valid whatever is called
+ *     later.  A call that would have to grow while its stream is being captured
+ *     returns NVMAI_ERR_SCRATCH and launches nothing: run the same call eagerly once,
+ *     or nvmai_hip_ctx_reserve, before capturing.
  * Data formats (reference file:line):
  *   - weights: affine group-64 codes, 4 bit (two per byte, element 2k in the low
  *     nibble of byte k) or 8 bit, plus one BF16 scale and one BF16 bias per group
@@ -65,6 +72,11 @@ typedef struct {
  * Attention.swift:117-126, sampler stages LogitOutput.swift:244-258). */
 int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** out);
 void nvmai_hip_ctx_destroy(nvmai_hip_ctx* ctx);
+/* Grow the ctx workspace to at least `bytes` now (the counterpart of the wrappers' scratch
+ * buffers allocated in init, Attention.swift:117-126, LogitOutput.swift:244-258), so that no
+ * later call has to; nvmai_hip_ctx_workspace_bytes reports the current size. */
+int nvmai_hip_ctx_reserve(nvmai_hip_ctx* ctx, size_t bytes);
+size_t nvmai_hip_ctx_workspace_bytes(const nvmai_hip_ctx* ctx);
 const char* nvmai_hip_status_string(int status);
 
 /* Per-kernel timing, the counterpart of the reference's NVMAI_KERNEL_STATS roles
@@ -200,6 +212,7 @@ int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream stream, const nv
                                uint32_t* stats);
 
 
+
 /* ---- prefill: permutation by expert and grouped expert GEMM ------------------------------- */
 
 /* PrefillTokenExpertPair (PrefillRouter.swift:5-28 == prefill.metal:220-225): 16 bytes;
@@ -270,7 +283,11 @@ int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream stream, cons
  * type.  hidden [query_count, hidden_stride]; act_scratch [n_pairs, f] and route_partials
  * [n_pairs, d] are caller-owned, 16-bit.  d and f must be multiples of 64.  The kernel addresses
  * each operand array with 32-bit byte offsets: hidden, act_scratch, an expert's blob and one weight
- * matrix must each span less than 4 GiB (NVMAI_ERR_UNSUPPORTED otherwise). */
+ * matrix must each span less than 4 GiB (NVMAI_ERR_UNSUPPORTED otherwise).
+ * A grouping whose validation failed on the device (grouping->info[2] != 0, where the reference
+ * throws before any compute) runs no product: the call still returns NVMAI_OK, because the
+ * failure is only known on the device, and route_partials is filled with zeros.  Read info[2]
+ * after synchronising before trusting the outputs. */
 int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* experts_base,
                                   uint64_t expert_stride, const nvmai_expert_offsets* off, uint32_t bits,
                                   uint32_t d, uint32_t f, uint32_t num_experts, const void* hidden,

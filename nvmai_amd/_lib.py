@@ -58,6 +58,7 @@ class PrefillGrouping(C.Structure):
 # name -> argtypes (every function returns int unless listed in _OTHER)
 SIGNATURES = {
     "nvmai_hip_ctx_create": [C.c_int, C.c_int, C.POINTER(vp)],
+    "nvmai_hip_ctx_reserve": [vp, C.c_size_t],
     "nvmai_hip_profile_enable": [vp, C.c_int],
     "nvmai_hip_profile_read": [vp, C.c_int, C.POINTER(C.c_double), C.POINTER(u32)],
     "nvmai_expert_offsets_for": [u32, u32, u32, C.POINTER(ExpertOffsets), C.POINTER(u64)],
@@ -105,6 +106,7 @@ SIGNATURES = {
 }
 _OTHER = {
     "nvmai_hip_ctx_destroy": (None, [vp]),
+    "nvmai_hip_ctx_workspace_bytes": (C.c_size_t, [vp]),
     "nvmai_hip_status_string": (C.c_char_p, [C.c_int]),
     "nvmai_int4_affine_gemv": (None, [vp, vp, vp, vp, C.c_size_t, C.c_size_t, vp]),
     "nvmai_sampler_seed_for": (u64, [u64, C.c_int64]),

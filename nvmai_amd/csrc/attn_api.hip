@@ -127,7 +127,7 @@ extern "C" int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream strea
     nc = ((len > 0 ? len : 1) + chunk_len - 1) / chunk_len;
     if (nc > ATTN_MAX_CHUNKS) return NVMAI_ERR_UNSUPPORTED;      // cannot happen: nc <= 512 by construction
     const size_t heads_total = (size_t)batch * num_q_heads;
-    rc = ws_begin(ctx, 2 * ws_round(heads_total * nc * 4) + ws_round(heads_total * nc * head_dim * 4));
+    rc = ws_begin(ctx, stream, 2 * ws_round(heads_total * nc * 4) + ws_round(heads_total * nc * head_dim * 4));
     if (rc) return rc;
     AttnParams p{};
     p.q = q; p.k = (const uint8_t*)k->base; p.v = (const uint8_t*)v->base; p.kv_batch_stride = kv_batch_stride;

@@ -16,6 +16,10 @@ struct nvmai_hip_ctx {
     uint8_t* ws;
     size_t ws_cap;
     size_t ws_used;
+    // Blocks the workspace has outgrown.  They stay allocated until the context is destroyed: a
+    // captured graph keeps the addresses it was recorded with, and replaying it must stay valid
+    // after a later, larger call has moved the workspace.
+    std::vector<void*> ws_retired;
     uint32_t* tickets;       // zero-initialised device words for last-block-done kernels (TICKET_WORDS)
     // Optional per-kernel timing: event pairs recorded around tagged launches.
     bool prof_on;
@@ -39,17 +43,27 @@ constexpr uint32_t TICKET_GROUPS = 64;
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Make the workspace at least `bytes` large and reset the bump pointer.  Growing
-// waits for the device (hipFree does) and is meant to happen during warm-up.
-inline int ws_begin(nvmai_hip_ctx* ctx, size_t bytes) {
+// Make the workspace at least `bytes` large and reset the bump pointer.  Growing allocates a new
+// block (sizes double, so the retired blocks together are smaller than the live one) and never
+// frees the old one: launches already recorded into a graph keep pointing at it.  A call that
+// would have to grow while `stream` is being captured returns NVMAI_ERR_SCRATCH instead of
+// allocating inside the capture: size the workspace first, with an eager call of the same shape
+// or with nvmai_hip_ctx_reserve.
+inline int ws_begin(nvmai_hip_ctx* ctx, nvmai_stream stream, size_t bytes) {
     ctx->ws_used = 0;
     if (bytes <= ctx->ws_cap) return NVMAI_OK;
+    hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &cap_status) != hipSuccess) {
+        (void)hipGetLastError();
+        cap_status = hipStreamCaptureStatusNone;
+    }
+    if (cap_status != hipStreamCaptureStatusNone) return NVMAI_ERR_SCRATCH;
     size_t cap = ctx->ws_cap ? ctx->ws_cap : (size_t)1 << 20;
     while (cap < bytes) cap *= 2;
-    if (ctx->ws) NVMAI_HIP_TRY(hipFree(ctx->ws));
-    ctx->ws = nullptr;
-    ctx->ws_cap = 0;
-    NVMAI_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&ctx->ws), cap));
+    uint8_t* block = nullptr;
+    NVMAI_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&block), cap));
+    if (ctx->ws) ctx->ws_retired.push_back(ctx->ws);
+    ctx->ws = block;
     ctx->ws_cap = cap;
     return NVMAI_OK;
 }

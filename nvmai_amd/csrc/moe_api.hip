@@ -39,11 +39,20 @@ extern "C" int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** o
 extern "C" void nvmai_hip_ctx_destroy(nvmai_hip_ctx* ctx) {
     if (!ctx) return;
     if (ctx->ws) (void)hipFree(ctx->ws);
+    for (void* block : ctx->ws_retired) (void)hipFree(block);
     if (ctx->tickets) (void)hipFree(ctx->tickets);
     for (auto& sp : ctx->prof_spans) { (void)hipEventDestroy(sp.start); (void)hipEventDestroy(sp.stop); }
     for (auto& e : ctx->prof_free) (void)hipEventDestroy(e);
     delete ctx;
 }
+
+extern "C" int nvmai_hip_ctx_reserve(nvmai_hip_ctx* ctx, size_t bytes) {
+    if (!ctx) return NVMAI_ERR_INVALID_ARG;
+    NVMAI_HIP_TRY(hipSetDevice(ctx->device));
+    return ws_begin(ctx, nullptr, bytes);
+}
+
+extern "C" size_t nvmai_hip_ctx_workspace_bytes(const nvmai_hip_ctx* ctx) { return ctx ? ctx->ws_cap : 0; }
 
 extern "C" int nvmai_hip_profile_enable(nvmai_hip_ctx* ctx, int on) {
     if (!ctx) return NVMAI_ERR_INVALID_ARG;
@@ -494,7 +503,7 @@ int affine_gemv_any(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weig
     const bool need_tmp = (y != nullptr) || y_stride != m;
     size_t need = ws_round(ents * sizeof(WorkEntry)) + ws_round(16) + 2 * ws_round(n_tokens * 4u) +
                   (need_tmp ? ws_round((size_t)n_tokens * m * 4u) : 0);
-    int rc = ws_begin(ctx, need);
+    int rc = ws_begin(ctx, stream, need);
     if (rc) return rc;
     WorkEntry* entries = ws_take<WorkEntry>(ctx, ents);
     uint32_t* n_entries = ws_take<uint32_t>(ctx, 4);
@@ -595,7 +604,7 @@ extern "C" int nvmai_hip_moe_router_topk(nvmai_hip_ctx* ctx, nvmai_stream stream
     hipStream_t s = (hipStream_t)stream;
     float* logits = logits_out;
     if (!logits) {
-        rc = ws_begin(ctx, ws_round((size_t)n_tokens * num_experts * 4));
+        rc = ws_begin(ctx, stream, ws_round((size_t)n_tokens * num_experts * 4));
         if (rc) return rc;
         logits = ws_take<float>(ctx, (size_t)n_tokens * num_experts);
     }
@@ -654,7 +663,7 @@ extern "C" int nvmai_hip_moe_phase1_gate_up_act_subset(
             return launch_status();
         }
     }
-    rc = ws_begin(ctx, ws_round(8 * sizeof(WorkEntry)) + 3 * ws_round(64));
+    rc = ws_begin(ctx, stream, ws_round(8 * sizeof(WorkEntry)) + 3 * ws_round(64));
     if (rc) return rc;
     WorkEntry* entries = ws_take<WorkEntry>(ctx, 8);
     uint32_t* n_entries = ws_take<uint32_t>(ctx, 4);
@@ -709,7 +718,7 @@ extern "C" int nvmai_hip_moe_phase2_down_reduce(nvmai_hip_ctx* ctx, nvmai_stream
             return launch_status();
         }
     }
-    rc = ws_begin(ctx, ws_round(8 * sizeof(WorkEntry)) + 3 * ws_round(64) + ws_round((size_t)top_k * d * 4));
+    rc = ws_begin(ctx, stream, ws_round(8 * sizeof(WorkEntry)) + 3 * ws_round(64) + ws_round((size_t)top_k * d * 4));
     if (rc) return rc;
     WorkEntry* entries = ws_take<WorkEntry>(ctx, 8);
     uint32_t* n_entries = ws_take<uint32_t>(ctx, 4);
@@ -755,7 +764,7 @@ extern "C" int nvmai_hip_shared_expert(nvmai_hip_ctx* ctx, nvmai_stream stream, 
     if (n_tokens >= 192 && (uint64_t)n_tokens * x_stride * 2 <= 0xFFFFFFFFull &&
         (uint64_t)n_tokens * d * 2 <= 0xFFFFFFFFull && (uint64_t)d * f * bits / 8 <= 0xFFFFFFFFull) {
         const bool gated_d = shared_gate && shared_gate->kind;
-        rc = ws_begin(ctx, ws_round((size_t)n_tokens * f * 2) + ws_round((size_t)n_tokens * d * 2) +
+        rc = ws_begin(ctx, stream, ws_round((size_t)n_tokens * f * 2) + ws_round((size_t)n_tokens * d * 2) +
                                ws_round(n_tokens * 4u) + ws_round(16));
         if (rc) return rc;
         uint16_t* act = ws_take<uint16_t>(ctx, (size_t)n_tokens * f);
@@ -783,7 +792,7 @@ extern "C" int nvmai_hip_shared_expert(nvmai_hip_ctx* ctx, nvmai_stream stream, 
         if (n_tokens <= 4 && (d * bits) % 128 == 0 && (c1 == 64 || c1 == 128) && (f * bits) % 128 == 0 &&
             (c2 == 16 || c2 == 32 || c2 == 64)) {
             const bool gated_s = shared_gate && shared_gate->kind;
-            rc = ws_begin(ctx, ws_round((size_t)n_tokens * f * 4) + ws_round(n_tokens * 4u) + ws_round(16));
+            rc = ws_begin(ctx, stream, ws_round((size_t)n_tokens * f * 4) + ws_round(n_tokens * 4u) + ws_round(16));
             if (rc) return rc;
             float* acts = ws_take<float>(ctx, (size_t)n_tokens * f);
             float* gate_logit = ws_take<float>(ctx, n_tokens);
@@ -815,7 +824,7 @@ extern "C" int nvmai_hip_shared_expert(nvmai_hip_ctx* ctx, nvmai_stream stream, 
     size_t need = ws_round(ents * sizeof(WorkEntry)) + ws_round(16) + 2 * ws_round(n_tokens * 4u) +
                   ws_round((size_t)n_tokens * f * 4) + ws_round((size_t)n_tokens * d * 4) +
                   ws_round(n_tokens * 4u) + ws_round(16);
-    rc = ws_begin(ctx, need);
+    rc = ws_begin(ctx, stream, need);
     if (rc) return rc;
     WorkEntry* entries = ws_take<WorkEntry>(ctx, ents);
     uint32_t* n_entries = ws_take<uint32_t>(ctx, 4);
@@ -859,10 +868,25 @@ extern "C" int nvmai_hip_shared_expert(nvmai_hip_ctx* ctx, nvmai_stream stream, 
 // ---------------------------------------------------------------------------
 // fused decode layer
 // ---------------------------------------------------------------------------
-extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream stream,
-                                          const nvmai_moe_layer* L, const void* x, uint32_t x_stride,
-                                          uint32_t n_tokens, void* y, uint32_t y_stride,
-                                          uint32_t* out_idx, uint16_t* out_w, uint32_t* stats) {
+namespace {
+
+// Intermediate buffers of a decode step, cut from one block by a bump pointer.
+struct Carver {
+    uint8_t* base;
+    size_t used;
+    template <typename T>
+    T* take(size_t count) {
+        T* p = reinterpret_cast<T*>(base + used);
+        used += ws_round(count * sizeof(T));
+        return p;
+    }
+};
+
+// fixed_ws == nullptr: the buffers come from the context's workspace (grown when needed);
+// otherwise from the fixed_cap bytes at fixed_ws, and a step that needs more is refused.
+int decode_layer_impl(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_moe_layer* L, const void* x,
+                      uint32_t x_stride, uint32_t n_tokens, void* y, uint32_t y_stride, uint32_t* out_idx,
+                      uint16_t* out_w, uint32_t* stats, uint8_t* fixed_ws, size_t fixed_cap) {
     if (!ctx || !L || !x || !y) return NVMAI_ERR_INVALID_ARG;
     int rc = check_shape(L->d, L->f, L->bits);
     if (rc) return rc;
@@ -893,18 +917,24 @@ extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream strea
                   ws_round(pairs * 2u) + ws_round(max_entries * sizeof(WorkEntry)) + ws_round(16) +
                   2 * ws_round(rows_total * 4u) + ws_round((size_t)rows_total * F * 4) +
                   ws_round((size_t)rows_total * D * 4);
-    rc = ws_begin(ctx, need);
-    if (rc) return rc;
-    float* logits = ws_take<float>(ctx, (size_t)T * E);
-    float* gate_logit = ws_take<float>(ctx, T);
-    uint32_t* idx = ws_take<uint32_t>(ctx, pairs);
-    uint16_t* wts = ws_take<uint16_t>(ctx, pairs);
-    WorkEntry* entries = ws_take<WorkEntry>(ctx, max_entries);
-    uint32_t* n_entries = ws_take<uint32_t>(ctx, 4);
-    uint32_t* pair_token = ws_take<uint32_t>(ctx, rows_total);
-    uint32_t* pair_id = ws_take<uint32_t>(ctx, rows_total);
-    float* acts = ws_take<float>(ctx, (size_t)rows_total * F);
-    float* partials = ws_take<float>(ctx, (size_t)rows_total * D);
+    Carver cv{fixed_ws, 0};
+    if (fixed_ws) {
+        if (need > fixed_cap) return NVMAI_ERR_SCRATCH;
+    } else {
+        rc = ws_begin(ctx, stream, need);
+        if (rc) return rc;
+        cv.base = ctx->ws;
+    }
+    float* logits = cv.take<float>((size_t)T * E);
+    float* gate_logit = cv.take<float>(T);
+    uint32_t* idx = cv.take<uint32_t>(pairs);
+    uint16_t* wts = cv.take<uint16_t>(pairs);
+    WorkEntry* entries = cv.take<WorkEntry>(max_entries);
+    uint32_t* n_entries = cv.take<uint32_t>(4);
+    uint32_t* pair_token = cv.take<uint32_t>(rows_total);
+    uint32_t* pair_id = cv.take<uint32_t>(rows_total);
+    float* acts = cv.take<float>((size_t)rows_total * F);
+    float* partials = cv.take<float>((size_t)rows_total * D);
     if (out_idx) idx = out_idx;
     if (out_w) wts = out_w;
 
@@ -969,4 +999,13 @@ extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream strea
     cp.y_stride = y_stride; cp.y = y;
     { ProfScope ps(ctx, NVMAI_PROF_COMBINE, s); run_combine(ctx->act, cp, s); }
     return launch_status();
+}
+
+}  // namespace
+
+extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                          const nvmai_moe_layer* L, const void* x, uint32_t x_stride,
+                                          uint32_t n_tokens, void* y, uint32_t y_stride,
+                                          uint32_t* out_idx, uint16_t* out_w, uint32_t* stats) {
+    return decode_layer_impl(ctx, stream, L, x, x_stride, n_tokens, y, y_stride, out_idx, out_w, stats, nullptr, 0);
 }

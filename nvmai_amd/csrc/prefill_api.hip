@@ -85,7 +85,7 @@ extern "C" int nvmai_hip_prefill_group_pairs(nvmai_hip_ctx* ctx, nvmai_stream st
         return NVMAI_ERR_INVALID_ARG;
     if (n_pairs >= (1u << 28) || num_experts > MAX_GROUP_EXPERTS) return NVMAI_ERR_UNSUPPORTED;
     const uint32_t n = (uint32_t)n_pairs, n_blocks = (n + GROUP_CHUNK - 1) / GROUP_CHUNK;
-    rc = ws_begin(ctx, 3 * ws_round((size_t)n * 4) + 2 * ws_round((size_t)n_blocks * num_experts * 4));
+    rc = ws_begin(ctx, stream, 3 * ws_round((size_t)n * 4) + 2 * ws_round((size_t)n_blocks * num_experts * 4));
     if (rc) return rc;
     uint32_t* first = ws_take<uint32_t>(ctx, n);
     uint32_t* slot_expert = ws_take<uint32_t>(ctx, n);
@@ -121,7 +121,7 @@ extern "C" int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream s
         return NVMAI_ERR_INVALID_ARG;
     if (n_pairs >= (1u << 28) || num_experts > MAX_GROUP_EXPERTS) return NVMAI_ERR_UNSUPPORTED;
     const uint32_t n = (uint32_t)n_pairs, n_blocks = (n + GROUP_CHUNK - 1) / GROUP_CHUNK;
-    rc = ws_begin(ctx, 2 * ws_round((size_t)n_blocks * num_experts * 4));
+    rc = ws_begin(ctx, stream, 2 * ws_round((size_t)n_blocks * num_experts * 4));
     if (rc) return rc;
     uint32_t* block_hist = ws_take<uint32_t>(ctx, (size_t)n_blocks * num_experts);
     uint32_t* block_base = ws_take<uint32_t>(ctx, (size_t)n_blocks * num_experts);
@@ -222,13 +222,14 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
     if (n_pairs == 0) return NVMAI_OK;
     // full tiles + one remainder per expert + the padding of the list's last long and short rows
     const uint32_t max_mtiles = (uint32_t)(n_pairs / GEMM_BM) + (num_experts < n_pairs ? num_experts : (uint32_t)n_pairs) + 14;
-    rc = ws_begin(ctx, ws_round((size_t)max_mtiles * sizeof(MTile)) + ws_round(64));
+    rc = ws_begin(ctx, stream, ws_round((size_t)max_mtiles * sizeof(MTile)) + ws_round(64));
     if (rc) return rc;
     MTile* mtiles = ws_take<MTile>(ctx, max_mtiles);
     uint32_t* n_mtiles = ws_take<uint32_t>(ctx, 16);
     hipStream_t s = (hipStream_t)stream;
     prefill_mtiles_kernel<<<1, 256, 0, s>>>(reinterpret_cast<const PrefillGroup*>(grouping->groups), grouping->info,
-                                            mtiles, n_mtiles);
+                                            mtiles, n_mtiles, reinterpret_cast<uint4*>(route_partials),
+                                            n_pairs * d * 2 / 16);
     const uint32_t nt = bits == 4 ? 4 : 2;        // 16-column tiles per wave: what the register file allows
     GemmParams g1{};
     g1.pool = (const uint8_t*)experts_base; g1.pool_stride = expert_stride;

@@ -422,13 +422,19 @@ constexpr uint32_t GEMM_SHORT_ROWS = 32;   // M tiles of at most this many rows 
 // with empty tiles.  Long tiles keep their groups' order by size (four coarse classes, largest
 // first) so that the experts with the most tiles start early.
 // n_mtiles <= pairs / GEMM_BM + groups + 14.
+// On a grouping that failed validation (info[2] != 0) no tile is listed, and this block zeroes the
+// caller's route partials instead (slowly: it is the error path), so that the reduce after it
+// returns zeros, never whatever the buffer held.
 __global__ __launch_bounds__(256) void prefill_mtiles_kernel(const PrefillGroup* groups, const uint32_t* info,
-                                                            MTile* mtiles, uint32_t* n_mtiles) {
+                                                            MTile* mtiles, uint32_t* n_mtiles,
+                                                            uint4* partials_on_error, uint64_t partials_chunks) {
     __shared__ uint32_t cls_long[4], cur_long[4], n_short, cur_short;
     if (threadIdx.x < 4) { cls_long[threadIdx.x] = 0; cur_long[threadIdx.x] = 0; }
     if (threadIdx.x == 0) { n_short = 0; cur_short = 0; }
     __syncthreads();
     const uint32_t ng = info[2] ? 0u : info[0];               // nothing runs on a grouping that failed
+    if (info[2] && partials_on_error)
+        for (uint64_t i = threadIdx.x; i < partials_chunks; i += 256) partials_on_error[i] = uint4{0, 0, 0, 0};
     // a group's tiles: t - 1 full ones and a last one of `last` rows; its class by t
     auto shape = [](const PrefillGroup& gr, uint32_t& t, uint32_t& last, uint32_t& nl, int& cls) {
         t = (gr.pair_count + GEMM_BM - 1) / GEMM_BM;

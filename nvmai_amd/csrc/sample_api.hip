@@ -22,7 +22,7 @@ extern "C" int nvmai_hip_softmax_tiled(nvmai_hip_ctx* ctx, nvmai_stream stream, 
     if (rows == 0) return NVMAI_OK;
     hipStream_t s = (hipStream_t)stream;
     const uint32_t tiles = (v + SOFTMAX_TILE - 1) / SOFTMAX_TILE;
-    int rc = ws_begin(ctx, 2 * ws_round((size_t)rows * tiles * 4));
+    int rc = ws_begin(ctx, stream, 2 * ws_round((size_t)rows * tiles * 4));
     if (rc) return rc;
     float* tmax = ws_take<float>(ctx, (size_t)rows * tiles);
     float* tsum = ws_take<float>(ctx, (size_t)rows * tiles);
@@ -51,7 +51,7 @@ extern "C" int nvmai_hip_sample_topk64(nvmai_hip_ctx* ctx, nvmai_stream stream, 
     hipStream_t s = (hipStream_t)stream;
     const uint32_t g1 = (v + SAMPLE_TILE - 1) / SAMPLE_TILE, c1 = g1 * SAMPLE_KEEP;
     const uint32_t g2 = (c1 + SAMPLE_TILE - 1) / SAMPLE_TILE, c2 = g2 * SAMPLE_KEEP;
-    int rc = ws_begin(ctx, ws_round((size_t)rows * c1 * 8) + ws_round((size_t)rows * c2 * 8));
+    int rc = ws_begin(ctx, stream, ws_round((size_t)rows * c1 * 8) + ws_round((size_t)rows * c2 * 8));
     if (rc) return rc;
     uint64_t* s1 = ws_take<uint64_t>(ctx, (size_t)rows * c1);
     uint64_t* s2 = ws_take<uint64_t>(ctx, (size_t)rows * c2);
@@ -78,7 +78,7 @@ extern "C" int nvmai_hip_sample(nvmai_hip_ctx* ctx, nvmai_stream stream, const u
     if (temperature > 0.0f && top_k == 0u && (top_p <= 0.0f || top_p >= 1.0f)) {   // logit.metal:391
         PosArray pa{};
         for (uint32_t r = 0; r < rows; ++r) pa.p[r] = positions ? positions[r] : 0u;
-        const int rc = ws_begin(ctx, ws_round((size_t)rows * GUMBEL_BLOCKS * 8));
+        const int rc = ws_begin(ctx, stream, ws_round((size_t)rows * GUMBEL_BLOCKS * 8));
         if (rc) return rc;
         uint64_t* block_best = ws_take<uint64_t>(ctx, (size_t)rows * GUMBEL_BLOCKS);
         sample_gumbel_kernel<<<dim3(GUMBEL_BLOCKS, rows), 256, 0, s>>>(probs, v, probs_stride, temperature, sa, pa,

@@ -463,7 +463,9 @@ __global__ __launch_bounds__(256) void sample_generic_kernel(const uint16_t* pro
         __syncthreads();
     }
     if (threadIdx.x == 0) {
-        if (temperature <= 0.0f) { out_token[row] = idx[0]; return; }
+        // greedy: with no value above -inf (all NaN or -inf) the reference's reduction ends at index 0
+        // (logit.metal:340-382: every lane starts at best_i = 0), never at an out-of-range id
+        if (temperature <= 0.0f) { out_token[row] = idx[0] == 0xFFFFFFFFu ? 0u : idx[0]; return; }
         uint32_t kept = 0;
         while (kept < k && idx[kept] < v && isfinite(val[kept])) kept++;
         out_token[row] = sample_select(val, idx, kept, temperature, top_p, seeds.s[row], kept > 0 ? idx[0] : 0u);

@@ -119,7 +119,7 @@ extern "C" int nvmai_hip_lm_head_greedy(nvmai_hip_ctx* ctx, nvmai_stream stream,
     if (n_tokens == 0) return NVMAI_OK;
     hipStream_t s = (hipStream_t)stream;
     const uint32_t n_blocks = (vocab + LMH_ROWS - 1) / LMH_ROWS;
-    int rc = ws_begin(ctx, ws_round((size_t)n_tokens * n_blocks * sizeof(float2)));
+    int rc = ws_begin(ctx, stream, ws_round((size_t)n_tokens * n_blocks * sizeof(float2)));
     if (rc) return rc;
     LmHeadParams p{};
     p.hidden = (const uint16_t*)hidden; p.hidden_stride = hidden_stride; p.norm_weight = norm_weight;

@@ -35,6 +35,14 @@ class Context:
         check(lib.nvmai_hip_ctx_create(device, act, C.byref(h)), "ctx_create")
         self.handle = h
 
+    def reserve(self, nbytes):
+        """Size the workspace now, so that no later call (a captured one above all) has to grow it."""
+        check(lib.nvmai_hip_ctx_reserve(self.handle, nbytes), "ctx_reserve")
+
+    @property
+    def workspace_bytes(self):
+        return lib.nvmai_hip_ctx_workspace_bytes(self.handle)
+
     def profile_enable(self, on=True):
         check(lib.nvmai_hip_profile_enable(self.handle, int(on)), "profile_enable")
 

@@ -968,7 +968,8 @@ uint32_t orc_sample_generic(const uint16_t *probs_f16, size_t v, float temperatu
             float p = orc_f16_to_float(probs_f16[i]);
             if (p > best) { best = p; bi = (uint32_t)i; }
         }
-        return bi;
+        /* no value above -inf (all NaN or -inf): every lane of the reference keeps best_i = 0 */
+        return bi == 0xFFFFFFFFu ? 0u : bi;
     }
     size_t k = (top_k == 0) ? v : top_k;                      /* :464-467 */
     if (k > 256) k = 256;

@@ -200,3 +200,63 @@ def test_attention_long_context_properties(nv):
     assert O.rel_error(act_np(out)[0], want) < 1e-2
     torch.cuda.synchronize()
     ctx.close()
+
+
+def _long_cache(nv, ctx, gen, batch, seq, elements, bits):
+    """K and V caches of `batch` sequences filled by quantize-on-write from seeded bf16 rows made on
+    the GPU; returns the caches and, per sequence, a few source rows for the code check."""
+    kc, vc = nv.KVCache(batch, seq, elements, bits), nv.KVCache(batch, seq, elements, bits)
+    quant = nv.KVCacheQuantizer(ctx)
+    probes = []
+    for b in range(batch):
+        k = torch.empty((seq, elements), device="cuda").normal_(0.0, 1.0, generator=gen).to(torch.bfloat16)
+        v = torch.empty((seq, elements), device="cuda").normal_(0.0, 1.0, generator=gen).to(torch.bfloat16)
+        quant.encode(k, elements, kc.view(b), seq, elements)
+        quant.encode(v, elements, vc.view(b), seq, elements)
+        rows = np.r_[0:32, seq // 2 - 16:seq // 2 + 16, seq - 32:seq]
+        probes.append((rows, k[torch.from_numpy(rows).cuda()].float().cpu().numpy()))
+    torch.cuda.synchronize()
+    return kc, vc, probes
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("batch,seq,kv_start", [(8, 32768, 0), (1, 131072, 0), (8, 131072, 0), (2, 131067, 77)],
+                         ids=["32Kx8", "128Kx1", "128Kx8", "128K-ragged"])
+def test_attention_configs3_long_context(nv, bits, batch, seq, kv_start):
+    # configs[3] at its long contexts and at batch 8: the production kernel's size-dependent parts
+    # (32-bit row offsets, buffer bounds of seq * stride bytes, up to 512 chunks) against the oracle
+    # on EVERY sequence, KV codes of the quantize-on-write bit-exact on sampled rows, a start
+    # offset and a length that is not a multiple of the 32-token step, and two different chunk
+    # counts (a sequence alone, and inside the batch) giving the same output.
+    say("attention long context", bits, batch, seq, kv_start)
+    ctx = nv.Context(0, 0)
+    nq, nkv, hd = 16, 2, 256
+    elements = nkv * hd
+    gen = torch.Generator(device="cuda").manual_seed(seq % 1000 + 10 * batch + bits)
+    kc, vc, probes = _long_cache(nv, ctx, gen, batch, seq, elements, bits)
+    q = O.round_bf16(gauss(np.random.default_rng(seq + bits), (batch, nq, hd)))
+    attn = nv.Attention(ctx)
+    out = act_np(attn.encode_full(act_tensor(q, ctx), kc, vc, hd, nq, nkv, seq, kv_start=kv_start))
+    torch.cuda.synchronize()
+    worst = 0.0
+    for b in range(batch):
+        rows, src = probes[b]
+        got_rows = kc.rows[b][torch.from_numpy(rows).cuda()].cpu().numpy()
+        assert np.array_equal(got_rows, O.kv_quantize(src, bits)), "KV codes, sequence %d" % b
+        kq, vq = kc.rows[b].cpu().numpy(), vc.rows[b].cpu().numpy()
+        want = O.attention_decode(q[b], kq, vq, bits, nq, nkv, hd, seq, 1 / 16.0, kv_start)
+        err = O.rel_error(out[b], want)
+        worst = max(worst, err)
+        assert err < 1e-2, "sequence %d rel %g" % (b, err)
+        del kq, vq
+    print("worst rel", worst, flush=True)
+    if batch > 1:
+        # the last sequence on its own: batch 1 cuts the range into more chunks than batch 8 does
+        b = batch - 1
+        k1, v1 = nv.KVCache(1, 1, elements, bits), nv.KVCache(1, 1, elements, bits)
+        k1.rows, v1.rows = kc.rows[b:b + 1], vc.rows[b:b + 1]
+        alone = act_np(attn.encode_full(act_tensor(q[b:b + 1], ctx), k1, v1, hd, nq, nkv, seq, kv_start=kv_start))
+        torch.cuda.synchronize()
+        assert O.rel_error(alone[0], out[b]) < 1e-2
+    torch.cuda.synchronize()
+    ctx.close()

@@ -477,3 +477,62 @@ def test_decode_layer_replays_from_a_captured_graph(nv, ctx_bf16, tokens):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y_static, want)
+
+
+def test_captured_graph_survives_workspace_growth(nv):
+    # A captured step keeps the workspace addresses it was recorded with.  A later, larger call on the
+    # same context moves the workspace to a new block; the old block must stay allocated, so that a
+    # replay after the growth still equals the eager result bit for bit.  A call that would have to
+    # grow the workspace while its stream is being captured reports "scratch" and launches nothing.
+    say("graph replay after workspace growth")
+    ctx = nv.Context(0, nv.ACT_BF16)
+    d, f, E, k, bits, tokens = 1024, 256, 24, 8, 8, 12
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    off, stride = nv.expert_offsets(d, f, bits)
+    pool = torch.empty((E + 1, stride), dtype=torch.uint8, device="cuda")
+    mk = lambda r, c, s=0.03: torch.empty((r, c), device="cuda").normal_(0.0, s, generator=gen).to(torch.bfloat16)
+    for e in range(E + 1):
+        nv.pack_expert(ctx, mk(f, d), mk(f, d), mk(d, f), bits, pool[e])
+    router = mk(E, d, 0.05)
+    layer = nv.moe_layer_desc(d, f, E, k, bits, nv.rows_desc(16, router.view(torch.int16)), pool[:E], pool[E])
+    moe = nv.MoE(ctx, bits)
+    x_static = mk(tokens, d, 1.0)
+    y_static = torch.empty((tokens, d), dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.Stream()
+    # (a) no warm-up: the workspace would have to grow inside the capture
+    assert ctx.workspace_bytes == 0
+    refused = torch.cuda.CUDAGraph()
+    err = None
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(refused, stream=stream):
+            y_static.zero_()
+            try:
+                moe.decode_layer(layer, x_static, y_static)
+            except nv.NvmaiError as e:
+                err = e
+    torch.cuda.synchronize()
+    assert err is not None and err.name == "scratch" and ctx.workspace_bytes == 0
+    # (b) reserve a small workspace, capture, then grow it with a 100-token call and replay
+    ctx.reserve(1 << 20)
+    moe.decode_layer(layer, x_static, y_static)
+    torch.cuda.synchronize()
+    before = ctx.workspace_bytes
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            moe.decode_layer(layer, x_static, y_static)
+    torch.cuda.synchronize()
+    big = moe.decode_layer(layer, mk(100, d, 1.0))
+    torch.cuda.synchronize()
+    assert ctx.workspace_bytes > before and bool(torch.isfinite(big.float()).all())
+    for _ in range(3):
+        x = mk(tokens, d, 1.0)
+        want = moe.decode_layer(layer, x).clone()
+        junk = torch.full((1 << 20,), 1.0, device="cuda")          # eager work between the replays
+        torch.cuda.synchronize()
+        del junk
+        x_static.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_static, want)
+    ctx.close()

@@ -345,3 +345,28 @@ def test_dense_qmm_rejects_bad_arguments(nv, ctx_bf16):
     assert e.value.name == "invalid_arg"
     with pytest.raises(nv.NvmaiError):
         nv.MPPPrefillInt4QMM(ctx_bf16, 3)
+
+
+def test_grouped_moe_on_a_failed_grouping_returns_zeros_and_the_error(nv, ctx_bf16):
+    # An expert id out of range: the reference throws expertOutOfRange before any compute
+    # (PrefillMoEGrouping.swift:121-138).  Here the failure is found on the device: the products do
+    # not run, the route partials (handed in full of junk) come back as zeros, so the reduce gives
+    # zeros, and validate() raises the reference's error with the first failing pair.
+    say("prefill grouped moe on a failed grouping")
+    ctx, d, f, E, k, tokens, bits = ctx_bf16, 128, 64, 4, 2, 40, 4
+    rng = np.random.default_rng(11)
+    blobs = np.stack([O.pack_expert(gauss(rng, (f, d), .05), gauss(rng, (f, d), .05), gauss(rng, (d, f), .05), bits)
+                      for _ in range(E)])
+    idx, w = _zipf_routes(rng, tokens, E, k)
+    idx[17, 1] = E + 3
+    off, _ = nv.expert_offsets(d, f, bits)
+    routes = nv.PrefillMoEGrouping(ctx).group_routes(dev(idx.view(np.int32)), dev(w.view(np.int16)), E)
+    junk = torch.full((tokens * k, d), 7.0, dtype=ctx.dtype, device="cuda")
+    partials, _ = nv.PrefillGroupedRoutedMoE(ctx, bits).encode(dev(blobs), off, act_tensor(gauss(rng, (tokens, d)), ctx),
+                                                               d, f, routes, route_partials=junk)
+    h2 = nv.PrefillMoE(ctx).encode_reduce_token_major(partials, dev(w.view(np.int16)), tokens, k, d)
+    torch.cuda.synchronize()
+    assert not act_np(partials).any() and not act_np(h2).any()
+    with pytest.raises(nv.PrefillMoEGroupingError) as e:
+        routes.validate()
+    assert e.value.name == "expertOutOfRange" and e.value.pair_index == 17 * k + 1

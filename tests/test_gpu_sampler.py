@@ -107,6 +107,10 @@ def test_sampler_ties_flat_geometric_and_greedy(nv, ctx):
     tie = np.zeros(512, np.float32)
     tie[[40, 7, 300]] = 0.3
     assert int(gen.encode(_probs_dev(O.f16_bits(tie)), 0.0)[0]) == 7       # lowest index wins a tie
+    # greedy with nothing above -inf (all NaN, all -inf): token 0 as the reference's reduction gives
+    # (logit.metal:340-382), never an out-of-range id
+    assert int(gen.encode(_probs_dev(np.full(512, 0x7E00, np.uint16)), 0.0)[0]) == 0
+    assert int(gen.encode(_probs_dev(np.full(512, 0xFC00, np.uint16)), 0.0)[0]) == 0
     with pytest.raises(nv.NvmaiError):                                     # temperature must be > 0
         nv.SampleTopK64(ctx, 512).encode(pd, 0.0, 0.95, 1, 20)
     with pytest.raises(nv.NvmaiError):                                     # k in 1...64

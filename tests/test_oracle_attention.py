@@ -53,6 +53,31 @@ def test_kv_quantizer_closed_form_and_invariants():
         assert np.all(np.abs(rec - v) <= 0.5 * step + 2e-3 * np.maximum(np.abs(v), 1))
 
 
+def test_kv_codes_are_the_nearest_codes():
+    # The property itself in float64, no rounding rule restated: against the UNROUNDED fp32 scale and
+    # bias of its group (kv_cache_quantize.metal:56-59 quantizes before the pair is rounded to fp16)
+    # every code is at least as close to its value as both neighbouring codes, ties aside.
+    rng = np.random.default_rng(23)
+    for v in (O.round_bf16(rng.standard_normal((64, 512)).astype(np.float32)),
+              rng.uniform(-0.5, 0.5, (16, 512)).astype(np.float32),
+              (rng.standard_normal((8, 512)) * 3 + 20).astype(np.float32)):
+        for bits in (4, 8):
+            levels = 15 if bits == 4 else 255
+            rows = O.kv_quantize(v, bits)
+            _, vb = O.kv_row_layout(512, bits)
+            q = np.stack([O.unpack_codes(r[:vb], bits) for r in rows]).astype(np.float64)
+            g = v.reshape(v.shape[0], -1, 64)
+            mn, mx = g.min(2), g.max(2)
+            s = ((mx - mn) / np.float32(levels)).astype(np.float32).astype(np.float64).repeat(64, axis=1)
+            b = mn.astype(np.float64).repeat(64, axis=1)
+            w = v.astype(np.float64)
+            err = np.abs(w - (q * s + b))
+            tol = 1e-4 * s + 1e-12
+            up_ok = (q >= levels) | (err <= np.abs(w - ((q + 1) * s + b)) + tol)
+            down_ok = (q <= 0) | (err <= np.abs(w - ((q - 1) * s + b)) + tol)
+            assert np.all(up_ok & down_ok), "%d-bit KV codes are not the nearest" % bits
+
+
 def test_kv_quantizer_partial_tail_group():
     v = np.linspace(-1, 1, 3 * 100, dtype=np.float32).reshape(3, 100)
     for bits in (4, 8):

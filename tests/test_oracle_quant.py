@@ -128,6 +128,38 @@ def test_quantizer_matches_brute_force_and_error_bound():
         assert np.array_equal(b, O.bf16_bits(wg.min(2)))
 
 
+def _assert_codes_are_argmin(w, codes, scale, bias, levels, what):
+    """The property itself, in float64 and without any rounding rule: the chosen code is at least as
+    close to the value as both neighbouring codes (|w - (q s + b)| <= |w - ((q +- 1) s + b)|), except
+    within a hair of an exact tie, where the fp32 product decides.  Clamped ends only have one
+    neighbour inside the range.  A quantizer that truncates, rounds the wrong way, is off by one
+    code or swaps scale and bias fails this for most elements."""
+    w, s, b, q = (np.asarray(a, np.float64) for a in (w, scale, bias, codes))
+    err = np.abs(w - (q * s + b))
+    tol = 1e-4 * np.abs(s) + 1e-12
+    up_ok = (q >= levels) | (err <= np.abs(w - ((q + 1) * s + b)) + tol)
+    down_ok = (q <= 0) | (err <= np.abs(w - ((q - 1) * s + b)) + tol)
+    bad = ~(up_ok & down_ok) & (s > 0)
+    assert not bad.any(), "%s: %d codes are not the nearest" % (what, int(bad.sum()))
+    # and values outside the representable range sit on the clamped end
+    assert np.all(q[(w < b) & (s > 0)] == 0) and np.all(q[(w > levels * s + b) & (s > 0)] == levels)
+
+
+def test_quantizer_codes_are_the_nearest_codes():
+    # argmin over codes against the STORED (bf16) scale and bias: that is what makes the packed
+    # codes the reference's (Quantization.swift:80-99 quantizes against the rounded pair)
+    rng = np.random.default_rng(17)
+    for bits in (4, 8):
+        levels = (1 << bits) - 1
+        for w in (O.round_bf16((rng.standard_normal((48, 2048)) * 0.02).astype(np.float32)),
+                  rng.uniform(-1, 1, (16, 512)).astype(np.float32),
+                  (rng.standard_normal((8, 256)) * 30 + 100).astype(np.float32)):      # positive-only groups
+            p, s, b = O.quantize_affine(w, bits)
+            codes = O.unpack_codes(p, bits).reshape(w.shape)
+            _assert_codes_are_argmin(w, codes, O.bf16_to_float(s).repeat(64, axis=1),
+                                     O.bf16_to_float(b).repeat(64, axis=1), levels, "weights %d bit" % bits)
+
+
 def test_expert_offsets_known_answers():
     # CPUExpertFFNTests.swift:56-67
     o = O.expert_offsets(2048, 512, 4)

@@ -102,6 +102,11 @@ def test_sampler_distribution_and_greedy():
     got = np.array([counts[10], counts[20], counts[30]]) / n
     assert np.abs(got - w).max() < 0.03
     assert O.sample_generic(pb, 0.0, 20, 0.95, 1) == 10          # greedy argmax
+    # nothing above -inf: the reference's reduction starts every lane at index 0 and ends there
+    # (logit.metal:340-382); an out-of-range id must never reach the generation loop
+    nan_bits = np.full(512, 0x7E00, np.uint16)
+    assert O.sample_generic(nan_bits, 0.0, 20, 0.95, 1) == 0
+    assert O.sample_generic(np.full(512, 0xFC00, np.uint16), 0.0, 0, 1.0, 1) == 0      # all -inf
     assert O.sample_topk64(pb, 1.0, 0.4, 77, 20) == 10           # nucleus cut at the first entry
 
 
