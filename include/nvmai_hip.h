@@ -211,6 +211,23 @@ int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream stream, const nv
                                uint32_t y_stride, uint32_t* out_idx, uint16_t* out_w,
                                uint32_t* stats);
 
+/* nvmai_hip_moe_decode_layer for callers that cannot allocate.  It has no counterpart in the
+ * reference: it is for code under HIP graph capture, tight serving loops and harnesses that
+ * forbid hipMalloc.  Same arguments, same results bit for bit, but the step's intermediate
+ * buffers (router logits, work list, activations, partial sums) live in a static device array
+ * of nvmai_hip_moe_decode_layer_noalloc_scratch_bytes() = 4 MiB inside the library, whose
+ * device address the ctx looked up when it was created: the call allocates nothing, frees
+ * nothing and records no memset, only kernel launches.  A step that needs more than the array
+ * holds (the production shape fits 32 tokens: hidden 2048, intermediate 512, 256 experts,
+ * top-8, shared expert) returns NVMAI_ERR_SCRATCH and launches nothing.  Every call on one
+ * GPU shares that GPU's array and finds the previous call's contents in it (each call writes
+ * what it reads, nothing has to be cleared): calls that overlap on one GPU, from different
+ * streams or contexts, race. */
+int nvmai_hip_moe_decode_layer_noalloc(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                       const nvmai_moe_layer* layer, const void* x, uint32_t x_stride,
+                                       uint32_t n_tokens, void* y, uint32_t y_stride, uint32_t* out_idx,
+                                       uint16_t* out_w, uint32_t* stats);
+size_t nvmai_hip_moe_decode_layer_noalloc_scratch_bytes(void);
 
 
 /* ---- prefill: permutation by expert and grouped expert GEMM ------------------------------- */

@@ -76,6 +76,7 @@ SIGNATURES = {
     "nvmai_hip_shared_expert": [vp, vp, vp, C.POINTER(ExpertOffsets), u32, C.POINTER(Rows), vp,
                                 u32, u32, vp, u32, u32, u32],
     "nvmai_hip_moe_decode_layer": [vp, vp, C.POINTER(MoeLayer), vp, u32, u32, vp, u32, vp, vp, vp],
+    "nvmai_hip_moe_decode_layer_noalloc": [vp, vp, C.POINTER(MoeLayer), vp, u32, u32, vp, u32, vp, vp, vp],
     "nvmai_kv_row_layout": [u32, u32, C.POINTER(u32), C.POINTER(u32)],
     "nvmai_hip_kv_quantize_affine": [vp, vp, vp, u32, C.POINTER(KvView), u32, u32],
     "nvmai_hip_rope_neox_subdim": [vp, vp, vp, u32, u32, u32, u32, vp, u32, C.c_float],
@@ -107,6 +108,7 @@ SIGNATURES = {
 _OTHER = {
     "nvmai_hip_ctx_destroy": (None, [vp]),
     "nvmai_hip_ctx_workspace_bytes": (C.c_size_t, [vp]),
+    "nvmai_hip_moe_decode_layer_noalloc_scratch_bytes": (C.c_size_t, []),
     "nvmai_hip_status_string": (C.c_char_p, [C.c_int]),
     "nvmai_int4_affine_gemv": (None, [vp, vp, vp, vp, C.c_size_t, C.c_size_t, vp]),
     "nvmai_sampler_seed_for": (u64, [u64, C.c_int64]),

@@ -20,6 +20,7 @@ struct nvmai_hip_ctx {
     // captured graph keeps the addresses it was recorded with, and replaying it must stay valid
     // after a later, larger call has moved the workspace.
     std::vector<void*> ws_retired;
+    uint8_t* static_scratch; // device address of the library's static scratch array on this device (moe_api.hip)
     uint32_t* tickets;       // zero-initialised device words for last-block-done kernels (TICKET_WORDS)
     // Optional per-kernel timing: event pairs recorded around tagged launches.
     bool prof_on;

@@ -9,6 +9,34 @@
 
 using namespace nvmai;
 
+namespace {
+
+// Scratch of the allocation-free decode entry point: one array per device, in the library's image,
+// so that a caller which may not allocate (HIP graph capture, a serving loop, a harness that
+// forbids hipMalloc) still has the step's intermediate buffers.  Host code never uses the
+// array's name as an address: the device address comes from hipGetSymbolAddress, once per device.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)4 << 20;
+static __device__ __align__(256) __attribute__((used)) uint8_t scratch[STATIC_SCRATCH_BYTES];
+constexpr int STATIC_SCRATCH_MAX_DEVICES = 64;
+uint8_t* g_static_scratch[STATIC_SCRATCH_MAX_DEVICES];   // device address of `scratch` on each device, nullptr = not asked yet
+
+// The device address of this device's copy of the array (the device must be current).
+int static_scratch_ptr(int device, uint8_t** out) {
+    if (device < 0 || device >= STATIC_SCRATCH_MAX_DEVICES) return NVMAI_ERR_INVALID_ARG;
+    if (!g_static_scratch[device]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            return NVMAI_ERR_HIP;
+        }
+        g_static_scratch[device] = static_cast<uint8_t*>(ptr);
+    }
+    *out = g_static_scratch[device];
+    return NVMAI_OK;
+}
+
+}  // namespace
+
 // ---------------------------------------------------------------------------
 // context
 // ---------------------------------------------------------------------------
@@ -32,6 +60,10 @@ extern "C" int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** o
         delete ctx;
         return NVMAI_ERR_HIP;
     }
+    // device address of this device's static scratch array (nullptr if the lookup fails: only the
+    // allocation-free entry point needs it, and it then reports the failure)
+    ctx->static_scratch = nullptr;
+    (void)static_scratch_ptr(device, &ctx->static_scratch);
     *out = ctx;
     return NVMAI_OK;
 }
@@ -1008,4 +1040,19 @@ extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream strea
                                           uint32_t n_tokens, void* y, uint32_t y_stride,
                                           uint32_t* out_idx, uint16_t* out_w, uint32_t* stats) {
     return decode_layer_impl(ctx, stream, L, x, x_stride, n_tokens, y, y_stride, out_idx, out_w, stats, nullptr, 0);
+}
+
+extern "C" size_t nvmai_hip_moe_decode_layer_noalloc_scratch_bytes(void) { return STATIC_SCRATCH_BYTES; }
+
+// The same step with its intermediate buffers in the library's static device array: no hipMalloc,
+// no hipFree, no memset, nothing but kernel launches.  The array's device address was fetched when
+// the context was created; every call on a device shares that device's one array.
+extern "C" int nvmai_hip_moe_decode_layer_noalloc(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                                  const nvmai_moe_layer* L, const void* x, uint32_t x_stride,
+                                                  uint32_t n_tokens, void* y, uint32_t y_stride,
+                                                  uint32_t* out_idx, uint16_t* out_w, uint32_t* stats) {
+    if (!ctx) return NVMAI_ERR_INVALID_ARG;
+    if (!ctx->static_scratch) return NVMAI_ERR_HIP;     // the symbol lookup failed at context creation
+    return decode_layer_impl(ctx, stream, L, x, x_stride, n_tokens, y, y_stride, out_idx, out_w, stats,
+                             ctx->static_scratch, STATIC_SCRATCH_BYTES);
 }

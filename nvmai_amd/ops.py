@@ -213,6 +213,15 @@ class MoE:
               "moe_decode_layer")
         return (y, idx, w) if want_routes else y
 
+    def decode_layer_noalloc(self, layer, x, y, idx=None, w=None, stats=None):
+        """nvmai_hip_moe_decode_layer_noalloc: the same step with its intermediate buffers in the
+        library's static device array; every output is the caller's, nothing is allocated."""
+        x2 = x.reshape(-1, x.shape[-1])
+        check(lib.nvmai_hip_moe_decode_layer_noalloc(self.ctx.handle, _stream(), C.byref(layer), _ptr(x2),
+                                                     x2.stride(0), x2.shape[0], _ptr(y), y.stride(0), _ptr(idx),
+                                                     _ptr(w), _ptr(stats)), "moe_decode_layer_noalloc")
+        return y
+
 
 def moe_layer_desc(d, f, num_experts, top_k, bits, router, experts, shared_blob=None, shared_gate=None,
                    eff_scale=None, per_expert_scale=None):
