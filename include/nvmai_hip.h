@@ -409,6 +409,43 @@ int nvmai_hip_sample(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint16_t* pr
                      uint32_t top_k, float top_p, const uint64_t* seeds, const uint32_t* positions,
                      uint32_t* out_token);
 
+/* Sampler.applyRepetitionPenaltyInPlace (Sampler.swift:259-293) on the device, in place on one row
+ * of `v` logits (activations): for every distinct id of history_ids (device int32 [n_ids]; ids
+ * outside the vocabulary are skipped, repeats count once) a positive logit is divided by
+ * `penalty`, a negative one multiplied; with logit_softcap > 0 the penalty acts on the capped
+ * logit and is mapped back through atanh.  penalty == 1 or n_ids == 0 does nothing. */
+int nvmai_hip_repetition_penalty(nvmai_hip_ctx* ctx, nvmai_stream stream, void* logits, uint32_t v,
+                                 const int32_t* history_ids, uint32_t n_ids, float penalty,
+                                 float logit_softcap);
+
+/* GenerationConfig (Sampler.swift:19-81), the fields Sampler.sample reads.  top_k 0 and top_p 0
+ * stand for the reference's nil (no top-k cap; top-p 1.0); has_seed 0 = clock-derived seed. */
+typedef struct {
+    float temperature;          /* >= 0; 0 = greedy */
+    int32_t top_k;              /* 0 = nil, else 1..256 */
+    float top_p;                /* 0 = nil, else (0, 1] */
+    float repetition_penalty;   /* 1 = off */
+    uint64_t seed;
+    int32_t has_seed;
+} nvmai_generation_config;
+enum { NVMAI_SAMPLER_TILED = 0, NVMAI_SAMPLER_GENERIC = 1 };                     /* RuntimeSamplerPath */
+enum { NVMAI_SAMPLE_PATH_GREEDY = 0, NVMAI_SAMPLE_PATH_SAMPLED = 1, NVMAI_SAMPLE_PATH_PENALTY = 2 };   /* SamplePath */
+
+/* Sampler.sample (Sampler.swift:171-234) for one row: the repetition penalty over the history
+ * (when the penalty is not 1 and the history is not empty; edits `logits` in place), softcap +
+ * softmax into probs (FP16 [v] scratch), then the tiled top-64 sampler when sampler_path is
+ * NVMAI_SAMPLER_TILED, temperature > 0, top_k is 1..64 and v is within that sampler's 262,144,
+ * else the generic kernel (greedy at
+ * temperature 0, Gumbel-max without top-k and top-p, k argmax passes otherwise), with the seed
+ * of Sampler.seedFor(config, position).  path_taken (optional, host) receives the SamplePath.
+ * A configuration GenerationConfig.validate refuses returns NVMAI_ERR_INVALID_ARG; top_p below
+ * one without top_k returns NVMAI_ERR_UNSUPPORTED, as it throws there. */
+int nvmai_hip_sampler_sample(nvmai_hip_ctx* ctx, nvmai_stream stream, void* logits, uint16_t* probs,
+                             uint32_t v, const int32_t* history_ids, uint32_t n_history,
+                             const nvmai_generation_config* config, int64_t position,
+                             float logit_softcap, int sampler_path, uint32_t* out_token,
+                             int* path_taken);
+
 /* ---- the small operators around the MoE block of a decode step ---------------------------- */
 
 /* RMSNorm.encodeBF16W / encodeNoScale / encodeBF16WPerHead / encodeNoScalePerHead

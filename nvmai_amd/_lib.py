@@ -50,6 +50,12 @@ class KvView(C.Structure):
     _fields_ = [("base", vp), ("stride", u32), ("value_bytes", u32), ("bits", u32), ("group_size", u32)]
 
 
+class GenerationConfig(C.Structure):
+    """nvmai_generation_config"""
+    _fields_ = [("temperature", C.c_float), ("top_k", i32), ("top_p", C.c_float), ("repetition_penalty", C.c_float),
+                ("seed", u64), ("has_seed", i32)]
+
+
 class PrefillGrouping(C.Structure):
     """nvmai_prefill_grouping"""
     _fields_ = [(n, vp) for n in ("sorted_pairs", "expert_offsets", "expert_counts", "groups", "tiles", "info")]
@@ -103,6 +109,9 @@ SIGNATURES = {
     "nvmai_hip_rmsnorm": [vp, vp, vp, u32, vp, vp, u32, u32, u32, C.c_float],
     "nvmai_hip_embed_lookup": [vp, vp, vp, vp, vp, u32, vp, u32, u32, vp, u32, u32, u32, C.c_float],
     "nvmai_hip_lm_head_greedy": [vp, vp, vp, u32, u32, vp, vp, vp, vp, u32, vp, u32, u32, C.c_float],
+    "nvmai_hip_repetition_penalty": [vp, vp, vp, u32, vp, u32, C.c_float, C.c_float],
+    "nvmai_hip_sampler_sample": [vp, vp, vp, vp, u32, vp, u32, C.POINTER(GenerationConfig), C.c_int64, C.c_float,
+                                 C.c_int, vp, C.POINTER(C.c_int)],
     "nvmai_hip_sample": [vp, vp, vp, u32, u32, u32, C.c_float, u32, C.c_float, C.POINTER(u64), C.POINTER(u32), vp],
 }
 _OTHER = {

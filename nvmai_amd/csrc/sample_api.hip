@@ -1,4 +1,8 @@
 // Entry points: tiled softmax over the vocabulary, top-64 and generic samplers.
+#include <time.h>
+
+#include <atomic>
+
 #include "ctx.hpp"
 #include "sample_kernels.cuh"
 
@@ -88,4 +92,72 @@ extern "C" int nvmai_hip_sample(nvmai_hip_ctx* ctx, nvmai_stream stream, const u
     }
     sample_generic_kernel<<<dim3(rows), 256, 0, s>>>(probs, v, probs_stride, temperature, top_k, top_p, sa, out_token);
     return launch_status();
+}
+
+extern "C" int nvmai_hip_repetition_penalty(nvmai_hip_ctx* ctx, nvmai_stream stream, void* logits, uint32_t v,
+                                            const int32_t* history_ids, uint32_t n_ids, float penalty,
+                                            float logit_softcap) {
+    if (!ctx || !logits || v == 0 || (n_ids && !history_ids)) return NVMAI_ERR_INVALID_ARG;
+    if (!(penalty > 0.0f)) return NVMAI_ERR_INVALID_ARG;
+    if (n_ids == 0 || penalty == 1.0f) return NVMAI_OK;          // Sampler.swift:181
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((n_ids + 255) / 256);
+    if (ctx->act == ACT_BF16)
+        repetition_penalty_kernel<ACT_BF16><<<grid, 256, 0, s>>>((uint16_t*)logits, v, history_ids, n_ids, penalty, logit_softcap);
+    else
+        repetition_penalty_kernel<ACT_FP16><<<grid, 256, 0, s>>>((uint16_t*)logits, v, history_ids, n_ids, penalty, logit_softcap);
+    return launch_status();
+}
+
+namespace {
+// Sampler.seedFor without a configured seed (Sampler.swift:311-323): the monotonic clock mixed
+// with a process-wide counter, never zero.
+uint64_t clock_seed() {
+    static std::atomic<uint64_t> counter{0};
+    timespec t{};
+    clock_gettime(CLOCK_MONOTONIC, &t);
+    const uint64_t c = counter.fetch_add(1, std::memory_order_relaxed) + 1;
+    const uint64_t raw = ((uint64_t)t.tv_nsec + c) * 0x9E3779B97F4A7C15ull + (uint64_t)t.tv_sec;
+    return raw == 0 ? 0x9E3779B97F4A7C15ull : raw;
+}
+}  // namespace
+
+extern "C" int nvmai_hip_sampler_sample(nvmai_hip_ctx* ctx, nvmai_stream stream, void* logits, uint16_t* probs,
+                                        uint32_t v, const int32_t* history_ids, uint32_t n_history,
+                                        const nvmai_generation_config* config, int64_t position,
+                                        float logit_softcap, int sampler_path, uint32_t* out_token,
+                                        int* path_taken) {
+    if (!ctx || !logits || !probs || !config || !out_token || v == 0) return NVMAI_ERR_INVALID_ARG;
+    if (sampler_path != NVMAI_SAMPLER_TILED && sampler_path != NVMAI_SAMPLER_GENERIC) return NVMAI_ERR_INVALID_ARG;
+    // GenerationConfig.validate (Sampler.swift:54-80), the parts the sampler reads
+    const float T = config->temperature;
+    if (!(T >= 0.0f) || T > 3.4e38f) return NVMAI_ERR_INVALID_ARG;
+    if (config->top_k < 0 || config->top_k > 256) return NVMAI_ERR_INVALID_ARG;
+    if (config->top_p < 0.0f || config->top_p > 1.0f || config->top_p != config->top_p) return NVMAI_ERR_INVALID_ARG;
+    const bool has_k = config->top_k > 0, has_p = config->top_p > 0.0f;
+    if (T > 0.0f && !has_k && has_p && config->top_p < 1.0f) return NVMAI_ERR_UNSUPPORTED;   // :76-79
+    const bool penalty = config->repetition_penalty != 1.0f && n_history > 0;                // :180
+    if (penalty) {
+        const int rc = nvmai_hip_repetition_penalty(ctx, stream, logits, v, history_ids, n_history,
+                                                    config->repetition_penalty, logit_softcap);
+        if (rc) return rc;
+    }
+    // one front end serves both paths here: the tiled and the single-group softmax of the
+    // reference agree to 1e-5 and differ only in how the work is cut
+    int rc = nvmai_hip_softmax_tiled(ctx, stream, logits, v, probs, v, 1, v, logit_softcap);
+    if (rc) return rc;
+    const uint64_t seed = config->has_seed ? nvmai_sampler_seed_for(config->seed, position) : clock_seed();
+    const float top_p = has_p ? config->top_p : 1.0f;
+    if (sampler_path == NVMAI_SAMPLER_TILED && T > 0.0f && has_k && config->top_k <= 64 && v <= 262144) {   // :211-214
+        rc = nvmai_hip_sample_topk64(ctx, stream, probs, v, 1, v, T, top_p, &seed, (uint32_t)config->top_k, out_token,
+                                     nullptr);
+    } else {
+        const uint32_t pos = (uint32_t)position;
+        rc = nvmai_hip_sample(ctx, stream, probs, v, 1, v, T, has_k ? (uint32_t)config->top_k : 0u, top_p, &seed, &pos,
+                              out_token);
+    }
+    if (rc) return rc;
+    if (path_taken)
+        *path_taken = penalty ? NVMAI_SAMPLE_PATH_PENALTY : (T == 0.0f ? NVMAI_SAMPLE_PATH_GREEDY : NVMAI_SAMPLE_PATH_SAMPLED);
+    return NVMAI_OK;
 }

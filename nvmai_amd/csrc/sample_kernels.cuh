@@ -472,6 +472,33 @@ __global__ __launch_bounds__(256) void sample_generic_kernel(const uint16_t* pro
     }
 }
 
+// Sampler.applyRepetitionPenaltyInPlace (Sampler.swift:259-293) on the device: one thread per history
+// id.  The reference walks the distinct ids of its history dictionary; here a thread drops out when
+// an earlier entry of the list holds the same id, so a list with repeats gives the same result.
+// Without a softcap the new logit is one IEEE division or product, rounded to the activation type.
+template <int ACT>
+__global__ __launch_bounds__(256) void repetition_penalty_kernel(uint16_t* logits, uint32_t v, const int32_t* ids,
+                                                                 uint32_t n_ids, float penalty, float softcap) {
+    const uint32_t j = blockIdx.x * 256u + threadIdx.x;
+    if (j >= n_ids) return;
+    const int32_t id = ids[j];
+    if (id < 0 || (uint32_t)id >= v) return;
+    for (uint32_t h = 0; h < j; ++h)
+        if (ids[h] == id) return;
+    const float z = act_to_f32<ACT>(logits[id]);
+    float out;
+    if (softcap > 0.0f) {
+        const float capped = softcap * tanhf(z / softcap);
+        const float pen = capped > 0.0f ? capped / penalty : capped * penalty;
+        const float limit = softcap * 0.9999f;
+        const float clamped = fmaxf(fminf(pen, limit), -limit);
+        out = softcap * atanhf(clamped / softcap);
+    } else {
+        out = z > 0.0f ? z / penalty : z * penalty;
+    }
+    logits[id] = f32_to_act<ACT>(out);
+}
+
 // Gumbel-max draw the reference takes when neither top-k nor top-p is set (logit.metal:296-313,
 // 391-429): argmax_i(log(p_i) / T + g_i), g_i = -log(-log(u_i)), u_i from SplitMix64 of
 // (seed, position, i).  Logarithms in double, rounded to float once per step, so that scores

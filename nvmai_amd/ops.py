@@ -7,7 +7,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._lib import ExpertOffsets, KvView, MoeLayer, PrefillGrouping, Rows, check, lib
+from ._lib import ExpertOffsets, GenerationConfig as _CGenerationConfig, KvView, MoeLayer, PrefillGrouping, Rows, check, lib
 
 ACT_BF16, ACT_FP16 = 0, 1
 (PROF_ROUTER, PROF_SELECT, PROF_GROUP, PROF_PHASE1, PROF_PHASE2, PROF_COMBINE, PROF_KV_QUANT,
@@ -587,6 +587,79 @@ class Sample:
                                    top_k, top_p, _seed_array(seed, rows), (C.c_uint32 * rows)(*pos), _ptr(out)),
               "sample")
         return out
+
+
+class GenerationConfig:
+    """GenerationConfig (Sampler.swift:19-81), the fields the sampler reads; top_k / top_p / seed may be
+    None as in the reference (defaults: GenerationDefaults, Sampler.swift:6-11)."""
+
+    def __init__(self, temperature=0.6, top_k=20, top_p=0.95, repetition_penalty=1.0, seed=None):
+        self.temperature, self.top_k, self.top_p = temperature, top_k, top_p
+        self.repetition_penalty, self.seed = repetition_penalty, seed
+
+    def _c(self):
+        c = _CGenerationConfig()
+        c.temperature = self.temperature
+        c.top_k = 0 if self.top_k is None else self.top_k
+        c.top_p = 0.0 if self.top_p is None else self.top_p
+        c.repetition_penalty = self.repetition_penalty
+        c.seed, c.has_seed = (0, 0) if self.seed is None else (self.seed, 1)
+        return c
+
+
+class Sampler:
+    """Mirror of Sampler (Sampler.swift:133-325): logits -> one token id through the repetition
+    penalty, softcap + softmax and the tiled or generic sampler.  The penalty history is kept as the
+    reference keeps it (a table of distinct ids, seeded from the first call's history, then one id
+    per call) and lives on the device as an id list."""
+    PATHS = {0: "greedyGPU", 1: "gpuSampled", 2: "hostPenalty"}
+
+    def __init__(self, ctx, vocab=262144, logit_softcap=30.0, sampler_path="tiled"):
+        if sampler_path not in ("tiled", "generic"):
+            raise ValueError("invalid sampler path %r" % sampler_path)       # GeneratorError.invalidSamplerPath
+        self.ctx, self.vocab, self.logit_softcap = ctx, vocab, logit_softcap
+        self.sampler_path = 0 if sampler_path == "tiled" else 1
+        self.probs = torch.empty(vocab, dtype=torch.float16, device=ctx.device)
+        self.reset_penalty_history()
+
+    def reset_penalty_history(self):
+        self._seen, self._ids, self._seeded = set(), [], False
+        self._ids_dev, self._ids_count = None, 0
+
+    def _fold_history(self, history):
+        new = list(history) if not self._seeded else list(history[-1:])
+        self._seeded = True
+        for i in new:
+            if 0 <= i < self.vocab and i not in self._seen:
+                self._seen.add(i)
+                self._ids.append(i)
+        if self._ids_count != len(self._ids):
+            self._ids_dev = torch.tensor(self._ids, dtype=torch.int32, device=self.ctx.device)
+            self._ids_count = len(self._ids)
+
+    def sample(self, logits, history, config, position, out_token=None):
+        """Sampler.sample (Sampler.swift:171-234); logits: activations [vocab], edited in place by the
+        penalty.  Returns (token tensor, path name)."""
+        if out_token is None:
+            out_token = torch.empty(1, dtype=torch.int32, device=logits.device)
+        penalty = config.repetition_penalty != 1.0 and len(history) > 0
+        if penalty:
+            self._fold_history(history)
+        path = C.c_int(-1)
+        cfg = config._c()
+        check(lib.nvmai_hip_sampler_sample(self.ctx.handle, _stream(), _ptr(logits), _ptr(self.probs), self.vocab,
+                                           _ptr(self._ids_dev) if penalty else None,
+                                           self._ids_count if penalty else 0, C.byref(cfg), position,
+                                           self.logit_softcap, self.sampler_path, _ptr(out_token), C.byref(path)),
+              "sampler_sample")
+        return out_token, self.PATHS[path.value]
+
+
+def repetition_penalty(ctx, logits, history_ids, penalty, logit_softcap=0.0):
+    """Sampler.applyRepetitionPenaltyInPlace (Sampler.swift:259-293) on the device, in place."""
+    check(lib.nvmai_hip_repetition_penalty(ctx.handle, _stream(), _ptr(logits), logits.shape[-1], _ptr(history_ids),
+                                           history_ids.numel(), penalty, logit_softcap), "repetition_penalty")
+    return logits
 
 
 class RMSNorm:

@@ -81,6 +81,11 @@ _sig("orc_sample", C.c_uint32, u16p, size_t, C.c_float, C.c_uint32, C.c_float, C
 _sig("orc_gumbel_for", C.c_float, C.c_uint64, C.c_uint32, C.c_uint32)
 _sig("orc_sample_topk64", C.c_uint32, u16p, size_t, C.c_float, C.c_float, C.c_uint64,
      C.c_uint32, C.c_void_p, C.c_void_p)
+_sig("orc_repetition_penalty", None, f32p, C.c_int, size_t, np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS"),
+     size_t, C.c_float, C.c_float)
+_sig("orc_sampler_route", C.c_int, C.c_int, C.c_float, C.c_int)
+_sig("orc_sampler_sample", C.c_uint32, f32p, size_t, C.c_float, C.c_int, C.c_float, C.c_int, C.c_float,
+     C.c_uint64, C.c_int64, u16p)
 _sig("orc_rel_error", C.c_float, f32p, f32p, size_t)
 _sig("orc_rmsnorm", None, f32p, size_t, C.c_void_p, size_t, size_t, C.c_float, f32p, size_t)
 _sig("orc_elementwise", None, C.c_int, f32p, f32p, size_t, f32p)
@@ -429,6 +434,29 @@ def sample_generic(probs_f16, temperature, top_k, top_p, seed):
 def sample_gumbel(probs_f16, temperature, seed, position=0):
     p = np.ascontiguousarray(probs_f16, np.uint16)
     return lib.orc_sample_gumbel(p, p.size, temperature, seed, position)
+
+
+def repetition_penalty(logits, act, history, penalty, softcap=0.0):
+    """Sampler.applyRepetitionPenaltyInPlace (Sampler.swift:259-293) on a copy of `logits`
+    (16-bit activation values as float32; act 0 = bf16, 1 = fp16)."""
+    out = np.ascontiguousarray(logits, np.float32).copy()
+    ids = np.ascontiguousarray(history, np.int32)
+    lib.orc_repetition_penalty(out, act, out.size, ids, ids.size, penalty, softcap)
+    return out
+
+
+def sampler_route(tiled_path, temperature, top_k):
+    """2 = tiled top-64 sampler, 1 = generic kernel, 0 = generic greedy (Sampler.swift:196-231)."""
+    return lib.orc_sampler_route(int(tiled_path), temperature, 0 if top_k is None else top_k)
+
+
+def sampler_sample(logits, softcap, temperature, top_k, top_p, seed, position, tiled_path=True):
+    """Sampler.sample after the penalty; returns (token, fp16 probability bits)."""
+    lg = np.ascontiguousarray(logits, np.float32)
+    probs = np.empty(lg.size, np.uint16)
+    tok = lib.orc_sampler_sample(lg, lg.size, softcap, int(tiled_path), temperature, 0 if top_k is None else top_k,
+                                 0.0 if top_p is None else top_p, seed, position, probs)
+    return tok, probs
 
 
 def sample(probs_f16, temperature, top_k, top_p, seed, position=0):

@@ -1096,6 +1096,53 @@ uint32_t orc_sample_topk64(const uint16_t *probs_f16, size_t v, float temperatur
     return sample_tail(val, idx, kept, temperature, top_p, seed, idx[0]);
 }
 
+/* Sampler.applyRepetitionPenaltyInPlace (Sampler.swift:259-293): for every DISTINCT id of the
+ * history inside the vocabulary, a positive logit is divided by the penalty and a negative one
+ * multiplied; with a logit softcap the penalty acts on the capped logit and is mapped back through
+ * atanh.  logits are 16-bit activations held as floats; act 0 = bf16, 1 = fp16 (the reference). */
+void orc_repetition_penalty(float *logits, int act, size_t v, const int32_t *ids, size_t n_ids,
+                            float penalty, float softcap) {
+    for (size_t j = 0; j < n_ids; ++j) {
+        int seen = 0;                                          /* once per distinct id */
+        for (size_t h = 0; h < j && !seen; ++h) seen = ids[h] == ids[j];
+        if (seen || ids[j] < 0 || (size_t)ids[j] >= v) continue;
+        const float z = logits[ids[j]];
+        float out;
+        if (softcap > 0.0f) {
+            const float capped = softcap * tanhf(z / softcap);
+            const float pen = capped > 0.0f ? capped / penalty : capped * penalty;
+            const float limit = softcap * 0.9999f;
+            const float clamped = fmaxf(fminf(pen, limit), -limit);
+            out = softcap * atanhf(clamped / softcap);
+        } else {
+            out = z > 0.0f ? z / penalty : z * penalty;
+        }
+        logits[ids[j]] = act == 0 ? orc_bf16_to_float(orc_bf16_bits(out)) : orc_f16_to_float(orc_f16_bits(out));
+    }
+}
+
+/* Sampler.sample's choice of kernel (Sampler.swift:196-231): 2 = the tiled top-64 sampler, 1 = the
+ * generic kernel with its own three paths, 0 = generic greedy.  top_k <= 0 stands for nil. */
+int orc_sampler_route(int tiled_path, float temperature, int top_k) {
+    if (tiled_path && temperature > 0.0f && top_k >= 1 && top_k <= 64) return 2;
+    return temperature == 0.0f ? 0 : 1;
+}
+
+/* Sampler.sample after the penalty: softcap + softmax, then the routed sampler with
+ * seedFor(seed, position); top_p <= 0 stands for nil (1.0).  probs_f16 receives the probabilities. */
+uint32_t orc_sampler_sample(const float *logits, size_t v, float softcap, int tiled_path,
+                            float temperature, int top_k, float top_p, uint64_t seed,
+                            int64_t position, uint16_t *probs_f16) {
+    if (tiled_path) orc_softmax_tiled_f16(logits, v, softcap, probs_f16);
+    else orc_softmax_f16(logits, v, softcap, probs_f16);
+    const uint64_t s = orc_seed_for(seed, position);
+    const float p = top_p > 0.0f ? top_p : 1.0f;
+    if (orc_sampler_route(tiled_path, temperature, top_k) == 2)
+        return orc_sample_topk64(probs_f16, v, temperature, p, s, (uint32_t)top_k, NULL, NULL);
+    return orc_sample(probs_f16, v, temperature == 0.0f ? 0.0f : temperature,
+                      top_k > 0 ? (uint32_t)top_k : 0u, p, s, (uint32_t)position);
+}
+
 float orc_rel_error(const float *actual, const float *reference, size_t n) {
     float max_diff = 0.0f, ref_norm = 0.0f;
     for (size_t i = 0; i < n; ++i) {

@@ -198,6 +198,15 @@ uint32_t orc_sample_topk64(const uint16_t *probs_f16, size_t v, float temperatur
                            float top_p, uint64_t seed, uint32_t top_k,
                            uint32_t *top64_idx, float *top64_val);
 
+/* Sampler.sample's front end (Sampler.swift:171-293): the repetition penalty over the distinct
+ * history ids, the choice between the tiled and the generic sampler, and the whole call. */
+void orc_repetition_penalty(float *logits, int act, size_t v, const int32_t *ids, size_t n_ids,
+                            float penalty, float softcap);
+int orc_sampler_route(int tiled_path, float temperature, int top_k);
+uint32_t orc_sampler_sample(const float *logits, size_t v, float softcap, int tiled_path,
+                            float temperature, int top_k, float top_p, uint64_t seed,
+                            int64_t position, uint16_t *probs_f16);
+
 /* RelError.swift:5-16 */
 /* ---- rest of the decode step ------------------------------------------- */
 void orc_rmsnorm(const float *x, size_t x_stride, const uint16_t *weight_bf16, size_t rows,

@@ -158,3 +158,126 @@ def test_gumbel_max_path_matches_oracle(nv, ctx):
     assert np.array_equal(batch, again)
     z = np.zeros(512, np.uint16)
     assert int(gen.encode(_probs_dev(z), 1.0, 0, 1.0, 1, 0)[0]) == 0   # nothing eligible -> token 0
+
+
+def test_sampler_sample_front_end(nv, ctx):
+    # Sampler.sample (Sampler.swift:171-234): penalty over the history, softcap + softmax, then the
+    # tiled sampler for k in 1...64 at T > 0 and the generic kernel otherwise.  Tokens must equal the
+    # oracle's samplers run on the probabilities the GPU produced; the path names are the reference's.
+    say("Sampler.sample", ctx.act)
+    v = 248320
+    rng = np.random.default_rng(31)
+    base = (rng.standard_normal(v) * 2.5).astype(np.float32)
+    base[[17, 4000, 99999]] += 9.0
+    base = round_act(base, ctx.act)
+    history = [17, 4000, 17, 5, v + 3, -1, 4000]
+    for softcap in (0.0, 30.0):
+        for cfg, path_name, tiled in [
+                (nv.GenerationConfig(seed=1234), "gpuSampled", True),                       # production default
+                (nv.GenerationConfig(top_k=64, top_p=None, seed=9), "gpuSampled", True),
+                (nv.GenerationConfig(top_k=100, top_p=0.9, seed=9), "gpuSampled", False),   # k > 64: generic
+                (nv.GenerationConfig(temperature=0.8, top_k=None, top_p=None, seed=5), "gpuSampled", False),   # Gumbel
+                (nv.GenerationConfig(temperature=0.0, seed=1), "greedyGPU", False),
+                (nv.GenerationConfig(repetition_penalty=1.3, seed=77), "hostPenalty", True),
+                (nv.GenerationConfig(temperature=0.0, repetition_penalty=4.0, seed=1), "hostPenalty", False)]:
+            for which in ("tiled", "generic"):
+                sampler = nv.Sampler(ctx, v, softcap, which)
+                logits = act_tensor(base, ctx)
+                position = 41
+                tok, path = sampler.sample(logits, history, cfg, position)
+                torch.cuda.synchronize()
+                assert path == path_name
+                want_logits = base
+                if cfg.repetition_penalty != 1.0:
+                    want_logits = O.repetition_penalty(base, ctx.act, history, cfg.repetition_penalty, softcap)
+                    got_logits = act_np(logits)
+                    if softcap == 0.0:
+                        assert np.array_equal(got_logits, want_logits)         # one IEEE operation per id
+                    else:
+                        assert np.abs(got_logits - want_logits).max() <= 2 ** -5   # tanh / atanh from two libraries
+                    assert np.array_equal(np.delete(got_logits, [17, 4000, 5]), np.delete(base, [17, 4000, 5]))
+                probs = sampler.probs.cpu().numpy().view(np.uint16)
+                ref = O.f16_to_float(O.softmax_f16(act_np(logits), softcap=softcap, tiled=True))
+                assert np.abs(O.f16_to_float(probs) - ref).max() <= 2e-3 * ref.max() + 1e-7
+                seed = O.seed_for(cfg.seed, position)
+                k = 0 if cfg.top_k is None else cfg.top_k
+                p = 1.0 if cfg.top_p is None else cfg.top_p
+                if which == "tiled" and tiled and cfg.temperature > 0:
+                    want = O.sample_topk64(probs, cfg.temperature, p, seed, top_k=k)
+                else:
+                    want = O.sample(probs, cfg.temperature, k, p, seed, position)
+                assert int(tok[0]) == want, (softcap, which, cfg.__dict__)
+                if cfg.temperature == 0.0 and cfg.repetition_penalty == 4.0 and softcap == 0.0:
+                    assert want not in (17, 4000, 99999) or want == 99999       # the penalized peaks lost
+    # the incremental history of the reference: the first call folds the whole history, later calls
+    # only the last id (Sampler.swift:262-270)
+    sampler = nv.Sampler(ctx, v, 0.0)
+    cfg = nv.GenerationConfig(temperature=0.0, repetition_penalty=2.0, seed=1)
+    logits = act_tensor(base, ctx)
+    sampler.sample(logits, [17], cfg, 0)
+    logits2 = act_tensor(base, ctx)
+    sampler.sample(logits2, [99999, 4000], cfg, 1)          # only 4000 joins the table
+    torch.cuda.synchronize()
+    want = O.repetition_penalty(base, ctx.act, [17, 4000], 2.0)
+    assert np.array_equal(act_np(logits2), want)
+    with pytest.raises(nv.NvmaiError) as e:                 # top-p below one without top-k is not implemented
+        nv.Sampler(ctx, v, 0.0).sample(logits, [], nv.GenerationConfig(top_k=None, top_p=0.5), 0)
+    assert e.value.name == "unsupported"
+    with pytest.raises(nv.NvmaiError):
+        nv.Sampler(ctx, v, 0.0).sample(logits, [], nv.GenerationConfig(top_k=300), 0)
+
+
+def test_sampler_sample_reference_properties(nv, ctx):
+    # The reference's own Sampler tests (tests/NVMAI/Core/Runtime/Generation/SamplerTests.swift:68-197)
+    # through the C ABI, default softcap 30 as there.
+    say("Sampler.sample reference properties", ctx.act)
+
+    def draw(sampler, values, cfg, position=0, history=()):
+        tok, path = sampler.sample(act_tensor(np.asarray(values, np.float32), ctx), list(history), cfg, position)
+        torch.cuda.synchronize()
+        return int(tok[0]), path
+
+    # degenerateDistributionStillReturnsAnInRangeToken (:68-80)
+    s = nv.Sampler(ctx, 64)
+    for fill in (-np.inf, np.nan):
+        for seed in range(1, 9):
+            tok, _ = draw(s, np.full(64, fill, np.float32), nv.GenerationConfig(1.0, 64, 0.95, seed=seed), seed)
+            assert tok < 64
+    # greedy_picksArgmax (:82-91)
+    lg = np.full(2048, 0.1, np.float32)
+    lg[1337] = 9.0
+    assert draw(nv.Sampler(ctx, 2048), lg, nv.GenerationConfig(temperature=0.0)) == (1337, "greedyGPU")
+    # seeded_isDeterministicAtPosition / reproducibleAcrossPositions (:93-121)
+    g = O.seed_tree(0x51A71006, "sampler-position-replay")
+    lg = g.uniform_array(1024, -2.0, 2.0)
+    s = nv.Sampler(ctx, 1024)
+    cfg = nv.GenerationConfig(temperature=1.0, seed=42)
+    run1 = [draw(s, lg, cfg, p)[0] for p in range(5)]
+    run2 = [draw(s, lg, cfg, p)[0] for p in range(5)]
+    assert run1 == run2 and draw(s, lg, cfg, 0)[1] == "gpuSampled"
+    assert [draw(s, lg, nv.GenerationConfig(temperature=1.0, seed=43), p)[0] for p in range(5)] != run1
+    # topK_restrictsToTop (:123-135)
+    lg = np.full(1024, -8.0, np.float32)
+    lg[[10, 200, 500, 900]] = [4.0, 3.0, 2.0, 1.0]
+    for t in range(32):
+        assert draw(s, lg, nv.GenerationConfig(1.0, 4, 0.95, seed=t + 1), t)[0] in (10, 200, 500, 900)
+    # topP_restrictsToNucleus (:137-147)
+    lg = np.full(512, -10.0, np.float32)
+    lg[7], lg[42] = 6.0, 5.6
+    s = nv.Sampler(ctx, 512)
+    for t in range(32):
+        assert draw(s, lg, nv.GenerationConfig(1.0, 20, 0.9, seed=t + 1), t)[0] in (7, 42)
+    # repetitionPenalty_suppressesHistory (:149-169)
+    s = nv.Sampler(ctx, 64)
+    count5 = 0
+    for t in range(200):
+        tok, path = draw(s, np.full(64, 8.0, np.float32), nv.GenerationConfig(1.0, 20, 0.95, 2.0, seed=t + 1), t, [5, 5, 5])
+        assert path == "hostPenalty"
+        count5 += tok == 5
+    assert count5 < 0.5 * 200 / 64
+    # repetitionPenalty_bitesOnSaturatedLogits (:177-197)
+    s = nv.Sampler(ctx, 64)
+    lg = np.full(64, 300.0, np.float32)
+    lg[5] = 400.0
+    count5 = sum(draw(s, lg, nv.GenerationConfig(1.0, 20, 0.95, 1.3, seed=t + 1), t, [5])[0] == 5 for t in range(64))
+    assert count5 < 64 // 8

@@ -160,3 +160,38 @@ def test_gumbel_max_samples_p_to_the_one_over_t():
         top = np.argsort(-w)[:6]
         sigma = np.sqrt(w[top] * (1 - w[top]) / n)
         assert np.all(np.abs(cnt[top] / n - w[top]) <= 5 * sigma + 1e-3)
+
+
+def test_repetition_penalty_and_sampler_policy():
+    # Sampler.applyRepetitionPenaltyInPlace (Sampler.swift:259-293), HF convention: a positive logit
+    # is divided, a negative one multiplied, once per DISTINCT history id, ids outside the
+    # vocabulary ignored.  Exactly representable values pin the arithmetic.
+    lg = np.array([2.0, -2.0, 0.0, 4.0, -1.0, 8.0], np.float32)
+    out = O.repetition_penalty(lg, 1, [0, 1, 1, 2, 0, 99, -3], 1.25)
+    assert list(out) == [1.599609375, -2.5, 0.0, 4.0, -1.0, 8.0]     # 2 / 1.25 = 1.6 -> fp16 1638 / 1024
+    assert np.array_equal(O.repetition_penalty(lg, 0, [3, 5], 2.0), [2.0, -2.0, 0.0, 2.0, -1.0, 4.0])
+    # with a softcap the PENALIZED CAPPED logit is what the downstream softcap reproduces
+    cap, pen = 30.0, 1.1
+    z = np.array([50.0, -50.0, 3.0, 200.0], np.float32)
+    got = O.repetition_penalty(z, 1, [0, 1, 2, 3], pen, cap).astype(np.float64)
+    capped = cap * np.tanh(z.astype(np.float64) / cap)
+    want_capped = np.where(capped > 0, capped / pen, capped * pen)
+    want_capped = np.clip(want_capped, -cap * 0.9999, cap * 0.9999)
+    # fp16 rounding of the stored logit moves the capped value by at most ulp * (1 - tanh^2)
+    assert np.abs(cap * np.tanh(got / cap) - want_capped).max() < 0.05
+    assert np.all(np.isfinite(got))                                 # the clamp keeps atanh finite (:283-286)
+    # path choice (Sampler.swift:196-231): tiled for k in 1...64 at T > 0, generic otherwise
+    assert [O.sampler_route(True, 0.6, k) for k in (1, 20, 64, 65, 256, None)] == [2, 2, 2, 1, 1, 1]
+    assert O.sampler_route(True, 0.0, 20) == 0 and O.sampler_route(False, 0.6, 20) == 1
+    # the whole call equals its parts
+    rng = np.random.default_rng(8)
+    logits = O.round_bf16((rng.standard_normal(5000) * 3).astype(np.float32))
+    tok, probs = O.sampler_sample(logits, 30.0, 0.6, 20, 0.95, 1234, 7)
+    assert np.array_equal(probs, O.softmax_f16(logits, softcap=30.0, tiled=True))
+    assert tok == O.sample_topk64(probs, 0.6, 0.95, O.seed_for(1234, 7), top_k=20)
+    tok, probs = O.sampler_sample(logits, 0.0, 0.0, None, None, 1234, 7)
+    assert tok == int(np.argmax(logits))                            # greedy
+    tok, probs = O.sampler_sample(logits, 0.0, 0.8, None, None, 5, 3)
+    assert tok == O.sample_gumbel(probs, 0.8, O.seed_for(5, 3), 3)  # neither top-k nor top-p: Gumbel-max
+    tok, probs = O.sampler_sample(logits, 0.0, 0.8, 100, 0.9, 5, 3)
+    assert tok == O.sample_generic(probs, 0.8, 100, 0.9, O.seed_for(5, 3))
