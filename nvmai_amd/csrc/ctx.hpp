@@ -10,6 +10,7 @@
 
 struct nvmai_hip_ctx {
     int device;
+    int compute_units;       // of the device (persistent grids are sized from it)
     int act;                 // NVMAI_ACT_BF16 / NVMAI_ACT_FP16
     // Workspace: one device buffer carved by a bump pointer inside each entry
     // point.  Work on one stream is ordered, so consecutive calls may reuse it.

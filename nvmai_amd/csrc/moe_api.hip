@@ -49,6 +49,12 @@ extern "C" int nvmai_hip_ctx_create(int device, int act_dtype, nvmai_hip_ctx** o
     nvmai_hip_ctx* ctx = new (std::nothrow) nvmai_hip_ctx();
     if (!ctx) return NVMAI_ERR_HIP;
     ctx->device = device;
+    ctx->compute_units = 256;
+    {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus > 0)
+            ctx->compute_units = cus;
+    }
     ctx->act = act_dtype;
     ctx->ws = nullptr;
     ctx->ws_cap = 0;

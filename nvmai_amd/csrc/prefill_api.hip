@@ -133,21 +133,32 @@ extern "C" int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream s
 
 namespace {
 
-// Blocks of a launch over at most max_mtiles M tiles: whole units, dealt over eight XCDs.
-uint32_t gemm_grid(uint32_t max_mtiles, const GemmParams& g) {
-    const uint32_t units = max_mtiles * g.units_per_tile;
+// Blocks of a dense launch over `tiles` M tiles: whole units, dealt over eight XCDs.
+uint32_t gemm_grid(uint32_t tiles, const GemmParams& g) {
+    const uint32_t units = tiles * g.units_per_tile;
     return (units + 7) / 8 * 8 * GEMM_UNIT;
 }
 
+// Blocks of a grouped launch.  The work lists are dealt in serpentine order from a sorted sequence of
+// items of at most max(2, ceil(tiles / 64)) M tiles, so no list is longer than an eighth of the
+// tiles plus one item; every column tile of every list position is a block, and blocks past the
+// end of their list leave at once.
+uint32_t grouped_list_max(uint32_t max_mtiles) { return (max_mtiles + 7) / 8 + (max_mtiles + 63) / 64 + 2; }
+uint32_t grouped_grid(uint32_t max_mtiles, const GemmParams& g) {
+    return GEMM_XCDS * grouped_list_max(max_mtiles) * g.n_tiles_n;
+}
+
+// dense: grid over `tiles` M tiles cut by the kernel; grouped: a block per column tile of every list position.
 template <int ACT, int BITS, int NT>
-void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t max_mtiles, nvmai_hip_ctx* ctx, hipStream_t s) {
+void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t tiles, nvmai_hip_ctx* ctx, hipStream_t s) {
+    const bool dense = g1.dense_rows != 0;
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM1, s);
-        prefill_gemm_kernel<ACT, BITS, true, NT><<<gemm_grid(max_mtiles, g1), 256, 0, s>>>(g1);
+        prefill_gemm_kernel<ACT, BITS, true, NT><<<dense ? gemm_grid(tiles, g1) : grouped_grid(tiles, g1), 256, 0, s>>>(g1);
     }
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM2, s);
-        prefill_gemm_kernel<ACT, BITS, false, NT><<<gemm_grid(max_mtiles, g2), 256, 0, s>>>(g2);
+        prefill_gemm_kernel<ACT, BITS, false, NT><<<dense ? gemm_grid(tiles, g2) : grouped_grid(tiles, g2), 256, 0, s>>>(g2);
     }
 }
 
@@ -220,22 +231,24 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
         (uint64_t)d * f * bits / 8 > 0xFFFFFFFFull)
         return NVMAI_ERR_UNSUPPORTED;
     if (n_pairs == 0) return NVMAI_OK;
-    // full tiles + one remainder per expert + the padding of the list's last long and short rows
-    const uint32_t max_mtiles = (uint32_t)(n_pairs / GEMM_BM) + (num_experts < n_pairs ? num_experts : (uint32_t)n_pairs) + 14;
-    rc = ws_begin(ctx, stream, ws_round((size_t)max_mtiles * sizeof(MTile)) + ws_round(64));
+    // full tiles + one remainder per expert: what all eight work lists hold together, and a bound
+    // for each of them
+    const uint32_t max_mtiles = (uint32_t)(n_pairs / GEMM_BM) + (num_experts < n_pairs ? num_experts : (uint32_t)n_pairs);
+    rc = ws_begin(ctx, stream, ws_round((size_t)GEMM_XCDS * max_mtiles * sizeof(MTile)) + ws_round(GEMM_XCDS * 4));
     if (rc) return rc;
-    MTile* mtiles = ws_take<MTile>(ctx, max_mtiles);
-    uint32_t* n_mtiles = ws_take<uint32_t>(ctx, 16);
+    MTile* mtiles = ws_take<MTile>(ctx, (size_t)GEMM_XCDS * max_mtiles);
+    uint32_t* qwords = ws_take<uint32_t>(ctx, GEMM_XCDS);   // list lengths
     hipStream_t s = (hipStream_t)stream;
     prefill_mtiles_kernel<<<1, 256, 0, s>>>(reinterpret_cast<const PrefillGroup*>(grouping->groups), grouping->info,
-                                            mtiles, n_mtiles, reinterpret_cast<uint4*>(route_partials),
+                                            mtiles, max_mtiles, grouped_list_max(max_mtiles), qwords,
+                                            reinterpret_cast<uint4*>(route_partials),
                                             n_pairs * d * 2 / 16);
     const uint32_t nt = bits == 4 ? 4 : 2;        // 16-column tiles per wave: what the register file allows
     GemmParams g1{};
     g1.pool = (const uint8_t*)experts_base; g1.pool_stride = expert_stride;
     g1.wA = off->gate_w; g1.sA = off->gate_s; g1.bA = off->gate_b;
     g1.wB = off->up_w; g1.sB = off->up_s; g1.bB = off->up_b;
-    g1.mtiles = mtiles; g1.n_mtiles = n_mtiles;
+    g1.mtiles = mtiles; g1.list_cap = max_mtiles; g1.list_len = qwords;
     g1.pairs = reinterpret_cast<const PrefillPair*>(grouping->sorted_pairs);
     g1.x = hidden; g1.x_stride = hidden_stride;
     g1.out = act_scratch; g1.out_stride = f;

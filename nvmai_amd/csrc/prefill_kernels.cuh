@@ -413,75 +413,121 @@ constexpr int GEMM_BM = 128;
 
 constexpr uint32_t GEMM_SHORT_ROWS = 32;   // M tiles of at most this many rows take the kernel's short body
 
-// One block: cuts every group into runs of at most GEMM_BM sorted pairs and orders the runs for
-// the GEMM grid.  Long tiles are bound by instruction issue, short ones (a whole expert streamed
-// for a few rows) by memory, so the two kinds are interleaved: both then share every compute
-// unit for the whole launch instead of taking it in turns.  The list is made of rows of eight
-// tiles of one kind, because the grid deals consecutive tiles to the eight XCDs, and a kind's
-// rows are spread evenly among the other's (first row long, last row short); rows are padded
-// with empty tiles.  Long tiles keep their groups' order by size (four coarse classes, largest
-// first) so that the experts with the most tiles start early.
-// n_mtiles <= pairs / GEMM_BM + groups + 14.
+// Work lists of the grouped GEMM: one list of M tiles per XCD.
+//
+// An M tile (at most GEMM_BM sorted pairs of one expert) streams and dequantizes the codes of its
+// expert's matrix; M tiles of one expert that run on one XCD at about the same time find those
+// codes in that XCD's L2 instead of fetching them again.  The GEMM grid is dealt to the XCDs
+// round-robin and XCD x works through list x in order, so the lists are made per expert: the
+// groups are cut into items of at most cap = max(2, ceil(tiles / 64)) consecutive M tiles (an item
+// never spans two experts; the cap keeps one very popular expert from unbalancing the lists), the
+// items are sorted by cost, largest first, and dealt over the eight lists in serpentine order
+// (0..7, 7..0, ...), which keeps the totals of a sorted sequence within one item of each other.
+// Inside a list the most expensive items come first and the short tiles last.
+// No list may be longer than list_max, what the GEMM grid covers; lists that would be, and
+// groupings with more items than the tables below hold, are dealt tile by tile instead.
+//
+// list_len: [GEMM_XCDS] tiles in each list.  mtiles: list x at mtiles + x * list_cap.
+constexpr uint32_t GEMM_XCDS = 8;
+constexpr uint32_t MTILES_MAX_ITEMS = 1280;            // items that are sorted
+
+__device__ __forceinline__ uint32_t mtile_cost(uint32_t rows) {   // in sixteenths of a full tile
+    return rows > 64 ? 16u : rows > GEMM_SHORT_ROWS ? 11u : rows > 16 ? 8u : 7u;
+}
+
 // On a grouping that failed validation (info[2] != 0) no tile is listed, and this block zeroes the
 // caller's route partials instead (slowly: it is the error path), so that the reduce after it
 // returns zeros, never whatever the buffer held.
 __global__ __launch_bounds__(256) void prefill_mtiles_kernel(const PrefillGroup* groups, const uint32_t* info,
-                                                            MTile* mtiles, uint32_t* n_mtiles,
-                                                            uint4* partials_on_error, uint64_t partials_chunks) {
-    __shared__ uint32_t cls_long[4], cur_long[4], n_short, cur_short;
-    if (threadIdx.x < 4) { cls_long[threadIdx.x] = 0; cur_long[threadIdx.x] = 0; }
-    if (threadIdx.x == 0) { n_short = 0; cur_short = 0; }
+                                                            MTile* mtiles, uint32_t list_cap, uint32_t list_max,
+                                                            uint32_t* list_len, uint4* partials_on_error,
+                                                            uint64_t partials_chunks) {
+    __shared__ uint32_t it_group[MTILES_MAX_ITEMS], it_first[MTILES_MAX_ITEMS];
+    __shared__ __attribute__((aligned(16))) uint32_t it_key[MTILES_MAX_ITEMS];   // all different: the item index is part of the key
+    __shared__ uint32_t it_at[MTILES_MAX_ITEMS];        // M tiles of the item, then: list << 24 | offset in the list
+    __shared__ uint32_t by_rank[MTILES_MAX_ITEMS];
+    __shared__ uint32_t total_tiles, n_extra, too_long;
+    const uint32_t tid = threadIdx.x;
+    if (tid == 0) { total_tiles = 0; n_extra = 0; too_long = 0; }
     __syncthreads();
     const uint32_t ng = info[2] ? 0u : info[0];               // nothing runs on a grouping that failed
     if (info[2] && partials_on_error)
-        for (uint64_t i = threadIdx.x; i < partials_chunks; i += 256) partials_on_error[i] = uint4{0, 0, 0, 0};
-    // a group's tiles: t - 1 full ones and a last one of `last` rows; its class by t
-    auto shape = [](const PrefillGroup& gr, uint32_t& t, uint32_t& last, uint32_t& nl, int& cls) {
-        t = (gr.pair_count + GEMM_BM - 1) / GEMM_BM;
-        last = gr.pair_count - (t - 1) * GEMM_BM;
-        nl = t - 1 + (last > GEMM_SHORT_ROWS ? 1u : 0u);
-        cls = t >= 16 ? 3 : t >= 4 ? 2 : t >= 2 ? 1 : 0;
+        for (uint64_t i = tid; i < partials_chunks; i += 256) partials_on_error[i] = uint4{0, 0, 0, 0};
+    for (uint32_t g = tid; g < ng; g += 256) atomicAdd(&total_tiles, (groups[g].pair_count + GEMM_BM - 1) / GEMM_BM);
+    __syncthreads();
+    const uint32_t cap_tiles = max(2u, (total_tiles + 63u) / 64u);
+    // tile by tile in group order: list lengths differ by at most one
+    auto deal_tiles = [&]() {
+        if (tid == 0) {
+            uint32_t n = 0;
+            for (uint32_t g = 0; g < ng; ++g) {
+                const PrefillGroup gr = groups[g];
+                for (uint32_t r = 0; r < gr.pair_count; r += GEMM_BM, ++n)
+                    mtiles[(size_t)(n % GEMM_XCDS) * list_cap + n / GEMM_XCDS] =
+                        MTile{gr.expert, gr.pair_start + r, gr.pair_count - r < (uint32_t)GEMM_BM ? gr.pair_count - r : (uint32_t)GEMM_BM};
+            }
+            for (uint32_t x = 0; x < GEMM_XCDS; ++x) list_len[x] = n / GEMM_XCDS + (x < n % GEMM_XCDS ? 1u : 0u);
+        }
     };
-    // the first 256 groups (usually all of them) are read once and stay in registers
-    PrefillGroup first_gr{0, 0, 0};
-    if (threadIdx.x < ng) first_gr = groups[threadIdx.x];
-    for (uint32_t g = threadIdx.x; g < ng; g += 256) {
-        const PrefillGroup gr = g < 256 ? first_gr : groups[g];
-        uint32_t t, last, nl; int cls;
-        shape(gr, t, last, nl, cls);
-        if (nl) atomicAdd(&cls_long[cls], nl);
-        if (nl != t) atomicAdd(&n_short, 1u);
+    if (ng + 68u > MTILES_MAX_ITEMS) { deal_tiles(); return; }
+    // items: the first of a group at the group's index, further ones behind the groups
+    auto item_key = [&](const PrefillGroup& gr, uint32_t first, uint32_t item) {
+        const uint32_t t = (gr.pair_count + GEMM_BM - 1) / GEMM_BM;
+        const uint32_t n = min(cap_tiles, t - first);
+        const uint32_t cost = (n - 1) * 16u + mtile_cost(first + n == t ? gr.pair_count - (t - 1) * GEMM_BM : (uint32_t)GEMM_BM);
+        return (cost << 12) | (0xFFFu - (item & 0xFFFu));     // larger cost first, then lower index
+    };
+    for (uint32_t g = tid; g < ng; g += 256) {
+        const PrefillGroup gr = groups[g];
+        const uint32_t t = (gr.pair_count + GEMM_BM - 1) / GEMM_BM;
+        it_group[g] = g; it_first[g] = 0; it_key[g] = item_key(gr, 0, g); it_at[g] = min(cap_tiles, t);
+        for (uint32_t first = cap_tiles; first < t; first += cap_tiles) {
+            const uint32_t i = ng + atomicAdd(&n_extra, 1u);  // at most 64 of them: total_tiles / cap_tiles
+            it_group[i] = g; it_first[i] = first; it_key[i] = item_key(gr, first, i); it_at[i] = min(cap_tiles, t - first);
+        }
     }
     __syncthreads();
-    const uint32_t base3 = 0, base2 = cls_long[3], base1 = base2 + cls_long[2], base0 = base1 + cls_long[1];
-    const uint32_t L = base0 + cls_long[0], S = n_short;
-    const uint32_t lr = (L + 7) / 8, sr = (S + 7) / 8, rows = lr + sr;
-    // position of the i-th long / short tile: row a of lr long rows sits at floor(a * rows / lr),
-    // row b of sr short rows at ceil((b + 1) * rows / sr) - 1; the two sets partition 0..rows-1
-    const bool small = rows <= 0xFFFFu;                           // 32-bit products suffice
-    auto long_at = [&](uint32_t i) {
-        const uint32_t a = i / 8;
-        return (small ? a * rows / lr : (uint32_t)((uint64_t)a * rows / lr)) * 8 + i % 8;
-    };
-    auto short_at = [&](uint32_t j) {
-        const uint32_t b1 = j / 8 + 1;
-        return (small ? (b1 * rows + sr - 1) / sr - 1 : (uint32_t)(((uint64_t)b1 * rows + sr - 1) / sr - 1)) * 8 + j % 8;
-    };
-    for (uint32_t i = L + threadIdx.x; i < lr * 8; i += 256) mtiles[long_at(i)] = MTile{0, 0, 0};
-    for (uint32_t j = S + threadIdx.x; j < sr * 8; j += 256) mtiles[short_at(j)] = MTile{0, 0, 0};
-    for (uint32_t g = threadIdx.x; g < ng; g += 256) {
-        const PrefillGroup gr = g < 256 ? first_gr : groups[g];
-        uint32_t t, last, nl; int cls;
-        shape(gr, t, last, nl, cls);
-        if (nl) {
-            const uint32_t at = (cls == 3 ? base3 : cls == 2 ? base2 : cls == 1 ? base1 : base0) + atomicAdd(&cur_long[cls], nl);
-            for (uint32_t j = 0; j < nl; ++j)
-                mtiles[long_at(at + j)] = MTile{gr.expert, gr.pair_start + j * GEMM_BM, min((uint32_t)GEMM_BM, gr.pair_count - j * GEMM_BM)};
+    const uint32_t n_items = ng + n_extra;
+    if (tid < 4 && n_items + tid < MTILES_MAX_ITEMS) it_key[n_items + tid] = 0;   // pads the last group of four
+    __syncthreads();
+    for (uint32_t i = tid; i < n_items; i += 256) {           // rank = keys above this one, four keys per read
+        const uint32_t k = it_key[i];
+        uint32_t r = 0;
+        for (uint32_t j = 0; j < n_items; j += 4) {
+            const uint4 o = *reinterpret_cast<const uint4*>(&it_key[j]);
+            r += (o.x > k ? 1u : 0u) + (o.y > k ? 1u : 0u) + (o.z > k ? 1u : 0u) + (o.w > k ? 1u : 0u);
         }
-        if (nl != t)
-            mtiles[short_at(atomicAdd(&cur_short, 1u))] = MTile{gr.expert, gr.pair_start + (t - 1) * GEMM_BM, last};
+        by_rank[r] = i;
     }
-    if (threadIdx.x == 0) *n_mtiles = rows * 8;
+    __syncthreads();
+    // serpentine deal: rank r -> row r / 8, list r % 8 on even rows, 7 - r % 8 on odd ones; one
+    // thread per list walks its items in rank order and hands out the offsets (a chain of
+    // dependent reads: everything it touches is in LDS)
+    if (tid < GEMM_XCDS) {
+        uint32_t at = 0;
+        for (uint32_t row = 0; row * GEMM_XCDS < n_items; ++row) {
+            const uint32_t r = row * GEMM_XCDS + ((row & 1u) ? GEMM_XCDS - 1u - tid : tid);
+            if (r >= n_items) continue;
+            const uint32_t i = by_rank[r];
+            const uint32_t n = it_at[i];
+            it_at[i] = (tid << 24) | at;
+            at += n;
+        }
+        list_len[tid] = at;
+        if (at > list_max) too_long = 1;
+    }
+    __syncthreads();
+    if (too_long) { deal_tiles(); return; }                   // not reached for a sorted sequence; kept as the guarantee
+    for (uint32_t i = tid; i < n_items; i += 256) {
+        const PrefillGroup gr = groups[it_group[i]];
+        const uint32_t t = (gr.pair_count + GEMM_BM - 1) / GEMM_BM;
+        const uint32_t n = min(cap_tiles, t - it_first[i]);
+        MTile* dst = mtiles + (size_t)(it_at[i] >> 24) * list_cap + (it_at[i] & 0xFFFFFFu);
+        for (uint32_t j = 0; j < n; ++j) {
+            const uint32_t r0 = (it_first[i] + j) * GEMM_BM;
+            dst[j] = MTile{gr.expert, gr.pair_start + r0, min((uint32_t)GEMM_BM, gr.pair_count - r0)};
+        }
+    }
 }
 
 // ---- grouped GEMM ---------------------------------------------------------------------------
@@ -509,8 +555,9 @@ struct GemmParams {
     const uint8_t* pool;
     uint64_t pool_stride;
     int64_t wA, sA, bA, wB, sB, bB;     // A: gate or down; B: up
-    const MTile* mtiles;
-    const uint32_t* n_mtiles;
+    const MTile* mtiles;                // grouped product: list x of M tiles at mtiles + x * list_cap
+    uint32_t list_cap;
+    const uint32_t* list_len;           // [GEMM_XCDS] tiles in each list
     const PrefillPair* pairs;           // sorted
     const void* x;                      // DUAL: hidden rows by token; else act rows by sorted position
     uint32_t x_stride;
@@ -629,23 +676,29 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     // then fold every read of them away: a store that never executes keeps them alive (the
     // entry points reject K = 0).
     if (p.K == 0) { xs1[threadIdx.x] = 0; ws[threadIdx.x] = 0; }
-    // Blocks are dealt to the eight XCDs round-robin.  A unit = up to GEMM_UNIT consecutive column
-    // tiles of one M tile; its blocks run back to back on one XCD, so that the tile's activation
-    // rows are fetched into that L2 once, and the units (M tiles sorted by size, then columns)
-    // are dealt over the XCDs in turn, which balances them whether there are many M tiles (the
-    // grouped product) or one (a dense product with few rows).
+    // Blocks are dealt to the eight XCDs round-robin: block b runs on XCD b % 8, and an XCD takes
+    // its blocks in the order of their indices.
+    // Dense product: a unit = up to GEMM_UNIT consecutive column tiles of one M tile; its blocks
+    // run back to back on one XCD, so that the tile's activation rows are fetched into that L2
+    // once, and the units are dealt over the XCDs in turn, which balances them whether there are
+    // many M tiles or one (few rows, many columns).
+    // Grouped product: XCD x works through list x of the M tiles, every column tile of an M tile in
+    // turn.  The column tiles of an M tile share its activation rows and the M tiles of an expert
+    // (neighbours in a list) share its codes: both meet in that XCD's L2.
     const uint32_t on_xcd = blockIdx.x >> 3;
-    const uint32_t unit = (on_xcd / GEMM_UNIT) * 8 + (blockIdx.x & 7u);
-    const uint32_t tile_id = unit / p.units_per_tile;
-    const uint32_t nt = (unit % p.units_per_tile) * GEMM_UNIT + on_xcd % GEMM_UNIT;
     MTile mt;
+    uint32_t nt;
     if (p.dense_rows) {
+        const uint32_t unit = (on_xcd / GEMM_UNIT) * 8 + (blockIdx.x & 7u);
+        const uint32_t tile_id = unit / p.units_per_tile;
+        nt = (unit % p.units_per_tile) * GEMM_UNIT + on_xcd % GEMM_UNIT;
         if (tile_id * GEMM_BM >= p.dense_rows || nt >= p.n_tiles_n) return;
         mt = MTile{0u, tile_id * GEMM_BM, min((uint32_t)GEMM_BM, p.dense_rows - tile_id * GEMM_BM)};
     } else {
-        if (tile_id >= *p.n_mtiles || nt >= p.n_tiles_n) return;
-        mt = p.mtiles[tile_id];
-        if (mt.rows == 0) return;                       // padding of the tile list
+        const uint32_t list = blockIdx.x & (GEMM_XCDS - 1u), at = on_xcd / p.n_tiles_n;
+        nt = on_xcd % p.n_tiles_n;
+        if (at >= p.list_len[list]) return;
+        mt = p.mtiles[(size_t)list * p.list_cap + at];
     }
     const uint8_t* blob = p.pool + (uint64_t)mt.expert * p.pool_stride;
     const int tid = threadIdx.x, lane = tid & 63;
