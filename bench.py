@@ -34,6 +34,8 @@ def parse():
     ap.add_argument("--layers", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--sweep", action="store_true", help="also print batch/bits sweep lines to stderr")
+    ap.add_argument("--no-extra", action="store_true", help="skip the `extra` object (the other cells of the metric) "
+                    "that the default invocation appends")
     ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "sampler", "greedy", "copy"],
                     help="decode = configs[1] (the headline line); prefill = configs[2] grouped GEMM; "
                          "attention = configs[3] quantized-KV decode attention; sampler = the end of configs[4]: "
@@ -123,8 +125,11 @@ def run_config(nv, ctx, torch, layers, stride, bits, batch, steps, warmup, profi
 
 
 def cpu_baseline(layers, stride, bits, batch, torch):
-    """The CPU oracle (a scalar C port of the reference's CPU path) on a bounded sample: the
-    first tokens of one step of layer 0, one thread."""
+    """The CPU oracle (a C port of the reference's CPU path, rebuilt here at -O3 -march=native) on a
+    bounded sample of the same workload: one decode step of layer 0, timed inside the C library
+    (median of the repetitions), on one thread over the first 8 tokens and on all host cores over
+    the whole batch (tokens shared out over the threads: the reference kernel has no threads of
+    its own)."""
     import oracle as O
     L = layers[0]
     pool = L["pool"].cpu().numpy()
@@ -132,37 +137,43 @@ def cpu_baseline(layers, stride, bits, batch, torch):
     gq = [t.cpu().numpy() for t in L["gate"]]
     gate = (8, gq[0], gq[1].view(np.uint16), gq[2].view(np.uint16))
     rng = np.random.default_rng(7)
-    n = min(batch, 8)
-    x = O.round_bf16(rng.standard_normal((n, D)).astype(np.float32))
-    t0 = time.perf_counter()
-    reps = 0
-    while True:
-        idx, _, _ = O.moe_layer_forward(x, D, F, K, bits, (16, router, None, None), pool[:E], pool[E], gate)
-        reps += 1
-        if time.perf_counter() - t0 > 10.0 or reps >= 20:
-            break
-    dt = (time.perf_counter() - t0) / reps
-    # the scalar port evaluates every (token, slot) pair separately: its bytes are per pair
-    bytes_ = n * (K + 1) * stride + n * (E * D * 2) + n * D * 8
-    algo = step_bytes(len(np.unique(idx)), n, stride)
-    return dict(value=algo / dt / 1e9, unit="GB/s", cores=1, kind="port",
-                sample="oracle moe_layer_forward, %d tokens of one %d-bit layer, %d reps, %.2f s each; "
-                       "%.1f MB algorithmic (%.1f MB touched by the scalar path)"
-                       % (n, bits, reps, dt, algo / 1e6, bytes_ / 1e6))
+    model, cores = O.host_cpu()
+    _, flags = O.timing_lib()
+    x = O.round_bf16(rng.standard_normal((max(batch, cores), D)).astype(np.float32))
+    rows = {}
+    for name, n, threads, reps in (("one_thread", min(batch, 8), 1, 21), ("all_cores", max(batch, cores), cores, 41)):
+        dt, idx = O.time_moe_layer(x[:n], D, F, K, bits, (16, router, None, None), pool[:E], pool[E], gate,
+                                   threads, warmup=1, reps=reps)
+        algo = step_bytes(len(np.unique(idx)), n, stride)
+        rows[name] = dict(value=round(algo / dt / 1e9, 3), unit="GB/s", cores=threads,
+                          sample="%d tokens of one %d-bit layer, median of %d repetitions of %.3f s; %.1f MB "
+                                 "algorithmic (each distinct expert once), %.1f MB touched by the per-pair path"
+                                 % (n, bits, reps, dt, algo / 1e6, (n * (K + 1) * stride + n * E * D * 2) / 1e6))
+    out = dict(rows["all_cores"])
+    out.update(kind="port", cpu_model=model, build="oracle/nvmai_oracle.c, gcc " + flags,
+               one_thread=rows["one_thread"])
+    out["sample"] = "oracle orc_moe_layer_forward, " + out["sample"]
+    return out
 
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
-# HBM bytes per launch of the roofline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this file (KiB per dispatch, FETCH_SIZE scaled x2.00 and WRITE_SIZE x1.00 after calibration on
-# `--workload copy`); the summaries live under profiles/.  Keyed by (workload, bits, batch or
-# tokens); other configurations report null.
+# HBM bytes per launch of the roofline kernel: RECORDED figures from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of this file (KiB per dispatch, FETCH_SIZE scaled x2.00 and WRITE_SIZE x1.00 after
+# calibration on `--workload copy`), not something this run measures; each comes with the summary
+# under profiles/ it was read from and goes stale when its kernel changes.  Keyed by (workload,
+# bits, batch or tokens); other configurations report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("decode", 8, 32): (181300 * 2.00 + 1196 * 1.00) * 1024,
-    ("prefill", 4, 4096): (377200 * 2.00 + 36140 * 1.00) * 1024,
-    ("attention", 8, 8, 131072): (599800 * 2.00 + 4383 * 1.00) * 1024,
-    ("attention", 4, 8, 131072): (295900 * 2.00 + 4356 * 1.00) * 1024,
+    ("decode", 8, 32): ((181300 * 2.00 + 1196 * 1.00) * 1024, "profiles/expert_rows_fast_decode_configs1_8bit_batch32.txt"),
+    ("prefill", 4, 4096): ((279700 * 2.00 + 36140 * 1.00) * 1024, "profiles/prefill_gemm_kernel_configs2_4bit_4096tokens.txt"),
+    ("attention", 8, 8, 131072): ((599800 * 2.00 + 4383 * 1.00) * 1024, "profiles/attn_partial_mfma_kernel_configs3_8bit_128k_batch8.txt"),
+    ("attention", 4, 8, 131072): ((295900 * 2.00 + 4356 * 1.00) * 1024, "profiles/attn_partial_mfma_kernel_configs3_8bit_128k_batch8.txt"),
 }
+
+
+def recorded_traffic(key):
+    """(bytes or None, source or None) for a roofline object."""
+    return MEASURED_TRAFFIC_BYTES.get(key, (None, None))
 
 
 def run_prefill(nv, ctx, torch, a):
@@ -244,22 +255,21 @@ def run_prefill(nv, ctx, torch, a):
     cpu = None
     if not a.no_cpu:
         import oracle as O
-        n = 4                                           # tokens of the same step on the CPU oracle
+        model, cores = O.host_cpu()
+        _, flags = O.timing_lib()
         blobs = pool.cpu().numpy()
-        x0 = xs[0, :n].float().cpu().numpy()
-        i0 = idx[0, :n].cpu().numpy().astype(np.uint32)
-        w0 = w[0, :n].view(torch.int16).cpu().numpy().view(np.uint16)
-        t0 = time.perf_counter()
-        reps = 0
-        while True:
-            O.prefill_moe(blobs, bits, x0, D, F, i0, w0)
-            reps += 1
-            if time.perf_counter() - t0 > 10.0 or reps >= 20:
-                break
-        dtc = (time.perf_counter() - t0) / reps
-        cpu = dict(value=n * K * 6.0 * D * F / dtc / 1e12, unit="TFLOP/s", cores=1, kind="port",
-                   sample="oracle prefill_moe, %d tokens x top-%d of the same step, %d reps, %.3f s each"
-                          % (n, K, reps, dtc))
+        rows = {}
+        for name, n, threads, reps in (("one_thread", 4, 1, 5), ("all_cores", 4 * cores, cores, 5)):
+            x0 = xs[0, :n].float().cpu().numpy()     # the first tokens of the same step on the CPU oracle
+            i0 = idx[0, :n].cpu().numpy().astype(np.uint32)
+            w0 = w[0, :n].view(torch.int16).cpu().numpy().view(np.uint16)
+            dtc = O.time_prefill_moe(blobs, bits, x0, D, F, i0, w0, threads, warmup=1, reps=reps)
+            rows[name] = dict(value=n * K * 6.0 * D * F / dtc / 1e12, unit="TFLOP/s", cores=threads,
+                              sample="%d tokens x top-%d of the same step, median of %d repetitions of %.3f s"
+                                     % (n, K, reps, dtc))
+        cpu = dict(rows["all_cores"])
+        cpu.update(kind="port", cpu_model=model, build="oracle/nvmai_oracle.c, gcc " + flags, one_thread=rows["one_thread"])
+        cpu["sample"] = "oracle orc_prefill_moe, " + cpu["sample"]
     return {
         "metric": METRIC, "value": round(flops / dt / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
@@ -274,7 +284,8 @@ def run_prefill(nv, ctx, torch, a):
         "roofline": {"kernel": "prefill_gemm_kernel<DUAL> (gate/up + SwiGLU)", "bound": "mfma",
                      "achieved": round(g1, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(g1 / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(("prefill", bits, T)),
+                     "traffic": recorded_traffic(("prefill", bits, T))[0],
+                     "traffic_source": recorded_traffic(("prefill", bits, T))[1],
                      "flops_per_launch": T * K * 4.0 * D * F, "avg_launch_us": round(kern["gemm_gate_up"], 2)},
         "cpu_baseline": cpu,
     }
@@ -329,23 +340,38 @@ def run_attention(nv, ctx, torch, a):
     kern["kv_quantize_%d_tokens" % nq] = ms / max(n, 1) * 1e3
     stride = caches[0][0].stride
     cpu = None
-    if not a.no_cpu:
+    parity = None
+    if True:
         import oracle as O
-        n = min(ctx_len, 8192)                          # first rows of sequence 0 on the CPU oracle
-        kr = caches[0][0].rows[0, :n].cpu().numpy()
-        vr = caches[0][1].rows[0, :n].cpu().numpy()
-        q0 = q[0].float().cpu().numpy()
-        t0 = time.perf_counter()
-        reps = 0
-        while True:
-            O.attention_decode(q0, kr, vr, bits, HQ, HKV, HD, n, 1.0 / 16.0)
-            reps += 1
-            if time.perf_counter() - t0 > 10.0 or reps >= 20:
-                break
-        dtc = (time.perf_counter() - t0) / reps
-        cpu = dict(value=2.0 * n * stride / dtc / 1e9, unit="GB/s", cores=1, kind="port",
-                   sample="oracle attention_decode, one sequence, %d cached tokens, %d reps, %.3f s each"
-                          % (n, reps, dtc))
+        # the numbers above are only worth printing if the kernel is right at this size: the last
+        # 4096 positions of sequence 0 (a start offset deep in the cache) against the oracle
+        start = max(0, ctx_len - 4096)
+        got = att.encode_full(q[:1], caches[0][0], caches[0][1], HD, HQ, HKV, ctx_len, kv_start=start)
+        torch.cuda.synchronize()
+        kr = caches[0][0].rows[0].cpu().numpy()
+        vr = caches[0][1].rows[0].cpu().numpy()
+        want = O.attention_decode(q[0].float().cpu().numpy(), kr, vr, bits, HQ, HKV, HD, ctx_len, 1.0 / 16.0, start)
+        rel = float(O.rel_error(got[0].float().cpu().numpy(), want))
+        assert rel < 1e-2, "attention differs from the oracle at context %d: max-rel %g" % (ctx_len, rel)
+        parity = {"max_rel": round(rel, 6), "against": "oracle attention_decode, sequence 0, positions %d..%d" % (start, ctx_len)}
+    if not a.no_cpu:
+        model, cores = O.host_cpu()
+        _, flags = O.timing_lib()
+        n = min(ctx_len, 8192)                          # first rows of the sequences on the CPU oracle
+        nb = max(1, min(B, cores))
+        krs = np.stack([caches[0][0].rows[b, :n].cpu().numpy() for b in range(nb)])
+        vrs = np.stack([caches[0][1].rows[b, :n].cpu().numpy() for b in range(nb)])
+        qs = q[:nb].float().cpu().numpy()
+        rows = {}
+        for name, seqs, threads in (("one_thread", 1, 1), ("all_cores", nb, nb)):
+            dtc = O.time_attention(qs[:seqs], krs[:seqs], vrs[:seqs], bits, HQ, HKV, HD, n, 1.0 / 16.0, threads,
+                                   warmup=1, reps=5)
+            rows[name] = dict(value=2.0 * seqs * n * stride / dtc / 1e9, unit="GB/s", cores=threads,
+                              sample="%d sequence(s) of %d cached tokens, one thread per sequence, median of 5 "
+                                     "repetitions of %.3f s" % (seqs, n, dtc))
+        cpu = dict(rows["all_cores"])
+        cpu.update(kind="port", cpu_model=model, build="oracle/nvmai_oracle.c, gcc " + flags, one_thread=rows["one_thread"])
+        cpu["sample"] = "oracle orc_attention_decode, " + cpu["sample"]
     kv_bytes = 2.0 * B * ctx_len * stride
     step_b = kv_bytes + 2 * B * HQ * HD * 2
     part = kv_bytes / (kern["partial"] * 1e-6) / 1e9
@@ -361,9 +387,10 @@ def run_attention(nv, ctx, torch, a):
                    "kernel_us": {k: round(v, 2) for k, v in kern.items()}},
         "roofline": {"kernel": "attn_partial_mfma_kernel", "bound": "hbm", "achieved": round(part, 2),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(part / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(("attention", bits, B, ctx_len)),
+                     "traffic": recorded_traffic(("attention", bits, B, ctx_len))[0],
+                     "traffic_source": recorded_traffic(("attention", bits, B, ctx_len))[1],
                      "bytes_per_launch": kv_bytes, "avg_launch_us": round(kern["partial"], 2)},
-        "cpu_baseline": cpu,
+        "cpu_baseline": cpu, "parity_check": parity,
     }
 
 
@@ -584,25 +611,7 @@ def main():
     layers, stride = build_layers(nv, ctx, torch, a.bits, a.layers)
     torch.cuda.synchronize()
     r = run_config(nv, ctx, torch, layers, stride, a.bits, a.batch, a.steps, a.warmup, profile=True)
-    line = {
-        "metric": METRIC, "value": round(r["gbps"], 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps,
-        "warmup": a.warmup, "ms_per_step": round(r["ms_per_step"], 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "u%d codes, f32 accumulate" % a.bits,
-        "data": "synthetic",
-        "config": {"workload": "configs[1]: one MoE-layer decode step, %d-bit group-64 experts, hidden 2048, "
-                               "256 experts top-8 + gated shared expert, intermediate 512, bf16 activations, "
-                               "all experts resident in HBM" % a.bits,
-                   "batch_tokens": a.batch, "layers_rotated": a.layers,
-                   "mean_distinct_experts": round(r["mean_distinct"], 2),
-                   "frac_of_hbm_peak": round(r["gbps"] / HBM_PEAK_GBPS, 4),
-                   "kernel_us": {k: round(v, 2) for k, v in r["kernel_us"].items()}},
-        "roofline": {"kernel": "expert_rows_fast (routed + shared gate/up SwiGLU, phase 1)", "bound": "hbm",
-                     "achieved": round(r["phase1_gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(r["phase1_gbps"] / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(("decode", a.bits, a.batch)),
-                     "bytes_per_launch": round(r["phase1_bytes"]),
-                     "avg_launch_us": round(r["kernel_us"]["phase1"], 2)},
-    }
+    line = decode_line(a, r, a.bits, a.batch, a.steps, a.warmup)
     if a.sweep:
         for bits in (8, 4):
             ls, st = (layers, stride) if bits == a.bits else build_layers(nv, ctx, torch, bits, a.layers)
@@ -619,7 +628,74 @@ def main():
         line["cpu_baseline"] = cpu_baseline(layers, stride, a.bits, a.batch, torch)
     else:
         line["cpu_baseline"] = None
+    if not a.no_extra and a.bits == 8 and a.batch == 32:
+        line["extra"] = extra_cells(nv, ctx, torch, a, layers, stride)
     print(json.dumps(line), flush=True)
+
+
+def compact(line):
+    """The figures of a full line that the `extra` object keeps."""
+    r = line["roofline"]
+    out = {"workload": line["config"]["workload"], "value": line["value"], "unit": line["unit"],
+           "ms_per_step": line["ms_per_step"],
+           "roofline": {k: r[k] for k in ("kernel", "bound", "achieved", "peak", "unit", "frac", "avg_launch_us")}}
+    for k in ("batch_tokens", "mean_distinct_experts", "tokens_per_s", "frac_of_hbm_peak"):
+        if k in line["config"]:
+            out[k] = line["config"][k]
+    if line.get("parity_check"):
+        out["parity_check"] = line["parity_check"]
+    return out
+
+
+def decode_line(a, r, bits, batch, steps, warmup):
+    return {
+        "metric": METRIC, "value": round(r["gbps"], 2), "unit": "GB/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": round(r["ms_per_step"], 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u%d codes, f32 accumulate" % bits, "data": "synthetic",
+        "config": {"workload": "configs[1]: one MoE-layer decode step, %d-bit group-64 experts, hidden 2048, "
+                               "256 experts top-8 + gated shared expert, intermediate 512, bf16 activations, "
+                               "all experts resident in HBM" % bits,
+                   "batch_tokens": batch, "layers_rotated": a.layers,
+                   "mean_distinct_experts": round(r["mean_distinct"], 2),
+                   "frac_of_hbm_peak": round(r["gbps"] / HBM_PEAK_GBPS, 4),
+                   "kernel_us": {k: round(v, 2) for k, v in r["kernel_us"].items()}},
+        "roofline": {"kernel": "expert_rows_fast (routed + shared gate/up SwiGLU, phase 1)" if batch > 4 else
+                               "expert_rows_routed / expert_rows_fast (gate/up SwiGLU, phase 1)", "bound": "hbm",
+                     "achieved": round(r["phase1_gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(r["phase1_gbps"] / HBM_PEAK_GBPS, 4),
+                     "traffic": recorded_traffic(("decode", bits, batch))[0],
+                     "traffic_source": recorded_traffic(("decode", bits, batch))[1],
+                     "bytes_per_launch": round(r["phase1_bytes"]),
+                     "avg_launch_us": round(r["kernel_us"]["phase1"], 2)},
+    }
+
+
+def extra_cells(nv, ctx, torch, a, layers8, stride8):
+    """The other cells of the metric, each measured like its own --workload line but shorter:
+    4-bit decode at batch 32, 8-bit decode at one token, the configs[2] prefill grouped GEMM, and
+    configs[3] attention at 128K x 8 and 32K x 1 with 8- and 4-bit KV (each checked against the
+    oracle before it is reported)."""
+    import argparse
+    out = {}
+    r = run_config(nv, ctx, torch, layers8, stride8, 8, 1, 200, 20, profile=True)
+    out["decode_8bit_batch1"] = compact(decode_line(a, r, 8, 1, 200, 20))
+    layers4, stride4 = build_layers(nv, ctx, torch, 4, a.layers)
+    torch.cuda.synchronize()
+    r = run_config(nv, ctx, torch, layers4, stride4, 4, 32, 200, 20, profile=True)
+    out["decode_4bit_batch32"] = compact(decode_line(a, r, 4, 32, 200, 20))
+    del layers4
+    torch.cuda.empty_cache()
+    sub = argparse.Namespace(**vars(a))
+    sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.tokens = True, 30, 5, 4, 4096
+    out["prefill_4bit_4096tokens"] = compact(run_prefill(nv, ctx, torch, sub))
+    torch.cuda.empty_cache()
+    for bits in (8, 4):
+        for context, batch in ((131072, 8), (32768, 1)):
+            sub = argparse.Namespace(**vars(a))
+            sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.context, sub.batch = True, 30, 5, bits, context, batch
+            out["attention_%dbit_%dk_batch%d" % (bits, context // 1024, batch)] = compact(run_attention(nv, ctx, torch, sub))
+            torch.cuda.empty_cache()
+    return out
 
 
 if __name__ == "__main__":

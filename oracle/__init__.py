@@ -27,6 +27,20 @@ def _load():
 
 lib = _load()
 
+
+def build_native(path):
+    """The same two C files at -O3 -march=native (still -ffp-contract=off, no fast-math: the same
+    results, only faster) for the timed cpu_baseline legs of bench.py; compiled where it runs,
+    because a binary made for another CPU's instruction set may not.  Returns a CDLL, or None
+    when there is no compiler."""
+    cmd = ["gcc", "-O3", "-march=native", "-std=c11", "-ffp-contract=off", "-fPIC", "-shared", "-o", path,
+           os.path.join(_HERE, "nvmai_oracle.c"), os.path.join(_HERE, "nvmai_oracle_bench.c"), "-lm", "-lpthread"]
+    try:
+        subprocess.run(cmd, check=True, capture_output=True)
+        return C.CDLL(path)
+    except (OSError, subprocess.CalledProcessError):
+        return None
+
 u8p = np.ctypeslib.ndpointer(np.uint8, flags="C_CONTIGUOUS")
 u16p = np.ctypeslib.ndpointer(np.uint16, flags="C_CONTIGUOUS")
 u32p = np.ctypeslib.ndpointer(np.uint32, flags="C_CONTIGUOUS")
@@ -265,11 +279,7 @@ lib.orc_moe_layer_forward.restype = None
 lib.orc_moe_layer_forward.argtypes = [C.POINTER(OrcMoeLayer), f32p, size_t, u32p, u16p, f32p]
 
 
-def moe_layer_forward(x, d, f, top_k, bits, router, expert_blobs, shared_blob=None, gate=None):
-    """router / gate: (kind, weights, scales, biases).  expert_blobs: uint8 [E, stride].
-    Returns (idx [T,k] u32, w [T,k] f16 bits, y [T,d] f32)."""
-    x = np.ascontiguousarray(x, np.float32).reshape(-1, d)
-    tokens = x.shape[0]
+def _moe_layer_struct(d, f, top_k, bits, router, expert_blobs, shared_blob, gate):
     ne = expert_blobs.shape[0]
     L = OrcMoeLayer()
     L.d, L.f, L.num_experts, L.top_k, L.bits = d, f, ne, top_k, bits
@@ -281,11 +291,104 @@ def moe_layer_forward(x, d, f, top_k, bits, router, expert_blobs, shared_blob=No
     if gate is not None:
         L.gate_kind = gate[0]
         L.gate_w, L.gate_s, L.gate_b = _ptr(gate[1]), _ptr(gate[2]), _ptr(gate[3])
+    L._keep = (ptrs, router, expert_blobs, shared_blob, gate)
+    return L
+
+
+def moe_layer_forward(x, d, f, top_k, bits, router, expert_blobs, shared_blob=None, gate=None):
+    """router / gate: (kind, weights, scales, biases).  expert_blobs: uint8 [E, stride].
+    Returns (idx [T,k] u32, w [T,k] f16 bits, y [T,d] f32)."""
+    x = np.ascontiguousarray(x, np.float32).reshape(-1, d)
+    tokens = x.shape[0]
+    L = _moe_layer_struct(d, f, top_k, bits, router, expert_blobs, shared_blob, gate)
     idx = np.zeros((tokens, top_k), np.uint32)
     w = np.zeros((tokens, top_k), np.uint16)
     y = np.zeros((tokens, d), np.float32)
     lib.orc_moe_layer_forward(C.byref(L), x, tokens, idx, w, y)
     return idx, w, y
+
+
+# ---------------------------------------------------------------- timed legs (bench.py's cpu_baseline only)
+def host_cpu():
+    """(model string, threads this process may use, capped at the GPU box's CPU share of 16)."""
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    return model, max(1, min(16, n))
+
+
+_timing = {}
+
+
+def timing_lib():
+    """(CDLL, flags string): the oracle rebuilt at -O3 -march=native in a temporary file, or the
+    -O2 library that ships with the tree when no compiler is at hand."""
+    if "lib" not in _timing:
+        import tempfile
+        path = os.path.join(tempfile.gettempdir(), "libnvmai_oracle_native_%d.so" % os.getpid())
+        native = build_native(path)
+        _timing["lib"] = (native, "-O3 -march=native -ffp-contract=off") if native is not None else \
+            (lib, "-O2 -ffp-contract=off (prebuilt)")
+    return _timing["lib"]
+
+
+def time_moe_layer(x, d, f, top_k, bits, router, expert_blobs, shared_blob, gate, threads, warmup=1, reps=5):
+    """Median seconds of one decode step of the layer over the tokens of x, tokens shared out over
+    `threads` threads; also returns the routing indices of the step."""
+    clib, _ = timing_lib()
+    x = np.ascontiguousarray(x, np.float32).reshape(-1, d)
+    tokens = x.shape[0]
+    L = _moe_layer_struct(d, f, top_k, bits, router, expert_blobs, shared_blob, gate)
+    idx = np.zeros((tokens, top_k), np.uint32)
+    w = np.zeros((tokens, top_k), np.uint16)
+    y = np.zeros((tokens, d), np.float32)
+    fn = clib.orc_time_moe_layer
+    fn.restype = C.c_double
+    fn.argtypes = [C.POINTER(OrcMoeLayer), f32p, size_t, C.c_int, C.c_int, C.c_int, u32p, u16p, f32p]
+    return fn(C.byref(L), x, tokens, threads, warmup, reps, idx, w, y), idx
+
+
+def time_attention(q, k_rows, v_rows, bits, nq, nkv, hd, seq, scale, threads, warmup=1, reps=5):
+    """q [B, nq, hd] float32; k_rows, v_rows uint8 [B, seq, stride]: median seconds of one decode
+    attention call over the B sequences, sequences shared out over the threads."""
+    clib, _ = timing_lib()
+    q = np.ascontiguousarray(q, np.float32)
+    k_rows, v_rows = np.ascontiguousarray(k_rows), np.ascontiguousarray(v_rows)
+    b = q.shape[0]
+    stride, vb = kv_row_layout(nkv * hd, bits)
+    out = np.zeros_like(q)
+    fn = clib.orc_time_attention
+    fn.restype = C.c_double
+    fn.argtypes = [f32p, u8p, u8p, size_t, size_t, C.c_int, size_t, size_t, size_t, size_t, size_t, size_t,
+                   C.c_float, C.c_int, C.c_int, C.c_int, f32p]
+    return fn(q, k_rows.reshape(-1), v_rows.reshape(-1), k_rows.strides[0], b, bits, stride, vb, nq, nkv, hd, seq,
+              scale, threads, warmup, reps, out)
+
+
+def time_prefill_moe(expert_blobs, bits, x, d, f, idx, w_f16, threads, warmup=1, reps=5):
+    clib, _ = timing_lib()
+    x = np.ascontiguousarray(x, np.float32).reshape(-1, d)
+    tokens = x.shape[0]
+    idx = np.ascontiguousarray(idx, np.uint32)
+    k = idx.shape[1]
+    ne = expert_blobs.shape[0]
+    ptrs = (C.c_void_p * ne)(*[expert_blobs[e].ctypes.data for e in range(ne)])
+    h2 = np.zeros((tokens, d), np.float32)
+    fn = clib.orc_time_prefill_moe
+    fn.restype = C.c_double
+    fn.argtypes = [C.POINTER(C.c_void_p), u32p, C.c_int, f32p, size_t, size_t, size_t, size_t, u32p, u16p,
+                   C.c_int, C.c_int, C.c_int, f32p]
+    return fn(ptrs, expert_offsets(d, f, bits), bits, x, tokens, d, f, k, idx,
+              np.ascontiguousarray(w_f16, np.uint16), threads, warmup, reps, h2)
 
 
 # ---------------------------------------------------------------- prefill
