@@ -117,7 +117,10 @@ int nvmai_hip_dequantize_affine(nvmai_hip_ctx* ctx, nvmai_stream stream, const u
  * and, with y_f32 != NULL, nvmai_int4_affine_gemv (nvmai_kernels.h:22-28):
  * y[t, :] = W x[t, :] for n_tokens inputs.  y (activations) or y_f32 may be NULL.
  * More than four inputs against a matrix of 1024 rows or more, 16-bit outputs only and 16-byte
- * aligned operands: runs as nvmai_hip_affine_qmm (the matrix is read once for all inputs). */
+ * aligned operands: runs as nvmai_hip_affine_qmm (the matrix is read once for all inputs).
+ * bits == 16: `weights` holds dense BF16 rows [m, n] (scales and biases unused, may be NULL; the
+ * BF16 LM head): a BF16 context only, n a multiple of 64 and at most 4096, any number of inputs
+ * (the matrix is read once per 16 of them). */
 int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
                           const uint16_t* scales, const uint16_t* biases, uint32_t bits,
                           const void* x, uint32_t x_stride, uint32_t n_tokens, uint32_t m,
@@ -499,6 +502,63 @@ int nvmai_hip_lm_head_greedy(nvmai_hip_ctx* ctx, nvmai_stream stream, const void
                              const uint8_t* weights, const uint16_t* scales, const uint16_t* biases,
                              uint32_t bits, uint32_t* out_tokens, uint32_t d, uint32_t vocab,
                              float rms_eps);
+
+/* hidden[r] += delta[r] (Elementwise.encodeResidualAdd, utility.metal:95-104), then
+ * out[r] = RMSNorm(hidden[r]) * weight (RMSNorm.encodeBF16W, rmsnorm.metal:64-110): the residual add
+ * that ends one block of a layer and the norm that opens the next (RealForwardRunner.swift:1897-1905)
+ * in one launch, same results as the two calls.  weight: BF16 [d] or NULL. */
+int nvmai_hip_residual_add_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, void* hidden, uint32_t hidden_stride,
+                                   const void* delta, uint32_t delta_stride, const uint16_t* weight, void* out,
+                                   uint32_t out_stride, uint32_t rows, uint32_t d, float eps);
+
+/* ---- gated-DeltaNet linear attention ------------------------------------------------------- */
+
+/* LinearAttentionConfig (ModelTypes.swift:15-41).  Rows of qkv / conv_out are
+ * [q: Hk * Dk][k: Hk * Dk][v: Hv * Dv]. */
+typedef struct {
+    uint32_t num_k_heads, num_v_heads, key_head_dim, value_head_dim, conv_kernel_size;
+} nvmai_gdn_config;
+
+/* GDN.encodeConvDecode / encodeConvPrefill + encodeConvTailUpdate + encodeQKNorm (GDN.swift:130-246;
+ * kernels gdn.metal:241-366, 386-441): conv_out = silu(causal depthwise conv of [tail | rows]),
+ * then the q and k heads normalised without weight and scaled by 1 / Dk and 1 / sqrt(Dk), and the
+ * tail replaced by the last K - 1 raw rows.  `batch` sequences of `rows` tokens each (1 = a decode
+ * step): qkv_raw and conv_out are [batch * rows, stride] activations, tail is [batch, K - 1, C]
+ * activations, conv_weight BF16 [C, K].  K <= 8. */
+int nvmai_hip_gdn_conv_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_gdn_config* config,
+                            const void* qkv_raw, uint32_t qkv_stride, void* tail, const uint16_t* conv_weight,
+                            void* conv_out, uint32_t conv_out_stride, uint32_t rows, uint32_t batch);
+
+/* GDN.encodeDeltaStepDecode / encodeDeltaStepPrefill + encodeGatedNorm (GDN.swift:248-341; kernels
+ * gdn.metal:443-587, 589-642): the gated delta rule over the rows of each sequence in order, state
+ * [batch, Hv, Dv, Dk] updated in place -- fp32 as the reference keeps it, or BF16 when
+ * state_is_bf16 (half the bytes per token, arithmetic still fp32) -- and
+ * out = rmsnorm(y) * norm_weight * silu(z) per value head.  a_proj, b_proj: [batch * rows, ab_stride]
+ * activations; a_log, dt_bias: BF16 [Hv]; z, out: [batch * rows, stride] activations; norm_weight
+ * BF16 [Dv].  (Dk, Dv) in {(128, 128), (64, 64), (32, 32), (64, 128), (128, 64)}. */
+int nvmai_hip_gdn_delta_gated_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_gdn_config* config,
+                                   const void* conv_out, uint32_t conv_out_stride, const void* a_proj,
+                                   const void* b_proj, uint32_t ab_stride, const uint16_t* a_log,
+                                   const uint16_t* dt_bias, void* state, int state_is_bf16, const void* z,
+                                   uint32_t z_stride, const uint16_t* norm_weight, void* out, uint32_t out_stride,
+                                   uint32_t rows, uint32_t batch);
+
+/* GDN.encodeInputProjections (GDN.swift:85-128; kernel gdn_in_proj_gemv_simd, gdn.metal:179-239) and
+ * FusedQKVGEMV.encode (kernel dequant_int4_qkv_gemv_simd, dequant_int4.metal:279-329): several
+ * projections of the same input rows.  parts[i]: y_i = W_i x.  When the parts' codes, scales,
+ * biases and outputs each lie back to back in memory (and there is one input row) the call is ONE
+ * launch over the concatenated rows; otherwise one launch per part.  Same results either way. */
+typedef struct {
+    const uint8_t* weights;
+    const uint16_t* scales;
+    const uint16_t* biases;
+    uint32_t rows;
+    void* y;                /* activations [n_tokens, y_stride] */
+    uint32_t y_stride;
+} nvmai_gemv_part;
+int nvmai_hip_affine_gemv_fused(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_gemv_part* parts,
+                                uint32_t n_parts, uint32_t bits, const void* x, uint32_t x_stride,
+                                uint32_t n_tokens, uint32_t n);
 
 /* Sampler.seedFor (Sampler.swift:304-325): splitmix64(seed + position), 0 mapped away. */
 uint64_t nvmai_sampler_seed_for(uint64_t seed, int64_t position);

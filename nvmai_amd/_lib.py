@@ -56,6 +56,16 @@ class GenerationConfig(C.Structure):
                 ("seed", u64), ("has_seed", i32)]
 
 
+class GdnConfig(C.Structure):
+    """nvmai_gdn_config"""
+    _fields_ = [(n, u32) for n in ("num_k_heads", "num_v_heads", "key_head_dim", "value_head_dim", "conv_kernel_size")]
+
+
+class GemvPart(C.Structure):
+    """nvmai_gemv_part"""
+    _fields_ = [("weights", vp), ("scales", vp), ("biases", vp), ("rows", u32), ("y", vp), ("y_stride", u32)]
+
+
 class PrefillGrouping(C.Structure):
     """nvmai_prefill_grouping"""
     _fields_ = [(n, vp) for n in ("sorted_pairs", "expert_offsets", "expert_counts", "groups", "tiles", "info")]
@@ -112,6 +122,11 @@ SIGNATURES = {
     "nvmai_hip_repetition_penalty": [vp, vp, vp, u32, vp, u32, C.c_float, C.c_float],
     "nvmai_hip_sampler_sample": [vp, vp, vp, vp, u32, vp, u32, C.POINTER(GenerationConfig), C.c_int64, C.c_float,
                                  C.c_int, vp, C.POINTER(C.c_int)],
+    "nvmai_hip_residual_add_rmsnorm": [vp, vp, vp, u32, vp, u32, vp, vp, u32, u32, u32, C.c_float],
+    "nvmai_hip_gdn_conv_norm": [vp, vp, C.POINTER(GdnConfig), vp, u32, vp, vp, vp, u32, u32, u32],
+    "nvmai_hip_gdn_delta_gated_norm": [vp, vp, C.POINTER(GdnConfig), vp, u32, vp, vp, u32, vp, vp, vp, C.c_int, vp, u32,
+                                       vp, vp, u32, u32, u32],
+    "nvmai_hip_affine_gemv_fused": [vp, vp, C.POINTER(GemvPart), u32, u32, vp, u32, u32, u32],
     "nvmai_hip_sample": [vp, vp, vp, u32, u32, u32, C.c_float, u32, C.c_float, C.POINTER(u64), C.POINTER(u32), vp],
 }
 _OTHER = {

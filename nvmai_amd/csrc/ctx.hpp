@@ -103,6 +103,10 @@ int expert_ffn_dense(nvmai_hip_ctx* ctx, hipStream_t s, const uint8_t* blob, con
                      uint32_t bits, const void* x, uint32_t x_stride, uint32_t tokens, uint32_t d, uint32_t f,
                      void* act, void* tmp, const float* gate_logit, void* y, uint32_t y_stride);
 
+// Dense BF16 rows against BF16 inputs on the matrix cores (step_api.hip).
+int dense_bf16_gemv(nvmai_hip_ctx* ctx, hipStream_t s, const uint16_t* w, const void* x, uint32_t x_stride,
+                    uint32_t n_tokens, uint32_t m, uint32_t n, void* y, float* y_f32, uint32_t y_stride);
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? NVMAI_OK : NVMAI_ERR_HIP; }
 
 }  // namespace nvmai

@@ -1,0 +1,126 @@
+// Entry points: gated-DeltaNet linear attention (conv + q / k norm, delta rule + gated output norm)
+// and the fused input projections of an attention block.
+#include "ctx.hpp"
+#include "gdn_kernels.cuh"
+
+using namespace nvmai;
+
+namespace {
+
+int check_gdn(const nvmai_gdn_config* c, uint32_t rows, uint32_t batch) {
+    if (!c || rows == 0 || batch == 0) return NVMAI_ERR_INVALID_ARG;
+    // GDN.init preconditions (GDN.swift:38-45)
+    if (c->key_head_dim == 0 || c->key_head_dim % 32 || c->value_head_dim == 0 || c->value_head_dim % 4 ||
+        c->num_k_heads == 0 || c->num_v_heads == 0 || c->num_v_heads % c->num_k_heads)
+        return NVMAI_ERR_INVALID_ARG;
+    if (c->conv_kernel_size == 0 || c->conv_kernel_size > GDN_MAX_TAPS) return NVMAI_ERR_UNSUPPORTED;
+    return NVMAI_OK;
+}
+
+GdnShape shape_of(const nvmai_gdn_config* c, uint32_t rows, uint32_t batch) {
+    return GdnShape{c->num_k_heads, c->num_v_heads, c->key_head_dim, c->value_head_dim, c->conv_kernel_size, rows, batch};
+}
+
+template <int ACT, int DK, int DV>
+void launch_delta(const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
+    const dim3 grid(p.sh.v_heads, p.sh.batch);
+    if (state_bf16) gdn_delta_gated_kernel<ACT, DK, DV, true><<<grid, 256, 0, s>>>(p);
+    else gdn_delta_gated_kernel<ACT, DK, DV, false><<<grid, 256, 0, s>>>(p);
+}
+
+template <int ACT>
+int launch_delta_shape(const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
+    const uint32_t dk = p.sh.dk, dv = p.sh.dv;
+    if (dk == 128 && dv == 128) launch_delta<ACT, 128, 128>(p, state_bf16, s);
+    else if (dk == 64 && dv == 64) launch_delta<ACT, 64, 64>(p, state_bf16, s);
+    else if (dk == 32 && dv == 32) launch_delta<ACT, 32, 32>(p, state_bf16, s);
+    else if (dk == 64 && dv == 128) launch_delta<ACT, 64, 128>(p, state_bf16, s);
+    else if (dk == 128 && dv == 64) launch_delta<ACT, 128, 64>(p, state_bf16, s);
+    else return NVMAI_ERR_UNSUPPORTED;
+    return NVMAI_OK;
+}
+
+}  // namespace
+
+extern "C" int nvmai_hip_gdn_conv_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_gdn_config* config,
+                                       const void* qkv_raw, uint32_t qkv_stride, void* tail, const uint16_t* conv_weight,
+                                       void* conv_out, uint32_t conv_out_stride, uint32_t rows, uint32_t batch) {
+    if (!ctx || !qkv_raw || !tail || !conv_weight || !conv_out) return NVMAI_ERR_INVALID_ARG;
+    int rc = check_gdn(config, rows, batch);
+    if (rc) return rc;
+    const uint32_t C = 2 * config->num_k_heads * config->key_head_dim + config->num_v_heads * config->value_head_dim;
+    if (qkv_stride < C || conv_out_stride < C) return NVMAI_ERR_INVALID_ARG;
+    const GdnShape sh = shape_of(config, rows, batch);
+    const dim3 grid(2 * sh.k_heads + sh.v_heads, batch);
+    hipStream_t s = (hipStream_t)stream;
+    if (ctx->act == ACT_BF16)
+        gdn_conv_norm_kernel<ACT_BF16><<<grid, 256, 0, s>>>((const uint16_t*)qkv_raw, qkv_stride, (uint16_t*)tail, conv_weight,
+                                                            (uint16_t*)conv_out, conv_out_stride, sh);
+    else
+        gdn_conv_norm_kernel<ACT_FP16><<<grid, 256, 0, s>>>((const uint16_t*)qkv_raw, qkv_stride, (uint16_t*)tail, conv_weight,
+                                                            (uint16_t*)conv_out, conv_out_stride, sh);
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_gdn_delta_gated_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_gdn_config* config,
+                                              const void* conv_out, uint32_t conv_out_stride, const void* a_proj,
+                                              const void* b_proj, uint32_t ab_stride, const uint16_t* a_log,
+                                              const uint16_t* dt_bias, void* state, int state_is_bf16, const void* z,
+                                              uint32_t z_stride, const uint16_t* norm_weight, void* out,
+                                              uint32_t out_stride, uint32_t rows, uint32_t batch) {
+    if (!ctx || !conv_out || !a_proj || !b_proj || !a_log || !dt_bias || !state || !z || !norm_weight || !out)
+        return NVMAI_ERR_INVALID_ARG;
+    int rc = check_gdn(config, rows, batch);
+    if (rc) return rc;
+    const uint32_t C = 2 * config->num_k_heads * config->key_head_dim + config->num_v_heads * config->value_head_dim;
+    const uint32_t vd = config->num_v_heads * config->value_head_dim;
+    if (conv_out_stride < C || ab_stride < config->num_v_heads || z_stride < vd || out_stride < vd) return NVMAI_ERR_INVALID_ARG;
+    GdnDeltaParams p{};
+    p.conv_out = (const uint16_t*)conv_out; p.conv_stride = conv_out_stride;
+    p.a_proj = (const uint16_t*)a_proj; p.b_proj = (const uint16_t*)b_proj; p.ab_stride = ab_stride;
+    p.a_log = a_log; p.dt_bias = dt_bias; p.state = state;
+    p.z = (const uint16_t*)z; p.z_stride = z_stride; p.norm_w = norm_weight;
+    p.out = (uint16_t*)out; p.out_stride = out_stride;
+    p.sh = shape_of(config, rows, batch);
+    hipStream_t s = (hipStream_t)stream;
+    rc = ctx->act == ACT_BF16 ? launch_delta_shape<ACT_BF16>(p, state_is_bf16 != 0, s)
+                              : launch_delta_shape<ACT_FP16>(p, state_is_bf16 != 0, s);
+    if (rc) return rc;
+    return launch_status();
+}
+
+// One GEMV launch over the concatenated rows of several matrices when they lie back to back in
+// memory (codes, scales and biases each, and the outputs), one launch per matrix otherwise.
+extern "C" int nvmai_hip_affine_gemv_fused(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_gemv_part* parts,
+                                           uint32_t n_parts, uint32_t bits, const void* x, uint32_t x_stride,
+                                           uint32_t n_tokens, uint32_t n) {
+    if (!ctx || !parts || n_parts == 0 || !x) return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    if (n == 0 || n % NVMAI_GROUP) return NVMAI_ERR_INVALID_ARG;
+    const uint64_t row_bytes = (uint64_t)n * bits / 8, meta_bytes = (uint64_t)(n / NVMAI_GROUP) * 2;
+    bool adjacent = n_tokens == 1;        // rows of one input are contiguous in the output; more inputs need a common stride
+    uint32_t total = 0;
+    for (uint32_t i = 0; i < n_parts; ++i) {
+        const nvmai_gemv_part& a = parts[i];
+        if (!a.weights || !a.scales || !a.biases || !a.y || a.y_stride < a.rows) return NVMAI_ERR_INVALID_ARG;
+        total += a.rows;
+        if (i + 1 < n_parts) {
+            const nvmai_gemv_part& b = parts[i + 1];
+            adjacent = adjacent && b.weights == a.weights + a.rows * row_bytes &&
+                       (const uint8_t*)b.scales == (const uint8_t*)a.scales + a.rows * meta_bytes &&
+                       (const uint8_t*)b.biases == (const uint8_t*)a.biases + a.rows * meta_bytes &&
+                       (const uint8_t*)b.y == (const uint8_t*)a.y + (size_t)a.rows * 2;
+        }
+    }
+    if (adjacent)
+        return nvmai_hip_affine_gemv(ctx, stream, parts[0].weights, parts[0].scales, parts[0].biases, bits, x, x_stride,
+                                     n_tokens, total, n, parts[0].y, nullptr, total);
+    for (uint32_t i = 0; i < n_parts; ++i) {
+        const nvmai_gemv_part& a = parts[i];
+        if (a.rows == 0) continue;
+        const int rc = nvmai_hip_affine_gemv(ctx, stream, a.weights, a.scales, a.biases, bits, x, x_stride, n_tokens,
+                                             a.rows, n, a.y, nullptr, a.y_stride);
+        if (rc) return rc;
+    }
+    return NVMAI_OK;
+}

@@ -1,0 +1,197 @@
+// Gated-DeltaNet linear attention for gfx950: the causal depthwise conv + SiLU with the q / k head
+// norm in one kernel, the gated delta rule with the gated output norm in another.  They replace the
+// reference's gdn_conv_mix_decode / _prefill, gdn_conv_tail_update, gdn_qk_norm,
+// gdn_delta_step_decode / _prefill and gdn_gated_norm (gdn.metal:241-642): a decode step is rows = 1,
+// a prefill chunk rows > 1 with the recurrence sequential inside the kernel, and every sequence of
+// a batch has its own conv tail and recurrent state.
+#pragma once
+
+#include "common.cuh"
+
+namespace nvmai {
+
+constexpr float GDN_RMS_EPS = 1e-6f;        // kGdnRmsEps, gdn.metal:28
+constexpr int GDN_MAX_TAPS = 8;
+
+struct GdnShape {
+    uint32_t k_heads, v_heads, dk, dv, taps;
+    uint32_t rows;                          // tokens per sequence in this call (1 = decode)
+    uint32_t batch;
+};
+
+__device__ __forceinline__ float gdn_silu(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float gdn_softplus(float x) { return x > 20.0f ? x : logf(1.0f + expf(x)); }
+
+// Sum over the 256 threads of a block, result in every thread.  part: 4 floats of LDS.
+__device__ __forceinline__ float gdn_block_sum(float v, float* part) {
+    v = wave_sum_bcast(v);
+    __syncthreads();                        // part may still be read from the previous use
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (part[0] + part[1]) + (part[2] + part[3]);
+}
+
+// ---- conv + SiLU + q / k norm (+ tail update) -------------------------------------------------
+// Block (head segment, sequence): segments 0 .. 2 Hk - 1 are the q then the k heads (Dk channels
+// each, normalised: x / rms * (1 / Dk for q, 1 / sqrt(Dk) for k), gdn.metal:386-441), segments from
+// 2 Hk on the value heads (Dv channels, conv only).  A thread owns channels tid, tid + 256, ... of its
+// segment for all rows of the call, reads the K - 1 tail rows of its channels once, and writes the
+// new tail (the last K - 1 raw rows of [old tail | chunk], gdn.metal:309-366) when it is done: no
+// other thread touches those columns.  conv_out is rounded to the activation type before the norm
+// reads it, as the two kernels of the reference hand it over in 16 bits.
+template <int ACT>
+__global__ __launch_bounds__(256) void gdn_conv_norm_kernel(const uint16_t* qkv_raw, uint32_t qkv_stride,
+                                                           uint16_t* tail, const uint16_t* conv_w,
+                                                           uint16_t* conv_out, uint32_t out_stride, GdnShape sh) {
+    __shared__ float part[4];
+    const uint32_t seg = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const uint32_t C = 2 * sh.k_heads * sh.dk + sh.v_heads * sh.dv;
+    const bool is_qk = seg < 2 * sh.k_heads;
+    const uint32_t seg_len = is_qk ? sh.dk : sh.dv;
+    const uint32_t base = is_qk ? seg * sh.dk : 2 * sh.k_heads * sh.dk + (seg - 2 * sh.k_heads) * sh.dv;
+    const uint32_t hist = sh.taps - 1;
+    uint16_t* tl = tail + (size_t)b * hist * C;
+    const uint16_t* raw = qkv_raw + (size_t)b * sh.rows * qkv_stride;
+    uint16_t* out = conv_out + (size_t)b * sh.rows * out_stride;
+    const float scale = seg < sh.k_heads ? 1.0f / (float)sh.dk : rsqrtf((float)sh.dk);
+    for (uint32_t t = 0; t < sh.rows; ++t) {
+        float sumsq = 0.0f;
+        for (uint32_t i = tid; i < seg_len; i += 256) {
+            const uint32_t ch = base + i;
+            float acc = 0.0f;
+            for (uint32_t j = 0; j < sh.taps; ++j) {
+                // input row in the virtual sequence [tail rows | chunk rows]
+                const int src = (int)t + (int)j - (int)hist;
+                const uint16_t v = src >= 0 ? raw[(size_t)src * qkv_stride + ch] : tl[(size_t)((int)hist + src) * C + ch];
+                acc = fmaf(act_to_f32<ACT>(v), bf16_to_f32(conv_w[ch * sh.taps + j]), acc);
+            }
+            const uint16_t r = f32_to_act<ACT>(gdn_silu(acc));
+            out[(size_t)t * out_stride + ch] = r;
+            const float x = act_to_f32<ACT>(r);
+            sumsq = fmaf(x, x, sumsq);
+        }
+        if (is_qk) {                                      // block-uniform
+            const float total = gdn_block_sum(sumsq, part);
+            const float inv = rsqrtf(total / (float)sh.dk + GDN_RMS_EPS);
+            for (uint32_t i = tid; i < seg_len; i += 256) {   // a thread rereads only what it wrote
+                uint16_t* o = out + (size_t)t * out_stride + base + i;
+                *o = f32_to_act<ACT>(act_to_f32<ACT>(*o) * inv * scale);
+            }
+        }
+    }
+    // new tail row j = virtual row rows + j - hist
+    for (uint32_t i = tid; i < seg_len; i += 256) {
+        const uint32_t ch = base + i;
+        uint16_t keep[GDN_MAX_TAPS];
+#pragma unroll
+        for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+            if (j >= hist) break;
+            const int src = (int)sh.rows + (int)j - (int)hist;
+            keep[j] = src >= 0 ? raw[(size_t)src * qkv_stride + ch] : tl[(size_t)((int)hist + src) * C + ch];
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+            if (j >= hist) break;
+            tl[(size_t)j * C + ch] = keep[j];
+        }
+    }
+}
+
+// ---- gated delta rule + gated output norm -------------------------------------------------------
+// Per value head h with state S [Dv, Dk] (gdn.metal:10-25, 443-587):
+//   g = exp(-exp(A_log[h]) * softplus(a[h] + dt_bias[h])),  beta = sigmoid(b[h])
+//   S *= g;  kv = S k;  S += outer((v - kv) * beta, k);  y = S q
+// then out = rmsnorm(y) * weight * silu(z) over the head's Dv outputs (gdn.metal:589-642).
+// Block (value head, sequence), four waves.  Sixteen lanes own one state row (Dk / 16 elements
+// each), so a wave works on four rows at once and the block on sixteen; a thread keeps its share of
+// all Dv / 16 row groups in registers across the rows of the call, so a prefill chunk reads and
+// writes the state once.  STATE_BF16: the state is stored in BF16 (half the bytes per token; the
+// arithmetic stays fp32), else in fp32 as the reference keeps it.
+struct GdnDeltaParams {
+    const uint16_t* conv_out;   // [batch * rows, conv_stride]: normed q, k and conv'd v
+    uint32_t conv_stride;
+    const uint16_t* a_proj;     // [batch * rows, ab_stride]
+    const uint16_t* b_proj;
+    uint32_t ab_stride;
+    const uint16_t* a_log;      // BF16 [Hv]
+    const uint16_t* dt_bias;    // BF16 [Hv]
+    void* state;                // [batch, Hv, Dv, Dk]
+    const uint16_t* z;          // [batch * rows, z_stride]
+    uint32_t z_stride;
+    const uint16_t* norm_w;     // BF16 [Dv]
+    uint16_t* out;              // [batch * rows, out_stride]
+    uint32_t out_stride;
+    GdnShape sh;
+};
+
+template <int ACT, int DK, int DV, bool STATE_BF16>
+__global__ __launch_bounds__(256) void gdn_delta_gated_kernel(GdnDeltaParams p) {
+    constexpr int EPL = DK / 16;                // state elements per lane
+    constexpr int GROUPS = DV / 16;             // sixteen rows per block pass
+    static_assert(DK % 16 == 0 && DV % 16 == 0 && EPL >= 1 && EPL <= 16, "shape");
+    __shared__ float y_s[DV];
+    __shared__ float part[4];
+    const uint32_t h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const uint32_t sub = tid & 15u, row_in_pass = tid >> 4;     // 16 rows per pass
+    const GdnShape& sh = p.sh;
+    const uint32_t hk = h / (sh.v_heads / sh.k_heads);
+    const float exp_a = expf(bf16_to_f32(p.a_log[h]));
+    const float dtb = bf16_to_f32(p.dt_bias[h]);
+    const size_t state_base = (((size_t)b * sh.v_heads + h) * DV) * DK;
+    float s[GROUPS][EPL];
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+        const size_t at = state_base + (size_t)(g * 16 + row_in_pass) * DK + sub * EPL;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e)
+            s[g][e] = STATE_BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(p.state)[at + e])
+                                 : reinterpret_cast<const float*>(p.state)[at + e];
+    }
+    for (uint32_t t = 0; t < sh.rows; ++t) {
+        const size_t row = (size_t)b * sh.rows + t;
+        const uint16_t* cq = p.conv_out + row * p.conv_stride + hk * DK + sub * EPL;
+        const uint16_t* ck = cq + sh.k_heads * DK;
+        const uint16_t* cv = p.conv_out + row * p.conv_stride + 2 * sh.k_heads * DK + h * DV;
+        float q[EPL], k[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) { q[e] = act_to_f32<ACT>(cq[e]); k[e] = act_to_f32<ACT>(ck[e]); }
+        const float g_decay = expf(-exp_a * gdn_softplus(act_to_f32<ACT>(p.a_proj[row * p.ab_stride + h]) + dtb));
+        const float beta = 1.0f / (1.0f + expf(-act_to_f32<ACT>(p.b_proj[row * p.ab_stride + h])));
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            const uint32_t dv = g * 16 + row_in_pass;
+            float kv = 0.0f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) { s[g][e] *= g_decay; kv = fmaf(s[g][e], k[e], kv); }
+            kv = seg_reduce_sum<16>(kv);
+            const float delta = (act_to_f32<ACT>(cv[dv]) - kv) * beta;
+            float o = 0.0f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) { s[g][e] = fmaf(k[e], delta, s[g][e]); o = fmaf(s[g][e], q[e], o); }
+            o = seg_reduce_sum<16>(o);
+            if (sub == 0) y_s[dv] = act_to_f32<ACT>(f32_to_act<ACT>(o));     // y is handed over in 16 bits
+        }
+        __syncthreads();
+        float sumsq = 0.0f;
+        for (uint32_t i = tid; i < DV; i += 256) sumsq = fmaf(y_s[i], y_s[i], sumsq);
+        const float total = gdn_block_sum(sumsq, part);
+        const float inv = rsqrtf(total / (float)DV + GDN_RMS_EPS);
+        for (uint32_t i = tid; i < DV; i += 256) {
+            const float normed = y_s[i] * inv * bf16_to_f32(p.norm_w[i]);
+            const float gate = gdn_silu(act_to_f32<ACT>(p.z[row * p.z_stride + h * DV + i]));
+            p.out[row * p.out_stride + h * DV + i] = f32_to_act<ACT>(normed * gate);
+        }
+        __syncthreads();                                    // y_s is rewritten by the next row
+    }
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+        const size_t at = state_base + (size_t)(g * 16 + row_in_pass) * DK + sub * EPL;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            if (STATE_BF16) reinterpret_cast<uint16_t*>(p.state)[at + e] = f32_to_bf16(s[g][e]);
+            else reinterpret_cast<float*>(p.state)[at + e] = s[g][e];
+        }
+    }
+}
+
+}  // namespace nvmai

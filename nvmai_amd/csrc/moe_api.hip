@@ -573,6 +573,11 @@ extern "C" int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, co
                                      const void* x, uint32_t x_stride, uint32_t n_tokens,
                                      uint32_t m, uint32_t n, void* y, float* y_f32,
                                      uint32_t y_stride) {
+    if (bits == 16) {                     // dense BF16 rows: the BF16 LM head
+        if (!ctx || !weights || !x || (!y && !y_f32)) return NVMAI_ERR_INVALID_ARG;
+        return nvmai::dense_bf16_gemv(ctx, (hipStream_t)stream, reinterpret_cast<const uint16_t*>(weights), x, x_stride,
+                                      n_tokens, m, n, y, y_f32, y_stride);
+    }
     // More than four input rows of a large matrix: the row engine would stream the matrix once per
     // four rows; the matrix-core product reads and dequantizes it once (from five rows on it is
     // the faster of the two at LM-head sizes).  Only where its preconditions hold and 16-bit

@@ -18,6 +18,52 @@ extern "C" int nvmai_hip_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const 
     return launch_status();
 }
 
+extern "C" int nvmai_hip_residual_add_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, void* hidden,
+                                              uint32_t hidden_stride, const void* delta, uint32_t delta_stride,
+                                              const uint16_t* weight, void* out, uint32_t out_stride, uint32_t rows,
+                                              uint32_t d, float eps) {
+    if (!ctx || !hidden || !delta || !out || d == 0 || hidden_stride < d || delta_stride < d || out_stride < d)
+        return NVMAI_ERR_INVALID_ARG;
+    if (rows == 0) return NVMAI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((rows + 3) / 4);
+    if (ctx->act == ACT_BF16)
+        residual_add_rmsnorm_kernel<ACT_BF16><<<grid, 256, 0, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta,
+                                                                   delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);
+    else
+        residual_add_rmsnorm_kernel<ACT_FP16><<<grid, 256, 0, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta,
+                                                                   delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);
+    return launch_status();
+}
+
+// Dense BF16 rows [m, n] against n_tokens BF16 inputs: the bits == 16 case of nvmai_hip_affine_gemv.
+namespace nvmai {
+int dense_bf16_gemv(nvmai_hip_ctx* ctx, hipStream_t s, const uint16_t* w, const void* x, uint32_t x_stride,
+                    uint32_t n_tokens, uint32_t m, uint32_t n, void* y, float* y_f32, uint32_t y_stride) {
+    if (ctx->act != ACT_BF16) return NVMAI_ERR_UNSUPPORTED;
+    if (n == 0 || n % 64 || n > 4096 || x_stride < n || y_stride < m) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(w) || !aligned16(x) || x_stride % 8) return NVMAI_ERR_ALIGNMENT;
+    if (m == 0 || n_tokens == 0) return NVMAI_OK;
+    static bool lds_raised = false;
+    if (!lds_raised) {
+        NVMAI_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(dense_bf16_gemv_kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, DENSE_TOK * (4096 * 2 + 16)));
+        lds_raised = true;
+    }
+    const uint32_t groups = (m + 63) / 64;                   // 64 rows per block pass
+    const uint32_t per_block = groups >= 4 * 1024 ? 4u : 1u; // long launches: fewer, longer blocks (the inputs are staged once per block)
+    const dim3 grid((groups + per_block - 1) / per_block);
+    for (uint32_t t0 = 0; t0 < n_tokens; t0 += DENSE_TOK) {
+        const uint32_t nt = n_tokens - t0 < (uint32_t)DENSE_TOK ? n_tokens - t0 : (uint32_t)DENSE_TOK;
+        dense_bf16_gemv_kernel<<<grid, 256, DENSE_TOK * (n * 2 + 16), s>>>(
+            w, (const uint16_t*)x + (size_t)t0 * x_stride, x_stride, nt, m, n,
+            y ? (uint16_t*)y + (size_t)t0 * y_stride : nullptr, y_f32 ? y_f32 + (size_t)t0 * y_stride : nullptr, y_stride,
+            per_block);
+    }
+    return launch_status();
+}
+}  // namespace nvmai
+
 namespace {
 
 template <int OP>

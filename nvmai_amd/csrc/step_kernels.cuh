@@ -45,6 +45,111 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* x, uint32_
     }
 }
 
+// hidden += delta (rounded to the activation type and stored, utility.metal:95-104), then
+// out = RMSNorm(hidden) * weight of the updated row (rmsnorm.metal:64-110): the residual add that
+// ends one block of a layer and the norm that opens the next, in one pass over the row.  Same
+// arithmetic and summation order as the two kernels one after the other.
+template <int ACT>
+__global__ __launch_bounds__(256) void residual_add_rmsnorm_kernel(uint16_t* hidden, uint32_t hidden_stride,
+                                                                   const uint16_t* delta, uint32_t delta_stride,
+                                                                   const uint16_t* weight, uint16_t* out,
+                                                                   uint32_t out_stride, uint32_t rows, uint32_t d,
+                                                                   float eps) {
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;                       // uniform per wave
+    const uint32_t lane = threadIdx.x & 63;
+    uint16_t* hr = hidden + (size_t)row * hidden_stride;
+    const uint16_t* dr = delta + (size_t)row * delta_stride;
+    float acc = 0.0f;
+    for (uint32_t i = lane; i < d; i += 64) {
+        const uint16_t sum = f32_to_act<ACT>(__fadd_rn(act_to_f32<ACT>(hr[i]), act_to_f32<ACT>(dr[i])));
+        hr[i] = sum;
+        const float v = act_to_f32<ACT>(sum);
+        acc = fmaf(v, v, acc);
+    }
+    const float inv = rms_inverse(rms_wave_sum(acc), d, eps);
+    uint16_t* o = out + (size_t)row * out_stride;
+    for (uint32_t i = lane; i < d; i += 64) {       // a lane rereads only what it wrote
+        float v = __fmul_rn(act_to_f32<ACT>(hr[i]), inv);
+        if (weight) v = __fmul_rn(v, bf16_to_f32(weight[i]));
+        o[i] = f32_to_act<ACT>(v);
+    }
+}
+
+// ---- dense BF16 rows against a few BF16 inputs (the BF16 LM head) ---------------------------------
+// y[t, r] = sum_k W[r, k] x[t, k] for up to 16 inputs per pass, on the matrix cores: the weight rows
+// are the B operand of v_mfma_f32_16x16x32_bf16 exactly as they lie in memory -- lane (i = lane % 16,
+// q = lane / 16) loads the 32 bytes W[r0 + i, k0 + 16 q .. + 16), so four lanes cover 128 contiguous
+// bytes of a row and every byte of the matrix is read once -- and the inputs are the A operand,
+// staged once per block in LDS (rows 16 bytes apart from a power of two, so the sixteen inputs of a
+// fragment read fall into different banks).  A wave owns 16 rows at a time and keeps DEPTH
+// super-steps of 64 k in flight.  The product is bound by the matrix's bytes: the matrix cores
+// idle most of the time, which is what lets one kernel serve 1 to 16 inputs at the same speed.
+typedef __bf16 dg_bf8_t __attribute__((ext_vector_type(8)));
+typedef float dg_fl4_t __attribute__((ext_vector_type(4)));
+constexpr int DENSE_TOK = 16;
+constexpr int DENSE_DEPTH = 4;
+
+__global__ __launch_bounds__(256) void dense_bf16_gemv_kernel(const uint16_t* w, const uint16_t* x, uint32_t x_stride,
+                                                             uint32_t tokens, uint32_t m, uint32_t n, uint16_t* y,
+                                                             float* y_f32, uint32_t y_stride, uint32_t row_groups_per_block) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t dense_lds[];
+    const uint32_t ld = n * 2u + 16u;                       // bytes between two inputs in LDS
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t li = lane & 15u, lq = lane >> 4;
+    // inputs -> LDS, zero rows for the inputs that are not there
+    for (uint32_t c = tid; c < DENSE_TOK * (n / 8u); c += 256u) {
+        const uint32_t t = c / (n / 8u), k8 = c % (n / 8u);
+        uint4 v = uint4{0, 0, 0, 0};
+        if (t < tokens) v = *reinterpret_cast<const uint4*>(x + (size_t)t * x_stride + k8 * 8u);
+        *reinterpret_cast<uint4*>(dense_lds + t * ld + k8 * 16u) = v;
+    }
+    __syncthreads();
+    const uint32_t steps = n / 64u;                         // super-steps of 64 k: two MFMAs each
+    const uint8_t* xa = dense_lds + li * ld + lq * 32u;      // this lane's A fragments
+    for (uint32_t g = 0; g < row_groups_per_block; ++g) {
+        const uint32_t r0 = ((blockIdx.x * row_groups_per_block + g) * 4u + wave) * 16u;
+        if (r0 >= m) break;                                 // wave-uniform
+        const uint32_t r = min(r0 + li, m - 1u);            // rows past the end repeat the last one, never stored
+        const uint4* wp = reinterpret_cast<const uint4*>(w + (size_t)r * n + lq * 16u);
+        dg_fl4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        uint4 buf[DENSE_DEPTH][2];
+#pragma unroll
+        for (int d = 0; d < DENSE_DEPTH; ++d) {
+            const uint32_t st = min((uint32_t)d, steps - 1u);
+            buf[d][0] = wp[st * 8u];
+            buf[d][1] = wp[st * 8u + 1u];
+        }
+        for (uint32_t s0 = 0; s0 < steps; s0 += DENSE_DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DENSE_DEPTH; ++d) {
+                const uint32_t st = s0 + d;
+                const uint4 b0 = buf[d][0], b1 = buf[d][1];
+                const uint32_t nx = min(st + DENSE_DEPTH, steps - 1u);     // unconditional: past the end rereads the last step
+                buf[d][0] = wp[nx * 8u];
+                buf[d][1] = wp[nx * 8u + 1u];
+                if (st < steps) {                           // uniform
+                    const uint4 a0 = *reinterpret_cast<const uint4*>(xa + st * 128u);
+                    const uint4 a1 = *reinterpret_cast<const uint4*>(xa + st * 128u + 16u);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dg_bf8_t, a0), __builtin_bit_cast(dg_bf8_t, b0), acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dg_bf8_t, a1), __builtin_bit_cast(dg_bf8_t, b1), acc, 0, 0, 0);
+                }
+            }
+        }
+        // acc[j] = y[input 4 q + j, row r0 + i]
+        if (r0 + li < m) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t t = lq * 4u + j;
+                if (t < tokens) {
+                    if (y) y[(size_t)t * y_stride + r0 + li] = f32_to_bf16(acc[j]);
+                    if (y_f32) y_f32[(size_t)t * y_stride + r0 + li] = acc[j];
+                }
+            }
+        }
+    }
+}
+
 // ---- elementwise helpers of the layer loop (utility.metal) -----------------------------------
 // 16-bit activations in and out, fp32 arithmetic, one rounding at the end.
 enum ElementwiseOp : int {

@@ -7,7 +7,7 @@ import ctypes as C
 import torch
 
 from . import _lib
-from ._lib import ExpertOffsets, GenerationConfig as _CGenerationConfig, KvView, MoeLayer, PrefillGrouping, Rows, check, lib
+from ._lib import ExpertOffsets, GdnConfig, GemvPart, GenerationConfig as _CGenerationConfig, KvView, MoeLayer, PrefillGrouping, Rows, check, lib
 
 ACT_BF16, ACT_FP16 = 0, 1
 (PROF_ROUTER, PROF_SELECT, PROF_GROUP, PROF_PHASE1, PROF_PHASE2, PROF_COMBINE, PROF_KV_QUANT,
@@ -586,6 +586,75 @@ class Sample:
         check(lib.nvmai_hip_sample(self.ctx.handle, _stream(), _ptr(p), p.stride(0), rows, p.shape[1], temperature,
                                    top_k, top_p, _seed_array(seed, rows), (C.c_uint32 * rows)(*pos), _ptr(out)),
               "sample")
+        return out
+
+
+def residual_add_rmsnorm(ctx, hidden, delta, weight, out=None, eps=1e-6):
+    """Elementwise.encodeResidualAdd + RMSNorm.encodeBF16W in one launch: hidden += delta (in place),
+    returns RMSNorm(hidden) * weight.  hidden, delta: [rows, d] activations."""
+    h2, d2 = hidden.reshape(-1, hidden.shape[-1]), delta.reshape(-1, delta.shape[-1])
+    if out is None:
+        out = torch.empty_like(h2)
+    check(lib.nvmai_hip_residual_add_rmsnorm(ctx.handle, _stream(), _ptr(h2), h2.stride(0), _ptr(d2), d2.stride(0),
+                                             _ptr(weight), _ptr(out), out.stride(0), h2.shape[0], h2.shape[1], eps),
+          "residual_add_rmsnorm")
+    return out
+
+
+def affine_gemv_fused(ctx, parts, bits, x, n):
+    """GDN.encodeInputProjections / FusedQKVGEMV.encode: parts = [(weights, scales, biases, rows, y), ...],
+    y_i = W_i x for the rows of x; one launch when the parts lie back to back in memory."""
+    x2 = x.reshape(-1, x.shape[-1])
+    arr = (GemvPart * len(parts))()
+    for i, (w, s_, b_, rows, y) in enumerate(parts):
+        arr[i].weights, arr[i].scales, arr[i].biases = w.data_ptr(), s_.data_ptr(), b_.data_ptr()
+        arr[i].rows, arr[i].y, arr[i].y_stride = rows, y.data_ptr(), (y.stride(0) if y.dim() > 1 else rows)
+    check(lib.nvmai_hip_affine_gemv_fused(ctx.handle, _stream(), arr, len(parts), bits, _ptr(x2), x2.stride(0),
+                                          x2.shape[0], n), "affine_gemv_fused")
+
+
+class GDN:
+    """Mirror of GDN (GDN.swift:13-341), gated-DeltaNet linear attention.  The reference's conv,
+    tail-update and q / k norm dispatches are one call here, the delta step and the gated output
+    norm another; `rows` tokens per sequence (1 = decode) for `batch` sequences."""
+
+    def __init__(self, ctx, num_k_heads, num_v_heads, key_head_dim, value_head_dim, conv_kernel_size=4):
+        self.ctx = ctx
+        self.cfg = GdnConfig(num_k_heads, num_v_heads, key_head_dim, value_head_dim, conv_kernel_size)
+        self.qkv_dim = 2 * num_k_heads * key_head_dim + num_v_heads * value_head_dim
+        self.value_dim = num_v_heads * value_head_dim
+
+    def new_state(self, batch=1, bf16=False):
+        """(conv tail [batch, K - 1, C] activations, recurrent state [batch, Hv, Dv, Dk]) zeroed
+        (GDNStateManager's buffers)."""
+        c = self.cfg
+        tail = torch.zeros((batch, c.conv_kernel_size - 1, self.qkv_dim), dtype=self.ctx.dtype, device=self.ctx.device)
+        state = torch.zeros((batch, c.num_v_heads, c.value_head_dim, c.key_head_dim),
+                            dtype=torch.bfloat16 if bf16 else torch.float32, device=self.ctx.device)
+        return tail, state
+
+    def encode_conv_norm(self, qkv_raw, tail, conv_weight, conv_out=None, rows=1):
+        """encodeConvDecode / encodeConvPrefill + encodeConvTailUpdate + encodeQKNorm."""
+        q2 = qkv_raw.reshape(-1, qkv_raw.shape[-1])
+        batch = q2.shape[0] // rows
+        if conv_out is None:
+            conv_out = torch.empty((q2.shape[0], self.qkv_dim), dtype=self.ctx.dtype, device=q2.device)
+        check(lib.nvmai_hip_gdn_conv_norm(self.ctx.handle, _stream(), C.byref(self.cfg), _ptr(q2), q2.stride(0),
+                                          _ptr(tail), _ptr(conv_weight), _ptr(conv_out), conv_out.stride(0), rows, batch),
+              "gdn_conv_norm")
+        return conv_out
+
+    def encode_delta_gated_norm(self, conv_out, a_proj, b_proj, a_log, dt_bias, state, z, norm_weight, out=None, rows=1):
+        """encodeDeltaStepDecode / encodeDeltaStepPrefill + encodeGatedNorm."""
+        batch = conv_out.shape[0] // rows
+        if out is None:
+            out = torch.empty((conv_out.shape[0], self.value_dim), dtype=self.ctx.dtype, device=conv_out.device)
+        check(lib.nvmai_hip_gdn_delta_gated_norm(self.ctx.handle, _stream(), C.byref(self.cfg), _ptr(conv_out),
+                                                 conv_out.stride(0), _ptr(a_proj), _ptr(b_proj), a_proj.stride(0),
+                                                 _ptr(a_log), _ptr(dt_bias), _ptr(state),
+                                                 int(state.dtype == torch.bfloat16), _ptr(z), z.stride(0),
+                                                 _ptr(norm_weight), _ptr(out), out.stride(0), rows, batch),
+              "gdn_delta_gated_norm")
         return out
 
 

@@ -100,6 +100,8 @@ _sig("orc_repetition_penalty", None, f32p, C.c_int, size_t, np.ctypeslib.ndpoint
 _sig("orc_sampler_route", C.c_int, C.c_int, C.c_float, C.c_int)
 _sig("orc_sampler_sample", C.c_uint32, f32p, size_t, C.c_float, C.c_int, C.c_float, C.c_int, C.c_float,
      C.c_uint64, C.c_int64, u16p)
+_sig("orc_gdn_step", None, f32p, f32p, f32p, f32p, u16p, u16p, u16p, u16p, size_t, size_t, size_t, size_t, size_t,
+     C.c_int, f32p, f32p, f32p)
 _sig("orc_rel_error", C.c_float, f32p, f32p, size_t)
 _sig("orc_rmsnorm", None, f32p, size_t, C.c_void_p, size_t, size_t, C.c_float, f32p, size_t)
 _sig("orc_elementwise", None, C.c_int, f32p, f32p, size_t, f32p)
@@ -537,6 +539,27 @@ def sample_generic(probs_f16, temperature, top_k, top_p, seed):
 def sample_gumbel(probs_f16, temperature, seed, position=0):
     p = np.ascontiguousarray(probs_f16, np.uint16)
     return lib.orc_sample_gumbel(p, p.size, temperature, seed, position)
+
+
+class GdnLayerState:
+    """Conv tail [(taps - 1), C] and recurrent state [Hv, Dv, Dk] of one gated-DeltaNet layer, fp32."""
+
+    def __init__(self, k_heads, v_heads, dk, dv, taps):
+        self.shape = (k_heads, v_heads, dk, dv, taps)
+        self.tail = np.zeros((taps - 1, 2 * k_heads * dk + v_heads * dv), np.float32)
+        self.state = np.zeros((v_heads, dv, dk), np.float32)
+
+
+def gdn_step(st, qkv_raw, a, b, z, conv_w, a_log, dt_bias, norm_w, act=0):
+    """GDNReference.step (GDNReference.swift:41-114) on st (updated in place); weights as BF16 bits.
+    Returns the gated output [Hv * Dv], not rounded."""
+    kh, vh, dk, dv, taps = st.shape
+    out = np.zeros(vh * dv, np.float32)
+    f = lambda v: np.ascontiguousarray(v, np.float32)
+    u = lambda v: np.ascontiguousarray(v, np.uint16)
+    lib.orc_gdn_step(f(qkv_raw), f(a), f(b), f(z), u(conv_w), u(a_log), u(dt_bias), u(norm_w), kh, vh, dk, dv,
+                     taps, act, st.tail, st.state, out)
+    return out
 
 
 def repetition_penalty(logits, act, history, penalty, softcap=0.0):

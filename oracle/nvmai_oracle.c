@@ -1096,6 +1096,75 @@ uint32_t orc_sample_topk64(const uint16_t *probs_f16, size_t v, float temperatur
     return sample_tail(val, idx, kept, temperature, top_p, seed, idx[0]);
 }
 
+/* ------------------------------------------------------------------------ */
+/* gated DeltaNet linear attention                                            */
+/* ------------------------------------------------------------------------ */
+
+static float round_act(float v, int act) {
+    return act == 0 ? orc_bf16_to_float(orc_bf16_bits(v)) : orc_f16_to_float(orc_f16_bits(v));
+}
+static float gdn_silu(float x) { return x / (1.0f + expf(-x)); }                 /* gdn.metal:71-73 */
+static float gdn_softplus(float x) { return x > 20.0f ? x : logf(1.0f + expf(x)); }   /* :75-79 */
+
+/* GDNReference.step (GDNReference.swift:41-114), the CPU model of one token through the kernels of
+ * gdn.metal:241-271 (conv + SiLU, tail shift), :386-441 (q / k norm with the folded scales 1 / Dk and
+ * 1 / sqrt(Dk)), :443-508 (gated delta rule) and :589-642 (gated output norm), with the reference's
+ * rounding points: conv output, normed q / k and y are rounded to the activation type (act 0 = bf16,
+ * 1 = fp16, the reference's), the tail keeps the raw row rounded to it, the state stays fp32.
+ *   qkv_raw [C], a, b [Hv], z [Hv * Dv]: projection outputs (activation values as floats)
+ *   conv_w [C, taps], a_log, dt_bias [Hv], norm_w [Dv]: BF16 bits
+ *   tail [(taps - 1), C] and state [Hv, Dv, Dk] are updated in place; out [Hv * Dv] is NOT rounded. */
+void orc_gdn_step(const float *qkv_raw, const float *a, const float *b, const float *z,
+                  const uint16_t *conv_w, const uint16_t *a_log, const uint16_t *dt_bias,
+                  const uint16_t *norm_w, size_t k_heads, size_t v_heads, size_t dk, size_t dv,
+                  size_t taps, int act, float *tail, float *state, float *out) {
+    const size_t C = 2 * k_heads * dk + v_heads * dv, hist = taps - 1;
+    float *conv = (float *)malloc(C * sizeof(float));
+    float *normed = (float *)malloc(C * sizeof(float));
+    float *y = (float *)malloc(v_heads * dv * sizeof(float));
+    for (size_t ch = 0; ch < C; ++ch) {                       /* GDNReference.swift:50-58 */
+        float acc = qkv_raw[ch] * orc_bf16_to_float(conv_w[ch * taps + hist]);
+        for (size_t j = 0; j < hist; ++j) acc += tail[j * C + ch] * orc_bf16_to_float(conv_w[ch * taps + j]);
+        conv[ch] = round_act(gdn_silu(acc), act);
+    }
+    for (size_t j = 0; j + 1 < hist; ++j) memcpy(tail + j * C, tail + (j + 1) * C, C * sizeof(float));
+    if (hist) for (size_t ch = 0; ch < C; ++ch) tail[(hist - 1) * C + ch] = round_act(qkv_raw[ch], act);
+    memcpy(normed, conv, C * sizeof(float));
+    for (size_t hi = 0; hi < 2 * k_heads; ++hi) {             /* :62-74 */
+        const int is_q = hi < k_heads;
+        const size_t base = (is_q ? 0 : k_heads * dk) + (is_q ? hi : hi - k_heads) * dk;
+        float sumsq = 0.0f;
+        for (size_t i = 0; i < dk; ++i) sumsq += conv[base + i] * conv[base + i];
+        const float inv = 1.0f / sqrtf(sumsq / (float)dk + 1e-6f);
+        const float scale = is_q ? 1.0f / (float)dk : 1.0f / sqrtf((float)dk);
+        for (size_t i = 0; i < dk; ++i) normed[base + i] = round_act(conv[base + i] * inv * scale, act);
+    }
+    for (size_t h = 0; h < v_heads; ++h) {                    /* :77-99 */
+        const size_t hk = h / (v_heads / k_heads);
+        const float *q = normed + hk * dk, *k = normed + k_heads * dk + hk * dk;
+        const float *v = normed + 2 * k_heads * dk + h * dv;
+        const float g = expf(-expf(orc_bf16_to_float(a_log[h])) * gdn_softplus(a[h] + orc_bf16_to_float(dt_bias[h])));
+        const float beta = 1.0f / (1.0f + expf(-b[h]));
+        for (size_t d = 0; d < dv; ++d) {
+            float *srow = state + (h * dv + d) * dk;
+            float kv = 0.0f;
+            for (size_t i = 0; i < dk; ++i) { srow[i] *= g; kv += srow[i] * k[i]; }
+            const float delta = (v[d] - kv) * beta;
+            float o = 0.0f;
+            for (size_t i = 0; i < dk; ++i) { srow[i] += k[i] * delta; o += srow[i] * q[i]; }
+            y[h * dv + d] = round_act(o, act);
+        }
+    }
+    for (size_t h = 0; h < v_heads; ++h) {                    /* :102-112 */
+        float sumsq = 0.0f;
+        for (size_t i = 0; i < dv; ++i) sumsq += y[h * dv + i] * y[h * dv + i];
+        const float inv = 1.0f / sqrtf(sumsq / (float)dv + 1e-6f);
+        for (size_t i = 0; i < dv; ++i)
+            out[h * dv + i] = y[h * dv + i] * inv * orc_bf16_to_float(norm_w[i]) * gdn_silu(z[h * dv + i]);
+    }
+    free(y); free(normed); free(conv);
+}
+
 /* Sampler.applyRepetitionPenaltyInPlace (Sampler.swift:259-293): for every DISTINCT id of the
  * history inside the vocabulary, a positive logit is divided by the penalty and a negative one
  * multiplied; with a logit softcap the penalty acts on the capped logit and is mapped back through

@@ -198,6 +198,13 @@ uint32_t orc_sample_topk64(const uint16_t *probs_f16, size_t v, float temperatur
                            float top_p, uint64_t seed, uint32_t top_k,
                            uint32_t *top64_idx, float *top64_val);
 
+/* GDNReference.step (GDNReference.swift:41-114): one token of gated-DeltaNet linear attention --
+ * causal depthwise conv + SiLU, q / k norm with folded scales, gated delta rule, gated output norm. */
+void orc_gdn_step(const float *qkv_raw, const float *a, const float *b, const float *z,
+                  const uint16_t *conv_w, const uint16_t *a_log, const uint16_t *dt_bias,
+                  const uint16_t *norm_w, size_t k_heads, size_t v_heads, size_t dk, size_t dv,
+                  size_t taps, int act, float *tail, float *state, float *out);
+
 /* Sampler.sample's front end (Sampler.swift:171-293): the repetition penalty over the distinct
  * history ids, the choice between the tiled and the generic sampler, and the whole call. */
 void orc_repetition_penalty(float *logits, int act, size_t v, const int32_t *ids, size_t n_ids,

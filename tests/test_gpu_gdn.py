@@ -1,0 +1,219 @@
+"""GPU parity: gated-DeltaNet linear attention (conv + q / k norm, delta rule + gated output norm), the
+fused residual add + RMSNorm, the fused input projections and the dense BF16 GEMV, through the C ABI
+against the CPU oracle.
+
+GDN bar: the reference's own, for its kernels against its CPU model (GDNKernelTests.swift:170-185):
+|got - want| <= max(2e-2, 4e-2 |want|) per output and 5e-2 on the recurrent state, with fp16
+activations as there; with bf16 activations (three mantissa bits fewer at every hand-over) the same
+form at 8e-2 / 1.6e-1."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from gpu_util import act_np, act_tensor, dev, gauss, round_act, say
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def nv():
+    import nvmai_amd
+    return nvmai_amd
+
+
+@pytest.fixture(scope="module", params=[0, 1], ids=["bf16", "fp16"])
+def ctx(request, nv):
+    c = nv.Context(0, request.param)
+    yield c
+    torch.cuda.synchronize()
+    c.close()
+
+
+def _fixture(cfg, rows, seed, act):
+    kh, vh, dk, dv, taps = cfg
+    C = 2 * kh * dk + vh * dv
+    rng = np.random.default_rng(seed)
+    u = lambda lo, hi, n: rng.uniform(lo, hi, n).astype(np.float32)
+    r = lambda a: round_act(a, act)
+    return dict(conv_w=O.bf16_bits(u(-0.4, 0.4, C * taps)), a_log=O.bf16_bits(u(-1.0, 1.5, vh)),
+                dt_bias=O.bf16_bits(u(-0.5, 0.5, vh)), norm_w=O.bf16_bits(u(0.5, 1.5, dv)),
+                qkv=r(u(-1, 1, rows * C)).reshape(rows, C), a=r(u(-1, 1, rows * vh)).reshape(rows, vh),
+                b=r(u(-1, 1, rows * vh)).reshape(rows, vh), z=r(u(-1, 1, rows * vh * dv)).reshape(rows, vh * dv))
+
+
+def _bits(a):
+    return dev(np.ascontiguousarray(a).view(np.int16))
+
+
+def _close(got, want, act):
+    lo, rel = (2e-2, 4e-2) if act == 1 else (8e-2, 1.6e-1)
+    return np.all(np.abs(got - want) <= np.maximum(lo, np.abs(want) * rel))
+
+
+def _gpu_rows(nv, ctx, gdn, fx, tail, state, t0, rows, batch_rows=None):
+    """rows tokens of one sequence (or of each sequence when batch_rows is given) in one call."""
+    sl = slice(t0, t0 + rows)
+    conv = gdn.encode_conv_norm(act_tensor(fx["qkv"][sl], ctx), tail, _bits(fx["conv_w"]), rows=rows)
+    return gdn.encode_delta_gated_norm(conv, act_tensor(fx["a"][sl], ctx), act_tensor(fx["b"][sl], ctx),
+                                       _bits(fx["a_log"]), _bits(fx["dt_bias"]), state, act_tensor(fx["z"][sl], ctx),
+                                       _bits(fx["norm_w"]), rows=rows)
+
+
+@pytest.mark.parametrize("cfg", [(2, 4, 32, 32, 4), (16, 32, 128, 128, 4), (2, 2, 64, 64, 2), (1, 2, 64, 128, 3)],
+                         ids=["reference-toy", "production", "dk64", "dk64-dv128"])
+def test_gdn_decode_chain_matches_oracle(nv, ctx, cfg):
+    # decodeChainMatchesReference (GDNKernelTests.swift:130-187): six tokens, outputs, tail and state
+    say("gdn decode chain", ctx.act, cfg)
+    rows = 6
+    fx = _fixture(cfg, rows, 0x51D, ctx.act)
+    gdn = nv.GDN(ctx, *cfg)
+    tail, state = gdn.new_state()
+    ref = O.GdnLayerState(*cfg)
+    for t in range(rows):
+        got = act_np(_gpu_rows(nv, ctx, gdn, fx, tail, state, t, 1))[0]
+        want = O.gdn_step(ref, fx["qkv"][t], fx["a"][t], fx["b"][t], fx["z"][t], fx["conv_w"], fx["a_log"],
+                          fx["dt_bias"], fx["norm_w"], ctx.act)
+        torch.cuda.synchronize()
+        assert _close(got, want, ctx.act), "token %d" % t
+    assert np.array_equal(act_np(tail[0]), ref.tail)               # raw rows, copied
+    assert np.abs(state[0].cpu().numpy() - ref.state).max() <= 5e-2
+
+
+def test_gdn_prefill_chunk_equals_sequential_decode(nv, ctx):
+    # prefillChunkMatchesSequentialDecode (GDNKernelTests.swift:189-290): seven rows in one call against seven
+    # calls; and a chunk shorter than the conv history (the ordered tail shift, gdn.metal:337-366)
+    for cfg, rows in (((2, 4, 32, 32, 4), 7), ((16, 32, 128, 128, 4), 5), ((2, 4, 32, 32, 4), 2)):
+        say("gdn prefill chunk", ctx.act, cfg, rows)
+        fx = _fixture(cfg, rows + 3, 0xBEEF, ctx.act)
+        gdn = nv.GDN(ctx, *cfg)
+        tail_a, state_a = gdn.new_state()
+        tail_b, state_b = gdn.new_state()
+        seq = []
+        for t in range(3):                                        # a common prefix, so that the tail is not zero
+            _gpu_rows(nv, ctx, gdn, fx, tail_a, state_a, t, 1)
+            _gpu_rows(nv, ctx, gdn, fx, tail_b, state_b, t, 1)
+        for t in range(3, 3 + rows):
+            seq.append(act_np(_gpu_rows(nv, ctx, gdn, fx, tail_a, state_a, t, 1))[0])
+        chunk = act_np(_gpu_rows(nv, ctx, gdn, fx, tail_b, state_b, 3, rows))
+        torch.cuda.synchronize()
+        assert _close(chunk, np.array(seq), ctx.act)
+        assert torch.equal(tail_a, tail_b)
+        assert (state_a - state_b).abs().max().item() <= 5e-2
+
+
+@pytest.mark.parametrize("bf16_state", [False, True])
+def test_gdn_batch_of_sequences_and_bf16_state(nv, ctx, bf16_state):
+    # three sequences with their own tails and states in one call per token; the BF16 state is the
+    # measured variant (half the state bytes per token) and tracks the fp32 oracle more loosely
+    say("gdn batch", ctx.act, bf16_state)
+    cfg, batch, steps = (16, 32, 128, 128, 4), 3, 4
+    kh, vh, dk, dv, taps = cfg
+    fxs = [_fixture(cfg, steps, 100 + b, ctx.act) for b in range(batch)]
+    gdn = nv.GDN(ctx, *cfg)
+    tail, state = gdn.new_state(batch, bf16=bf16_state)
+    refs = [O.GdnLayerState(*cfg) for _ in range(batch)]
+    w = fxs[0]
+    for t in range(steps):
+        stack = lambda key: act_tensor(np.stack([fx[key][t] for fx in fxs]), ctx)
+        conv = gdn.encode_conv_norm(stack("qkv"), tail, _bits(w["conv_w"]))
+        out = act_np(gdn.encode_delta_gated_norm(conv, stack("a"), stack("b"), _bits(w["a_log"]), _bits(w["dt_bias"]),
+                                                 state, stack("z"), _bits(w["norm_w"])))
+        torch.cuda.synchronize()
+        for b in range(batch):
+            want = O.gdn_step(refs[b], fxs[b]["qkv"][t], fxs[b]["a"][t], fxs[b]["b"][t], fxs[b]["z"][t], w["conv_w"],
+                              w["a_log"], w["dt_bias"], w["norm_w"], ctx.act)
+            if bf16_state:
+                assert np.all(np.abs(out[b] - want) <= np.maximum(0.15, np.abs(want) * 0.3))
+            else:
+                assert _close(out[b], want, ctx.act), (t, b)
+    got_state = state.float().cpu().numpy()
+    for b in range(batch):
+        assert np.abs(got_state[b] - refs[b].state).max() <= (5e-2 if not bf16_state else 1e-1)
+
+
+def test_gdn_rejects_bad_shapes(nv, ctx):
+    say("gdn errors")
+    with pytest.raises(nv.NvmaiError) as e:            # numVHeads must be a multiple of numKHeads (GDN.swift:44-45)
+        g = nv.GDN(ctx, 3, 4, 32, 32, 4)
+        tail, state = g.new_state()
+        g.encode_conv_norm(torch.zeros((1, g.qkv_dim), dtype=ctx.dtype, device="cuda"), tail,
+                           torch.zeros(g.qkv_dim * 4, dtype=torch.int16, device="cuda"))
+    assert e.value.name == "invalid_arg"
+    with pytest.raises(nv.NvmaiError) as e:            # keyHeadDim must be a positive multiple of 32 (GDN.swift:38-39)
+        g = nv.GDN(ctx, 2, 4, 48, 32, 4)
+        tail, state = g.new_state()
+        g.encode_conv_norm(torch.zeros((1, g.qkv_dim), dtype=ctx.dtype, device="cuda"), tail,
+                           torch.zeros(g.qkv_dim * 4, dtype=torch.int16, device="cuda"))
+    assert e.value.name == "invalid_arg"
+
+
+def test_residual_add_rmsnorm_equals_the_two_calls(nv, ctx):
+    say("residual add + rmsnorm", ctx.act)
+    rng = np.random.default_rng(5)
+    for rows, d in ((1, 2048), (5, 2048), (3, 192), (16, 4096)):
+        h = round_act(gauss(rng, (rows, d)), ctx.act)
+        delta = round_act(gauss(rng, (rows, d), 0.3), ctx.act)
+        w = _bits(O.bf16_bits(rng.uniform(0.5, 1.5, d).astype(np.float32)))
+        h1, h2 = act_tensor(h, ctx), act_tensor(h, ctx)
+        out = nv.residual_add_rmsnorm(ctx, h1, act_tensor(delta, ctx), w)
+        nv.Elementwise(ctx).encode_residual_add(h2, act_tensor(delta, ctx))
+        want = nv.RMSNorm(ctx).encode_bf16w(h2, w)
+        torch.cuda.synchronize()
+        assert torch.equal(h1, h2) and torch.equal(out, want)
+        # and against the oracle: the sum rounded to the activation type, then the norm (bit-exact)
+        hs = round_act(h + delta, ctx.act)
+        assert np.array_equal(act_np(out), round_act(O.rmsnorm(hs, w.cpu().numpy().view(np.uint16), 1e-6), ctx.act))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_fused_projections_equal_separate_gemvs(nv, ctx, bits):
+    # GDN.encodeInputProjections (qkv, z, a, b) and FusedQKVGEMV: bit-identical to the separate GEMVs,
+    # whether the parts lie back to back (one launch) or not
+    say("fused projections", ctx.act, bits)
+    rng = np.random.default_rng(bits)
+    n, rows_list = 2048, [1024, 512, 32, 32]
+    total = sum(rows_list)
+    wq = O.quantize_affine(O.round_bf16(gauss(rng, (total, n), 0.02)), bits)
+    W, S, B = dev(wq[0]), dev(wq[1].view(np.int16)), dev(wq[2].view(np.int16))
+    x = act_tensor(round_act(gauss(rng, (1, n)), ctx.act), ctx)
+    want = nv.affine_gemv(ctx, W, S, B, bits, x, total, n)
+    y = torch.zeros((1, total), dtype=ctx.dtype, device="cuda")
+    parts, at = [], 0
+    for r in rows_list:
+        parts.append((W[at:at + r], S[at:at + r], B[at:at + r], r, y[0, at:at + r]))
+        at += r
+    nv.affine_gemv_fused(ctx, parts, bits, x, n)
+    torch.cuda.synchronize()
+    assert torch.equal(y, want)
+    # scattered outputs: one launch per part, same bits
+    outs = [torch.zeros(r + 8, dtype=ctx.dtype, device="cuda") for r in rows_list]
+    parts = [(p[0], p[1], p[2], p[3], o[:p[3]]) for p, o in zip(parts, outs)]
+    nv.affine_gemv_fused(ctx, parts, bits, x, n)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([o[:r] for o, r in zip(outs, rows_list)]), want[0])
+
+
+def test_dense_bf16_gemv(nv):
+    # bits == 16: dense BF16 rows (the BF16 LM head), 1..16 inputs per pass and more than 16; against
+    # a float64 product of the same BF16 values (fp32 accumulate: 2e-3 on the fp32 output, 1e-2 on BF16)
+    say("dense bf16 gemv")
+    ctx = nv.Context(0, 0)
+    rng = np.random.default_rng(9)
+    for m, n, tokens in ((1000, 2048, 1), (70, 256, 3), (4096, 2048, 16), (515, 1024, 21), (64, 64, 2)):
+        w = O.round_bf16(gauss(rng, (m, n), 0.02))
+        x = O.round_bf16(gauss(rng, (tokens, n)))
+        wd = dev(O.bf16_bits(w).view(np.int16))
+        y = nv.affine_gemv(ctx, wd, None, None, 16, act_tensor(x, ctx), m, n)
+        yf = nv.affine_gemv(ctx, wd, None, None, 16, act_tensor(x, ctx), m, n, out_f32=True)
+        torch.cuda.synchronize()
+        want = x.astype(np.float64) @ w.astype(np.float64).T
+        assert O.rel_error(yf.cpu().numpy(), want.astype(np.float32)) < 2e-3
+        assert O.rel_error(act_np(y), want.astype(np.float32)) < 1e-2
+    c16 = nv.Context(0, 1)
+    with pytest.raises(nv.NvmaiError) as e:            # dense BF16 rows need BF16 activations
+        nv.affine_gemv(c16, wd, None, None, 16, torch.zeros((1, 64), dtype=torch.float16, device="cuda"), 64, 64)
+    assert e.value.name == "unsupported"
+    torch.cuda.synchronize()
+    ctx.close()
+    c16.close()
