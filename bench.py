@@ -36,11 +36,12 @@ def parse():
     ap.add_argument("--sweep", action="store_true", help="also print batch/bits sweep lines to stderr")
     ap.add_argument("--no-extra", action="store_true", help="skip the `extra` object (the other cells of the metric) "
                     "that the default invocation appends")
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "sampler", "greedy", "copy"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "sampler", "greedy", "step", "copy"],
                     help="decode = configs[1] (the headline line); prefill = configs[2] grouped GEMM; "
                          "attention = configs[3] quantized-KV decode attention; sampler = the end of configs[4]: "
                          "quantized LM head GEMV over 248,320 rows, tiled softmax, top-k sampler; greedy = the fused greedy LM head "
-                         "(RMSNorm + logits in a fixed order + argmax) over the same head; copy = a plain 1 GiB device copy, "
+                         "(RMSNorm + logits in a fixed order + argmax) over the same head; step = configs[4], the full 40-layer decode "
+                         "step (tok/s at --batch 1..16, KV at --context); copy = a plain 1 GiB device copy, "
                          "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated on")
     ap.add_argument("--context", type=int, default=32768, help="attention: tokens in the KV cache")
     ap.add_argument("--tokens", type=int, default=4096, help="prefill: tokens per step")
@@ -570,6 +571,70 @@ def run_greedy(nv, ctx, torch, a):
     }
 
 
+def run_step(nv, ctx, torch, a):
+    """configs[4]: the full synthetic decode step of the 40-layer hybrid model (30 gated-DeltaNet layers with
+    a BF16 recurrent state, 10 full-attention layers over an 8-bit KV cache at `--context`, 4-bit experts and
+    projections, BF16 LM head over 248,320, tiled top-k sampler), captured once into a HIP graph and replayed:
+    tok/s for `--batch` sequences and the fraction of the bytes-per-token roofline."""
+    from nvmai_amd.decoder import HybridConfig, HybridDecoder, HybridWeights
+    B, context = min(a.batch, 16), a.context
+    cfg = HybridConfig(layers=40, expert_bits=4, attn_bits=4, kv_bits=8, head_bits=16, gdn_state_bf16=True)
+    w = HybridWeights(ctx, cfg, seed=2024)
+    dec = HybridDecoder(ctx, cfg, w, batch=B, max_context=context)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    quant = nv.KVCacheQuantizer(ctx)
+    for L, (kc, vc) in dec.kv.items():                      # a cache full of quantized N(0, 1) rows
+        for c in (kc, vc):
+            for b in range(B):
+                for start in range(0, context, 8192):
+                    n = min(8192, context - start)
+                    src = torch.empty((n, cfg.kv_dim), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
+                    quant.encode(src, cfg.kv_dim, c.view(b, start), n, cfg.kv_dim)
+    dec.tokens.copy_(torch.randint(0, cfg.vocab, (B,), generator=gen, device="cuda", dtype=torch.int32))
+    position = context - 1
+    seeds = [nv.sampler_seed_for(1234, position + b) for b in range(B)]
+    dec.step(position, seeds)                               # warm-up: sizes the workspace
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            dec.step(position, seeds)
+    torch.cuda.synchronize()
+    for _ in range(a.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    # the same step launched eagerly (every call through the C ABI from Python), for comparison
+    t0 = time.perf_counter()
+    for _ in range(5):
+        dec.step(position, seeds)
+    torch.cuda.synchronize()
+    dt_eager = (time.perf_counter() - t0) / 5
+    bpt = cfg.bytes_per_token(B, context)
+    gbps = bpt * B / dt / 1e9
+    assert bool(((dec.next_tokens >= 0) & (dec.next_tokens < cfg.vocab)).all()) and bool(torch.isfinite(dec.logits.float()).all())
+    return {
+        "metric": METRIC, "value": round(B / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u4 codes, f32 accumulate; bf16 activations, recurrent state and LM head; u8 KV", "data": "synthetic",
+        "config": {"workload": "configs[4]: full decode step of the 40-layer hybrid MoE model (30 gated-DeltaNet + 10 "
+                               "full-attention layers, 256 experts top-8 + shared, 4-bit), 8-bit KV at context %d, bf16 LM "
+                               "head over 248,320, tiled top-k sampler; batch %d, one HIP graph per step" % (context, B),
+                   "batch": B, "context": context, "bytes_per_token_MB": round(bpt / 1e6, 1),
+                   "roofline_tok_per_s_at_8TBps": round(HBM_PEAK_GBPS * 1e9 / bpt, 1),
+                   "eager_ms_per_step": round(dt_eager * 1e3, 3)},
+        "roofline": {"kernel": "whole step (all kernels of one graph replay)", "bound": "hbm", "achieved": round(gbps, 2),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "traffic_source": None, "bytes_per_launch": round(bpt * B), "avg_launch_us": round(dt * 1e6, 2)},
+        "cpu_baseline": None,
+    }
+
+
 def run_copy(torch, a):
     """A plain copy kernel of known size: 1 GiB read + 1 GiB written per launch."""
     n = 1 << 30
@@ -605,7 +670,8 @@ def main():
         line = (run_prefill(nv, ctx, torch, a) if a.workload == "prefill" else
                 run_attention(nv, ctx, torch, a) if a.workload == "attention" else
                 run_sampler(nv, ctx, torch, a) if a.workload == "sampler" else
-                run_greedy(nv, ctx, torch, a) if a.workload == "greedy" else run_copy(torch, a))
+                run_greedy(nv, ctx, torch, a) if a.workload == "greedy" else
+                run_step(nv, ctx, torch, a) if a.workload == "step" else run_copy(torch, a))
         print(json.dumps(line), flush=True)
         return
     layers, stride = build_layers(nv, ctx, torch, a.bits, a.layers)
@@ -673,8 +739,8 @@ def decode_line(a, r, bits, batch, steps, warmup):
 def extra_cells(nv, ctx, torch, a, layers8, stride8):
     """The other cells of the metric, each measured like its own --workload line but shorter:
     4-bit decode at batch 32, 8-bit decode at one token, the configs[2] prefill grouped GEMM, and
-    configs[3] attention at 128K x 8 and 32K x 1 with 8- and 4-bit KV (each checked against the
-    oracle before it is reported)."""
+    configs[4] (the full 40-layer decode step, tok/s at batch 1 and 16), and configs[3] attention at
+    128K x 8 and 32K x 1 with 8- and 4-bit KV (each checked against the oracle before it is reported)."""
     import argparse
     out = {}
     r = run_config(nv, ctx, torch, layers8, stride8, 8, 1, 200, 20, profile=True)
@@ -689,6 +755,15 @@ def extra_cells(nv, ctx, torch, a, layers8, stride8):
     sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.tokens = True, 30, 5, 4, 4096
     out["prefill_4bit_4096tokens"] = compact(run_prefill(nv, ctx, torch, sub))
     torch.cuda.empty_cache()
+    for batch in (1, 16):
+        sub = argparse.Namespace(**vars(a))
+        sub.no_cpu, sub.steps, sub.warmup, sub.batch, sub.context = True, 30, 3, batch, 32768
+        cell = run_step(nv, ctx, torch, sub)
+        c = compact(cell)
+        c["bytes_per_token_MB"] = cell["config"]["bytes_per_token_MB"]
+        c["roofline_tok_per_s_at_8TBps"] = cell["config"]["roofline_tok_per_s_at_8TBps"]
+        out["decode_step_configs4_batch%d" % batch] = c
+        torch.cuda.empty_cache()
     for bits in (8, 4):
         for context, batch in ((131072, 8), (32768, 1)):
             sub = argparse.Namespace(**vars(a))

@@ -116,7 +116,7 @@ int nvmai_hip_dequantize_affine(nvmai_hip_ctx* ctx, nvmai_stream stream, const u
  * (DequantInt4GEMV.swift:66-110, DequantInt8GEMV.swift:50-86, AffineQuant.swift:58)
  * and, with y_f32 != NULL, nvmai_int4_affine_gemv (nvmai_kernels.h:22-28):
  * y[t, :] = W x[t, :] for n_tokens inputs.  y (activations) or y_f32 may be NULL.
- * More than four inputs against a matrix of 1024 rows or more, 16-bit outputs only and 16-byte
+ * More than four inputs against a matrix of 32,768 rows or more (more than 32 inputs: 1024 rows), 16-bit outputs only and 16-byte
  * aligned operands: runs as nvmai_hip_affine_qmm (the matrix is read once for all inputs).
  * bits == 16: `weights` holds dense BF16 rows [m, n] (scales and biases unused, may be NULL; the
  * BF16 LM head): a BF16 context only, n a multiple of 64 and at most 4096, any number of inputs
@@ -510,6 +510,20 @@ int nvmai_hip_lm_head_greedy(nvmai_hip_ctx* ctx, nvmai_stream stream, const void
 int nvmai_hip_residual_add_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, void* hidden, uint32_t hidden_stride,
                                    const void* delta, uint32_t delta_stride, const uint16_t* weight, void* out,
                                    uint32_t out_stride, uint32_t rows, uint32_t d, float eps);
+
+/* The epilogue of the q / k / v projection of a full-attention layer in one launch:
+ * Elementwise.encodeSplitQGate + RMSNorm.encodeBF16WPerHead (q, k) + RoPE.encodeNeoxSubdim (q, k)
+ * (RealForwardRunner.swift:2213-2255), or with q_packed = 0 and v_norm = 1 the reference's own
+ * FusedQKVEpilogue (fused.metal:72-162).  proj: [tokens, proj_stride] activations, per token the q
+ * heads (packed [q ; gate] pairs of 2 head_dim when q_packed), then the k heads, then the v heads, as the
+ * fused projection writes them.  q_out, gate_out: [tokens, num_q_heads, head_dim]; k_out, v_out:
+ * [tokens, kv_stride] stage rows for nvmai_hip_kv_quantize_affine.  positions: device array of one
+ * position per token, or NULL = `position` for all.  Same bits as the separate calls.  head_dim <= 512. */
+int nvmai_hip_attn_qkv_epilogue(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* proj, uint32_t proj_stride,
+                                int q_packed, const uint16_t* q_weight, const uint16_t* k_weight, void* q_out,
+                                void* gate_out, void* k_out, void* v_out, uint32_t kv_stride, uint32_t tokens,
+                                uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t head_dim, uint32_t rotary_dim,
+                                int v_norm, const uint32_t* positions, uint32_t position, float theta, float eps);
 
 /* ---- gated-DeltaNet linear attention ------------------------------------------------------- */
 

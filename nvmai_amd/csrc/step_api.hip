@@ -4,6 +4,15 @@
 
 using namespace nvmai;
 
+namespace {
+// Rows travel through LDS when they can be moved 16 bytes at a time: four rows and the weight, 10 d bytes.
+bool rms_staged_ok(const void* a, uint32_t a_stride, const void* b, uint32_t b_stride, const void* c, uint32_t c_stride,
+                   const void* weight, uint32_t d) {
+    return d % 8 == 0 && d <= 6144 && aligned16(a) && a_stride % 8 == 0 && (!b || (aligned16(b) && b_stride % 8 == 0)) &&
+           aligned16(c) && c_stride % 8 == 0 && (!weight || aligned16(weight));
+}
+}  // namespace
+
 extern "C" int nvmai_hip_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* x, uint32_t x_stride,
                                  const uint16_t* weight, void* out, uint32_t out_stride, uint32_t rows,
                                  uint32_t d, float eps) {
@@ -11,10 +20,16 @@ extern "C" int nvmai_hip_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const 
     if (rows == 0) return NVMAI_OK;
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((rows + 3) / 4);
-    if (ctx->act == ACT_BF16)
-        rmsnorm_kernel<ACT_BF16><<<grid, 256, 0, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);
-    else
-        rmsnorm_kernel<ACT_FP16><<<grid, 256, 0, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);
+    const bool staged = rms_staged_ok(x, x_stride, nullptr, 0, out, out_stride, weight, d);
+    const size_t lds = staged ? (size_t)d * 10 : 0;
+#define NVMAI_RMS(ACT)                                                                                              \
+    do {                                                                                                            \
+        if (staged && d == 2048) rmsnorm_kernel<ACT, true, 2048><<<grid, 256, lds, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps); \
+        else if (staged) rmsnorm_kernel<ACT, true, 0><<<grid, 256, lds, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps); \
+        else rmsnorm_kernel<ACT, false, 0><<<grid, 256, 0, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);        \
+    } while (0)
+    if (ctx->act == ACT_BF16) NVMAI_RMS(ACT_BF16); else NVMAI_RMS(ACT_FP16);
+#undef NVMAI_RMS
     return launch_status();
 }
 
@@ -27,12 +42,42 @@ extern "C" int nvmai_hip_residual_add_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream s
     if (rows == 0) return NVMAI_OK;
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((rows + 3) / 4);
-    if (ctx->act == ACT_BF16)
-        residual_add_rmsnorm_kernel<ACT_BF16><<<grid, 256, 0, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta,
-                                                                   delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);
-    else
-        residual_add_rmsnorm_kernel<ACT_FP16><<<grid, 256, 0, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta,
-                                                                   delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);
+    const bool staged = rms_staged_ok(hidden, hidden_stride, delta, delta_stride, out, out_stride, weight, d);
+    const size_t lds = staged ? (size_t)d * 10 : 0;
+#define NVMAI_RES(ACT)                                                                                              \
+    do {                                                                                                            \
+        if (staged && d == 2048) residual_add_rmsnorm_kernel<ACT, true, 2048><<<grid, 256, lds, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta, delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps); \
+        else if (staged) residual_add_rmsnorm_kernel<ACT, true, 0><<<grid, 256, lds, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta, delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps); \
+        else residual_add_rmsnorm_kernel<ACT, false, 0><<<grid, 256, 0, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta, delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);        \
+    } while (0)
+    if (ctx->act == ACT_BF16) NVMAI_RES(ACT_BF16); else NVMAI_RES(ACT_FP16);
+#undef NVMAI_RES
+    return launch_status();
+}
+
+extern "C" int nvmai_hip_attn_qkv_epilogue(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* proj,
+                                           uint32_t proj_stride, int q_packed, const uint16_t* q_weight,
+                                           const uint16_t* k_weight, void* q_out, void* gate_out, void* k_out,
+                                           void* v_out, uint32_t kv_stride, uint32_t tokens, uint32_t num_q_heads,
+                                           uint32_t num_kv_heads, uint32_t head_dim, uint32_t rotary_dim, int v_norm,
+                                           const uint32_t* positions, uint32_t position, float theta, float eps) {
+    if (!ctx || !proj || !q_out || !k_out || !v_out || (q_packed && !gate_out)) return NVMAI_ERR_INVALID_ARG;
+    if (head_dim == 0 || head_dim > 512 || num_q_heads == 0 || num_kv_heads == 0) return NVMAI_ERR_INVALID_ARG;   // kFusedMaxHeadDim
+    if (rotary_dim > head_dim || (rotary_dim & 1u)) return NVMAI_ERR_INVALID_ARG;
+    const uint32_t span = (q_packed ? 2u : 1u) * num_q_heads * head_dim + 2u * num_kv_heads * head_dim;
+    if (proj_stride < span || kv_stride < num_kv_heads * head_dim) return NVMAI_ERR_INVALID_ARG;
+    if (tokens == 0) return NVMAI_OK;
+    QkvEpilogueParams p{};
+    p.proj = (const uint16_t*)proj; p.proj_stride = proj_stride; p.q_packed = q_packed ? 1u : 0u;
+    p.q_weight = q_weight; p.k_weight = k_weight;
+    p.q_out = (uint16_t*)q_out; p.gate_out = (uint16_t*)gate_out; p.k_out = (uint16_t*)k_out; p.v_out = (uint16_t*)v_out;
+    p.kv_stride = kv_stride; p.tokens = tokens; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads;
+    p.head_dim = head_dim; p.rotary_dim = rotary_dim; p.v_norm = v_norm ? 1u : 0u;
+    p.positions = positions; p.position0 = position; p.theta = theta; p.eps = eps;
+    const dim3 grid((num_q_heads + 2 * num_kv_heads + 3) / 4, tokens);
+    hipStream_t s = (hipStream_t)stream;
+    if (ctx->act == ACT_BF16) qkv_epilogue_kernel<ACT_BF16><<<grid, 256, 0, s>>>(p);
+    else qkv_epilogue_kernel<ACT_FP16><<<grid, 256, 0, s>>>(p);
     return launch_status();
 }
 

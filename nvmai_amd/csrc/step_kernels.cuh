@@ -23,56 +23,199 @@ __device__ __forceinline__ float rms_inverse(float sum, uint32_t d, float eps) {
     return __fdiv_rn(1.0f, sqrtf(__fadd_rn(mean, eps)));     // sqrtf: correctly rounded (the _rn intrinsic is not)
 }
 
-template <int ACT>
-__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* x, uint32_t x_stride, const uint16_t* weight,
-                                                      uint16_t* out, uint32_t out_stride, uint32_t rows, uint32_t d,
-                                                      float eps) {
-    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;                       // uniform per wave
-    const uint32_t lane = threadIdx.x & 63;
-    const uint16_t* xr = x + (size_t)row * x_stride;
+// One wave per row.  STAGED: the row travels through LDS -- 16-byte loads in, the per-lane sums
+// and products read and written two bytes at a time there, 16-byte stores out -- so that a lane's
+// 32 strided elements of a 2048-wide row are not 32 dependent trips to memory (23 us per row that
+// way, a few us staged); the arithmetic and its order are the same either way.  delta != nullptr:
+// the row is first replaced by round(row + delta) (the residual add, utility.metal:95-104) and
+// stored back.  Rows need 16-byte alignment and d a multiple of 8 for the staged form (the entry
+// point checks); lds holds 4 rows of d elements.
+// DFIX: the row length when it is known at compile time (the loops then unroll and a lane's
+// LDS reads are all in flight together), 0 = any.
+template <int ACT, bool STAGED, int DFIX>
+__device__ __forceinline__ void rms_row(uint16_t* xr, const uint16_t* dr, const uint16_t* weight, uint16_t* o,
+                                        uint32_t d_any, float eps, uint16_t* row_s, uint32_t lane) {
+    const uint32_t d = DFIX ? (uint32_t)DFIX : d_any;
+    if (STAGED) {
+        for (uint32_t c = lane; c < d / 8; c += 64) {
+            uint4 v = *reinterpret_cast<const uint4*>(xr + c * 8);
+            if (dr) {
+                const uint4 dl = *reinterpret_cast<const uint4*>(dr + c * 8);
+                uint32_t* vv = reinterpret_cast<uint32_t*>(&v);
+                const uint32_t* dd = reinterpret_cast<const uint32_t*>(&dl);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float a0, a1, b0, b1;
+                    act2_to_f32<ACT>(vv[j], a0, a1);
+                    act2_to_f32<ACT>(dd[j], b0, b1);
+                    vv[j] = (uint32_t)f32_to_act<ACT>(__fadd_rn(a0, b0)) | ((uint32_t)f32_to_act<ACT>(__fadd_rn(a1, b1)) << 16);
+                }
+                *reinterpret_cast<uint4*>(xr + c * 8) = v;
+            }
+            *reinterpret_cast<uint4*>(row_s + c * 8) = v;
+        }
+        __builtin_amdgcn_wave_barrier();
+    } else if (dr) {
+        for (uint32_t i = lane; i < d; i += 64)
+            xr[i] = f32_to_act<ACT>(__fadd_rn(act_to_f32<ACT>(xr[i]), act_to_f32<ACT>(dr[i])));
+    }
+    const uint16_t* src = STAGED ? row_s : xr;
     float acc = 0.0f;
+#pragma unroll
     for (uint32_t i = lane; i < d; i += 64) {
-        const float v = act_to_f32<ACT>(xr[i]);
+        const float v = act_to_f32<ACT>(src[i]);
         acc = fmaf(v, v, acc);
     }
     const float inv = rms_inverse(rms_wave_sum(acc), d, eps);
-    uint16_t* o = out + (size_t)row * out_stride;
+    uint16_t* dst = STAGED ? row_s : o;
+#pragma unroll
     for (uint32_t i = lane; i < d; i += 64) {       // in place is fine: a lane rereads only what it writes
-        float v = __fmul_rn(act_to_f32<ACT>(xr[i]), inv);
+        float v = __fmul_rn(act_to_f32<ACT>(src[i]), inv);
         if (weight) v = __fmul_rn(v, bf16_to_f32(weight[i]));
-        o[i] = f32_to_act<ACT>(v);
+        dst[i] = f32_to_act<ACT>(v);
     }
+    if (STAGED) {
+        __builtin_amdgcn_wave_barrier();
+        for (uint32_t c = lane; c < d / 8; c += 64)
+            *reinterpret_cast<uint4*>(o + c * 8) = *reinterpret_cast<const uint4*>(row_s + c * 8);
+    }
+}
+
+// weight_s: the block's copy of the norm weight in LDS (staged form), read two bytes at a time
+template <int ACT, bool STAGED, int DFIX>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* x, uint32_t x_stride, const uint16_t* weight,
+                                                      uint16_t* out, uint32_t out_stride, uint32_t rows, uint32_t d,
+                                                      float eps) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t rms_lds[];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint16_t* w = weight;
+    if (STAGED && weight) {
+        for (uint32_t c = threadIdx.x; c < d / 8; c += 256)
+            *reinterpret_cast<uint4*>(rms_lds + 4 * d + c * 8) = *reinterpret_cast<const uint4*>(weight + c * 8);
+        __syncthreads();
+        w = rms_lds + 4 * d;
+    }
+    const uint32_t row = blockIdx.x * 4 + wave;
+    if (row >= rows) return;                       // uniform per wave, after the block's only barrier
+    // out may be x: the row is complete in LDS (or every lane rereads only its own elements) before it is written
+    rms_row<ACT, STAGED, DFIX>(const_cast<uint16_t*>(x) + (size_t)row * x_stride, nullptr, w, out + (size_t)row * out_stride,
+                         d, eps, rms_lds + wave * d, lane);
 }
 
 // hidden += delta (rounded to the activation type and stored, utility.metal:95-104), then
 // out = RMSNorm(hidden) * weight of the updated row (rmsnorm.metal:64-110): the residual add that
 // ends one block of a layer and the norm that opens the next, in one pass over the row.  Same
 // arithmetic and summation order as the two kernels one after the other.
-template <int ACT>
+template <int ACT, bool STAGED, int DFIX>
 __global__ __launch_bounds__(256) void residual_add_rmsnorm_kernel(uint16_t* hidden, uint32_t hidden_stride,
                                                                    const uint16_t* delta, uint32_t delta_stride,
                                                                    const uint16_t* weight, uint16_t* out,
                                                                    uint32_t out_stride, uint32_t rows, uint32_t d,
                                                                    float eps) {
-    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;                       // uniform per wave
-    const uint32_t lane = threadIdx.x & 63;
-    uint16_t* hr = hidden + (size_t)row * hidden_stride;
-    const uint16_t* dr = delta + (size_t)row * delta_stride;
-    float acc = 0.0f;
-    for (uint32_t i = lane; i < d; i += 64) {
-        const uint16_t sum = f32_to_act<ACT>(__fadd_rn(act_to_f32<ACT>(hr[i]), act_to_f32<ACT>(dr[i])));
-        hr[i] = sum;
-        const float v = act_to_f32<ACT>(sum);
-        acc = fmaf(v, v, acc);
+    extern __shared__ __attribute__((aligned(16))) uint16_t rms_lds[];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint16_t* w = weight;
+    if (STAGED && weight) {
+        for (uint32_t c = threadIdx.x; c < d / 8; c += 256)
+            *reinterpret_cast<uint4*>(rms_lds + 4 * d + c * 8) = *reinterpret_cast<const uint4*>(weight + c * 8);
+        __syncthreads();
+        w = rms_lds + 4 * d;
     }
-    const float inv = rms_inverse(rms_wave_sum(acc), d, eps);
-    uint16_t* o = out + (size_t)row * out_stride;
-    for (uint32_t i = lane; i < d; i += 64) {       // a lane rereads only what it wrote
-        float v = __fmul_rn(act_to_f32<ACT>(hr[i]), inv);
-        if (weight) v = __fmul_rn(v, bf16_to_f32(weight[i]));
-        o[i] = f32_to_act<ACT>(v);
+    const uint32_t row = blockIdx.x * 4 + wave;
+    if (row >= rows) return;                       // uniform per wave, after the block's only barrier
+    rms_row<ACT, STAGED, DFIX>(hidden + (size_t)row * hidden_stride, delta + (size_t)row * delta_stride, w,
+                         out + (size_t)row * out_stride, d, eps, rms_lds + wave * d, lane);
+}
+
+// ---- epilogue of the fused q / k / v projection of a full-attention layer --------------------------
+// One wave per head of one token, replacing split_q_gate + rmsnorm_bf16w_perhead (q, k) + rope_neox_subdim
+// (q, k) (RealForwardRunner.swift:2213-2255; the reference's own fusion of the norm and the rotation is
+// fused_qkv_epilogue, fused.metal:72-162):
+//   q head h:  packed [q ; gate] -> gate copied out, q = rope(round(rmsnorm(q) * q_weight))
+//   k head h:  k = rope(round(rmsnorm(k) * k_weight)) into the K stage row
+//   v head h:  copied into the V stage row (v_norm: RMS norm without weight first, as the
+//              reference's fused kernel has it for models that norm V)
+// The norm is the arithmetic of rmsnorm_kernel (same summation order), the result is rounded to the
+// activation type before the rotation as the separate kernels hand it over, and the rotation is the
+// arithmetic of rope_neox_subdim_kernel: the outputs are the same bits as the five launches.
+struct QkvEpilogueParams {
+    const uint16_t* proj;       // [tokens, proj_stride]: q heads packed [q ; gate], then k heads, then v heads
+    uint32_t proj_stride;
+    uint32_t q_packed;          // 1: q heads are [q ; gate] pairs (2 head_dim each); 0: plain q heads, no gate
+    const uint16_t* q_weight;   // BF16 [head_dim] or NULL
+    const uint16_t* k_weight;
+    uint16_t* q_out;            // [tokens, num_q_heads, head_dim]
+    uint16_t* gate_out;         // [tokens, num_q_heads, head_dim] (q_packed only)
+    uint16_t* k_out;            // [tokens, kv_stride]
+    uint16_t* v_out;
+    uint32_t kv_stride;
+    uint32_t tokens, num_q_heads, num_kv_heads, head_dim, rotary_dim;
+    uint32_t v_norm;
+    const uint32_t* positions;  // one per token, or NULL = position0
+    uint32_t position0;
+    float theta, eps;
+};
+
+template <int ACT>
+__global__ __launch_bounds__(256) void qkv_epilogue_kernel(QkvEpilogueParams p) {
+    __shared__ uint16_t head_s[4][512];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t heads = p.num_q_heads + 2 * p.num_kv_heads;
+    const uint32_t hidx = blockIdx.x * 4 + wave, token = blockIdx.y;
+    if (hidx >= heads) return;                              // wave-uniform; no block-wide barrier below
+    const uint32_t hd = p.head_dim;
+    const bool is_q = hidx < p.num_q_heads, is_k = !is_q && hidx < p.num_q_heads + p.num_kv_heads;
+    const uint32_t q_span = p.q_packed ? 2 * hd : hd;
+    const uint16_t* src;
+    uint16_t* dst;
+    const uint16_t* w = nullptr;
+    if (is_q) {
+        src = p.proj + (size_t)token * p.proj_stride + hidx * q_span;
+        dst = p.q_out + ((size_t)token * p.num_q_heads + hidx) * hd;
+        w = p.q_weight;
+        if (p.q_packed) {
+            uint16_t* g = p.gate_out + ((size_t)token * p.num_q_heads + hidx) * hd;
+            for (uint32_t i = lane; i < hd; i += 64) g[i] = src[hd + i];
+        }
+    } else {
+        const uint32_t kvh = hidx - p.num_q_heads - (is_k ? 0 : p.num_kv_heads);
+        src = p.proj + (size_t)token * p.proj_stride + p.num_q_heads * q_span + (is_k ? 0 : p.num_kv_heads * hd) + kvh * hd;
+        dst = (is_k ? p.k_out : p.v_out) + (size_t)token * p.kv_stride + kvh * hd;
+        w = is_k ? p.k_weight : nullptr;
+    }
+    uint16_t* hs = head_s[wave];
+    const bool norm = is_q || is_k || p.v_norm;
+    if (norm) {
+        float acc = 0.0f;
+        for (uint32_t i = lane; i < hd; i += 64) {
+            const float v = act_to_f32<ACT>(src[i]);
+            acc = fmaf(v, v, acc);
+        }
+        const float inv = rms_inverse(rms_wave_sum(acc), hd, p.eps);
+        for (uint32_t i = lane; i < hd; i += 64) {
+            float v = __fmul_rn(act_to_f32<ACT>(src[i]), inv);
+            if (w) v = __fmul_rn(v, bf16_to_f32(w[i]));
+            hs[i] = f32_to_act<ACT>(v);
+        }
+    } else {
+        for (uint32_t i = lane; i < hd; i += 64) hs[i] = src[i];
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xC07F);                      // lgkmcnt(0): this wave's LDS writes have landed
+    const uint32_t half_rot = (is_q || is_k) ? p.rotary_dim / 2 : 0;
+    const uint32_t pos = p.positions ? p.positions[token] : p.position0;
+    for (uint32_t i = lane; i < hd; i += 64) {
+        uint16_t o = hs[i];
+        if (i < 2 * half_rot) {
+            const uint32_t pair = i < half_rot ? i : i - half_rot;
+            const float exponent = __fdiv_rn(-(float)(2u * pair), (float)p.rotary_dim);
+            const float angle = __fmul_rn((float)pos, powf(p.theta, exponent));
+            const float c = cosf(angle), s = sinf(angle);
+            const float x0 = act_to_f32<ACT>(hs[pair]), x1 = act_to_f32<ACT>(hs[half_rot + pair]);
+            o = i < half_rot ? f32_to_act<ACT>(__fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s)))
+                             : f32_to_act<ACT>(__fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c)));
+        }
+        dst[i] = o;
     }
 }
 

@@ -1,0 +1,267 @@
+"""Decode step of the hybrid MoE model over the C ABI: the host-side counterpart of
+RealForwardRunner.step (RealForwardRunner.swift:1820-2050) for experts resident in HBM.
+
+A layer is: input RMSNorm -> attention branch (gated-DeltaNet linear attention, or full attention
+with an output gate over a quantized KV cache; RealForwardRunner.swift:2066-2131, 2178-2283) ->
+residual add -> post-attention RMSNorm -> MoE block (router, shared expert, routed experts) ->
+residual add; then the final norm, the LM head, softmax and the sampler.  Every call only enqueues
+kernels on the current stream, so a whole step can be captured into a HIP graph and replayed.
+
+Weights are laid out for one launch per projection group: the four input projections of a linear
+layer (qkv, z, a, b) and the three of a full-attention layer (packed q / gate, k, v) are rows of one
+matrix each.
+"""
+import ctypes as C
+
+import torch
+
+from . import ops
+from ._lib import check, lib
+
+
+class HybridConfig:
+    """The architecture fields the step reads (ArchConfig, ModelTypes.swift:48-204)."""
+
+    def __init__(self, hidden=2048, layers=40, full_every=4, num_heads=16, num_kv_heads=2, head_dim=256,
+                 rotary_dim=64, rope_theta=1e7, gdn=(16, 32, 128, 128, 4), num_experts=256, top_k=8,
+                 moe_intermediate=512, vocab=248320, expert_bits=4, attn_bits=4, kv_bits=8, head_bits=16,
+                 embed_bits=4, rms_eps=1e-6, logit_softcap=0.0, gdn_state_bf16=True):
+        self.hidden, self.layers, self.full_every = hidden, layers, full_every
+        self.num_heads, self.num_kv_heads, self.head_dim = num_heads, num_kv_heads, head_dim
+        self.rotary_dim, self.rope_theta, self.gdn = rotary_dim, rope_theta, gdn
+        self.num_experts, self.top_k, self.moe_intermediate, self.vocab = num_experts, top_k, moe_intermediate, vocab
+        self.expert_bits, self.attn_bits, self.kv_bits = expert_bits, attn_bits, kv_bits
+        self.head_bits, self.embed_bits = head_bits, embed_bits
+        self.rms_eps, self.logit_softcap, self.gdn_state_bf16 = rms_eps, logit_softcap, gdn_state_bf16
+
+    def is_linear(self, layer):
+        """layerIsLinear: every full_every-th layer is full attention, the others gated DeltaNet."""
+        return (layer + 1) % self.full_every != 0
+
+    @property
+    def q_dim(self):
+        return self.num_heads * self.head_dim
+
+    @property
+    def kv_dim(self):
+        return self.num_kv_heads * self.head_dim
+
+    @property
+    def gdn_qkv_dim(self):
+        kh, vh, dk, dv, _ = self.gdn
+        return 2 * kh * dk + vh * dv
+
+    @property
+    def gdn_value_dim(self):
+        return self.gdn[1] * self.gdn[3]
+
+    def bytes_per_token(self, batch=1, context=32768):
+        """Algorithmic HBM bytes of one decode step divided by the batch: every weight the step
+        touches once (routed experts: the expected number of distinct ones for uniform routing), the
+        recurrent states read and written, the KV rows read."""
+        D, F, E, k = self.hidden, self.moe_intermediate, self.num_experts, self.top_k
+        mat = lambda rows, cols, bits: rows * cols * bits / 8 + (0 if bits == 16 else 2 * rows * (cols // 64) * 2)
+        expert = 2 * mat(F, D, self.expert_bits) + mat(D, F, self.expert_bits)
+        distinct = E * (1.0 - (1.0 - k / E) ** batch)
+        moe = (distinct + 1) * expert + E * D * 2 + mat(1, D, 8)
+        kh, vh, dk, dv, taps = self.gdn
+        lin = mat(self.gdn_qkv_dim + self.gdn_value_dim + 2 * vh, D, self.attn_bits) + mat(D, self.gdn_value_dim, self.attn_bits) \
+            + self.gdn_qkv_dim * taps * 2
+        lin_state = batch * 2 * vh * dv * dk * (2 if self.gdn_state_bf16 else 4)
+        full = mat(2 * self.q_dim + 2 * self.kv_dim, D, self.attn_bits) + mat(D, self.q_dim, self.attn_bits)
+        kv_stride = ops.kv_row_layout(self.kv_dim, self.kv_bits)[0]
+        kv = batch * context * 2 * kv_stride
+        n_lin = sum(self.is_linear(L) for L in range(self.layers))
+        n_full = self.layers - n_lin
+        total = self.layers * moe + n_lin * (lin + lin_state) + n_full * (full + kv) + mat(self.vocab, D, self.head_bits)
+        return total / batch
+
+
+def _randn(gen, shape, std, device):
+    return torch.empty(shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen).to(torch.bfloat16)
+
+
+class HybridWeights:
+    """Random-init weights of the model, quantized on the device by the library's own quantizer
+    (the same bits as the reference's quantizer gives for the same values)."""
+
+    def __init__(self, ctx, cfg, seed=1234, std=0.02):
+        self.ctx, self.cfg = ctx, cfg
+        dev = ctx.device
+        gen = torch.Generator(device=dev).manual_seed(seed)
+        D = cfg.hidden
+        q = lambda rows, cols, bits, s=std: ops.quantize_affine(ctx, _randn(gen, (rows, cols), s, dev), bits)
+        normw = lambda n: torch.empty(n, dtype=torch.float32, device=dev).uniform_(0.8, 1.2, generator=gen) \
+            .to(torch.bfloat16).view(torch.int16)
+        self.embed = q(cfg.vocab, D, cfg.embed_bits, 1.0)
+        self.final_norm = normw(D)
+        if cfg.head_bits == 16:
+            self.lm_head = (_randn(gen, (cfg.vocab, D), std, dev).view(torch.int16), None, None)
+        else:
+            self.lm_head = q(cfg.vocab, D, cfg.head_bits)
+        off, stride = ops.expert_offsets(D, cfg.moe_intermediate, cfg.expert_bits)
+        self.layers = []
+        kh, vh, dk, dv, taps = cfg.gdn
+        for L in range(cfg.layers):
+            w = dict(in_norm=normw(D), post_norm=normw(D))
+            if cfg.is_linear(L):
+                rows = cfg.gdn_qkv_dim + cfg.gdn_value_dim + 2 * vh
+                w["in_proj"] = q(rows, D, cfg.attn_bits)
+                w["conv_w"] = torch.empty((cfg.gdn_qkv_dim, taps), dtype=torch.float32, device=dev) \
+                    .uniform_(-0.4, 0.4, generator=gen).to(torch.bfloat16).view(torch.int16)
+                u = lambda lo, hi, n: torch.empty(n, dtype=torch.float32, device=dev).uniform_(lo, hi, generator=gen) \
+                    .to(torch.bfloat16).view(torch.int16)
+                w["a_log"], w["dt_bias"], w["gdn_norm"] = u(-1.0, 1.5, vh), u(-0.5, 0.5, vh), u(0.5, 1.5, dv)
+                w["out_proj"] = q(D, cfg.gdn_value_dim, cfg.attn_bits)
+            else:
+                w["qkv"] = q(2 * cfg.q_dim + 2 * cfg.kv_dim, D, cfg.attn_bits)
+                w["q_norm"], w["k_norm"] = normw(cfg.head_dim), normw(cfg.head_dim)
+                w["o_proj"] = q(D, cfg.q_dim, cfg.attn_bits)
+            pool = torch.empty((cfg.num_experts + 1, stride), dtype=torch.uint8, device=dev)
+            F = cfg.moe_intermediate
+            for (rows, n, wo, so, bo) in ((F, D, off.gate_w, off.gate_s, off.gate_b), (F, D, off.up_w, off.up_s, off.up_b),
+                                          (D, F, off.down_w, off.down_s, off.down_b)):
+                p_, s_, b_ = q((cfg.num_experts + 1) * rows, n, cfg.expert_bits)
+                wb, mb = rows * n * cfg.expert_bits // 8, rows * n // 32
+                pool[:, wo:wo + wb] = p_.view(cfg.num_experts + 1, wb)
+                pool[:, so:so + mb] = s_.view(torch.uint8).view(cfg.num_experts + 1, mb)
+                pool[:, bo:bo + mb] = b_.view(torch.uint8).view(cfg.num_experts + 1, mb)
+                del p_, s_, b_
+            w["pool"] = pool
+            w["router"] = _randn(gen, (cfg.num_experts, D), std, dev).view(torch.int16)
+            w["gate"] = q(1, D, 8)
+            w["moe"] = ops.moe_layer_desc(D, F, cfg.num_experts, cfg.top_k, cfg.expert_bits,
+                                          ops.rows_desc(16, w["router"]), pool[:cfg.num_experts], pool[cfg.num_experts],
+                                          ops.rows_desc(8, *w["gate"]))
+            self.layers.append(w)
+
+
+class HybridDecoder:
+    """One decode step for `batch` sequences: buffers, recurrent states and KV caches are allocated
+    once; step() only enqueues kernels."""
+
+    def __init__(self, ctx, cfg, weights, batch=1, max_context=32768):
+        self.ctx, self.cfg, self.w, self.batch = ctx, cfg, weights, batch
+        dev, dt = ctx.device, ctx.dtype
+        D = cfg.hidden
+        buf = lambda *shape: torch.zeros(shape, dtype=dt, device=dev)
+        self.hidden, self.normed, self.branch = buf(batch, D), buf(batch, D), buf(batch, D)
+        self.moe_out = buf(batch, D)
+        kh, vh, dk, dv, taps = cfg.gdn
+        self.gdn = ops.GDN(ctx, kh, vh, dk, dv, taps)
+        self.lin_rows = cfg.gdn_qkv_dim + cfg.gdn_value_dim + 2 * vh
+        self.lin_proj, self.conv_out, self.gdn_out = buf(batch, self.lin_rows), buf(batch, cfg.gdn_qkv_dim), buf(batch, cfg.gdn_value_dim)
+        self.full_rows = 2 * cfg.q_dim + 2 * cfg.kv_dim
+        self.full_proj = buf(batch, self.full_rows)
+        self.q, self.gate, self.attn_out = buf(batch, cfg.num_heads, cfg.head_dim), buf(batch, cfg.num_heads, cfg.head_dim), \
+            buf(batch, cfg.num_heads, cfg.head_dim)
+        self.k_stage, self.v_stage = buf(batch, cfg.kv_dim), buf(batch, cfg.kv_dim)
+        self.logits = buf(batch, cfg.vocab)
+        self.probs = torch.zeros((batch, cfg.vocab), dtype=torch.float16, device=dev)
+        self.tokens = torch.zeros(batch, dtype=torch.int32, device=dev)
+        self.next_tokens = torch.zeros(batch, dtype=torch.int32, device=dev)
+        self.positions = torch.zeros(batch, dtype=torch.int32, device=dev)
+        self.gdn_states, self.kv = {}, {}
+        for L in range(cfg.layers):
+            if cfg.is_linear(L):
+                self.gdn_states[L] = self.gdn.new_state(batch, bf16=cfg.gdn_state_bf16)
+            else:
+                self.kv[L] = (ops.KVCache(batch, max_context, cfg.kv_dim, cfg.kv_bits, dev),
+                              ops.KVCache(batch, max_context, cfg.kv_dim, cfg.kv_bits, dev))
+        self.moe = ops.MoE(ctx, cfg.expert_bits)
+        self.attn = ops.Attention(ctx)
+        self.quant = ops.KVCacheQuantizer(ctx)
+        self.softmax = ops.LogitSoftcapSoftmaxTiled(ctx, cfg.vocab)
+        self.sampler = ops.SampleTopK64(ctx, cfg.vocab) if cfg.vocab <= 262144 else None
+        self.ew = ops.Elementwise(ctx)
+
+    # -- attention branches ---------------------------------------------------------------------
+    def _linear_attention(self, L, w):
+        cfg, B = self.cfg, self.batch
+        vh = cfg.gdn[1]
+        p_, s_, b_ = w["in_proj"]
+        ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, self.normed, self.lin_rows, cfg.hidden, y=self.lin_proj)
+        qkv = self.lin_proj[:, :cfg.gdn_qkv_dim]
+        z = self.lin_proj[:, cfg.gdn_qkv_dim:cfg.gdn_qkv_dim + cfg.gdn_value_dim]
+        a = self.lin_proj[:, cfg.gdn_qkv_dim + cfg.gdn_value_dim:cfg.gdn_qkv_dim + cfg.gdn_value_dim + vh]
+        b = self.lin_proj[:, cfg.gdn_qkv_dim + cfg.gdn_value_dim + vh:]
+        tail, state = self.gdn_states[L]
+        g = self.gdn
+        check(lib.nvmai_hip_gdn_conv_norm(self.ctx.handle, ops._stream(), C.byref(g.cfg), ops._ptr(qkv), self.lin_rows,
+                                          ops._ptr(tail), ops._ptr(w["conv_w"]), ops._ptr(self.conv_out),
+                                          cfg.gdn_qkv_dim, 1, B), "gdn_conv_norm")
+        check(lib.nvmai_hip_gdn_delta_gated_norm(self.ctx.handle, ops._stream(), C.byref(g.cfg), ops._ptr(self.conv_out),
+                                                 cfg.gdn_qkv_dim, ops._ptr(a), ops._ptr(b), self.lin_rows,
+                                                 ops._ptr(w["a_log"]), ops._ptr(w["dt_bias"]), ops._ptr(state),
+                                                 int(state.dtype == torch.bfloat16), ops._ptr(z), self.lin_rows,
+                                                 ops._ptr(w["gdn_norm"]), ops._ptr(self.gdn_out), cfg.gdn_value_dim, 1, B),
+              "gdn_delta_gated_norm")
+        p_, s_, b_ = w["out_proj"]
+        ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, self.gdn_out, cfg.hidden, cfg.gdn_value_dim, y=self.branch)
+
+    def _full_attention(self, L, w, position):
+        cfg, B = self.cfg, self.batch
+        p_, s_, b_ = w["qkv"]
+        ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, self.normed, self.full_rows, cfg.hidden, y=self.full_proj)
+        check(lib.nvmai_hip_attn_qkv_epilogue(self.ctx.handle, ops._stream(), ops._ptr(self.full_proj), self.full_rows, 1,
+                                              ops._ptr(w["q_norm"]), ops._ptr(w["k_norm"]), ops._ptr(self.q),
+                                              ops._ptr(self.gate), ops._ptr(self.k_stage), ops._ptr(self.v_stage),
+                                              cfg.kv_dim, B, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim,
+                                              cfg.rotary_dim, 0, None, position, cfg.rope_theta, cfg.rms_eps),
+              "attn_qkv_epilogue")
+        kc, vc = self.kv[L]
+        # one row per sequence, all at `position`: a view whose row pitch is the distance between sequences
+        for cache, stage in ((kc, self.k_stage), (vc, self.v_stage)):
+            view = cache.view(0, position)
+            view.stride = cache.batch_stride
+            self.quant.encode(stage, cfg.kv_dim, view, B, cfg.kv_dim)
+        self.attn.encode_full(self.q, kc, vc, cfg.head_dim, cfg.num_heads, cfg.num_kv_heads, position + 1,
+                              out=self.attn_out)
+        self.ew.encode_sigmoid_gate_mul(self.attn_out, self.gate)
+        p_, s_, b_ = w["o_proj"]
+        ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, self.attn_out.view(B, cfg.q_dim), cfg.hidden, cfg.q_dim,
+                        y=self.branch)
+
+    # -- the step ---------------------------------------------------------------------------------
+    def forward_hidden(self, position):
+        """Embedding lookup of self.tokens through the last layer; leaves the final-normed rows in
+        self.normed.  `position` is the index of these tokens in their sequences."""
+        cfg, ctx = self.cfg, self.ctx
+        e_p, e_s, e_b = self.w.embed
+        check(lib.nvmai_hip_embed_lookup(ctx.handle, ops._stream(), ops._ptr(e_p), ops._ptr(e_s), ops._ptr(e_b),
+                                         cfg.embed_bits, ops._ptr(self.tokens), 0, self.batch, ops._ptr(self.hidden),
+                                         cfg.hidden, cfg.hidden, cfg.vocab, 1.0), "embed_lookup")
+        ops.RMSNorm(ctx).encode_bf16w(self.hidden, self.w.layers[0]["in_norm"], out=self.normed, eps=cfg.rms_eps)
+        for L, w in enumerate(self.w.layers):
+            if cfg.is_linear(L):
+                self._linear_attention(L, w)
+            else:
+                self._full_attention(L, w, position)
+            ops.residual_add_rmsnorm(ctx, self.hidden, self.branch, w["post_norm"], out=self.normed, eps=cfg.rms_eps)
+            self.moe.decode_layer(w["moe"], self.normed, self.moe_out)
+            nxt = self.w.layers[L + 1]["in_norm"] if L + 1 < cfg.layers else self.w.final_norm
+            ops.residual_add_rmsnorm(ctx, self.hidden, self.moe_out, nxt, out=self.normed, eps=cfg.rms_eps)
+        return self.normed
+
+    def head(self):
+        """LM head over the final-normed rows: logits in self.logits."""
+        cfg = self.cfg
+        p_, s_, b_ = self.w.lm_head
+        ops.affine_gemv(self.ctx, p_, s_, b_, cfg.head_bits, self.normed, cfg.vocab, cfg.hidden, y=self.logits)
+        return self.logits
+
+    def sample(self, seeds, temperature=0.6, top_k=20, top_p=0.95):
+        """Softcap + softmax and the tiled top-k sampler (Sampler.sample's production path): tokens in
+        self.next_tokens."""
+        self.softmax.encode(self.logits, self.probs, softcap=self.cfg.logit_softcap)
+        check(lib.nvmai_hip_sample_topk64(self.ctx.handle, ops._stream(), ops._ptr(self.probs), self.probs.stride(0),
+                                          self.batch, self.cfg.vocab, temperature, top_p,
+                                          (C.c_uint64 * self.batch)(*seeds), top_k, ops._ptr(self.next_tokens), None),
+              "sample_topk64")
+        return self.next_tokens
+
+    def step(self, position, seeds, temperature=0.6, top_k=20, top_p=0.95):
+        """tokens (self.tokens) at `position` -> next tokens (self.next_tokens)."""
+        self.forward_hidden(position)
+        self.head()
+        return self.sample(seeds, temperature, top_k, top_p)
