@@ -36,18 +36,23 @@ def parse():
     ap.add_argument("--sweep", action="store_true", help="also print batch/bits sweep lines to stderr")
     ap.add_argument("--no-extra", action="store_true", help="skip the `extra` object (the other cells of the metric) "
                     "that the default invocation appends")
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "sampler", "greedy", "step", "copy"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "prefill_attention", "sampler", "greedy", "step", "copy"],
                     help="decode = configs[1] (the headline line); prefill = configs[2] grouped GEMM; "
-                         "attention = configs[3] quantized-KV decode attention; sampler = the end of configs[4]: "
+                         "attention = configs[3] quantized-KV decode attention; prefill_attention = causal attention of --tokens queries "
+                         "at the end of a --context cache; sampler = the end of configs[4]: "
                          "quantized LM head GEMV over 248,320 rows, tiled softmax, top-k sampler; greedy = the fused greedy LM head "
                          "(RMSNorm + logits in a fixed order + argmax) over the same head; step = configs[4], the full 40-layer decode "
                          "step (tok/s at --batch 1..16, KV at --context); copy = a plain 1 GiB device copy, "
                          "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated on")
-    ap.add_argument("--context", type=int, default=32768, help="attention: tokens in the KV cache")
+    ap.add_argument("--context", type=int, default=None, help="attention: tokens in the KV cache (default 32768; "
+                    "prefill_attention: the chunk itself)")
     ap.add_argument("--tokens", type=int, default=4096, help="prefill: tokens per step")
     a = ap.parse_args()
     if a.bits is None:
         a.bits = 4 if a.workload == "prefill" else 8
+    a.context_given = a.context is not None
+    if a.context is None:
+        a.context = 32768
     return a
 
 
@@ -395,6 +400,68 @@ def run_attention(nv, ctx, torch, a):
     }
 
 
+def run_prefill_attention(nv, ctx, torch, a):
+    """The attention half of a configs[2] prefill step: `--tokens` query tokens (16 query / 2 KV
+    heads, head_dim 256) at the end of a quantized KV cache of `--context` tokens (at least the
+    chunk itself), causal.  A step = one PrefillAttention.encodeCausal call."""
+    bits, T = a.bits, a.tokens
+    HQ, HKV, HD = 16, 2, 256
+    kv_valid = max(a.context, T) if a.context_given else T
+    start = kv_valid - T
+    gen = torch.Generator(device="cuda").manual_seed(37)
+    quant, pa = nv.KVCacheQuantizer(ctx), nv.PrefillAttention(ctx)
+    kc, vc = nv.KVCache(1, kv_valid, HKV * HD, bits), nv.KVCache(1, kv_valid, HKV * HD, bits)
+    for at in range(0, kv_valid, 8192):
+        n = min(8192, kv_valid - at)
+        for c in (kc, vc):
+            src = torch.empty((n, HKV * HD), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
+            quant.encode(src, HKV * HD, c.view(0, at), n, HKV * HD)
+    q = torch.empty((T, HQ, HD), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
+    out = torch.empty_like(q)
+    call = lambda: pa.encode_causal(q, kc.view(), vc.view(), out, start, T, HD, HQ, HKV, kv_valid)
+    for _ in range(a.warmup):
+        call()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        call()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    ctx.profile_enable(True)
+    for _ in range(a.steps):
+        call()
+    torch.cuda.synchronize()
+    ctx.profile_enable(False)
+    ms, n = ctx.profile_read(nv.PROF_ATTN_PARTIAL)
+    kern_us = ms / max(n, 1) * 1e3
+    import oracle as O
+    kr, vr = kc.rows[0].cpu().numpy(), vc.rows[0].cpu().numpy()
+    rows = sorted({0, 1, T // 2, T - 1}) if kv_valid <= 16384 else [0, T - 1]
+    worst = 0.0
+    for t in rows:                                     # the oracle walks one query's keys in about a second at 128K
+        want = O.attention_prefill_causal(q[t].float().cpu().numpy().reshape(1, -1), kr, vr, bits, HQ, HKV, HD,
+                                          start + t, start + t + 1, 1.0 / 16.0)
+        worst = max(worst, float(O.rel_error(out[t].float().cpu().numpy(), want)))
+    assert worst < 1e-2, "prefill attention differs from the oracle: max-rel %g" % worst
+    pairs = float(sum(min(kv_valid, start + t + 1) for t in range(T)))
+    flops = 4.0 * pairs * HD * HQ                      # q.k and p.v, one multiply-add each per (query, key, head, dim)
+    tf = flops / (kern_us * 1e-6) / 1e12
+    return {
+        "metric": METRIC, "value": round(flops / dt / 1e12, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u%d KV codes, f16 MFMA, f32 softmax" % bits, "data": "synthetic",
+        "config": {"workload": "attention of a configs[2] prefill step: causal, %d query tokens at positions %d..%d, "
+                               "16 query / 2 KV heads, head_dim 256, %d-bit KV" % (T, start, kv_valid - 1, bits),
+                   "tokens_per_s": round(T / dt), "query_key_pairs": pairs},
+        "roofline": {"kernel": "attn_partial_mfma_kernel (causal, %d queries per block)" % (16 // (HQ // HKV)),
+                     "bound": "mfma", "achieved": round(tf, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "flops_per_launch": flops, "avg_launch_us": round(kern_us, 2)},
+        "cpu_baseline": None,
+        "parity_check": {"max_rel": round(worst, 6), "against": "oracle attention_prefill_causal, query rows %s" % rows},
+    }
+
+
 def run_sampler(nv, ctx, torch, a):
     """The end of configs[4]: logits = LM head (4/8-bit affine [248320, 2048]) x hidden, softcap +
     tiled softmax, tiled top-k sampler (k 20, top-p 0.95, T 0.6, fixed seed) for `--batch` rows."""
@@ -669,6 +736,7 @@ def main():
     if a.workload != "decode":
         line = (run_prefill(nv, ctx, torch, a) if a.workload == "prefill" else
                 run_attention(nv, ctx, torch, a) if a.workload == "attention" else
+                run_prefill_attention(nv, ctx, torch, a) if a.workload == "prefill_attention" else
                 run_sampler(nv, ctx, torch, a) if a.workload == "sampler" else
                 run_greedy(nv, ctx, torch, a) if a.workload == "greedy" else
                 run_step(nv, ctx, torch, a) if a.workload == "step" else run_copy(torch, a))
@@ -763,6 +831,11 @@ def extra_cells(nv, ctx, torch, a, layers8, stride8):
         c["bytes_per_token_MB"] = cell["config"]["bytes_per_token_MB"]
         c["roofline_tok_per_s_at_8TBps"] = cell["config"]["roofline_tok_per_s_at_8TBps"]
         out["decode_step_configs4_batch%d" % batch] = c
+        torch.cuda.empty_cache()
+    for bits in (8, 4):
+        sub = argparse.Namespace(**vars(a))
+        sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.tokens, sub.context_given = True, 20, 3, bits, 4096, False
+        out["prefill_attention_%dbit_4096tokens" % bits] = compact(run_prefill_attention(nv, ctx, torch, sub))
         torch.cuda.empty_cache()
     for bits in (8, 4):
         for context, batch in ((131072, 8), (32768, 1)):

@@ -375,6 +375,37 @@ int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream stream, const vo
                                uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
                                uint32_t seq_len, uint32_t kv_start, float scale);
 
+/* The same call for sequences of different lengths: sequence b reads rows
+ * [kv_starts[b], min(seq_lens[b], max_seq_len)) of its cache (kv_starts NULL: from row 0).
+ * seq_lens and kv_starts are device arrays of `batch` words read by the kernels, so a captured
+ * graph follows them; max_seq_len bounds every row the call may touch and sizes the chunking.
+ * The reference issues one encodeFull per sequence (Attention.swift:207-239); an empty range
+ * writes zeros as there. */
+int nvmai_hip_attention_decode_ragged(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
+                                      const nvmai_kv_view* k, const nvmai_kv_view* v,
+                                      uint64_t kv_batch_stride, void* out, uint32_t batch,
+                                      uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                      const uint32_t* seq_lens, const uint32_t* kv_starts,
+                                      uint32_t max_seq_len, float scale);
+
+/* PrefillAttention.encodeCausal on the causalTiled path (PrefillAttention.swift:97-167; kernel
+ * attention_prefill_causal_tiled, prefill.metal:709-830) over fp16, 8-bit or 4-bit K/V rows:
+ * query token t of the chunk (row q + t * q_token_stride elements, [num_q_heads, head_dim]) sits
+ * at absolute position start_position + t and attends to the keys
+ * [first, min(kv_valid_count, start_position + t + 1)), first = max(0, start_position + t + 1 -
+ * sliding_window) when sliding_window != 0, else 0; its output row is out + t * o_token_stride
+ * elements.  kv_ring_capacity != 0: the row of key p is p % kv_ring_capacity (function constant
+ * 76 of the reference).  Errors follow PrefillAttention.validate (PrefillAttention.swift:169-191):
+ * strides below num_q_heads * head_dim, query_count == 0, or start_position + query_count >
+ * kv_valid_count give NVMAI_ERR_INVALID_ARG.  scale <= 0 selects 1/sqrt(head_dim). */
+int nvmai_hip_attention_prefill_causal(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
+                                       uint32_t q_token_stride, const nvmai_kv_view* k,
+                                       const nvmai_kv_view* v, void* out, uint32_t o_token_stride,
+                                       uint32_t start_position, uint32_t query_count,
+                                       uint32_t kv_valid_count, uint32_t sliding_window,
+                                       uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                       uint32_t kv_ring_capacity, float scale);
+
 /* Attention.splitGeometry (Attention.swift:148-168): the reference's chunking of a KV range,
  * reported for callers that size scratch the way it does.  Host arithmetic. */
 int nvmai_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len,

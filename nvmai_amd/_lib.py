@@ -98,6 +98,10 @@ SIGNATURES = {
     "nvmai_hip_rope_neox_subdim": [vp, vp, vp, u32, u32, u32, u32, vp, u32, C.c_float],
     "nvmai_hip_attention_decode": [vp, vp, vp, C.POINTER(KvView), C.POINTER(KvView), u64, vp, u32, u32, u32,
                                    u32, u32, u32, C.c_float],
+    "nvmai_hip_attention_decode_ragged": [vp, vp, vp, C.POINTER(KvView), C.POINTER(KvView), u64, vp, u32, u32, u32,
+                                          u32, vp, vp, u32, C.c_float],
+    "nvmai_hip_attention_prefill_causal": [vp, vp, vp, u32, C.POINTER(KvView), C.POINTER(KvView), vp, u32, u32, u32,
+                                           u32, u32, u32, u32, u32, u32, C.c_float],
     "nvmai_attention_split_geometry": [u32, u32, u32, u32, C.c_int, C.POINTER(u32), C.POINTER(u32),
                                        C.POINTER(u32), C.POINTER(u32)],
     "nvmai_hip_softmax_tiled": [vp, vp, vp, u32, vp, u32, u32, u32, C.c_float],

@@ -93,32 +93,26 @@ extern "C" int nvmai_hip_rope_neox_subdim(nvmai_hip_ctx* ctx, nvmai_stream strea
     return launch_status();
 }
 
-extern "C" int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
-                                          const nvmai_kv_view* k, const nvmai_kv_view* v,
-                                          uint64_t kv_batch_stride, void* out, uint32_t batch,
-                                          uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
-                                          uint32_t seq_len, uint32_t kv_start, float scale) {
-    if (!ctx || !q || !out || batch == 0 || head_dim == 0 || num_kv_heads == 0) return NVMAI_ERR_INVALID_ARG;
-    if (num_q_heads % num_kv_heads) return NVMAI_ERR_INVALID_ARG;      // Attention.swift:221-222
-    if (head_dim > 512) return NVMAI_ERR_INVALID_ARG;                  // Attention.swift:223-224
-    if (kv_start > seq_len) return NVMAI_ERR_INVALID_ARG;
-    const uint32_t elements = num_kv_heads * head_dim;
-    int rc = check_view(k, elements);
-    if (rc) return rc;
-    rc = check_view(v, elements);
-    if (rc) return rc;
-    if (k->bits != v->bits || k->stride != v->stride) return NVMAI_ERR_INVALID_ARG;
-    if (!aligned16(q)) return NVMAI_ERR_ALIGNMENT;
+namespace {
+// Shared by the decode, ragged decode and causal prefill entry points.  p holds the problem (q, out
+// and their strides, the views' format, the per-sequence range rule, batch, heads); max_len is the
+// longest key range any block may have to walk, pack_ok says that every sequence reads the same
+// cache so several of them may share a block's K/V reads.
+int run_attention(nvmai_hip_ctx* ctx, nvmai_stream stream, AttnParams p, const nvmai_kv_view* k,
+                  const nvmai_kv_view* v, uint32_t max_len, bool pack_ok) {
     hipStream_t s = (hipStream_t)stream;
-    const uint32_t len = seq_len - kv_start;
-    const uint32_t qpk = num_q_heads / num_kv_heads;
-    const bool fast = head_dim == ATTN_HD && (k->bits == 4 || k->bits == 8) && qpk <= 16 &&
+    const uint32_t qpk = p.num_q_heads / p.num_kv_heads;
+    const bool fast = p.head_dim == ATTN_HD && (k->bits == 4 || k->bits == 8) && qpk <= 16 && p.ring == 0 &&
                       aligned16(k->base) && aligned16(v->base) && (k->stride % 16 == 0) &&
-                      (kv_batch_stride % 16 == 0) &&
-                      (uint64_t)seq_len * k->stride < (1ull << 32);        // 32-bit row offsets in the kernel
+                      (p.kv_batch_stride % 16 == 0) && aligned16(p.q) && (p.q_stride % 8 == 0) &&
+                      (uint64_t)p.seq_len * k->stride < (1ull << 32);      // 32-bit row offsets in the kernel
+    p.cols_q = (fast && pack_ok) ? 16 / qpk : 1;
+    const uint32_t seq_blocks = (p.batch + p.cols_q - 1) / p.cols_q;
+    if (p.cols_q > 1) max_len = max_len + p.cols_q - 1 < p.seq_len ? max_len + p.cols_q - 1 : p.seq_len;
     // Chunking: enough blocks to fill the device, chunks a multiple of the 32-token step.
-    const uint32_t units = fast ? batch * num_kv_heads : batch * num_q_heads;
-    uint32_t nc = (512 + units - 1) / units;
+    const uint64_t units = fast ? (uint64_t)seq_blocks * p.num_kv_heads : (uint64_t)p.batch * p.num_q_heads;
+    const uint32_t len = max_len;
+    uint32_t nc = units >= 512 ? 1 : (uint32_t)((512 + units - 1) / units);
     const uint32_t max_nc = (len + 127) / 128 ? (len + 127) / 128 : 1;
     if (nc > max_nc) nc = max_nc;
     if (nc < 1) nc = 1;
@@ -126,38 +120,114 @@ extern "C" int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream strea
     chunk_len = (chunk_len + 31) & ~31u;
     nc = ((len > 0 ? len : 1) + chunk_len - 1) / chunk_len;
     if (nc > ATTN_MAX_CHUNKS) return NVMAI_ERR_UNSUPPORTED;      // cannot happen: nc <= 512 by construction
-    const size_t heads_total = (size_t)batch * num_q_heads;
-    rc = ws_begin(ctx, stream, 2 * ws_round(heads_total * nc * 4) + ws_round(heads_total * nc * head_dim * 4));
-    if (rc) return rc;
-    AttnParams p{};
-    p.q = q; p.k = (const uint8_t*)k->base; p.v = (const uint8_t*)v->base; p.kv_batch_stride = kv_batch_stride;
-    p.f = KvFormat{k->bits, k->stride, k->value_bytes, elements};
-    p.head_dim = head_dim; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads; p.batch = batch;
-    p.seq_len = seq_len; p.kv_start = kv_start; p.num_chunks = nc; p.chunk_len = chunk_len;
-    p.scale = scale > 0.0f ? scale : 1.0f / std::sqrt((float)head_dim);
-    p.m_part = ws_take<float>(ctx, heads_total * nc);
-    p.d_part = ws_take<float>(ctx, heads_total * nc);
-    p.o_part = ws_take<float>(ctx, heads_total * nc * head_dim);
-    p.out = out;
+    const size_t heads_total = (size_t)p.batch * p.num_q_heads;
+    // one chunk: the partial kernel writes the rows itself (the matrix-core one in 8-byte pieces)
+    p.direct = nc == 1 && (!fast || ((reinterpret_cast<uintptr_t>(p.out) & 7u) == 0 && p.out_stride % 4 == 0));
+    p.num_chunks = nc; p.chunk_len = chunk_len;
+    if (!p.direct) {
+        const int rc = ws_begin(ctx, stream, 2 * ws_round(heads_total * nc * 4) + ws_round(heads_total * nc * p.head_dim * 4));
+        if (rc) return rc;
+        p.m_part = ws_take<float>(ctx, heads_total * nc);
+        p.d_part = ws_take<float>(ctx, heads_total * nc);
+        p.o_part = ws_take<float>(ctx, heads_total * nc * p.head_dim);
+    }
     {
         ProfScope ps(ctx, NVMAI_PROF_ATTN_PARTIAL, s);
         if (fast) {
-            dim3 grid(batch * num_kv_heads * nc);
+            dim3 grid(seq_blocks * p.num_kv_heads * nc);
 #define NVMAI_ATTN(ACT, BITS) attn_partial_mfma_kernel<ACT, BITS><<<grid, 256, 0, s>>>(p)
             if (ctx->act == ACT_BF16) { if (k->bits == 8) NVMAI_ATTN(ACT_BF16, 8); else NVMAI_ATTN(ACT_BF16, 4); }
             else { if (k->bits == 8) NVMAI_ATTN(ACT_FP16, 8); else NVMAI_ATTN(ACT_FP16, 4); }
 #undef NVMAI_ATTN
         } else {
-            dim3 grid(batch * num_q_heads * nc);
+            dim3 grid(p.batch * p.num_q_heads * nc);
             if (ctx->act == ACT_BF16) attn_partial_generic_kernel<ACT_BF16><<<grid, 256, 0, s>>>(p);
             else attn_partial_generic_kernel<ACT_FP16><<<grid, 256, 0, s>>>(p);
         }
     }
-    {
+    if (!p.direct) {
         ProfScope ps(ctx, NVMAI_PROF_ATTN_COMBINE, s);
-        const dim3 cgrid((uint32_t)heads_total, (head_dim + 63) / 64);
+        const dim3 cgrid((uint32_t)heads_total, (p.head_dim + 63) / 64);
         if (ctx->act == ACT_BF16) attn_combine_kernel<ACT_BF16><<<cgrid, 256, 0, s>>>(p);
         else attn_combine_kernel<ACT_FP16><<<cgrid, 256, 0, s>>>(p);
     }
     return launch_status();
+}
+
+// Argument checks common to the three entry points; fills the shape and format fields of p.
+int attention_setup(nvmai_hip_ctx* ctx, const void* q, const nvmai_kv_view* k, const nvmai_kv_view* v, void* out,
+                    uint32_t batch, uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads, float scale,
+                    AttnParams& p) {
+    if (!ctx || !q || !out || batch == 0 || head_dim == 0 || num_kv_heads == 0 || num_q_heads == 0) return NVMAI_ERR_INVALID_ARG;
+    if (num_q_heads % num_kv_heads) return NVMAI_ERR_INVALID_ARG;      // Attention.swift:221-222
+    if (head_dim > 512) return NVMAI_ERR_INVALID_ARG;                  // Attention.swift:223-224
+    const uint32_t elements = num_kv_heads * head_dim;
+    int rc = check_view(k, elements);
+    if (rc) return rc;
+    rc = check_view(v, elements);
+    if (rc) return rc;
+    if (k->bits != v->bits || k->stride != v->stride) return NVMAI_ERR_INVALID_ARG;
+    p = AttnParams{};
+    p.q = q; p.out = out; p.k = (const uint8_t*)k->base; p.v = (const uint8_t*)v->base;
+    p.f = KvFormat{k->bits, k->stride, k->value_bytes, elements};
+    p.head_dim = head_dim; p.num_q_heads = num_q_heads; p.num_kv_heads = num_kv_heads; p.batch = batch;
+    p.q_stride = p.out_stride = num_q_heads * head_dim;
+    p.scale = scale > 0.0f ? scale : 1.0f / std::sqrt((float)head_dim);
+    return NVMAI_OK;
+}
+}  // namespace
+
+extern "C" int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
+                                          const nvmai_kv_view* k, const nvmai_kv_view* v,
+                                          uint64_t kv_batch_stride, void* out, uint32_t batch,
+                                          uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                          uint32_t seq_len, uint32_t kv_start, float scale) {
+    AttnParams p;
+    const int rc = attention_setup(ctx, q, k, v, out, batch, head_dim, num_q_heads, num_kv_heads, scale, p);
+    if (rc) return rc;
+    if (kv_start > seq_len) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(q)) return NVMAI_ERR_ALIGNMENT;
+    p.kv_batch_stride = kv_batch_stride;
+    p.seq_len = seq_len; p.kv_start = kv_start;
+    return run_attention(ctx, stream, p, k, v, seq_len - kv_start, false);
+}
+
+extern "C" int nvmai_hip_attention_decode_ragged(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
+                                                 const nvmai_kv_view* k, const nvmai_kv_view* v,
+                                                 uint64_t kv_batch_stride, void* out, uint32_t batch,
+                                                 uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                                 const uint32_t* seq_lens, const uint32_t* kv_starts,
+                                                 uint32_t max_seq_len, float scale) {
+    AttnParams p;
+    const int rc = attention_setup(ctx, q, k, v, out, batch, head_dim, num_q_heads, num_kv_heads, scale, p);
+    if (rc) return rc;
+    if (!seq_lens) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(q)) return NVMAI_ERR_ALIGNMENT;
+    p.kv_batch_stride = kv_batch_stride;
+    p.seq_len = max_seq_len; p.kv_start = 0;
+    p.seq_lens = seq_lens; p.kv_starts = kv_starts;
+    return run_attention(ctx, stream, p, k, v, max_seq_len, false);
+}
+
+extern "C" int nvmai_hip_attention_prefill_causal(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
+                                                  uint32_t q_token_stride, const nvmai_kv_view* k,
+                                                  const nvmai_kv_view* v, void* out, uint32_t o_token_stride,
+                                                  uint32_t start_position, uint32_t query_count,
+                                                  uint32_t kv_valid_count, uint32_t sliding_window,
+                                                  uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                                  uint32_t kv_ring_capacity, float scale) {
+    AttnParams p;
+    // PrefillAttention.validate, PrefillAttention.swift:169-191
+    const int rc = attention_setup(ctx, q, k, v, out, query_count, head_dim, num_q_heads, num_kv_heads, scale, p);
+    if (rc) return rc;
+    if (q_token_stride < num_q_heads * head_dim || o_token_stride < num_q_heads * head_dim) return NVMAI_ERR_INVALID_ARG;
+    if ((uint64_t)start_position + query_count > kv_valid_count) return NVMAI_ERR_INVALID_ARG;
+    p.q_stride = q_token_stride; p.out_stride = o_token_stride;
+    p.kv_batch_stride = 0;
+    p.seq_len = kv_valid_count; p.kv_start = 0;
+    p.causal = 1; p.causal_start = start_position; p.window = sliding_window;
+    p.ring = kv_ring_capacity;
+    const uint32_t longest = start_position + query_count;          // keys of the last query without a window
+    const uint32_t max_len = sliding_window != 0 && sliding_window < longest ? sliding_window : longest;
+    return run_attention(ctx, stream, p, k, v, max_len, true);
 }

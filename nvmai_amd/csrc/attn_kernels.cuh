@@ -129,22 +129,46 @@ __global__ void rope_neox_subdim_kernel(void* data, uint32_t tokens, uint32_t he
     head[half_rot + pair] = f32_to_act<ACT>(__fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c)));
 }
 
-// ---- decode attention ------------------------------------------------------------------------
+// ---- decode and causal prefill attention -----------------------------------------------------
+// "Sequence" b is one query row: a decode step of sequence b, or query token b of a prefill chunk
+// (then every b reads the same cache: kv_batch_stride 0).
 struct AttnParams {
-    const void* q;             // [batch, num_q_heads, head_dim] activations
+    const void* q;             // query row of sequence b at q + b * q_stride: [num_q_heads, head_dim]
     const uint8_t* k;          // cache of sequence b at k + b * kv_batch_stride
     const uint8_t* v;
     uint64_t kv_batch_stride;  // bytes
     KvFormat f;
     uint32_t head_dim, num_q_heads, num_kv_heads, batch;
-    uint32_t seq_len, kv_start;
+    uint32_t seq_len, kv_start;     // keys [kv_start, seq_len) unless a per-sequence rule below applies;
+                                    // seq_len also bounds every row the kernels may touch
     uint32_t num_chunks, chunk_len;
     float scale;
     float* m_part;             // [batch, num_q_heads, num_chunks]
     float* d_part;
     float* o_part;             // [batch, num_q_heads, num_chunks, head_dim]
-    void* out;                 // [batch, num_q_heads, head_dim] activations
+    void* out;                 // row of sequence b at out + b * out_stride: [num_q_heads, head_dim]
+    uint32_t q_stride, out_stride;  // elements
+    // per-sequence key ranges: causal (prefill.metal:760-764) or read from device arrays
+    uint32_t causal;           // 1: keys [first, min(seq_len, start + b + 1)), first from the window
+    uint32_t causal_start, window;
+    const uint32_t* seq_lens;  // causal == 0, not null: keys [kv_starts[b] (or kv_start), min(seq_lens[b], seq_len))
+    const uint32_t* kv_starts;
+    uint32_t ring;             // not 0: row of key p is p % ring (generic kernel only)
+    uint32_t cols_q;           // sequences sharing one block of the matrix-core kernel
+    uint32_t direct;           // num_chunks == 1: the partial kernel normalises and writes out itself
 };
+
+__device__ __forceinline__ void attn_range(const AttnParams& p, uint32_t b, uint32_t& lo, uint32_t& hi) {
+    if (p.causal) {
+        const uint32_t a = p.causal_start + b + 1u;
+        hi = min(p.seq_len, a);
+        lo = (p.window != 0u && a > p.window) ? a - p.window : 0u;
+    } else {
+        hi = p.seq_lens ? min(p.seq_lens[b], p.seq_len) : p.seq_len;
+        lo = p.kv_starts ? p.kv_starts[b] : p.kv_start;
+    }
+    if (lo > hi) lo = hi;
+}
 
 __device__ __forceinline__ float kv_load(const uint8_t* row, const KvFormat& f, uint32_t e) {   // attention.metal:89-117
     if (f.bits == 16) return f16_to_f32(reinterpret_cast<const uint16_t*>(row)[e]);
@@ -155,7 +179,7 @@ __device__ __forceinline__ float kv_load(const uint8_t* row, const KvFormat& f, 
 }
 
 // Generic split-KV partial (attention.metal:163-261): any head_dim <= 512, any format.
-// One block per (batch, q head, chunk); thread i owns dims i, i+256.
+// One block per (sequence, q head, chunk); thread i owns dims i, i+256.
 template <int ACT>
 __global__ __launch_bounds__(256) void attn_partial_generic_kernel(AttnParams p) {
     __shared__ float red[4];
@@ -163,16 +187,19 @@ __global__ __launch_bounds__(256) void attn_partial_generic_kernel(AttnParams p)
     const uint32_t head = (blockIdx.x / p.num_chunks) % p.num_q_heads;
     const uint32_t b = blockIdx.x / (p.num_chunks * p.num_q_heads);
     const uint32_t kvh = head / (p.num_q_heads / p.num_kv_heads);
-    const uint32_t p0 = p.kv_start + chunk * p.chunk_len, p1 = min(p0 + p.chunk_len, p.seq_len);
-    const uint16_t* qh = (const uint16_t*)p.q + ((size_t)b * p.num_q_heads + head) * p.head_dim;
+    uint32_t lo, hi;
+    attn_range(p, b, lo, hi);
+    const uint32_t p0 = min(lo + chunk * p.chunk_len, hi), p1 = min(p0 + p.chunk_len, hi);
+    const uint16_t* qh = (const uint16_t*)p.q + (size_t)b * p.q_stride + (size_t)head * p.head_dim;
     const uint32_t tid = threadIdx.x;
     float qv[2], o[2] = {0.0f, 0.0f};
 #pragma unroll
     for (int s = 0; s < 2; ++s) qv[s] = tid + 256 * s < p.head_dim ? act_to_f32<ACT>(qh[tid + 256 * s]) : 0.0f;
     float m = -INFINITY, d = 0.0f;
     for (uint32_t pos = p0; pos < p1; ++pos) {
-        const uint8_t* kr = p.k + b * p.kv_batch_stride + (size_t)pos * p.f.stride;
-        const uint8_t* vr = p.v + b * p.kv_batch_stride + (size_t)pos * p.f.stride;
+        const uint32_t slot = p.ring ? pos % p.ring : pos;
+        const uint8_t* kr = p.k + b * p.kv_batch_stride + (size_t)slot * p.f.stride;
+        const uint8_t* vr = p.v + b * p.kv_batch_stride + (size_t)slot * p.f.stride;
         float part = 0.0f;
 #pragma unroll
         for (int s = 0; s < 2; ++s)
@@ -190,6 +217,13 @@ __global__ __launch_bounds__(256) void attn_partial_generic_kernel(AttnParams p)
             if (tid + 256 * s < p.head_dim)
                 o[s] = o[s] * alpha + pe * kv_load(vr, p.f, kvh * p.head_dim + tid + 256 * s);
         m = mn;
+    }
+    if (p.direct) {                                       // one chunk: no partials, no combine
+        uint16_t* orow = (uint16_t*)p.out + (size_t)b * p.out_stride + (size_t)head * p.head_dim;
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+            if (tid + 256 * s < p.head_dim) orow[tid + 256 * s] = f32_to_act<ACT>(d > 0.0f ? o[s] / d : 0.0f);
+        return;
     }
     const size_t base = ((size_t)b * p.num_q_heads + head) * p.num_chunks + chunk;
     if (tid == 0) { p.m_part[base] = m; p.d_part[base] = d; }
@@ -214,6 +248,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     const float* dr = p.d_part + bh * p.num_chunks;
     const float* orow = p.o_part + bh * p.num_chunks * p.head_dim;
     const uint32_t dim = blockIdx.y * 64 + lane;
+    uint16_t* out_row = (uint16_t*)p.out + (bh / p.num_q_heads) * p.out_stride + (bh % p.num_q_heads) * p.head_dim;
     float mloc = -INFINITY;
     for (uint32_t c = threadIdx.x; c < p.num_chunks; c += 256) mloc = fmaxf(mloc, mr[c]);
     mloc = wave_max_f32(mloc);
@@ -221,7 +256,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     __syncthreads();
     const float mg = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     if (mg == -INFINITY) {                                   // uniform over the block
-        if (wave == 0 && dim < p.head_dim) ((uint16_t*)p.out)[bh * p.head_dim + dim] = f32_to_act<ACT>(0.0f);
+        if (wave == 0 && dim < p.head_dim) out_row[dim] = f32_to_act<ACT>(0.0f);
         return;
     }
     float dloc = 0.0f;
@@ -244,7 +279,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     __syncthreads();
     if (wave == 0 && dim < p.head_dim) {
         const float tot = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
-        ((uint16_t*)p.out)[bh * p.head_dim + dim] = f32_to_act<ACT>(D > 0.0f ? tot / D : 0.0f);
+        out_row[dim] = f32_to_act<ACT>(D > 0.0f ? tot / D : 0.0f);
     }
 }
 
@@ -314,9 +349,28 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
     float* merge = reinterpret_cast<float*>(kst);                  // after the loop
     const uint32_t chunk = blockIdx.x % p.num_chunks;
     const uint32_t kvh = (blockIdx.x / p.num_chunks) % p.num_kv_heads;
-    const uint32_t b = blockIdx.x / (p.num_chunks * p.num_kv_heads);
+    const uint32_t n_qb = (p.batch + p.cols_q - 1) / p.cols_q;
+    uint32_t qb = blockIdx.x / (p.num_chunks * p.num_kv_heads);
+    if (p.causal) qb = n_qb - 1u - qb;                             // the longest key ranges start first
+    const uint32_t b = qb * p.cols_q;                              // first sequence of this block
     const uint32_t qpk = p.num_q_heads / p.num_kv_heads;           // <= 16
-    const uint32_t p0 = p.kv_start + chunk * p.chunk_len, p1 = min(p0 + p.chunk_len, p.seq_len);
+    // Column i of the score tile is (sequence b + i / qpk, q head i % qpk of this kv head): a decode
+    // step has cols_q = 1, a prefill chunk packs 16 / qpk query tokens into the sixteen columns.
+    const uint32_t cols = min(p.cols_q, p.batch - b) * qpk;        // live columns
+    const bool live = (uint32_t)i < cols;
+    const uint32_t my_b = b + (live ? (uint32_t)i / qpk : 0u), my_h = kvh * qpk + (live ? (uint32_t)i % qpk : 0u);
+    uint32_t lo_i, hi_i;                                           // key range of this lane's column
+    attn_range(p, my_b, lo_i, hi_i);
+    uint32_t blo = live ? lo_i : 0xFFFFFFFFu, bhi = live ? hi_i : 0u;
+    if (!live) lo_i = hi_i = 0u;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        blo = min(blo, shfl_xor_u(blo, off));
+        bhi = max(bhi, shfl_xor_u(bhi, off));
+    }
+    blo = __builtin_amdgcn_readfirstlane(blo);                     // the union of the block's ranges
+    bhi = __builtin_amdgcn_readfirstlane(bhi);
+    const uint32_t p0 = min(blo + chunk * p.chunk_len, bhi), p1 = min(p0 + p.chunk_len, bhi);
     const uint32_t groups_total = (p.f.elements + 63) / 64;
     const uint32_t code_off = kvh * ATTN_HD * BITS / 8;            // this head's codes inside a row
     const uint32_t meta_sc = p.f.value_bytes + 2 * (kvh * 4);      // 4 fp16 scales of this head
@@ -329,8 +383,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
     float qsum[4];
     float q_unscale;                                               // scale * 2^-k of head i
     {
-        const bool live = (uint32_t)i < qpk;
-        const uint16_t* qh = (const uint16_t*)p.q + ((size_t)b * p.num_q_heads + kvh * qpk + (live ? i : 0)) * ATTN_HD;
+        const uint16_t* qh = (const uint16_t*)p.q + (size_t)my_b * p.q_stride + (size_t)my_h * ATTN_HD;
         float qf[4][2][8];
         float amax = 0.0f;
 #pragma unroll
@@ -428,7 +481,10 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
         __builtin_amdgcn_s_waitcnt(gemm_like_vmcnt(N_LOADS));
         bool tok_ok[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) tok_ok[t] = s0 + slot_tok(t) < p1;
+        for (int t = 0; t < 8; ++t) {
+            const uint32_t pos = s0 + slot_tok(t);
+            tok_ok[t] = pos < p1 && pos >= lo_i && pos < hi_i;
+        }
 
         // ---- S^T = K . Q^T per group, then the exact affine correction
         float sv[8];                                                // scores of head i at this lane's 8 tokens
@@ -492,11 +548,12 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
         for (int t = 1; t < 8; ++t) mx = fmaxf(mx, sv[t]);
         mx = fmaxf(mx, shfl_xor_f(mx, 16));
         mx = fmaxf(mx, shfl_xor_f(mx, 32));
-        const float m_new = fmaxf(m_run, mx);                       // finite: the step holds >= 1 valid token
-        const float alpha = expf(m_run - m_new);
+        const float m_new = fmaxf(m_run, mx);                       // -inf while the column has seen no key yet
+        const bool none = m_new == -INFINITY;
+        const float alpha = none ? 1.0f : expf(m_run - m_new);
         float pe[8], psum = 0.0f;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) { pe[t] = expf(sv[t] - m_new); psum += pe[t]; }
+        for (int t = 0; t < 8; ++t) { pe[t] = none ? 0.0f : expf(sv[t] - m_new); psum += pe[t]; }
         d_run = d_run * alpha + psum;
         m_run = m_new;
 
@@ -640,16 +697,40 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
     __syncthreads();
     if (wave != 0) return;
     take_state(merge);
-    const size_t hbase = (size_t)b * p.num_q_heads + kvh * qpk;
-    if (r == 0 && (uint32_t)i < qpk) {
-        p.m_part[(hbase + i) * p.num_chunks + chunk] = m_run;
-        p.d_part[(hbase + i) * p.num_chunks + chunk] = d_run;
+    // column c -> (sequence b + c / qpk, q head kvh * qpk + c % qpk)
+    if (p.direct) {                                                 // one chunk: normalise and write the rows
+        if (r == 0) bc[i] = d_run;
+        __builtin_amdgcn_wave_barrier();
+        const float4 d4 = *reinterpret_cast<const float4*>(bc + 4 * r);
+        __builtin_amdgcn_wave_barrier();
+        const float dd[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t c = 4 * r + t;
+            if (c >= cols) continue;
+            uint16_t* dst = (uint16_t*)p.out + (size_t)(b + c / qpk) * p.out_stride + (size_t)(kvh * qpk + c % qpk) * ATTN_HD;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint2 o2;
+                o2.x = f32_to_act<ACT>(dd[t] > 0.0f ? oacc[g][0][t] / dd[t] : 0.0f) |
+                       ((uint32_t)f32_to_act<ACT>(dd[t] > 0.0f ? oacc[g][1][t] / dd[t] : 0.0f) << 16);
+                o2.y = f32_to_act<ACT>(dd[t] > 0.0f ? oacc[g][2][t] / dd[t] : 0.0f) |
+                       ((uint32_t)f32_to_act<ACT>(dd[t] > 0.0f ? oacc[g][3][t] / dd[t] : 0.0f) << 16);
+                *reinterpret_cast<uint2*>(dst + 64 * g + 4 * i) = o2;
+            }
+        }
+        return;
+    }
+    if (r == 0 && live) {
+        const size_t at = ((size_t)my_b * p.num_q_heads + my_h) * p.num_chunks + chunk;
+        p.m_part[at] = m_run;
+        p.d_part[at] = d_run;
     }
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-        const uint32_t head = 4 * r + t;
-        if (head >= qpk) continue;
-        float* dst = p.o_part + ((hbase + head) * p.num_chunks + chunk) * ATTN_HD;
+        const uint32_t c = 4 * r + t;
+        if (c >= cols) continue;
+        float* dst = p.o_part + (((size_t)(b + c / qpk) * p.num_q_heads + kvh * qpk + c % qpk) * p.num_chunks + chunk) * ATTN_HD;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const float4 o4 = {oacc[g][0][t], oacc[g][1][t], oacc[g][2][t], oacc[g][3][t]};

@@ -515,6 +515,41 @@ class Attention:
         return self.encode_full(q, k_cache, v_cache, head_dim, num_q_heads, num_kv_heads, seq_len, scale,
                                 kv_start=seq_len - window if seq_len > window else 0)
 
+    def encode_ragged(self, q, k_cache, v_cache, head_dim, num_q_heads, num_kv_heads, seq_lens, max_seq_len,
+                      kv_starts=None, scale=None, out=None):
+        """One decode query per sequence, each with its own key range: seq_lens / kv_starts are
+        uint32 device tensors of one word per sequence."""
+        batch = q.shape[0]
+        if out is None:
+            out = torch.empty_like(q)
+        kview, vview = k_cache.view(), v_cache.view()
+        check(lib.nvmai_hip_attention_decode_ragged(self.ctx.handle, _stream(), _ptr(q), C.byref(kview),
+                                                    C.byref(vview), k_cache.batch_stride, _ptr(out), batch, head_dim,
+                                                    num_q_heads, num_kv_heads, _ptr(seq_lens), _ptr(kv_starts),
+                                                    max_seq_len, 0.0 if scale is None else scale),
+              "attention_decode_ragged")
+        return out
+
+
+class PrefillAttention:
+    """Mirror of PrefillAttention (PrefillAttention.swift:70-167), causalTiled path."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+
+    def encode_causal(self, q, k_view, v_view, out, start_position, query_count, head_dim, num_q_heads,
+                      num_kv_heads, kv_valid_count, sliding_window=0, q_token_stride=None, o_token_stride=None,
+                      scale=None, kv_ring_capacity=0):
+        """q / out: tensors whose row t starts t * token stride elements in; k_view / v_view:
+        KvView of the cache rows from position 0."""
+        row = num_q_heads * head_dim
+        check(lib.nvmai_hip_attention_prefill_causal(
+            self.ctx.handle, _stream(), _ptr(q), row if q_token_stride is None else q_token_stride,
+            C.byref(k_view), C.byref(v_view), _ptr(out), row if o_token_stride is None else o_token_stride,
+            start_position, query_count, kv_valid_count, sliding_window, head_dim, num_q_heads, num_kv_heads,
+            kv_ring_capacity, 0.0 if scale is None else scale), "attention_prefill_causal")
+        return out
+
 
 # ---------------------------------------------------------------------------------------------
 # logits -> token

@@ -522,6 +522,24 @@ def attention_decode(q, k, v, kv_bits, nq, nkv, hd, seq_len, scale, kv_start=0,
     return out
 
 
+def attention_prefill_causal(q, k, v, kv_bits, nq, nkv, hd, start, kv_valid, scale, window=0, ring=0):
+    """q float32 [count, nq*hd]; k, v: float32 [rows, nkv*hd] (kv_bits=32) or uint8 [rows, stride].
+    Returns float32 [count, nq*hd]."""
+    q = np.ascontiguousarray(q, np.float32)
+    count = q.shape[0]
+    q = q.reshape(count, nq * hd)
+    stride, vb = (0, 0) if kv_bits == 32 else kv_row_layout(nkv * hd, kv_bits)
+    k, v = np.ascontiguousarray(k), np.ascontiguousarray(v)
+    out = np.zeros((count, nq * hd), np.float32)
+    fn = lib.orc_attention_prefill_causal
+    fn.restype = None
+    fn.argtypes = [f32p, size_t, C.c_void_p, C.c_void_p, C.c_int, size_t, size_t, size_t, size_t, size_t,
+                   size_t, size_t, size_t, size_t, size_t, C.c_float, f32p, size_t]
+    fn(q, nq * hd, k.ctypes.data, v.ctypes.data, kv_bits, stride, vb, nq, nkv, hd, start, count, kv_valid,
+       window, ring, scale, out, nq * hd)
+    return out
+
+
 # ---------------------------------------------------------------- sampler
 def softmax_f16(logits, softcap=0.0, tiled=False):
     logits = np.ascontiguousarray(logits, np.float32)

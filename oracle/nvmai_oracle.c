@@ -768,6 +768,53 @@ void orc_attention_decode(const float *q, const void *k, const void *v, int kv_b
     free(o); free(dsum); free(m); free(vt); free(kt);
 }
 
+void orc_attention_prefill_causal(const float *q, size_t q_stride, const void *k, const void *v,
+                                  int kv_bits, size_t stride, size_t value_bytes,
+                                  size_t num_q_heads, size_t num_kv_heads, size_t head_dim,
+                                  size_t start, size_t count, size_t kv_valid, size_t window,
+                                  size_t ring, float scale, float *out, size_t out_stride) {
+    const size_t elements = num_kv_heads * head_dim;
+    const size_t q_per_kv = num_q_heads / num_kv_heads;
+    float *kt = (float *)malloc(elements * sizeof(float));
+    float *vt = (float *)malloc(elements * sizeof(float));
+    float *row_max = (float *)malloc(num_q_heads * sizeof(float));
+    float *row_sum = (float *)malloc(num_q_heads * sizeof(float));
+    float *acc = (float *)malloc(num_q_heads * head_dim * sizeof(float));
+    for (size_t t = 0; t < count; ++t) {
+        const size_t abs_q = start + t;
+        const size_t first = (window != 0 && abs_q + 1 > window) ? abs_q + 1 - window : 0;
+        const size_t last = kv_valid < abs_q + 1 ? kv_valid : abs_q + 1;
+        for (size_t h = 0; h < num_q_heads; ++h) { row_max[h] = -INFINITY; row_sum[h] = 0.0f; }
+        memset(acc, 0, num_q_heads * head_dim * sizeof(float));
+        for (size_t key = first; key < last; ++key) {
+            const size_t slot = ring ? key % ring : key;
+            const float *kr, *vr;
+            kv_row_as_float(k, kv_bits, stride, value_bytes, elements, slot, kt, &kr);
+            kv_row_as_float(v, kv_bits, stride, value_bytes, elements, slot, vt, &vr);
+            for (size_t h = 0; h < num_q_heads; ++h) {
+                const size_t kvh = h / q_per_kv;
+                const float *qh = q + t * q_stride + h * head_dim;
+                float s = 0.0f;
+                for (size_t i = 0; i < head_dim; ++i) s = fmaf(qh[i], kr[kvh * head_dim + i], s);
+                s *= scale;
+                const float new_max = fmaxf(row_max[h], s);
+                const float old_scale = row_sum[h] > 0.0f ? expf(row_max[h] - new_max) : 0.0f;
+                const float new_scale = expf(s - new_max);
+                float *a = acc + h * head_dim;
+                for (size_t i = 0; i < head_dim; ++i)
+                    a[i] = fmaf(new_scale, vr[kvh * head_dim + i], a[i] * old_scale);
+                row_sum[h] = row_sum[h] * old_scale + new_scale;
+                row_max[h] = new_max;
+            }
+        }
+        for (size_t h = 0; h < num_q_heads; ++h)
+            for (size_t i = 0; i < head_dim; ++i)
+                out[t * out_stride + h * head_dim + i] =
+                    row_sum[h] > 0.0f ? acc[h * head_dim + i] / row_sum[h] : 0.0f;
+    }
+    free(acc); free(row_sum); free(row_max); free(vt); free(kt);
+}
+
 /* ------------------------------------------------------------------------ */
 /* softmax + sampler                                                         */
 /* ------------------------------------------------------------------------ */

@@ -174,6 +174,19 @@ void orc_attention_decode(const float *q, const void *k, const void *v, int kv_b
                           size_t kv_start, float scale, size_t num_chunks,
                           size_t chunk_len, float *out);
 
+/* Causal prefill attention, attention_prefill_causal_tiled (prefill.metal:709-830): query t
+ * (row q + t * q_stride, [num_q_heads, head_dim]) at absolute position start + t attends to
+ * keys [first, min(kv_valid, start + t + 1)) with first = start + t + 1 - window when window
+ * != 0 and that is positive, else 0 (:760-764); online softmax over the keys in ascending
+ * order (:771-792), out = acc / row_sum, zeros for an empty row (:794-797).  The row of key p
+ * is p % ring when ring != 0 (:732-737).  K/V rows as for orc_attention_decode.  out row t at
+ * out + t * out_stride, not rounded. */
+void orc_attention_prefill_causal(const float *q, size_t q_stride, const void *k, const void *v,
+                                  int kv_bits, size_t stride, size_t value_bytes,
+                                  size_t num_q_heads, size_t num_kv_heads, size_t head_dim,
+                                  size_t start, size_t count, size_t kv_valid, size_t window,
+                                  size_t ring, float scale, float *out, size_t out_stride);
+
 /* ---- softmax + sampler (logit.metal) ------------------------------------ */
 /* two-pass fp32 softmax with optional softcap (<=0 disables), fp16 probs */
 void orc_softmax_f16(const float *logits, size_t v, float softcap, uint16_t *probs_f16);

@@ -260,3 +260,185 @@ def test_attention_configs3_long_context(nv, bits, batch, seq, kv_start):
         assert O.rel_error(alone[0], out[b]) < 1e-2
     torch.cuda.synchronize()
     ctx.close()
+
+
+# ---------------------------------------------------------------- causal prefill attention
+def _prefill_case(nv, ctx, seed, bits, start, chunk, window, hd, nq, nkv, extra_kv=0, pad=True, ring=0, lo=-0.35,
+                  hi=0.35, tol=1e-2, scale=1.0):
+    """One PrefillAttention.encodeCausal call against the oracle over the same rows.  pad: strided
+    q / out rows and offset buffers as PrefillAttentionTests.swift:179-258 builds them."""
+    rng = np.random.default_rng(seed)
+    kv_valid = start + chunk + extra_kv
+    elements, row = nkv * hd, nq * hd
+    q = round_act(rng.uniform(lo, hi, (chunk, row)).astype(np.float32), ctx.act)
+    k = round_act(rng.uniform(lo, hi, (kv_valid, elements)).astype(np.float32), ctx.act)
+    v = round_act(rng.uniform(lo, hi, (kv_valid, elements)).astype(np.float32), ctx.act)
+    q_stride, o_stride, q_off, o_off = (row + 3, row + 7, 17, 29) if pad else (row, row, 0, 0)
+    q_buf = torch.zeros(q_off + chunk * q_stride, dtype=ctx.dtype, device="cuda")
+    q_buf[q_off:].view(chunk, q_stride)[:, :row] = act_tensor(q, ctx)
+    out_buf = torch.full((o_off + chunk * o_stride,), 7.0, dtype=ctx.dtype, device="cuda")
+    rows = ring if ring else kv_valid
+    kc, vc = nv.KVCache(1, rows, elements, bits), nv.KVCache(1, rows, elements, bits)
+    if bits == 16:
+        k, v = O.f16_to_float(O.f16_bits(k)), O.f16_to_float(O.f16_bits(v))
+        ko, vo = k, v
+        if ring:
+            ko, vo = np.zeros((ring, elements), np.float32), np.zeros((ring, elements), np.float32)
+            for p in range(kv_valid):
+                ko[p % ring], vo[p % ring] = k[p], v[p]
+        kc.rows[0].copy_(dev(ko).to(torch.float16).view(torch.uint8).view(rows, -1))
+        vc.rows[0].copy_(dev(vo).to(torch.float16).view(torch.uint8).view(rows, -1))
+        obits = 32
+    else:
+        assert not ring
+        quant = nv.KVCacheQuantizer(ctx)
+        quant.encode(act_tensor(k, ctx), elements, kc.view(), kv_valid, elements)
+        quant.encode(act_tensor(v, ctx), elements, vc.view(), kv_valid, elements)
+        ko, vo = kc.rows[0].cpu().numpy(), vc.rows[0].cpu().numpy()
+        obits = bits
+    nv.PrefillAttention(ctx).encode_causal(q_buf[q_off:], kc.view(), vc.view(), out_buf[o_off:], start, chunk, hd, nq, nkv,
+                                           kv_valid, sliding_window=window, q_token_stride=q_stride,
+                                           o_token_stride=o_stride, scale=scale, kv_ring_capacity=ring)
+    torch.cuda.synchronize()
+    flat = act_np(out_buf)
+    got = flat[o_off:].reshape(chunk, o_stride)[:, :row]
+    want = O.attention_prefill_causal(q, ko, vo, obits, nq, nkv, hd, start, kv_valid, scale, window=window, ring=ring)
+    err = O.rel_error(got, want)
+    assert err < tol, "rel %g" % err
+    # nothing outside the output rows is written
+    assert np.all(flat[:o_off] == 7.0) and np.all(flat[o_off:].reshape(chunk, o_stride)[:, row:] == 7.0)
+    return got, want, (q, k, v)
+
+
+def test_prefill_attention_reference_cases(nv, ctx):
+    # PrefillAttentionTests.swift:10-25, 79-116: fp16 rows, strided and offset buffers
+    cases = [(0, 3, 0, 8, 4, 2), (4, 3, 0, 8, 4, 2), (2, 4, 16, 8, 4, 2), (7, 4, 5, 8, 4, 2),
+             (1023, 1, 1, 256, 16, 8), (1024, 1, 1, 256, 16, 8), (4095, 1, 1, 256, 16, 8), (0, 1, 0, 512, 16, 2),
+             (3, 1, 0, 512, 16, 2), (1023, 4, 1024, 256, 16, 8), (31, 8, 0, 512, 16, 2)]
+    for n, (start, chunk, window, hd, nq, nkv) in enumerate(cases):
+        say("prefill attention fp16 rows", ctx.act, start, chunk, window, hd, nq, nkv)
+        _prefill_case(nv, ctx, 0xA510 + n, 16, start, chunk, window, hd, nq, nkv)
+    say("prefill attention ring", ctx.act)                         # PrefillAttentionTests.swift:27-56
+    _prefill_case(nv, ctx, 0xA611, 16, 20, 4, 8, 32, 4, 2, ring=16)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_prefill_attention_quantized_rows(nv, ctx, bits):
+    # KVCacheQuantizedAttentionTests.swift:91-157 (start 4, four queries, qwen shape) and beyond it:
+    # chunks that start deep in the cache, windows, kv_valid past the chunk, odd query counts, the
+    # generic path (head_dim 128 and padded rows) beside the matrix-core one
+    say("prefill attention vs unquantized", ctx.act, bits)
+    got, want, (q, k, v) = _prefill_case(nv, ctx, 0x5052, bits, 4, 4, 0, 256, 16, 2, pad=False, lo=-0.5, hi=0.5,
+                                         scale=1 / 16.0)
+    dense = O.attention_prefill_causal(q, k, v, 32, 16, 2, 256, 4, 8, 1 / 16.0)
+    assert O.rel_error(got, dense) < (0.025 if bits == 8 else 0.20)
+    for start, chunk, window, hd, nq, nkv, extra, pad in [
+            (0, 1, 0, 256, 16, 2, 0, False), (0, 67, 0, 256, 16, 2, 0, False), (130, 33, 0, 256, 16, 2, 5, False),
+            (500, 40, 64, 256, 16, 2, 0, False), (100, 9, 7, 256, 16, 8, 0, False), (64, 5, 0, 256, 16, 16, 0, False),
+            (31, 6, 0, 256, 6, 2, 0, False), (40, 7, 16, 256, 16, 2, 0, True), (9, 5, 0, 128, 8, 2, 3, False)]:
+        say("prefill attention quantized", ctx.act, bits, start, chunk, window, hd, nq, nkv, extra, pad)
+        _prefill_case(nv, ctx, start + chunk, bits, start, chunk, window, hd, nq, nkv, extra_kv=extra, pad=pad,
+                      lo=-1.0, hi=1.0, scale=1.0 / np.sqrt(hd))
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_prefill_attention_chunk_equals_decode_steps(nv, bits):
+    # size-independent property at a prefill size the scalar oracle cannot walk: query t of a
+    # 512-token chunk at the end of an 8K context is the decode call with seq_len = start + t + 1
+    # (the same kernels, a different packing of queries into blocks), and the oracle agrees on a few rows
+    say("prefill chunk vs decode", bits)
+    ctx = nv.Context(0, 0)
+    gen = torch.Generator(device="cuda").manual_seed(11 + bits)
+    nq, nkv, hd, start, chunk = 16, 2, 256, 7680, 512
+    kv_valid, elements = start + chunk, nkv * hd
+    kc, vc, _ = _long_cache(nv, ctx, gen, 1, kv_valid, elements, bits)
+    q = torch.randn((chunk, nq, hd), generator=gen, device="cuda", dtype=torch.float32).to(ctx.dtype)
+    out = torch.empty_like(q)
+    nv.PrefillAttention(ctx).encode_causal(q, kc.view(), vc.view(), out, start, chunk, hd, nq, nkv, kv_valid)
+    att = nv.Attention(ctx)
+    kq, vq = kc.rows[0].cpu().numpy(), vc.rows[0].cpu().numpy()
+    for t in (0, 1, 255, 510, 511):
+        one = att.encode_full(q[t:t + 1], kc, vc, hd, nq, nkv, start + t + 1)
+        torch.cuda.synchronize()
+        assert O.rel_error(act_np(out[t]), act_np(one[0])) < 1e-2       # two bf16 roundings of differently ordered sums
+    for t in (0, 511):
+        want = O.attention_decode(act_np(q[t]), kq, vq, bits, nq, nkv, hd, start + t + 1, 1 / 16.0)
+        assert O.rel_error(act_np(out[t]), want) < 1e-2
+    # ragged decode: the same rows again, every query as its own "sequence" of the one cache
+    lens = torch.arange(start + 1, start + chunk + 1, device="cuda", dtype=torch.int32)
+    ragged = att.encode_ragged(q, _Shared(kc), _Shared(vc), hd, nq, nkv, lens, kv_valid)
+    torch.cuda.synchronize()
+    assert O.rel_error(act_np(ragged), act_np(out)) < 1e-2
+    ctx.close()
+
+
+class _Shared:
+    """A cache whose every sequence is sequence 0 (batch stride 0)."""
+
+    def __init__(self, cache):
+        self.cache, self.batch_stride = cache, 0
+
+    def view(self):
+        return self.cache.view()
+
+
+def test_attention_ragged_batch(nv, ctx):
+    # sequences of different lengths and starts in one call, an empty one included
+    say("attention ragged", ctx.act)
+    rng = np.random.default_rng(41)
+    nq, nkv, hd, batch, cap = 16, 2, 256, 5, 700
+    for bits in (8, 4, 16):
+        elements = nkv * hd
+        q = round_act(gauss(rng, (batch, nq, hd)), ctx.act)
+        k = round_act(gauss(rng, (batch, cap, elements)), ctx.act)
+        v = round_act(gauss(rng, (batch, cap, elements)), ctx.act)
+        kc, vc = nv.KVCache(batch, cap, elements, bits), nv.KVCache(batch, cap, elements, bits)
+        if bits == 16:
+            kc.rows.copy_(dev(k).to(torch.float16).view(torch.uint8).view(batch, cap, -1))
+            vc.rows.copy_(dev(v).to(torch.float16).view(torch.uint8).view(batch, cap, -1))
+        else:
+            quant = nv.KVCacheQuantizer(ctx)
+            for b in range(batch):
+                quant.encode(act_tensor(k[b], ctx), elements, kc.view(b), cap, elements)
+                quant.encode(act_tensor(v[b], ctx), elements, vc.view(b), cap, elements)
+        lens = np.array([700, 1, 333, 64, 0], np.uint32)
+        starts = np.array([0, 0, 300, 63, 0], np.uint32)
+        for use_starts in (False, True):
+            out = nv.Attention(ctx).encode_ragged(act_tensor(q, ctx), kc, vc, hd, nq, nkv,
+                                                  dev(lens.view(np.int32)), cap,
+                                                  kv_starts=dev(starts.view(np.int32)) if use_starts else None)
+            torch.cuda.synchronize()
+            got = act_np(out)
+            for b in range(batch):
+                s0 = int(starts[b]) if use_starts else 0
+                if bits == 16:
+                    want = O.attention_decode(q[b], O.f16_to_float(O.f16_bits(k[b])), O.f16_to_float(O.f16_bits(v[b])),
+                                              32, nq, nkv, hd, int(lens[b]), 1 / 16.0, s0)
+                else:
+                    want = O.attention_decode(q[b], kc.rows[b].cpu().numpy(), vc.rows[b].cpu().numpy(), bits, nq, nkv,
+                                              hd, int(lens[b]), 1 / 16.0, s0)
+                if lens[b] == 0:
+                    assert not got[b].any() and not want.any()
+                else:
+                    assert O.rel_error(got[b], want) < 1e-2, (bits, b)
+
+
+def test_prefill_attention_rejects_what_validate_rejects(nv, ctx):
+    say("prefill attention errors")
+    kc, vc = nv.KVCache(1, 16, 512, 8), nv.KVCache(1, 16, 512, 8)
+    q = torch.zeros((4, 16 * 256), dtype=ctx.dtype, device="cuda")
+    out = torch.zeros_like(q)
+    pa = nv.PrefillAttention(ctx)
+    for kwargs in (dict(q_token_stride=100), dict(o_token_stride=100)):       # PrefillAttention.swift:176-179
+        with pytest.raises(nv.NvmaiError) as e:
+            pa.encode_causal(q, kc.view(), vc.view(), out, 0, 4, 256, 16, 2, 4, **kwargs)
+        assert e.value.name == "invalid_arg"
+    with pytest.raises(nv.NvmaiError) as e:                                      # :189-190
+        pa.encode_causal(q, kc.view(), vc.view(), out, 2, 4, 256, 16, 2, 5)
+    assert e.value.name == "invalid_arg"
+    with pytest.raises(nv.NvmaiError) as e:                                      # queryCount must be positive
+        pa.encode_causal(q, kc.view(), vc.view(), out, 0, 0, 256, 16, 2, 4)
+    assert e.value.name == "invalid_arg"
+    with pytest.raises(nv.NvmaiError) as e:                                      # :174-175
+        pa.encode_causal(q, kc.view(), vc.view(), out, 0, 4, 256, 15, 2, 4)
+    assert e.value.name == "invalid_arg"

@@ -163,3 +163,103 @@ def test_quantized_attention_tracks_unquantized_reference():
         kd = O.kv_dequant(O.kv_quantize(k, bits), nkv * hd, bits)
         vd = O.kv_dequant(O.kv_quantize(v, bits), nkv * hd, bits)
         assert O.rel_error(got, _attention64(q, kd, vd, nq, nkv, hd, 0.0625)) < 1e-5
+
+
+# ---------------------------------------------------------------- causal prefill attention
+def _prefill_model_f64(q, k, v, nq, nkv, hd, start, kv_valid, window, scale):
+    """softmax(q K^T * scale) V per query over its visible keys, float64: what
+    PrefillAttentionRef.apply (PrefillAttentionRef.swift:57-99) computes, written with matrix
+    products instead of the kernel's running maximum."""
+    count = q.shape[0]
+    out = np.zeros((count, nq, hd))
+    q = q.astype(np.float64).reshape(count, nq, hd)
+    k = k.astype(np.float64).reshape(-1, nkv, hd)
+    v = v.astype(np.float64).reshape(-1, nkv, hd)
+    for t in range(count):
+        a = start + t
+        first = max(0, a + 1 - window) if window else 0
+        last = min(kv_valid, a + 1)
+        if last <= first:
+            continue
+        for h in range(nq):
+            kvh = h // (nq // nkv)
+            s = k[first:last, kvh] @ q[t, h] * scale
+            w = np.exp(s - s.max())
+            out[t, h] = (w / w.sum()) @ v[first:last, kvh]
+    return out.reshape(count, nq * hd)
+
+
+def _prefill_fixture(seed, start, chunk, hd, nq, nkv, extra_kv=0, lo=-0.35, hi=0.35):
+    rng = np.random.default_rng(seed)
+    kv_valid = start + chunk + extra_kv
+    q = rng.uniform(lo, hi, (chunk, nq * hd)).astype(np.float32)
+    k = rng.uniform(lo, hi, (kv_valid, nkv * hd)).astype(np.float32)
+    v = rng.uniform(lo, hi, (kv_valid, nkv * hd)).astype(np.float32)
+    return q, k, v, kv_valid
+
+
+def test_prefill_attention_matches_the_softmax_model():
+    # the shapes of PrefillAttentionTests.swift:11-16, 81-87, 101-104 (start, chunk, window, hd, nq, nkv)
+    cases = [(0, 3, 0, 8, 4, 2), (4, 3, 0, 8, 4, 2), (2, 4, 16, 8, 4, 2), (7, 4, 5, 8, 4, 2),
+             (1023, 1, 1, 256, 16, 8), (1024, 1, 1, 256, 16, 8), (0, 1, 0, 512, 16, 2), (3, 1, 0, 512, 16, 2),
+             (1023, 4, 1024, 256, 16, 8), (31, 8, 0, 512, 16, 2)]
+    for n, (start, chunk, window, hd, nq, nkv) in enumerate(cases):
+        q, k, v, kv_valid = _prefill_fixture(0xA510 + n, start, chunk, hd, nq, nkv)
+        got = O.attention_prefill_causal(q, k, v, 32, nq, nkv, hd, start, kv_valid, 1.0, window=window)
+        want = _prefill_model_f64(q, k, v, nq, nkv, hd, start, kv_valid, window, 1.0)
+        assert np.abs(got - want).max() < 2e-6, (start, chunk, window)
+        # query t alone is the decode call over its own key range
+        for t in range(chunk):
+            a = start + t
+            first = max(0, a + 1 - window) if window else 0
+            one = O.attention_decode(q[t], k, v, 32, nq, nkv, hd, a + 1, 1.0, kv_start=first)
+            assert np.abs(one.reshape(-1) - got[t]).max() < 2e-6
+
+
+def test_prefill_attention_masks_future_and_invalid_keys():
+    # PrefillAttentionTests.swift:58-77: the chunk's own later rows carry huge scores; a query must not see them
+    start, chunk, hd, nq, nkv = 5, 4, 8, 4, 2
+    q, k, v, kv_valid = _prefill_fixture(0xA620, start, chunk, hd, nq, nkv)
+    for row in range(start, kv_valid):
+        k[row] = np.tile((row - start + 1) * 2.0 + np.arange(hd) * 0.125, nkv)
+        v[row] = np.tile((row - start + 1) * -2.0 - np.arange(hd) * 0.125, nkv)
+    got = O.attention_prefill_causal(q, k, v, 32, nq, nkv, hd, start, kv_valid, 1.0)
+    want = _prefill_model_f64(q, k, v, nq, nkv, hd, start, kv_valid, 0, 1.0)
+    assert np.abs(got - want).max() < 1e-5
+    # rows past a query's own position may hold anything, NaN included
+    k2, v2 = k.copy(), v.copy()
+    k2[start + 1:], v2[start + 1:] = np.nan, np.nan
+    first = O.attention_prefill_causal(q[:1], k2, v2, 32, nq, nkv, hd, start, kv_valid, 1.0)
+    assert np.array_equal(first, got[:1])
+    # kv_valid below the causal limit clamps the range (prefill.metal:765): rows >= kv_valid unseen
+    q3, k3, v3, _ = _prefill_fixture(77, 6, 3, 8, 4, 2, extra_kv=0)
+    got3 = O.attention_prefill_causal(q3, k3, v3, 32, 4, 2, 8, 6, 7, 1.0)     # all three queries see keys [0, 7)
+    want3 = _prefill_model_f64(q3, k3, v3, 4, 2, 8, 6, 7, 0, 1.0)
+    assert np.abs(got3 - want3).max() < 2e-6
+    assert np.abs(got3[1] - O.attention_decode(q3[1], k3, v3, 32, 4, 2, 8, 7, 1.0).reshape(-1)).max() < 2e-6
+
+
+def test_prefill_attention_ring_and_quantized_rows():
+    # PrefillAttentionTests.swift:27-56: rows stored at p % capacity give the linear answer
+    start, chunk, window, hd, nq, nkv, cap = 20, 4, 8, 32, 4, 2, 16
+    q, k, v, kv_valid = _prefill_fixture(0xA611, start, chunk, hd, nq, nkv)
+    k_ring, v_ring = np.zeros((cap, nkv * hd), np.float32), np.zeros((cap, nkv * hd), np.float32)
+    for p in range(kv_valid):
+        k_ring[p % cap], v_ring[p % cap] = k[p], v[p]
+    linear = O.attention_prefill_causal(q, k, v, 32, nq, nkv, hd, start, kv_valid, 1.0, window=window)
+    ring = O.attention_prefill_causal(q, k_ring, v_ring, 32, nq, nkv, hd, start, kv_valid, 1.0, window=window,
+                                      ring=cap)
+    assert np.array_equal(ring, linear)
+    # quantized rows: the answer over the dequantized rows (KVCacheQuantizedAttentionTests.swift:91-157)
+    hd, nq, nkv, start, chunk = 256, 16, 2, 4, 4
+    q, k, v, kv_valid = _prefill_fixture(0x5052, start, chunk, hd, nq, nkv, lo=-0.5, hi=0.5)
+    scale = 1.0 / np.sqrt(hd)
+    dense = O.attention_prefill_causal(q, k, v, 32, nq, nkv, hd, start, kv_valid, scale)
+    for bits, tol in ((8, 0.025), (4, 0.20)):
+        kr, vr = O.kv_quantize(k, bits), O.kv_quantize(v, bits)
+        got = O.attention_prefill_causal(q, kr, vr, bits, nq, nkv, hd, start, kv_valid, scale)
+        deq = O.attention_prefill_causal(q, O.kv_dequant(kr, nkv * hd, bits), O.kv_dequant(vr, nkv * hd, bits), 32,
+                                         nq, nkv, hd, start, kv_valid, scale)
+        assert np.array_equal(got, deq)
+        rel = O.rel_error(got, dense)                    # RelError.swift:5-16
+        assert rel < tol, (bits, rel)
