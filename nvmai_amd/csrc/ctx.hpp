@@ -107,6 +107,15 @@ int expert_ffn_dense(nvmai_hip_ctx* ctx, hipStream_t s, const uint8_t* blob, con
 int dense_bf16_gemv(nvmai_hip_ctx* ctx, hipStream_t s, const uint16_t* w, const void* x, uint32_t x_stride,
                     uint32_t n_tokens, uint32_t m, uint32_t n, void* y, float* y_f32, uint32_t y_stride);
 
+// Affine 4 / 8-bit rows against 1 .. 32 input rows on the matrix cores, the matrix read once
+// (gemv_mfma_api.hip).  gemv_mfma_ok: the shapes and alignments it takes.
+bool gemv_mfma_ok(const uint8_t* w, const uint16_t* s, const uint16_t* b, uint32_t bits, const void* x,
+                  uint32_t x_stride, uint32_t n_tokens, uint32_t m, uint32_t n, const void* y, const float* y_f32,
+                  uint32_t y_stride);
+int gemv_mfma(nvmai_hip_ctx* ctx, hipStream_t s, const uint8_t* w, const uint16_t* scales, const uint16_t* biases,
+              uint32_t bits, const void* x, uint32_t x_stride, uint32_t n_tokens, uint32_t m, uint32_t n, void* y,
+              float* y_f32, uint32_t y_stride);
+
 inline int launch_status() { return hipGetLastError() == hipSuccess ? NVMAI_OK : NVMAI_ERR_HIP; }
 
 }  // namespace nvmai

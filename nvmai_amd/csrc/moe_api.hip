@@ -254,6 +254,13 @@ bool launch_dense_rows_t(RowsParams& p, int maxtok, uint32_t ents, hipStream_t s
         return true;                                                                               \
     } while (0)
     const bool few = ents <= 40;      // the same block shapes as the work-list launches
+    // a projection of a decode step (a few thousand rows): blocks of 8 or 16 rows, so that the
+    // launch covers the device; the long blocks below are for matrices like the LM head
+    const uint64_t total_rows = (uint64_t)ents * p.rows;
+    if (total_rows <= 4096 && chunks == 64) NVMAI_DENSE(64, 1, 1, 2);
+    if (total_rows <= 4096 && chunks == 128) NVMAI_DENSE(64, 2, 1, 2);
+    if (total_rows <= 16384 && chunks == 64) NVMAI_DENSE(64, 1, 2, 2);
+    if (total_rows <= 16384 && chunks == 128) NVMAI_DENSE(64, 2, 1, 4);
     if (few && chunks == 16) NVMAI_DENSE(16, 1, 1, 2);
     if (few && chunks == 32) NVMAI_DENSE(32, 1, 2, 2);
     if (chunks == 16) NVMAI_DENSE(16, 1, 2, 2);
@@ -578,6 +585,11 @@ extern "C" int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, co
         return nvmai::dense_bf16_gemv(ctx, (hipStream_t)stream, reinterpret_cast<const uint16_t*>(weights), x, x_stride,
                                       n_tokens, m, n, y, y_f32, y_stride);
     }
+    // Five to 32 input rows: the matrix-core GEMV reads the matrix once for all of them.
+    if (ctx && n_tokens > 4 && n_tokens <= 32 &&
+        nvmai::gemv_mfma_ok(weights, scales, biases, bits, x, x_stride, n_tokens, m, n, y, y_f32, y_stride))
+        return nvmai::gemv_mfma(ctx, (hipStream_t)stream, weights, scales, biases, bits, x, x_stride, n_tokens, m, n, y,
+                                y_f32, y_stride);
     // More than four input rows of a large matrix: the row engine would stream the matrix once per
     // four rows; the matrix-core product reads and dequantizes it once (from five rows on it is
     // the faster of the two at LM-head sizes).  Only where its preconditions hold and 16-bit

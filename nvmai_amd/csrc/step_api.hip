@@ -11,6 +11,8 @@ bool rms_staged_ok(const void* a, uint32_t a_stride, const void* b, uint32_t b_s
     return d % 8 == 0 && d <= 6144 && aligned16(a) && a_stride % 8 == 0 && (!b || (aligned16(b) && b_stride % 8 == 0)) &&
            aligned16(c) && c_stride % 8 == 0 && (!weight || aligned16(weight));
 }
+// Up to this many 2048-wide rows take one wave per block and row with no LDS (rms_direct_kernel).
+constexpr uint32_t RMS_DIRECT_ROWS = 256;
 }  // namespace
 
 extern "C" int nvmai_hip_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* x, uint32_t x_stride,
@@ -22,9 +24,11 @@ extern "C" int nvmai_hip_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const 
     const dim3 grid((rows + 3) / 4);
     const bool staged = rms_staged_ok(x, x_stride, nullptr, 0, out, out_stride, weight, d);
     const size_t lds = staged ? (size_t)d * 10 : 0;
+    const bool direct = d == 2048 && rows <= RMS_DIRECT_ROWS;
 #define NVMAI_RMS(ACT)                                                                                              \
     do {                                                                                                            \
-        if (staged && d == 2048) rmsnorm_kernel<ACT, true, 2048><<<grid, 256, lds, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps); \
+        if (direct) rms_direct_kernel<ACT, 2048, false><<<rows, 64, 0, s>>>((uint16_t*)x, x_stride, nullptr, 0, weight, (uint16_t*)out, out_stride, eps); \
+        else if (staged && d == 2048) rmsnorm_kernel<ACT, true, 2048><<<grid, 256, lds, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps); \
         else if (staged) rmsnorm_kernel<ACT, true, 0><<<grid, 256, lds, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps); \
         else rmsnorm_kernel<ACT, false, 0><<<grid, 256, 0, s>>>((const uint16_t*)x, x_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);        \
     } while (0)
@@ -44,9 +48,11 @@ extern "C" int nvmai_hip_residual_add_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream s
     const dim3 grid((rows + 3) / 4);
     const bool staged = rms_staged_ok(hidden, hidden_stride, delta, delta_stride, out, out_stride, weight, d);
     const size_t lds = staged ? (size_t)d * 10 : 0;
+    const bool direct = d == 2048 && rows <= RMS_DIRECT_ROWS;
 #define NVMAI_RES(ACT)                                                                                              \
     do {                                                                                                            \
-        if (staged && d == 2048) residual_add_rmsnorm_kernel<ACT, true, 2048><<<grid, 256, lds, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta, delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps); \
+        if (direct) rms_direct_kernel<ACT, 2048, true><<<rows, 64, 0, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta, delta_stride, weight, (uint16_t*)out, out_stride, eps); \
+        else if (staged && d == 2048) residual_add_rmsnorm_kernel<ACT, true, 2048><<<grid, 256, lds, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta, delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps); \
         else if (staged) residual_add_rmsnorm_kernel<ACT, true, 0><<<grid, 256, lds, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta, delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps); \
         else residual_add_rmsnorm_kernel<ACT, false, 0><<<grid, 256, 0, s>>>((uint16_t*)hidden, hidden_stride, (const uint16_t*)delta, delta_stride, weight, (uint16_t*)out, out_stride, rows, d, eps);        \
     } while (0)

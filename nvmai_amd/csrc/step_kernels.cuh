@@ -127,6 +127,51 @@ __global__ __launch_bounds__(256) void residual_add_rmsnorm_kernel(uint16_t* hid
                          out + (size_t)row * out_stride, d, eps, rms_lds + wave * d, lane);
 }
 
+// A few rows of a width known at compile time (a decode step's hidden rows): one wave per block and
+// row, no LDS.  Lane l loads its elements l, l + 64, ... with two-byte loads -- the 64 lanes of one
+// instruction read 128 contiguous bytes, and with the width fixed all of a lane's loads (row,
+// delta, weight) are in flight together, so the kernel is one trip to memory, the fma chain, the
+// butterfly and the stores.  Same arithmetic and order as rms_row.
+template <int ACT, int DFIX, bool RESIDUAL>
+__global__ __launch_bounds__(64) void rms_direct_kernel(uint16_t* x, uint32_t x_stride, const uint16_t* delta,
+                                                        uint32_t delta_stride, const uint16_t* weight, uint16_t* out,
+                                                        uint32_t out_stride, float eps) {
+    constexpr int N = DFIX / 64;
+    const uint32_t row = blockIdx.x, lane = threadIdx.x;
+    uint16_t* xr = x + (size_t)row * x_stride;
+    const uint16_t* dr = RESIDUAL ? delta + (size_t)row * delta_stride : nullptr;
+    uint16_t* o = out + (size_t)row * out_stride;
+    uint16_t xv[N], dv[N], wv[N];
+#pragma unroll
+    for (int j = 0; j < N; ++j) xv[j] = xr[lane + 64 * j];
+    if (RESIDUAL) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) dv[j] = dr[lane + 64 * j];
+    }
+    if (weight) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) wv[j] = weight[lane + 64 * j];
+    }
+    float v[N];
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        if (RESIDUAL) {
+            xv[j] = f32_to_act<ACT>(__fadd_rn(act_to_f32<ACT>(xv[j]), act_to_f32<ACT>(dv[j])));
+            xr[lane + 64 * j] = xv[j];
+        }
+        v[j] = act_to_f32<ACT>(xv[j]);
+        acc = fmaf(v[j], v[j], acc);
+    }
+    const float inv = rms_inverse(rms_wave_sum(acc), DFIX, eps);
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        float y = __fmul_rn(v[j], inv);
+        if (weight) y = __fmul_rn(y, bf16_to_f32(wv[j]));
+        o[lane + 64 * j] = f32_to_act<ACT>(y);
+    }
+}
+
 // ---- epilogue of the fused q / k / v projection of a full-attention layer --------------------------
 // One wave per head of one token, replacing split_q_gate + rmsnorm_bf16w_perhead (q, k) + rope_neox_subdim
 // (q, k) (RealForwardRunner.swift:2213-2255; the reference's own fusion of the norm and the rotation is

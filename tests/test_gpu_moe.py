@@ -84,6 +84,42 @@ def test_affine_gemv_matches_oracle(nv, ctx, bits, m, n, tokens):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
+def test_affine_gemv_small_batch_on_the_matrix_cores(nv, ctx, bits):
+    # 5 .. 32 input rows against rows of whole 512-code stages: the matrix is read once for all of
+    # them.  Ragged row counts (last block, last wave, last four rows), one and two token tiles,
+    # one and two input panels, padded output rows, an all-zero input row and one with a huge entry
+    rng = np.random.default_rng(300 + bits)
+    for m, n, tokens in [(64, 512, 5), (100, 1024, 16), (203, 2048, 17), (2048, 4096, 9), (1001, 2048, 32),
+                         (130, 4096, 31), (12352, 2048, 16)]:
+        say("gemv mfma", ctx.act, bits, m, n, tokens)
+        p, s, b = O.quantize_affine(gauss(rng, (m, n), 0.05), bits)
+        x = gauss(rng, (tokens, n))
+        x[1] = 0.0
+        x[2, 7] = 3.0e4 if ctx.act == 1 else 1.0e30
+        x[3] *= 1e-3
+        x = round_act(x, ctx.act)
+        want = np.stack([O.affine_gemv(p, s, b, x[t], bits) for t in range(tokens)])
+        stride = m + 12
+        y = torch.full((tokens, stride), 7.0, dtype=ctx.dtype, device="cuda")
+        yf = torch.full((tokens, stride), 7.0, dtype=torch.float32, device="cuda")
+        pd, sd, bd = dev(p), dev(s.view(np.int16)), dev(b.view(np.int16))
+        nv.affine_gemv(ctx, pd, sd, bd, bits, act_tensor(x, ctx), m, n, y=y, y_f32=yf)
+        torch.cuda.synchronize()
+        got32, got16 = yf[:, :m].cpu().numpy(), act_np(y[:, :m])
+        for t in range(tokens):                         # per input row: a small row must not hide behind a large one
+            assert O.rel_error(got32[t], want[t]) < TOL_F32, (m, n, tokens, t)
+            if np.isfinite(round_act(want[t], ctx.act)).all():
+                assert O.rel_error(got16[t], want[t]) < TOL_ACT, (m, n, tokens, t)
+        assert not got32[1].any()
+        assert (yf[:, m:] == 7.0).all() and (y[:, m:].float() == 7.0).all()     # padding untouched
+        # the same product through the row engine (four rows at a time): both paths within the bar of each other
+        y4 = torch.cat([nv.affine_gemv(ctx, pd, sd, bd, bits, act_tensor(x[t0:t0 + 4], ctx), m, n, out_f32=True)
+                        for t0 in range(0, tokens, 4)])
+        torch.cuda.synchronize()
+        assert O.rel_error(got32, y4.cpu().numpy()) < TOL_F32
+
+
+@pytest.mark.parametrize("bits", [4, 8])
 def test_affine_gemv_both_outputs_padded_stride(nv, ctx, bits):
     # 16-bit and fp32 results in one call, rows of the outputs further apart than m; shapes with a
     # single-launch instantiation (any chunk count 16 / 32 / 64 / 128) and one without (n = 192)

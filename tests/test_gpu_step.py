@@ -36,7 +36,7 @@ def _bits(t):
 
 
 # ------------------------------------------------------------------ RMSNorm
-@pytest.mark.parametrize("rows,d", [(1, 256), (1, 2048), (3, 2816), (16, 256), (5, 100), (9, 64)])
+@pytest.mark.parametrize("rows,d", [(1, 256), (1, 2048), (16, 2048), (300, 2048), (3, 2816), (16, 256), (5, 100), (9, 64)])
 def test_rmsnorm_bit_exact(nv, ctx, rows, d):
     say("rmsnorm", ctx.act, rows, d)
     rng = np.random.default_rng(rows * 31 + d)
