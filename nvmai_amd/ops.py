@@ -224,13 +224,18 @@ class MoE:
 
 
 def moe_layer_desc(d, f, num_experts, top_k, bits, router, experts, shared_blob=None, shared_gate=None,
-                   eff_scale=None, per_expert_scale=None):
-    """Fill an nvmai_moe_layer.  experts: uint8 tensor [num_experts, stride] (resident pool)."""
+                   eff_scale=None, per_expert_scale=None, offsets=None):
+    """Fill an nvmai_moe_layer.  experts: uint8 tensor [num_experts, stride] (resident pool).
+    offsets: the nine sub-tensor offsets inside a blob when they come from a packed-experts layout
+    (Model.routedExpertOffsets); default = CPUExpertFFN.Offsets(d:f:)."""
     L = MoeLayer()
     L.d, L.f, L.num_experts, L.top_k, L.bits = d, f, num_experts, top_k, bits
     L.router = router
     L.experts_base, L.expert_stride = experts.data_ptr(), experts.stride(0)
-    L.offsets, _ = expert_offsets(d, f, bits)
+    if offsets is None:
+        L.offsets, _ = expert_offsets(d, f, bits)
+    else:
+        L.offsets = ExpertOffsets(*[int(v) for v in offsets])
     L.shared_blob = 0 if shared_blob is None else shared_blob.data_ptr()
     if shared_gate is not None:
         L.shared_gate = shared_gate

@@ -1,0 +1,79 @@
+"""GPU: a model directory in the reference's .gturbo format (written here from quantized random
+weights, experts stored in a permuted physical order) is read into HBM by nvmai_amd.gturbo and
+driven through the decode layer; the result is compared with the oracle over the arrays the
+directory was written from.  No model file of the reference is available offline, so the weights are
+synthetic; the format rules themselves are pinned on the CPU in tests/test_gturbo_format.py."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from gpu_util import act_np, act_tensor, gauss, round_act, say, u16, u32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_model_directory_to_decode_layer(tmp_path, bits):
+    import nvmai_amd as nv
+    from nvmai_amd import gturbo as G
+    say("gturbo directory -> decode layer", bits)
+    rng = np.random.default_rng(70 + bits)
+    d, f, E, k, layers = 256, 128, 16, 4, 2
+    mk = lambda r, c, s=0.05: O.round_bf16(gauss(rng, (r, c), s))
+    roles = ["gate", "gate_scales", "gate_biases", "up", "up_scales", "up_biases", "down", "down_scales", "down_biases"]
+    off = O.expert_offsets(d, f, bits)                     # CPUExpertFFN.Offsets: the order the repack tool writes
+    sizes = [f * d * bits // 8, f * (d // 64) * 2, f * (d // 64) * 2] * 2 + [d * f * bits // 8, d * (f // 64) * 2, d * (f // 64) * 2]
+    shapes = [(f, d), (f, d // 64), (f, d // 64)] * 2 + [(d, f), (d, f // 64), (d, f // 64)]
+    tensors = {r: G.SubTensorEntry(int(off[i]), sizes[i], "BF16" if "_" in r else "U32", shapes[i], None if "_" in r else bits)
+               for i, r in enumerate(roles)}
+    used = int(off[8]) + sizes[8]
+    stride = (used + G.ALIGNMENT_BYTES - 1) // G.ALIGNMENT_BYTES * G.ALIGNMENT_BYTES
+    ranks = list(rng.permutation(E))
+    lays, resident, truth = [], [], []
+    for L in range(layers):
+        blobs = np.zeros((E, stride), np.uint8)
+        for e in range(E):
+            blobs[e, :used] = O.pack_expert(mk(f, d), mk(f, d), mk(d, f), bits)[:used]
+        lays.append({"blobs": blobs, "tensors": tensors, "ranks": [int(r) for r in ranks]})
+        p = "language_model.model.layers.%d.mlp." % L
+        router = O.bf16_bits(mk(E, d, 0.02))
+        resident.append((p + "gate.weight", 1, (E, d), router.tobytes(), None, None))
+        shared = []
+        for proj, (rows, cols) in (("gate_proj", (f, d)), ("up_proj", (f, d)), ("down_proj", (d, f))):
+            q = O.quantize_affine(mk(rows, cols), bits)
+            shared.append(q)
+            resident.append((p + "shared_expert.%s.weight" % proj, 0, (rows, cols), q[0].tobytes(), q[1].tobytes(), q[2].tobytes()))
+        gate = O.quantize_affine(mk(1, d), bits)
+        resident.append((p + "shared_expert_gate.weight", 0, (1, d), gate[0].tobytes(), gate[1].tobytes(), gate[2].tobytes()))
+        truth.append((router, blobs, shared, gate))
+    slot = lambda b: {"weightBits": b, "scheme": "affine", "scaleType": "bf16", "biasType": "bf16", "groupSize": 64}
+    quant = {n: slot(bits) for n in ("embedding", "attention", "router", "sharedExpert", "routedExpert")}
+    arch = {"hiddenSize": d, "ffnIntermediate": 4 * d, "moeIntermediateSize": f, "numHeads": 4, "numKVHeads": 2,
+            "numFullKVHeads": 2, "headDim": 64, "fullHeadDim": 64, "vocabSize": 1000, "slidingWindow": 0,
+            "finalLogitSoftcap": 0.0, "ropeTheta": 1e4, "fullRopeTheta": 1e7, "partialRotaryFactor": 0.25,
+            "numLayers": layers, "numExperts": E, "topKExperts": k, "tieWordEmbeddings": False, "attentionKEqV": False,
+            "hiddenActivation": "silu", "fullAttentionLayerMask": [0, 1]}
+    G.write_model(str(tmp_path), arch, quant, lays, resident)
+
+    model = G.GTurboModel(str(tmp_path))
+    ctx = nv.Context(0, 0)
+    x = round_act(gauss(rng, (5, d)), 0)
+    for L in range(layers):
+        pool = model.expert_pool(L)
+        assert pool.shape == (E + 1, stride)
+        assert np.array_equal(pool[:E].cpu().numpy(), lays[L]["blobs"])        # logical order in HBM
+        desc, keep = model.moe_layer(L, pool)
+        y, idx, w = nv.MoE(ctx, bits).decode_layer(desc, act_tensor(x, ctx), want_routes=True)
+        torch.cuda.synchronize()
+        router, blobs, shared, gate = truth[L]
+        shared_blob = np.zeros(stride, np.uint8)
+        for i, q in enumerate(shared):
+            for arr, at in zip(q, (int(off[3 * i]), int(off[3 * i + 1]), int(off[3 * i + 2]))):
+                raw = arr.view(np.uint8).reshape(-1)
+                shared_blob[at:at + raw.size] = raw
+        io, wo, yo = O.moe_layer_forward(x, d, f, k, bits, (16, router, None, None), blobs, shared_blob, (bits,) + gate)
+        assert np.array_equal(u32(idx), io), "routing indices"
+        assert np.abs(u16(w).astype(np.int32) - wo.astype(np.int32)).max() <= 1
+        assert O.rel_error(act_np(y), yo) < 1e-2
+    ctx.close()
