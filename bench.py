@@ -170,9 +170,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # under profiles/ it was read from and goes stale when its kernel changes.  Keyed by (workload,
 # bits, batch or tokens); other configurations report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("decode", 8, 32): ((181300 * 2.00 + 1196 * 1.00) * 1024, "profiles/expert_rows_fast_decode_configs1_8bit_batch32.txt"),
-    ("prefill", 4, 4096): ((279700 * 2.00 + 36140 * 1.00) * 1024, "profiles/prefill_gemm_kernel_configs2_4bit_4096tokens.txt"),
-    ("attention", 8, 8, 131072): ((599800 * 2.00 + 4383 * 1.00) * 1024, "profiles/attn_partial_mfma_kernel_configs3_8bit_128k_batch8.txt"),
+    ("decode", 8, 32): ((181300 * 2.00 + 1229 * 1.00) * 1024, "profiles/expert_rows_fast_decode_configs1_8bit_batch32.txt"),
+    ("prefill", 4, 4096): ((279390 * 2.00 + 36142 * 1.00) * 1024, "profiles/prefill_gemm_kernel_configs2_4bit_4096tokens.txt"),
+    ("attention", 8, 8, 131072): ((565650 * 2.00 + 4383 * 1.00) * 1024, "profiles/attn_partial_mfma_kernel_configs3_8bit_128k_batch8.txt"),
     ("attention", 4, 8, 131072): ((295900 * 2.00 + 4356 * 1.00) * 1024, "profiles/attn_partial_mfma_kernel_configs3_8bit_128k_batch8.txt"),
 }
 
@@ -478,16 +478,15 @@ def run_sampler(nv, ctx, torch, a):
     probs = torch.empty((rows, V), dtype=torch.float16, device="cuda")
     seeds = [nv.sampler_seed_for(1234, r) for r in range(rows)]
 
-    qmm = nv.MPPPrefillInt4QMM(ctx, bits)
     logits_buf = torch.empty((rows, V), dtype=torch.bfloat16, device="cuda")
 
     def head(i):
-        # a few rows: the GEMV (each weight row read once per group of 4 inputs); more: the
-        # matrix-core product (weights read and dequantized once for all rows)
+        # the GEMV entry point: the row engine for 1-4 rows; for more rows it hands a matrix of this
+        # size to the dense matrix-core product (weights read and dequantized once for all rows)
         p_, s_, b_ = heads[i % n_heads]
         if rows <= 4:
             return nv.affine_gemv(ctx, p_, s_, b_, bits, xs[i % 8], V, D)
-        return qmm.encode(p_, s_, b_, xs[i % 8], V, D, logits_buf)
+        return nv.affine_gemv(ctx, p_, s_, b_, bits, xs[i % 8], V, D, y=logits_buf)[0]
 
     def step(i):
         logits = head(i)

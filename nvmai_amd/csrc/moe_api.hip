@@ -585,8 +585,11 @@ extern "C" int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, co
         return nvmai::dense_bf16_gemv(ctx, (hipStream_t)stream, reinterpret_cast<const uint16_t*>(weights), x, x_stride,
                                       n_tokens, m, n, y, y_f32, y_stride);
     }
-    // Five to 32 input rows: the matrix-core GEMV reads the matrix once for all of them.
-    if (ctx && n_tokens > 4 && n_tokens <= 32 &&
+    // Five to 32 input rows against a projection-sized matrix: the matrix-core GEMV reads the matrix
+    // once for all of them.  (Every block of it stages the inputs for itself, which a matrix of
+    // LM-head size pays thousands of times: 165 / 280 us at 16 / 32 rows against 116 us through the
+    // dense product below -- so that one keeps the large matrices unless fp32 results are asked for.)
+    if (ctx && n_tokens > 4 && n_tokens <= 32 && (m < 32768 || y_f32 || !y) &&
         nvmai::gemv_mfma_ok(weights, scales, biases, bits, x, x_stride, n_tokens, m, n, y, y_f32, y_stride))
         return nvmai::gemv_mfma(ctx, (hipStream_t)stream, weights, scales, biases, bits, x, x_stride, n_tokens, m, n, y,
                                 y_f32, y_stride);
