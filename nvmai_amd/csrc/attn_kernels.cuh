@@ -317,6 +317,10 @@ __device__ __forceinline__ f4_t mfma16(const H8& a, const H8& b, f4_t c) {
 // s_waitcnt operand: at most n vector-memory loads still in flight, the other counters free.
 constexpr int gemm_like_vmcnt(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
+// e^x for x <= 0 in two instructions (a multiply and the hardware's 2^x, good to about one ulp; -inf gives
+// 0): the library's expf costs a dozen, and the softmax of a step needs nine of them per lane.
+__device__ __forceinline__ float attn_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+
 constexpr int ATTN_HD = 256;
 constexpr int ATTN_STEP = 32;
 
@@ -377,42 +381,6 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
     const uint32_t meta_bi = p.f.value_bytes + 2 * groups_total + 2 * (kvh * 4);
     const uint8_t* kbase = p.k + b * p.kv_batch_stride;
     const uint8_t* vbase = p.v + b * p.kv_batch_stride;
-
-    auto slot_tok = [&](int t) { return (uint32_t)((t >> 2) * 16 + 4 * r + (t & 3)); };   // token of slot t inside the step
-    // Buffer loads: a scalar resource per cache, 32-bit offsets; reads past the end of the
-    // sequence's rows return zero instead of faulting (tokens past the chunk are masked anyway).
-    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(kbase), 0, (int)(p.seq_len * p.f.stride), 0x00020000);
-    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(vbase), 0, (int)(p.seq_len * p.f.stride), 0x00020000);
-    // One load instruction moves 1 KB = the codes of 4 (8 bit) or 8 (4 bit) tokens: lane l takes
-    // chunk (l % LPT) ^ token of token l / LPT, which lands in slot l % LPT of that token.
-    constexpr int LPT = CODE_ROW / 16;                              // lanes (16-byte chunks) per token
-    constexpr int TPI = 64 / LPT;                                   // tokens per instruction
-    const uint32_t d_tok = lane / LPT, d_slot = lane % LPT;
-    const uint32_t d_chunk16 = ((d_slot ^ d_tok) & (LPT - 1)) * 16u;  // 8 bit: ^ 64 (j & 3) per instruction
-    const uint32_t m_part = (lane & 3) < 2 ? meta_sc + 4 * (lane & 3) : meta_bi + 4 * ((lane & 3) - 2);
-    uint8_t* const myk = kst + wave * REGION;
-    uint8_t* const myv = vst + wave * REGION;
-    constexpr int N_LOADS = 32 / TPI + 2;                           // load instructions of one region
-    auto issue_region = [&](uint32_t s0, const __amdgpu_buffer_rsrc_t& rs, uint8_t* st) {
-        const uint32_t row = (s0 + d_tok) * p.f.stride;
-#pragma unroll
-        for (int j = 0; j < 32 / TPI; ++j) {
-            const uint32_t voff = row + (BITS == 8 ? (d_chunk16 ^ (64u * (j & 3))) : d_chunk16);
-            const uint32_t soff = (uint32_t)(j * TPI) * p.f.stride + code_off;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(st + j * 1024), 16, voff, soff, 0, 0);
-        }
-        const uint32_t mrow = (s0 + (lane >> 2)) * p.f.stride + m_part;
-#pragma unroll
-        for (int m = 0; m < 2; ++m)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(st + OFF_META + m * 256), 4, mrow,
-                                                     (uint32_t)(16 * m) * p.f.stride, 0, 0);
-    };
-    // the first step's rows are requested before the queries are prepared: neither depends on the other
-    const uint32_t s_first = p0 + wave * ATTN_STEP;
-    if (s_first < p1) { issue_region(s_first, krsrc, myk); issue_region(s_first, vrsrc, myv); }
-
 
     // ---- Q: head i (zero for i >= qpk), scaled to fp16; operands and per-group sums
     H8 qop[4][2];
@@ -476,6 +444,42 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
         for (int n = 0; n < 4; ++n) oacc[g][n] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
     float m_run = -INFINITY, d_run = 0.0f;                          // head i; d over this lane's tokens only
     float corr[4] = {0.0f, 0.0f, 0.0f, 0.0f};                       // head i, this lane's tokens only
+
+    auto slot_tok = [&](int t) { return (uint32_t)((t >> 2) * 16 + 4 * r + (t & 3)); };   // token of slot t inside the step
+    // Buffer loads: a scalar resource per cache, 32-bit offsets; reads past the end of the
+    // sequence's rows return zero instead of faulting (tokens past the chunk are masked anyway).
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(kbase), 0, (int)(p.seq_len * p.f.stride), 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(vbase), 0, (int)(p.seq_len * p.f.stride), 0x00020000);
+    // One load instruction moves 1 KB = the codes of 4 (8 bit) or 8 (4 bit) tokens: lane l takes
+    // chunk (l % LPT) ^ token of token l / LPT, which lands in slot l % LPT of that token.
+    constexpr int LPT = CODE_ROW / 16;                              // lanes (16-byte chunks) per token
+    constexpr int TPI = 64 / LPT;                                   // tokens per instruction
+    const uint32_t d_tok = lane / LPT, d_slot = lane % LPT;
+    const uint32_t d_chunk16 = ((d_slot ^ d_tok) & (LPT - 1)) * 16u;  // 8 bit: ^ 64 (j & 3) per instruction
+    const uint32_t m_part = (lane & 3) < 2 ? meta_sc + 4 * (lane & 3) : meta_bi + 4 * ((lane & 3) - 2);
+    uint8_t* const myk = kst + wave * REGION;
+    uint8_t* const myv = vst + wave * REGION;
+    constexpr int N_LOADS = 32 / TPI + 2;                           // load instructions of one region
+    auto issue_region = [&](uint32_t s0, const __amdgpu_buffer_rsrc_t& rs, uint8_t* st) {
+        const uint32_t row = (s0 + d_tok) * p.f.stride;
+#pragma unroll
+        for (int j = 0; j < 32 / TPI; ++j) {
+            const uint32_t voff = row + (BITS == 8 ? (d_chunk16 ^ (64u * (j & 3))) : d_chunk16);
+            const uint32_t soff = (uint32_t)(j * TPI) * p.f.stride + code_off;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(st + j * 1024), 16, voff, soff, 0, 0);
+        }
+        const uint32_t mrow = (s0 + (lane >> 2)) * p.f.stride + m_part;
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(st + OFF_META + m * 256), 4, mrow,
+                                                     (uint32_t)(16 * m) * p.f.stride, 0, 0);
+    };
+    // (requested after the query loads: loads return in order, and the queries' preparation then
+    // overlaps the flight of the rows -- the other order was measured 0.7 us slower per launch)
+    const uint32_t s_first = p0 + wave * ATTN_STEP;
+    if (s_first < p1) { issue_region(s_first, krsrc, myk); issue_region(s_first, vrsrc, myv); }
 
     for (uint32_t s0 = s_first; s0 < p1; s0 += 4 * ATTN_STEP) {
         const bool more = s0 + 4 * ATTN_STEP < p1;                  // wave-uniform
@@ -552,10 +556,10 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
         mx = fmaxf(mx, shfl_xor_f(mx, 32));
         const float m_new = fmaxf(m_run, mx);                       // -inf while the column has seen no key yet
         const bool none = m_new == -INFINITY;
-        const float alpha = none ? 1.0f : expf(m_run - m_new);
+        const float alpha = none ? 1.0f : attn_exp(m_run - m_new);
         float pe[8], psum = 0.0f;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) { pe[t] = none ? 0.0f : expf(sv[t] - m_new); psum += pe[t]; }
+        for (int t = 0; t < 8; ++t) { pe[t] = none ? 0.0f : attn_exp(sv[t] - m_new); psum += pe[t]; }
         d_run = d_run * alpha + psum;
         m_run = m_new;
 
