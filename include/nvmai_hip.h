@@ -214,6 +214,24 @@ int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream stream, const nv
                                uint32_t y_stride, uint32_t* out_idx, uint16_t* out_w,
                                uint32_t* stats);
 
+/* The MoE block of a layer together with the residual add and the RMSNorm that open it
+ * (RealForwardRunner's encodeResidualAdd, utility.metal:95-104, RMSNorm.encodeBF16W,
+ * rmsnorm.metal:64-110, then the MoE calls of nvmai_hip_moe_decode_layer):
+ *   hidden_out = round(hidden + delta)      (delta NULL: hidden_out = hidden)
+ *   normed     = rmsnorm(hidden_out) * norm_weight
+ *   y          = MoE(normed)
+ * with the bits of nvmai_hip_residual_add_rmsnorm followed by nvmai_hip_moe_decode_layer.  Below 64
+ * tokens, with 16-byte aligned rows and hidden_out, normed and hidden three different buffers, the
+ * router launch norms its input itself (one launch fewer per layer); otherwise the steps run one
+ * after the other.  normed is written for the caller too (the reference keeps it for the
+ * shared-expert and the next projections). */
+int nvmai_hip_moe_decode_layer_prenorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_moe_layer* layer,
+                                       const void* hidden, uint32_t hidden_stride, const void* delta,
+                                       uint32_t delta_stride, const uint16_t* norm_weight, float eps,
+                                       void* hidden_out, uint32_t hidden_out_stride, void* normed,
+                                       uint32_t normed_stride, uint32_t n_tokens, void* y, uint32_t y_stride,
+                                       uint32_t* out_idx, uint16_t* out_w, uint32_t* stats);
+
 /* nvmai_hip_moe_decode_layer for callers that cannot allocate.  It has no counterpart in the
  * reference: it is for code under HIP graph capture, tight serving loops and harnesses that
  * forbid hipMalloc.  Same arguments, same results bit for bit, but the step's intermediate

@@ -174,6 +174,20 @@ __device__ __forceinline__ void unpack4(uint32_t w, float* q) {
 }
 
 // Codes per 16-byte chunk.
+// ---- RMSNorm pieces shared by the norm kernels and the kernels that norm their own input ------
+// Sum of squares in a stated order: lane l runs acc = fma(x, x, acc) over the elements l, l + 64,
+// ..., then this xor butterfly 32, 16, 8, 4, 2, 1; mean, sqrt and the divide are single IEEE steps.
+__device__ __forceinline__ float rms_wave_sum(float acc) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) acc = __fadd_rn(acc, shfl_xor_f(acc, off));
+    return acc;
+}
+
+__device__ __forceinline__ float rms_inverse(float sum, uint32_t d, float eps) {
+    const float mean = __fdiv_rn(sum, (float)d);
+    return __fdiv_rn(1.0f, sqrtf(__fadd_rn(mean, eps)));     // sqrtf: correctly rounded (the _rn intrinsic is not)
+}
+
 template <int BITS>
 struct Chunk { static constexpr int elems = 128 / BITS; };
 

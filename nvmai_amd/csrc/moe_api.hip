@@ -334,7 +334,8 @@ uint32_t rows_chunks(int kind, uint32_t d) { return kind == 16 ? d / 8 : (kind =
 
 template <int ACT>
 void run_router_t(const RouterParams& rp, uint32_t cpl, dim3 grid, hipStream_t s) {
-    const size_t lds = (size_t)ROUTER_TOK * rp.d * 2;             // the block's token rows
+    // the block's token rows (+ the raw row and the inverse norm of the prologue)
+    const size_t lds = (size_t)ROUTER_TOK * rp.d * 2 + (rp.pre_weight ? (size_t)rp.d * 2 + 16 : 0);
     if (cpl <= 1) router_logits_kernel<ACT, 1><<<grid, 256, lds, s>>>(rp);
     else if (cpl <= 2) router_logits_kernel<ACT, 2><<<grid, 256, lds, s>>>(rp);
     else if (cpl <= 4) router_logits_kernel<ACT, 4><<<grid, 256, lds, s>>>(rp);
@@ -943,11 +944,22 @@ struct Carver {
     }
 };
 
+// The residual add + RMSNorm that opens the MoE block, done by the router launch (every block of it
+// norms its token row for itself) instead of a launch of its own.  x of the layer call is then the
+// residual stream; the normed rows land in `normed` for the launches that follow.
+struct PreNorm {
+    const void* delta; uint32_t delta_stride;      // may be null: norm only
+    const uint16_t* weight; float eps;
+    void* hidden_out; uint32_t hidden_out_stride;
+    void* normed; uint32_t normed_stride;
+};
+
 // fixed_ws == nullptr: the buffers come from the context's workspace (grown when needed);
 // otherwise from the fixed_cap bytes at fixed_ws, and a step that needs more is refused.
 int decode_layer_impl(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_moe_layer* L, const void* x,
                       uint32_t x_stride, uint32_t n_tokens, void* y, uint32_t y_stride, uint32_t* out_idx,
-                      uint16_t* out_w, uint32_t* stats, uint8_t* fixed_ws, size_t fixed_cap) {
+                      uint16_t* out_w, uint32_t* stats, uint8_t* fixed_ws, size_t fixed_cap,
+                      const PreNorm* pre = nullptr) {
     if (!ctx || !L || !x || !y) return NVMAI_ERR_INVALID_ARG;
     int rc = check_shape(L->d, L->f, L->bits);
     if (rc) return rc;
@@ -1004,6 +1016,13 @@ int decode_layer_impl(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_moe_l
     if (gated) rp.gate = to_desc(&L->shared_gate);
     rp.x = x; rp.eff_scale = L->eff_scale; rp.x_stride = x_stride; rp.tokens = T;
     rp.num_experts = E; rp.d = D; rp.logits = logits; rp.gate_logit = gate_logit;
+    if (pre) {
+        rp.pre_delta = (const uint16_t*)pre->delta; rp.pre_delta_stride = pre->delta_stride;
+        rp.pre_weight = pre->weight; rp.pre_eps = pre->eps;
+        rp.pre_hidden_out = (uint16_t*)pre->hidden_out; rp.pre_hidden_stride = pre->hidden_out_stride;
+        rp.pre_normed_out = (uint16_t*)pre->normed; rp.pre_normed_stride = pre->normed_stride;
+        x = pre->normed; x_stride = pre->normed_stride;     // what the expert launches read
+    }
     SelectParams sp{logits, L->per_expert_scale, T, E, K, idx, wts};
     GroupParams gp{sp, (uint32_t)maxtok, has_shared ? 1 : 0, entries, n_entries, stats, pair_token, pair_id,
                    ctx->tickets};
@@ -1069,6 +1088,42 @@ extern "C" int nvmai_hip_moe_decode_layer(nvmai_hip_ctx* ctx, nvmai_stream strea
                                           uint32_t n_tokens, void* y, uint32_t y_stride,
                                           uint32_t* out_idx, uint16_t* out_w, uint32_t* stats) {
     return decode_layer_impl(ctx, stream, L, x, x_stride, n_tokens, y, y_stride, out_idx, out_w, stats, nullptr, 0);
+}
+
+extern "C" int nvmai_hip_moe_decode_layer_prenorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_moe_layer* L,
+                                                  const void* hidden, uint32_t hidden_stride, const void* delta,
+                                                  uint32_t delta_stride, const uint16_t* norm_weight, float eps,
+                                                  void* hidden_out, uint32_t hidden_out_stride, void* normed,
+                                                  uint32_t normed_stride, uint32_t n_tokens, void* y,
+                                                  uint32_t y_stride, uint32_t* out_idx, uint16_t* out_w,
+                                                  uint32_t* stats) {
+    if (!ctx || !L || !hidden || !norm_weight || !hidden_out || !normed || !y) return NVMAI_ERR_INVALID_ARG;
+    const uint32_t D = L->d;
+    if (hidden_stride < D || hidden_out_stride < D || normed_stride < D || (delta && delta_stride < D))
+        return NVMAI_ERR_INVALID_ARG;
+    if (n_tokens == 0) return NVMAI_OK;
+    const bool rows16 = aligned16(hidden) && hidden_stride % 8 == 0 && aligned16(hidden_out) && hidden_out_stride % 8 == 0 &&
+                        aligned16(normed) && normed_stride % 8 == 0 && aligned16(norm_weight) && D % 8 == 0 &&
+                        (!delta || (aligned16(delta) && delta_stride % 8 == 0));
+    // the router launch norms for itself when it is the per-token kernel, the rows can be moved 16 bytes
+    // at a time and the updated residual rows do not overwrite the ones other blocks still read
+    if (n_tokens < 64 && rows16 && D <= 8192 && hidden_out != hidden && normed != hidden && normed != hidden_out) {
+        const PreNorm pre{delta, delta_stride, norm_weight, eps, hidden_out, hidden_out_stride, normed, normed_stride};
+        return decode_layer_impl(ctx, stream, L, hidden, hidden_stride, n_tokens, y, y_stride, out_idx, out_w, stats,
+                                 nullptr, 0, &pre);
+    }
+    // otherwise the two steps one after the other
+    if (hidden_out != hidden) {
+        const hipError_t e = hipMemcpy2DAsync(hidden_out, (size_t)hidden_out_stride * 2, hidden, (size_t)hidden_stride * 2,
+                                              (size_t)D * 2, n_tokens, hipMemcpyDeviceToDevice, (hipStream_t)stream);
+        if (e != hipSuccess) return NVMAI_ERR_HIP;
+    }
+    int rc = delta ? nvmai_hip_residual_add_rmsnorm(ctx, stream, hidden_out, hidden_out_stride, delta, delta_stride,
+                                                    norm_weight, normed, normed_stride, n_tokens, D, eps)
+                   : nvmai_hip_rmsnorm(ctx, stream, hidden_out, hidden_out_stride, norm_weight, normed, normed_stride,
+                                       n_tokens, D, eps);
+    if (rc) return rc;
+    return decode_layer_impl(ctx, stream, L, normed, normed_stride, n_tokens, y, y_stride, out_idx, out_w, stats, nullptr, 0);
 }
 
 extern "C" size_t nvmai_hip_moe_decode_layer_noalloc_scratch_bytes(void) { return STATIC_SCRATCH_BYTES; }

@@ -564,6 +564,17 @@ struct RouterParams {
     uint32_t x_stride, tokens, num_experts, d;
     float* logits;                 // [tokens, num_experts]
     float* gate_logit;             // [tokens]
+    // Optional prologue (pre_weight != null): x holds the residual stream's rows and the block's
+    // input row is rmsnorm(round(x + pre_delta)) * pre_weight, computed by every block for itself
+    // with the arithmetic of residual_add_rmsnorm_kernel (same bits); the block of the first rows
+    // also stores the updated residual row to pre_hidden_out (not x: other blocks still read it)
+    // and the normed row to pre_normed_out for the kernels that follow.  Rows 16-byte aligned.
+    const uint16_t* pre_delta;     // [tokens, pre_delta_stride], may be null (norm only)
+    const uint16_t* pre_weight;    // BF16 [d]
+    uint16_t* pre_hidden_out;      // [tokens, pre_hidden_stride]
+    uint16_t* pre_normed_out;      // [tokens, pre_normed_stride]
+    uint32_t pre_delta_stride, pre_hidden_stride, pre_normed_stride;
+    float pre_eps;
 };
 
 // Tokens per block in y.  One: the launch is a chain of latencies (stage the row, load eight
@@ -607,32 +618,122 @@ __device__ __forceinline__ void router_stage_x(const RouterParams& p, uint32_t t
     __syncthreads();
 }
 
+// The same with the prologue: the block's rows are summed with their delta, normed and staged.
+// raw: d 16-bit values of LDS.  A thread keeps its 16-byte pieces of the row in registers between
+// the add and the scaling (d <= 8192), every load is issued before the first use, and every wave
+// sums the squares for itself (the same 64-lane order, so the same bits) -- no broadcast, one
+// barrier less.  Ends with a barrier.
+constexpr int ROUTER_PRE_PIECES = 4;                 // 16-byte pieces per thread: d <= 8192
+
+template <int ACT>
+__device__ __forceinline__ void router_stage_prenorm(const RouterParams& p, uint32_t t0, uint32_t nt, uint16_t* xl,
+                                                     uint16_t* raw) {
+    const bool writer = blockIdx.x == 0;
+    const uint32_t per_row = p.d / 8, lane = threadIdx.x & 63;
+    for (uint32_t t = 0; t < nt; ++t) {
+        const uint16_t* h = (const uint16_t*)p.x + (size_t)(t0 + t) * p.x_stride;
+        uint4 v[ROUTER_PRE_PIECES], dl[ROUTER_PRE_PIECES], w[ROUTER_PRE_PIECES];
+#pragma unroll
+        for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
+            const uint32_t c = threadIdx.x + 256 * k;
+            if (c >= per_row) break;
+            v[k] = *reinterpret_cast<const uint4*>(h + c * 8);
+            if (p.pre_delta) dl[k] = *reinterpret_cast<const uint4*>(p.pre_delta + (size_t)(t0 + t) * p.pre_delta_stride + c * 8);
+            w[k] = *reinterpret_cast<const uint4*>(p.pre_weight + c * 8);
+        }
+#pragma unroll
+        for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
+            const uint32_t c = threadIdx.x + 256 * k;
+            if (c >= per_row) break;
+            if (p.pre_delta) {
+                uint32_t* vv = reinterpret_cast<uint32_t*>(&v[k]);
+                const uint32_t* dd = reinterpret_cast<const uint32_t*>(&dl[k]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float a0, a1, b0, b1;
+                    act2_to_f32<ACT>(vv[j], a0, a1);
+                    act2_to_f32<ACT>(dd[j], b0, b1);
+                    vv[j] = (uint32_t)f32_to_act<ACT>(__fadd_rn(a0, b0)) | ((uint32_t)f32_to_act<ACT>(__fadd_rn(a1, b1)) << 16);
+                }
+            }
+            reinterpret_cast<uint4*>(raw)[c] = v[k];
+            if (writer && p.pre_hidden_out)
+                *reinterpret_cast<uint4*>(p.pre_hidden_out + (size_t)(t0 + t) * p.pre_hidden_stride + c * 8) = v[k];
+        }
+        __syncthreads();
+        // the stated order: lane l over the elements l, l + 64, ...; eight reads in flight at a time
+        float acc = 0.0f;
+        for (uint32_t i0 = lane; i0 < p.d; i0 += 512) {
+            uint16_t e[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) e[j] = i0 + 64 * j < p.d ? raw[i0 + 64 * j] : (uint16_t)0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                if (i0 + 64 * j >= p.d) break;
+                const float x = act_to_f32<ACT>(e[j]);
+                acc = fmaf(x, x, acc);
+            }
+        }
+        const float inv = rms_inverse(rms_wave_sum(acc), p.d, p.pre_eps);
+#pragma unroll
+        for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
+            const uint32_t c = threadIdx.x + 256 * k;
+            if (c >= per_row) break;
+            const uint32_t* vv = reinterpret_cast<const uint32_t*>(&v[k]);
+            const uint32_t* ww = reinterpret_cast<const uint32_t*>(&w[k]);
+            uint4 o;
+            uint32_t* oo = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float a0, a1, w0, w1;
+                act2_to_f32<ACT>(vv[j], a0, a1);
+                act2_to_f32<ACT_BF16>(ww[j], w0, w1);
+                oo[j] = (uint32_t)f32_to_act<ACT>(__fmul_rn(__fmul_rn(a0, inv), w0)) |
+                        ((uint32_t)f32_to_act<ACT>(__fmul_rn(__fmul_rn(a1, inv), w1)) << 16);
+            }
+            reinterpret_cast<uint4*>(xl)[t * per_row + c] = o;
+            if (writer && p.pre_normed_out)
+                *reinterpret_cast<uint4*>(p.pre_normed_out + (size_t)(t0 + t) * p.pre_normed_stride + c * 8) = o;
+        }
+        __syncthreads();                             // xl is complete; raw is rewritten by the next row
+    }
+}
+
 // One row against up to ROUTER_TOK tokens; hl = lane in the half-wave, CPL =
 // chunks per lane (compile time) so that every load is issued before the first
 // use: a dependent round trip to HBM costs more than the whole arithmetic.
 // Per token the lane accumulates over its chunks in ascending order.
-template <int ACT, int KIND, int CPL>
-__device__ __forceinline__ void router_row_dots(const RouterParams& p, const RowsDesc& r, uint32_t row,
-                                                const uint16_t* xl, uint32_t nt, int hl, float* acc) {
-    constexpr int EPC = KIND == 16 ? 8 : (KIND == 8 ? 16 : 32);
-    constexpr int XV = EPC / 8;
-    const uint32_t chunks = p.d / EPC;
-    const uint32_t groups = p.d / NVMAI_GROUP;
-    const uint8_t* wr = (const uint8_t*)r.w + (size_t)row * ((size_t)p.d * KIND / 8);
-    uint4 wraw[CPL];
-    uint16_t sraw[CPL], braw[CPL];
+// A half-wave's share of one weight row, fetched before the inputs are staged: the two do not depend
+// on each other, and a trip to memory costs more than the arithmetic that follows.
+template <int CPL>
+struct RouterRowRegs { uint4 w[CPL]; uint16_t s[CPL], b[CPL]; };
+
+template <int CPL>
+__device__ __forceinline__ void router_row_prefetch(const RouterParams& p, const RowsDesc& r, uint32_t row, int hl,
+                                                    RouterRowRegs<CPL>& g) {
+    const uint32_t epc = r.kind == 16 ? 8u : (r.kind == 8 ? 16u : 32u);
+    const uint32_t chunks = p.d / epc, groups = p.d / NVMAI_GROUP;
+    const uint8_t* wr = (const uint8_t*)r.w + (size_t)row * ((size_t)p.d * r.kind / 8);
 #pragma unroll
     for (int i = 0; i < CPL; ++i) {
         const uint32_t c = hl + 32 * i;
         if (c < chunks) {
-            wraw[i] = *reinterpret_cast<const uint4*>(wr + (size_t)c * 16);
-            if (KIND != 16) {
-                const uint32_t g = c * EPC / NVMAI_GROUP;
-                sraw[i] = r.s[(size_t)row * groups + g];
-                braw[i] = r.b[(size_t)row * groups + g];
+            g.w[i] = *reinterpret_cast<const uint4*>(wr + (size_t)c * 16);
+            if (r.kind != 16) {
+                const uint32_t gi = c * epc / NVMAI_GROUP;
+                g.s[i] = r.s[(size_t)row * groups + gi];
+                g.b[i] = r.b[(size_t)row * groups + gi];
             }
         }
     }
+}
+
+template <int ACT, int KIND, int CPL>
+__device__ __forceinline__ void router_row_dots(const RouterParams& p, const RouterRowRegs<CPL>& g,
+                                                const uint16_t* xl, uint32_t nt, int hl, float* acc) {
+    constexpr int EPC = KIND == 16 ? 8 : (KIND == 8 ? 16 : 32);
+    constexpr int XV = EPC / 8;
+    const uint32_t chunks = p.d / EPC;
 #pragma unroll
     for (int t = 0; t < ROUTER_TOK; ++t) acc[t] = 0.0f;
 #pragma unroll
@@ -641,10 +742,10 @@ __device__ __forceinline__ void router_row_dots(const RouterParams& p, const Row
         if (c >= chunks) break;
         float q[EPC];
         if (KIND == 16) {
-            act2_to_f32<ACT_BF16>(wraw[i].x, q[0], q[1]); act2_to_f32<ACT_BF16>(wraw[i].y, q[2], q[3]);
-            act2_to_f32<ACT_BF16>(wraw[i].z, q[4], q[5]); act2_to_f32<ACT_BF16>(wraw[i].w, q[6], q[7]);
+            act2_to_f32<ACT_BF16>(g.w[i].x, q[0], q[1]); act2_to_f32<ACT_BF16>(g.w[i].y, q[2], q[3]);
+            act2_to_f32<ACT_BF16>(g.w[i].z, q[4], q[5]); act2_to_f32<ACT_BF16>(g.w[i].w, q[6], q[7]);
         } else {
-            unpack_chunk<KIND == 16 ? 8 : KIND>(wraw[i], q);
+            unpack_chunk<KIND == 16 ? 8 : KIND>(g.w[i], q);
         }
 #pragma unroll
         for (int t = 0; t < ROUTER_TOK; ++t) {
@@ -664,8 +765,8 @@ __device__ __forceinline__ void router_row_dots(const RouterParams& p, const Row
                     dot = fmaf(q[j], xv[j], dot);
                     xs = __fadd_rn(xs, xv[j]);
                 }
-                acc[t] = fmaf(bf16_to_f32(sraw[i]), dot, acc[t]);
-                acc[t] = fmaf(bf16_to_f32(braw[i]), xs, acc[t]);
+                acc[t] = fmaf(bf16_to_f32(g.s[i]), dot, acc[t]);
+                acc[t] = fmaf(bf16_to_f32(g.b[i]), xs, acc[t]);
             }
         }
     }
@@ -676,11 +777,11 @@ __device__ __forceinline__ void router_row_dots(const RouterParams& p, const Row
 }
 
 template <int ACT, int CPL>
-__device__ __forceinline__ void router_row_any(const RouterParams& p, const RowsDesc& r, uint32_t row,
+__device__ __forceinline__ void router_row_any(const RouterParams& p, int kind, const RouterRowRegs<CPL>& g,
                                                const uint16_t* xl, uint32_t nt, int hl, float* acc) {
-    if (r.kind == 16) router_row_dots<ACT, 16, CPL>(p, r, row, xl, nt, hl, acc);
-    else if (r.kind == 8) router_row_dots<ACT, 8, CPL>(p, r, row, xl, nt, hl, acc);
-    else router_row_dots<ACT, 4, CPL>(p, r, row, xl, nt, hl, acc);
+    if (kind == 16) router_row_dots<ACT, 16, CPL>(p, g, xl, nt, hl, acc);
+    else if (kind == 8) router_row_dots<ACT, 8, CPL>(p, g, xl, nt, hl, acc);
+    else router_row_dots<ACT, 4, CPL>(p, g, xl, nt, hl, acc);
 }
 
 // Largest chunk count per lane over the router and gate rows must be <= CPL.
@@ -693,12 +794,19 @@ __global__ __launch_bounds__(256) void router_logits_kernel(RouterParams p) {
     const uint32_t total_rows = p.num_experts + (p.gate.kind ? 1u : 0u);
     const uint32_t t0 = blockIdx.y * ROUTER_TOK;
     const uint32_t nt = min((uint32_t)ROUTER_TOK, p.tokens - t0);
-    router_stage_x(p, t0, nt, reinterpret_cast<uint16_t*>(router_lds));
-    if (row >= total_rows) return;                   // uniform per half-wave
-    const bool is_gate = row >= p.num_experts;
+    const bool live = row < total_rows, is_gate = row >= p.num_experts;
+    const RowsDesc& rd = is_gate ? p.gate : p.router;
+    RouterRowRegs<CPL> g;
+    if (live) router_row_prefetch<CPL>(p, rd, is_gate ? 0u : row, hl, g);      // in flight while the inputs are staged
+    if (p.pre_weight) {
+        uint16_t* raw = reinterpret_cast<uint16_t*>(router_lds) + (size_t)ROUTER_TOK * p.d;
+        router_stage_prenorm<ACT>(p, t0, nt, reinterpret_cast<uint16_t*>(router_lds), raw);
+    } else {
+        router_stage_x(p, t0, nt, reinterpret_cast<uint16_t*>(router_lds));
+    }
+    if (!live) return;                               // uniform per half-wave
     float acc[ROUTER_TOK];
-    if (is_gate) router_row_any<ACT, CPL>(p, p.gate, 0, xl, nt, hl, acc);
-    else router_row_any<ACT, CPL>(p, p.router, row, xl, nt, hl, acc);
+    router_row_any<ACT, CPL>(p, rd.kind, g, xl, nt, hl, acc);
     if (hl == 0) {
         for (uint32_t t = 0; t < nt; ++t) {
             if (is_gate) p.gate_logit[t0 + t] = acc[t];

@@ -12,16 +12,7 @@ namespace nvmai {
 // One wave per row.  The sum of squares has a fixed order so that a CPU run of the same order
 // gives the same bits: lane l runs acc = fma(x, x, acc) over the elements l, l + 64, ...,
 // then an xor butterfly 32, 16, 8, 4, 2, 1; every later step is one IEEE operation.
-__device__ __forceinline__ float rms_wave_sum(float acc) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) acc = __fadd_rn(acc, shfl_xor_f(acc, off));
-    return acc;
-}
-
-__device__ __forceinline__ float rms_inverse(float sum, uint32_t d, float eps) {
-    const float mean = __fdiv_rn(sum, (float)d);
-    return __fdiv_rn(1.0f, sqrtf(__fadd_rn(mean, eps)));     // sqrtf: correctly rounded (the _rn intrinsic is not)
-}
+// (rms_wave_sum and rms_inverse, the stated order and the single IEEE steps, are in common.cuh)
 
 // One wave per row.  STAGED: the row travels through LDS -- 16-byte loads in, the per-lane sums
 // and products read and written two bytes at a time there, 16-byte stores out -- so that a lane's

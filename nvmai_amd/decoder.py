@@ -146,6 +146,7 @@ class HybridDecoder:
         D = cfg.hidden
         buf = lambda *shape: torch.zeros(shape, dtype=dt, device=dev)
         self.hidden, self.normed, self.branch = buf(batch, D), buf(batch, D), buf(batch, D)
+        self.hidden_alt = buf(batch, D)            # the residual rows alternate between two buffers
         self.moe_out = buf(batch, D)
         kh, vh, dk, dv, taps = cfg.gdn
         self.gdn = ops.GDN(ctx, kh, vh, dk, dv, taps)
@@ -237,8 +238,11 @@ class HybridDecoder:
                 self._linear_attention(L, w)
             else:
                 self._full_attention(L, w, position)
-            ops.residual_add_rmsnorm(ctx, self.hidden, self.branch, w["post_norm"], out=self.normed, eps=cfg.rms_eps)
-            self.moe.decode_layer(w["moe"], self.normed, self.moe_out)
+            # residual add + post-attention norm + MoE: the router launch does the add and the norm itself,
+            # so the updated residual rows go to the second buffer (other blocks still read the first)
+            self.moe.decode_layer_prenorm(w["moe"], self.hidden, self.branch, w["post_norm"], self.hidden_alt, self.normed,
+                                          self.moe_out, eps=cfg.rms_eps)
+            self.hidden, self.hidden_alt = self.hidden_alt, self.hidden
             nxt = self.w.layers[L + 1]["in_norm"] if L + 1 < cfg.layers else self.w.final_norm
             ops.residual_add_rmsnorm(ctx, self.hidden, self.moe_out, nxt, out=self.normed, eps=cfg.rms_eps)
         return self.normed

@@ -222,6 +222,19 @@ class MoE:
                                                      _ptr(w), _ptr(stats)), "moe_decode_layer_noalloc")
         return y
 
+    def decode_layer_prenorm(self, layer, hidden, delta, norm_weight, hidden_out, normed, y, eps=1e-6, idx=None,
+                             w=None, stats=None):
+        """nvmai_hip_moe_decode_layer_prenorm: hidden_out = hidden + delta (delta None: a copy),
+        normed = rmsnorm(hidden_out) * norm_weight, y = MoE(normed); below 64 tokens the router
+        launch does the add and the norm itself.  Every buffer is the caller's."""
+        h2 = hidden.reshape(-1, hidden.shape[-1])
+        check(lib.nvmai_hip_moe_decode_layer_prenorm(
+            self.ctx.handle, _stream(), C.byref(layer), _ptr(h2), h2.stride(0), _ptr(delta),
+            0 if delta is None else delta.stride(0), _ptr(norm_weight), eps, _ptr(hidden_out), hidden_out.stride(0),
+            _ptr(normed), normed.stride(0), h2.shape[0], _ptr(y), y.stride(0), _ptr(idx), _ptr(w), _ptr(stats)),
+            "moe_decode_layer_prenorm")
+        return y
+
 
 def moe_layer_desc(d, f, num_experts, top_k, bits, router, experts, shared_blob=None, shared_gate=None,
                    eff_scale=None, per_expert_scale=None, offsets=None):

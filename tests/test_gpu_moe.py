@@ -572,3 +572,47 @@ def test_captured_graph_survives_workspace_growth(nv):
         torch.cuda.synchronize()
         assert torch.equal(y_static, want)
     ctx.close()
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_decode_layer_prenorm_equals_the_separate_calls(nv, ctx, bits):
+    # residual add + RMSNorm done by the router launch: the same bits as nvmai_hip_residual_add_rmsnorm
+    # followed by the plain decode layer, for the three-launch path (1-4 tokens), the work-list path
+    # (5-63) and the fallback (64 and more; or the residual rows updated in place)
+    rng = np.random.default_rng(500 + bits)
+    d, f, E, k = 256, 128, 16, 4
+    off, stride = nv.expert_offsets(d, f, bits)
+    pool = torch.empty((E + 1, stride), dtype=torch.uint8, device="cuda")
+    for e in range(E + 1):
+        mk = lambda r, c: torch.randn((r, c), device="cuda").mul_(0.05).to(torch.bfloat16)
+        nv.pack_expert(ctx, mk(f, d), mk(f, d), mk(d, f), bits, pool[e])
+    rdesc = nv.rows_desc(16, dev(O.bf16_bits(gauss(rng, (E, d), 0.02)).view(np.int16)))
+    gh = O.quantize_affine(O.round_bf16(gauss(rng, (1, d), 0.05)), 8)
+    gdesc = nv.rows_desc(8, dev(gh[0]), dev(gh[1].view(np.int16)), dev(gh[2].view(np.int16)))
+    layer = nv.moe_layer_desc(d, f, E, k, bits, rdesc, pool[:E], pool[E], gdesc)
+    w = dev(O.bf16_bits(rng.uniform(0.5, 1.5, d).astype(np.float32)).view(np.int16))
+    moe = nv.MoE(ctx, bits)
+    for tokens, with_delta, in_place in [(1, True, False), (3, False, False), (5, True, False), (32, True, False),
+                                         (70, True, False), (4, True, True)]:
+        say("decode layer prenorm", ctx.act, bits, tokens, with_delta, in_place)
+        h = act_tensor(round_act(gauss(rng, (tokens, d)), ctx.act), ctx)
+        delta = act_tensor(round_act(gauss(rng, (tokens, d), 0.3), ctx.act), ctx) if with_delta else None
+        # reference: the separate calls
+        h_ref = h.clone()
+        if with_delta:
+            n_ref = nv.residual_add_rmsnorm(ctx, h_ref, delta, w)
+        else:
+            n_ref = nv.RMSNorm(ctx).encode_bf16w(h_ref, w)
+        y_ref, i_ref, w_ref = moe.decode_layer(layer, n_ref, want_routes=True)
+        h_in = h.clone()
+        h_out = h_in if in_place else torch.full_like(h, 9.0)
+        normed, y = torch.full_like(h, 9.0), torch.full_like(h, 9.0)
+        idx = torch.zeros((tokens, k), dtype=torch.int32, device="cuda")
+        wt = torch.zeros((tokens, k), dtype=torch.int16, device="cuda")
+        moe.decode_layer_prenorm(layer, h_in, delta, w, h_out, normed, y, idx=idx, w=wt)
+        torch.cuda.synchronize()
+        assert torch.equal(h_out, h_ref) and torch.equal(normed, n_ref)
+        assert torch.equal(idx, i_ref.view(torch.int32).reshape(tokens, k)) and torch.equal(wt, w_ref.view(torch.int16).reshape(tokens, k))
+        assert torch.equal(y, y_ref)
+        if not in_place:
+            assert torch.equal(h_in, h)                      # the residual rows read by the launch are untouched
