@@ -22,19 +22,25 @@ int gemv_mfma(nvmai_hip_ctx* ctx, hipStream_t s, const uint8_t* w, const uint16_
     // rows per block: 64 for a large matrix, 32 or 16 where that would leave compute units without a block
     const int wr = m >= 8192 ? 4 : m >= 4096 ? 2 : 1;
     const dim3 grid((m + 16 * wr - 1) / (16 * wr));
-#define NVMAI_GM_T(ACT, BITS, TT)                                                        \
-    do {                                                                                 \
-        if (wr == 4) gemv_mfma_kernel<ACT, BITS, TT, 4><<<grid, 256, 0, s>>>(p);         \
-        else if (wr == 2) gemv_mfma_kernel<ACT, BITS, TT, 2><<<grid, 256, 0, s>>>(p);    \
-        else gemv_mfma_kernel<ACT, BITS, TT, 1><<<grid, 256, 0, s>>>(p);                 \
+    // eight waves per block for 4-bit rows (8-bit rows would need 200 KB of LDS for them)
+#define NVMAI_GM_N(ACT, BITS, TT, NW)                                                          \
+    do {                                                                                       \
+        if (wr == 4) gemv_mfma_kernel<ACT, BITS, TT, 4, NW><<<grid, 64 * NW, 0, s>>>(p);       \
+        else if (wr == 2) gemv_mfma_kernel<ACT, BITS, TT, 2, NW><<<grid, 64 * NW, 0, s>>>(p);  \
+        else gemv_mfma_kernel<ACT, BITS, TT, 1, NW><<<grid, 64 * NW, 0, s>>>(p);               \
     } while (0)
-#define NVMAI_GM(ACT, BITS)                                                              \
-    do {                                                                                 \
-        if (n_tokens <= 16) NVMAI_GM_T(ACT, BITS, 1); else NVMAI_GM_T(ACT, BITS, 2);     \
+#define NVMAI_GM_T(ACT, BITS, TT)                                                              \
+    do {                                                                                       \
+        NVMAI_GM_N(ACT, BITS, TT, (BITS == 4 ? 8 : 4));                                        \
+    } while (0)
+#define NVMAI_GM(ACT, BITS)                                                                    \
+    do {                                                                                       \
+        if (n_tokens <= 16) NVMAI_GM_T(ACT, BITS, 1); else NVMAI_GM_T(ACT, BITS, 2);           \
     } while (0)
     if (ctx->act == ACT_BF16) { if (bits == 8) NVMAI_GM(ACT_BF16, 8); else NVMAI_GM(ACT_BF16, 4); }
     else { if (bits == 8) NVMAI_GM(ACT_FP16, 8); else NVMAI_GM(ACT_FP16, 4); }
 #undef NVMAI_GM_T
+#undef NVMAI_GM_N
 #undef NVMAI_GM
     return launch_status();
 }

@@ -62,9 +62,11 @@ __device__ __forceinline__ void gm_pow2_scale(float amax, float& sc, float& isc)
 
 constexpr uint32_t GM_STAGE_CODES = 512;        // codes of a row per stage: 8 groups
 
-template <int ACT, int BITS, int TT, int WR>
-__global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p) {
-    constexpr int KW = 4 / WR;                           // waves sharing out the stages of K
+// NW = waves per block (4 or 8): eight halve what a wave has to stage and to multiply, which is
+// what a projection of a few thousand rows -- one block per compute unit at most -- is short of.
+template <int ACT, int BITS, int TT, int WR, int NW>
+__global__ __launch_bounds__(64 * NW) void gemv_mfma_kernel(GemvMfmaParams p) {
+    constexpr int KW = NW / WR;                          // waves sharing out the stages of K
     constexpr uint32_t KP = 2048 / TT;                   // elements of an input panel
     constexpr uint32_t XROW = KP * 2 + 16;               // bytes of a staged input row
     constexpr uint32_t NTOK = 16 * TT;
@@ -76,10 +78,10 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p) {
     constexpr int N_LOADS = NLD + 2;                     // + scales + biases
     constexpr uint32_t GPP = KP / 64;                    // groups per panel
     __shared__ __attribute__((aligned(16))) uint8_t x_s[NTOK * XROW];
-    __shared__ __attribute__((aligned(16))) uint8_t wa[4 * WREG];
-    __shared__ __attribute__((aligned(16))) uint8_t wb[4 * WREG];
-    __shared__ __attribute__((aligned(16))) uint8_t ma[4 * 512];     // per wave: 16 rows x 16 B scales | 16 x 16 B biases
-    __shared__ __attribute__((aligned(16))) uint8_t mb[4 * 512];
+    __shared__ __attribute__((aligned(16))) uint8_t wa[NW * WREG];
+    __shared__ __attribute__((aligned(16))) uint8_t wb[NW * WREG];
+    __shared__ __attribute__((aligned(16))) uint8_t ma[NW * 512];    // per wave: 16 rows x 16 B scales | 16 x 16 B biases
+    __shared__ __attribute__((aligned(16))) uint8_t mb[NW * 512];
     __shared__ __attribute__((aligned(16))) float xsum_s[NTOK * GPP];
     __shared__ float isc_s[NTOK];
     // the stage arrays are written by load instructions only; a store that never runs keeps the
@@ -134,16 +136,16 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p) {
     if (n_my > 0) issue_stage(wave_k, wa_w, ma_w);
     if (n_my > 1) issue_stage(wave_k + KW, wb_w, mb_w);
 
-    // ---- inputs of one panel: a wave converts whole rows (tokens wave, wave + 4, ...)
+    // ---- inputs of one panel: a wave converts whole rows (tokens wave, wave + NW, ...)
     auto stage_inputs = [&](uint32_t k0) {
         constexpr int CH = KP / 512;                         // 16-byte pieces per lane and row
         const uint32_t kp_len = min(KP, p.n - k0);
         // every load of the wave's rows is issued before the first is used
-        constexpr int TPW = NTOK / 4;                        // rows per wave
+        constexpr int TPW = NTOK / NW;                       // rows per wave
         uint4 raw_all[TPW][CH];
 #pragma unroll
         for (int q = 0; q < TPW; ++q) {
-            const uint32_t t = wave + 4 * q;
+            const uint32_t t = wave + NW * q;
 #pragma unroll
             for (int c = 0; c < CH; ++c) {
                 const uint32_t e = (c * 64 + lane) * 8;
@@ -154,7 +156,7 @@ __global__ __launch_bounds__(256) void gemv_mfma_kernel(GemvMfmaParams p) {
         }
 #pragma unroll
         for (int q = 0; q < TPW; ++q) {
-            const uint32_t t = wave + 4 * q;
+            const uint32_t t = wave + NW * q;
             const uint4* raw = raw_all[q];
             float v[CH][8];
             float amax = 0.0f;
