@@ -393,6 +393,17 @@ int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream stream, const vo
                                uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
                                uint32_t seq_len, uint32_t kv_start, float scale);
 
+/* nvmai_hip_attention_decode followed by Elementwise.encodeSigmoidGateMul over its output
+ * (RealForwardRunner.swift:2257-2276; utility.metal:47-58) in the same launches:
+ * out = round(attention) / (1 + exp(-gate)), gate rows [batch, gate_stride] activations laid out
+ * like out.  Same bits as the two calls one after the other. */
+int nvmai_hip_attention_decode_gated(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
+                                     const nvmai_kv_view* k, const nvmai_kv_view* v,
+                                     uint64_t kv_batch_stride, void* out, const void* gate,
+                                     uint32_t gate_stride, uint32_t batch, uint32_t head_dim,
+                                     uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len,
+                                     uint32_t kv_start, float scale);
+
 /* The same call for sequences of different lengths: sequence b reads rows
  * [kv_starts[b], min(seq_lens[b], max_seq_len)) of its cache (kv_starts NULL: from row 0).
  * seq_lens and kv_starts are device arrays of `batch` words read by the kernels, so a captured
@@ -573,6 +584,19 @@ int nvmai_hip_attn_qkv_epilogue(nvmai_hip_ctx* ctx, nvmai_stream stream, const v
                                 void* gate_out, void* k_out, void* v_out, uint32_t kv_stride, uint32_t tokens,
                                 uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t head_dim, uint32_t rotary_dim,
                                 int v_norm, const uint32_t* positions, uint32_t position, float theta, float eps);
+
+/* The same epilogue with KVCacheQuantizer.encode (KVCacheQuantizer.swift:17-60;
+ * kv_cache_quantize.metal:7-73) of the finished k and v rows in the same launch: token t's rows
+ * go to k_cache->base + t * k_cache->stride and v_cache->base + t * v_cache->stride as
+ * [codes | fp16 scales | fp16 biases] (4 or 8 bit, group 64; head_dim a multiple of 64; both views of
+ * one format).  k_out / v_out (the 16-bit stage rows) may both be NULL.  Same bits as
+ * nvmai_hip_attn_qkv_epilogue followed by two nvmai_hip_kv_quantize_affine calls. */
+int nvmai_hip_attn_qkv_epilogue_kv(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* proj, uint32_t proj_stride,
+                                   int q_packed, const uint16_t* q_weight, const uint16_t* k_weight, void* q_out,
+                                   void* gate_out, void* k_out, void* v_out, uint32_t kv_stride,
+                                   const nvmai_kv_view* k_cache, const nvmai_kv_view* v_cache, uint32_t tokens,
+                                   uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t head_dim, uint32_t rotary_dim,
+                                   int v_norm, const uint32_t* positions, uint32_t position, float theta, float eps);
 
 /* ---- gated-DeltaNet linear attention ------------------------------------------------------- */
 

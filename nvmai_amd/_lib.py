@@ -100,6 +100,8 @@ SIGNATURES = {
     "nvmai_hip_rope_neox_subdim": [vp, vp, vp, u32, u32, u32, u32, vp, u32, C.c_float],
     "nvmai_hip_attention_decode": [vp, vp, vp, C.POINTER(KvView), C.POINTER(KvView), u64, vp, u32, u32, u32,
                                    u32, u32, u32, C.c_float],
+    "nvmai_hip_attention_decode_gated": [vp, vp, vp, C.POINTER(KvView), C.POINTER(KvView), u64, vp, vp, u32, u32, u32,
+                                         u32, u32, u32, u32, C.c_float],
     "nvmai_hip_attention_decode_ragged": [vp, vp, vp, C.POINTER(KvView), C.POINTER(KvView), u64, vp, u32, u32, u32,
                                           u32, vp, vp, u32, C.c_float],
     "nvmai_hip_attention_prefill_causal": [vp, vp, vp, u32, C.POINTER(KvView), C.POINTER(KvView), vp, u32, u32, u32,
@@ -131,6 +133,8 @@ SIGNATURES = {
     "nvmai_hip_residual_add_rmsnorm": [vp, vp, vp, u32, vp, u32, vp, vp, u32, u32, u32, C.c_float],
     "nvmai_hip_attn_qkv_epilogue": [vp, vp, vp, u32, C.c_int, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32,
                                     C.c_int, vp, u32, C.c_float, C.c_float],
+    "nvmai_hip_attn_qkv_epilogue_kv": [vp, vp, vp, u32, C.c_int, vp, vp, vp, vp, vp, vp, u32, C.POINTER(KvView),
+                                       C.POINTER(KvView), u32, u32, u32, u32, u32, C.c_int, vp, u32, C.c_float, C.c_float],
     "nvmai_hip_gdn_conv_norm": [vp, vp, C.POINTER(GdnConfig), vp, u32, vp, vp, vp, u32, u32, u32],
     "nvmai_hip_gdn_delta_gated_norm": [vp, vp, C.POINTER(GdnConfig), vp, u32, vp, vp, u32, vp, vp, vp, C.c_int, vp, u32,
                                        vp, vp, u32, u32, u32],

@@ -122,7 +122,8 @@ int run_attention(nvmai_hip_ctx* ctx, nvmai_stream stream, AttnParams p, const n
     if (nc > ATTN_MAX_CHUNKS) return NVMAI_ERR_UNSUPPORTED;      // cannot happen: nc <= 512 by construction
     const size_t heads_total = (size_t)p.batch * p.num_q_heads;
     // one chunk: the partial kernel writes the rows itself (the matrix-core one in 8-byte pieces)
-    p.direct = nc == 1 && (!fast || ((reinterpret_cast<uintptr_t>(p.out) & 7u) == 0 && p.out_stride % 4 == 0));
+    // (a gated call keeps the combine launch: the gate is applied where the rows are written)
+    p.direct = nc == 1 && !p.gate && (!fast || ((reinterpret_cast<uintptr_t>(p.out) & 7u) == 0 && p.out_stride % 4 == 0));
     p.num_chunks = nc; p.chunk_len = chunk_len;
     if (!p.direct) {
         const int rc = ws_begin(ctx, stream, 2 * ws_round(heads_total * nc * 4) + ws_round(heads_total * nc * p.head_dim * 4));
@@ -189,6 +190,23 @@ extern "C" int nvmai_hip_attention_decode(nvmai_hip_ctx* ctx, nvmai_stream strea
     if (!aligned16(q)) return NVMAI_ERR_ALIGNMENT;
     p.kv_batch_stride = kv_batch_stride;
     p.seq_len = seq_len; p.kv_start = kv_start;
+    return run_attention(ctx, stream, p, k, v, seq_len - kv_start, false);
+}
+
+extern "C" int nvmai_hip_attention_decode_gated(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
+                                                const nvmai_kv_view* k, const nvmai_kv_view* v,
+                                                uint64_t kv_batch_stride, void* out, const void* gate,
+                                                uint32_t gate_stride, uint32_t batch, uint32_t head_dim,
+                                                uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len,
+                                                uint32_t kv_start, float scale) {
+    AttnParams p;
+    const int rc = attention_setup(ctx, q, k, v, out, batch, head_dim, num_q_heads, num_kv_heads, scale, p);
+    if (rc) return rc;
+    if (kv_start > seq_len || !gate || gate_stride < num_q_heads * head_dim) return NVMAI_ERR_INVALID_ARG;
+    if (!aligned16(q)) return NVMAI_ERR_ALIGNMENT;
+    p.kv_batch_stride = kv_batch_stride;
+    p.seq_len = seq_len; p.kv_start = kv_start;
+    p.gate = (const uint16_t*)gate; p.gate_stride = gate_stride;
     return run_attention(ctx, stream, p, k, v, seq_len - kv_start, false);
 }
 

@@ -156,6 +156,11 @@ struct AttnParams {
     uint32_t ring;             // not 0: row of key p is p % ring (generic kernel only)
     uint32_t cols_q;           // sequences sharing one block of the matrix-core kernel
     uint32_t direct;           // num_chunks == 1: the partial kernel normalises and writes out itself
+    // optional output gate (RealForwardRunner.swift:2272-2276, utility.metal:47-58): the combine
+    // kernel writes round(out) / (1 + exp(-gate)) -- the rounded row first, as the separate
+    // elementwise launch reads it, so the bits are the same.  Row of sequence b at gate + b * gate_stride.
+    const uint16_t* gate;
+    uint32_t gate_stride;
 };
 
 __device__ __forceinline__ void attn_range(const AttnParams& p, uint32_t b, uint32_t& lo, uint32_t& hi) {
@@ -249,6 +254,12 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     const float* orow = p.o_part + bh * p.num_chunks * p.head_dim;
     const uint32_t dim = blockIdx.y * 64 + lane;
     uint16_t* out_row = (uint16_t*)p.out + (bh / p.num_q_heads) * p.out_stride + (bh % p.num_q_heads) * p.head_dim;
+    const uint16_t* gate_row = p.gate ? p.gate + (bh / p.num_q_heads) * p.gate_stride + (bh % p.num_q_heads) * p.head_dim : nullptr;
+    auto gated = [&](float v) -> uint16_t {
+        uint16_t o = f32_to_act<ACT>(v);
+        if (gate_row) o = f32_to_act<ACT>(__fdiv_rn(act_to_f32<ACT>(o), __fadd_rn(1.0f, expf(-act_to_f32<ACT>(gate_row[dim])))));
+        return o;
+    };
     float mloc = -INFINITY;
     for (uint32_t c = threadIdx.x; c < p.num_chunks; c += 256) mloc = fmaxf(mloc, mr[c]);
     mloc = wave_max_f32(mloc);
@@ -256,7 +267,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     __syncthreads();
     const float mg = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     if (mg == -INFINITY) {                                   // uniform over the block
-        if (wave == 0 && dim < p.head_dim) out_row[dim] = f32_to_act<ACT>(0.0f);
+        if (wave == 0 && dim < p.head_dim) out_row[dim] = gated(0.0f);
         return;
     }
     float dloc = 0.0f;
@@ -279,7 +290,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     __syncthreads();
     if (wave == 0 && dim < p.head_dim) {
         const float tot = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
-        out_row[dim] = f32_to_act<ACT>(D > 0.0f ? tot / D : 0.0f);
+        out_row[dim] = gated(D > 0.0f ? tot / D : 0.0f);
     }
 }
 

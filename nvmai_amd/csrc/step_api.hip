@@ -1,4 +1,6 @@
 // Entry points: RMSNorm, the elementwise helpers of the layer loop, affine embedding lookup, fused greedy LM head.
+#include <initializer_list>
+
 #include "ctx.hpp"
 #include "step_kernels.cuh"
 
@@ -61,19 +63,36 @@ extern "C" int nvmai_hip_residual_add_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream s
     return launch_status();
 }
 
-extern "C" int nvmai_hip_attn_qkv_epilogue(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* proj,
-                                           uint32_t proj_stride, int q_packed, const uint16_t* q_weight,
-                                           const uint16_t* k_weight, void* q_out, void* gate_out, void* k_out,
-                                           void* v_out, uint32_t kv_stride, uint32_t tokens, uint32_t num_q_heads,
-                                           uint32_t num_kv_heads, uint32_t head_dim, uint32_t rotary_dim, int v_norm,
-                                           const uint32_t* positions, uint32_t position, float theta, float eps) {
-    if (!ctx || !proj || !q_out || !k_out || !v_out || (q_packed && !gate_out)) return NVMAI_ERR_INVALID_ARG;
+namespace {
+int qkv_epilogue_impl(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* proj, uint32_t proj_stride, int q_packed,
+                      const uint16_t* q_weight, const uint16_t* k_weight, void* q_out, void* gate_out, void* k_out,
+                      void* v_out, uint32_t kv_stride, uint32_t tokens, uint32_t num_q_heads, uint32_t num_kv_heads,
+                      uint32_t head_dim, uint32_t rotary_dim, int v_norm, const uint32_t* positions, uint32_t position,
+                      float theta, float eps, const nvmai_kv_view* k_cache, const nvmai_kv_view* v_cache) {
+    const bool cached = k_cache || v_cache;
+    if (!ctx || !proj || !q_out || (q_packed && !gate_out)) return NVMAI_ERR_INVALID_ARG;
+    if (cached ? (!k_cache || !v_cache) : (!k_out || !v_out)) return NVMAI_ERR_INVALID_ARG;
+    if ((k_out == nullptr) != (v_out == nullptr)) return NVMAI_ERR_INVALID_ARG;
     if (head_dim == 0 || head_dim > 512 || num_q_heads == 0 || num_kv_heads == 0) return NVMAI_ERR_INVALID_ARG;   // kFusedMaxHeadDim
     if (rotary_dim > head_dim || (rotary_dim & 1u)) return NVMAI_ERR_INVALID_ARG;
     const uint32_t span = (q_packed ? 2u : 1u) * num_q_heads * head_dim + 2u * num_kv_heads * head_dim;
-    if (proj_stride < span || kv_stride < num_kv_heads * head_dim) return NVMAI_ERR_INVALID_ARG;
-    if (tokens == 0) return NVMAI_OK;
+    if (proj_stride < span || (k_out && kv_stride < num_kv_heads * head_dim)) return NVMAI_ERR_INVALID_ARG;
     QkvEpilogueParams p{};
+    if (cached) {
+        // KVCacheQuantizer.encode's checks (KVCacheQuantizer.swift:17-30) on both destinations
+        if (head_dim % 64) return NVMAI_ERR_UNSUPPORTED;      // a group must not straddle two heads
+        uint32_t stride = 0, vb = 0;
+        for (const nvmai_kv_view* c : {k_cache, v_cache}) {
+            if (!c->base) return NVMAI_ERR_INVALID_ARG;
+            if ((c->bits != 4 && c->bits != 8) || c->group_size != 64) return NVMAI_ERR_UNSUPPORTED;
+            if (nvmai_kv_row_layout(num_kv_heads * head_dim, c->bits, &stride, &vb) != NVMAI_OK) return NVMAI_ERR_INVALID_ARG;
+            if (c->value_bytes != vb || c->stride < stride || (c->stride & 1u)) return NVMAI_ERR_INVALID_ARG;
+        }
+        if (k_cache->bits != v_cache->bits || k_cache->stride != v_cache->stride) return NVMAI_ERR_INVALID_ARG;
+        p.kc = (uint8_t*)k_cache->base; p.vc = (uint8_t*)v_cache->base;
+        p.kv_bits = k_cache->bits; p.kv_row_stride = k_cache->stride; p.kv_value_bytes = k_cache->value_bytes;
+    }
+    if (tokens == 0) return NVMAI_OK;
     p.proj = (const uint16_t*)proj; p.proj_stride = proj_stride; p.q_packed = q_packed ? 1u : 0u;
     p.q_weight = q_weight; p.k_weight = k_weight;
     p.q_out = (uint16_t*)q_out; p.gate_out = (uint16_t*)gate_out; p.k_out = (uint16_t*)k_out; p.v_out = (uint16_t*)v_out;
@@ -85,6 +104,31 @@ extern "C" int nvmai_hip_attn_qkv_epilogue(nvmai_hip_ctx* ctx, nvmai_stream stre
     if (ctx->act == ACT_BF16) qkv_epilogue_kernel<ACT_BF16><<<grid, 256, 0, s>>>(p);
     else qkv_epilogue_kernel<ACT_FP16><<<grid, 256, 0, s>>>(p);
     return launch_status();
+}
+}  // namespace
+
+extern "C" int nvmai_hip_attn_qkv_epilogue(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* proj,
+                                           uint32_t proj_stride, int q_packed, const uint16_t* q_weight,
+                                           const uint16_t* k_weight, void* q_out, void* gate_out, void* k_out,
+                                           void* v_out, uint32_t kv_stride, uint32_t tokens, uint32_t num_q_heads,
+                                           uint32_t num_kv_heads, uint32_t head_dim, uint32_t rotary_dim, int v_norm,
+                                           const uint32_t* positions, uint32_t position, float theta, float eps) {
+    return qkv_epilogue_impl(ctx, stream, proj, proj_stride, q_packed, q_weight, k_weight, q_out, gate_out, k_out, v_out,
+                             kv_stride, tokens, num_q_heads, num_kv_heads, head_dim, rotary_dim, v_norm, positions,
+                             position, theta, eps, nullptr, nullptr);
+}
+
+extern "C" int nvmai_hip_attn_qkv_epilogue_kv(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* proj,
+                                              uint32_t proj_stride, int q_packed, const uint16_t* q_weight,
+                                              const uint16_t* k_weight, void* q_out, void* gate_out, void* k_out,
+                                              void* v_out, uint32_t kv_stride, const nvmai_kv_view* k_cache,
+                                              const nvmai_kv_view* v_cache, uint32_t tokens, uint32_t num_q_heads,
+                                              uint32_t num_kv_heads, uint32_t head_dim, uint32_t rotary_dim, int v_norm,
+                                              const uint32_t* positions, uint32_t position, float theta, float eps) {
+    if (!k_cache || !v_cache) return NVMAI_ERR_INVALID_ARG;
+    return qkv_epilogue_impl(ctx, stream, proj, proj_stride, q_packed, q_weight, k_weight, q_out, gate_out, k_out, v_out,
+                             kv_stride, tokens, num_q_heads, num_kv_heads, head_dim, rotary_dim, v_norm, positions,
+                             position, theta, eps, k_cache, v_cache);
 }
 
 // Dense BF16 rows [m, n] against n_tokens BF16 inputs: the bits == 16 case of nvmai_hip_affine_gemv.

@@ -190,6 +190,14 @@ struct QkvEpilogueParams {
     const uint32_t* positions;  // one per token, or NULL = position0
     uint32_t position0;
     float theta, eps;
+    // Optional quantize-on-write of the finished k / v heads (KVCacheQuantizer.encode,
+    // kv_cache_quantize.metal:7-73), head_dim a multiple of 64: token t's row at
+    // kc / vc + t * kv_row_stride bytes = [codes | fp16 scales | fp16 biases] of kv_bits bits.  A wave
+    // holds one group of 64 elements per pass of its store loop, so the group's extremes are two
+    // butterflies over the lanes: the arithmetic, and so the bits, of kv_quantize_kernel.
+    uint8_t* kc;
+    uint8_t* vc;
+    uint32_t kv_bits, kv_row_stride, kv_value_bytes;
 };
 
 template <int ACT>
@@ -205,6 +213,8 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(QkvEpilogueParams p) 
     const uint16_t* src;
     uint16_t* dst;
     const uint16_t* w = nullptr;
+    uint8_t* cache = nullptr;                                // this token's cache row (k / v heads of a fused call)
+    uint32_t kv_elem0 = 0;                                  // first element of this head in the row
     if (is_q) {
         src = p.proj + (size_t)token * p.proj_stride + hidx * q_span;
         dst = p.q_out + ((size_t)token * p.num_q_heads + hidx) * hd;
@@ -216,8 +226,12 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(QkvEpilogueParams p) 
     } else {
         const uint32_t kvh = hidx - p.num_q_heads - (is_k ? 0 : p.num_kv_heads);
         src = p.proj + (size_t)token * p.proj_stride + p.num_q_heads * q_span + (is_k ? 0 : p.num_kv_heads * hd) + kvh * hd;
-        dst = (is_k ? p.k_out : p.v_out) + (size_t)token * p.kv_stride + kvh * hd;
+        uint16_t* stage = is_k ? p.k_out : p.v_out;
+        dst = stage ? stage + (size_t)token * p.kv_stride + kvh * hd : nullptr;
         w = is_k ? p.k_weight : nullptr;
+        uint8_t* cbase = is_k ? p.kc : p.vc;
+        if (cbase) cache = cbase + (size_t)token * p.kv_row_stride;
+        kv_elem0 = kvh * hd;
     }
     uint16_t* hs = head_s[wave];
     const bool norm = is_q || is_k || p.v_norm;
@@ -251,7 +265,33 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(QkvEpilogueParams p) 
             o = i < half_rot ? f32_to_act<ACT>(__fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s)))
                              : f32_to_act<ACT>(__fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c)));
         }
-        dst[i] = o;
+        if (dst) dst[i] = o;
+        if (cache) {                                        // wave-uniform; hd % 64 == 0: every lane holds an element
+            const float v = act_to_f32<ACT>(o);
+            float mn = v, mx = v;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) {
+                mn = fminf(mn, shfl_xor_f(mn, off));
+                mx = fmaxf(mx, shfl_xor_f(mx, off));
+            }
+            const float levels = p.kv_bits == 4 ? 15.0f : 255.0f;
+            const float bias = mn;
+            const float scale = mx > mn ? __fdiv_rn(__fsub_rn(mx, mn), levels) : 0.0f;
+            const uint32_t groups = p.num_kv_heads * hd / 64, g = (kv_elem0 + i) / 64, e = kv_elem0 + i;
+            if (lane == 0) {
+                reinterpret_cast<uint16_t*>(cache + p.kv_value_bytes)[g] = f32_to_f16(scale);
+                reinterpret_cast<uint16_t*>(cache + p.kv_value_bytes)[groups + g] = f32_to_f16(bias);
+            }
+            float q = 0.0f;
+            if (scale > 0.0f) q = roundf(fminf(fmaxf(__fdiv_rn(__fsub_rn(v, bias), scale), 0.0f), levels));
+            const uint32_t code = (uint32_t)q;
+            if (p.kv_bits == 8) {
+                cache[e] = (uint8_t)code;
+            } else {
+                const uint32_t hi = shfl_xor_u(code, 1);
+                if ((lane & 1) == 0) cache[e / 2] = (uint8_t)(code | (hi << 4));
+            }
+        }
     }
 }
 

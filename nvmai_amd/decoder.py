@@ -204,21 +204,32 @@ class HybridDecoder:
         cfg, B = self.cfg, self.batch
         p_, s_, b_ = w["qkv"]
         ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, self.normed, self.full_rows, cfg.hidden, y=self.full_proj)
-        check(lib.nvmai_hip_attn_qkv_epilogue(self.ctx.handle, ops._stream(), ops._ptr(self.full_proj), self.full_rows, 1,
-                                              ops._ptr(w["q_norm"]), ops._ptr(w["k_norm"]), ops._ptr(self.q),
-                                              ops._ptr(self.gate), ops._ptr(self.k_stage), ops._ptr(self.v_stage),
-                                              cfg.kv_dim, B, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim,
-                                              cfg.rotary_dim, 0, None, position, cfg.rope_theta, cfg.rms_eps),
-              "attn_qkv_epilogue")
         kc, vc = self.kv[L]
-        # one row per sequence, all at `position`: a view whose row pitch is the distance between sequences
-        for cache, stage in ((kc, self.k_stage), (vc, self.v_stage)):
-            view = cache.view(0, position)
-            view.stride = cache.batch_stride
-            self.quant.encode(stage, cfg.kv_dim, view, B, cfg.kv_dim)
-        self.attn.encode_full(self.q, kc, vc, cfg.head_dim, cfg.num_heads, cfg.num_kv_heads, position + 1,
-                              out=self.attn_out)
-        self.ew.encode_sigmoid_gate_mul(self.attn_out, self.gate)
+        if cfg.head_dim % 64 == 0 and cfg.kv_bits in (4, 8):
+            # split + per-head norm + RoPE + quantize-on-write in one launch: one cache row per sequence,
+            # all at `position` (views whose row pitch is the distance between two sequences)
+            kview, vview = kc.view(0, position), vc.view(0, position)
+            kview.stride, vview.stride = kc.batch_stride, vc.batch_stride
+            check(lib.nvmai_hip_attn_qkv_epilogue_kv(self.ctx.handle, ops._stream(), ops._ptr(self.full_proj), self.full_rows,
+                                                     1, ops._ptr(w["q_norm"]), ops._ptr(w["k_norm"]), ops._ptr(self.q),
+                                                     ops._ptr(self.gate), None, None, cfg.kv_dim, C.byref(kview),
+                                                     C.byref(vview), B, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim,
+                                                     cfg.rotary_dim, 0, None, position, cfg.rope_theta, cfg.rms_eps),
+                  "attn_qkv_epilogue_kv")
+        else:
+            check(lib.nvmai_hip_attn_qkv_epilogue(self.ctx.handle, ops._stream(), ops._ptr(self.full_proj), self.full_rows, 1,
+                                                  ops._ptr(w["q_norm"]), ops._ptr(w["k_norm"]), ops._ptr(self.q),
+                                                  ops._ptr(self.gate), ops._ptr(self.k_stage), ops._ptr(self.v_stage),
+                                                  cfg.kv_dim, B, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim,
+                                                  cfg.rotary_dim, 0, None, position, cfg.rope_theta, cfg.rms_eps),
+                  "attn_qkv_epilogue")
+            for cache, stage in ((kc, self.k_stage), (vc, self.v_stage)):
+                view = cache.view(0, position)
+                view.stride = cache.batch_stride
+                self.quant.encode(stage, cfg.kv_dim, view, B, cfg.kv_dim)
+        # attention and its sigmoid output gate in the same launches
+        self.attn.encode_full_gated(self.q, kc, vc, self.gate, cfg.head_dim, cfg.num_heads, cfg.num_kv_heads,
+                                    position + 1, out=self.attn_out)
         p_, s_, b_ = w["o_proj"]
         ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, self.attn_out.view(B, cfg.q_dim), cfg.hidden, cfg.q_dim,
                         y=self.branch)

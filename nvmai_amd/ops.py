@@ -528,6 +528,21 @@ class Attention:
               "attention_decode")
         return out
 
+    def encode_full_gated(self, q, k_cache, v_cache, gate, head_dim, num_q_heads, num_kv_heads, seq_len, scale=None,
+                          kv_start=0, out=None):
+        """encode_full followed by Elementwise.encodeSigmoidGateMul(out, gate) in the same launches
+        (RealForwardRunner.swift:2257-2276); gate is laid out like q.  Same bits as the two calls."""
+        batch = q.shape[0]
+        if out is None:
+            out = torch.empty_like(q)
+        kview, vview = k_cache.view(), v_cache.view()
+        check(lib.nvmai_hip_attention_decode_gated(self.ctx.handle, _stream(), _ptr(q), C.byref(kview), C.byref(vview),
+                                                   k_cache.batch_stride, _ptr(out), _ptr(gate), gate.stride(0), batch,
+                                                   head_dim, num_q_heads, num_kv_heads, seq_len, kv_start,
+                                                   0.0 if scale is None else scale),
+              "attention_decode_gated")
+        return out
+
     def encode_swa(self, q, k_cache, v_cache, head_dim, num_q_heads, num_kv_heads, seq_len, window, scale=None):
         """Attention.encodeSWA (Attention.swift:170-205): the last `window` positions."""
         return self.encode_full(q, k_cache, v_cache, head_dim, num_q_heads, num_kv_heads, seq_len, scale,

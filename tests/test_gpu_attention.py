@@ -442,3 +442,46 @@ def test_prefill_attention_rejects_what_validate_rejects(nv, ctx):
     with pytest.raises(nv.NvmaiError) as e:                                      # :174-175
         pa.encode_causal(q, kc.view(), vc.view(), out, 0, 4, 256, 15, 2, 4)
     assert e.value.name == "invalid_arg"
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_attention_with_output_gate_equals_the_two_calls(nv, ctx, bits):
+    # attention + sigmoid output gate in the same launches: the bits of encode_full followed by
+    # encode_sigmoid_gate_mul, at a context with many chunks and at one that fits one chunk
+    # (where the ungated call writes its rows from the partial kernel), and against the oracle
+    say("attention with output gate", ctx.act, bits)
+    rng = np.random.default_rng(77 + bits)
+    nq, nkv, hd = 16, 2, 256
+    attn, ew, quant = nv.Attention(ctx), nv.Elementwise(ctx), nv.KVCacheQuantizer(ctx)
+    for batch, seq in ((3, 1500), (2, 96), (1, 1)):
+        elements = nkv * hd
+        q = round_act(gauss(rng, (batch, nq, hd)), ctx.act)
+        gate = round_act(gauss(rng, (batch, nq, hd)) * 2.0, ctx.act)
+        kc, vc = nv.KVCache(batch, seq, elements, bits), nv.KVCache(batch, seq, elements, bits)
+        ks, vs = [], []
+        for b in range(batch):
+            k = round_act(gauss(rng, (seq, elements)), ctx.act)
+            v = round_act(gauss(rng, (seq, elements)), ctx.act)
+            quant.encode(act_tensor(k, ctx), elements, kc.view(b), seq, elements)
+            quant.encode(act_tensor(v, ctx), elements, vc.view(b), seq, elements)
+            ks.append(k); vs.append(v)
+        qd, gd = act_tensor(q, ctx), act_tensor(gate, ctx)
+        two = attn.encode_full(qd, kc, vc, hd, nq, nkv, seq)
+        ew.encode_sigmoid_gate_mul(two, gd)
+        one = attn.encode_full_gated(qd, kc, vc, gd, hd, nq, nkv, seq)
+        torch.cuda.synchronize()
+        assert torch.equal(one.view(torch.int16), two.view(torch.int16))
+        for b in range(batch):
+            want = O.attention_decode(q[b], O.kv_quantize(ks[b], bits), O.kv_quantize(vs[b], bits), bits, nq, nkv, hd,
+                                      seq, 1.0 / np.sqrt(hd))
+            want = O.elementwise(O.EW_SIGMOID_MUL, round_act(want, ctx.act), gate[b])
+            assert O.rel_error(act_np(one[b]), want) < 1e-2
+    # the gate is required and must cover a row
+    import ctypes as C
+    qd = act_tensor(round_act(gauss(rng, (1, nq, hd)), ctx.act), ctx)
+    kc = nv.KVCache(1, 8, nkv * hd, bits)
+    kview = kc.view()
+    for gate_ptr, gate_stride in ((None, nq * hd), (qd.data_ptr(), 16)):
+        rc = nv.lib.nvmai_hip_attention_decode_gated(ctx.handle, None, qd.data_ptr(), C.byref(kview), C.byref(kview), 0,
+                                                     qd.data_ptr(), gate_ptr, gate_stride, 1, hd, nq, nkv, 8, 0, 0.0)
+        assert rc != 0

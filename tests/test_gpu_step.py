@@ -219,3 +219,107 @@ def test_elementwise_helpers_match_oracle(nv, ctx):
     assert np.array_equal(act_np(ew.encode_concat_rows(q, g)), packed)
     torch.cuda.synchronize()
     assert nv.lib.nvmai_hip_silu_mul(ctx.handle, None, None, None, None, 4) == -1
+
+
+# ------------------------------------------------------------------ q / k / v epilogue
+def _qkv_epilogue_case(nv, ctx, rng, tokens, nq, nkv, hd, rot, pad):
+    span = 2 * nq * hd + 2 * nkv * hd
+    proj = np.zeros((tokens, span + pad), np.float32)
+    proj[:, :span] = round_act(gauss(rng, (tokens, span)), ctx.act)
+    qw = O.bf16_bits(1.0 + 0.1 * gauss(rng, (hd,)))
+    kw = O.bf16_bits(1.0 + 0.1 * gauss(rng, (hd,)))
+    positions = rng.integers(0, 5000, tokens).astype(np.uint32)
+    return proj, qw, kw, positions
+
+
+def _run_epilogue(nv, ctx, proj, qw, kw, positions, nq, nkv, hd, rot, kviews=None, stage=True):
+    import ctypes as C
+    tokens = proj.shape[0]
+    pd = act_tensor(proj, ctx)
+    q = torch.zeros((tokens, nq, hd), dtype=pd.dtype, device="cuda")
+    gate, k, v = torch.zeros_like(q), torch.zeros((tokens, nkv * hd), dtype=pd.dtype, device="cuda"), None
+    v = torch.zeros_like(k)
+    ptr = lambda t: None if t is None else t.data_ptr()
+    qwd, kwd, posd = dev(qw), dev(kw), dev(positions)       # held until the call has run
+    args = [ctx.handle, None, pd.data_ptr(), pd.stride(0), 1, qwd.data_ptr(), kwd.data_ptr(), q.data_ptr(),
+            gate.data_ptr(), ptr(k if stage else None), ptr(v if stage else None), nkv * hd]
+    tail = [tokens, nq, nkv, hd, rot, 0, posd.data_ptr(), 0, 1e4, 1e-6]
+    if kviews is None:
+        rc = nv.lib.nvmai_hip_attn_qkv_epilogue(*args, *tail)
+    else:
+        rc = nv.lib.nvmai_hip_attn_qkv_epilogue_kv(*args, C.byref(kviews[0]), C.byref(kviews[1]), *tail)
+    torch.cuda.synchronize()
+    return rc, q, gate, k, v
+
+
+@pytest.mark.parametrize("tokens,nq,nkv,hd,rot", [(1, 16, 2, 256, 64), (5, 4, 2, 64, 16), (3, 6, 3, 128, 128), (2, 3, 1, 40, 8)])
+def test_qkv_epilogue_equals_the_separate_operators(nv, ctx, tokens, nq, nkv, hd, rot):
+    # split + per-head RMSNorm (q, k) + partial RoPE (q, k) in one launch: the bits of the oracle's
+    # operators applied one after the other with a 16-bit hand-over between them
+    say("qkv epilogue", ctx.act, tokens, nq, nkv, hd, rot)
+    rng = np.random.default_rng(500 + hd + tokens)
+    proj, qw, kw, positions = _qkv_epilogue_case(nv, ctx, rng, tokens, nq, nkv, hd, rot, pad=8)
+    rc, q, gate, k, v = _run_epilogue(nv, ctx, proj, qw, kw, positions, nq, nkv, hd, rot)
+    assert rc == 0
+    r = lambda a: round_act(a, ctx.act)
+    for t in range(tokens):
+        want_q, want_gate = O.split_q_gate(proj[t, :2 * nq * hd], nq, hd)
+        want_k = proj[t, 2 * nq * hd:2 * nq * hd + nkv * hd].reshape(nkv, hd)
+        want_v = proj[t, 2 * nq * hd + nkv * hd:2 * nq * hd + 2 * nkv * hd]
+        want_q = r(O.rmsnorm(want_q, qw, 1e-6))
+        want_k = r(O.rmsnorm(want_k, kw, 1e-6))
+        want_q = O.rope_neox_subdim(want_q[None], rot, positions[t:t + 1], 1e4)[0]
+        want_k = O.rope_neox_subdim(want_k[None], rot, positions[t:t + 1], 1e4)[0]
+        assert np.array_equal(_bits(gate[t]).reshape(nq, hd), _act_bits(want_gate, ctx.act))
+        assert np.array_equal(_bits(v[t]), _act_bits(want_v, ctx.act))
+        # the rotation's sine and cosine come from two libraries: one 16-bit ulp
+        assert O.rel_error(act_np(q[t]), want_q) < 1e-2 and O.rel_error(act_np(k[t]).reshape(nkv, hd), want_k) < 1e-2
+        unrot = slice(rot, hd)
+        assert np.array_equal(_bits(q[t])[:, unrot], _act_bits(r(want_q), ctx.act)[:, unrot])
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("tokens,nq,nkv,hd,rot", [(1, 16, 2, 256, 64), (4, 4, 2, 64, 16), (3, 6, 3, 128, 128)])
+def test_qkv_epilogue_with_kv_write_equals_the_separate_calls(nv, ctx, bits, tokens, nq, nkv, hd, rot):
+    # the epilogue that also quantizes the finished k and v rows into the cache: q, gate and the
+    # cache rows are the bits of the epilogue followed by two KVCacheQuantizer.encode calls, with
+    # and without the 16-bit stage rows; the codes also equal the oracle's for the GPU's own rows
+    say("qkv epilogue + kv write", ctx.act, bits, tokens, nq, nkv, hd, rot)
+    rng = np.random.default_rng(900 + hd + tokens + bits)
+    proj, qw, kw, positions = _qkv_epilogue_case(nv, ctx, rng, tokens, nq, nkv, hd, rot, pad=0)
+    elements = nkv * hd
+    rc, q0, gate0, k0, v0 = _run_epilogue(nv, ctx, proj, qw, kw, positions, nq, nkv, hd, rot)
+    assert rc == 0
+    quant = nv.KVCacheQuantizer(ctx)
+    ref_k, ref_v = nv.KVCache(1, tokens + 2, elements, bits), nv.KVCache(1, tokens + 2, elements, bits)
+    quant.encode(k0, elements, ref_k.view(0, 1), tokens, elements)
+    quant.encode(v0, elements, ref_v.view(0, 1), tokens, elements)
+    for stage in (True, False):
+        kc, vc = nv.KVCache(1, tokens + 2, elements, bits), nv.KVCache(1, tokens + 2, elements, bits)
+        rc, q1, gate1, k1, v1 = _run_epilogue(nv, ctx, proj, qw, kw, positions, nq, nkv, hd, rot,
+                                              kviews=(kc.view(0, 1), vc.view(0, 1)), stage=stage)
+        assert rc == 0
+        assert torch.equal(q1.view(torch.int16), q0.view(torch.int16)) and torch.equal(gate1.view(torch.int16), gate0.view(torch.int16))
+        if stage:
+            assert torch.equal(k1.view(torch.int16), k0.view(torch.int16)) and torch.equal(v1.view(torch.int16), v0.view(torch.int16))
+        else:
+            assert int(k1.view(torch.int16).abs().max()) == 0      # untouched
+        assert torch.equal(kc.rows, ref_k.rows) and torch.equal(vc.rows, ref_v.rows)
+        stride = kc.rows.shape[-1]
+        want = O.kv_quantize(act_np(k0), bits)
+        assert np.array_equal(kc.rows[0, 1:1 + tokens].cpu().numpy()[:, :want.shape[1]], want[:, :stride])
+
+
+def test_qkv_epilogue_with_kv_write_rejects_bad_arguments(nv, ctx):
+    rng = np.random.default_rng(5)
+    tokens, nq, nkv, hd, rot = 2, 4, 2, 40, 8
+    proj, qw, kw, positions = _qkv_epilogue_case(nv, ctx, rng, tokens, nq, nkv, 64, rot, pad=0)
+    kc, vc = nv.KVCache(1, 4, nkv * 64, 8), nv.KVCache(1, 4, nkv * 64, 4)
+    # views of two formats
+    rc = _run_epilogue(nv, ctx, proj, qw, kw, positions, nq, nkv, 64, rot, kviews=(kc.view(0, 0), vc.view(0, 0)))[0]
+    assert rc != 0
+    # a head that is not whole groups of 64
+    proj, qw, kw, positions = _qkv_epilogue_case(nv, ctx, rng, tokens, nq, nkv, hd, rot, pad=0)
+    k40 = nv.KVCache(1, 4, 128, 8)
+    rc = _run_epilogue(nv, ctx, proj, qw, kw, positions, nq, nkv, hd, rot, kviews=(k40.view(0, 0), k40.view(0, 0)))[0]
+    assert rc != 0
