@@ -630,6 +630,19 @@ int nvmai_hip_gdn_delta_gated_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, cons
                                    uint32_t z_stride, const uint16_t* norm_weight, void* out, uint32_t out_stride,
                                    uint32_t rows, uint32_t batch);
 
+/* One decode token per sequence: nvmai_hip_gdn_conv_norm followed by nvmai_hip_gdn_delta_gated_norm
+ * (rows = 1) in ONE launch -- a block per (key head, sequence) runs the conv of its q / k channels
+ * once and the delta rule of each of its Hv / Hk value heads, and shifts its tail columns in place.
+ * Same bits as the two calls (out, state, tail).  Fused for (Dk, Dv) in {(128, 128), (32, 32)} with
+ * Hv / Hk in {1, 2}; any other shape runs the two kernels through conv_scratch ([batch,
+ * conv_scratch_stride] activations), and returns NVMAI_ERR_UNSUPPORTED when that is NULL. */
+int nvmai_hip_gdn_decode_step(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_gdn_config* config,
+                              const void* qkv_raw, uint32_t qkv_stride, void* tail, const uint16_t* conv_weight,
+                              void* conv_scratch, uint32_t conv_scratch_stride, const void* a_proj,
+                              const void* b_proj, uint32_t ab_stride, const uint16_t* a_log, const uint16_t* dt_bias,
+                              void* state, int state_is_bf16, const void* z, uint32_t z_stride,
+                              const uint16_t* norm_weight, void* out, uint32_t out_stride, uint32_t batch);
+
 /* GDN.encodeInputProjections (GDN.swift:85-128; kernel gdn_in_proj_gemv_simd, gdn.metal:179-239) and
  * FusedQKVGEMV.encode (kernel dequant_int4_qkv_gemv_simd, dequant_int4.metal:279-329): several
  * projections of the same input rows.  parts[i]: y_i = W_i x.  When the parts' codes, scales,

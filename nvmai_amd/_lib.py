@@ -136,6 +136,8 @@ SIGNATURES = {
     "nvmai_hip_attn_qkv_epilogue_kv": [vp, vp, vp, u32, C.c_int, vp, vp, vp, vp, vp, vp, u32, C.POINTER(KvView),
                                        C.POINTER(KvView), u32, u32, u32, u32, u32, C.c_int, vp, u32, C.c_float, C.c_float],
     "nvmai_hip_gdn_conv_norm": [vp, vp, C.POINTER(GdnConfig), vp, u32, vp, vp, vp, u32, u32, u32],
+    "nvmai_hip_gdn_decode_step": [vp, vp, C.POINTER(GdnConfig), vp, u32, vp, vp, vp, u32, vp, vp, u32, vp, vp, vp, C.c_int,
+                                  vp, u32, vp, vp, u32, u32],
     "nvmai_hip_gdn_delta_gated_norm": [vp, vp, C.POINTER(GdnConfig), vp, u32, vp, vp, u32, vp, vp, vp, C.c_int, vp, u32,
                                        vp, vp, u32, u32, u32],
     "nvmai_hip_affine_gemv_fused": [vp, vp, C.POINTER(GemvPart), u32, u32, vp, u32, u32, u32],

@@ -89,6 +89,68 @@ extern "C" int nvmai_hip_gdn_delta_gated_norm(nvmai_hip_ctx* ctx, nvmai_stream s
     return launch_status();
 }
 
+namespace {
+template <int ACT, int DK, int DV>
+bool launch_decode_fused(const GdnDecodeParams& p, uint32_t ratio, bool state_bf16, hipStream_t s) {
+    const dim3 grid(p.d.sh.k_heads, p.d.sh.batch);
+#define NVMAI_GDN_FUSED(R)                                                                             \
+    do {                                                                                               \
+        if (state_bf16) gdn_decode_fused_kernel<ACT, DK, DV, R, true><<<grid, 256 * R, 0, s>>>(p);      \
+        else gdn_decode_fused_kernel<ACT, DK, DV, R, false><<<grid, 256 * R, 0, s>>>(p);                \
+        return true;                                                                                   \
+    } while (0)
+    if (ratio == 1) NVMAI_GDN_FUSED(1);
+    if (ratio == 2) NVMAI_GDN_FUSED(2);
+#undef NVMAI_GDN_FUSED
+    return false;
+}
+
+template <int ACT>
+bool launch_decode_fused_shape(const GdnDecodeParams& p, uint32_t ratio, bool state_bf16, hipStream_t s) {
+    const uint32_t dk = p.d.sh.dk, dv = p.d.sh.dv;
+    if (dk == 128 && dv == 128) return launch_decode_fused<ACT, 128, 128>(p, ratio, state_bf16, s);
+    if (dk == 32 && dv == 32) return launch_decode_fused<ACT, 32, 32>(p, ratio, state_bf16, s);
+    return false;
+}
+}  // namespace
+
+extern "C" int nvmai_hip_gdn_decode_step(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_gdn_config* config,
+                                         const void* qkv_raw, uint32_t qkv_stride, void* tail, const uint16_t* conv_weight,
+                                         void* conv_scratch, uint32_t conv_scratch_stride, const void* a_proj,
+                                         const void* b_proj, uint32_t ab_stride, const uint16_t* a_log,
+                                         const uint16_t* dt_bias, void* state, int state_is_bf16, const void* z,
+                                         uint32_t z_stride, const uint16_t* norm_weight, void* out, uint32_t out_stride,
+                                         uint32_t batch) {
+    if (!ctx || !qkv_raw || !tail || !conv_weight || !a_proj || !b_proj || !a_log || !dt_bias || !state || !z ||
+        !norm_weight || !out)
+        return NVMAI_ERR_INVALID_ARG;
+    int rc = check_gdn(config, 1, batch);
+    if (rc) return rc;
+    const uint32_t C = 2 * config->num_k_heads * config->key_head_dim + config->num_v_heads * config->value_head_dim;
+    const uint32_t vd = config->num_v_heads * config->value_head_dim;
+    if (qkv_stride < C || ab_stride < config->num_v_heads || z_stride < vd || out_stride < vd) return NVMAI_ERR_INVALID_ARG;
+    GdnDecodeParams p{};
+    p.d.a_proj = (const uint16_t*)a_proj; p.d.b_proj = (const uint16_t*)b_proj; p.d.ab_stride = ab_stride;
+    p.d.a_log = a_log; p.d.dt_bias = dt_bias; p.d.state = state;
+    p.d.z = (const uint16_t*)z; p.d.z_stride = z_stride; p.d.norm_w = norm_weight;
+    p.d.out = (uint16_t*)out; p.d.out_stride = out_stride;
+    p.d.sh = shape_of(config, 1, batch);
+    p.qkv_raw = (const uint16_t*)qkv_raw; p.qkv_stride = qkv_stride; p.tail = (uint16_t*)tail; p.conv_w = conv_weight;
+    hipStream_t s = (hipStream_t)stream;
+    const uint32_t ratio = config->num_v_heads / config->num_k_heads;
+    const bool fused = ctx->act == ACT_BF16 ? launch_decode_fused_shape<ACT_BF16>(p, ratio, state_is_bf16 != 0, s)
+                                            : launch_decode_fused_shape<ACT_FP16>(p, ratio, state_is_bf16 != 0, s);
+    if (fused) return launch_status();
+    // a shape without a fused instantiation: the two kernels one after the other through the scratch rows
+    if (!conv_scratch || conv_scratch_stride < C) return NVMAI_ERR_UNSUPPORTED;
+    rc = nvmai_hip_gdn_conv_norm(ctx, stream, config, qkv_raw, qkv_stride, tail, conv_weight, conv_scratch,
+                                 conv_scratch_stride, 1, batch);
+    if (rc) return rc;
+    return nvmai_hip_gdn_delta_gated_norm(ctx, stream, config, conv_scratch, conv_scratch_stride, a_proj, b_proj, ab_stride,
+                                          a_log, dt_bias, state, state_is_bf16, z, z_stride, norm_weight, out, out_stride,
+                                          1, batch);
+}
+
 // One GEMV launch over the concatenated rows of several matrices when they lie back to back in
 // memory (codes, scales and biases each, and the outputs), one launch per matrix otherwise.
 extern "C" int nvmai_hip_affine_gemv_fused(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_gemv_part* parts,

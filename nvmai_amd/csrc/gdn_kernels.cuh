@@ -194,4 +194,150 @@ __global__ __launch_bounds__(256) void gdn_delta_gated_kernel(GdnDeltaParams p) 
     }
 }
 
+
+// ---- one decode token: both kernels above in one launch --------------------------------------------
+// Block (key head, sequence) of 256 R threads, R = Hv / Hk value heads per key head: the first 256
+// threads run the conv + SiLU + norm of the key head's q and k channels (q on waves 0 - 1, k on
+// waves 2 - 3: each channel on the lane it has in gdn_conv_norm_kernel, wave sums added in that
+// kernel's order, so the same bits), group r of 256 threads the conv of value head Hk-head * R + r
+// and then its delta rule and gated norm exactly as gdn_delta_gated_kernel does, with q, k and v
+// taken from LDS instead of a conv_out row in memory.  The thread that computes a channel holds the
+// channel's tail column in registers and writes it back shifted: the block is the only reader of
+// its channels, so the tail is updated in place with no ordering between blocks.  The state rows
+// are requested before the conv so that they arrive while it runs.
+struct GdnDecodeParams {
+    GdnDeltaParams d;           // conv_out unused
+    const uint16_t* qkv_raw;    // [batch, qkv_stride]
+    uint32_t qkv_stride;
+    uint16_t* tail;             // [batch, taps - 1, C]
+    const uint16_t* conv_w;     // BF16 [C, taps]
+};
+
+template <int ACT, int DK, int DV, int R, bool STATE_BF16>
+__global__ __launch_bounds__(256 * R) void gdn_decode_fused_kernel(GdnDecodeParams pp) {
+    constexpr int EPL = DK / 16;
+    constexpr int GROUPS = DV / 16;
+    static_assert(DK <= 128 && DV <= 256 /* one channel per thread */ && DK % 16 == 0 && DV % 16 == 0, "shape");
+    __shared__ float q_s[DK], k_s[DK];
+    __shared__ float v_s[R][DV], y_s[R][DV];
+    __shared__ float part_qk[4], part[R][4];
+    const GdnDeltaParams& p = pp.d;
+    const GdnShape& sh = p.sh;
+    const uint32_t hk = blockIdx.x, b = blockIdx.y;
+    const uint32_t r = threadIdx.x >> 8, lt = threadIdx.x & 255u;          // value head of the group, thread in the group
+    const uint32_t lane = lt & 63u, wave = lt >> 6;
+    const uint32_t h = hk * R + r;
+    const uint32_t sub = lt & 15u, row_in_pass = lt >> 4;
+    const uint32_t C = 2 * sh.k_heads * DK + sh.v_heads * DV;
+    const uint32_t hist = sh.taps - 1;
+
+    // ---- the state rows of this value head
+    const size_t state_base = (((size_t)b * sh.v_heads + h) * DV) * DK;
+    float s[GROUPS][EPL];
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+        const size_t at = state_base + (size_t)(g * 16 + row_in_pass) * DK + sub * EPL;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e)
+            s[g][e] = STATE_BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(p.state)[at + e])
+                                 : reinterpret_cast<const float*>(p.state)[at + e];
+    }
+
+    // everything else the token needs from memory is requested now as well, ahead of the conv's barriers
+    const size_t row = b;
+    const uint16_t a_raw = p.a_proj[row * p.ab_stride + h], b_raw = p.b_proj[row * p.ab_stride + h];
+    const uint16_t a_log_raw = p.a_log[h], dt_raw = p.dt_bias[h];
+    const uint16_t z_raw = lt < (uint32_t)DV ? p.z[row * p.z_stride + h * DV + lt] : (uint16_t)0;
+    const uint16_t nw_raw = lt < (uint32_t)DV ? p.norm_w[lt] : (uint16_t)0;
+
+    // ---- conv + SiLU of one channel, tail column shifted in place; returns the 16-bit result as a float
+    uint16_t* tl = pp.tail + (size_t)b * hist * C;
+    const uint16_t* raw = pp.qkv_raw + (size_t)b * pp.qkv_stride;
+    auto conv_channel = [&](uint32_t ch) -> float {
+        uint16_t x[GDN_MAX_TAPS];
+#pragma unroll
+        for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+            if (j > hist) break;
+            x[j] = j < hist ? tl[(size_t)j * C + ch] : raw[ch];
+        }
+        float acc = 0.0f;
+#pragma unroll
+        for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+            if (j > hist) break;
+            acc = fmaf(act_to_f32<ACT>(x[j]), bf16_to_f32(pp.conv_w[ch * sh.taps + j]), acc);
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+            if (j >= hist) break;
+            tl[(size_t)j * C + ch] = x[j + 1];
+        }
+        return act_to_f32<ACT>(f32_to_act<ACT>(gdn_silu(acc)));
+    };
+    // q: threads 0 .. DK - 1 of group 0; k: threads 128 .. 128 + DK - 1 of group 0
+    const bool is_q = r == 0 && lt < (uint32_t)DK, is_k = r == 0 && lt >= 128u && lt < 128u + (uint32_t)DK;
+    float qk = 0.0f;
+    if (is_q) qk = conv_channel(hk * DK + lt);
+    if (is_k) qk = conv_channel(sh.k_heads * DK + hk * DK + (lt - 128u));
+    if (lt < (uint32_t)DV) v_s[r][lt] = conv_channel(2 * sh.k_heads * DK + h * DV + lt);
+    if (r == 0) {
+        const float ws = wave_sum_bcast(qk * qk);               // fma(x, x, 0) of the separate kernel
+        if (lane == 0) part_qk[wave] = ws;
+    }
+    __syncthreads();
+    if (is_q || is_k) {
+        const float total = is_q ? (part_qk[0] + part_qk[1]) + (0.0f + 0.0f) : (part_qk[2] + part_qk[3]) + (0.0f + 0.0f);
+        // the divisor and the k scale from the run-time shape, as gdn_conv_norm_kernel takes them
+        const float inv = rsqrtf(total / (float)sh.dk + GDN_RMS_EPS);
+        const float scale = is_q ? 1.0f / (float)sh.dk : rsqrtf((float)sh.dk);
+        const float o = act_to_f32<ACT>(f32_to_act<ACT>(qk * inv * scale));
+        if (is_q) q_s[lt] = o; else k_s[lt - 128u] = o;
+    }
+    __syncthreads();
+
+    // ---- delta rule + gated norm of value head h (gdn_delta_gated_kernel, one row)
+    const float exp_a = expf(bf16_to_f32(a_log_raw));
+    const float dtb = bf16_to_f32(dt_raw);
+    float q[EPL], k[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) { q[e] = q_s[sub * EPL + e]; k[e] = k_s[sub * EPL + e]; }
+    const float g_decay = expf(-exp_a * gdn_softplus(act_to_f32<ACT>(a_raw) + dtb));
+    const float beta = 1.0f / (1.0f + expf(-act_to_f32<ACT>(b_raw)));
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+        const uint32_t dv = g * 16 + row_in_pass;
+        float kv = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) { s[g][e] *= g_decay; kv = fmaf(s[g][e], k[e], kv); }
+        kv = seg_reduce_sum<16>(kv);
+        const float delta = (v_s[r][dv] - kv) * beta;
+        float o = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) { s[g][e] = fmaf(k[e], delta, s[g][e]); o = fmaf(s[g][e], q[e], o); }
+        o = seg_reduce_sum<16>(o);
+        if (sub == 0) y_s[r][dv] = act_to_f32<ACT>(f32_to_act<ACT>(o));
+    }
+    __syncthreads();
+    float sumsq = 0.0f;
+    if (lt < (uint32_t)DV) sumsq = fmaf(y_s[r][lt], y_s[r][lt], sumsq);
+    sumsq = wave_sum_bcast(sumsq);
+    if (lane == 0) part[r][wave] = sumsq;
+    __syncthreads();
+    const float total = (part[r][0] + part[r][1]) + (part[r][2] + part[r][3]);
+    const float inv = rsqrtf(total / (float)DV + GDN_RMS_EPS);
+    if (lt < (uint32_t)DV) {
+        const float normed = y_s[r][lt] * inv * bf16_to_f32(nw_raw);
+        const float gate = gdn_silu(act_to_f32<ACT>(z_raw));
+        p.out[row * p.out_stride + h * DV + lt] = f32_to_act<ACT>(normed * gate);
+    }
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+        const size_t at = state_base + (size_t)(g * 16 + row_in_pass) * DK + sub * EPL;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            if (STATE_BF16) reinterpret_cast<uint16_t*>(p.state)[at + e] = f32_to_bf16(s[g][e]);
+            else reinterpret_cast<float*>(p.state)[at + e] = s[g][e];
+        }
+    }
+}
+
 }  // namespace nvmai

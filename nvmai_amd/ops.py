@@ -726,6 +726,24 @@ class GDN:
         return out
 
 
+    def encode_decode_step(self, qkv_raw, tail, conv_weight, a_proj, b_proj, a_log, dt_bias, state, z, norm_weight,
+                           out=None, conv_scratch=None):
+        """One token per sequence: encode_conv_norm + encode_delta_gated_norm in one launch (same bits);
+        conv_scratch [batch, C] is only used for shapes without a fused kernel."""
+        q2 = qkv_raw.reshape(-1, qkv_raw.shape[-1])
+        batch = q2.shape[0]
+        if out is None:
+            out = torch.empty((batch, self.value_dim), dtype=self.ctx.dtype, device=q2.device)
+        check(lib.nvmai_hip_gdn_decode_step(self.ctx.handle, _stream(), C.byref(self.cfg), _ptr(q2), q2.stride(0),
+                                            _ptr(tail), _ptr(conv_weight), _ptr(conv_scratch),
+                                            0 if conv_scratch is None else conv_scratch.stride(0), _ptr(a_proj),
+                                            _ptr(b_proj), a_proj.stride(0), _ptr(a_log), _ptr(dt_bias), _ptr(state),
+                                            int(state.dtype == torch.bfloat16), _ptr(z), z.stride(0), _ptr(norm_weight),
+                                            _ptr(out), out.stride(0), batch),
+              "gdn_decode_step")
+        return out
+
+
 class GenerationConfig:
     """GenerationConfig (Sampler.swift:19-81), the fields the sampler reads; top_k / top_p / seed may be
     None as in the reference (defaults: GenerationDefaults, Sampler.swift:6-11)."""

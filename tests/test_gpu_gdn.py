@@ -132,6 +132,45 @@ def test_gdn_batch_of_sequences_and_bf16_state(nv, ctx, bf16_state):
         assert np.abs(got_state[b] - refs[b].state).max() <= (5e-2 if not bf16_state else 1e-1)
 
 
+@pytest.mark.parametrize("bf16_state", [False, True])
+@pytest.mark.parametrize("cfg", [(2, 4, 32, 32, 4), (16, 32, 128, 128, 4), (4, 4, 32, 32, 2), (2, 2, 64, 64, 2), (2, 8, 32, 32, 4)],
+                         ids=["toy", "production", "ratio1-taps2", "two-kernel-shape", "two-kernel-ratio"])
+def test_gdn_decode_step_in_one_launch_equals_the_two_calls(nv, ctx, cfg, bf16_state):
+    # conv + q / k norm + tail update + delta rule + gated norm of one token per sequence in one launch:
+    # outputs, recurrent state and conv tail are the bits of the two calls, token after token, for a
+    # batch of three sequences; the fused shapes and the shapes that go through the scratch rows
+    say("gdn decode step, one launch", ctx.act, cfg, bf16_state)
+    batch, steps = 3, 5
+    fxs = [_fixture(cfg, steps, 300 + b, ctx.act) for b in range(batch)]
+    gdn = nv.GDN(ctx, *cfg)
+    tail_a, state_a = gdn.new_state(batch, bf16=bf16_state)
+    tail_b, state_b = gdn.new_state(batch, bf16=bf16_state)
+    w = fxs[0]
+    ref = O.GdnLayerState(*cfg)
+    scratch = torch.empty((batch, gdn.qkv_dim), dtype=ctx.dtype, device="cuda")
+    for t in range(steps):
+        stack = lambda key: act_tensor(np.stack([fx[key][t] for fx in fxs]), ctx)
+        qkv, a, b, z = stack("qkv"), stack("a"), stack("b"), stack("z")
+        weights = (_bits(w["a_log"]), _bits(w["dt_bias"]))
+        conv = gdn.encode_conv_norm(qkv, tail_a, _bits(w["conv_w"]))
+        two = gdn.encode_delta_gated_norm(conv, a, b, weights[0], weights[1], state_a, z, _bits(w["norm_w"]))
+        one = gdn.encode_decode_step(qkv, tail_b, _bits(w["conv_w"]), a, b, weights[0], weights[1], state_b, z,
+                                     _bits(w["norm_w"]), conv_scratch=scratch)
+        torch.cuda.synchronize()
+        assert torch.equal(one.view(torch.int16), two.view(torch.int16)), "token %d" % t
+        assert torch.equal(tail_a.view(torch.int16), tail_b.view(torch.int16))
+        assert torch.equal(state_a.view(torch.int32 if not bf16_state else torch.int16),
+                           state_b.view(torch.int32 if not bf16_state else torch.int16))
+        if not bf16_state:
+            want = O.gdn_step(ref, fxs[0]["qkv"][t], fxs[0]["a"][t], fxs[0]["b"][t], fxs[0]["z"][t], w["conv_w"],
+                              w["a_log"], w["dt_bias"], w["norm_w"], ctx.act)
+            assert _close(act_np(one)[0], want, ctx.act)
+    # a shape without a fused kernel and no scratch rows
+    if cfg == (2, 2, 64, 64, 2):
+        with pytest.raises(nv.NvmaiError):
+            gdn.encode_decode_step(qkv, tail_b, _bits(w["conv_w"]), a, b, weights[0], weights[1], state_b, z, _bits(w["norm_w"]))
+
+
 def test_gdn_rejects_bad_shapes(nv, ctx):
     say("gdn errors")
     with pytest.raises(nv.NvmaiError) as e:            # numVHeads must be a multiple of numKHeads (GDN.swift:44-45)
