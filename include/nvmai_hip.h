@@ -333,6 +333,33 @@ int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream stream, const
                                   const nvmai_prefill_grouping* grouping, void* act_scratch,
                                   void* route_partials);
 
+/* PrefillGroupedRoutedMoEStreamedParams (PrefillGroupedRoutedMoE.swift:104-183 == prefill.metal:231-264):
+ * the per-tile parameter block, 128 bytes, field for field (the reference's layout test:
+ * PrefillGroupedRoutedMoETests+Layout.swift:7-30).  local_expert[i] = global id of the expert in
+ * local slot i, 0xFFFFFFFF for the unused slots. */
+typedef struct {
+    uint32_t pair_start, pair_count, d, routed_intermediate, top_k, hidden_stride_elements, live_expert_count;
+    uint32_t local_expert[16];
+    uint32_t gate_w_off, gate_s_off, gate_b_off, up_w_off, up_s_off, up_b_off, down_w_off, down_s_off, down_b_off;
+} nvmai_prefill_streamed_params;
+
+/* PrefillGroupedRoutedMoE.encodeStreamedBatched for ONE tile (PrefillGroupedRoutedMoE.swift:413-489) with
+ * the tile's experts bound one by one, as PrefillStreamedTileBinding (:185-323) binds the buffers
+ * they were fetched into: expert_blobs is a HOST array of params->live_expert_count device pointers,
+ * blob i = the expert params->local_expert[i] (16-byte aligned, any offset inside a larger buffer).
+ * Runs gate/up + SwiGLU and down over the sorted pairs [pair_start, pair_start + pair_count) and
+ * writes act_scratch[p, :] and route_partials[token * top_k + rank, :] for exactly those pairs;
+ * sorted_pairs is the whole sorted array (n_sorted_pairs records), hidden [tokens,
+ * hidden_stride_elements].  The binding's own checks (1..16 experts, unique ids) and the pair
+ * range return NVMAI_ERR_INVALID_ARG; a pair whose expert is not bound (validateCoversPairs,
+ * :274-287) is found on the device: nothing is computed and err (optional, 2 device words) =
+ * (1, index of the first such pair), else (0, 0).  Same kernels as nvmai_hip_prefill_grouped_moe. */
+int nvmai_hip_prefill_grouped_moe_streamed(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                           const nvmai_prefill_streamed_params* params,
+                                           const void* const* expert_blobs, uint32_t bits, const void* hidden,
+                                           const nvmai_prefill_pair* sorted_pairs, uint64_t n_sorted_pairs,
+                                           void* act_scratch, void* route_partials, uint32_t* err);
+
 /* MPPPrefillInt4QMM.encode (MPPPrefillInt4QMM.swift:63-128; kernel tensorops.metal:29-121):
  * the dense prefill product y[m, n] = x[m, k] . W[n, k]^T for m rows of activations against
  * one affine 4/8-bit matrix (group 64 along k, BF16 scale/bias), on the matrix cores: weights

@@ -66,6 +66,15 @@ class GemvPart(C.Structure):
     _fields_ = [("weights", vp), ("scales", vp), ("biases", vp), ("rows", u32), ("y", vp), ("y_stride", u32)]
 
 
+class PrefillStreamedParams(C.Structure):
+    """nvmai_prefill_streamed_params == PrefillGroupedRoutedMoEStreamedParams, 128 bytes"""
+    _fields_ = ([(n, u32) for n in ("pair_start", "pair_count", "d", "routed_intermediate", "top_k",
+                                    "hidden_stride_elements", "live_expert_count")] +
+                [("local_expert", u32 * 16)] +
+                [(n, u32) for n in ("gate_w_off", "gate_s_off", "gate_b_off", "up_w_off", "up_s_off", "up_b_off",
+                                    "down_w_off", "down_s_off", "down_b_off")])
+
+
 class PrefillGrouping(C.Structure):
     """nvmai_prefill_grouping"""
     _fields_ = [(n, vp) for n in ("sorted_pairs", "expert_offsets", "expert_counts", "groups", "tiles", "info")]
@@ -116,6 +125,8 @@ SIGNATURES = {
     "nvmai_hip_prefill_group_routes": [vp, vp, vp, vp, u32, u32, u32, u32, vp, u64, C.POINTER(PrefillGrouping)],
     "nvmai_hip_prefill_grouped_moe": [vp, vp, vp, u64, C.POINTER(ExpertOffsets), u32, u32, u32, u32, vp, u32,
                                       u32, u32, C.POINTER(PrefillGrouping), vp, vp],
+    "nvmai_hip_prefill_grouped_moe_streamed": [vp, vp, C.POINTER(PrefillStreamedParams), C.POINTER(vp), u32, vp, vp, u64,
+                                               vp, vp, vp],
     "nvmai_hip_affine_qmm": [vp, vp, vp, vp, vp, u32, vp, u32, vp, u32, u32, u32, u32],
     "nvmai_hip_prefill_moe_reduce_token_major": [vp, vp, vp, vp, vp, u32, u32, u32, u32],
     "nvmai_hip_silu_mul": [vp, vp, vp, vp, vp, u32],

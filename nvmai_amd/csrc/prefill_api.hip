@@ -271,6 +271,93 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
     return launch_status();
 }
 
+// One streamed tile: PrefillGroupedRoutedMoE.encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:413-489)
+// with the tile's experts bound through separate blobs.
+extern "C" int nvmai_hip_prefill_grouped_moe_streamed(nvmai_hip_ctx* ctx, nvmai_stream stream,
+                                                      const nvmai_prefill_streamed_params* params,
+                                                      const void* const* expert_blobs, uint32_t bits,
+                                                      const void* hidden, const nvmai_prefill_pair* sorted_pairs,
+                                                      uint64_t n_sorted_pairs, void* act_scratch, void* route_partials,
+                                                      uint32_t* err) {
+    static_assert(sizeof(nvmai_prefill_streamed_params) == 128, "PrefillGroupedRoutedMoEStreamedParams is 128 bytes");
+    if (!ctx || !params || !expert_blobs || !hidden || !sorted_pairs || !act_scratch || !route_partials)
+        return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    const uint32_t d = params->d, f = params->routed_intermediate, top_k = params->top_k;
+    const uint32_t live = params->live_expert_count;
+    // PrefillStreamedTileBinding.init (PrefillGroupedRoutedMoE.swift:189-214): 1 .. 16 experts, ids unique
+    if (live == 0 || live > STREAMED_MAX_EXPERTS) return NVMAI_ERR_INVALID_ARG;
+    for (uint32_t i = 0; i < live; ++i) {
+        if (!expert_blobs[i] || params->local_expert[i] == 0xFFFFFFFFu) return NVMAI_ERR_INVALID_ARG;
+        if (!aligned16(expert_blobs[i])) return NVMAI_ERR_ALIGNMENT;
+        for (uint32_t j = 0; j < i; ++j)
+            if (params->local_expert[j] == params->local_expert[i]) return NVMAI_ERR_INVALID_ARG;
+    }
+    if (d == 0 || f == 0 || d % NVMAI_GROUP || f % NVMAI_GROUP || top_k == 0 || params->hidden_stride_elements < d)
+        return NVMAI_ERR_INVALID_ARG;
+    // validateCoversPairs' range check (:274-279)
+    if ((uint64_t)params->pair_start + params->pair_count > n_sorted_pairs) return NVMAI_ERR_INVALID_ARG;
+    const uint32_t offs[9] = {params->gate_w_off, params->gate_s_off, params->gate_b_off, params->up_w_off,
+                              params->up_s_off, params->up_b_off, params->down_w_off, params->down_s_off,
+                              params->down_b_off};
+    for (int i = 0; i < 9; ++i)
+        if (offs[i] % (i % 3 == 0 ? 16 : 2)) return NVMAI_ERR_ALIGNMENT;
+    if (!aligned16(hidden) || params->hidden_stride_elements % 8 || !aligned16(act_scratch) || !aligned16(route_partials))
+        return NVMAI_ERR_ALIGNMENT;
+    if (n_sorted_pairs >= (1u << 28)) return NVMAI_ERR_UNSUPPORTED;
+    if (n_sorted_pairs * f * 2 > 0xFFFFFFFFull || n_sorted_pairs * d * 2 > 0xFFFFFFFFull ||
+        (uint64_t)d * f * bits / 8 > 0xFFFFFFFFull)
+        return NVMAI_ERR_UNSUPPORTED;
+    if (params->pair_count == 0) return NVMAI_OK;
+    // the extent of a blob, from its last array: the bound of the kernel's scale / bias resources
+    uint64_t extent = 0;
+    const uint64_t w_bytes = (uint64_t)d * f * bits / 8, gu_meta = (uint64_t)f * (d / NVMAI_GROUP) * 2,
+                   dn_meta = (uint64_t)d * (f / NVMAI_GROUP) * 2;
+    const uint64_t ends[9] = {offs[0] + w_bytes, offs[1] + gu_meta, offs[2] + gu_meta, offs[3] + w_bytes, offs[4] + gu_meta,
+                              offs[5] + gu_meta, offs[6] + w_bytes, offs[7] + dn_meta, offs[8] + dn_meta};
+    for (int i = 0; i < 9; ++i) extent = ends[i] > extent ? ends[i] : extent;
+    if (extent > 0xFFFFFFFFull) return NVMAI_ERR_UNSUPPORTED;
+    const uint32_t max_mtiles = params->pair_count / GEMM_BM + live;
+    int rc = ws_begin(ctx, stream, ws_round((size_t)GEMM_XCDS * max_mtiles * sizeof(MTile)) + ws_round(GEMM_XCDS * 4) +
+                                       ws_round(STREAMED_MAX_EXPERTS * sizeof(void*)));
+    if (rc) return rc;
+    MTile* mtiles = ws_take<MTile>(ctx, (size_t)GEMM_XCDS * max_mtiles);
+    uint32_t* qwords = ws_take<uint32_t>(ctx, GEMM_XCDS);
+    const uint8_t** table = ws_take<const uint8_t*>(ctx, STREAMED_MAX_EXPERTS);
+    StreamedBind b{};
+    for (uint32_t i = 0; i < live; ++i) { b.blob[i] = (const uint8_t*)expert_blobs[i]; b.expert[i] = params->local_expert[i]; }
+    b.live = live; b.pair_start = params->pair_start; b.pair_count = params->pair_count;
+    hipStream_t s = (hipStream_t)stream;
+    prefill_streamed_mtiles_kernel<<<1, 256, 0, s>>>(reinterpret_cast<const PrefillPair*>(sorted_pairs), b, table, mtiles,
+                                                     max_mtiles, qwords, err);
+    const uint32_t nt = bits == 4 ? 4 : 2;
+    GemmParams g1{};
+    g1.pool = nullptr; g1.pool_stride = extent; g1.blob_table = table;
+    g1.wA = offs[0]; g1.sA = offs[1]; g1.bA = offs[2];
+    g1.wB = offs[3]; g1.sB = offs[4]; g1.bB = offs[5];
+    g1.mtiles = mtiles; g1.list_cap = max_mtiles; g1.list_len = qwords;
+    g1.pairs = reinterpret_cast<const PrefillPair*>(sorted_pairs);
+    g1.x = hidden; g1.x_stride = params->hidden_stride_elements;
+    g1.out = act_scratch; g1.out_stride = f;
+    g1.K = d; g1.N = f; g1.top_k = top_k; g1.n_tiles_n = (f + 32 * nt - 1) / (32 * nt);
+    g1.units_per_tile = (g1.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
+    GemmParams g2 = g1;
+    g2.wA = offs[6]; g2.sA = offs[7]; g2.bA = offs[8];
+    g2.wB = g2.sB = g2.bB = 0;
+    g2.x = act_scratch; g2.x_stride = f;
+    g2.out = route_partials; g2.out_stride = d;
+    g2.K = f; g2.N = d; g2.n_tiles_n = (d + 64 * nt - 1) / (64 * nt);
+    g2.units_per_tile = (g2.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
+    if (ctx->act == ACT_BF16) {
+        if (bits == 4) launch_gemms<ACT_BF16, 4, 4>(g1, g2, max_mtiles, ctx, s);
+        else launch_gemms<ACT_BF16, 8, 2>(g1, g2, max_mtiles, ctx, s);
+    } else {
+        if (bits == 4) launch_gemms<ACT_FP16, 4, 4>(g1, g2, max_mtiles, ctx, s);
+        else launch_gemms<ACT_FP16, 8, 2>(g1, g2, max_mtiles, ctx, s);
+    }
+    return launch_status();
+}
+
 namespace {
 template <int ACT, int BITS, int NT>
 void launch_qmm(const GemmParams& g, uint32_t blocks, hipStream_t s) {

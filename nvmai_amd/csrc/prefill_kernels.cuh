@@ -530,6 +530,61 @@ __global__ __launch_bounds__(256) void prefill_mtiles_kernel(const PrefillGroup*
     }
 }
 
+// ---- one streamed tile: experts bound one by one ----------------------------------------------
+// The reference runs a tile of at most sixteen experts whose blobs were fetched into separate
+// buffers (PrefillStreamedTileBinding, PrefillGroupedRoutedMoE.swift:185-323) over the sorted pairs
+// [pair_start, pair_start + pair_count) (PrefillGroupedRoutedMoEStreamedParams, :104-183 ==
+// prefill.metal:231-264).  This kernel turns such a call into the GEMM's work lists: the run of
+// each bound expert inside the pair range (the pairs are sorted, so an expert's pairs are one
+// run) is cut into M tiles whose `expert` is the LOCAL slot, dealt tile by tile over the lists,
+// and the slots' blob addresses go into the table the GEMM reads.  A pair whose expert is not
+// bound (validateCoversPairs, :274-287) lists nothing and reports (1, pair index) in err.
+constexpr uint32_t STREAMED_MAX_EXPERTS = 16;
+struct StreamedBind {
+    const uint8_t* blob[STREAMED_MAX_EXPERTS];
+    uint32_t expert[STREAMED_MAX_EXPERTS];      // global expert id of local slot i
+    uint32_t live, pair_start, pair_count;
+};
+
+__global__ __launch_bounds__(256) void prefill_streamed_mtiles_kernel(const PrefillPair* pairs, StreamedBind b,
+                                                                     const uint8_t** table, MTile* mtiles,
+                                                                     uint32_t list_cap, uint32_t* list_len,
+                                                                     uint32_t* err) {
+    __shared__ uint32_t start[STREAMED_MAX_EXPERTS], stop[STREAMED_MAX_EXPERTS];
+    __shared__ uint32_t bad;
+    const uint32_t tid = threadIdx.x;
+    if (tid < STREAMED_MAX_EXPERTS) {
+        start[tid] = 0; stop[tid] = 0;
+        table[tid] = tid < b.live ? b.blob[tid] : nullptr;
+    }
+    if (tid == 0) bad = 0xFFFFFFFFu;
+    __syncthreads();
+    const uint32_t lo = b.pair_start, hi = b.pair_start + b.pair_count;
+    for (uint32_t i = lo + tid; i < hi; i += 256) {
+        const uint32_t e = pairs[i].expert;
+        const bool first = i == lo || pairs[i - 1].expert != e;
+        const bool last = i + 1 == hi || pairs[i + 1].expert != e;
+        if (!first && !last) continue;
+        uint32_t slot = STREAMED_MAX_EXPERTS;
+        for (uint32_t j = 0; j < b.live; ++j)
+            if (b.expert[j] == e) { slot = j; break; }
+        if (slot == STREAMED_MAX_EXPERTS) { atomicMin(&bad, i); continue; }
+        if (first) start[slot] = i;
+        if (last) stop[slot] = i + 1;
+    }
+    __syncthreads();
+    if (tid != 0) return;
+    if (err) { err[0] = bad != 0xFFFFFFFFu ? 1u : 0u; err[1] = bad != 0xFFFFFFFFu ? bad : 0u; }
+    uint32_t n = 0;
+    if (bad == 0xFFFFFFFFu) {
+        for (uint32_t slot = 0; slot < b.live; ++slot)
+            for (uint32_t r = start[slot]; r < stop[slot]; r += GEMM_BM, ++n)
+                mtiles[(size_t)(n % GEMM_XCDS) * list_cap + n / GEMM_XCDS] =
+                    MTile{slot, r, stop[slot] - r < (uint32_t)GEMM_BM ? stop[slot] - r : (uint32_t)GEMM_BM};
+    }
+    for (uint32_t x = 0; x < GEMM_XCDS; ++x) list_len[x] = n / GEMM_XCDS + (x < n % GEMM_XCDS ? 1u : 0u);
+}
+
 // ---- grouped GEMM ---------------------------------------------------------------------------
 // out[m, n] = sum_k X[row(m), k] * W_e[n, k] for the rows of one M tile (<= 128 sorted pairs of
 // one expert) and GEMM_BN output columns: DUAL -> gate and up rows of the same columns,
@@ -554,6 +609,8 @@ typedef float fl4_t __attribute__((ext_vector_type(4)));
 struct GemmParams {
     const uint8_t* pool;
     uint64_t pool_stride;
+    const uint8_t* const* blob_table;   // optional: expert e's blob at blob_table[e] (experts bound one by one,
+                                        // PrefillStreamedTileBinding) instead of pool + e * pool_stride
     int64_t wA, sA, bA, wB, sB, bB;     // A: gate or down; B: up
     const MTile* mtiles;                // grouped product: list x of M tiles at mtiles + x * list_cap
     uint32_t list_cap;
@@ -700,7 +757,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
         if (at >= p.list_len[list]) return;
         mt = p.mtiles[(size_t)list * p.list_cap + at];
     }
-    const uint8_t* blob = p.pool + (uint64_t)mt.expert * p.pool_stride;
+    const uint8_t* blob = p.blob_table ? p.blob_table[mt.expert] : p.pool + (uint64_t)mt.expert * p.pool_stride;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lq = lane >> 4;

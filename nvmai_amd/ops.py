@@ -417,6 +417,127 @@ class PrefillGroupedRoutedMoE:
         return route_partials, act_scratch
 
 
+    def encode_streamed_batched(self, hidden, sorted_pairs, route_partials, act_scratch, binding, params, err=None):
+        """encodeStreamedBatched for one tile (PrefillGroupedRoutedMoE.swift:413-489): the pairs
+        [params.pair_start, + params.pair_count) of sorted_pairs through the experts of `binding`."""
+        if params.live_expert_count != len(binding.expert_ids):
+            raise PrefillGroupedRoutedMoEError("params were made for another binding")
+        ptrs = (C.c_void_p * len(binding.views))(*binding.pointers())
+        check(lib.nvmai_hip_prefill_grouped_moe_streamed(self.ctx.handle, _stream(), C.byref(params), ptrs, self.bits,
+                                                         _ptr(hidden), _ptr(sorted_pairs), sorted_pairs.shape[0],
+                                                         _ptr(act_scratch), _ptr(route_partials), _ptr(err)),
+              "prefill_grouped_moe_streamed")
+        return route_partials
+
+
+class PrefillGroupedRoutedMoEError(Exception):
+    """PrefillGroupedRoutedMoEError.invalidStreamedTileBinding (PrefillGroupedRoutedMoE.swift:325-337)."""
+
+
+class PrefillStreamedTileLifetimeError(Exception):
+    """PrefillStreamedTileLifetimeError (PrefillGroupedRoutedMoE.swift:49-64): .kind is 'duplicateSlots',
+    'slotReuseBeforeCompletion' or 'completeWithoutInFlightTile'."""
+
+    def __init__(self, kind, tile_index, conflicting_tile_index=None, slots=()):
+        super().__init__("prefill streamed tile %d: %s %s" % (tile_index, kind, list(slots)))
+        self.kind, self.tile_index = kind, tile_index
+        self.conflicting_tile_index, self.slots = conflicting_tile_index, list(slots)
+
+
+class PrefillStreamedTileSlotLifetime:
+    """PrefillStreamedTileSlotLifetime (PrefillGroupedRoutedMoE.swift:66-102): which cache slots the
+    tiles in flight hold, so that a slot is not refilled before the tile reading it has completed."""
+
+    def __init__(self):
+        self.in_flight = {}
+
+    def begin(self, tile_index, planned_slots):
+        slots = set()
+        for slot in planned_slots:
+            if slot in slots:
+                raise PrefillStreamedTileLifetimeError("duplicateSlots", tile_index, slots=sorted(planned_slots))
+            slots.add(slot)
+        for other, other_slots in self.in_flight.items():
+            overlap = slots & other_slots
+            if overlap:
+                raise PrefillStreamedTileLifetimeError("slotReuseBeforeCompletion", tile_index, other, sorted(overlap))
+        self.in_flight[tile_index] = slots
+
+    def complete(self, tile_index):
+        if self.in_flight.pop(tile_index, None) is None:
+            raise PrefillStreamedTileLifetimeError("completeWithoutInFlightTile", tile_index)
+
+
+class PrefillStreamedTileBinding:
+    """PrefillStreamedTileBinding (PrefillGroupedRoutedMoE.swift:185-323): the experts of one tile, at
+    most sixteen, each with the view (a device tensor, or (tensor, byte offset)) its blob was fetched
+    into; a global expert id maps to its index here, the kernel's local slot."""
+
+    def __init__(self, expert_ids, views):
+        expert_ids = [int(e) for e in expert_ids]
+        if not expert_ids:
+            raise PrefillGroupedRoutedMoEError("tile binding must include at least one expert")
+        if len(expert_ids) > 16:
+            raise PrefillGroupedRoutedMoEError("tile binding has %d experts; maximum is 16" % len(expert_ids))
+        if len(expert_ids) != len(views):
+            raise PrefillGroupedRoutedMoEError("expertIDs.count %d != views.count %d" % (len(expert_ids), len(views)))
+        seen = set()
+        for e in expert_ids:
+            if e < 0:
+                raise PrefillGroupedRoutedMoEError("expert id %d must be non-negative" % e)
+            if e in seen:
+                raise PrefillGroupedRoutedMoEError("duplicate expert id %d in tile binding" % e)
+            seen.add(e)
+        self.expert_ids, self.views = expert_ids, list(views)
+
+    def local_slot(self, expert):
+        return self.expert_ids.index(int(expert)) if int(expert) in self.expert_ids else None
+
+    def pointers(self):
+        out = []
+        for v in self.views:
+            t, off = v if isinstance(v, tuple) else (v, 0)
+            out.append(t.data_ptr() + int(off))
+        return out
+
+    @staticmethod
+    def expert_ids_for_tile(tile_index, groups, tiles):
+        """expertIDs(forTile:routes:): groups / tiles are the host copies of a grouping's records
+        (rows of (expert, pair_start, pair_count) and (group_start, group_count, pair_start, pair_count))."""
+        if not 0 <= tile_index < len(tiles):
+            raise PrefillGroupedRoutedMoEError("tile index %d is out of range" % tile_index)
+        group_start, group_count = int(tiles[tile_index][0]), int(tiles[tile_index][1])
+        if not 0 < group_count <= 16:
+            raise PrefillGroupedRoutedMoEError("tile has %d live experts; expected 1...16" % group_count)
+        if group_start < 0 or group_start + group_count > len(groups):
+            raise PrefillGroupedRoutedMoEError("tile group range %d..<%d exceeds %d"
+                                               % (group_start, group_start + group_count, len(groups)))
+        return [int(groups[g][0]) for g in range(group_start, group_start + group_count)]
+
+    def validate_covers_pairs(self, pair_experts, pair_start, pair_count):
+        """validateCoversPairs: pair_experts = the expert of every sorted pair (host sequence)."""
+        if pair_start < 0 or pair_count < 0 or pair_start + pair_count > len(pair_experts):
+            raise PrefillGroupedRoutedMoEError("pair range %d..<%d exceeds %d"
+                                               % (pair_start, pair_start + pair_count, len(pair_experts)))
+        for e in pair_experts[pair_start:pair_start + pair_count]:
+            if self.local_slot(e) is None:
+                raise PrefillGroupedRoutedMoEError("route expert %d is not bound in tile" % int(e))
+
+
+def prefill_streamed_params(pair_start, pair_count, d, routed_intermediate, top_k, hidden_stride_elements, binding,
+                            offsets):
+    """PrefillGroupedRoutedMoEStreamedParams.init (PrefillGroupedRoutedMoE.swift:139-183)."""
+    p = _lib.PrefillStreamedParams()
+    p.pair_start, p.pair_count, p.d, p.routed_intermediate = pair_start, pair_count, d, routed_intermediate
+    p.top_k, p.hidden_stride_elements, p.live_expert_count = top_k, hidden_stride_elements, len(binding.expert_ids)
+    for i in range(16):
+        p.local_expert[i] = binding.expert_ids[i] if i < len(binding.expert_ids) else 0xFFFFFFFF
+    p.gate_w_off, p.gate_s_off, p.gate_b_off = offsets.gate_w, offsets.gate_s, offsets.gate_b
+    p.up_w_off, p.up_s_off, p.up_b_off = offsets.up_w, offsets.up_s, offsets.up_b
+    p.down_w_off, p.down_s_off, p.down_b_off = offsets.down_w, offsets.down_s, offsets.down_b
+    return p
+
+
 class MPPPrefillInt4QMM:
     """MPPPrefillInt4QMM.encode (MPPPrefillInt4QMM.swift:63-128): y[m, n] = x[m, k] . W[n, k]^T on the
     matrix cores for one affine 4/8-bit matrix."""

@@ -370,3 +370,130 @@ def test_grouped_moe_on_a_failed_grouping_returns_zeros_and_the_error(nv, ctx_bf
     with pytest.raises(nv.PrefillMoEGroupingError) as e:
         routes.validate()
     assert e.value.name == "expertOutOfRange" and e.value.pair_index == 17 * k + 1
+
+
+# ------------------------------------------------------------------ streamed tiles (experts bound one by one)
+def _scattered_views(blobs, expert_ids, gap=4096, first=256):
+    """Each expert's blob copied to its own place inside one big device buffer, at a nonzero
+    16-byte-aligned offset (streamedViewsWithNonzeroOffsets)."""
+    stride = blobs.shape[1]
+    pitch = (stride + gap + 15) // 16 * 16
+    buf = torch.zeros(first + pitch * len(expert_ids), dtype=torch.uint8, device="cuda")
+    views = []
+    for i, e in enumerate(expert_ids):
+        off = first + i * pitch
+        buf[off:off + stride] = dev(blobs[e])
+        views.append((buf, off))
+    return buf, views
+
+
+def _route_partials_oracle(blobs, bits, x, d, f, idx, act):
+    """cpuSyntheticRoutePartials (PrefillGroupedRoutedMoETests.swift:293-378): per (token, rank) the
+    expert's FFN of the token's row, through the oracle's single-route call."""
+    tokens, k = idx.shape
+    one = O.f16_bits(np.ones((1, 1), np.float32))
+    out = np.zeros((tokens * k, d), np.float32)
+    for t in range(tokens):
+        for r in range(k):
+            out[t * k + r] = O.prefill_moe(blobs, bits, x[t:t + 1], d, f, idx[t:t + 1, r:r + 1], one)[0]
+    return out
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_streamed_tile_matches_reference_case(nv, ctx, bits):
+    # streamedBatchedMatchesReferenceAcrossPartialMicrobatch (PrefillGroupedRoutedMoETests+Execution.swift:8-110):
+    # d = f = 64, three rows, top-2 of 16 experts, every expert bound through a view at a nonzero offset
+    say("prefill streamed tile, reference case", ctx.act, bits)
+    d = f = 64
+    rows, k, E = 3, 2, 16
+    idx = np.array([[2, 0], [1, 2], [0, 1]], np.uint32)
+    w = O.f16_bits(np.ones((rows, k), np.float32))
+
+    def mat(expert, role, r, c):                     # makeSyntheticExpertPool's closed form
+        i, j = np.meshgrid(np.arange(r), np.arange(c), indexing="ij")
+        return ((expert + 1) * 1e-3 + (role + 1) * 3e-3 + ((i % 7) - 3) * 4e-4 + ((j % 11) - 5) * 2e-4).astype(np.float32)
+    blobs = np.stack([O.pack_expert(mat(e, 0, f, d), mat(e, 1, f, d), mat(e, 2, d, f), bits) for e in range(E)])
+    hidden = np.array([(i % 17) - 8 for i in range(rows * d)], np.float32).reshape(rows, d)
+    off, _ = nv.expert_offsets(d, f, bits)
+    routes = nv.PrefillMoEGrouping(ctx).group_routes(dev(idx.view(np.int32)), dev(w.view(np.int16)), E)
+    torch.cuda.synchronize()
+    routes.validate()
+    expert_ids = list(range(E))
+    buf, views = _scattered_views(blobs, expert_ids)
+    binding = nv.PrefillStreamedTileBinding(expert_ids, views)
+    n = rows * k
+    params = nv.prefill_streamed_params(0, n, d, f, k, d, binding, off)
+    partials = torch.full((n, d), -77.0, dtype=ctx.dtype, device="cuda")
+    act = torch.zeros((n, f), dtype=ctx.dtype, device="cuda")
+    err = torch.full((2,), 9, dtype=torch.int32, device="cuda")
+    nv.PrefillGroupedRoutedMoE(ctx, bits).encode_streamed_batched(act_tensor(hidden, ctx), routes.sorted_pairs, partials,
+                                                                 act, binding, params, err=err)
+    torch.cuda.synchronize()
+    assert err.tolist() == [0, 0]
+    want = _route_partials_oracle(blobs, bits, hidden, d, f, idx, ctx.act)
+    assert O.rel_error(act_np(partials), want) <= TOL_ACT
+    assert all(o > 0 for _, o in views)
+    binding.validate_covers_pairs(u32(routes.sorted_pairs).reshape(-1, 4)[:, 1].tolist(), 0, n)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_streamed_tiles_equal_the_resident_pool_call(nv, ctx_bf16, bits):
+    # tile after tile (at most 16 experts each, bound from scattered copies, only the tile's pair
+    # range computed) gives the bits of the one call over the resident pool; a tile that leaves an
+    # expert of its range unbound computes nothing and reports the first such pair
+    say("prefill streamed tiles vs pool", bits)
+    ctx = ctx_bf16
+    rng = np.random.default_rng(31 + bits)
+    d, f, E, k, tokens = 256, 128, 40, 4, 700
+    mats = [(gauss(rng, (f, d), 0.05), gauss(rng, (f, d), 0.05), gauss(rng, (d, f), 0.05)) for _ in range(E)]
+    blobs = np.stack([O.pack_expert(*m, bits) for m in mats])
+    x = O.round_bf16(gauss(rng, (tokens, d)))
+    idx, w = _zipf_routes(rng, tokens, E, k)
+    off, stride = nv.expert_offsets(d, f, bits)
+    routes = nv.PrefillMoEGrouping(ctx).group_routes(dev(idx.view(np.int32)), dev(w.view(np.int16)), E)
+    moe = nv.PrefillGroupedRoutedMoE(ctx, bits)
+    xd = act_tensor(x, ctx)
+    want, want_act = moe.encode(dev(blobs), off, xd, d, f, routes)
+    torch.cuda.synchronize()
+    info = routes.validate()
+    groups = u32(routes.groups).reshape(-1, 3)[:info[0]].tolist()
+    tiles = u32(routes.tiles).reshape(-1, 4)[:info[1]].tolist()
+    assert len(tiles) == 3                                     # 40 experts in tiles of 16
+    n = tokens * k
+    got = torch.zeros((n, d), dtype=ctx.dtype, device="cuda")
+    act = torch.zeros((n, f), dtype=ctx.dtype, device="cuda")
+    err = torch.zeros(2, dtype=torch.int32, device="cuda")
+    lifetime = nv.PrefillStreamedTileSlotLifetime()
+    keep = []
+    for t, tile in enumerate(tiles):
+        ids = nv.PrefillStreamedTileBinding.expert_ids_for_tile(t, groups, tiles)
+        lifetime.begin(t, list(range(len(ids))))
+        buf, views = _scattered_views(blobs, ids, gap=16 * (t + 1))
+        keep.append(buf)
+        binding = nv.PrefillStreamedTileBinding(ids, views)
+        params = nv.prefill_streamed_params(tile[2], tile[3], d, f, k, xd.stride(0), binding, off)
+        moe.encode_streamed_batched(xd, routes.sorted_pairs, got, act, binding, params, err=err)
+        torch.cuda.synchronize()
+        assert err.tolist() == [0, 0]
+        lifetime.complete(t)
+    assert torch.equal(got, want) and torch.equal(act, want_act)
+    # the second tile with its last expert left out
+    ids = nv.PrefillStreamedTileBinding.expert_ids_for_tile(1, groups, tiles)
+    buf, views = _scattered_views(blobs, ids[:-1])
+    binding = nv.PrefillStreamedTileBinding(ids[:-1], views)
+    params = nv.prefill_streamed_params(tiles[1][2], tiles[1][3], d, f, k, xd.stride(0), binding, off)
+    before = got.clone()
+    moe.encode_streamed_batched(xd, routes.sorted_pairs, got, act, binding, params, err=err)
+    torch.cuda.synchronize()
+    first_unbound = groups[tiles[1][0] + tiles[1][1] - 1][1]
+    assert err.tolist() == [1, first_unbound] and torch.equal(got, before)
+    with pytest.raises(nv.PrefillGroupedRoutedMoEError):
+        binding.validate_covers_pairs(u32(routes.sorted_pairs).reshape(-1, 4)[:, 1].tolist(), tiles[1][2], tiles[1][3])
+    # argument checks of the entry point: a pair range past the end, a misaligned blob
+    bad = nv.prefill_streamed_params(n - 4, 8, d, f, k, xd.stride(0), binding, off)
+    with pytest.raises(nv.NvmaiError):
+        moe.encode_streamed_batched(xd, routes.sorted_pairs, got, act, binding, bad)
+    crooked = nv.PrefillStreamedTileBinding(ids[:1], [(buf, 257)])
+    with pytest.raises(nv.NvmaiError):
+        moe.encode_streamed_batched(xd, routes.sorted_pairs, got, act, crooked,
+                                    nv.prefill_streamed_params(0, 4, d, f, k, xd.stride(0), crooked, off))
