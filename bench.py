@@ -806,8 +806,9 @@ def decode_line(a, r, bits, batch, steps, warmup):
 def extra_cells(nv, ctx, torch, a, layers8, stride8):
     """The other cells of the metric, each measured like its own --workload line but shorter:
     4-bit decode at batch 32, 8-bit decode at one token, the configs[2] prefill grouped GEMM, and
-    configs[4] (the full 40-layer decode step, tok/s at batch 1 and 16), and configs[3] attention at
-    128K x 8 and 32K x 1 with 8- and 4-bit KV (each checked against the oracle before it is reported)."""
+    configs[4] (the full 40-layer decode step, tok/s at batch 1 and 16), and every cell of configs[3]
+    (attention at 4K / 32K / 128K context x batch 1 / 8 with 8- and 4-bit KV, each checked against the
+    oracle before it is reported)."""
     import argparse
     out = {}
     r = run_config(nv, ctx, torch, layers8, stride8, 8, 1, 200, 20, profile=True)
@@ -837,7 +838,7 @@ def extra_cells(nv, ctx, torch, a, layers8, stride8):
         out["prefill_attention_%dbit_4096tokens" % bits] = compact(run_prefill_attention(nv, ctx, torch, sub))
         torch.cuda.empty_cache()
     for bits in (8, 4):
-        for context, batch in ((131072, 8), (32768, 1)):
+        for context, batch in ((131072, 8), (131072, 1), (32768, 8), (32768, 1), (4096, 8), (4096, 1)):
             sub = argparse.Namespace(**vars(a))
             sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.context, sub.batch = True, 30, 5, bits, context, batch
             out["attention_%dbit_%dk_batch%d" % (bits, context // 1024, batch)] = compact(run_attention(nv, ctx, torch, sub))
