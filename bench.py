@@ -36,17 +36,19 @@ def parse():
     ap.add_argument("--sweep", action="store_true", help="also print batch/bits sweep lines to stderr")
     ap.add_argument("--no-extra", action="store_true", help="skip the `extra` object (the other cells of the metric) "
                     "that the default invocation appends")
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "prefill_attention", "sampler", "greedy", "step", "copy"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "prefill_attention", "sampler", "greedy", "step", "prefill_step", "copy"],
                     help="decode = configs[1] (the headline line); prefill = configs[2] grouped GEMM; "
                          "attention = configs[3] quantized-KV decode attention; prefill_attention = causal attention of --tokens queries "
                          "at the end of a --context cache; sampler = the end of configs[4]: "
                          "quantized LM head GEMV over 248,320 rows, tiled softmax, top-k sampler; greedy = the fused greedy LM head "
                          "(RMSNorm + logits in a fixed order + argmax) over the same head; step = configs[4], the full 40-layer decode "
-                         "step (tok/s at --batch 1..16, KV at --context); copy = a plain 1 GiB device copy, "
+                         "step (tok/s at --batch 1..16, KV at --context); prefill_step = --tokens prompt tokens of one sequence through the "
+                         "same 40 layers with the prefill kernels, in chunks of --chunk; copy = a plain 1 GiB device copy, "
                          "the known-size kernel the FETCH_SIZE / WRITE_SIZE counters are calibrated on")
     ap.add_argument("--context", type=int, default=None, help="attention: tokens in the KV cache (default 32768; "
                     "prefill_attention: the chunk itself)")
     ap.add_argument("--tokens", type=int, default=4096, help="prefill: tokens per step")
+    ap.add_argument("--chunk", type=int, default=4096, help="prefill_step: tokens per chunk")
     a = ap.parse_args()
     if a.bits is None:
         a.bits = 4 if a.workload == "prefill" else 8
@@ -701,6 +703,60 @@ def run_step(nv, ctx, torch, a):
     }
 
 
+def run_prefill_step(nv, ctx, torch, a):
+    """The prompt side of configs[4]: `--tokens` tokens of one sequence through all 40 layers of the same
+    hybrid model with the prefill kernels (HybridDecoder.prefill_chunked, chunks of `--chunk` tokens): dense
+    matrix-core projections, gated-DeltaNet over the rows of a chunk, causal attention over the 8-bit
+    cache, tiled router + permutation + grouped GEMM + reduce, shared expert.  Prompt tokens per second;
+    the flops counted are the matrix products of the model (2 flop per weight and token)."""
+    from nvmai_amd.decoder import HybridConfig, HybridDecoder, HybridWeights
+    cfg = HybridConfig(layers=40, expert_bits=4, attn_bits=4, kv_bits=8, head_bits=16, gdn_state_bf16=True)
+    w = HybridWeights(ctx, cfg, seed=2024)
+    T, chunk = a.tokens, a.chunk
+    dec = HybridDecoder(ctx, cfg, w, batch=1, max_context=T)
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    tokens = torch.randint(0, cfg.vocab, (T,), generator=gen, device="cuda", dtype=torch.int32)
+
+    def once():
+        for L in dec.gdn_states:
+            for buf in dec.gdn_states[L]:
+                buf.zero_()
+        return dec.prefill_chunked(tokens, 0, 0, chunk)
+    ctx.profile_enable(False)
+    for _ in range(max(1, a.warmup)):
+        last = once()
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(last.float()).all())
+    steps = max(1, a.steps)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        once()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    D, F, K = cfg.hidden, cfg.moe_intermediate, cfg.top_k
+    kh, vh, dk, dv, taps = cfg.gdn
+    n_lin = sum(cfg.is_linear(L) for L in range(cfg.layers))
+    n_full = cfg.layers - n_lin
+    lin_w = (cfg.gdn_qkv_dim + cfg.gdn_value_dim + 2 * vh) * D + D * cfg.gdn_value_dim
+    full_w = (2 * cfg.q_dim + 2 * cfg.kv_dim) * D + D * cfg.q_dim
+    moe_w = (K + 1) * 3 * D * F + cfg.num_experts * D
+    attn_flops = n_full * 4.0 * cfg.num_heads * cfg.head_dim * (T * (T + 1) / 2)
+    flops = 2.0 * T * (n_lin * lin_w + n_full * full_w + cfg.layers * moe_w) + attn_flops
+    tf = flops / dt / 1e12
+    return {
+        "metric": METRIC, "value": round(T / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": a.warmup,
+        "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u4 codes dequantized to bf16 MFMA operands, f32 accumulate; bf16 recurrent state; u8 KV", "data": "synthetic",
+        "config": {"workload": "prompt side of configs[4]: %d tokens of one sequence through the 40-layer hybrid MoE model "
+                               "in chunks of %d (prefill kernels; launched eagerly through the C ABI)" % (T, chunk),
+                   "tokens": T, "chunk": chunk, "model_gflop_per_token": round(flops / T / 1e9, 2)},
+        "roofline": {"kernel": "whole prompt (all kernels)", "bound": "mfma", "achieved": round(tf, 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "traffic_source": None,
+                     "flops_per_launch": flops, "avg_launch_us": round(dt * 1e6, 1)},
+        "cpu_baseline": None,
+    }
+
+
 def run_copy(torch, a):
     """A plain copy kernel of known size: 1 GiB read + 1 GiB written per launch."""
     n = 1 << 30
@@ -738,7 +794,8 @@ def main():
                 run_prefill_attention(nv, ctx, torch, a) if a.workload == "prefill_attention" else
                 run_sampler(nv, ctx, torch, a) if a.workload == "sampler" else
                 run_greedy(nv, ctx, torch, a) if a.workload == "greedy" else
-                run_step(nv, ctx, torch, a) if a.workload == "step" else run_copy(torch, a))
+                run_step(nv, ctx, torch, a) if a.workload == "step" else
+                run_prefill_step(nv, ctx, torch, a) if a.workload == "prefill_step" else run_copy(torch, a))
         print(json.dumps(line), flush=True)
         return
     layers, stride = build_layers(nv, ctx, torch, a.bits, a.layers)

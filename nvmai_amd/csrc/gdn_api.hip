@@ -21,9 +21,21 @@ GdnShape shape_of(const nvmai_gdn_config* c, uint32_t rows, uint32_t batch) {
     return GdnShape{c->num_k_heads, c->num_v_heads, c->key_head_dim, c->value_head_dim, c->conv_kernel_size, rows, batch};
 }
 
+// From this many rows per sequence on a call takes the kernels that keep only the recurrence
+// sequential (two or three launches instead of one or two, so not for a handful of rows).
+constexpr uint32_t GDN_ROWS_PARALLEL_FROM = 8;
+
 template <int ACT, int DK, int DV>
 void launch_delta(const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
     const dim3 grid(p.sh.v_heads, p.sh.batch);
+    if (p.sh.rows >= GDN_ROWS_PARALLEL_FROM && (p.sh.rows + 1) / 2 <= 65535 && aligned16(p.conv_out) && p.conv_stride % 8 == 0) {
+        const dim3 rgrid(p.sh.v_heads, p.sh.batch, DV / 16);      // one group of sixteen state rows per block
+        if (state_bf16) gdn_delta_rows_kernel<ACT, DK, DV, true, 1><<<rgrid, 256, 0, s>>>(p);
+        else gdn_delta_rows_kernel<ACT, DK, DV, false, 1><<<rgrid, 256, 0, s>>>(p);
+        const dim3 ngrid(p.sh.v_heads, p.sh.batch, (p.sh.rows + 1) / 2);
+        gdn_gated_norm_rows_kernel<ACT><<<ngrid, 256, 0, s>>>(p.out, p.out_stride, p.z, p.z_stride, p.norm_w, p.sh);
+        return;
+    }
     if (state_bf16) gdn_delta_gated_kernel<ACT, DK, DV, true><<<grid, 256, 0, s>>>(p);
     else gdn_delta_gated_kernel<ACT, DK, DV, false><<<grid, 256, 0, s>>>(p);
 }
@@ -53,6 +65,20 @@ extern "C" int nvmai_hip_gdn_conv_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, 
     const GdnShape sh = shape_of(config, rows, batch);
     const dim3 grid(2 * sh.k_heads + sh.v_heads, batch);
     hipStream_t s = (hipStream_t)stream;
+    if (rows >= GDN_ROWS_PARALLEL_FROM && sh.dk <= 128 && sh.dv <= 128 && (rows + 1) / 2 <= 65535) {
+        // a chunk of rows: every (row, head segment) on a pair of waves, then the tail in a launch of its own
+        const dim3 rgrid(2 * sh.k_heads + sh.v_heads, batch, (rows + 1) / 2);
+        if (ctx->act == ACT_BF16)
+            gdn_conv_norm_rows_kernel<ACT_BF16><<<rgrid, 256, 0, s>>>((const uint16_t*)qkv_raw, qkv_stride, (const uint16_t*)tail,
+                                                                     conv_weight, (uint16_t*)conv_out, conv_out_stride, sh);
+        else
+            gdn_conv_norm_rows_kernel<ACT_FP16><<<rgrid, 256, 0, s>>>((const uint16_t*)qkv_raw, qkv_stride, (const uint16_t*)tail,
+                                                                     conv_weight, (uint16_t*)conv_out, conv_out_stride, sh);
+        if (sh.taps > 1)
+            gdn_tail_update_kernel<<<dim3((C + 255) / 256, batch), 256, 0, s>>>((const uint16_t*)qkv_raw, qkv_stride,
+                                                                               (uint16_t*)tail, sh);
+        return launch_status();
+    }
     if (ctx->act == ACT_BF16)
         gdn_conv_norm_kernel<ACT_BF16><<<grid, 256, 0, s>>>((const uint16_t*)qkv_raw, qkv_stride, (uint16_t*)tail, conv_weight,
                                                             (uint16_t*)conv_out, conv_out_stride, sh);

@@ -195,6 +195,223 @@ __global__ __launch_bounds__(256) void gdn_delta_gated_kernel(GdnDeltaParams p) 
 }
 
 
+// ---- a chunk of rows: the parts that do not recur, spread over the device ---------------------------
+// The conv of row t reads the raw rows t - K + 1 .. t only, and the gated output norm of row t reads
+// y[t] only: with many rows per call (a prefill chunk) both run with a pair of waves per (row,
+// head segment) instead of inside the sequential loops above, which leaves the recurrence itself --
+// S and the rows it produces -- as the only sequential part.  Channel i of a segment sits on lane
+// i % 64 of the pair's wave i / 64 and the two wave sums are added first, as in the kernels above:
+// the same bits.  Segments of at most 128 channels.
+
+// conv + SiLU + q / k norm of rows [0, rows) of every sequence; the tail is read, not written.
+template <int ACT>
+__global__ __launch_bounds__(256) void gdn_conv_norm_rows_kernel(const uint16_t* qkv_raw, uint32_t qkv_stride,
+                                                                const uint16_t* tail, const uint16_t* conv_w,
+                                                                uint16_t* conv_out, uint32_t out_stride, GdnShape sh) {
+    __shared__ float part[4];
+    const uint32_t seg = blockIdx.x, b = blockIdx.y;
+    const uint32_t pair = threadIdx.x >> 7, i = threadIdx.x & 127u;         // row of the block, channel of the segment
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t t = blockIdx.z * 2u + pair;
+    const uint32_t C = 2 * sh.k_heads * sh.dk + sh.v_heads * sh.dv;
+    const bool is_qk = seg < 2 * sh.k_heads;
+    const uint32_t seg_len = is_qk ? sh.dk : sh.dv;
+    const uint32_t base = is_qk ? seg * sh.dk : 2 * sh.k_heads * sh.dk + (seg - 2 * sh.k_heads) * sh.dv;
+    const uint32_t hist = sh.taps - 1;
+    const uint16_t* tl = tail + (size_t)b * hist * C;
+    const uint16_t* raw = qkv_raw + (size_t)b * sh.rows * qkv_stride;
+    const bool live = t < sh.rows && i < seg_len;
+    const uint32_t ch = base + i;
+    float x = 0.0f;
+    uint16_t r = 0;
+    if (live) {
+        float acc = 0.0f;
+        for (uint32_t j = 0; j < sh.taps; ++j) {
+            const int src = (int)t + (int)j - (int)hist;
+            const uint16_t v = src >= 0 ? raw[(size_t)src * qkv_stride + ch] : tl[(size_t)((int)hist + src) * C + ch];
+            acc = fmaf(act_to_f32<ACT>(v), bf16_to_f32(conv_w[ch * sh.taps + j]), acc);
+        }
+        r = f32_to_act<ACT>(gdn_silu(acc));
+        x = act_to_f32<ACT>(r);
+    }
+    uint16_t* o = conv_out + ((size_t)b * sh.rows + t) * out_stride + ch;
+    if (!is_qk) {                                             // block-uniform
+        if (live) *o = r;
+        return;
+    }
+    const float ws = wave_sum_bcast(x * x);
+    if (lane == 0) part[wave] = ws;
+    __syncthreads();
+    if (live) {
+        const float total = (part[2 * pair] + part[2 * pair + 1]) + (0.0f + 0.0f);
+        const float inv = rsqrtf(total / (float)sh.dk + GDN_RMS_EPS);
+        const float scale = seg < sh.k_heads ? 1.0f / (float)sh.dk : rsqrtf((float)sh.dk);
+        *o = f32_to_act<ACT>(x * inv * scale);
+    }
+}
+
+// The new tail of every sequence: the last K - 1 raw rows of [old tail | rows].  One thread per channel
+// reads its column before it writes it, so the update is in place.
+__global__ __launch_bounds__(256) void gdn_tail_update_kernel(const uint16_t* qkv_raw, uint32_t qkv_stride, uint16_t* tail,
+                                                             GdnShape sh) {
+    const uint32_t C = 2 * sh.k_heads * sh.dk + sh.v_heads * sh.dv;
+    const uint32_t ch = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+    if (ch >= C) return;
+    const uint32_t hist = sh.taps - 1;
+    uint16_t* tl = tail + (size_t)b * hist * C;
+    const uint16_t* raw = qkv_raw + (size_t)b * sh.rows * qkv_stride;
+    uint16_t keep[GDN_MAX_TAPS];
+#pragma unroll
+    for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+        if (j >= hist) break;
+        const int src = (int)sh.rows + (int)j - (int)hist;
+        keep[j] = src >= 0 ? raw[(size_t)src * qkv_stride + ch] : tl[(size_t)((int)hist + src) * C + ch];
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+        if (j >= hist) break;
+        tl[(size_t)j * C + ch] = keep[j];
+    }
+}
+
+// out[row, head] = rmsnorm(y) * weight * silu(z) in place over the 16-bit y rows the recurrence left in out.
+template <int ACT>
+__global__ __launch_bounds__(256) void gdn_gated_norm_rows_kernel(uint16_t* out, uint32_t out_stride, const uint16_t* z,
+                                                                 uint32_t z_stride, const uint16_t* norm_w, GdnShape sh) {
+    __shared__ float part[4];
+    const uint32_t h = blockIdx.x, b = blockIdx.y;
+    const uint32_t pair = threadIdx.x >> 7, i = threadIdx.x & 127u;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t t = blockIdx.z * 2u + pair;
+    const bool live = t < sh.rows && i < sh.dv;
+    const size_t row = (size_t)b * sh.rows + t;
+    float y = 0.0f;
+    if (live) y = act_to_f32<ACT>(out[row * out_stride + h * sh.dv + i]);
+    const float ws = wave_sum_bcast(fmaf(y, y, 0.0f));
+    if (lane == 0) part[wave] = ws;
+    __syncthreads();
+    if (!live) return;
+    const float total = (part[2 * pair] + part[2 * pair + 1]) + (0.0f + 0.0f);
+    const float inv = rsqrtf(total / (float)sh.dv + GDN_RMS_EPS);
+    const float normed = y * inv * bf16_to_f32(norm_w[i]);
+    const float gate = gdn_silu(act_to_f32<ACT>(z[row * z_stride + h * sh.dv + i]));
+    out[row * out_stride + h * sh.dv + i] = f32_to_act<ACT>(normed * gate);
+}
+
+// The recurrence alone over the rows of a call: S, and y[t] = S q rounded to 16 bits into out (the
+// kernel above norms it).  A row costs a few hundred cycles of arithmetic and a trip to memory costs
+// several times that, so the rows arrive a tile of 32 at a time: all 256 threads fetch the next
+// tile's q, k and v rows of this head (16 bytes per load, six loads per thread at 128 x 128) into
+// registers while the current tile is worked on from LDS, the threads of the first rows compute the
+// tile's decays and betas, and one barrier per tile hands both over.  Inside a tile nothing waits
+// for the block.  The rows of S do not depend on one another (kv, delta and y of row dv read S[dv, :]
+// only), so a head's DV rows are shared out over DV / (16 GPB) blocks, each with GPB groups of sixteen
+// rows: eight times as many blocks as heads at GPB = 1, and an eighth of the arithmetic per row and
+// thread.  conv_out rows 16-byte aligned, DK and DV multiples of 8.
+template <int ACT, int DK, int DV, bool STATE_BF16, int GPB>
+__global__ __launch_bounds__(256) void gdn_delta_rows_kernel(GdnDeltaParams p) {
+    constexpr int EPL = DK / 16;
+    constexpr int GROUPS = DV / 16;
+    constexpr uint32_t TR = 32;                             // rows per tile
+    constexpr uint32_t ROW_E = 2 * DK + DV;                 // elements of a staged row: q | k | v
+    constexpr uint32_t CPR = ROW_E / 8;                     // 16-byte chunks per row
+    constexpr uint32_t NLD = (TR * CPR + 255) / 256;        // chunks per thread and tile
+    static_assert(DK % 16 == 0 && DV % 16 == 0 && EPL >= 1 && EPL <= 16 && ROW_E % 8 == 0 && GROUPS % GPB == 0, "shape");
+    const uint32_t g0 = blockIdx.z * GPB;                   // first of this block's groups of sixteen state rows
+    __shared__ __attribute__((aligned(16))) uint16_t rows_s[2][TR][ROW_E];
+    __shared__ float decay_s[2][TR], beta_s[2][TR];
+    const uint32_t h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const uint32_t sub = tid & 15u, row_in_pass = tid >> 4;
+    const GdnShape& sh = p.sh;
+    const uint32_t hk = h / (sh.v_heads / sh.k_heads);
+    const float exp_a = expf(bf16_to_f32(p.a_log[h]));
+    const float dtb = bf16_to_f32(p.dt_bias[h]);
+    const size_t state_base = (((size_t)b * sh.v_heads + h) * DV) * DK;
+    float s[GPB][EPL];
+#pragma unroll
+    for (int g = 0; g < GPB; ++g) {
+        const size_t at = state_base + (size_t)((g0 + g) * 16 + row_in_pass) * DK + sub * EPL;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e)
+            s[g][e] = STATE_BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(p.state)[at + e])
+                                 : reinterpret_cast<const float*>(p.state)[at + e];
+    }
+    // this thread's chunks of a tile: chunk c of the tile is row c / CPR, elements 8 (c % CPR) ..
+    uint4 stage[NLD];
+    uint16_t a_raw = 0, b_raw = 0;
+    auto fetch_tile = [&](uint32_t t0) {
+#pragma unroll
+        for (uint32_t j = 0; j < NLD; ++j) {
+            const uint32_t c = tid + 256 * j, r = c / CPR, e = (c % CPR) * 8;
+            stage[j] = uint4{0u, 0u, 0u, 0u};
+            if (c < TR * CPR && t0 + r < sh.rows) {
+                const size_t row = (size_t)b * sh.rows + t0 + r;
+                const uint16_t* base = p.conv_out + row * p.conv_stride;
+                const uint16_t* src = e < (uint32_t)DK ? base + hk * DK + e
+                                    : e < 2u * DK ? base + (sh.k_heads + hk) * DK + (e - DK)
+                                                  : base + 2 * sh.k_heads * DK + h * DV + (e - 2 * DK);
+                stage[j] = *reinterpret_cast<const uint4*>(src);
+            }
+        }
+        if (tid < TR && t0 + tid < sh.rows) {
+            const size_t row = (size_t)b * sh.rows + t0 + tid;
+            a_raw = p.a_proj[row * p.ab_stride + h];
+            b_raw = p.b_proj[row * p.ab_stride + h];
+        }
+    };
+    auto store_tile = [&](uint32_t buf) {
+#pragma unroll
+        for (uint32_t j = 0; j < NLD; ++j) {
+            const uint32_t c = tid + 256 * j;
+            if (c < TR * CPR) *reinterpret_cast<uint4*>(&rows_s[buf][c / CPR][(c % CPR) * 8]) = stage[j];
+        }
+        if (tid < TR) {
+            decay_s[buf][tid] = expf(-exp_a * gdn_softplus(act_to_f32<ACT>(a_raw) + dtb));
+            beta_s[buf][tid] = 1.0f / (1.0f + expf(-act_to_f32<ACT>(b_raw)));
+        }
+    };
+    fetch_tile(0);
+    store_tile(0);
+    __syncthreads();
+    for (uint32_t t0 = 0, buf = 0; t0 < sh.rows; t0 += TR, buf ^= 1u) {
+        const uint32_t n = min(TR, sh.rows - t0);
+        if (t0 + TR < sh.rows) fetch_tile(t0 + TR);
+        for (uint32_t u = 0; u < n; ++u) {
+            const uint16_t* rs = rows_s[buf][u];
+            float q[EPL], k[EPL];
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) { q[e] = act_to_f32<ACT>(rs[sub * EPL + e]); k[e] = act_to_f32<ACT>(rs[DK + sub * EPL + e]); }
+            const float g_decay = decay_s[buf][u], beta = beta_s[buf][u];
+            uint16_t* yrow = p.out + ((size_t)b * sh.rows + t0 + u) * p.out_stride + h * DV;
+#pragma unroll
+            for (int g = 0; g < GPB; ++g) {
+                const uint32_t dv = (g0 + g) * 16 + row_in_pass;
+                float kv = 0.0f;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) { s[g][e] *= g_decay; kv = fmaf(s[g][e], k[e], kv); }
+                kv = seg_reduce_sum<16>(kv);
+                const float delta = (act_to_f32<ACT>(rs[2 * DK + dv]) - kv) * beta;
+                float o = 0.0f;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) { s[g][e] = fmaf(k[e], delta, s[g][e]); o = fmaf(s[g][e], q[e], o); }
+                o = seg_reduce_sum<16>(o);
+                if (sub == 0) yrow[dv] = f32_to_act<ACT>(o);
+            }
+        }
+        if (t0 + TR < sh.rows) store_tile(buf ^ 1u);        // the other buffer: nobody reads it during this tile
+        __syncthreads();
+    }
+#pragma unroll
+    for (int g = 0; g < GPB; ++g) {
+        const size_t at = state_base + (size_t)((g0 + g) * 16 + row_in_pass) * DK + sub * EPL;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            if (STATE_BF16) reinterpret_cast<uint16_t*>(p.state)[at + e] = f32_to_bf16(s[g][e]);
+            else reinterpret_cast<float*>(p.state)[at + e] = s[g][e];
+        }
+    }
+}
+
 // ---- one decode token: both kernels above in one launch --------------------------------------------
 // Block (key head, sequence) of 256 R threads, R = Hv / Hk value heads per key head: the first 256
 // threads run the conv + SiLU + norm of the key head's q and k channels (q on waves 0 - 1, k on

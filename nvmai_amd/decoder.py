@@ -141,7 +141,7 @@ class HybridDecoder:
     once; step() only enqueues kernels."""
 
     def __init__(self, ctx, cfg, weights, batch=1, max_context=32768):
-        self.ctx, self.cfg, self.w, self.batch = ctx, cfg, weights, batch
+        self.ctx, self.cfg, self.w, self.batch, self.max_context = ctx, cfg, weights, batch, max_context
         dev, dt = ctx.device, ctx.dtype
         D = cfg.hidden
         buf = lambda *shape: torch.zeros(shape, dtype=dt, device=dev)
@@ -269,6 +269,112 @@ class HybridDecoder:
             nxt = self.w.layers[L + 1]["in_norm"] if L + 1 < cfg.layers else self.w.final_norm
             ops.residual_add_rmsnorm(ctx, self.hidden, self.moe_out, nxt, out=self.normed, eps=cfg.rms_eps)
         return self.normed
+
+    # -- prefill: the tokens of ONE sequence, a chunk at a time, through every layer ------------------------
+    # RealForwardRunner.prefillChunked / executePrefillChunk (RealForwardRunner.swift:1323-1388, 1503-1733):
+    # per chunk encodeLinearAttentionPrefill (:2605-2742) or encodeFullAttentionPrefill (:2744-2913), then
+    # encodeRoutedMoEPrefill (:3244+).  The kernels are the prefill ones -- the dense matrix-core product
+    # for the projections, the recurrent kernels over the rows of the chunk, causal attention over the
+    # quantized cache, the tiled router, the permutation by expert and the grouped GEMM, the shared expert
+    # in dense mode -- and they leave the sequence's KV rows, conv tails and recurrent states exactly
+    # where step() expects them, so decoding continues at start_position + len(tokens).
+    def prefill_chunked(self, tokens, sequence=0, start_position=0, chunk_tokens=2048):
+        """tokens: int32 device tensor [n] of sequence `sequence`, the first of them at start_position.
+        Returns the final-normed row of the last token, [1, hidden] (the input of head())."""
+        n = tokens.numel()
+        if n == 0:
+            raise ValueError("prefill_chunked needs at least one token")
+        if start_position + n > self.max_context:
+            raise ValueError("prefill of %d tokens from %d exceeds the cache (%d rows)" % (n, start_position, self.max_context))
+        last = None
+        for c0 in range(0, n, chunk_tokens):
+            last = self._execute_prefill_chunk(tokens[c0:min(n, c0 + chunk_tokens)].contiguous(), sequence,
+                                               start_position + c0)
+        return last
+
+    def _execute_prefill_chunk(self, tokens, b, start):
+        cfg, ctx = self.cfg, self.ctx
+        T = tokens.numel()
+        e_p, e_s, e_b = self.w.embed
+        hidden = torch.empty((T, cfg.hidden), dtype=ctx.dtype, device=ctx.device)
+        check(lib.nvmai_hip_embed_lookup(ctx.handle, ops._stream(), ops._ptr(e_p), ops._ptr(e_s), ops._ptr(e_b),
+                                         cfg.embed_bits, ops._ptr(tokens), 0, T, ops._ptr(hidden), cfg.hidden, cfg.hidden,
+                                         cfg.vocab, 1.0), "embed_lookup")
+        norm = ops.RMSNorm(ctx)
+        normed = norm.encode_bf16w(hidden, self.w.layers[0]["in_norm"], eps=cfg.rms_eps)
+        positions = torch.arange(start, start + T, dtype=torch.int32, device=ctx.device)
+        for L, w in enumerate(self.w.layers):
+            if cfg.is_linear(L):
+                branch = self._linear_attention_prefill(L, w, normed, b, T)
+            else:
+                branch = self._full_attention_prefill(L, w, normed, b, start, positions, T)
+            routed_x = ops.residual_add_rmsnorm(ctx, hidden, branch, w["post_norm"], eps=cfg.rms_eps)
+            y = self._routed_moe_prefill(w, routed_x, T)
+            nxt = self.w.layers[L + 1]["in_norm"] if L + 1 < cfg.layers else self.w.final_norm
+            normed = ops.residual_add_rmsnorm(ctx, hidden, y, nxt, eps=cfg.rms_eps)
+        return normed[T - 1:T]
+
+    def _linear_attention_prefill(self, L, w, normed, b, T):
+        cfg = self.cfg
+        vh = cfg.gdn[1]
+        p_, s_, b_ = w["in_proj"]
+        proj = ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, normed, self.lin_rows, cfg.hidden)
+        C_, V = cfg.gdn_qkv_dim, cfg.gdn_value_dim
+        qkv, z, a, bb = proj[:, :C_], proj[:, C_:C_ + V], proj[:, C_ + V:C_ + V + vh], proj[:, C_ + V + vh:]
+        tail, state = self.gdn_states[L]
+        conv = self.gdn.encode_conv_norm(qkv, tail[b:b + 1], w["conv_w"], rows=T)
+        out = self.gdn.encode_delta_gated_norm(conv, a, bb, w["a_log"], w["dt_bias"], state[b:b + 1], z, w["gdn_norm"], rows=T)
+        p_, s_, b_ = w["out_proj"]
+        return ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, out, cfg.hidden, cfg.gdn_value_dim)
+
+    def _full_attention_prefill(self, L, w, normed, b, start, positions, T):
+        cfg, ctx = self.cfg, self.ctx
+        p_, s_, b_ = w["qkv"]
+        proj = ops.affine_gemv(ctx, p_, s_, b_, cfg.attn_bits, normed, self.full_rows, cfg.hidden)
+        q = torch.empty((T, cfg.num_heads, cfg.head_dim), dtype=ctx.dtype, device=ctx.device)
+        gate, out = torch.empty_like(q), torch.empty_like(q)
+        kc, vc = self.kv[L]
+        if cfg.head_dim % 64 == 0 and cfg.kv_bits in (4, 8):
+            # the chunk's K / V rows go into the cache rows start .. start + T - 1 of this sequence
+            kview, vview = kc.view(b, start), vc.view(b, start)
+            check(lib.nvmai_hip_attn_qkv_epilogue_kv(ctx.handle, ops._stream(), ops._ptr(proj), proj.stride(0), 1,
+                                                     ops._ptr(w["q_norm"]), ops._ptr(w["k_norm"]), ops._ptr(q), ops._ptr(gate),
+                                                     None, None, cfg.kv_dim, C.byref(kview), C.byref(vview), T, cfg.num_heads,
+                                                     cfg.num_kv_heads, cfg.head_dim, cfg.rotary_dim, 0, ops._ptr(positions), 0,
+                                                     cfg.rope_theta, cfg.rms_eps), "attn_qkv_epilogue_kv")
+        else:
+            k = torch.empty((T, cfg.kv_dim), dtype=ctx.dtype, device=ctx.device)
+            v = torch.empty_like(k)
+            check(lib.nvmai_hip_attn_qkv_epilogue(ctx.handle, ops._stream(), ops._ptr(proj), proj.stride(0), 1,
+                                                  ops._ptr(w["q_norm"]), ops._ptr(w["k_norm"]), ops._ptr(q), ops._ptr(gate),
+                                                  ops._ptr(k), ops._ptr(v), cfg.kv_dim, T, cfg.num_heads, cfg.num_kv_heads,
+                                                  cfg.head_dim, cfg.rotary_dim, 0, ops._ptr(positions), 0, cfg.rope_theta,
+                                                  cfg.rms_eps), "attn_qkv_epilogue")
+            self.quant.encode(k, cfg.kv_dim, kc.view(b, start), T, cfg.kv_dim)
+            self.quant.encode(v, cfg.kv_dim, vc.view(b, start), T, cfg.kv_dim)
+        ops.PrefillAttention(ctx).encode_causal(q, kc.view(b, 0), vc.view(b, 0), out, start, T, cfg.head_dim, cfg.num_heads,
+                                                cfg.num_kv_heads, start + T)
+        self.ew.encode_sigmoid_gate_mul(out, gate)
+        p_, s_, b_ = w["o_proj"]
+        return ops.affine_gemv(ctx, p_, s_, b_, cfg.attn_bits, out.view(T, cfg.q_dim), cfg.hidden, cfg.q_dim)
+
+    def _routed_moe_prefill(self, w, x, T):
+        """The MoE block of a chunk: below 64 rows the decode call (a work list over the distinct
+        experts), from 64 rows on the prefill path -- tiled router, permutation by expert, grouped
+        GEMM, rank-order reduce -- with the shared expert beside it."""
+        cfg, ctx = self.cfg, self.ctx
+        D, F, E, K = cfg.hidden, cfg.moe_intermediate, cfg.num_experts, cfg.top_k
+        if T < 64 and T * K <= 4096:
+            return self.moe.decode_layer(w["moe"], x)
+        layer = w["moe"]
+        idx, wts = self.moe.encode_router(layer.router, x, E, D, K)
+        routes = ops.PrefillMoEGrouping(ctx).group_routes(idx, wts, E)
+        pool = w["pool"]
+        partials, _ = ops.PrefillGroupedRoutedMoE(ctx, cfg.expert_bits).encode(pool[:E], layer.offsets, x, D, F, routes)
+        h2 = ops.PrefillMoE(ctx).encode_reduce_token_major(partials, wts, T, K, D)
+        shared = ops.SharedExpertRuntime(ctx, cfg.expert_bits).encode(pool[E], layer.offsets, x, D, F,
+                                                                      shared_gate=layer.shared_gate)
+        return self.ew.encode_residual_add(h2, shared)
 
     def head(self):
         """LM head over the final-normed rows: logits in self.logits."""

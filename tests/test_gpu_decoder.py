@@ -173,3 +173,55 @@ def test_step_replays_from_a_captured_graph():
         torch.cuda.synchronize()
         assert torch.equal(graphed.logits, eager.logits) and torch.equal(graphed.next_tokens, want)
     ctx.close()
+
+
+@pytest.mark.parametrize("prompt,chunk", [(80, 512), (80, 48), (200, 512)], ids=["one-chunk", "two-chunks", "dense-shared"])
+def test_prefill_chunks_leave_the_state_that_decode_steps_leave(prompt, chunk):
+    # RealForwardRunner.prefillChunked against its own serial decode loop: the prompt through the prefill
+    # kernels (dense matrix-core projections, recurrent kernels over the rows of a chunk, causal attention
+    # over the quantized cache, tiled router + permutation + grouped GEMM + reduce, shared expert) and
+    # through one decode step per token end in the same final-normed row, the same KV rows and recurrent
+    # states, and the next decode step from either gives the same logits -- within the 16-bit hand-over
+    # tolerance, the two paths round at different places.  Every expert is selected (top_k = experts), so
+    # that no near-tie of the router can send the two paths to different experts.
+    import nvmai_amd as nv
+    from nvmai_amd.decoder import HybridConfig, HybridDecoder, HybridWeights
+    say("prefill chunks vs decode steps", prompt, chunk)
+    ctx = nv.Context(0, nv.ACT_BF16)
+    cfg = HybridConfig(hidden=256, layers=4, full_every=2, num_heads=4, num_kv_heads=2, head_dim=64, rotary_dim=16,
+                       rope_theta=1e4, gdn=(2, 4, 32, 32, 4), num_experts=4, top_k=4, moe_intermediate=128, vocab=1024,
+                       expert_bits=4, attn_bits=4, kv_bits=8, head_bits=16, gdn_state_bf16=False)
+    w = HybridWeights(ctx, cfg, seed=11, std=0.06)
+    serial, chunked = HybridDecoder(ctx, cfg, w, 1, 256), HybridDecoder(ctx, cfg, w, 1, 256)
+    gen = torch.Generator(device="cuda").manual_seed(prompt)
+    tokens = torch.randint(0, cfg.vocab, (prompt,), generator=gen, device="cuda", dtype=torch.int32)
+    for position in range(prompt):
+        serial.tokens.copy_(tokens[position:position + 1])
+        want_last = serial.forward_hidden(position)
+    got_last = chunked.prefill_chunked(tokens, sequence=0, start_position=0, chunk_tokens=chunk)
+    torch.cuda.synchronize()
+    err = O.rel_error(act_np(got_last), act_np(want_last))
+    print("final-normed row of the last prompt token: rel", err, flush=True)
+    assert err < 2e-2
+    for L in serial.gdn_states:
+        (tail_a, state_a), (tail_b, state_b) = serial.gdn_states[L], chunked.gdn_states[L]
+        assert O.rel_error(act_np(tail_b), act_np(tail_a)) < 3e-2
+        assert (state_a - state_b).abs().max().item() <= 5e-2 * max(1.0, state_a.abs().max().item())
+    for L in serial.kv:
+        for ca, cb in zip(serial.kv[L], chunked.kv[L]):
+            ka = O.kv_dequant(ca.rows[0, :prompt].cpu().numpy(), cfg.kv_dim, cfg.kv_bits)
+            kb = O.kv_dequant(cb.rows[0, :prompt].cpu().numpy(), cfg.kv_dim, cfg.kv_bits)
+            assert O.rel_error(kb, ka) < 3e-2
+            assert int(cb.rows[0, prompt:].abs().max()) == 0          # nothing written past the prompt
+    # the next token from either state
+    nxt = torch.tensor([7], dtype=torch.int32, device="cuda")
+    outs = []
+    for dec in (serial, chunked):
+        dec.tokens.copy_(nxt)
+        dec.forward_hidden(prompt)
+        outs.append(act_np(dec.head()).copy())
+    torch.cuda.synchronize()
+    err = O.rel_error(outs[1], outs[0])
+    print("logits of the next decode step: rel", err, flush=True)
+    assert err < 3e-2
+    ctx.close()

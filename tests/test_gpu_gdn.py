@@ -83,7 +83,10 @@ def test_gdn_decode_chain_matches_oracle(nv, ctx, cfg):
 def test_gdn_prefill_chunk_equals_sequential_decode(nv, ctx):
     # prefillChunkMatchesSequentialDecode (GDNKernelTests.swift:189-290): seven rows in one call against seven
     # calls; and a chunk shorter than the conv history (the ordered tail shift, gdn.metal:337-366)
-    for cfg, rows in (((2, 4, 32, 32, 4), 7), ((16, 32, 128, 128, 4), 5), ((2, 4, 32, 32, 4), 2)):
+    # (from 8 rows on the call runs the conv and the output norm spread over the device and only the
+    # recurrence in sequence: 19, 33 and 12 rows, and 300 rows across two sets of precomputed gates)
+    for cfg, rows in (((2, 4, 32, 32, 4), 7), ((16, 32, 128, 128, 4), 5), ((2, 4, 32, 32, 4), 2), ((2, 4, 32, 32, 4), 19),
+                      ((16, 32, 128, 128, 4), 33), ((2, 2, 64, 64, 2), 12), ((1, 2, 64, 128, 3), 300)):
         say("gdn prefill chunk", ctx.act, cfg, rows)
         fx = _fixture(cfg, rows + 3, 0xBEEF, ctx.act)
         gdn = nv.GDN(ctx, *cfg)
