@@ -863,7 +863,8 @@ def decode_line(a, r, bits, batch, steps, warmup):
 def extra_cells(nv, ctx, torch, a, layers8, stride8):
     """The other cells of the metric, each measured like its own --workload line but shorter:
     4-bit decode at batch 32, 8-bit decode at one token, the configs[2] prefill grouped GEMM, and
-    configs[4] (the full 40-layer decode step, tok/s at batch 1 and 16), and every cell of configs[3]
+    configs[4] (the full 40-layer decode step, tok/s at batch 1 and 16, and its prompt side: 4096 tokens
+    through the same layers with the prefill kernels), and every cell of configs[3]
     (attention at 4K / 32K / 128K context x batch 1 / 8 with 8- and 4-bit KV, each checked against the
     oracle before it is reported)."""
     import argparse
@@ -889,6 +890,13 @@ def extra_cells(nv, ctx, torch, a, layers8, stride8):
         c["roofline_tok_per_s_at_8TBps"] = cell["config"]["roofline_tok_per_s_at_8TBps"]
         out["decode_step_configs4_batch%d" % batch] = c
         torch.cuda.empty_cache()
+    sub = argparse.Namespace(**vars(a))
+    sub.no_cpu, sub.steps, sub.warmup, sub.tokens, sub.chunk = True, 2, 1, 4096, 4096
+    cell = run_prefill_step(nv, ctx, torch, sub)
+    c = compact(cell)
+    c["model_gflop_per_token"] = cell["config"]["model_gflop_per_token"]
+    out["prefill_step_configs4_4096tokens"] = c
+    torch.cuda.empty_cache()
     for bits in (8, 4):
         sub = argparse.Namespace(**vars(a))
         sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.tokens, sub.context_given = True, 20, 3, bits, 4096, False
