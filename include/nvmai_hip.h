@@ -598,6 +598,20 @@ int nvmai_hip_residual_add_rmsnorm(nvmai_hip_ctx* ctx, nvmai_stream stream, void
                                    const void* delta, uint32_t delta_stride, const uint16_t* weight, void* out,
                                    uint32_t out_stride, uint32_t rows, uint32_t d, float eps);
 
+/* nvmai_hip_residual_add_rmsnorm followed by nvmai_hip_affine_gemv over the normed rows -- the input
+ * norm of a layer and its fused input projection (RealForwardRunner.swift:1857-1875, 2066-2085) -- in ONE
+ * launch for up to four rows of at most 2048 elements against a projection of at most 16,384 rows:
+ * every block norms the rows for itself (same arithmetic and order, so the same bits), the first
+ * block stores the updated residual rows to hidden_out, which must not be `hidden` (other blocks
+ * still read it).  delta may be NULL (norm only).  Any other shape runs the steps one after the other
+ * through normed_scratch ([n_tokens, normed_stride] activations; NVMAI_ERR_UNSUPPORTED when NULL). */
+int nvmai_hip_affine_gemv_prenorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
+                                  const uint16_t* scales, const uint16_t* biases, uint32_t bits, const void* hidden,
+                                  uint32_t hidden_stride, const void* delta, uint32_t delta_stride,
+                                  const uint16_t* norm_weight, float eps, void* hidden_out,
+                                  uint32_t hidden_out_stride, void* normed_scratch, uint32_t normed_stride,
+                                  uint32_t n_tokens, uint32_t m, uint32_t n, void* y, uint32_t y_stride);
+
 /* The epilogue of the q / k / v projection of a full-attention layer in one launch:
  * Elementwise.encodeSplitQGate + RMSNorm.encodeBF16WPerHead (q, k) + RoPE.encodeNeoxSubdim (q, k)
  * (RealForwardRunner.swift:2213-2255), or with q_packed = 0 and v_norm = 1 the reference's own

@@ -142,6 +142,8 @@ SIGNATURES = {
     "nvmai_hip_sampler_sample": [vp, vp, vp, vp, u32, vp, u32, C.POINTER(GenerationConfig), C.c_int64, C.c_float,
                                  C.c_int, vp, C.POINTER(C.c_int)],
     "nvmai_hip_residual_add_rmsnorm": [vp, vp, vp, u32, vp, u32, vp, vp, u32, u32, u32, C.c_float],
+    "nvmai_hip_affine_gemv_prenorm": [vp, vp, vp, vp, vp, u32, vp, u32, vp, u32, vp, C.c_float, vp, u32, vp, u32, u32, u32, u32,
+                                      vp, u32],
     "nvmai_hip_attn_qkv_epilogue": [vp, vp, vp, u32, C.c_int, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32,
                                     C.c_int, vp, u32, C.c_float, C.c_float],
     "nvmai_hip_attn_qkv_epilogue_kv": [vp, vp, vp, u32, C.c_int, vp, vp, vp, vp, vp, vp, u32, C.POINTER(KvView),

@@ -31,8 +31,14 @@ __device__ __forceinline__ float f16_to_f32(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
 
+// Round an fp32 value to fp16 (v_cvt_f16_f32, nearest even) as a step of its own.  The empty asm
+// hides where x came from: left to itself the compiler folds "round(a * b)" into v_fma_mixlo_f16,
+// which rounds the exact product once instead of rounding the fp32 product again -- in some kernels
+// and not in others, so that two kernels written with the same arithmetic differ in the last bit
+// of about one element in eight thousand.
 __device__ __forceinline__ uint16_t f32_to_f16(float x) {
-    return __builtin_bit_cast(uint16_t, (_Float16)x);   // v_cvt_f16_f32, RNE
+    asm("" : "+v"(x));
+    return __builtin_bit_cast(uint16_t, (_Float16)x);
 }
 
 template <int ACT>

@@ -610,6 +610,81 @@ extern "C" int nvmai_hip_affine_gemv(nvmai_hip_ctx* ctx, nvmai_stream stream, co
                            y_f32, y_stride);
 }
 
+namespace {
+// The dense rows engine with the residual add + RMSNorm prologue, for the block shapes a projection of
+// a decode step takes (up to 16,384 rows of 2048 codes).  False, having launched nothing, otherwise.
+template <int ACT, int BITS>
+bool launch_dense_prenorm_t(RowsParams& p, int maxtok, hipStream_t s) {
+    if ((p.n * BITS) % 128) return false;
+    const uint32_t chunks = p.n * BITS / 128;
+#define NVMAI_PRE(SEG, NCH, RPI, ITERS)                                                            \
+    do {                                                                                           \
+        constexpr uint32_t rows_per_block = 4 * (64 / SEG) * RPI * ITERS;                          \
+        p.blocks_per_entry = (p.rows + rows_per_block - 1) / rows_per_block;                       \
+        const size_t lds = rows_fast_lds_bytes_prenorm(p.n, NCH, SEG);                             \
+        const dim3 grid(p.blocks_per_entry);                                                       \
+        if (maxtok == 1) expert_rows_fast<ACT, BITS, SEG, NCH, 1, false, false, RPI, ITERS, true, true><<<grid, 256, lds, s>>>(p); \
+        else expert_rows_fast<ACT, BITS, SEG, NCH, 4, false, false, RPI, ITERS, true, true><<<grid, 256, lds, s>>>(p);             \
+        return true;                                                                               \
+    } while (0)
+    if (p.rows <= 4096 && chunks == 64) NVMAI_PRE(64, 1, 1, 2);
+    if (p.rows <= 4096 && chunks == 128) NVMAI_PRE(64, 2, 1, 2);
+    if (p.rows <= 16384 && chunks == 64) NVMAI_PRE(64, 1, 2, 2);
+    if (p.rows <= 16384 && chunks == 128) NVMAI_PRE(64, 2, 1, 4);
+#undef NVMAI_PRE
+    return false;
+}
+}  // namespace
+
+extern "C" int nvmai_hip_affine_gemv_prenorm(nvmai_hip_ctx* ctx, nvmai_stream stream, const uint8_t* weights,
+                                             const uint16_t* scales, const uint16_t* biases, uint32_t bits,
+                                             const void* hidden, uint32_t hidden_stride, const void* delta,
+                                             uint32_t delta_stride, const uint16_t* norm_weight, float eps,
+                                             void* hidden_out, uint32_t hidden_out_stride, void* normed_scratch,
+                                             uint32_t normed_stride, uint32_t n_tokens, uint32_t m, uint32_t n, void* y,
+                                             uint32_t y_stride) {
+    if (!ctx || !weights || !scales || !biases || !hidden || !norm_weight || !hidden_out || !y) return NVMAI_ERR_INVALID_ARG;
+    if (bits != 4 && bits != 8) return NVMAI_ERR_UNSUPPORTED;
+    if (n == 0 || n % NVMAI_GROUP || hidden_stride < n || hidden_out_stride < n || (delta && delta_stride < n) || y_stride < m)
+        return NVMAI_ERR_INVALID_ARG;
+    if (m == 0 || n_tokens == 0) return NVMAI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const bool rows16 = aligned16(hidden) && hidden_stride % 8 == 0 && aligned16(hidden_out) && hidden_out_stride % 8 == 0 &&
+                        aligned16(norm_weight) && (!delta || (aligned16(delta) && delta_stride % 8 == 0));
+    // every block norms the rows for itself when they are few, short and may be moved 16 bytes at a time,
+    // and the updated residual rows do not overwrite the ones other blocks still read
+    if (n_tokens <= (uint32_t)MAX_TOK && n <= 2048 && rows16 && aligned16(weights) && hidden_out != hidden) {
+        RowsParams p{};
+        p.src.slot[0] = weights;
+        p.sA = reinterpret_cast<const uint8_t*>(scales) - weights;
+        p.bA = reinterpret_cast<const uint8_t*>(biases) - weights;
+        p.x = hidden; p.x_stride = hidden_stride; p.rows = m; p.n = n;
+        p.out = nullptr; p.out_stride = y_stride; p.out_act = y; p.out_act_stride = y_stride;
+        p.dense_count = n_tokens;
+        p.pre_delta = (const uint16_t*)delta; p.pre_delta_stride = delta_stride; p.pre_weight = norm_weight;
+        p.pre_hidden_out = (uint16_t*)hidden_out; p.pre_hidden_stride = hidden_out_stride; p.pre_eps = eps;
+        const int maxtok = n_tokens == 1 ? 1 : MAX_TOK;
+        const bool done = ctx->act == ACT_BF16
+                              ? (bits == 8 ? launch_dense_prenorm_t<ACT_BF16, 8>(p, maxtok, s) : launch_dense_prenorm_t<ACT_BF16, 4>(p, maxtok, s))
+                              : (bits == 8 ? launch_dense_prenorm_t<ACT_FP16, 8>(p, maxtok, s) : launch_dense_prenorm_t<ACT_FP16, 4>(p, maxtok, s));
+        if (done) return launch_status();
+    }
+    // otherwise the steps one after the other, through the caller's scratch rows
+    if (!normed_scratch || normed_stride < n) return NVMAI_ERR_UNSUPPORTED;
+    if (hidden_out != hidden) {
+        const hipError_t e = hipMemcpy2DAsync(hidden_out, (size_t)hidden_out_stride * 2, hidden, (size_t)hidden_stride * 2,
+                                              (size_t)n * 2, n_tokens, hipMemcpyDeviceToDevice, s);
+        if (e != hipSuccess) return NVMAI_ERR_HIP;
+    }
+    int rc = delta ? nvmai_hip_residual_add_rmsnorm(ctx, stream, hidden_out, hidden_out_stride, delta, delta_stride,
+                                                    norm_weight, normed_scratch, normed_stride, n_tokens, n, eps)
+                   : nvmai_hip_rmsnorm(ctx, stream, hidden_out, hidden_out_stride, norm_weight, normed_scratch, normed_stride,
+                                       n_tokens, n, eps);
+    if (rc) return rc;
+    return nvmai_hip_affine_gemv(ctx, stream, weights, scales, biases, bits, normed_scratch, normed_stride, n_tokens, m, n, y,
+                                 nullptr, y_stride);
+}
+
 // The reference's CPU entry point with its own signature (host pointers, fp32 x, out written,
 // nothing returned): the operands travel to the device, the GEMV runs there, the result
 // travels back, and the call returns when `out` is complete.  A failure cannot be returned,

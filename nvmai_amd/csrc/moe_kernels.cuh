@@ -49,6 +49,15 @@ struct RowsParams {
     uint32_t dense_count;
     void* out_act;               // optional 16-bit copy of the result, rows out_act_stride apart;
     uint32_t out_act_stride;     // `out` may then be null
+    // dense launches with the PRENORM body: x holds the residual stream's rows and the inputs are
+    // rmsnorm(round(x + pre_delta)) * pre_weight, made by every block for itself (stage_prenorm_rows);
+    // block 0 stores the updated residual rows to pre_hidden_out.  n <= 2048, rows 16-byte aligned.
+    const uint16_t* pre_delta;
+    const uint16_t* pre_weight;
+    uint16_t* pre_hidden_out;
+    uint16_t* pre_normed_out;    // optional: block 0 also stores the normed rows
+    uint32_t pre_delta_stride, pre_hidden_stride, pre_normed_stride;
+    float pre_eps;
 };
 
 // ---- input staging ----------------------------------------------------------
@@ -73,6 +82,110 @@ __device__ __forceinline__ void load_x(const void* x, size_t row_off, uint32_t e
             act2_to_f32<ACT>(v.w, dst[8 * i + 6], dst[8 * i + 7]);
         }
     }
+}
+
+// ---- residual add + RMSNorm as the prologue of a kernel that stages its input rows in LDS ----------
+// Rows t0 .. t0 + nt - 1 of x (the residual stream) are summed with their delta rows, rounded,
+// normed and left in xl [nt][d] as 16-bit activations: the arithmetic and the summation order of
+// residual_add_rmsnorm / rms_direct_kernel, so the same bits.  The `writer` block also stores the
+// updated residual rows to hidden_out (never x itself: other blocks still read it) and, when asked, the
+// normed rows to normed_out.
+// raw: d 16-bit values of LDS.  A thread keeps its 16-byte pieces of the row in registers between
+// the add and the scaling (d <= 8192), every load is issued before the first use, and every wave
+// sums the squares for itself (the same 64-lane order, so the same bits) -- no broadcast, one
+// barrier less.  Ends with a barrier.
+struct PreNormArgs {
+    const uint16_t* x;             // [rows, x_stride] residual stream
+    uint32_t x_stride;
+    const uint16_t* delta;         // [rows, delta_stride] or null (norm only)
+    uint32_t delta_stride;
+    const uint16_t* weight;        // BF16 [d]
+    uint16_t* hidden_out;          // [rows, hidden_stride] or null
+    uint32_t hidden_stride;
+    uint16_t* normed_out;          // [rows, normed_stride] or null
+    uint32_t normed_stride;
+    float eps;
+    uint32_t d;
+};
+constexpr int ROUTER_PRE_PIECES = 4;                 // 16-byte pieces per thread: d <= 8192
+
+template <int ACT>
+__device__ __forceinline__ void stage_prenorm_rows(const PreNormArgs& p, uint32_t t0, uint32_t nt, uint16_t* xl,
+                                                   uint16_t* raw, const bool writer) {
+    const uint32_t per_row = p.d / 8, lane = threadIdx.x & 63;
+    for (uint32_t t = 0; t < nt; ++t) {
+        const uint16_t* h = p.x + (size_t)(t0 + t) * p.x_stride;
+        uint4 v[ROUTER_PRE_PIECES], dl[ROUTER_PRE_PIECES], w[ROUTER_PRE_PIECES];
+#pragma unroll
+        for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
+            const uint32_t c = threadIdx.x + 256 * k;
+            if (c >= per_row) break;
+            v[k] = *reinterpret_cast<const uint4*>(h + c * 8);
+            if (p.delta) dl[k] = *reinterpret_cast<const uint4*>(p.delta + (size_t)(t0 + t) * p.delta_stride + c * 8);
+            w[k] = *reinterpret_cast<const uint4*>(p.weight + c * 8);
+        }
+#pragma unroll
+        for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
+            const uint32_t c = threadIdx.x + 256 * k;
+            if (c >= per_row) break;
+            if (p.delta) {
+                uint32_t* vv = reinterpret_cast<uint32_t*>(&v[k]);
+                const uint32_t* dd = reinterpret_cast<const uint32_t*>(&dl[k]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float a0, a1, b0, b1;
+                    act2_to_f32<ACT>(vv[j], a0, a1);
+                    act2_to_f32<ACT>(dd[j], b0, b1);
+                    vv[j] = (uint32_t)f32_to_act<ACT>(__fadd_rn(a0, b0)) | ((uint32_t)f32_to_act<ACT>(__fadd_rn(a1, b1)) << 16);
+                }
+            }
+            reinterpret_cast<uint4*>(raw)[c] = v[k];
+            if (writer && p.hidden_out)
+                *reinterpret_cast<uint4*>(p.hidden_out + (size_t)(t0 + t) * p.hidden_stride + c * 8) = v[k];
+        }
+        __syncthreads();
+        // the stated order: lane l over the elements l, l + 64, ...; eight reads in flight at a time
+        float acc = 0.0f;
+        for (uint32_t i0 = lane; i0 < p.d; i0 += 512) {
+            uint16_t e[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) e[j] = i0 + 64 * j < p.d ? raw[i0 + 64 * j] : (uint16_t)0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                if (i0 + 64 * j >= p.d) break;
+                const float x = act_to_f32<ACT>(e[j]);
+                acc = fmaf(x, x, acc);
+            }
+        }
+        const float inv = rms_inverse(rms_wave_sum(acc), p.d, p.eps);
+#pragma unroll
+        for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
+            const uint32_t c = threadIdx.x + 256 * k;
+            if (c >= per_row) break;
+            const uint32_t* vv = reinterpret_cast<const uint32_t*>(&v[k]);
+            const uint32_t* ww = reinterpret_cast<const uint32_t*>(&w[k]);
+            uint4 o;
+            uint32_t* oo = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float a0, a1, w0, w1;
+                act2_to_f32<ACT>(vv[j], a0, a1);
+                act2_to_f32<ACT_BF16>(ww[j], w0, w1);
+                oo[j] = (uint32_t)f32_to_act<ACT>(__fmul_rn(__fmul_rn(a0, inv), w0)) |
+                        ((uint32_t)f32_to_act<ACT>(__fmul_rn(__fmul_rn(a1, inv), w1)) << 16);
+            }
+            reinterpret_cast<uint4*>(xl)[t * per_row + c] = o;
+            if (writer && p.normed_out)
+                *reinterpret_cast<uint4*>(p.normed_out + (size_t)(t0 + t) * p.normed_stride + c * 8) = o;
+        }
+        __syncthreads();                             // xl is complete; raw is rewritten by the next row
+    }
+}
+
+// Offset, in the fast engine's dynamic LDS, of the area behind its own arrays (16-byte aligned).
+__host__ __device__ inline size_t rows_fast_lds_base(uint32_t n, int nch, int seg) {
+    const size_t own = (size_t)4 /* MAX_TOK */ * (n / 8) * 16 + (size_t)4 * nch * seg * 8 + 4 * 4 * 4 + 4 * 4;
+    return (own + 15) & ~(size_t)15;
 }
 
 // ---- fast engine ------------------------------------------------------------
@@ -198,9 +311,11 @@ __device__ __forceinline__ void pow2_scale(float amax, float& sc, float& isc) {
 // we.reserved, output row we.pair_start.  ROWS_DENSE: input and output row we.pair_start + t, and
 // the result goes to p.out (fp32) and / or p.out_act (16 bit), whichever is not null.
 constexpr int ROWS_TABLES = 0, ROWS_DIRECT = 1, ROWS_DENSE = 2;
-template <int ACT, int BITS, int SEG, int NCH, int TOKS, bool DUAL, bool XF32, int RPI, int ITERS, int MODE = ROWS_TABLES>
+template <int ACT, int BITS, int SEG, int NCH, int TOKS, bool DUAL, bool XF32, int RPI, int ITERS, int MODE = ROWS_TABLES,
+          bool PRENORM = false>
 __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const WorkEntry& we, uint32_t rb,
                                                  uint4* lds) {
+    static_assert(!PRENORM || (MODE == ROWS_DENSE && !XF32), "the prologue is for dense launches over 16-bit rows");
     static_assert(MODE != ROWS_DIRECT || TOKS == 1, "a direct entry holds one input");
     auto in_row = [&](int t) -> uint32_t {
         return MODE == ROWS_DIRECT ? we.reserved : MODE == ROWS_DENSE ? we.pair_start + t : p.pair_in[we.pair_start + t];
@@ -270,9 +385,26 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
         float v[MT][8], m[MT];
         const uint32_t e0 = threadIdx.x * 8;
         const bool live = e0 < p.n;
+        if (PRENORM) {
+            // the normed rows are made here, in LDS behind the engine's own arrays, and read from there
+            uint16_t* xl = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(lds) + rows_fast_lds_base(p.n, NCH, SEG));
+            uint16_t* raw = xl + (size_t)MAX_TOK * p.n;
+            const PreNormArgs a{(const uint16_t*)p.x, p.x_stride, p.pre_delta, p.pre_delta_stride, p.pre_weight,
+                                p.pre_hidden_out, p.pre_hidden_stride, p.pre_normed_out, p.pre_normed_stride, p.pre_eps, p.n};
+            stage_prenorm_rows<ACT>(a, we.pair_start, (uint32_t)ntok, xl, raw, blockIdx.x == 0);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                if (t >= ntok) break;
+                if (live) {
+                    const uint4 r = *reinterpret_cast<const uint4*>(xl + (size_t)t * p.n + e0);
+                    act2_to_f32<ACT>(r.x, v[t][0], v[t][1]); act2_to_f32<ACT>(r.y, v[t][2], v[t][3]);
+                    act2_to_f32<ACT>(r.z, v[t][4], v[t][5]); act2_to_f32<ACT>(r.w, v[t][6], v[t][7]);
+                }
+            }
+        }
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-            if (t >= ntok) break;
+            if (t >= ntok || PRENORM) break;
             if (live) load8<ACT, XF32>(p.x, (size_t)in_row(t) * p.x_stride + e0, v[t]);
         }
 #pragma unroll
@@ -435,9 +567,13 @@ __device__ __forceinline__ void expert_rows_body(const RowsParams& p, const Work
     }
 }
 
-// Bytes of dynamic LDS the fast engine needs for rows of n codes.
+// Bytes of dynamic LDS the fast engine needs for rows of n codes; with the prologue the normed rows
+// (MAX_TOK x n) and one raw row follow at a 16-byte boundary.
 __host__ __device__ inline size_t rows_fast_lds_bytes(uint32_t n, int nch, int seg) {
     return (size_t)MAX_TOK * (n / 8) * 16 + (size_t)MAX_TOK * nch * seg * 8 + MAX_TOK * 4 * 4 + MAX_TOK * 4;
+}
+__host__ __device__ inline size_t rows_fast_lds_bytes_prenorm(uint32_t n, int nch, int seg) {
+    return rows_fast_lds_base(n, nch, seg) + (size_t)(MAX_TOK + 1) * n * 2;
 }
 
 // MAXTOK = 1: single-input launches.  MAXTOK = 4: the body is chosen by the
@@ -445,7 +581,8 @@ __host__ __device__ inline size_t rows_fast_lds_bytes(uint32_t n, int nch, int s
 // does not pay for more.
 // DENSE: the matrix in blob slot 0 against the input rows 0 .. dense_count - 1, entry e = the
 // rows e * MAXTOK .. (a grid of exactly that many entries; no work list, no pair tables).
-template <int ACT, int BITS, int SEG, int NCH, int MAXTOK, bool DUAL, bool XF32, int RPI, int ITERS, bool DENSE = false>
+template <int ACT, int BITS, int SEG, int NCH, int MAXTOK, bool DUAL, bool XF32, int RPI, int ITERS, bool DENSE = false,
+          bool PRENORM = false>
 __global__ __launch_bounds__(256) void expert_rows_fast(RowsParams p) {
     extern __shared__ uint4 rows_lds[];
     const uint32_t entry = blockIdx.x / p.blocks_per_entry;
@@ -462,9 +599,9 @@ __global__ __launch_bounds__(256) void expert_rows_fast(RowsParams p) {
         we = p.entries[entry];
     }
     if (MAXTOK == 1 || we.pair_count == 1)
-        expert_rows_body<ACT, BITS, SEG, NCH, 1, DUAL, XF32, RPI, ITERS, MODE>(p, we, rb, rows_lds);
+        expert_rows_body<ACT, BITS, SEG, NCH, 1, DUAL, XF32, RPI, ITERS, MODE, PRENORM>(p, we, rb, rows_lds);
     else
-        expert_rows_body<ACT, BITS, SEG, NCH, 0, DUAL, XF32, RPI, ITERS, MODE>(p, we, rb, rows_lds);
+        expert_rows_body<ACT, BITS, SEG, NCH, 0, DUAL, XF32, RPI, ITERS, MODE, PRENORM>(p, we, rb, rows_lds);
 }
 
 // ---- generic engine -----------------------------------------------------------
@@ -618,85 +755,14 @@ __device__ __forceinline__ void router_stage_x(const RouterParams& p, uint32_t t
     __syncthreads();
 }
 
-// The same with the prologue: the block's rows are summed with their delta, normed and staged.
-// raw: d 16-bit values of LDS.  A thread keeps its 16-byte pieces of the row in registers between
-// the add and the scaling (d <= 8192), every load is issued before the first use, and every wave
-// sums the squares for itself (the same 64-lane order, so the same bits) -- no broadcast, one
-// barrier less.  Ends with a barrier.
-constexpr int ROUTER_PRE_PIECES = 4;                 // 16-byte pieces per thread: d <= 8192
-
+// The same with the prologue (stage_prenorm_rows): the block's rows are summed with their delta,
+// normed and staged.
 template <int ACT>
 __device__ __forceinline__ void router_stage_prenorm(const RouterParams& p, uint32_t t0, uint32_t nt, uint16_t* xl,
                                                      uint16_t* raw) {
-    const bool writer = blockIdx.x == 0;
-    const uint32_t per_row = p.d / 8, lane = threadIdx.x & 63;
-    for (uint32_t t = 0; t < nt; ++t) {
-        const uint16_t* h = (const uint16_t*)p.x + (size_t)(t0 + t) * p.x_stride;
-        uint4 v[ROUTER_PRE_PIECES], dl[ROUTER_PRE_PIECES], w[ROUTER_PRE_PIECES];
-#pragma unroll
-        for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
-            const uint32_t c = threadIdx.x + 256 * k;
-            if (c >= per_row) break;
-            v[k] = *reinterpret_cast<const uint4*>(h + c * 8);
-            if (p.pre_delta) dl[k] = *reinterpret_cast<const uint4*>(p.pre_delta + (size_t)(t0 + t) * p.pre_delta_stride + c * 8);
-            w[k] = *reinterpret_cast<const uint4*>(p.pre_weight + c * 8);
-        }
-#pragma unroll
-        for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
-            const uint32_t c = threadIdx.x + 256 * k;
-            if (c >= per_row) break;
-            if (p.pre_delta) {
-                uint32_t* vv = reinterpret_cast<uint32_t*>(&v[k]);
-                const uint32_t* dd = reinterpret_cast<const uint32_t*>(&dl[k]);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float a0, a1, b0, b1;
-                    act2_to_f32<ACT>(vv[j], a0, a1);
-                    act2_to_f32<ACT>(dd[j], b0, b1);
-                    vv[j] = (uint32_t)f32_to_act<ACT>(__fadd_rn(a0, b0)) | ((uint32_t)f32_to_act<ACT>(__fadd_rn(a1, b1)) << 16);
-                }
-            }
-            reinterpret_cast<uint4*>(raw)[c] = v[k];
-            if (writer && p.pre_hidden_out)
-                *reinterpret_cast<uint4*>(p.pre_hidden_out + (size_t)(t0 + t) * p.pre_hidden_stride + c * 8) = v[k];
-        }
-        __syncthreads();
-        // the stated order: lane l over the elements l, l + 64, ...; eight reads in flight at a time
-        float acc = 0.0f;
-        for (uint32_t i0 = lane; i0 < p.d; i0 += 512) {
-            uint16_t e[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) e[j] = i0 + 64 * j < p.d ? raw[i0 + 64 * j] : (uint16_t)0;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                if (i0 + 64 * j >= p.d) break;
-                const float x = act_to_f32<ACT>(e[j]);
-                acc = fmaf(x, x, acc);
-            }
-        }
-        const float inv = rms_inverse(rms_wave_sum(acc), p.d, p.pre_eps);
-#pragma unroll
-        for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
-            const uint32_t c = threadIdx.x + 256 * k;
-            if (c >= per_row) break;
-            const uint32_t* vv = reinterpret_cast<const uint32_t*>(&v[k]);
-            const uint32_t* ww = reinterpret_cast<const uint32_t*>(&w[k]);
-            uint4 o;
-            uint32_t* oo = reinterpret_cast<uint32_t*>(&o);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float a0, a1, w0, w1;
-                act2_to_f32<ACT>(vv[j], a0, a1);
-                act2_to_f32<ACT_BF16>(ww[j], w0, w1);
-                oo[j] = (uint32_t)f32_to_act<ACT>(__fmul_rn(__fmul_rn(a0, inv), w0)) |
-                        ((uint32_t)f32_to_act<ACT>(__fmul_rn(__fmul_rn(a1, inv), w1)) << 16);
-            }
-            reinterpret_cast<uint4*>(xl)[t * per_row + c] = o;
-            if (writer && p.pre_normed_out)
-                *reinterpret_cast<uint4*>(p.pre_normed_out + (size_t)(t0 + t) * p.pre_normed_stride + c * 8) = o;
-        }
-        __syncthreads();                             // xl is complete; raw is rewritten by the next row
-    }
+    const PreNormArgs a{(const uint16_t*)p.x, p.x_stride, p.pre_delta, p.pre_delta_stride, p.pre_weight, p.pre_hidden_out,
+                        p.pre_hidden_stride, p.pre_normed_out, p.pre_normed_stride, p.pre_eps, p.d};
+    stage_prenorm_rows<ACT>(a, t0, nt, xl, raw, blockIdx.x == 0);
 }
 
 // One row against up to ROUTER_TOK tokens; hl = lane in the half-wave, CPL =

@@ -177,11 +177,24 @@ class HybridDecoder:
         self.ew = ops.Elementwise(ctx)
 
     # -- attention branches ---------------------------------------------------------------------
-    def _linear_attention(self, L, w):
+    def _input_projection(self, p_, s_, b_, rows, out, pre):
+        """The fused input projections of a layer over its normed input rows.  pre = the norm weight
+        of this layer when the residual add of the MoE block before it and this norm are still to
+        be done: the projection launch then does both itself (up to four sequences; same bits)
+        and the updated residual rows go to the second buffer."""
+        cfg = self.cfg
+        if pre is None:
+            ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, self.normed, rows, cfg.hidden, y=out)
+            return
+        ops.affine_gemv_prenorm(self.ctx, p_, s_, b_, cfg.attn_bits, self.hidden, self.moe_out, pre, self.hidden_alt, rows,
+                                cfg.hidden, y=out, normed_scratch=self.normed, eps=cfg.rms_eps)
+        self.hidden, self.hidden_alt = self.hidden_alt, self.hidden
+
+    def _linear_attention(self, L, w, pre=None):
         cfg, B = self.cfg, self.batch
         vh = cfg.gdn[1]
         p_, s_, b_ = w["in_proj"]
-        ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, self.normed, self.lin_rows, cfg.hidden, y=self.lin_proj)
+        self._input_projection(p_, s_, b_, self.lin_rows, self.lin_proj, pre)
         qkv = self.lin_proj[:, :cfg.gdn_qkv_dim]
         z = self.lin_proj[:, cfg.gdn_qkv_dim:cfg.gdn_qkv_dim + cfg.gdn_value_dim]
         a = self.lin_proj[:, cfg.gdn_qkv_dim + cfg.gdn_value_dim:cfg.gdn_qkv_dim + cfg.gdn_value_dim + vh]
@@ -212,10 +225,10 @@ class HybridDecoder:
         p_, s_, b_ = w["out_proj"]
         ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, self.gdn_out, cfg.hidden, cfg.gdn_value_dim, y=self.branch)
 
-    def _full_attention(self, L, w, position):
+    def _full_attention(self, L, w, position, pre=None):
         cfg, B = self.cfg, self.batch
         p_, s_, b_ = w["qkv"]
-        ops.affine_gemv(self.ctx, p_, s_, b_, cfg.attn_bits, self.normed, self.full_rows, cfg.hidden, y=self.full_proj)
+        self._input_projection(p_, s_, b_, self.full_rows, self.full_proj, pre)
         kc, vc = self.kv[L]
         if cfg.head_dim % 64 == 0 and cfg.kv_bits in (4, 8):
             # split + per-head norm + RoPE + quantize-on-write in one launch: one cache row per sequence,
@@ -256,18 +269,23 @@ class HybridDecoder:
                                          cfg.embed_bits, ops._ptr(self.tokens), 0, self.batch, ops._ptr(self.hidden),
                                          cfg.hidden, cfg.hidden, cfg.vocab, 1.0), "embed_lookup")
         ops.RMSNorm(ctx).encode_bf16w(self.hidden, self.w.layers[0]["in_norm"], out=self.normed, eps=cfg.rms_eps)
+        # up to four sequences: the residual add after a MoE block and the input norm of the next layer
+        # run inside that layer's projection launch (one launch less per layer)
+        fold = self.batch <= 4
         for L, w in enumerate(self.w.layers):
+            pre = w["in_norm"] if (fold and L > 0) else None
             if cfg.is_linear(L):
-                self._linear_attention(L, w)
+                self._linear_attention(L, w, pre)
             else:
-                self._full_attention(L, w, position)
+                self._full_attention(L, w, position, pre)
             # residual add + post-attention norm + MoE: the router launch does the add and the norm itself,
             # so the updated residual rows go to the second buffer (other blocks still read the first)
             self.moe.decode_layer_prenorm(w["moe"], self.hidden, self.branch, w["post_norm"], self.hidden_alt, self.normed,
                                           self.moe_out, eps=cfg.rms_eps)
             self.hidden, self.hidden_alt = self.hidden_alt, self.hidden
-            nxt = self.w.layers[L + 1]["in_norm"] if L + 1 < cfg.layers else self.w.final_norm
-            ops.residual_add_rmsnorm(ctx, self.hidden, self.moe_out, nxt, out=self.normed, eps=cfg.rms_eps)
+            if not fold or L + 1 == cfg.layers:
+                nxt = self.w.layers[L + 1]["in_norm"] if L + 1 < cfg.layers else self.w.final_norm
+                ops.residual_add_rmsnorm(ctx, self.hidden, self.moe_out, nxt, out=self.normed, eps=cfg.rms_eps)
         return self.normed
 
     # -- prefill: the tokens of ONE sequence, a chunk at a time, through every layer ------------------------

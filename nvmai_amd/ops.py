@@ -790,6 +790,24 @@ def residual_add_rmsnorm(ctx, hidden, delta, weight, out=None, eps=1e-6):
     return out
 
 
+def affine_gemv_prenorm(ctx, weights, scales, biases, bits, hidden, delta, norm_weight, hidden_out, m, n, y=None,
+                        normed_scratch=None, eps=1e-6):
+    """hidden_out = round(hidden + delta); y = W . (rmsnorm(hidden_out) * norm_weight): a layer's input norm
+    and its input projection in one launch for up to four rows (same bits as the two calls).  delta may
+    be None; normed_scratch [rows, n] is only used for shapes without the one-launch form."""
+    h2 = hidden.reshape(-1, hidden.shape[-1])
+    rows = h2.shape[0]
+    if y is None:
+        y = torch.empty((rows, m), dtype=ctx.dtype, device=h2.device)
+    d2 = None if delta is None else delta.reshape(-1, delta.shape[-1])
+    check(lib.nvmai_hip_affine_gemv_prenorm(ctx.handle, _stream(), _ptr(weights), _ptr(scales), _ptr(biases), bits,
+                                            _ptr(h2), h2.stride(0), _ptr(d2), 0 if d2 is None else d2.stride(0),
+                                            _ptr(norm_weight), eps, _ptr(hidden_out), hidden_out.stride(0),
+                                            _ptr(normed_scratch), 0 if normed_scratch is None else normed_scratch.stride(0),
+                                            rows, m, n, _ptr(y), y.stride(0)), "affine_gemv_prenorm")
+    return y
+
+
 def affine_gemv_fused(ctx, parts, bits, x, n):
     """GDN.encodeInputProjections / FusedQKVGEMV.encode: parts = [(weights, scales, biases, rows, y), ...],
     y_i = W_i x for the rows of x; one launch when the parts lie back to back in memory."""

@@ -616,3 +616,40 @@ def test_decode_layer_prenorm_equals_the_separate_calls(nv, ctx, bits):
         assert torch.equal(y, y_ref)
         if not in_place:
             assert torch.equal(h_in, h)                      # the residual rows read by the launch are untouched
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_affine_gemv_prenorm_equals_the_separate_calls(nv, ctx, bits):
+    # a layer's input norm (with the residual add before it) done by the projection launch: the bits
+    # of nvmai_hip_residual_add_rmsnorm followed by nvmai_hip_affine_gemv, for the one-launch shapes
+    # (1-4 rows of 2048 against a projection of a decode step) and for the shapes that fall back to
+    # the two steps through the scratch rows (more rows, short rows, a long projection)
+    rng = np.random.default_rng(900 + bits)
+    for tokens, m, n, with_delta in [(1, 12352, 2048, True), (4, 9216, 2048, True), (2, 2048, 2048, False), (3, 4100, 2048, True),
+                                     (1, 320, 256, True), (6, 2048, 2048, True), (2, 17000, 2048, True)]:
+        say("affine gemv prenorm", ctx.act, bits, tokens, m, n, with_delta)
+        wmat = torch.empty((m, n), device="cuda").normal_(0.0, 0.03).to(torch.bfloat16)
+        p_, s_, b_ = nv.quantize_affine(ctx, wmat, bits)
+        h = act_tensor(round_act(gauss(rng, (tokens, n)), ctx.act), ctx)
+        delta = act_tensor(round_act(gauss(rng, (tokens, n), 0.3), ctx.act), ctx) if with_delta else None
+        w = dev(O.bf16_bits(rng.uniform(0.5, 1.5, n).astype(np.float32)).view(np.int16))
+        h_ref = h.clone()
+        n_ref = nv.residual_add_rmsnorm(ctx, h_ref, delta, w) if with_delta else nv.RMSNorm(ctx).encode_bf16w(h_ref, w)
+        y_ref = nv.affine_gemv(ctx, p_, s_, b_, bits, n_ref, m, n)
+        h_in, h_out = h.clone(), torch.full_like(h, 9.0)
+        scratch = torch.full_like(h, 7.0)
+        y = nv.affine_gemv_prenorm(ctx, p_, s_, b_, bits, h_in, delta, w, h_out, m, n, normed_scratch=scratch)
+        torch.cuda.synchronize()
+        assert torch.equal(h_out, h_ref), "residual rows"
+        assert torch.equal(y.view(torch.int16), y_ref.view(torch.int16)), "projection"
+        assert torch.equal(h_in, h)                          # the rows the launch reads are untouched
+        fused = tokens <= 4 and n == 2048 and m <= 16384
+        assert bool((scratch == 7.0).all()) == fused         # the one-launch form never touches the scratch rows
+        if not fused:                                        # and without them the other shapes are refused
+            with pytest.raises(nv.NvmaiError):
+                nv.affine_gemv_prenorm(ctx, p_, s_, b_, bits, h_in, delta, w, h_out, m, n)
+    # hidden_out must be a buffer of its own for the one-launch form; in place it takes the two steps
+    h_in = h.clone()
+    y2 = nv.affine_gemv_prenorm(ctx, p_, s_, b_, bits, h_in, delta, w, h_in, m, n, normed_scratch=scratch)
+    torch.cuda.synchronize()
+    assert torch.equal(h_in, h_ref) and torch.equal(y2.view(torch.int16), y_ref.view(torch.int16))
