@@ -663,6 +663,12 @@ __device__ __forceinline__ uint4 dequant8(const float* q, float s, float b) {
 // is rounded once in fp32 (error below 2^-14 of a quantization step).  mask (0x000F000F or
 // 0x00FF00FF) and magic (0x64006400) arrive in registers: as literals they would split every
 // AND-OR in two, a three-operand instruction takes no literal here.
+// Measured and not kept: the result written as fp16 halves by v_fma_mixlo_f16 / v_fma_mixhi_f16
+// (no pack instructions, but the two issue at half the rate of v_fma_mix_f32: 18 % fewer vector
+// instructions, 7 % more vector cycles, 5 % slower); 4-bit pairs without two of the three shifts
+// (a nibble at bits 4..7 of a half as 64 + q under 0x5400, with a second shifted bias): four
+// more registers live across the loop, which the 256-register kernels do not have (52 bytes of
+// scratch, 8 % slower); 8-bit pairs by one byte permute each instead of shift + AND-OR (equal).
 template <int ACT, int BITS>
 __device__ __forceinline__ uint4 dequant8_magic(uint32_t w0, uint32_t w1, float s, float b1024, uint32_t mask, uint32_t magic) {
     typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
