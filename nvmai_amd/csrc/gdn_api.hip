@@ -2,6 +2,7 @@
 // and the fused input projections of an attention block.
 #include "ctx.hpp"
 #include "gdn_kernels.cuh"
+#include "gdn_chunk_kernels.cuh"
 
 using namespace nvmai;
 
@@ -25,9 +26,33 @@ GdnShape shape_of(const nvmai_gdn_config* c, uint32_t rows, uint32_t batch) {
 // sequential (two or three launches instead of one or two, so not for a handful of rows).
 constexpr uint32_t GDN_ROWS_PARALLEL_FROM = 8;
 
+// From this many rows per sequence on the recurrence of a 128 x 128 head runs sixteen rows at a time on
+// the matrix cores (a launch more, and 2,304 bytes of workspace per head and chunk).
+constexpr uint32_t GDN_CHUNKED_FROM = 64;
+
 template <int ACT, int DK, int DV>
-void launch_delta(const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
+bool launch_delta_chunked(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
+    if (DK != 128 || DV != 128) return false;
+    const uint32_t nchunks = (p.sh.rows + 15) / 16;
+    const size_t count = (size_t)p.sh.batch * p.sh.v_heads * nchunks;
+    if (!ctx || nchunks > 65535 || p.sh.batch > 65535 || (p.sh.rows + 1) / 2 > 65535 || !aligned16(p.conv_out) || p.conv_stride % 8 ||
+        (!state_bf16 && !aligned16(p.state)) || (reinterpret_cast<uintptr_t>(p.state) & 7u))
+        return false;
+    if (ws_begin(ctx, (nvmai_stream)s, ws_round(count * sizeof(GdnChunkPrep))) != NVMAI_OK) return false;
+    GdnChunkPrep* prep = ws_take<GdnChunkPrep>(ctx, count);
+    gdn_chunk_prep_kernel<ACT, 128><<<dim3(nchunks, p.sh.v_heads, p.sh.batch), 64, 0, s>>>(p, prep, nchunks);
+    const dim3 cgrid(p.sh.v_heads, p.sh.batch, 128 / 16);
+    if (state_bf16) gdn_chunk_delta_kernel<ACT, 128, 128, true><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
+    else gdn_chunk_delta_kernel<ACT, 128, 128, false><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
+    const dim3 ngrid(p.sh.v_heads, p.sh.batch, (p.sh.rows + 1) / 2);
+    gdn_gated_norm_rows_kernel<ACT><<<ngrid, 256, 0, s>>>(p.out, p.out_stride, p.z, p.z_stride, p.norm_w, p.sh);
+    return true;
+}
+
+template <int ACT, int DK, int DV>
+void launch_delta(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
     const dim3 grid(p.sh.v_heads, p.sh.batch);
+    if (p.sh.rows >= GDN_CHUNKED_FROM && launch_delta_chunked<ACT, DK, DV>(ctx, p, state_bf16, s)) return;
     if (p.sh.rows >= GDN_ROWS_PARALLEL_FROM && (p.sh.rows + 1) / 2 <= 65535 && aligned16(p.conv_out) && p.conv_stride % 8 == 0) {
         const dim3 rgrid(p.sh.v_heads, p.sh.batch, DV / 16);      // one group of sixteen state rows per block
         if (state_bf16) gdn_delta_rows_kernel<ACT, DK, DV, true, 1><<<rgrid, 256, 0, s>>>(p);
@@ -41,13 +66,13 @@ void launch_delta(const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
 }
 
 template <int ACT>
-int launch_delta_shape(const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
+int launch_delta_shape(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
     const uint32_t dk = p.sh.dk, dv = p.sh.dv;
-    if (dk == 128 && dv == 128) launch_delta<ACT, 128, 128>(p, state_bf16, s);
-    else if (dk == 64 && dv == 64) launch_delta<ACT, 64, 64>(p, state_bf16, s);
-    else if (dk == 32 && dv == 32) launch_delta<ACT, 32, 32>(p, state_bf16, s);
-    else if (dk == 64 && dv == 128) launch_delta<ACT, 64, 128>(p, state_bf16, s);
-    else if (dk == 128 && dv == 64) launch_delta<ACT, 128, 64>(p, state_bf16, s);
+    if (dk == 128 && dv == 128) launch_delta<ACT, 128, 128>(ctx, p, state_bf16, s);
+    else if (dk == 64 && dv == 64) launch_delta<ACT, 64, 64>(ctx, p, state_bf16, s);
+    else if (dk == 32 && dv == 32) launch_delta<ACT, 32, 32>(ctx, p, state_bf16, s);
+    else if (dk == 64 && dv == 128) launch_delta<ACT, 64, 128>(ctx, p, state_bf16, s);
+    else if (dk == 128 && dv == 64) launch_delta<ACT, 128, 64>(ctx, p, state_bf16, s);
     else return NVMAI_ERR_UNSUPPORTED;
     return NVMAI_OK;
 }
@@ -109,8 +134,8 @@ extern "C" int nvmai_hip_gdn_delta_gated_norm(nvmai_hip_ctx* ctx, nvmai_stream s
     p.out = (uint16_t*)out; p.out_stride = out_stride;
     p.sh = shape_of(config, rows, batch);
     hipStream_t s = (hipStream_t)stream;
-    rc = ctx->act == ACT_BF16 ? launch_delta_shape<ACT_BF16>(p, state_is_bf16 != 0, s)
-                              : launch_delta_shape<ACT_FP16>(p, state_is_bf16 != 0, s);
+    rc = ctx->act == ACT_BF16 ? launch_delta_shape<ACT_BF16>(ctx, p, state_is_bf16 != 0, s)
+                              : launch_delta_shape<ACT_FP16>(ctx, p, state_is_bf16 != 0, s);
     if (rc) return rc;
     return launch_status();
 }

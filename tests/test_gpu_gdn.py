@@ -86,7 +86,10 @@ def test_gdn_prefill_chunk_equals_sequential_decode(nv, ctx):
     # (from 8 rows on the call runs the conv and the output norm spread over the device and only the
     # recurrence in sequence: 19, 33 and 12 rows, and 300 rows across two sets of precomputed gates)
     for cfg, rows in (((2, 4, 32, 32, 4), 7), ((16, 32, 128, 128, 4), 5), ((2, 4, 32, 32, 4), 2), ((2, 4, 32, 32, 4), 19),
-                      ((16, 32, 128, 128, 4), 33), ((2, 2, 64, 64, 2), 12), ((1, 2, 64, 128, 3), 300)):
+                      ((16, 32, 128, 128, 4), 33), ((2, 2, 64, 64, 2), 12), ((1, 2, 64, 128, 3), 300),
+                      # from 64 rows on a 128 x 128 head takes sixteen rows at a time on the matrix cores:
+                      # whole chunks, a ragged last chunk, a single chunk plus one row
+                      ((2, 4, 128, 128, 4), 64), ((16, 32, 128, 128, 4), 100), ((1, 2, 128, 128, 3), 177), ((2, 2, 128, 128, 2), 65)):
         say("gdn prefill chunk", ctx.act, cfg, rows)
         fx = _fixture(cfg, rows + 3, 0xBEEF, ctx.act)
         gdn = nv.GDN(ctx, *cfg)
@@ -133,6 +136,36 @@ def test_gdn_batch_of_sequences_and_bf16_state(nv, ctx, bf16_state):
     got_state = state.float().cpu().numpy()
     for b in range(batch):
         assert np.abs(got_state[b] - refs[b].state).max() <= (5e-2 if not bf16_state else 1e-1)
+
+
+@pytest.mark.parametrize("bf16_state", [False, True])
+def test_gdn_long_call_on_the_matrix_cores_batch_and_state_types(nv, ctx, bf16_state):
+    # two sequences of 83 rows each in one call (five chunks of sixteen and a ragged sixth, the
+    # chunked form of the recurrence) against 83 calls of one row per sequence: outputs, tails, states
+    say("gdn chunked batch", ctx.act, bf16_state)
+    cfg, batch, rows = (2, 4, 128, 128, 4), 2, 83
+    fxs = [_fixture(cfg, rows, 700 + b, ctx.act) for b in range(batch)]
+    w = fxs[0]
+    gdn = nv.GDN(ctx, *cfg)
+    tail_a, state_a = gdn.new_state(batch, bf16=bf16_state)
+    tail_b, state_b = gdn.new_state(batch, bf16=bf16_state)
+    args = (_bits(w["a_log"]), _bits(w["dt_bias"]))
+    seq = []
+    for t in range(rows):
+        stack = lambda key: act_tensor(np.stack([fx[key][t] for fx in fxs]), ctx)
+        conv = gdn.encode_conv_norm(stack("qkv"), tail_a, _bits(w["conv_w"]))
+        seq.append(act_np(gdn.encode_delta_gated_norm(conv, stack("a"), stack("b"), *args, state_a, stack("z"), _bits(w["norm_w"]))))
+    cat = lambda key: act_tensor(np.concatenate([fx[key] for fx in fxs]), ctx)
+    conv = gdn.encode_conv_norm(cat("qkv"), tail_b, _bits(w["conv_w"]), rows=rows)
+    chunk = act_np(gdn.encode_delta_gated_norm(conv, cat("a"), cat("b"), *args, state_b, cat("z"), _bits(w["norm_w"]), rows=rows))
+    torch.cuda.synchronize()
+    want = np.stack(seq, axis=1).reshape(batch * rows, -1)            # [batch, rows, :] like the call's rows
+    if bf16_state:      # the row-by-row calls round the state to BF16 after every row, the long call once
+        assert np.all(np.abs(chunk - want) <= np.maximum(0.15, np.abs(want) * 0.3))
+    else:
+        assert _close(chunk, want, ctx.act)
+    assert torch.equal(tail_a, tail_b)
+    assert (state_a.float() - state_b.float()).abs().max().item() <= (5e-2 if not bf16_state else 1e-1)
 
 
 @pytest.mark.parametrize("bf16_state", [False, True])
