@@ -132,13 +132,13 @@ __global__ __launch_bounds__(64) void gdn_chunk_prep_kernel(GdnDeltaParams p, Gd
 // index 4 g + step, the B operand of S k and S q.  It contracts S k and S q over its own columns,
 // the four partial sums meet in LDS (added in wave order by every wave, so all four hold the same
 // bits), every wave repeats the two small products T R and W D, and updates its own columns.
-constexpr int GDN_CHUNK_WAVES = 4;
+constexpr int GDN_CHUNK_WAVES = 8;
 
 template <int ACT, int DK, int DV, bool STATE_BF16>
 __global__ __launch_bounds__(64 * GDN_CHUNK_WAVES) void gdn_chunk_delta_kernel(GdnDeltaParams p, const GdnChunkPrep* prep, uint32_t nchunks) {
     constexpr int NW = GDN_CHUNK_WAVES;
     constexpr int NBW = DK / 16 / NW;                   // 16-column blocks of the state per wave
-    static_assert(DK % (16 * NW) == 0 && DV % 16 == 0 && DK * 2 == 256 && NW == 4, "a row of k is sixteen 16-byte pieces; a wave stages four rows");
+    static_assert(DK % (16 * NW) == 0 && DV % 16 == 0 && DK * 2 == 256 && (NW == 4 || NW == 8), "a row of k is sixteen 16-byte pieces; a wave stages four rows");
     __shared__ __attribute__((aligned(16))) uint16_t ks[2][16][DK];
     __shared__ __attribute__((aligned(16))) uint16_t qs[2][16][DK];
     __shared__ __attribute__((aligned(16))) float red[2][NW][64][8];     // partial S k (4) and S q (4) per lane
@@ -167,9 +167,10 @@ __global__ __launch_bounds__(64 * GDN_CHUNK_WAVES) void gdn_chunk_delta_kernel(G
     struct Stage { uint4 k, q; uint16_t v[4]; float4 T, W, G, bG, beta, c; float G15; };
     auto fetch = [&](uint32_t c, Stage& st) {
         const uint32_t t0 = c * 16;
-        const uint16_t* base = p.conv_out + ((size_t)b * sh.rows + min(t0 + 4 * w + g, sh.rows - 1)) * p.conv_stride;
-        st.k = *reinterpret_cast<const uint4*>(base + (sh.k_heads + hk) * DK + i16 * 8);
-        st.q = *reinterpret_cast<const uint4*>(base + hk * DK + i16 * 8);
+        // four waves: wave w stages rows 4 w .. 4 w + 3 of k and of q; eight: waves 0 - 3 those of k, 4 - 7 those of q
+        const uint16_t* base = p.conv_out + ((size_t)b * sh.rows + min(t0 + 4 * (w & 3u) + g, sh.rows - 1)) * p.conv_stride;
+        st.k = *reinterpret_cast<const uint4*>(base + ((NW == 8 && w >= 4) ? hk : sh.k_heads + hk) * DK + i16 * 8);
+        if (NW == 4) st.q = *reinterpret_cast<const uint4*>(base + hk * DK + i16 * 8);
 #pragma unroll
         for (int r = 0; r < 4; ++r)
             st.v[r] = p.conv_out[((size_t)b * sh.rows + min(t0 + 4 * g + r, sh.rows - 1)) * p.conv_stride + 2 * sh.k_heads * DK + h * DV + dv];
@@ -183,9 +184,11 @@ __global__ __launch_bounds__(64 * GDN_CHUNK_WAVES) void gdn_chunk_delta_kernel(G
         st.G15 = pc->G[15];
     };
     auto to_lds = [&](uint32_t c, uint32_t buf, const Stage& st) {
-        const uint32_t keep = c * 16 + 4 * w + g < sh.rows ? 0xFFFFFFFFu : 0u;
-        *reinterpret_cast<uint4*>(&ks[buf][4 * w + g][i16 * 8]) = uint4{st.k.x & keep, st.k.y & keep, st.k.z & keep, st.k.w & keep};
-        *reinterpret_cast<uint4*>(&qs[buf][4 * w + g][i16 * 8]) = uint4{st.q.x & keep, st.q.y & keep, st.q.z & keep, st.q.w & keep};
+        const uint32_t srow = 4 * (w & 3u) + g;
+        const uint32_t keep = c * 16 + srow < sh.rows ? 0xFFFFFFFFu : 0u;
+        uint16_t* first = (NW == 8 && w >= 4) ? &qs[buf][srow][i16 * 8] : &ks[buf][srow][i16 * 8];
+        *reinterpret_cast<uint4*>(first) = uint4{st.k.x & keep, st.k.y & keep, st.k.z & keep, st.k.w & keep};
+        if (NW == 4) *reinterpret_cast<uint4*>(&qs[buf][srow][i16 * 8]) = uint4{st.q.x & keep, st.q.y & keep, st.q.z & keep, st.q.w & keep};
     };
     auto chunk = [&](uint32_t c, uint32_t buf, const Stage& st) {
         const uint32_t t0 = c * 16;
@@ -253,22 +256,27 @@ __global__ __launch_bounds__(64 * GDN_CHUNK_WAVES) void gdn_chunk_delta_kernel(G
                     p.out[((size_t)b * sh.rows + t0 + 4 * g + r) * p.out_stride + h * DV + dv] = f32_to_act<ACT>(Y[r]);
         }
     };
-    Stage st[2];
+    // two chunks on their way while one is worked on: chunk c travels in stage c % 3 (the loop is
+    // unrolled by three so that the stages stay registers)
+    Stage st[3];
     fetch(0, st[0]);
     to_lds(0, 0, st[0]);
+    fetch(1, st[1]);
     __syncthreads();
-    for (uint32_t c = 0;; c += 2) {
-        fetch(c + 1, st[1]);
-        chunk(c, 0, st[0]);
-        if (c + 1 >= nchunks) break;
-        to_lds(c + 1, 1, st[1]);
-        __syncthreads();
-        fetch(c + 2, st[0]);
-        chunk(c + 1, 1, st[1]);
-        if (c + 2 >= nchunks) break;
-        to_lds(c + 2, 0, st[0]);
-        __syncthreads();
+    uint32_t c = 0;
+#define NVMAI_GDN_CHUNK_STEP(A, B, C)                   \
+    fetch(c + 2, st[C]);                                \
+    chunk(c, c & 1u, st[A]);                            \
+    if (c + 1 >= nchunks) break;                        \
+    to_lds(c + 1, (c + 1) & 1u, st[B]);                 \
+    __syncthreads();                                    \
+    ++c;
+    for (;;) {
+        NVMAI_GDN_CHUNK_STEP(0, 1, 2)
+        NVMAI_GDN_CHUNK_STEP(1, 2, 0)
+        NVMAI_GDN_CHUNK_STEP(2, 0, 1)
     }
+#undef NVMAI_GDN_CHUNK_STEP
 #pragma unroll
     for (int bb = 0; bb < NBW; ++bb) {
         if (STATE_BF16) {
