@@ -204,15 +204,20 @@ __global__ __launch_bounds__(256) void gdn_delta_gated_kernel(GdnDeltaParams p) 
 // the same bits.  Segments of at most 128 channels.
 
 // conv + SiLU + q / k norm of rows [0, rows) of every sequence; the tail is read, not written.
+// A block takes sixteen rows of one segment, eight consecutive rows per pair of waves: a thread keeps
+// the window of its channel in registers, so a row costs it one two-byte load instead of one per tap.
+constexpr uint32_t GDN_CONV_ROWS_PER_BLOCK = 16;
+
 template <int ACT>
 __global__ __launch_bounds__(256) void gdn_conv_norm_rows_kernel(const uint16_t* qkv_raw, uint32_t qkv_stride,
                                                                 const uint16_t* tail, const uint16_t* conv_w,
                                                                 uint16_t* conv_out, uint32_t out_stride, GdnShape sh) {
-    __shared__ float part[4];
+    constexpr uint32_t RPP = GDN_CONV_ROWS_PER_BLOCK / 2;                   // rows per pair of waves
+    __shared__ float part[2][4];
     const uint32_t seg = blockIdx.x, b = blockIdx.y;
-    const uint32_t pair = threadIdx.x >> 7, i = threadIdx.x & 127u;         // row of the block, channel of the segment
+    const uint32_t pair = threadIdx.x >> 7, i = threadIdx.x & 127u;         // half of the block, channel of the segment
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const uint32_t t = blockIdx.z * 2u + pair;
+    const uint32_t t_first = blockIdx.z * GDN_CONV_ROWS_PER_BLOCK + pair * RPP;
     const uint32_t C = 2 * sh.k_heads * sh.dk + sh.v_heads * sh.dv;
     const bool is_qk = seg < 2 * sh.k_heads;
     const uint32_t seg_len = is_qk ? sh.dk : sh.dv;
@@ -220,33 +225,52 @@ __global__ __launch_bounds__(256) void gdn_conv_norm_rows_kernel(const uint16_t*
     const uint32_t hist = sh.taps - 1;
     const uint16_t* tl = tail + (size_t)b * hist * C;
     const uint16_t* raw = qkv_raw + (size_t)b * sh.rows * qkv_stride;
-    const bool live = t < sh.rows && i < seg_len;
-    const uint32_t ch = base + i;
-    float x = 0.0f;
-    uint16_t r = 0;
-    if (live) {
-        float acc = 0.0f;
-        for (uint32_t j = 0; j < sh.taps; ++j) {
-            const int src = (int)t + (int)j - (int)hist;
-            const uint16_t v = src >= 0 ? raw[(size_t)src * qkv_stride + ch] : tl[(size_t)((int)hist + src) * C + ch];
-            acc = fmaf(act_to_f32<ACT>(v), bf16_to_f32(conv_w[ch * sh.taps + j]), acc);
+    const bool ch_live = i < seg_len;
+    const uint32_t ch = base + (ch_live ? i : 0u);
+    auto value_at = [&](int src) -> float {                  // row src of [old tail | rows]
+        return act_to_f32<ACT>(src >= 0 ? raw[(size_t)src * qkv_stride + ch] : tl[(size_t)((int)hist + src) * C + ch]);
+    };
+    float wt[GDN_MAX_TAPS], pre[GDN_MAX_TAPS];               // weights; the hist values before the current row
+#pragma unroll
+    for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+        wt[j] = 0.0f; pre[j] = 0.0f;
+        if (j < sh.taps) wt[j] = bf16_to_f32(conv_w[ch * sh.taps + j]);
+        if (j < hist && t_first < sh.rows) pre[j] = value_at((int)t_first - (int)hist + (int)j);
+    }
+    const float scale = seg < sh.k_heads ? 1.0f / (float)sh.dk : rsqrtf((float)sh.dk);
+    for (uint32_t k = 0; k < RPP; ++k) {
+        const uint32_t t = t_first + k;
+        const bool live = t < sh.rows && ch_live;
+        float x = 0.0f;
+        uint16_t r = 0;
+        if (t < sh.rows) {
+            const float cur = value_at((int)t);
+            float acc = 0.0f;
+#pragma unroll
+            for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+                if (j >= sh.taps) break;
+                acc = fmaf(j < hist ? pre[j] : cur, wt[j], acc);
+            }
+#pragma unroll
+            for (uint32_t j = 0; j + 1 < GDN_MAX_TAPS; ++j) pre[j] = j + 1 < hist ? pre[j + 1] : cur;
+            if (live) {
+                r = f32_to_act<ACT>(gdn_silu(acc));
+                x = act_to_f32<ACT>(r);
+            }
         }
-        r = f32_to_act<ACT>(gdn_silu(acc));
-        x = act_to_f32<ACT>(r);
-    }
-    uint16_t* o = conv_out + ((size_t)b * sh.rows + t) * out_stride + ch;
-    if (!is_qk) {                                             // block-uniform
-        if (live) *o = r;
-        return;
-    }
-    const float ws = wave_sum_bcast(x * x);
-    if (lane == 0) part[wave] = ws;
-    __syncthreads();
-    if (live) {
-        const float total = (part[2 * pair] + part[2 * pair + 1]) + (0.0f + 0.0f);
-        const float inv = rsqrtf(total / (float)sh.dk + GDN_RMS_EPS);
-        const float scale = seg < sh.k_heads ? 1.0f / (float)sh.dk : rsqrtf((float)sh.dk);
-        *o = f32_to_act<ACT>(x * inv * scale);
+        uint16_t* o = conv_out + ((size_t)b * sh.rows + t) * out_stride + ch;
+        if (!is_qk) {                                         // block-uniform
+            if (live) *o = r;
+            continue;
+        }
+        const float ws = wave_sum_bcast(x * x);
+        if (lane == 0) part[k & 1u][wave] = ws;
+        __syncthreads();
+        if (live) {
+            const float total = (part[k & 1u][2 * pair] + part[k & 1u][2 * pair + 1]) + (0.0f + 0.0f);
+            const float inv = rsqrtf(total / (float)sh.dk + GDN_RMS_EPS);
+            *o = f32_to_act<ACT>(x * inv * scale);
+        }
     }
 }
 
