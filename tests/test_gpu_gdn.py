@@ -168,6 +168,28 @@ def test_gdn_long_call_on_the_matrix_cores_batch_and_state_types(nv, ctx, bf16_s
     assert (state_a.float() - state_b.float()).abs().max().item() <= (5e-2 if not bf16_state else 1e-1)
 
 
+def test_gdn_full_size_prompt_is_the_same_in_one_call_or_in_pieces(nv, ctx):
+    # the production layer (16 key / 32 value heads of 128 x 128, four taps) over 4096 rows, the size of a
+    # configs[4] prompt chunk: one call against calls of 1000 rows (ragged pieces, a last one of 96) and
+    # against calls of 48 rows (below the chunked form: the row-by-row recurrence) -- outputs, conv tails
+    # and states of the three must agree, whatever route the rows take through the kernels
+    say("gdn full size", ctx.act)
+    cfg, rows = (16, 32, 128, 128, 4), 4096
+    fx = _fixture(cfg, rows, 0x4096, ctx.act)
+    gdn = nv.GDN(ctx, *cfg)
+    outs, tails, states = [], [], []
+    for piece in (rows, 1000, 48):
+        tail, state = gdn.new_state()
+        got = [act_np(_gpu_rows(nv, ctx, gdn, fx, tail, state, t0, min(piece, rows - t0))) for t0 in range(0, rows, piece)]
+        torch.cuda.synchronize()
+        outs.append(np.concatenate(got)); tails.append(tail); states.append(state)
+    assert np.isfinite(outs[0]).all()
+    for k in (1, 2):
+        assert _close(outs[k], outs[0], ctx.act), k
+        assert torch.equal(tails[k], tails[0])
+        assert (states[k] - states[0]).abs().max().item() <= 5e-2
+
+
 @pytest.mark.parametrize("bf16_state", [False, True])
 @pytest.mark.parametrize("cfg", [(2, 4, 32, 32, 4), (16, 32, 128, 128, 4), (4, 4, 32, 32, 2), (2, 2, 64, 64, 2), (2, 8, 32, 32, 4)],
                          ids=["toy", "production", "ratio1-taps2", "two-kernel-shape", "two-kernel-ratio"])
