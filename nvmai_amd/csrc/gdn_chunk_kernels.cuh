@@ -164,13 +164,17 @@ __global__ __launch_bounds__(64 * GDN_CHUNK_WAVES) void gdn_chunk_delta_kernel(G
     // this lane's v values and the chunk's T / W pieces and gate vectors.  Every load is unconditional
     // (rows past the end re-read the last row and are zeroed afterwards) so that the loads stay in
     // flight over a chunk.
-    struct Stage { uint4 k, q; uint16_t v[4]; float4 T, W, G, bG, beta, c; float G15; };
-    auto fetch = [&](uint32_t c, Stage& st) {
+    struct StageKQ { uint4 k, q; };
+    struct Stage { uint16_t v[4]; float4 T, W, G, bG, beta, c; float G15; };
+    auto fetch_kq = [&](uint32_t c, StageKQ& st) {
         const uint32_t t0 = c * 16;
         // four waves: wave w stages rows 4 w .. 4 w + 3 of k and of q; eight: waves 0 - 3 those of k, 4 - 7 those of q
         const uint16_t* base = p.conv_out + ((size_t)b * sh.rows + min(t0 + 4 * (w & 3u) + g, sh.rows - 1)) * p.conv_stride;
         st.k = *reinterpret_cast<const uint4*>(base + ((NW == 8 && w >= 4) ? hk : sh.k_heads + hk) * DK + i16 * 8);
         if (NW == 4) st.q = *reinterpret_cast<const uint4*>(base + hk * DK + i16 * 8);
+    };
+    auto fetch = [&](uint32_t c, Stage& st) {
+        const uint32_t t0 = c * 16;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
             st.v[r] = p.conv_out[((size_t)b * sh.rows + min(t0 + 4 * g + r, sh.rows - 1)) * p.conv_stride + 2 * sh.k_heads * DK + h * DV + dv];
@@ -183,16 +187,17 @@ __global__ __launch_bounds__(64 * GDN_CHUNK_WAVES) void gdn_chunk_delta_kernel(G
         st.c = *reinterpret_cast<const float4*>(&pc->c[4 * g]);
         st.G15 = pc->G[15];
     };
-    auto to_lds = [&](uint32_t c, uint32_t buf, const Stage& st) {
+    auto to_lds = [&](uint32_t c, uint32_t buf, const StageKQ& st) {
         const uint32_t srow = 4 * (w & 3u) + g;
         const uint32_t keep = c * 16 + srow < sh.rows ? 0xFFFFFFFFu : 0u;
         uint16_t* first = (NW == 8 && w >= 4) ? &qs[buf][srow][i16 * 8] : &ks[buf][srow][i16 * 8];
         *reinterpret_cast<uint4*>(first) = uint4{st.k.x & keep, st.k.y & keep, st.k.z & keep, st.k.w & keep};
         if (NW == 4) *reinterpret_cast<uint4*>(&qs[buf][srow][i16 * 8]) = uint4{st.q.x & keep, st.q.y & keep, st.q.z & keep, st.q.w & keep};
     };
-    auto chunk = [&](uint32_t c, uint32_t buf, const Stage& st) {
-        const uint32_t t0 = c * 16;
-        // this wave's share of S k and S q: contraction index dk = 16 (NBW w + bb) + 4 g + s
+    float ku[NBW][4];                                    // the k values of the coming update
+    // front of a chunk: this wave's share of S k and S q from the state as it is now, into red[c & 1]
+    auto front = [&](uint32_t c, uint32_t buf) {
+        // contraction index dk = 16 (NBW w + bb) + 4 g + s
         gc_f4 P = {0.0f, 0.0f, 0.0f, 0.0f}, Q = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int bb = 0; bb < NBW; ++bb) {
@@ -208,8 +213,6 @@ __global__ __launch_bounds__(64 * GDN_CHUNK_WAVES) void gdn_chunk_delta_kernel(G
                 Q = gc_mfma4(qf[s], acc[bb][s], Q);
             }
         }
-        // the k values of the update, read while the sums travel
-        float ku[NBW][4];
 #pragma unroll
         for (int bb = 0; bb < NBW; ++bb)
 #pragma unroll
@@ -217,14 +220,15 @@ __global__ __launch_bounds__(64 * GDN_CHUNK_WAVES) void gdn_chunk_delta_kernel(G
         float* mine = red[c & 1u][w][lane];
         *reinterpret_cast<float4*>(mine) = float4{P[0], P[1], P[2], P[3]};
         *reinterpret_cast<float4*>(mine + 4) = float4{Q[0], Q[1], Q[2], Q[3]};
-        __syncthreads();
-        float Ps[4] = {0.0f, 0.0f, 0.0f, 0.0f}, Qs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    };
+    // back of a chunk, after the barrier that follows its front: the sums, the deltas, the update, the rows
+    auto back = [&](uint32_t c, const Stage& st) {
+        const uint32_t t0 = c * 16;
+        float Ps[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int ww = 0; ww < NW; ++ww) {
             const float4 a = *reinterpret_cast<const float4*>(red[c & 1u][ww][lane]);
-            const float4 bq = *reinterpret_cast<const float4*>(red[c & 1u][ww][lane] + 4);
             Ps[0] += a.x; Ps[1] += a.y; Ps[2] += a.z; Ps[3] += a.w;
-            Qs[0] += bq.x; Qs[1] += bq.y; Qs[2] += bq.z; Qs[3] += bq.w;
         }
         // R = beta v - beta G (S k); rows past the end hold beta = 0
         const float betav[4] = {st.beta.x, st.beta.y, st.beta.z, st.beta.w}, bGv[4] = {st.bG.x, st.bG.y, st.bG.z, st.bG.w};
@@ -247,6 +251,12 @@ __global__ __launch_bounds__(64 * GDN_CHUNK_WAVES) void gdn_chunk_delta_kernel(G
         }
         // y = G (S q) + W D, stored by the first wave
         if (w == 0) {
+            float Qs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww) {
+                const float4 bq = *reinterpret_cast<const float4*>(red[c & 1u][ww][lane] + 4);
+                Qs[0] += bq.x; Qs[1] += bq.y; Qs[2] += bq.z; Qs[3] += bq.w;
+            }
             gc_f4 Y = {Gv[0] * Qs[0], Gv[1] * Qs[1], Gv[2] * Qs[2], Gv[3] * Qs[3]};
 #pragma unroll
             for (int s = 0; s < 4; ++s) Y = gc_mfma4(Wf[s], D[s], Y);
@@ -256,25 +266,40 @@ __global__ __launch_bounds__(64 * GDN_CHUNK_WAVES) void gdn_chunk_delta_kernel(G
                     p.out[((size_t)b * sh.rows + t0 + 4 * g + r) * p.out_stride + h * DV + dv] = f32_to_act<ACT>(Y[r]);
         }
     };
-    // two chunks on their way while one is worked on: chunk c travels in stage c % 3 (the loop is
-    // unrolled by three so that the stages stay registers)
+    // One barrier per chunk: an iteration runs the back of chunk c and then, with the state just updated,
+    // the front of chunk c + 1, whose k and q rows reached LDS an iteration earlier.  On their way
+    // meanwhile: the k / q pieces of chunks c + 2 (stored at the end of the iteration) and c + 3, the
+    // other operands of chunks c + 1 and c + 2.  Chunk c travels in kq[c % 2] and st[c % 3]; the loop is
+    // unrolled by six so that both stay registers.
+    StageKQ kq[2];
     Stage st[3];
+    fetch_kq(0, kq[0]);
+    fetch_kq(1, kq[1]);
     fetch(0, st[0]);
-    to_lds(0, 0, st[0]);
     fetch(1, st[1]);
+    to_lds(0, 0, kq[0]);
+    __syncthreads();
+    front(0, 0);
+    fetch_kq(2, kq[0]);
+    to_lds(1, 1, kq[1]);
     __syncthreads();
     uint32_t c = 0;
-#define NVMAI_GDN_CHUNK_STEP(A, B, C)                   \
+#define NVMAI_GDN_CHUNK_STEP(K0, K1, A, C)              \
+    fetch_kq(c + 3, kq[K1]);                            \
     fetch(c + 2, st[C]);                                \
-    chunk(c, c & 1u, st[A]);                            \
+    back(c, st[A]);                                     \
     if (c + 1 >= nchunks) break;                        \
-    to_lds(c + 1, (c + 1) & 1u, st[B]);                 \
+    front(c + 1, (c + 1) & 1u);                         \
+    to_lds(c + 2, c & 1u, kq[K0]);                      \
     __syncthreads();                                    \
     ++c;
     for (;;) {
-        NVMAI_GDN_CHUNK_STEP(0, 1, 2)
-        NVMAI_GDN_CHUNK_STEP(1, 2, 0)
-        NVMAI_GDN_CHUNK_STEP(2, 0, 1)
+        NVMAI_GDN_CHUNK_STEP(0, 1, 0, 2)
+        NVMAI_GDN_CHUNK_STEP(1, 0, 1, 0)
+        NVMAI_GDN_CHUNK_STEP(0, 1, 2, 1)
+        NVMAI_GDN_CHUNK_STEP(1, 0, 0, 2)
+        NVMAI_GDN_CHUNK_STEP(0, 1, 1, 0)
+        NVMAI_GDN_CHUNK_STEP(1, 0, 2, 1)
     }
 #undef NVMAI_GDN_CHUNK_STEP
 #pragma unroll
