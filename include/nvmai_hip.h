@@ -232,6 +232,25 @@ int nvmai_hip_moe_decode_layer_prenorm(nvmai_hip_ctx* ctx, nvmai_stream stream, 
                                        uint32_t normed_stride, uint32_t n_tokens, void* y, uint32_t y_stride,
                                        uint32_t* out_idx, uint16_t* out_w, uint32_t* stats);
 
+/* The same with the residual add that closes the layer and the RMSNorm that opens the next one
+ * (RealForwardRunner.swift:1857-1920: encodeResidualAdd after the MoE block, then the next layer's
+ * RMSNorm.encodeBF16W):
+ *   hidden_out  = round(hidden + delta);  normed = rmsnorm(hidden_out) * norm_weight;  y = MoE(normed)
+ *   hidden_out  = round(hidden_out + y)
+ *   next_normed = rmsnorm(hidden_out) * next_norm_weight
+ * with the bits of nvmai_hip_moe_decode_layer_prenorm followed by nvmai_hip_residual_add_rmsnorm.
+ * From five tokens on (the work-list path) the last two lines ride in the block's combine launch,
+ * one block per token; otherwise they are the residual-add-norm kernel after the block.  hidden_out
+ * ends as the residual stream after the layer; next_normed must be a buffer of its own. */
+int nvmai_hip_moe_decode_layer_norms(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_moe_layer* layer,
+                                     const void* hidden, uint32_t hidden_stride, const void* delta,
+                                     uint32_t delta_stride, const uint16_t* norm_weight, float eps,
+                                     void* hidden_out, uint32_t hidden_out_stride, void* normed,
+                                     uint32_t normed_stride, uint32_t n_tokens, void* y, uint32_t y_stride,
+                                     uint32_t* out_idx, uint16_t* out_w, uint32_t* stats,
+                                     const uint16_t* next_norm_weight, void* next_normed,
+                                     uint32_t next_normed_stride);
+
 /* nvmai_hip_moe_decode_layer for callers that cannot allocate.  It has no counterpart in the
  * reference: it is for code under HIP graph capture, tight serving loops and harnesses that
  * forbid hipMalloc.  Same arguments, same results bit for bit, but the step's intermediate

@@ -103,6 +103,8 @@ SIGNATURES = {
     "nvmai_hip_moe_decode_layer": [vp, vp, C.POINTER(MoeLayer), vp, u32, u32, vp, u32, vp, vp, vp],
     "nvmai_hip_moe_decode_layer_prenorm": [vp, vp, C.POINTER(MoeLayer), vp, u32, vp, u32, vp, C.c_float, vp, u32, vp, u32,
                                            u32, vp, u32, vp, vp, vp],
+    "nvmai_hip_moe_decode_layer_norms": [vp, vp, C.POINTER(MoeLayer), vp, u32, vp, u32, vp, C.c_float, vp, u32, vp, u32,
+                                         u32, vp, u32, vp, vp, vp, vp, vp, u32],
     "nvmai_hip_moe_decode_layer_noalloc": [vp, vp, C.POINTER(MoeLayer), vp, u32, u32, vp, u32, vp, vp, vp],
     "nvmai_kv_row_layout": [u32, u32, C.POINTER(u32), C.POINTER(u32)],
     "nvmai_hip_kv_quantize_affine": [vp, vp, vp, u32, C.POINTER(KvView), u32, u32],

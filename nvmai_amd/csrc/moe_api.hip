@@ -1029,12 +1029,21 @@ struct PreNorm {
     void* normed; uint32_t normed_stride;
 };
 
+// After the block: stream += y, next = rmsnorm(stream) * weight (the residual add that closes the layer
+// and the norm that opens the next one).
+struct PostNorm {
+    void* stream; uint32_t stream_stride;
+    const uint16_t* weight; float eps;
+    void* next; uint32_t next_stride;
+    bool done;                                     // set when the combine launch took it along
+};
+
 // fixed_ws == nullptr: the buffers come from the context's workspace (grown when needed);
 // otherwise from the fixed_cap bytes at fixed_ws, and a step that needs more is refused.
 int decode_layer_impl(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_moe_layer* L, const void* x,
                       uint32_t x_stride, uint32_t n_tokens, void* y, uint32_t y_stride, uint32_t* out_idx,
                       uint16_t* out_w, uint32_t* stats, uint8_t* fixed_ws, size_t fixed_cap,
-                      const PreNorm* pre = nullptr) {
+                      const PreNorm* pre = nullptr, PostNorm* post = nullptr) {
     if (!ctx || !L || !x || !y) return NVMAI_ERR_INVALID_ARG;
     int rc = check_shape(L->d, L->f, L->bits);
     if (rc) return rc;
@@ -1152,6 +1161,16 @@ int decode_layer_impl(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_moe_l
     cp.partials = partials; cp.w = wts; cp.residual = nullptr; cp.gate_logit = gated ? gate_logit : nullptr;
     cp.has_shared = has_shared ? 1 : 0; cp.tokens = T; cp.top_k = K; cp.d = D; cp.res_stride = 0;
     cp.y_stride = y_stride; cp.y = y;
+    if (post && D % 8 == 0 && D <= 8 * 256 * ROUTER_PRE_PIECES && aligned16(post->stream) && post->stream_stride % 8 == 0 &&
+        aligned16(post->next) && post->next_stride % 8 == 0 && aligned16(post->weight) && aligned16(y) && y_stride % 8 == 0) {
+        // the combine, the residual add and the next norm in one launch, one block per token
+        const PostNormArgs pa{(uint16_t*)post->stream, post->stream_stride, post->weight, post->eps, (uint16_t*)post->next, post->next_stride};
+        ProfScope ps(ctx, NVMAI_PROF_COMBINE, s);
+        if (ctx->act == ACT_BF16) combine_postnorm_kernel<ACT_BF16><<<T, 256, D * 2, s>>>(cp, pa);
+        else combine_postnorm_kernel<ACT_FP16><<<T, 256, D * 2, s>>>(cp, pa);
+        post->done = true;
+        return launch_status();
+    }
     { ProfScope ps(ctx, NVMAI_PROF_COMBINE, s); run_combine(ctx->act, cp, s); }
     return launch_status();
 }
@@ -1199,6 +1218,45 @@ extern "C" int nvmai_hip_moe_decode_layer_prenorm(nvmai_hip_ctx* ctx, nvmai_stre
                                        n_tokens, D, eps);
     if (rc) return rc;
     return decode_layer_impl(ctx, stream, L, normed, normed_stride, n_tokens, y, y_stride, out_idx, out_w, stats, nullptr, 0);
+}
+
+// The block of a layer between two norms: residual add + norm before it (as the entry point above), and
+// after it the residual add that closes the layer with the norm that opens the next one:
+// hidden_out += y, next_normed = rmsnorm(hidden_out) * next_norm_weight.  With the work-list path
+// (five tokens or more) the last of these rides in the combine launch; otherwise it is the
+// residual-add-norm kernel after the block.  Same bits as the separate calls either way.
+extern "C" int nvmai_hip_moe_decode_layer_norms(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_moe_layer* L,
+                                                const void* hidden, uint32_t hidden_stride, const void* delta,
+                                                uint32_t delta_stride, const uint16_t* norm_weight, float eps,
+                                                void* hidden_out, uint32_t hidden_out_stride, void* normed,
+                                                uint32_t normed_stride, uint32_t n_tokens, void* y, uint32_t y_stride,
+                                                uint32_t* out_idx, uint16_t* out_w, uint32_t* stats,
+                                                const uint16_t* next_norm_weight, void* next_normed,
+                                                uint32_t next_normed_stride) {
+    if (!ctx || !L || !hidden || !norm_weight || !hidden_out || !normed || !y || !next_norm_weight || !next_normed)
+        return NVMAI_ERR_INVALID_ARG;
+    const uint32_t D = L->d;
+    if (hidden_stride < D || hidden_out_stride < D || normed_stride < D || next_normed_stride < D || (delta && delta_stride < D))
+        return NVMAI_ERR_INVALID_ARG;
+    if (n_tokens == 0) return NVMAI_OK;
+    const bool rows16 = aligned16(hidden) && hidden_stride % 8 == 0 && aligned16(hidden_out) && hidden_out_stride % 8 == 0 &&
+                        aligned16(normed) && normed_stride % 8 == 0 && aligned16(norm_weight) && D % 8 == 0 &&
+                        (!delta || (aligned16(delta) && delta_stride % 8 == 0));
+    PostNorm post{hidden_out, hidden_out_stride, next_norm_weight, eps, next_normed, next_normed_stride, false};
+    int rc;
+    if (n_tokens < 64 && rows16 && D <= 8192 && hidden_out != hidden && normed != hidden && normed != hidden_out &&
+        next_normed != hidden_out && next_normed != y) {
+        const PreNorm pre{delta, delta_stride, norm_weight, eps, hidden_out, hidden_out_stride, normed, normed_stride};
+        rc = decode_layer_impl(ctx, stream, L, hidden, hidden_stride, n_tokens, y, y_stride, out_idx, out_w, stats,
+                               nullptr, 0, &pre, &post);
+    } else {
+        rc = nvmai_hip_moe_decode_layer_prenorm(ctx, stream, L, hidden, hidden_stride, delta, delta_stride, norm_weight, eps,
+                                                hidden_out, hidden_out_stride, normed, normed_stride, n_tokens, y, y_stride,
+                                                out_idx, out_w, stats);
+    }
+    if (rc || post.done) return rc;
+    return nvmai_hip_residual_add_rmsnorm(ctx, stream, hidden_out, hidden_out_stride, y, y_stride, next_norm_weight,
+                                          next_normed, next_normed_stride, n_tokens, D, eps);
 }
 
 extern "C" size_t nvmai_hip_moe_decode_layer_noalloc_scratch_bytes(void) { return STATIC_SCRATCH_BYTES; }

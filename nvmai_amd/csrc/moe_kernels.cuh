@@ -1280,6 +1280,117 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineParams p) {
     ((uint16_t*)p.y)[(size_t)t * p.y_stride + d] = f32_to_act<ACT>(acc);
 }
 
+// The combine, the residual add that follows the MoE block and the RMSNorm that opens the next block, one
+// block per token: acc as combine_kernel takes it (same terms, same order), y = round(acc) (stored when
+// asked for), hidden = round(hidden + y) in place, normed = rmsnorm(hidden) * weight with the stated
+// summation order of rms_wave_sum / rms_inverse -- the bits of combine_kernel followed by the
+// residual-add-norm kernel.  d a multiple of 8, at most 8192; rows 16-byte aligned.
+struct PostNormArgs {
+    uint16_t* hidden; uint32_t hidden_stride;      // residual stream, updated in place
+    const uint16_t* weight; float eps;             // BF16 [d]
+    uint16_t* normed; uint32_t normed_stride;
+};
+
+template <int ACT>
+__global__ __launch_bounds__(256) void combine_postnorm_kernel(CombineParams p, PostNormArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t post_raw[];
+    const uint32_t t = blockIdx.x, per_row = p.d / 8, lane = threadIdx.x & 63;
+    uint4 v[ROUTER_PRE_PIECES], wv[ROUTER_PRE_PIECES];
+    float gate = 1.0f;
+    if (p.has_shared && p.gate_logit) gate = __fadd_rn(1.0f, expf(-p.gate_logit[t]));
+#pragma unroll
+    for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
+        const uint32_t c = threadIdx.x + 256 * k;
+        if (c >= per_row) break;
+        float acc[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+        auto row8 = [&](size_t row, float* f) {
+            const float4 lo = *reinterpret_cast<const float4*>(p.partials + row * p.d + c * 8);
+            const float4 hi = *reinterpret_cast<const float4*>(p.partials + row * p.d + c * 8 + 4);
+            f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w; f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
+        };
+        // every row of the sum is requested before the first is used (up to eight routed rows at a time):
+        // a block has one token's rows to itself, so what it waits for is a trip to memory, not bytes
+        float sh[8];
+        if (p.has_shared) row8((size_t)p.tokens * p.top_k + t, sh);
+        v[k] = *reinterpret_cast<const uint4*>(a.hidden + (size_t)t * a.hidden_stride + c * 8);
+        wv[k] = *reinterpret_cast<const uint4*>(a.weight + c * 8);
+        if (p.has_shared) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float s = p.gate_logit ? __fdiv_rn(sh[j], gate) : sh[j];
+                acc[j] = __fadd_rn(acc[j], s);
+            }
+        }
+        for (uint32_t r0 = 0; r0 < p.top_k; r0 += 8) {
+            float pr[8][8], w[8];
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                if (r0 + r < p.top_k) {
+                    w[r] = f16_to_f32(p.w[(size_t)t * p.top_k + r0 + r]);
+                    row8((size_t)t * p.top_k + r0 + r, pr[r]);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                if (r0 + r < p.top_k) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[j] = __fadd_rn(acc[j], __fmul_rn(w[r], pr[r][j]));
+                }
+            }
+        }
+        uint4 y16;
+        uint32_t* yy = reinterpret_cast<uint32_t*>(&y16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) yy[j] = (uint32_t)f32_to_act<ACT>(acc[2 * j]) | ((uint32_t)f32_to_act<ACT>(acc[2 * j + 1]) << 16);
+        if (p.y) *reinterpret_cast<uint4*>((uint16_t*)p.y + (size_t)t * p.y_stride + c * 8) = y16;
+        uint32_t* vv = reinterpret_cast<uint32_t*>(&v[k]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float a0, a1, b0, b1;
+            act2_to_f32<ACT>(vv[j], a0, a1);
+            act2_to_f32<ACT>(yy[j], b0, b1);
+            vv[j] = (uint32_t)f32_to_act<ACT>(__fadd_rn(a0, b0)) | ((uint32_t)f32_to_act<ACT>(__fadd_rn(a1, b1)) << 16);
+        }
+        reinterpret_cast<uint4*>(post_raw)[c] = v[k];
+        *reinterpret_cast<uint4*>(a.hidden + (size_t)t * a.hidden_stride + c * 8) = v[k];
+    }
+    __syncthreads();
+    // the stated order: lane l over the elements l, l + 64, ...; every wave for itself
+    float sum = 0.0f;
+    for (uint32_t i0 = lane; i0 < p.d; i0 += 512) {
+        uint16_t e[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = i0 + 64 * j < p.d ? post_raw[i0 + 64 * j] : (uint16_t)0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (i0 + 64 * j >= p.d) break;
+            const float x = act_to_f32<ACT>(e[j]);
+            sum = fmaf(x, x, sum);
+        }
+    }
+    const float inv = rms_inverse(rms_wave_sum(sum), p.d, a.eps);
+#pragma unroll
+    for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
+        const uint32_t c = threadIdx.x + 256 * k;
+        if (c >= per_row) break;
+        const uint32_t* vv = reinterpret_cast<const uint32_t*>(&v[k]);
+        const uint32_t* ww = reinterpret_cast<const uint32_t*>(&wv[k]);
+        uint4 o;
+        uint32_t* oo = reinterpret_cast<uint32_t*>(&o);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float a0, a1, w0, w1;
+            act2_to_f32<ACT>(vv[j], a0, a1);
+            act2_to_f32<ACT_BF16>(ww[j], w0, w1);
+            oo[j] = (uint32_t)f32_to_act<ACT>(__fmul_rn(__fmul_rn(a0, inv), w0)) |
+                    ((uint32_t)f32_to_act<ACT>(__fmul_rn(__fmul_rn(a1, inv), w1)) << 16);
+        }
+        *reinterpret_cast<uint4*>(a.normed + (size_t)t * a.normed_stride + c * 8) = o;
+    }
+}
+
 // ---- small decode batches: three launches instead of five ---------------------------------
 // With a handful of tokens the step is bound by its chain of dependent launches, not by bytes.
 // (1) expert_rows_routed: the gate/up launch selects for itself.  Every wave repeats its token's

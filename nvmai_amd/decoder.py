@@ -280,11 +280,18 @@ class HybridDecoder:
                 self._full_attention(L, w, position, pre)
             # residual add + post-attention norm + MoE: the router launch does the add and the norm itself,
             # so the updated residual rows go to the second buffer (other blocks still read the first)
+            nxt = self.w.layers[L + 1]["in_norm"] if L + 1 < cfg.layers else self.w.final_norm
+            if not fold:
+                # five sequences or more: the residual add that closes the layer and the next norm ride in the
+                # block's combine launch (the post-attention rows in self.normed are dead by then)
+                self.moe.decode_layer_norms(w["moe"], self.hidden, self.branch, w["post_norm"], self.hidden_alt, self.normed,
+                                            self.moe_out, nxt, self.normed, eps=cfg.rms_eps)
+                self.hidden, self.hidden_alt = self.hidden_alt, self.hidden
+                continue
             self.moe.decode_layer_prenorm(w["moe"], self.hidden, self.branch, w["post_norm"], self.hidden_alt, self.normed,
                                           self.moe_out, eps=cfg.rms_eps)
             self.hidden, self.hidden_alt = self.hidden_alt, self.hidden
-            if not fold or L + 1 == cfg.layers:
-                nxt = self.w.layers[L + 1]["in_norm"] if L + 1 < cfg.layers else self.w.final_norm
+            if L + 1 == cfg.layers:
                 ops.residual_add_rmsnorm(ctx, self.hidden, self.moe_out, nxt, out=self.normed, eps=cfg.rms_eps)
         return self.normed
 

@@ -236,6 +236,20 @@ class MoE:
         return y
 
 
+    def decode_layer_norms(self, layer, hidden, delta, norm_weight, hidden_out, normed, y, next_norm_weight, next_normed,
+                           eps=1e-6, idx=None, w=None, stats=None):
+        """nvmai_hip_moe_decode_layer_norms: decode_layer_prenorm, then hidden_out += y and
+        next_normed = rmsnorm(hidden_out) * next_norm_weight (the residual add that closes the layer and
+        the norm that opens the next); from five tokens on in the block's combine launch."""
+        h2 = hidden.reshape(-1, hidden.shape[-1])
+        check(lib.nvmai_hip_moe_decode_layer_norms(
+            self.ctx.handle, _stream(), C.byref(layer), _ptr(h2), h2.stride(0), _ptr(delta),
+            0 if delta is None else delta.stride(0), _ptr(norm_weight), eps, _ptr(hidden_out), hidden_out.stride(0),
+            _ptr(normed), normed.stride(0), h2.shape[0], _ptr(y), y.stride(0), _ptr(idx), _ptr(w), _ptr(stats),
+            _ptr(next_norm_weight), _ptr(next_normed), next_normed.stride(0)), "moe_decode_layer_norms")
+        return y
+
+
 def moe_layer_desc(d, f, num_experts, top_k, bits, router, experts, shared_blob=None, shared_gate=None,
                    eff_scale=None, per_expert_scale=None, offsets=None):
     """Fill an nvmai_moe_layer.  experts: uint8 tensor [num_experts, stride] (resident pool).

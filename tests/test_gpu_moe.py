@@ -619,6 +619,46 @@ def test_decode_layer_prenorm_equals_the_separate_calls(nv, ctx, bits):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
+def test_decode_layer_with_both_norms_equals_the_separate_calls(nv, ctx, bits):
+    # the block between two norms in one call: residual add + norm before it, and after it the residual
+    # add that closes the layer with the norm that opens the next one -- in the combine launch from
+    # five tokens on, the residual-add-norm kernel after the block below that and from 64 tokens on; the
+    # next norm's rows may land in the buffer of the first norm's (dead by then)
+    rng = np.random.default_rng(900 + bits)
+    d, f, E, k = 256, 128, 16, 4
+    off, stride = nv.expert_offsets(d, f, bits)
+    pool = torch.empty((E + 1, stride), dtype=torch.uint8, device="cuda")
+    for e in range(E + 1):
+        mk = lambda r, c: torch.randn((r, c), device="cuda").mul_(0.05).to(torch.bfloat16)
+        nv.pack_expert(ctx, mk(f, d), mk(f, d), mk(d, f), bits, pool[e])
+    rdesc = nv.rows_desc(16, dev(O.bf16_bits(gauss(rng, (E, d), 0.02)).view(np.int16)))
+    gh = O.quantize_affine(O.round_bf16(gauss(rng, (1, d), 0.05)), 8)
+    gdesc = nv.rows_desc(8, dev(gh[0]), dev(gh[1].view(np.int16)), dev(gh[2].view(np.int16)))
+    w1 = dev(O.bf16_bits(rng.uniform(0.5, 1.5, d).astype(np.float32)).view(np.int16))
+    w2 = dev(O.bf16_bits(rng.uniform(0.5, 1.5, d).astype(np.float32)).view(np.int16))
+    moe = nv.MoE(ctx, bits)
+    for tokens, gated, alias in [(1, True, False), (4, True, True), (5, True, False), (16, True, True), (32, False, True),
+                                 (63, True, False), (70, True, True)]:
+        say("decode layer norms", ctx.act, bits, tokens, gated, alias)
+        layer = nv.moe_layer_desc(d, f, E, k, bits, rdesc, pool[:E], pool[E], gdesc if gated else None)
+        h = act_tensor(round_act(gauss(rng, (tokens, d)), ctx.act), ctx)
+        delta = act_tensor(round_act(gauss(rng, (tokens, d), 0.3), ctx.act), ctx)
+        # reference: the separate calls
+        h_ref, n_ref, y_ref = torch.full_like(h, 9.0), torch.full_like(h, 9.0), torch.full_like(h, 9.0)
+        moe.decode_layer_prenorm(layer, h.clone(), delta, w1, h_ref, n_ref, y_ref)
+        next_ref = nv.residual_add_rmsnorm(ctx, h_ref, y_ref, w2)
+        h_out, normed, y = torch.full_like(h, 9.0), torch.full_like(h, 9.0), torch.full_like(h, 9.0)
+        nxt = normed if alias else torch.full_like(h, 9.0)
+        moe.decode_layer_norms(layer, h.clone(), delta, w1, h_out, normed, y, w2, nxt)
+        torch.cuda.synchronize()
+        assert torch.equal(y, y_ref)
+        assert torch.equal(h_out, h_ref)                      # the stream after the layer
+        assert torch.equal(nxt, next_ref)
+        if not alias:
+            assert torch.equal(normed, n_ref)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
 def test_affine_gemv_prenorm_equals_the_separate_calls(nv, ctx, bits):
     # a layer's input norm (with the residual add before it) done by the projection launch: the bits
     # of nvmai_hip_residual_add_rmsnorm followed by nvmai_hip_affine_gemv, for the one-launch shapes
