@@ -146,11 +146,26 @@ int dense_bf16_gemv(nvmai_hip_ctx* ctx, hipStream_t s, const uint16_t* w, const 
         lds_raised = true;
     }
     const uint32_t groups = (m + 63) / 64;                   // 64 rows per block pass
-    const uint32_t per_block = groups >= 4 * 1024 ? 4u : 1u; // long launches: fewer, longer blocks (the inputs are staged once per block)
-    const dim3 grid((groups + per_block - 1) / per_block);
+    // Blocks per compute unit follow from the staged inputs (4 KB of LDS each at the usual width):
+    // five at one input, two at sixteen.  With three or more the hardware's own hand-out of short
+    // blocks is the fastest form (one pass per block; two or three passes, or one resident round,
+    // measured 3 to 14 % slower at 1..12 inputs: 180 us = 5.7 TB/s for 1.02 GB at one input).  At two
+    // blocks per unit the 64 KB staging of every block is what costs, and one resident round of long
+    // blocks wins (217 -> 202 us at sixteen inputs).
+    static int resident[DENSE_TOK + 1] = {};                 // blocks per compute unit by staged inputs
     for (uint32_t t0 = 0; t0 < n_tokens; t0 += DENSE_TOK) {
         const uint32_t nt = n_tokens - t0 < (uint32_t)DENSE_TOK ? n_tokens - t0 : (uint32_t)DENSE_TOK;
-        dense_bf16_gemv_kernel<<<grid, 256, DENSE_TOK * (n * 2 + 16), s>>>(
+        const uint32_t lds = nt * (n * 2 + 16);
+        int occ = n == 2048 ? resident[nt] : 0;              // cached for the usual width only
+        if (occ == 0) {
+            NVMAI_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, dense_bf16_gemv_kernel, 256, lds));
+            if (occ < 1) occ = 1;
+            if (n == 2048) resident[nt] = occ;
+        }
+        const uint32_t places = (uint32_t)occ * (uint32_t)ctx->compute_units;
+        const uint32_t per_block = occ >= 3 ? 1u : (groups + places - 1) / places;
+        const dim3 grid((groups + per_block - 1) / per_block);
+        dense_bf16_gemv_kernel<<<grid, 256, lds, s>>>(
             w, (const uint16_t*)x + (size_t)t0 * x_stride, x_stride, nt, m, n,
             y ? (uint16_t*)y + (size_t)t0 * y_stride : nullptr, y_f32 ? y_f32 + (size_t)t0 * y_stride : nullptr, y_stride,
             per_block);

@@ -301,7 +301,10 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(QkvEpilogueParams p) 
 // q = lane / 16) loads the 32 bytes W[r0 + i, k0 + 16 q .. + 16), so four lanes cover 128 contiguous
 // bytes of a row and every byte of the matrix is read once -- and the inputs are the A operand,
 // staged once per block in LDS (rows 16 bytes apart from a power of two, so the sixteen inputs of a
-// fragment read fall into different banks).  A wave owns 16 rows at a time and keeps DEPTH
+// fragment read fall into different banks).  Only the inputs that exist are staged: row t of A
+// reaches row t of the product alone, and the rows of absent inputs are never stored, so their lanes
+// read the last staged input again -- at one input a block holds 4 KB of LDS instead of 64 and the
+// resident waves per CU are bounded by registers.  A wave owns 16 rows at a time and keeps DEPTH
 // super-steps of 64 k in flight.  The product is bound by the matrix's bytes: the matrix cores
 // idle most of the time, which is what lets one kernel serve 1 to 16 inputs at the same speed.
 typedef __bf16 dg_bf8_t __attribute__((ext_vector_type(8)));
@@ -316,16 +319,15 @@ __global__ __launch_bounds__(256) void dense_bf16_gemv_kernel(const uint16_t* w,
     const uint32_t ld = n * 2u + 16u;                       // bytes between two inputs in LDS
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t li = lane & 15u, lq = lane >> 4;
-    // inputs -> LDS, zero rows for the inputs that are not there
-    for (uint32_t c = tid; c < DENSE_TOK * (n / 8u); c += 256u) {
+    // inputs -> LDS
+    for (uint32_t c = tid; c < tokens * (n / 8u); c += 256u) {
         const uint32_t t = c / (n / 8u), k8 = c % (n / 8u);
-        uint4 v = uint4{0, 0, 0, 0};
-        if (t < tokens) v = *reinterpret_cast<const uint4*>(x + (size_t)t * x_stride + k8 * 8u);
-        *reinterpret_cast<uint4*>(dense_lds + t * ld + k8 * 16u) = v;
+        *reinterpret_cast<uint4*>(dense_lds + t * ld + k8 * 16u) =
+            *reinterpret_cast<const uint4*>(x + (size_t)t * x_stride + k8 * 8u);
     }
     __syncthreads();
     const uint32_t steps = n / 64u;                         // super-steps of 64 k: two MFMAs each
-    const uint8_t* xa = dense_lds + li * ld + lq * 32u;      // this lane's A fragments
+    const uint8_t* xa = dense_lds + min(li, tokens - 1u) * ld + lq * 32u;   // this lane's A fragments
     for (uint32_t g = 0; g < row_groups_per_block; ++g) {
         const uint32_t r0 = ((blockIdx.x * row_groups_per_block + g) * 4u + wave) * 16u;
         if (r0 >= m) break;                                 // wave-uniform
