@@ -297,7 +297,9 @@ def test_dense_bf16_gemv(nv):
     say("dense bf16 gemv")
     ctx = nv.Context(0, 0)
     rng = np.random.default_rng(9)
-    for m, n, tokens in ((1000, 2048, 1), (70, 256, 3), (4096, 2048, 16), (515, 1024, 21), (64, 64, 2)):
+    # (70001 rows at 16 inputs: more 64-row passes than resident blocks, so blocks walk several passes)
+    for m, n, tokens in ((1000, 2048, 1), (70, 256, 3), (4096, 2048, 16), (515, 1024, 21), (64, 64, 2),
+                         (70001, 2048, 16), (40000, 2048, 1)):
         w = O.round_bf16(gauss(rng, (m, n), 0.02))
         x = O.round_bf16(gauss(rng, (tokens, n)))
         wd = dev(O.bf16_bits(w).view(np.int16))
