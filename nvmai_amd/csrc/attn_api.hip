@@ -1,7 +1,7 @@
 // Entry points: KV row layout, quantize-on-write, partial RoPE, GQA decode attention.
 #include <cmath>
 
-#include "attn_kernels.cuh"
+#include "attn_kernels.hpp"
 #include "ctx.hpp"
 
 using namespace nvmai;

@@ -2,7 +2,7 @@
 // gfx950, wave64.
 #pragma once
 
-#include "common.cuh"
+#include "common.hpp"
 
 namespace nvmai {
 

@@ -1,8 +1,8 @@
 // Entry points: gated-DeltaNet linear attention (conv + q / k norm, delta rule + gated output norm)
 // and the fused input projections of an attention block.
 #include "ctx.hpp"
-#include "gdn_kernels.cuh"
-#include "gdn_chunk_kernels.cuh"
+#include "gdn_kernels.hpp"
+#include "gdn_chunk_kernels.hpp"
 
 using namespace nvmai;
 

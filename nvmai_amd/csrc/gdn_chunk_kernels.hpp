@@ -18,7 +18,7 @@
 // operand layout of the next when the contraction index is taken as 4 (lane / 16) + step, so
 // nothing is transposed or moved between lanes.
 #pragma once
-#include "gdn_kernels.cuh"
+#include "gdn_kernels.hpp"
 
 namespace nvmai {
 

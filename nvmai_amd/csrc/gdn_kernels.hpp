@@ -6,7 +6,7 @@
 // a batch has its own conv tail and recurrent state.
 #pragma once
 
-#include "common.cuh"
+#include "common.hpp"
 
 namespace nvmai {
 

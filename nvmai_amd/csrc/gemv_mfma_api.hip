@@ -1,6 +1,6 @@
 // Host side of the matrix-core GEMV for 5 .. 32 input rows.
 #include "ctx.hpp"
-#include "gemv_mfma_kernels.cuh"
+#include "gemv_mfma_kernels.hpp"
 
 namespace nvmai {
 

@@ -28,7 +28,7 @@
 //   accumulators:                input i, rows 4 r .. 4 r + 3
 #pragma once
 
-#include "common.cuh"
+#include "common.hpp"
 
 namespace nvmai {
 

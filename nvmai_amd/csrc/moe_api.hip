@@ -5,7 +5,7 @@
 #include <new>
 
 #include "ctx.hpp"
-#include "moe_kernels.cuh"
+#include "moe_kernels.hpp"
 
 using namespace nvmai;
 

@@ -3,7 +3,7 @@
 // weighted combine, and the affine group-64 quantizer.  gfx950, wave64.
 #pragma once
 
-#include "common.cuh"
+#include "common.hpp"
 
 namespace nvmai {
 

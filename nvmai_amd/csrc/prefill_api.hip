@@ -1,6 +1,6 @@
 // Entry points: token-expert pairs, grouping by expert, grouped expert GEMMs, rank-order reduce.
 #include "ctx.hpp"
-#include "prefill_kernels.cuh"
+#include "prefill_kernels.hpp"
 
 using namespace nvmai;
 

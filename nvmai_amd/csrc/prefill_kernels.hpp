@@ -3,7 +3,7 @@
 // combine.  gfx950, wave64.
 #pragma once
 
-#include "common.cuh"
+#include "common.hpp"
 
 namespace nvmai {
 

@@ -4,7 +4,7 @@
 #include <atomic>
 
 #include "ctx.hpp"
-#include "sample_kernels.cuh"
+#include "sample_kernels.hpp"
 
 using namespace nvmai;
 

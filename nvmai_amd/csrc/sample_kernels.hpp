@@ -1,7 +1,7 @@
 // Softmax over the vocabulary and the tiled top-64 / generic samplers.  gfx950, wave64.
 #pragma once
 
-#include "common.cuh"
+#include "common.hpp"
 
 namespace nvmai {
 

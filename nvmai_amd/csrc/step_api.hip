@@ -2,7 +2,7 @@
 #include <initializer_list>
 
 #include "ctx.hpp"
-#include "step_kernels.cuh"
+#include "step_kernels.hpp"
 
 using namespace nvmai;
 

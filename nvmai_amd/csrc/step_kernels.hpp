@@ -2,7 +2,7 @@
 // and the fused greedy LM head (RMSNorm -> one logit per vocabulary row -> argmax).  gfx950.
 #pragma once
 
-#include "common.cuh"
+#include "common.hpp"
 
 namespace nvmai {
 
@@ -12,7 +12,7 @@ namespace nvmai {
 // One wave per row.  The sum of squares has a fixed order so that a CPU run of the same order
 // gives the same bits: lane l runs acc = fma(x, x, acc) over the elements l, l + 64, ...,
 // then an xor butterfly 32, 16, 8, 4, 2, 1; every later step is one IEEE operation.
-// (rms_wave_sum and rms_inverse, the stated order and the single IEEE steps, are in common.cuh)
+// (rms_wave_sum and rms_inverse, the stated order and the single IEEE steps, are in common.hpp)
 
 // One wave per row.  STAGED: the row travels through LDS -- 16-byte loads in, the per-lane sums
 // and products read and written two bytes at a time there, 16-byte stores out -- so that a lane's
