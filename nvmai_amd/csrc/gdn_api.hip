@@ -30,6 +30,21 @@ constexpr uint32_t GDN_ROWS_PARALLEL_FROM = 8;
 // the matrix cores (a launch more, and 2,304 bytes of workspace per head and chunk).
 constexpr uint32_t GDN_CHUNKED_FROM = 64;
 
+// The gated norm over the rows the recurrence left in out: heads of 128 values in 16-byte pieces where
+// the rows allow it (same bits), one value per thread otherwise.  (rows + 1) / 2 <= 65535 is the caller's.
+template <int ACT>
+void launch_gated_norm_rows(const GdnDeltaParams& p, hipStream_t s) {
+    const uint64_t units = (uint64_t)p.sh.batch * p.sh.rows * p.sh.v_heads;
+    if (p.sh.dv == 128 && units < (1ull << 31) && aligned16(p.out) && p.out_stride % 8 == 0 && aligned16(p.z) &&
+        p.z_stride % 8 == 0 && aligned16(p.norm_w)) {
+        gdn_gated_norm_rows128_kernel<ACT><<<dim3((uint32_t)((units + 15) / 16)), 256, 0, s>>>(
+            p.out, p.out_stride, p.z, p.z_stride, p.norm_w, p.sh, (uint32_t)units);
+        return;
+    }
+    const dim3 ngrid(p.sh.v_heads, p.sh.batch, (p.sh.rows + 1) / 2);
+    gdn_gated_norm_rows_kernel<ACT><<<ngrid, 256, 0, s>>>(p.out, p.out_stride, p.z, p.z_stride, p.norm_w, p.sh);
+}
+
 template <int ACT, int DK, int DV>
 bool launch_delta_chunked(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
     if (DK != 128 || DV != 128) return false;
@@ -44,8 +59,7 @@ bool launch_delta_chunked(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool stat
     const dim3 cgrid(p.sh.v_heads, p.sh.batch, 128 / 16);
     if (state_bf16) gdn_chunk_delta_kernel<ACT, 128, 128, true><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
     else gdn_chunk_delta_kernel<ACT, 128, 128, false><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
-    const dim3 ngrid(p.sh.v_heads, p.sh.batch, (p.sh.rows + 1) / 2);
-    gdn_gated_norm_rows_kernel<ACT><<<ngrid, 256, 0, s>>>(p.out, p.out_stride, p.z, p.z_stride, p.norm_w, p.sh);
+    launch_gated_norm_rows<ACT>(p, s);
     return true;
 }
 
@@ -57,8 +71,7 @@ void launch_delta(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, 
         const dim3 rgrid(p.sh.v_heads, p.sh.batch, DV / 16);      // one group of sixteen state rows per block
         if (state_bf16) gdn_delta_rows_kernel<ACT, DK, DV, true, 1><<<rgrid, 256, 0, s>>>(p);
         else gdn_delta_rows_kernel<ACT, DK, DV, false, 1><<<rgrid, 256, 0, s>>>(p);
-        const dim3 ngrid(p.sh.v_heads, p.sh.batch, (p.sh.rows + 1) / 2);
-        gdn_gated_norm_rows_kernel<ACT><<<ngrid, 256, 0, s>>>(p.out, p.out_stride, p.z, p.z_stride, p.norm_w, p.sh);
+        launch_gated_norm_rows<ACT>(p, s);
         return;
     }
     if (state_bf16) gdn_delta_gated_kernel<ACT, DK, DV, true><<<grid, 256, 0, s>>>(p);

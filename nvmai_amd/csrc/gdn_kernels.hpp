@@ -322,6 +322,46 @@ __global__ __launch_bounds__(256) void gdn_gated_norm_rows_kernel(uint16_t* out,
     out[row * out_stride + h * sh.dv + i] = f32_to_act<ACT>(normed * gate);
 }
 
+// The same for heads of 128 values in 16-byte pieces: sixteen lanes per (row, head), eight values per
+// lane, sixteen (row, head) units per block, no barrier and no LDS.  The sum of squares is the balanced
+// tree of the kernel above -- pairs, fours and eights inside the lane, then the lanes 1, 2, 4 and 8
+// apart, where the kernel above goes on to its second wave -- so the result has the same bits.
+// out, z and norm_w rows 16-byte aligned.
+template <int ACT>
+__global__ __launch_bounds__(256) void gdn_gated_norm_rows128_kernel(uint16_t* out, uint32_t out_stride, const uint16_t* z,
+                                                                    uint32_t z_stride, const uint16_t* norm_w, GdnShape sh,
+                                                                    uint32_t units) {
+    const uint32_t u = blockIdx.x * 16u + (threadIdx.x >> 4), sub = threadIdx.x & 15u;
+    const bool live = u < units;
+    const uint32_t uu = live ? u : units - 1u;             // every lane takes part in the sum
+    const uint32_t h = uu % sh.v_heads;
+    const size_t row = uu / sh.v_heads;                    // batch * rows + t
+    uint16_t* const op = out + row * out_stride + h * 128u + sub * 8u;
+    const uint4 yr = *reinterpret_cast<const uint4*>(op);
+    const uint4 zr = *reinterpret_cast<const uint4*>(z + row * z_stride + h * 128u + sub * 8u);
+    const uint4 wr = *reinterpret_cast<const uint4*>(norm_w + sub * 8u);
+    float y[8], g[8], w[8], q[8];
+    act2_to_f32<ACT>(yr.x, y[0], y[1]); act2_to_f32<ACT>(yr.y, y[2], y[3]);
+    act2_to_f32<ACT>(yr.z, y[4], y[5]); act2_to_f32<ACT>(yr.w, y[6], y[7]);
+    act2_to_f32<ACT>(zr.x, g[0], g[1]); act2_to_f32<ACT>(zr.y, g[2], g[3]);
+    act2_to_f32<ACT>(zr.z, g[4], g[5]); act2_to_f32<ACT>(zr.w, g[6], g[7]);
+    act2_to_f32<ACT_BF16>(wr.x, w[0], w[1]); act2_to_f32<ACT_BF16>(wr.y, w[2], w[3]);
+    act2_to_f32<ACT_BF16>(wr.z, w[4], w[5]); act2_to_f32<ACT_BF16>(wr.w, w[6], w[7]);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) q[j] = fmaf(y[j], y[j], 0.0f);
+    const float lane_sum = ((q[0] + q[1]) + (q[2] + q[3])) + ((q[4] + q[5]) + (q[6] + q[7]));
+    const float total = seg_reduce_sum<16>(lane_sum) + (0.0f + 0.0f);
+    const float inv = rsqrtf(total / (float)sh.dv + GDN_RMS_EPS);
+    uint32_t r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lo = y[2 * j] * inv * w[2 * j] * gdn_silu(g[2 * j]);
+        const float hi = y[2 * j + 1] * inv * w[2 * j + 1] * gdn_silu(g[2 * j + 1]);
+        r[j] = (uint32_t)f32_to_act<ACT>(lo) | ((uint32_t)f32_to_act<ACT>(hi) << 16);
+    }
+    if (live) *reinterpret_cast<uint4*>(op) = uint4{r[0], r[1], r[2], r[3]};
+}
+
 // The recurrence alone over the rows of a call: S, and y[t] = S q rounded to 16 bits into out (the
 // kernel above norms it).  A row costs a few hundred cycles of arithmetic and a trip to memory costs
 // several times that, so the rows arrive a tile of 32 at a time: all 256 threads fetch the next

@@ -195,6 +195,14 @@ int expert_ffn_dense(nvmai_hip_ctx* ctx, hipStream_t s, const uint8_t* blob, con
         if (bits == 4) launch_gemms<ACT_FP16, 4, 4>(g1, g2, tiles, ctx, s);
         else launch_gemms<ACT_FP16, 8, 2>(g1, g2, tiles, ctx, s);
     }
+    if (d % 8 == 0 && y_stride % 8 == 0 && aligned16(tmp) && aligned16(y)) {       // sixteen bytes per thread
+        dim3 grid8((d / 8 + 255) / 256, tokens);
+        if (ctx->act == ACT_BF16)
+            gate_rows8_kernel<ACT_BF16><<<grid8, 256, 0, s>>>((const uint16_t*)tmp, gate_logit, (uint16_t*)y, tokens, d, y_stride);
+        else
+            gate_rows8_kernel<ACT_FP16><<<grid8, 256, 0, s>>>((const uint16_t*)tmp, gate_logit, (uint16_t*)y, tokens, d, y_stride);
+        return launch_status();
+    }
     dim3 grid((d + 255) / 256, tokens);
     if (ctx->act == ACT_BF16)
         gate_rows_kernel<ACT_BF16><<<grid, 256, 0, s>>>((const uint16_t*)tmp, gate_logit, (uint16_t*)y, tokens, d, y_stride);

@@ -1352,6 +1352,27 @@ __global__ __launch_bounds__(256) void gate_rows_kernel(const uint16_t* rows, co
     y[(size_t)t * y_stride + c] = f32_to_act<ACT>(v);
 }
 
+// The same, eight values (16 bytes) per thread: d a multiple of 8, rows and y rows 16-byte aligned.
+template <int ACT>
+__global__ __launch_bounds__(256) void gate_rows8_kernel(const uint16_t* rows, const float* gate_logit, uint16_t* y,
+                                                        uint32_t tokens, uint32_t d, uint32_t y_stride) {
+    const uint32_t t = blockIdx.y, c = (blockIdx.x * 256 + threadIdx.x) * 8u;
+    if (c >= d) return;
+    const uint4 v = *reinterpret_cast<const uint4*>(rows + (size_t)t * d + c);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    float den = 1.0f;
+    if (gate_logit) den = __fadd_rn(1.0f, expf(-gate_logit[t]));
+    uint32_t r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float lo, hi;
+        act2_to_f32<ACT>(w[j], lo, hi);
+        if (gate_logit) { lo = __fdiv_rn(lo, den); hi = __fdiv_rn(hi, den); }
+        r[j] = (uint32_t)f32_to_act<ACT>(lo) | ((uint32_t)f32_to_act<ACT>(hi) << 16);
+    }
+    *reinterpret_cast<uint4*>(y + (size_t)t * y_stride + c) = uint4{r[0], r[1], r[2], r[3]};
+}
+
 // ---- combine (prefill.metal:437-458) -------------------------------------------------------
 // h2[t, d] = sum over ranks in rank order of fma(w[t, r], partial[t, r, d], acc).  VEC = 8:
 // sixteen bytes of a row per thread (rows 16-byte aligned); VEC = 2: any even d.

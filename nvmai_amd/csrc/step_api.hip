@@ -180,8 +180,16 @@ template <int OP>
 int run_elementwise(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* a, const void* b, void* out, uint32_t count) {
     if (!ctx || !a || !b || !out) return NVMAI_ERR_INVALID_ARG;
     if (count == 0) return NVMAI_OK;
-    const dim3 grid((count + 255) / 256);
     hipStream_t s = (hipStream_t)stream;
+    if (count >= 4096 && count % 8 == 0 && aligned16(a) && aligned16(out) && (OP == EW_SIGMOID_SCALAR || aligned16(b))) {
+        const dim3 grid8((count / 8 + 255) / 256);       // sixteen bytes per thread, the same arithmetic per value
+        if (ctx->act == ACT_BF16)
+            elementwise8_kernel<ACT_BF16, OP><<<grid8, 256, 0, s>>>((const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, count / 8);
+        else
+            elementwise8_kernel<ACT_FP16, OP><<<grid8, 256, 0, s>>>((const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, count / 8);
+        return launch_status();
+    }
+    const dim3 grid((count + 255) / 256);
     if (ctx->act == ACT_BF16)
         elementwise_kernel<ACT_BF16, OP><<<grid, 256, 0, s>>>((const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, count);
     else

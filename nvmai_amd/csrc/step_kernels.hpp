@@ -394,6 +394,36 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const uint16_t* a, con
     out[i] = f32_to_act<ACT>(r);
 }
 
+// The same, eight values (16 bytes) per thread: a, b and out 16-byte aligned, count a multiple of 8.
+template <int ACT, int OP>
+__global__ __launch_bounds__(256) void elementwise8_kernel(const uint16_t* a, const uint16_t* b, uint16_t* out,
+                                                           uint32_t count8) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= count8) return;
+    const uint4 av = reinterpret_cast<const uint4*>(a)[i];
+    uint4 bv = uint4{0, 0, 0, 0};
+    if (OP != EW_SIGMOID_SCALAR) bv = reinterpret_cast<const uint4*>(b)[i];
+    const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
+    float scalar = 0.0f;
+    if (OP == EW_SIGMOID_SCALAR) scalar = act_to_f32<ACT>(b[0]);
+    uint32_t r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float x[2], y[2], o[2];
+        act2_to_f32<ACT>(aw[j], x[0], x[1]);
+        act2_to_f32<ACT>(bw[j], y[0], y[1]);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if (OP == EW_SILU_MUL) o[h] = __fmul_rn(__fdiv_rn(x[h], __fadd_rn(1.0f, expf(-x[h]))), y[h]);
+            else if (OP == EW_ADD) o[h] = __fadd_rn(x[h], y[h]);
+            else if (OP == EW_SIGMOID_SCALAR) o[h] = __fdiv_rn(x[h], __fadd_rn(1.0f, expf(-scalar)));
+            else o[h] = __fdiv_rn(x[h], __fadd_rn(1.0f, expf(-y[h])));
+        }
+        r[j] = (uint32_t)f32_to_act<ACT>(o[0]) | ((uint32_t)f32_to_act<ACT>(o[1]) << 16);
+    }
+    reinterpret_cast<uint4*>(out)[i] = uint4{r[0], r[1], r[2], r[3]};
+}
+
 // split (JOIN = false): packed [rows, 2 dim] -> lo [rows, dim], hi [rows, dim]   (split_q_gate_fp16, :75-92)
 // join  (JOIN = true):  lo, hi [rows, dim]   -> packed [rows, 2 dim]             (concat_rows_fp16, :107-121)
 template <bool JOIN>

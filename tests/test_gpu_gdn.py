@@ -168,6 +168,33 @@ def test_gdn_long_call_on_the_matrix_cores_batch_and_state_types(nv, ctx, bf16_s
     assert (state_a.float() - state_b.float()).abs().max().item() <= (5e-2 if not bf16_state else 1e-1)
 
 
+@pytest.mark.parametrize("rows", [8, 37, 80])
+def test_gdn_gated_norm_in_16_byte_pieces_same_bits(nv, ctx, rows):
+    # heads of 128 values take the gated output norm in 16-byte pieces, sixteen lanes per (row, head);
+    # z rows at a stride that is not a multiple of 16 bytes take the one-value-per-thread kernel:
+    # the same rows through both must give the same bits (rows below and above the chunked form)
+    say("gdn gated norm pieces", ctx.act, rows)
+    cfg, batch = (2, 4, 128, 128, 4), 2
+    fxs = [_fixture(cfg, rows, 900 + b, ctx.act) for b in range(batch)]
+    w = fxs[0]
+    gdn = nv.GDN(ctx, *cfg)
+    cat = lambda key: act_tensor(np.concatenate([fx[key] for fx in fxs]), ctx)
+    outs = []
+    for pad in (0, 4):
+        tail, state = gdn.new_state(batch)
+        conv = gdn.encode_conv_norm(cat("qkv"), tail, _bits(w["conv_w"]), rows=rows)
+        z = cat("z")
+        if pad:
+            wide = torch.zeros((z.shape[0], z.shape[1] + pad), dtype=z.dtype, device=z.device)
+            wide[:, :z.shape[1]] = z
+            z = wide[:, :z.shape[1]]
+            assert z.stride(0) % 8 != 0
+        outs.append(gdn.encode_delta_gated_norm(conv, cat("a"), cat("b"), _bits(w["a_log"]), _bits(w["dt_bias"]), state, z,
+                                                _bits(w["norm_w"]), rows=rows))
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_gdn_full_size_prompt_is_the_same_in_one_call_or_in_pieces(nv, ctx):
     # the production layer (16 key / 32 value heads of 128 x 128, four taps) over 4096 rows, the size of a
     # configs[4] prompt chunk: one call against calls of 1000 rows (ragged pieces, a last one of 96) and

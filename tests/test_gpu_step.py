@@ -221,6 +221,37 @@ def test_elementwise_helpers_match_oracle(nv, ctx):
     assert nv.lib.nvmai_hip_silu_mul(ctx.handle, None, None, None, None, 4) == -1
 
 
+def test_elementwise_helpers_in_16_byte_pieces_same_bits(nv, ctx):
+    # 4096 values and more in 16-byte-aligned buffers go eight per thread; the same values in buffers
+    # that start two bytes later take the one-value-per-thread kernels: same bits from both
+    say("elementwise pieces", ctx.act)
+    rng = np.random.default_rng(78)
+    n = 8192
+    a = round_act(gauss(rng, (n,), 3.0), ctx.act)
+    b = round_act(gauss(rng, (n,), 3.0), ctx.act)
+    ew = nv.Elementwise(ctx)
+
+    def shifted(x):                       # the same values, first element two bytes past a 16-byte boundary
+        t = torch.zeros(n + 8, dtype=ctx.dtype, device="cuda")
+        t[1:n + 1] = act_tensor(x, ctx)
+        return t[1:n + 1]
+
+    for op in ("silu", "gate", "scalar", "add"):
+        outs = []
+        for make in (lambda x: act_tensor(x, ctx).clone(), shifted):
+            ta, tb = make(a), make(b)
+            if op == "silu":
+                outs.append(ew.encode_silu_mul(ta, tb, out=make(a)))
+            elif op == "gate":
+                outs.append(ew.encode_sigmoid_gate_mul(ta, tb))
+            elif op == "scalar":
+                outs.append(ew.encode_sigmoid_scalar_mul(ta, tb[:1]))
+            else:
+                outs.append(ew.encode_residual_add(ta, tb))
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1]), op
+
+
 # ------------------------------------------------------------------ q / k / v epilogue
 def _qkv_epilogue_case(nv, ctx, rng, tokens, nq, nkv, hd, rot, pad):
     span = 2 * nq * hd + 2 * nkv * hd
