@@ -346,6 +346,20 @@ void run_router_t(const RouterParams& rp, uint32_t cpl, dim3 grid, hipStream_t s
 template <int ACT>
 void run_router_tiled(const RouterParams& rp, const RowsDesc& r, uint32_t n_rows, float* out, uint32_t out_ld,
                       hipStream_t s) {
+    const uint32_t cpl = (rows_chunks(r.kind, rp.d) + 31) / 32;
+    if (n_rows == 1 && rp.x_vec && cpl <= 8) {      // one row (the shared expert's gate): a half-wave per token, no staging
+        const dim3 sgrid((rp.tokens + 7) / 8);
+#define NVMAI_SINGLE(KIND)                                                                        \
+        do {                                                                                      \
+            if (cpl <= 4) router_single_row_kernel<ACT, KIND, 4><<<sgrid, 256, 0, s>>>(rp, r, out, out_ld); \
+            else router_single_row_kernel<ACT, KIND, 8><<<sgrid, 256, 0, s>>>(rp, r, out, out_ld);         \
+        } while (0)
+        if (r.kind == 16) NVMAI_SINGLE(16);
+        else if (r.kind == 8) NVMAI_SINGLE(8);
+        else NVMAI_SINGLE(4);
+#undef NVMAI_SINGLE
+        return;
+    }
     const size_t lds = (size_t)RT_TOK * rp.d * 2;
     const uint32_t per_block = 8 * (r.kind == 4 ? 2 : 4);
     dim3 grid((n_rows + per_block - 1) / per_block, (rp.tokens + RT_TOK - 1) / RT_TOK);

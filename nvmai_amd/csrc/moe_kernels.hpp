@@ -997,6 +997,65 @@ __global__ __launch_bounds__(256, KIND == 16 ? 4 : 2) void router_logits_tiled_k
         }
 }
 
+// One row (the shared expert's gate row) against many tokens: a half-wave per token, its inputs read
+// straight from memory (16 bytes per lane and load; nothing is shared between tokens but the one row,
+// which every half-wave reads from cache), all of a lane's loads requested before the first sum.  The
+// same sums in the same order as the kernels above, so the same bits.  Rows of x 16-byte aligned.
+template <int ACT, int KIND, int CPL>
+__global__ __launch_bounds__(256) void router_single_row_kernel(RouterParams p, RowsDesc r, float* out, uint32_t out_ld) {
+    constexpr int EPC = KIND == 16 ? 8 : (KIND == 8 ? 16 : 32);
+    constexpr int XV = EPC / 8;
+    const int hw = threadIdx.x >> 5, hl = threadIdx.x & 31;
+    const uint32_t t = blockIdx.x * 8 + hw;
+    if (t >= p.tokens) return;                       // uniform per half-wave
+    const uint32_t chunks = p.d / EPC;
+    const uint16_t* xrow = (const uint16_t*)p.x + (size_t)t * p.x_stride;
+    uint4 wv[CPL], xraw[CPL][XV];
+    uint16_t sv[CPL], bv[CPL];
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) {
+        const uint32_t c = min((uint32_t)hl + 32u * i, chunks - 1u);      // past the end: the last chunk again, unused
+        wv[i] = *reinterpret_cast<const uint4*>((const uint8_t*)r.w + (size_t)c * 16);
+#pragma unroll
+        for (int v = 0; v < XV; ++v) xraw[i][v] = *reinterpret_cast<const uint4*>(xrow + c * EPC + 8 * v);
+        if (KIND != 16) {
+            sv[i] = r.s[c * EPC / NVMAI_GROUP];
+            bv[i] = r.b[c * EPC / NVMAI_GROUP];
+        }
+    }
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) {
+        const uint32_t c = hl + 32u * i;
+        if (c < chunks) {
+            float q[EPC], xv[EPC];
+            if (KIND == 16) {
+                act2_to_f32<ACT_BF16>(wv[i].x, q[0], q[1]); act2_to_f32<ACT_BF16>(wv[i].y, q[2], q[3]);
+                act2_to_f32<ACT_BF16>(wv[i].z, q[4], q[5]); act2_to_f32<ACT_BF16>(wv[i].w, q[6], q[7]);
+            } else {
+                unpack_chunk<KIND == 16 ? 8 : KIND>(wv[i], q);
+            }
+            router_x_from_raw<ACT, EPC>(p, xraw[i], c * EPC, xv);
+            if (KIND == 16) {
+#pragma unroll
+                for (int j = 0; j < EPC; ++j) acc = fmaf(q[j], xv[j], acc);
+            } else {
+                float dot = 0.0f, xs = 0.0f;
+#pragma unroll
+                for (int j = 0; j < EPC; ++j) {
+                    dot = fmaf(q[j], xv[j], dot);
+                    xs = __fadd_rn(xs, xv[j]);
+                }
+                acc = fmaf(bf16_to_f32(sv[i]), dot, acc);
+                acc = fmaf(bf16_to_f32(bv[i]), xs, acc);
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 16; off >= 1; off >>= 1) acc = __fadd_rn(acc, shfl_xor_f(acc, off));
+    if (hl == 0) out[(size_t)t * out_ld] = acc;
+}
+
 // ---- top-k select + softmax over the selected ------------------------------------
 // One wave per token.  Selection equals a stable sort by (score desc, index asc)
 // (moe.metal:233-285).  Weights: ex_i = exp(s_i - s_0), sum in slot order,

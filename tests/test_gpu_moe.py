@@ -234,7 +234,9 @@ def test_router_indices_and_logits_bit_exact(nv, ctx, kind):
 def test_router_many_tokens_same_bits(nv, ctx, kind):
     # 64 tokens and more take the register-tiled kernel: same sums in the same order, so the same bits
     rng = np.random.default_rng(100 + kind)
-    for E, D, tokens, k in [(256, 2048, 150, 8), (100, 512, 70, 4), (20, 192, 64, 8), (33, 2048, 97, 2)]:
+    # (one row: the form the shared expert's gate row takes, a half-wave per token)
+    for E, D, tokens, k in [(256, 2048, 150, 8), (100, 512, 70, 4), (20, 192, 64, 8), (33, 2048, 97, 2),
+                            (1, 2048, 131, 1), (1, 512, 64, 1), (1, 4096, 70, 1)]:
         say("router tiled", ctx.act, kind, E, D, tokens, k)
         _router_case(nv, ctx, kind, E, D, tokens, k, rng)
     say("router tiled scales", kind)
