@@ -898,7 +898,8 @@ __global__ __launch_bounds__(256, KIND == 16 ? 4 : 2) void router_logits_tiled_k
                                                                   float* out, uint32_t out_ld) {
     constexpr int EPC = KIND == 16 ? 8 : (KIND == 8 ? 16 : 32);
     constexpr int XV = EPC / 8;
-    constexpr int R = KIND == 4 ? 2 : 4;             // rows per half-wave: what the register file holds
+    constexpr int R = KIND == 4 ? 2 : 4;             // rows per half-wave: what the register file holds at four blocks per CU
+                                                     // (eight BF16 rows, 174 registers, two blocks: 117 against 91 us at 4096 tokens)
     extern __shared__ uint4 router_lds[];
     const uint16_t* xl = reinterpret_cast<const uint16_t*>(router_lds);
     const int hw = threadIdx.x >> 5, hl = threadIdx.x & 31;
