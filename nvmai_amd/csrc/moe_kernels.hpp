@@ -906,11 +906,29 @@ __global__ __launch_bounds__(256, KIND == 16 ? 4 : 2) void router_logits_tiled_k
     const uint32_t row0 = (blockIdx.x * 8 + hw) * R;
     const uint32_t t0 = blockIdx.y * RT_TOK;
     const uint32_t nt = min((uint32_t)RT_TOK, p.tokens - t0);
-    router_stage_x(p, t0, nt, reinterpret_cast<uint16_t*>(router_lds));
-    if (row0 >= n_rows) return;                      // uniform per half-wave
     const uint32_t chunks = p.d / EPC;
     const uint32_t groups = p.d / NVMAI_GROUP;
     const size_t row_bytes = (size_t)p.d * KIND / 8;
+    // the rows' chunks one iteration ahead of their use (the first ones while the inputs are staged):
+    // rows past the end repeat the last one, chunks past the end the lane's last one, both unused
+    uint4 wnext[R];
+    uint16_t snext[R], bnext[R];
+    auto fetch_rows = [&](uint32_t c) {
+        const uint32_t cc = min(c, chunks - 1u);
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const uint32_t row = min(row0 + i, n_rows - 1);
+            wnext[i] = *reinterpret_cast<const uint4*>((const uint8_t*)r.w + row * row_bytes + (size_t)cc * 16);
+            if (KIND != 16) {
+                const uint32_t g = cc * EPC / NVMAI_GROUP;
+                snext[i] = r.s[(size_t)row * groups + g];
+                bnext[i] = r.b[(size_t)row * groups + g];
+            }
+        }
+    };
+    fetch_rows(hl);
+    router_stage_x(p, t0, nt, reinterpret_cast<uint16_t*>(router_lds));
+    if (row0 >= n_rows) return;                      // uniform per half-wave
     float acc[R][RT_TOK];
 #pragma unroll
     for (int i = 0; i < R; ++i)
@@ -921,18 +939,17 @@ __global__ __launch_bounds__(256, KIND == 16 ? 4 : 2) void router_logits_tiled_k
         float q[R][EPC], sc[R], bi[R];
 #pragma unroll
         for (int i = 0; i < R; ++i) {
-            const uint32_t row = min(row0 + i, n_rows - 1);     // rows past the end repeat the last one, unstored
-            const uint4 w = *reinterpret_cast<const uint4*>((const uint8_t*)r.w + row * row_bytes + (size_t)c * 16);
+            const uint4 w = wnext[i];
             if (KIND == 16) {
                 act2_to_f32<ACT_BF16>(w.x, q[i][0], q[i][1]); act2_to_f32<ACT_BF16>(w.y, q[i][2], q[i][3]);
                 act2_to_f32<ACT_BF16>(w.z, q[i][4], q[i][5]); act2_to_f32<ACT_BF16>(w.w, q[i][6], q[i][7]);
             } else {
                 unpack_chunk<KIND == 16 ? 8 : KIND>(w, q[i]);
-                const uint32_t g = c * EPC / NVMAI_GROUP;
-                sc[i] = bf16_to_f32(r.s[(size_t)row * groups + g]);
-                bi[i] = bf16_to_f32(r.b[(size_t)row * groups + g]);
+                sc[i] = bf16_to_f32(snext[i]);
+                bi[i] = bf16_to_f32(bnext[i]);
             }
         }
+        fetch_rows(c + 32);
         float eff[EFF ? EPC : 1];
         if (EFF) {
 #pragma unroll
