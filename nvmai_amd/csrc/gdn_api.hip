@@ -104,7 +104,7 @@ extern "C" int nvmai_hip_gdn_conv_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, 
     const dim3 grid(2 * sh.k_heads + sh.v_heads, batch);
     hipStream_t s = (hipStream_t)stream;
     if (rows >= GDN_ROWS_PARALLEL_FROM && sh.dk <= 128 && sh.dv <= 128 && (rows + 1) / 2 <= 65535) {
-        // a chunk of rows: sixteen rows of a head segment per block, then the tail in a launch of its own
+        // a chunk of rows: thirty-two rows of a head segment per block, then the tail in a launch of its own
         const dim3 rgrid(2 * sh.k_heads + sh.v_heads, batch, (rows + GDN_CONV_ROWS_PER_BLOCK - 1) / GDN_CONV_ROWS_PER_BLOCK);
         if (ctx->act == ACT_BF16)
             gdn_conv_norm_rows_kernel<ACT_BF16><<<rgrid, 256, 0, s>>>((const uint16_t*)qkv_raw, qkv_stride, (const uint16_t*)tail,

@@ -199,25 +199,27 @@ __global__ __launch_bounds__(256) void gdn_delta_gated_kernel(GdnDeltaParams p) 
 // The conv of row t reads the raw rows t - K + 1 .. t only, and the gated output norm of row t reads
 // y[t] only: with many rows per call (a prefill chunk) both run with a pair of waves per (row,
 // head segment) instead of inside the sequential loops above, which leaves the recurrence itself --
-// S and the rows it produces -- as the only sequential part.  Channel i of a segment sits on lane
-// i % 64 of the pair's wave i / 64 and the two wave sums are added first, as in the kernels above:
-// the same bits.  Segments of at most 128 channels.
+// S and the rows it produces -- as the only sequential part.  The sum of squares over a segment is
+// taken as in the kernels above -- channels 0..63 over the lanes of a wave, channels 64..127 the same
+// way, the two sums added first: the same bits.  Segments of at most 128 channels.
 
 // conv + SiLU + q / k norm of rows [0, rows) of every sequence; the tail is read, not written.
-// A block takes sixteen rows of one segment, eight consecutive rows per pair of waves: a thread keeps
-// the window of its channel in registers, so a row costs it one two-byte load instead of one per tap.
-constexpr uint32_t GDN_CONV_ROWS_PER_BLOCK = 16;
+// A wave takes eight consecutive rows of one segment, channels lane and 64 + lane (a block four such
+// groups of rows): a thread keeps the windows of its two channels in registers, so a row costs it two
+// two-byte loads instead of one per tap, all sixteen in flight together, and the two halves of the sum
+// of squares are the wave's own two sums -- no barrier, no LDS, and nothing orders the rows of a wave,
+// so their exponentials and divisions overlap.
+constexpr uint32_t GDN_CONV_ROWS_PER_BLOCK = 32;
 
 template <int ACT>
 __global__ __launch_bounds__(256) void gdn_conv_norm_rows_kernel(const uint16_t* qkv_raw, uint32_t qkv_stride,
                                                                 const uint16_t* tail, const uint16_t* conv_w,
                                                                 uint16_t* conv_out, uint32_t out_stride, GdnShape sh) {
-    constexpr uint32_t RPP = GDN_CONV_ROWS_PER_BLOCK / 2;                   // rows per pair of waves
-    __shared__ float part[2][4];
+    constexpr uint32_t RPW = GDN_CONV_ROWS_PER_BLOCK / 4;                   // rows per wave
     const uint32_t seg = blockIdx.x, b = blockIdx.y;
-    const uint32_t pair = threadIdx.x >> 7, i = threadIdx.x & 127u;         // half of the block, channel of the segment
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const uint32_t t_first = blockIdx.z * GDN_CONV_ROWS_PER_BLOCK + pair * RPP;
+    const uint32_t t_first = blockIdx.z * GDN_CONV_ROWS_PER_BLOCK + wave * RPW;
+    if (t_first >= sh.rows) return;                                         // uniform per wave; no barrier below
     const uint32_t C = 2 * sh.k_heads * sh.dk + sh.v_heads * sh.dv;
     const bool is_qk = seg < 2 * sh.k_heads;
     const uint32_t seg_len = is_qk ? sh.dk : sh.dv;
@@ -225,52 +227,70 @@ __global__ __launch_bounds__(256) void gdn_conv_norm_rows_kernel(const uint16_t*
     const uint32_t hist = sh.taps - 1;
     const uint16_t* tl = tail + (size_t)b * hist * C;
     const uint16_t* raw = qkv_raw + (size_t)b * sh.rows * qkv_stride;
-    const bool ch_live = i < seg_len;
-    const uint32_t ch = base + (ch_live ? i : 0u);
-    auto value_at = [&](int src) -> float {                  // row src of [old tail | rows]
-        return act_to_f32<ACT>(src >= 0 ? raw[(size_t)src * qkv_stride + ch] : tl[(size_t)((int)hist + src) * C + ch]);
-    };
-    float wt[GDN_MAX_TAPS], pre[GDN_MAX_TAPS];               // weights; the hist values before the current row
+    bool ch_live[2];
+    uint32_t ch[2];
 #pragma unroll
-    for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
-        wt[j] = 0.0f; pre[j] = 0.0f;
-        if (j < sh.taps) wt[j] = bf16_to_f32(conv_w[ch * sh.taps + j]);
-        if (j < hist && t_first < sh.rows) pre[j] = value_at((int)t_first - (int)hist + (int)j);
+    for (int h = 0; h < 2; ++h) {
+        ch_live[h] = lane + 64u * h < seg_len;
+        ch[h] = base + (ch_live[h] ? lane + 64u * h : 0u);
     }
+    float wt[2][GDN_MAX_TAPS], pre[2][GDN_MAX_TAPS];         // weights; the hist values before the current row
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+            wt[h][j] = 0.0f; pre[h][j] = 0.0f;
+            if (j < sh.taps) wt[h][j] = bf16_to_f32(conv_w[ch[h] * sh.taps + j]);
+            if (j < hist) {
+                const int src = (int)t_first - (int)hist + (int)j;       // row src of [old tail | rows]
+                pre[h][j] = act_to_f32<ACT>(src >= 0 ? raw[(size_t)src * qkv_stride + ch[h]]
+                                                     : tl[(size_t)((int)hist + src) * C + ch[h]]);
+            }
+        }
+    // rows past the end read the last row again and are not used
+    uint16_t curv[2][RPW];
+#pragma unroll
+    for (uint32_t k = 0; k < RPW; ++k)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) curv[h][k] = raw[(size_t)min(t_first + k, sh.rows - 1u) * qkv_stride + ch[h]];
     const float scale = seg < sh.k_heads ? 1.0f / (float)sh.dk : rsqrtf((float)sh.dk);
-    for (uint32_t k = 0; k < RPP; ++k) {
+#pragma unroll
+    for (uint32_t k = 0; k < RPW; ++k) {
         const uint32_t t = t_first + k;
-        const bool live = t < sh.rows && ch_live;
-        float x = 0.0f;
-        uint16_t r = 0;
-        if (t < sh.rows) {
-            const float cur = value_at((int)t);
+        if (t >= sh.rows) break;                             // uniform
+        float x[2];
+        uint16_t r[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float cur = act_to_f32<ACT>(curv[h][k]);
             float acc = 0.0f;
 #pragma unroll
             for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
                 if (j >= sh.taps) break;
-                acc = fmaf(j < hist ? pre[j] : cur, wt[j], acc);
+                acc = fmaf(j < hist ? pre[h][j] : cur, wt[h][j], acc);
             }
 #pragma unroll
-            for (uint32_t j = 0; j + 1 < GDN_MAX_TAPS; ++j) pre[j] = j + 1 < hist ? pre[j + 1] : cur;
-            if (live) {
-                r = f32_to_act<ACT>(gdn_silu(acc));
-                x = act_to_f32<ACT>(r);
+            for (uint32_t j = 0; j + 1 < GDN_MAX_TAPS; ++j) pre[h][j] = j + 1 < hist ? pre[h][j + 1] : cur;
+            r[h] = 0;
+            x[h] = 0.0f;
+            if (ch_live[h]) {
+                r[h] = f32_to_act<ACT>(gdn_silu(acc));
+                x[h] = act_to_f32<ACT>(r[h]);
             }
         }
-        uint16_t* o = conv_out + ((size_t)b * sh.rows + t) * out_stride + ch;
+        uint16_t* o = conv_out + ((size_t)b * sh.rows + t) * out_stride;
         if (!is_qk) {                                         // block-uniform
-            if (live) *o = r;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                if (ch_live[h]) o[ch[h]] = r[h];
             continue;
         }
-        const float ws = wave_sum_bcast(x * x);
-        if (lane == 0) part[k & 1u][wave] = ws;
-        __syncthreads();
-        if (live) {
-            const float total = (part[k & 1u][2 * pair] + part[k & 1u][2 * pair + 1]) + (0.0f + 0.0f);
-            const float inv = rsqrtf(total / (float)sh.dk + GDN_RMS_EPS);
-            *o = f32_to_act<ACT>(x * inv * scale);
-        }
+        const float s0 = wave_sum_bcast(x[0] * x[0]), s1 = wave_sum_bcast(x[1] * x[1]);
+        const float total = (s0 + s1) + (0.0f + 0.0f);
+        const float inv = rsqrtf(total / (float)sh.dk + GDN_RMS_EPS);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            if (ch_live[h]) o[ch[h]] = f32_to_act<ACT>(x[h] * inv * scale);
     }
 }
 
