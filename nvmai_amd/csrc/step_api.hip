@@ -101,8 +101,11 @@ int qkv_epilogue_impl(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* proj,
     p.positions = positions; p.position0 = position; p.theta = theta; p.eps = eps;
     const dim3 grid((num_q_heads + 2 * num_kv_heads + 3) / 4, tokens);
     hipStream_t s = (hipStream_t)stream;
-    if (ctx->act == ACT_BF16) qkv_epilogue_kernel<ACT_BF16><<<grid, 256, 0, s>>>(p);
-    else qkv_epilogue_kernel<ACT_FP16><<<grid, 256, 0, s>>>(p);
+    if (head_dim == 256) {          // the production head: loops unrolled, a pass's loads in flight together
+        if (ctx->act == ACT_BF16) qkv_epilogue_kernel<ACT_BF16, 256><<<grid, 256, 0, s>>>(p);
+        else qkv_epilogue_kernel<ACT_FP16, 256><<<grid, 256, 0, s>>>(p);
+    } else if (ctx->act == ACT_BF16) qkv_epilogue_kernel<ACT_BF16, 0><<<grid, 256, 0, s>>>(p);
+    else qkv_epilogue_kernel<ACT_FP16, 0><<<grid, 256, 0, s>>>(p);
     return launch_status();
 }
 }  // namespace

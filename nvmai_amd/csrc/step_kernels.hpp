@@ -200,14 +200,16 @@ struct QkvEpilogueParams {
     uint32_t kv_bits, kv_row_stride, kv_value_bytes;
 };
 
-template <int ACT>
+template <int ACT, int HD>
 __global__ __launch_bounds__(256) void qkv_epilogue_kernel(QkvEpilogueParams p) {
+    // HD: the head size when it is known at compile time (0 = any, read from p): the loops over a
+    // head's elements then unroll, and a lane's loads of a pass are in flight together
     __shared__ uint16_t head_s[4][512];
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const uint32_t heads = p.num_q_heads + 2 * p.num_kv_heads;
     const uint32_t hidx = blockIdx.x * 4 + wave, token = blockIdx.y;
     if (hidx >= heads) return;                              // wave-uniform; no block-wide barrier below
-    const uint32_t hd = p.head_dim;
+    const uint32_t hd = HD ? (uint32_t)HD : p.head_dim;
     const bool is_q = hidx < p.num_q_heads, is_k = !is_q && hidx < p.num_q_heads + p.num_kv_heads;
     const uint32_t q_span = p.q_packed ? 2 * hd : hd;
     const uint16_t* src;
@@ -221,6 +223,7 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(QkvEpilogueParams p) 
         w = p.q_weight;
         if (p.q_packed) {
             uint16_t* g = p.gate_out + ((size_t)token * p.num_q_heads + hidx) * hd;
+#pragma unroll
             for (uint32_t i = lane; i < hd; i += 64) g[i] = src[hd + i];
         }
     } else {
@@ -237,23 +240,27 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(QkvEpilogueParams p) 
     const bool norm = is_q || is_k || p.v_norm;
     if (norm) {
         float acc = 0.0f;
+#pragma unroll
         for (uint32_t i = lane; i < hd; i += 64) {
             const float v = act_to_f32<ACT>(src[i]);
             acc = fmaf(v, v, acc);
         }
         const float inv = rms_inverse(rms_wave_sum(acc), hd, p.eps);
+#pragma unroll
         for (uint32_t i = lane; i < hd; i += 64) {
             float v = __fmul_rn(act_to_f32<ACT>(src[i]), inv);
             if (w) v = __fmul_rn(v, bf16_to_f32(w[i]));
             hs[i] = f32_to_act<ACT>(v);
         }
     } else {
+#pragma unroll
         for (uint32_t i = lane; i < hd; i += 64) hs[i] = src[i];
     }
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_s_waitcnt(0xC07F);                      // lgkmcnt(0): this wave's LDS writes have landed
     const uint32_t half_rot = (is_q || is_k) ? p.rotary_dim / 2 : 0;
     const uint32_t pos = p.positions ? p.positions[token] : p.position0;
+#pragma unroll
     for (uint32_t i = lane; i < hd; i += 64) {
         uint16_t o = hs[i];
         if (i < 2 * half_rot) {
