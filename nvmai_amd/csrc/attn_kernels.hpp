@@ -255,13 +255,24 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     const uint32_t dim = blockIdx.y * 64 + lane;
     uint16_t* out_row = (uint16_t*)p.out + (bh / p.num_q_heads) * p.out_stride + (bh % p.num_q_heads) * p.head_dim;
     const uint16_t* gate_row = p.gate ? p.gate + (bh / p.num_q_heads) * p.gate_stride + (bh % p.num_q_heads) * p.head_dim : nullptr;
+    // everything the block reads besides the partial rows is requested at once: a thread's (at most
+    // two) chunk maxima and sums, and the gate value of its output element
+    uint16_t gate_v = 0;
+    if (gate_row && dim < p.head_dim) gate_v = gate_row[dim];
+    float mv[2], dv[2];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+        const uint32_t c = threadIdx.x + 256u * s2, cc = min(c, p.num_chunks - 1u);
+        const float m_c = mr[cc], d_c = dr[cc];
+        mv[s2] = c < p.num_chunks ? m_c : -INFINITY;
+        dv[s2] = c < p.num_chunks ? d_c : 0.0f;
+    }
     auto gated = [&](float v) -> uint16_t {
         uint16_t o = f32_to_act<ACT>(v);
-        if (gate_row) o = f32_to_act<ACT>(__fdiv_rn(act_to_f32<ACT>(o), __fadd_rn(1.0f, expf(-act_to_f32<ACT>(gate_row[dim])))));
+        if (gate_row) o = f32_to_act<ACT>(__fdiv_rn(act_to_f32<ACT>(o), __fadd_rn(1.0f, expf(-act_to_f32<ACT>(gate_v)))));
         return o;
     };
-    float mloc = -INFINITY;
-    for (uint32_t c = threadIdx.x; c < p.num_chunks; c += 256) mloc = fmaxf(mloc, mr[c]);
+    float mloc = fmaxf(fmaxf(-INFINITY, mv[0]), mv[1]);
     mloc = wave_max_f32(mloc);
     if (lane == 0) red[wave] = mloc;
     __syncthreads();
@@ -271,10 +282,14 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
         return;
     }
     float dloc = 0.0f;
-    for (uint32_t c = threadIdx.x; c < p.num_chunks; c += 256) {
-        const float w = expf(mr[c] - mg);
-        wgt[c] = w;
-        dloc += dr[c] * w;
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+        const uint32_t c = threadIdx.x + 256u * s2;
+        if (c < p.num_chunks) {
+            const float w = expf(mv[s2] - mg);
+            wgt[c] = w;
+            dloc += dv[s2] * w;
+        }
     }
     dloc = wave_sum_bcast(dloc);
     if (lane == 0) red[4 + wave] = dloc;
@@ -283,7 +298,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     float acc = 0.0f;
     if (dim < p.head_dim) {
         const float* oc = orow + dim;
-#pragma unroll 8
+#pragma unroll 16
         for (uint32_t c = wave; c < p.num_chunks; c += 4) acc += oc[(size_t)c * p.head_dim] * wgt[c];
     }
     part[wave][lane] = acc;
