@@ -74,6 +74,11 @@ void launch_delta(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, 
         launch_gated_norm_rows<ACT>(p, s);
         return;
     }
+    if (DK == 128 && DV == 128 && aligned16(p.state)) {       // the production head, state rows in 16-byte pieces
+        if (state_bf16) gdn_delta_gated_kernel<ACT, DK, DV, true, DK == 128><<<grid, 256, 0, s>>>(p);
+        else gdn_delta_gated_kernel<ACT, DK, DV, false, DK == 128><<<grid, 256, 0, s>>>(p);
+        return;
+    }
     if (state_bf16) gdn_delta_gated_kernel<ACT, DK, DV, true><<<grid, 256, 0, s>>>(p);
     else gdn_delta_gated_kernel<ACT, DK, DV, false><<<grid, 256, 0, s>>>(p);
 }

@@ -124,11 +124,13 @@ struct GdnDeltaParams {
     GdnShape sh;
 };
 
-template <int ACT, int DK, int DV, bool STATE_BF16>
+// VEC: the state is 16-byte aligned and DK = 128 (a lane's eight values of a state row are one or two
+// 16-byte loads and stores); the host chooses.
+template <int ACT, int DK, int DV, bool STATE_BF16, bool VEC = false>
 __global__ __launch_bounds__(256) void gdn_delta_gated_kernel(GdnDeltaParams p) {
     constexpr int EPL = DK / 16;                // state elements per lane
     constexpr int GROUPS = DV / 16;             // sixteen rows per block pass
-    static_assert(DK % 16 == 0 && DV % 16 == 0 && EPL >= 1 && EPL <= 16, "shape");
+    static_assert(DK % 16 == 0 && DV % 16 == 0 && DV <= 256 && EPL >= 1 && EPL <= 16, "shape");
     __shared__ float y_s[DV];
     __shared__ float part[4];
     const uint32_t h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
@@ -139,14 +141,33 @@ __global__ __launch_bounds__(256) void gdn_delta_gated_kernel(GdnDeltaParams p) 
     const float dtb = bf16_to_f32(p.dt_bias[h]);
     const size_t state_base = (((size_t)b * sh.v_heads + h) * DV) * DK;
     float s[GROUPS][EPL];
+    static_assert(!VEC || EPL == 8, "VEC needs eight state values per lane");
+    constexpr bool vec = VEC;
 #pragma unroll
     for (int g = 0; g < GROUPS; ++g) {
         const size_t at = state_base + (size_t)(g * 16 + row_in_pass) * DK + sub * EPL;
+        if (EPL == 8 && vec) {
+            if (STATE_BF16) {
+                const uint4 r = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.state) + at);
+                act2_to_f32<ACT_BF16>(r.x, s[g][0], s[g][1 % EPL]); act2_to_f32<ACT_BF16>(r.y, s[g][2 % EPL], s[g][3 % EPL]);
+                act2_to_f32<ACT_BF16>(r.z, s[g][4 % EPL], s[g][5 % EPL]); act2_to_f32<ACT_BF16>(r.w, s[g][6 % EPL], s[g][7 % EPL]);
+            } else {
+                const float4 r0 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.state) + at);
+                const float4 r1 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.state) + at + 4);
+                s[g][0] = r0.x; s[g][1 % EPL] = r0.y; s[g][2 % EPL] = r0.z; s[g][3 % EPL] = r0.w;
+                s[g][4 % EPL] = r1.x; s[g][5 % EPL] = r1.y; s[g][6 % EPL] = r1.z; s[g][7 % EPL] = r1.w;
+            }
+        } else {
 #pragma unroll
-        for (int e = 0; e < EPL; ++e)
-            s[g][e] = STATE_BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(p.state)[at + e])
-                                 : reinterpret_cast<const float*>(p.state)[at + e];
+            for (int e = 0; e < EPL; ++e)
+                s[g][e] = STATE_BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(p.state)[at + e])
+                                     : reinterpret_cast<const float*>(p.state)[at + e];
+        }
     }
+    // the norm weight of this thread's output element (threads past DV read the last one: a load under a
+    // condition would be waited for on the spot, and every load in flight with it)
+    const uint32_t oi = min(tid, (uint32_t)DV - 1u);
+    const uint16_t nw_raw = p.norm_w[oi];
     for (uint32_t t = 0; t < sh.rows; ++t) {
         const size_t row = (size_t)b * sh.rows + t;
         const uint16_t* cq = p.conv_out + row * p.conv_stride + hk * DK + sub * EPL;
@@ -155,6 +176,7 @@ __global__ __launch_bounds__(256) void gdn_delta_gated_kernel(GdnDeltaParams p) 
         float q[EPL], k[EPL];
 #pragma unroll
         for (int e = 0; e < EPL; ++e) { q[e] = act_to_f32<ACT>(cq[e]); k[e] = act_to_f32<ACT>(ck[e]); }
+        const uint16_t z_raw = p.z[row * p.z_stride + h * DV + oi];      // requested with the row's operands, used after the barrier
         const float g_decay = expf(-exp_a * gdn_softplus(act_to_f32<ACT>(p.a_proj[row * p.ab_stride + h]) + dtb));
         const float beta = 1.0f / (1.0f + expf(-act_to_f32<ACT>(p.b_proj[row * p.ab_stride + h])));
 #pragma unroll
@@ -176,16 +198,31 @@ __global__ __launch_bounds__(256) void gdn_delta_gated_kernel(GdnDeltaParams p) 
         for (uint32_t i = tid; i < DV; i += 256) sumsq = fmaf(y_s[i], y_s[i], sumsq);
         const float total = gdn_block_sum(sumsq, part);
         const float inv = rsqrtf(total / (float)DV + GDN_RMS_EPS);
-        for (uint32_t i = tid; i < DV; i += 256) {
-            const float normed = y_s[i] * inv * bf16_to_f32(p.norm_w[i]);
-            const float gate = gdn_silu(act_to_f32<ACT>(p.z[row * p.z_stride + h * DV + i]));
-            p.out[row * p.out_stride + h * DV + i] = f32_to_act<ACT>(normed * gate);
+        if (tid < DV) {                                     // DV <= 256: one element per thread
+            const float normed = y_s[tid] * inv * bf16_to_f32(nw_raw);
+            const float gate = gdn_silu(act_to_f32<ACT>(z_raw));
+            p.out[row * p.out_stride + h * DV + tid] = f32_to_act<ACT>(normed * gate);
         }
         __syncthreads();                                    // y_s is rewritten by the next row
     }
 #pragma unroll
     for (int g = 0; g < GROUPS; ++g) {
         const size_t at = state_base + (size_t)(g * 16 + row_in_pass) * DK + sub * EPL;
+        if (EPL == 8 && vec) {
+            if (STATE_BF16) {
+                uint4 r;
+                r.x = (uint32_t)f32_to_bf16(s[g][0]) | ((uint32_t)f32_to_bf16(s[g][1 % EPL]) << 16);
+                r.y = (uint32_t)f32_to_bf16(s[g][2 % EPL]) | ((uint32_t)f32_to_bf16(s[g][3 % EPL]) << 16);
+                r.z = (uint32_t)f32_to_bf16(s[g][4 % EPL]) | ((uint32_t)f32_to_bf16(s[g][5 % EPL]) << 16);
+                r.w = (uint32_t)f32_to_bf16(s[g][6 % EPL]) | ((uint32_t)f32_to_bf16(s[g][7 % EPL]) << 16);
+                *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(p.state) + at) = r;
+            } else {
+                *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.state) + at) = float4{s[g][0], s[g][1 % EPL], s[g][2 % EPL], s[g][3 % EPL]};
+                *reinterpret_cast<float4*>(reinterpret_cast<float*>(p.state) + at + 4) =
+                    float4{s[g][4 % EPL], s[g][5 % EPL], s[g][6 % EPL], s[g][7 % EPL]};
+            }
+            continue;
+        }
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
             if (STATE_BF16) reinterpret_cast<uint16_t*>(p.state)[at + e] = f32_to_bf16(s[g][e]);
