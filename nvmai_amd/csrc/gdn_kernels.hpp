@@ -58,13 +58,22 @@ __global__ __launch_bounds__(256) void gdn_conv_norm_kernel(const uint16_t* qkv_
         float sumsq = 0.0f;
         for (uint32_t i = tid; i < seg_len; i += 256) {
             const uint32_t ch = base + i;
-            float acc = 0.0f;
-            for (uint32_t j = 0; j < sh.taps; ++j) {
+            // every tap's input and weight requested before the first product: the address is chosen, not
+            // the load (a load under a condition is waited for on the spot); taps past the last reread it
+            uint16_t vv[GDN_MAX_TAPS], ww[GDN_MAX_TAPS];
+#pragma unroll
+            for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
+                const uint32_t jj = min(j, hist);
                 // input row in the virtual sequence [tail rows | chunk rows]
-                const int src = (int)t + (int)j - (int)hist;
-                const uint16_t v = src >= 0 ? raw[(size_t)src * qkv_stride + ch] : tl[(size_t)((int)hist + src) * C + ch];
-                acc = fmaf(act_to_f32<ACT>(v), bf16_to_f32(conv_w[ch * sh.taps + j]), acc);
+                const int src = (int)t + (int)jj - (int)hist;
+                const uint16_t* at = src >= 0 ? raw + (size_t)src * qkv_stride + ch : tl + (size_t)((int)hist + src) * C + ch;
+                vv[j] = *at;
+                ww[j] = conv_w[ch * sh.taps + jj];
             }
+            float acc = 0.0f;
+#pragma unroll
+            for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j)
+                if (j < sh.taps) acc = fmaf(act_to_f32<ACT>(vv[j]), bf16_to_f32(ww[j]), acc);
             const uint16_t r = f32_to_act<ACT>(gdn_silu(acc));
             out[(size_t)t * out_stride + ch] = r;
             const float x = act_to_f32<ACT>(r);
@@ -87,7 +96,8 @@ __global__ __launch_bounds__(256) void gdn_conv_norm_kernel(const uint16_t* qkv_
         for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
             if (j >= hist) break;
             const int src = (int)sh.rows + (int)j - (int)hist;
-            keep[j] = src >= 0 ? raw[(size_t)src * qkv_stride + ch] : tl[(size_t)((int)hist + src) * C + ch];
+            const uint16_t* at = src >= 0 ? raw + (size_t)src * qkv_stride + ch : tl + (size_t)((int)hist + src) * C + ch;
+            keep[j] = *at;
         }
 #pragma unroll
         for (uint32_t j = 0; j < GDN_MAX_TAPS; ++j) {
