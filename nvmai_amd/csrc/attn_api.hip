@@ -112,7 +112,12 @@ int run_attention(nvmai_hip_ctx* ctx, nvmai_stream stream, AttnParams p, const n
     // Chunking: enough blocks to fill the device, chunks a multiple of the 32-token step.
     const uint64_t units = fast ? (uint64_t)seq_blocks * p.num_kv_heads : (uint64_t)p.batch * p.num_q_heads;
     const uint32_t len = max_len;
-    uint32_t nc = units >= 512 ? 1 : (uint32_t)((512 + units - 1) / units);
+    // blocks aimed at: two per compute unit, except the 8-bit matrix-core kernel, which is bound by bytes
+    // and does better with one block per unit and half the partial rows to write and merge (32K x 1:
+    // 20.2 -> 17.8 us, 128K x 1: 40.9 -> 35.1, 32K x 8: 62.2 -> 58.3; the 4-bit kernel, bound by its vector
+    // work, loses with one: 128K x 8 136 -> 165 us)
+    const uint32_t tgt = (fast && k->bits == 8) ? 256u : 512u;
+    uint32_t nc = units >= tgt ? 1 : (uint32_t)((tgt + units - 1) / units);
     const uint32_t max_nc = (len + 127) / 128 ? (len + 127) / 128 : 1;
     if (nc > max_nc) nc = max_nc;
     if (nc < 1) nc = 1;
