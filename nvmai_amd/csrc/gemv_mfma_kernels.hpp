@@ -94,11 +94,11 @@ __global__ __launch_bounds__(64 * NW) void gemv_mfma_kernel(GemvMfmaParams p) {
     const uint32_t row0 = blockIdx.x * (16 * WR) + wave_r * 16;
     const uint32_t groups = p.n / 64, row_bytes = p.n * BITS / 8;
     const uint32_t n_stages = p.n / GM_STAGE_CODES;
-    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t*>(p.w), 0, (int)(p.m * row_bytes), 0x00020000);
-    const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc(
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.s), 0, (int)(p.m * groups * 2), 0x00020000);
-    const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(p.b), 0, (int)(p.m * groups * 2), 0x00020000);
 
     // ---- weight stages: lane l of load j fetches chunk (l % CPR) ^ row of row j RPI + l / CPR,
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_mfma_kernel(GemvMfmaParams p) {
     // scales / biases of a stage: 16 rows x 16 bytes, one dword per lane (every lane takes part:
     // a load under a lane mask would sit in a block of its own, and the compiler then loses track of
     // which LDS array the loads in flight write)
-    const uint32_t meta_off = (min(row0 + (uint32_t)lane / 4u, p.m - 1) * groups) * 2u + ((uint32_t)lane % 4u) * 4u;
+    [[maybe_unused]] const uint32_t meta_off = (min(row0 + (uint32_t)lane / 4u, p.m - 1) * groups) * 2u + ((uint32_t)lane % 4u) * 4u;
     uint8_t* const wa_w = wa + wave * WREG;
     uint8_t* const wb_w = wb + wave * WREG;
     uint8_t* const ma_w = ma + wave * 512;
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(64 * NW) void gemv_mfma_kernel(GemvMfmaParams p) {
         // (read like the codes below, with instructions the compiler does not track)
         gm_u4_t sc4[4], bi4[4];
         {
-            const uint32_t maddr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)msrc + r * 64;
+            [[maybe_unused]] const uint32_t maddr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const uint8_t*)msrc + r * 64;
 #if defined(__HIP_DEVICE_COMPILE__)
             asm volatile(
                 "ds_read_b128 %0, %8\n ds_read_b128 %1, %8 offset:16\n ds_read_b128 %2, %8 offset:32\n ds_read_b128 %3, %8 offset:48\n"

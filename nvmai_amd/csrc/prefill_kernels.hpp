@@ -896,7 +896,7 @@ __global__ __launch_bounds__(256, 2) void prefill_gemm_kernel(GemmParams p) {
     // the fetching lanes' dwords of one super-step -> this lane's (scale, bias) per tile, packed:
     // scale in the high half, bias in the low half.  The cross-lane reads carry the tile in their
     // immediate offset, so one address register serves all of them.
-    const uint32_t bp_addr = 4u * li;
+    [[maybe_unused]] const uint32_t bp_addr = 4u * li;
     auto scales_from = [&](uint32_t s_dw, uint32_t b_dw, uint32_t ss, uint32_t* sb) {
         const bool dead = odd_tail && ss == nss - 1 && lq >= 2;
         uint32_t ds[4], db[4];
