@@ -1373,8 +1373,9 @@ __global__ __launch_bounds__(256) void combine_postnorm_kernel(CombineParams p, 
     extern __shared__ __attribute__((aligned(16))) uint16_t post_raw[];
     const uint32_t t = blockIdx.x, per_row = p.d / 8, lane = threadIdx.x & 63;
     uint4 v[ROUTER_PRE_PIECES], wv[ROUTER_PRE_PIECES];
-    float gate = 1.0f;
-    if (p.has_shared && p.gate_logit) gate = __fadd_rn(1.0f, expf(-p.gate_logit[t]));
+    // the gate logit is requested like every other input, unconditionally (a load under a condition is
+    // waited for on the spot, ahead of everything after it); without a gate the word read is not used
+    const float gate_in = *(p.has_shared && p.gate_logit ? p.gate_logit + t : p.partials);
 #pragma unroll
     for (int k = 0; k < ROUTER_PRE_PIECES; ++k) {
         const uint32_t c = threadIdx.x + 256 * k;
@@ -1394,6 +1395,7 @@ __global__ __launch_bounds__(256) void combine_postnorm_kernel(CombineParams p, 
         v[k] = *reinterpret_cast<const uint4*>(a.hidden + (size_t)t * a.hidden_stride + c * 8);
         wv[k] = *reinterpret_cast<const uint4*>(a.weight + c * 8);
         if (p.has_shared) {
+            const float gate = __fadd_rn(1.0f, expf(-gate_in));
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float s = p.gate_logit ? __fdiv_rn(sh[j], gate) : sh[j];
@@ -1403,11 +1405,10 @@ __global__ __launch_bounds__(256) void combine_postnorm_kernel(CombineParams p, 
         for (uint32_t r0 = 0; r0 < p.top_k; r0 += 8) {
             float pr[8][8], w[8];
 #pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                if (r0 + r < p.top_k) {
-                    w[r] = f16_to_f32(p.w[(size_t)t * p.top_k + r0 + r]);
-                    row8((size_t)t * p.top_k + r0 + r, pr[r]);
-                }
+            for (int r = 0; r < 8; ++r) {          // slots past the last reread it and are not used
+                const uint32_t rr = min(r0 + r, p.top_k - 1u);
+                w[r] = f16_to_f32(p.w[(size_t)t * p.top_k + rr]);
+                row8((size_t)t * p.top_k + rr, pr[r]);
             }
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
