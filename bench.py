@@ -22,6 +22,8 @@ import numpy as np
 D, F, E, K = 2048, 512, 256, 8
 HBM_PEAK_GBPS = 8000.0
 METRIC = "4/8-bit MoE expert GEMV GB/s (% HBM peak); prefill grouped-GEMM TFLOPS"
+RAMP_STEPS = 200       # untimed steps ahead of the --warmup steps of the decode workload: a fresh device takes a few
+                       # milliseconds of work to reach its clock, and --steps 20 of this workload are under 3 ms
 
 
 def parse():
@@ -99,7 +101,7 @@ def run_config(nv, ctx, torch, layers, stride, bits, batch, steps, warmup, profi
     xs = torch.empty((n_x, batch, D), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
     y = torch.empty((batch, D), dtype=torch.bfloat16, device="cuda")
     stats = torch.zeros((steps, 2), dtype=torch.int32, device="cuda")
-    for i in range(warmup):
+    for i in range(RAMP_STEPS + warmup):                    # untimed: the clock ramp, then the warm-up steps asked for
         moe.decode_layer(layers[i % len(layers)]["desc"], xs[i % n_x], y)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -154,13 +156,12 @@ def cpu_baseline(layers, stride, bits, batch, torch):
                                    threads, warmup=1, reps=reps)
         algo = step_bytes(len(np.unique(idx)), n, stride)
         rows[name] = dict(value=round(algo / dt / 1e9, 3), unit="GB/s", cores=threads,
-                          sample="%d tokens of one %d-bit layer, median of %d repetitions of %.3f s; %.1f MB "
-                                 "algorithmic (each distinct expert once), %.1f MB touched by the per-pair path"
+                          sample="%d tokens, one %d-bit layer, median of %d x %.3f s; %.0f MB algorithmic, %.0f MB touched per pair"
                                  % (n, bits, reps, dt, algo / 1e6, (n * (K + 1) * stride + n * E * D * 2) / 1e6))
     out = dict(rows["all_cores"])
     out.update(kind="port", cpu_model=model, build="oracle/nvmai_oracle.c, gcc " + flags,
-               one_thread=rows["one_thread"])
-    out["sample"] = "oracle orc_moe_layer_forward, " + out["sample"]
+               one_thread_value=rows["one_thread"]["value"], one_thread_sample=rows["one_thread"]["sample"])
+    out["sample"] = "orc_moe_layer_forward, " + out["sample"]
     return out
 
 
@@ -823,17 +824,16 @@ def main():
     print(json.dumps(line), flush=True)
 
 
-def compact(line):
-    """The figures of a full line that the `extra` object keeps."""
+def compact(line, **more):
+    """One cell of the `extra` object: value, unit, ms per step, and the roofline kernel's launch time, rate and
+    fraction of its peak (GB/s against 8 TB/s, or TFLOP/s against 2.5 PFLOP/s); the key names the cell."""
     r = line["roofline"]
-    out = {"workload": line["config"]["workload"], "value": line["value"], "unit": line["unit"],
-           "ms_per_step": line["ms_per_step"],
-           "roofline": {k: r[k] for k in ("kernel", "bound", "achieved", "peak", "unit", "frac", "avg_launch_us")}}
-    for k in ("batch_tokens", "mean_distinct_experts", "tokens_per_s", "frac_of_hbm_peak"):
+    out = {"v": line["value"], "u": line["unit"], "ms": line["ms_per_step"], "kern_us": r["avg_launch_us"],
+           "kern": r["achieved"], "frac": r["frac"]}
+    for k in ("mean_distinct_experts", "frac_of_hbm_peak"):
         if k in line["config"]:
             out[k] = line["config"][k]
-    if line.get("parity_check"):
-        out["parity_check"] = line["parity_check"]
+    out.update(more)
     return out
 
 
@@ -842,10 +842,9 @@ def decode_line(a, r, bits, batch, steps, warmup):
         "metric": METRIC, "value": round(r["gbps"], 2), "unit": "GB/s", "n_gpus": 1, "steps": steps,
         "warmup": warmup, "ms_per_step": round(r["ms_per_step"], 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "u%d codes, f32 accumulate" % bits, "data": "synthetic",
-        "config": {"workload": "configs[1]: one MoE-layer decode step, %d-bit group-64 experts, hidden 2048, "
-                               "256 experts top-8 + gated shared expert, intermediate 512, bf16 activations, "
-                               "all experts resident in HBM" % bits,
-                   "batch_tokens": batch, "layers_rotated": a.layers,
+        "config": {"workload": "configs[1]: MoE-layer decode step, %d-bit g64 experts, 256 top-8 + gated shared, D 2048, F 512, "
+                               "all in HBM" % bits,
+                   "batch_tokens": batch, "layers_rotated": a.layers, "untimed_clock_ramp_steps": RAMP_STEPS,
                    "mean_distinct_experts": round(r["mean_distinct"], 2),
                    "frac_of_hbm_peak": round(r["gbps"] / HBM_PEAK_GBPS, 4),
                    "kernel_us": {k: round(v, 2) for k, v in r["kernel_us"].items()}},
@@ -860,54 +859,120 @@ def decode_line(a, r, bits, batch, steps, warmup):
     }
 
 
+def run_config0(nv, ctx, torch, layers4, stride4, a):
+    """BASELINE configs[0]: ONE 4-bit expert (SwiGLU MLP, 512 x 2048 gate and up, 2048 x 512 down), one token,
+    through the shared-expert operator without a gate (the single-expert FFN of CPUExpertFFN.accumulate).  Every
+    call takes another expert of the 40 x 257 resident ones, so the 1.78 MB come from HBM.  At 8 TB/s the bytes
+    of one call are 0.22 us of traffic, less than a launch: the figure is a latency, stated as such."""
+    import oracle as O
+    off, _ = nv.expert_offsets(D, F, 4)
+    run = nv.SharedExpertRuntime(ctx, 4)
+    gen = torch.Generator(device="cuda").manual_seed(404)
+    xs = torch.empty((64, 1, D), dtype=torch.bfloat16, device="cuda").normal_(0.0, 1.0, generator=gen)
+    y = torch.empty((1, D), dtype=torch.bfloat16, device="cuda")
+    blob_of = lambda i: layers4[i % len(layers4)]["pool"][(i * 37) % (E + 1)]
+    call = lambda i: run.encode(blob_of(i), off, xs[i % 64], D, F, shared_gate=None, y=y)
+    steps, warm = 400, 20
+    for i in range(warm):
+        call(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        call(warm + i)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    ev[0].record()
+    for i in range(steps):
+        call(i)
+    ev[1].record()
+    torch.cuda.synchronize()
+    ev_us = ev[0].elapsed_time(ev[1]) / steps * 1e3
+    lat = []
+    for i in range(20):                                     # one call alone: submit to completion, host clock
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        call(1000 + i)
+        torch.cuda.synchronize()
+        lat.append(time.perf_counter() - t0)
+    i = 1019
+    want = np.zeros(D, np.float32)
+    O.expert_ffn_accumulate(blob_of(i).cpu().numpy(), 4, xs[i % 64, 0].float().cpu().numpy(), D, F, 1.0, want)
+    rel = float(O.rel_error(y[0].float().cpu().numpy(), want))
+    assert rel < 1e-2, "configs[0] expert differs from the oracle: max-rel %g" % rel
+    nbytes = stride4 + 2 * D * 2
+    out = {"v": round(nbytes / dt / 1e9, 1), "u": "GB/s", "ms": round(dt * 1e3, 5), "kern_us": round(ev_us, 2),
+           "frac": round(nbytes / dt / 1e9 / HBM_PEAK_GBPS, 4), "bytes_per_call": nbytes,
+           "single_call_latency_us": round(float(np.median(lat)) * 1e6, 1), "launches_per_call": 2, "max_rel": round(rel, 6)}
+    if not a.no_cpu:
+        blobs = layers4[0]["pool"][:64].cpu().numpy()
+        x0 = xs[0, 0].float().cpu().numpy()
+        t_ref, _ = O.time_expert_ffn(blobs, D, F, x0, reps=41, reference=True)
+        t_port, _ = O.time_expert_ffn(blobs, D, F, x0, reps=41, reference=False)
+        row = lambda t, kind, what: {"value": round(nbytes / t / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": kind,
+                                     "ms_per_expert": round(t * 1e3, 4), "sample": what}
+        out["cpu_baseline"] = [
+            row(t_ref, "reference", "the reference's nvmai_int4_affine_gemv (oracle/_ref, gcc -O2) x3 + silu in numpy, "
+                                    "41 experts, median") if t_ref else None,
+            row(t_port, "port", "oracle orc_expert_ffn_accumulate (gcc -O3 -march=native), 41 experts, median")]
+    return out
+
+
 def extra_cells(nv, ctx, torch, a, layers8, stride8):
-    """The other cells of the metric, each measured like its own --workload line but shorter:
-    4-bit decode at batch 32, 8-bit decode at one token, the configs[2] prefill grouped GEMM, and
-    configs[4] (the full 40-layer decode step, tok/s at batch 1 and 16, and its prompt side: 4096 tokens
-    through the same layers with the prefill kernels), and every cell of configs[3]
-    (attention at 4K / 32K / 128K context x batch 1 / 8 with 8- and 4-bit KV, each checked against the
-    oracle before it is reported)."""
+    """The other cells of the metric, each measured like its own --workload line but shorter and printed in
+    compact form (the key names the cell; v = value, u = unit, ms = per step, kern_us / kern / frac = the
+    roofline kernel's launch time, rate and fraction of its peak).  The twelve cells of configs[3] come first as
+    one table, the metric's own cells last: configs[0], the configs[2] prefill grouped GEMM, 4-bit decode at batch
+    32, 8-bit decode at one token, configs[4] at batch 1 and 16."""
     import argparse
     out = {}
-    r = run_config(nv, ctx, torch, layers8, stride8, 8, 1, 200, 20, profile=True)
-    out["decode_8bit_batch1"] = compact(decode_line(a, r, 8, 1, 200, 20))
-    layers4, stride4 = build_layers(nv, ctx, torch, 4, a.layers)
-    torch.cuda.synchronize()
-    r = run_config(nv, ctx, torch, layers4, stride4, 4, 32, 200, 20, profile=True)
-    out["decode_4bit_batch32"] = compact(decode_line(a, r, 4, 32, 200, 20))
-    del layers4
-    torch.cuda.empty_cache()
-    sub = argparse.Namespace(**vars(a))
-    sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.tokens = True, 30, 5, 4, 4096
-    out["prefill_4bit_4096tokens"] = compact(run_prefill(nv, ctx, torch, sub))
-    torch.cuda.empty_cache()
-    for batch in (1, 16):
-        sub = argparse.Namespace(**vars(a))
-        sub.no_cpu, sub.steps, sub.warmup, sub.batch, sub.context = True, 30, 3, batch, 32768
-        cell = run_step(nv, ctx, torch, sub)
-        c = compact(cell)
-        c["bytes_per_token_MB"] = cell["config"]["bytes_per_token_MB"]
-        c["roofline_tok_per_s_at_8TBps"] = cell["config"]["roofline_tok_per_s_at_8TBps"]
-        out["decode_step_configs4_batch%d" % batch] = c
-        torch.cuda.empty_cache()
-    sub = argparse.Namespace(**vars(a))
-    sub.no_cpu, sub.steps, sub.warmup, sub.tokens, sub.chunk = True, 2, 1, 4096, 4096
-    cell = run_prefill_step(nv, ctx, torch, sub)
-    c = compact(cell)
-    c["model_gflop_per_token"] = cell["config"]["model_gflop_per_token"]
-    out["prefill_step_configs4_4096tokens"] = c
-    torch.cuda.empty_cache()
-    for bits in (8, 4):
-        sub = argparse.Namespace(**vars(a))
-        sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.tokens, sub.context_given = True, 20, 3, bits, 4096, False
-        out["prefill_attention_%dbit_4096tokens" % bits] = compact(run_prefill_attention(nv, ctx, torch, sub))
-        torch.cuda.empty_cache()
+    rows = []
     for bits in (8, 4):
         for context, batch in ((131072, 8), (131072, 1), (32768, 8), (32768, 1), (4096, 8), (4096, 1)):
             sub = argparse.Namespace(**vars(a))
             sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.context, sub.batch = True, 30, 5, bits, context, batch
-            out["attention_%dbit_%dk_batch%d" % (bits, context // 1024, batch)] = compact(run_attention(nv, ctx, torch, sub))
+            c = run_attention(nv, ctx, torch, sub)
+            r = c["roofline"]
+            rows.append([bits, context // 1024, batch, c["value"], c["config"]["frac_of_hbm_peak"], r["avg_launch_us"],
+                         r["frac"], c["parity_check"]["max_rel"]])
             torch.cuda.empty_cache()
+    out["attention_configs3"] = {"cols": ["kv_bits", "ctx_k", "batch", "GB/s", "frac", "kern_us", "kern_frac", "max_rel_vs_oracle"],
+                                 "rows": rows}
+    for bits in (8, 4):
+        sub = argparse.Namespace(**vars(a))
+        sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.tokens, sub.context_given = True, 20, 3, bits, 4096, False
+        c = run_prefill_attention(nv, ctx, torch, sub)
+        out["prefill_attention_%dbit_4096tokens" % bits] = compact(c, max_rel=c["parity_check"]["max_rel"])
+        torch.cuda.empty_cache()
+    sub = argparse.Namespace(**vars(a))
+    sub.no_cpu, sub.steps, sub.warmup, sub.tokens, sub.chunk = True, 2, 1, 4096, 4096
+    cell = run_prefill_step(nv, ctx, torch, sub)
+    out["prefill_step_configs4_4096tokens"] = compact(cell, model_gflop_per_token=cell["config"]["model_gflop_per_token"])
+    torch.cuda.empty_cache()
+    layers4, stride4 = build_layers(nv, ctx, torch, 4, a.layers)
+    torch.cuda.synchronize()
+    out["configs0_4bit_one_expert_one_token"] = run_config0(nv, ctx, torch, layers4, stride4, a)
+    sub = argparse.Namespace(**vars(a))
+    sub.no_cpu, sub.steps, sub.warmup, sub.bits, sub.tokens = True, 30, 5, 4, 4096
+    c = run_prefill(nv, ctx, torch, sub)
+    out["prefill_4bit_4096tokens"] = compact(c, kernel_us=c["config"]["kernel_us"], tokens_per_s=c["config"]["tokens_per_s"])
+    torch.cuda.empty_cache()
+    r = run_config(nv, ctx, torch, layers4, stride4, 4, 32, 200, 20, profile=True)
+    c = decode_line(a, r, 4, 32, 200, 20)
+    out["decode_4bit_batch32"] = compact(c, kernel_us=c["config"]["kernel_us"])
+    del layers4
+    torch.cuda.empty_cache()
+    r = run_config(nv, ctx, torch, layers8, stride8, 8, 1, 200, 20, profile=True)
+    c = decode_line(a, r, 8, 1, 200, 20)
+    out["decode_8bit_batch1"] = compact(c, kernel_us=c["config"]["kernel_us"])
+    for batch in (1, 16):
+        sub = argparse.Namespace(**vars(a))
+        sub.no_cpu, sub.steps, sub.warmup, sub.batch, sub.context = True, 30, 3, batch, 32768
+        cell = run_step(nv, ctx, torch, sub)
+        out["decode_step_configs4_batch%d" % batch] = compact(
+            cell, bytes_per_token_MB=cell["config"]["bytes_per_token_MB"],
+            roofline_tok_per_s_at_8TBps=cell["config"]["roofline_tok_per_s_at_8TBps"])
+        torch.cuda.empty_cache()
     return out
 
 

@@ -661,60 +661,146 @@ class GTurboModel:
         ranks = [e.physicalRank for e in lay.experts]
         return data if ranks == list(range(len(ranks))) else data[ranks]
 
+    def shared_matches_routed(self):
+        """Whether the shared expert has the routed experts' bit width and group size, so that its
+        arrays fit the routed sub-tensor regions and it can sit in the pool as one more expert.  The
+        reference keeps the two in separate quant slots (Model.swift:59-60; validateLayerTensors checks
+        the shared projections against quant.sharedExpert), and its repacker's default profile writes
+        an 8-bit shared expert beside 4-bit routed experts (RemoteStreamingRepacker.swift:678-683)."""
+        q = self.manifest.quant
+        return (q["sharedExpert"].weightBits == q["routedExpert"].weightBits and
+                q["sharedExpert"].groupSize == q["routedExpert"].groupSize)
+
+    def shared_expert_offsets(self, layer):
+        """(nine offsets, blob bytes, bits) of the shared expert's blob: the layer's routed-expert
+        offsets when the widths agree, else CPUExpertFFN.Offsets(d:f:) at the shared expert's own
+        width (CPUExpertFFN.swift:42-59)."""
+        a, q = self.manifest.arch, self.manifest.quant
+        bits, group = q["sharedExpert"].weightBits, q["sharedExpert"].groupSize
+        if bits not in (4, 8) or group != 64:
+            raise ModelError("unsupportedArch", "shared expert quantization %d-bit group %d (this build runs 4 / 8-bit, group 64)"
+                             % (bits, group))
+        if self.shared_matches_routed():
+            return routed_expert_offsets(self.layout, layer), self.layout.expertStride, bits
+        d, f = a["hiddenSize"], a["moeIntermediateSize"]
+        sizes = [f * d * bits // 8, f * (d // 64) * 2, f * (d // 64) * 2] * 2 + [d * f * bits // 8, d * (f // 64) * 2, d * (f // 64) * 2]
+        off, at = [], 0
+        for n in sizes:
+            off.append(at)
+            at += n
+        return tuple(off), at, bits
+
     def shared_expert_blob(self, layer):
-        """The shared expert's nine arrays gathered from the resident file into one blob with the
-        layer's routed-expert offsets, so that it can sit in the pool as one more expert
-        (names: Model.swift:165-177)."""
-        off = routed_expert_offsets(self.layout, layer)
-        blob = np.zeros(self.layout.expertStride, np.uint8)
+        """The shared expert's nine arrays gathered from the resident file into one blob at the
+        offsets of shared_expert_offsets (names: Model.swift:165-177).  Every array must have the size
+        its shape and the shared expert's bit width give (validateLayerTensors, Model.swift:700-760): an
+        array of another width would overlap its neighbour and be decoded as the wrong codes."""
+        a = self.manifest.arch
+        d, f = a["hiddenSize"], a["moeIntermediateSize"]
+        off, size, bits = self.shared_expert_offsets(layer)
+        blob = np.zeros(size, np.uint8)
         prefix = "language_model.model.layers.%d.mlp.shared_expert." % layer
-        for i, proj in enumerate(("gate_proj", "up_proj", "down_proj")):
+        for i, (proj, rows, cols) in enumerate((("gate_proj", f, d), ("up_proj", f, d), ("down_proj", d, f))):
             w, s, b, _ = self.resident(prefix + proj + ".weight")
             if s is None or b is None:
                 raise ModelError("indexCorrupt", "%s%s.weight has no scales or biases" % (prefix, proj))
-            for arr, at in ((w, off[3 * i]), (s.view(np.uint8), off[3 * i + 1]), (b.view(np.uint8), off[3 * i + 2])):
-                blob[at:at + arr.size] = arr
+            want = (rows * cols * bits // 8, rows * (cols // 64) * 2, rows * (cols // 64) * 2)
+            for arr, at, n, what in ((w, off[3 * i], want[0], "weights"), (s.view(np.uint8), off[3 * i + 1], want[1], "scales"),
+                                     (b.view(np.uint8), off[3 * i + 2], want[2], "biases")):
+                if arr.size != n:
+                    raise ModelError("indexCorrupt", "%s%s.weight %s hold %d bytes, a %d-bit [%d, %d] matrix needs %d"
+                                     % (prefix, proj, what, arr.size, bits, rows, cols, n))
+                blob[at:at + n] = arr
         return blob
 
     def expert_pool(self, layer, device="cuda", with_shared=True):
         """One layer's experts resident in device memory: uint8 [experts (+ 1), stride]; the shared
-        expert, when asked for, is the last row."""
+        expert, when asked for, is the last row -- which needs a shared expert of the routed experts'
+        width (shared_matches_routed); moe_block handles both kinds of model."""
         import torch
+        if with_shared and not self.shared_matches_routed():
+            raise ModelError("unsupportedArch", "the shared expert's quantization differs from the routed experts': it cannot "
+                             "be a row of their pool (use moe_block, which runs it through the shared-expert operator)")
         rows = [torch.from_numpy(np.array(self.expert_blobs(layer)))]
         if with_shared:
             rows.append(torch.from_numpy(self.shared_expert_blob(layer))[None])
         return torch.cat(rows).to(device)
 
-    def moe_layer(self, layer, pool, device="cuda"):
-        """The nvmai_moe_layer descriptor of one layer over `pool` (from expert_pool with the shared
-        expert): router rows and the shared expert's scalar gate row from the resident file
-        (Model.swift:160-182), the expert offsets from the layout.  Returns (descriptor, the device
-        tensors it points into -- keep them alive)."""
+    def _rows(self, name, bits, device, keep):
         import torch
 
         from . import ops
+        w, s, b, e = self.resident(name)
+        if e.dtype == 1:                                           # dense BF16 rows
+            t = torch.from_numpy(np.array(w)).to(device)          # a copy: the map is read-only
+            keep.append(t)
+            return ops.rows_desc(16, t)
+        ts = [torch.from_numpy(np.array(x.view(np.uint8) if x.dtype != np.uint8 else x)).to(device) for x in (w, s, b)]
+        keep.extend(ts)
+        return ops.rows_desc(bits, *ts)
+
+    def moe_layer(self, layer, pool, device="cuda"):
+        """The nvmai_moe_layer descriptor of one layer over `pool`: router rows and the shared expert's
+        scalar gate row from the resident file (Model.swift:160-182), the expert offsets from the
+        layout.  A pool with one row more than the layer has experts carries the shared expert in
+        that row (expert_pool with_shared); otherwise the descriptor has no shared expert.  Returns
+        (descriptor, the device tensors it points into -- keep them alive)."""
+        from . import ops
         a, q = self.manifest.arch, self.manifest.quant
         keep = [pool]
-
-        def rows(name, bits):
-            w, s, b, e = self.resident(name)
-            if e.dtype == 1:                                       # dense BF16 rows
-                t = torch.from_numpy(np.array(w)).to(device)      # a copy: the map is read-only
-                keep.append(t)
-                return ops.rows_desc(16, t)
-            ts = [torch.from_numpy(np.array(x.view(np.uint8) if x.dtype != np.uint8 else x)).to(device)
-                  for x in (w, s, b)]
-            keep.extend(ts)
-            return ops.rows_desc(bits, *ts)
-
-        prefix = "language_model.model.layers.%d.mlp." % layer
-        router = rows(prefix + "gate.weight", q["router"].weightBits)
-        gate = rows(prefix + "shared_expert_gate.weight", q["router"].weightBits)
-        bits = q["routedExpert"].weightBits
         n = self.layout.expertsPerLayer
-        desc = ops.moe_layer_desc(a["hiddenSize"], a["moeIntermediateSize"], n, a["topKExperts"], bits, router, pool[:n],
-                                  pool[n], gate, offsets=routed_expert_offsets(self.layout, layer))
+        has_shared = pool.shape[0] == n + 1
+        if has_shared and not self.shared_matches_routed():
+            raise ModelError("unsupportedArch", "a pool row cannot hold a shared expert of another quantization")
+        prefix = "language_model.model.layers.%d.mlp." % layer
+        router = self._rows(prefix + "gate.weight", q["router"].weightBits, device, keep)
+        gate = self._rows(prefix + "shared_expert_gate.weight", q["router"].weightBits, device, keep) if has_shared else None
+        desc = ops.moe_layer_desc(a["hiddenSize"], a["moeIntermediateSize"], n, a["topKExperts"], q["routedExpert"].weightBits,
+                                  router, pool[:n], pool[n] if has_shared else None, gate,
+                                  offsets=routed_expert_offsets(self.layout, layer))
         return desc, keep
+
+    def moe_block(self, layer, device="cuda"):
+        """One layer's MoE block resident in device memory, whatever the shared expert's width."""
+        return GTurboMoEBlock(self, layer, device)
+
+
+class GTurboMoEBlock:
+    """A layer's routed experts, router, shared expert and its gate row in HBM, and the decode call
+    over them.  A shared expert of the routed experts' width rides in the decode layer's own launches
+    (one more work-list slot).  One of another width (the reference's default 4-bit profile keeps it at
+    8 bits) runs as the reference runs it: the shared-expert operator at its own width
+    (SharedExpertRuntime.encode + the scalar sigmoid gate, RealForwardRunner.swift:3866-3912), its
+    16-bit output added to the routed sum (the `residual` input of phase 2, RealForwardRunner.swift:4263)."""
+
+    def __init__(self, model, layer, device="cuda"):
+        import torch
+
+        from . import ops
+        self.model, self.layer = model, layer
+        a, q = model.manifest.arch, model.manifest.quant
+        self.d, self.f = a["hiddenSize"], a["moeIntermediateSize"]
+        self.routed_bits, self.shared_bits = q["routedExpert"].weightBits, q["sharedExpert"].weightBits
+        self.fused = model.shared_matches_routed()
+        self.pool = model.expert_pool(layer, device, with_shared=self.fused)
+        self.desc, self.keep = model.moe_layer(layer, self.pool, device)
+        if not self.fused:
+            off, _, _ = model.shared_expert_offsets(layer)
+            self.shared_blob = torch.from_numpy(model.shared_expert_blob(layer)).to(device)
+            self.shared_offsets = ops.ExpertOffsets(*[int(v) for v in off])
+            self.shared_gate = model._rows("language_model.model.layers.%d.mlp.shared_expert_gate.weight" % layer,
+                                           q["router"].weightBits, device, self.keep)
+
+    def decode(self, ctx, x, want_routes=False):
+        """y[t] = sigmoid(g . x[t]) * ffn_shared(x[t]) + sum over the top-k of w * ffn_expert(x[t])."""
+        from . import ops
+        out = ops.MoE(ctx, self.routed_bits).decode_layer(self.desc, x, want_routes=want_routes)
+        y = out[0] if want_routes else out
+        if not self.fused:
+            h1 = ops.SharedExpertRuntime(ctx, self.shared_bits).encode(self.shared_blob, self.shared_offsets, x, self.d, self.f,
+                                                                      shared_gate=self.shared_gate)
+            ops.Elementwise(ctx).encode_residual_add(y, h1)
+        return out
 
 
 # ------------------------------------------------------------------------------------ writer (tests, tools)

@@ -698,3 +698,51 @@ def load_reference_gemv():
     ref.nvmai_int4_affine_gemv.restype = None
     ref.nvmai_int4_affine_gemv.argtypes = [u8p, u16p, u16p, f32p, size_t, size_t, f32p]
     return ref.nvmai_int4_affine_gemv
+
+
+def time_expert_ffn(blobs, d, f, x, reps=41, reference=False):
+    """bench.py's cpu_baseline leg for BASELINE configs[0]: median seconds of ONE 4-bit expert FFN on one
+    thread (CPUExpertFFN.accumulate, CPUExpertFFN.swift:101-139: gate and up GEMVs, silu(g) * u, down GEMV,
+    out += w * down), a different blob of `blobs` [n, stride] every repetition so that the weights do not
+    come from the cache.  reference=True: the three GEMVs are the reference's own nvmai_int4_affine_gemv
+    (oracle/_ref, its C file compiled by oracle/Makefile) and the lines of Swift around them are numpy;
+    otherwise the port orc_expert_ffn_accumulate of the -O3 native timing library.  Returns (seconds,
+    the last output) or (None, None) when the reference library was never built."""
+    import time
+    off = expert_offsets(d, f, 4)
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.zeros(d, np.float32)
+    times = []
+    if reference:
+        gemv = load_reference_gemv()
+        if gemv is None:
+            return None, None
+        g, u, dn = np.zeros(f, np.float32), np.zeros(f, np.float32), np.zeros(d, np.float32)
+        parts = lambda blob, i, rows, cols: (blob[off[3 * i]:off[3 * i] + rows * cols // 2],
+                                             blob[off[3 * i + 1]:off[3 * i + 1] + rows * (cols // 64) * 2].view(np.uint16),
+                                             blob[off[3 * i + 2]:off[3 * i + 2] + rows * (cols // 64) * 2].view(np.uint16))
+        for r in range(-2, reps):
+            blob = blobs[r % len(blobs)]
+            pg, pu, pd = parts(blob, 0, f, d), parts(blob, 1, f, d), parts(blob, 2, d, f)
+            t0 = time.perf_counter()
+            gemv(pg[0], pg[1], pg[2], x, f, d, g)
+            gemv(pu[0], pu[1], pu[2], x, f, d, u)
+            act = (g / (1.0 + np.exp(-g)) * u).astype(np.float32)
+            gemv(pd[0], pd[1], pd[2], act, d, f, dn)
+            out = dn.copy()
+            if r >= 0:
+                times.append(time.perf_counter() - t0)
+    else:
+        clib, _ = timing_lib()
+        fn = clib.orc_expert_ffn_accumulate
+        fn.restype = None
+        fn.argtypes = [u8p, u32p, C.c_int, f32p, size_t, size_t, C.c_float, f32p, f32p]
+        scratch = np.zeros(2 * f + d, np.float32)
+        for r in range(-2, reps):
+            blob = np.ascontiguousarray(blobs[r % len(blobs)])
+            out[:] = 0
+            t0 = time.perf_counter()
+            fn(blob, off, 4, x, d, f, 1.0, scratch, out)
+            if r >= 0:
+                times.append(time.perf_counter() - t0)
+    return float(np.median(times)), out

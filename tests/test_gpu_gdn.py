@@ -2,10 +2,13 @@
 fused residual add + RMSNorm, the fused input projections and the dense BF16 GEMV, through the C ABI
 against the CPU oracle.
 
-GDN bar: the reference's own, for its kernels against its CPU model (GDNKernelTests.swift:170-185):
-|got - want| <= max(2e-2, 4e-2 |want|) per output and 5e-2 on the recurrent state, with fp16
-activations as there; with bf16 activations (three mantissa bits fewer at every hand-over) the same
-form at 8e-2 / 1.6e-1."""
+GDN bars, both asserted for every comparison of outputs:
+ * max|got - want| / max|want| < 1e-2 (the measure and the 16-bit bar of this build, RelError.swift:5-16);
+   measured: fp16 activations <= 5e-4, bf16 activations <= 3.2e-3, bf16 activations with the BF16 state
+   <= 5.9e-3 (the oracle then rounds its own state to BF16 after every token, as the kernels store it);
+ * the reference's own per-element bar for its kernels against its CPU model (GDNKernelTests.swift:170-185),
+   |got - want| <= max(2e-2, 4e-2 |want|), with fp16 AND with bf16 activations (measured: no element uses
+   more than a quarter of it), and 5e-2 on the fp32 recurrent state."""
 import numpy as np
 import pytest
 import torch
@@ -46,9 +49,21 @@ def _bits(a):
     return dev(np.ascontiguousarray(a).view(np.int16))
 
 
-def _close(got, want, act):
-    lo, rel = (2e-2, 4e-2) if act == 1 else (8e-2, 1.6e-1)
-    return np.all(np.abs(got - want) <= np.maximum(lo, np.abs(want) * rel))
+MEASURED = []          # (label, max|diff| / max|ref|, worst element as a fraction of its bar)
+
+
+def _rel(got, want):
+    """The measure the tolerances of this build are stated in: max|got - want| / max|want| (RelError.swift:5-16)."""
+    return float(np.abs(got - want).max() / max(float(np.abs(want).max()), 1e-30))
+
+
+def _close(got, want, act, label=""):
+    lo, rel = 2e-2, 4e-2                                   # GDNKernelTests.swift:170-185, for both activation types
+    use = float((np.abs(got - want) / np.maximum(lo, np.abs(want) * rel)).max())
+    MEASURED.append((label, _rel(got, want), use))
+    print("[measure] gdn %-28s act=%d max|d|/max|ref| %.3e  worst element at %.2f of its bar" % (label, act, MEASURED[-1][1], use),
+          flush=True)
+    return use <= 1.0 and MEASURED[-1][1] < 1e-2
 
 
 def _gpu_rows(nv, ctx, gdn, fx, tail, state, t0, rows, batch_rows=None):
@@ -75,7 +90,7 @@ def test_gdn_decode_chain_matches_oracle(nv, ctx, cfg):
         want = O.gdn_step(ref, fx["qkv"][t], fx["a"][t], fx["b"][t], fx["z"][t], fx["conv_w"], fx["a_log"],
                           fx["dt_bias"], fx["norm_w"], ctx.act)
         torch.cuda.synchronize()
-        assert _close(got, want, ctx.act), "token %d" % t
+        assert _close(got, want, ctx.act, "decode chain"), "token %d" % t
     assert np.array_equal(act_np(tail[0]), ref.tail)               # raw rows, copied
     assert np.abs(state[0].cpu().numpy() - ref.state).max() <= 5e-2
 
@@ -103,7 +118,7 @@ def test_gdn_prefill_chunk_equals_sequential_decode(nv, ctx):
             seq.append(act_np(_gpu_rows(nv, ctx, gdn, fx, tail_a, state_a, t, 1))[0])
         chunk = act_np(_gpu_rows(nv, ctx, gdn, fx, tail_b, state_b, 3, rows))
         torch.cuda.synchronize()
-        assert _close(chunk, np.array(seq), ctx.act)
+        assert _close(chunk, np.array(seq), ctx.act, "chunk vs sequential %d" % rows)
         assert torch.equal(tail_a, tail_b)
         assert (state_a - state_b).abs().max().item() <= 5e-2
 
@@ -129,13 +144,12 @@ def test_gdn_batch_of_sequences_and_bf16_state(nv, ctx, bf16_state):
         for b in range(batch):
             want = O.gdn_step(refs[b], fxs[b]["qkv"][t], fxs[b]["a"][t], fxs[b]["b"][t], fxs[b]["z"][t], w["conv_w"],
                               w["a_log"], w["dt_bias"], w["norm_w"], ctx.act)
-            if bf16_state:
-                assert np.all(np.abs(out[b] - want) <= np.maximum(0.15, np.abs(want) * 0.3))
-            else:
-                assert _close(out[b], want, ctx.act), (t, b)
+            if bf16_state:                              # the kernels store the state as BF16 after every token
+                refs[b].state[...] = O.round_bf16(refs[b].state)
+            assert _close(out[b], want, ctx.act, "batch, bf16 state" if bf16_state else "batch, fp32 state"), (t, b)
     got_state = state.float().cpu().numpy()
     for b in range(batch):
-        assert np.abs(got_state[b] - refs[b].state).max() <= (5e-2 if not bf16_state else 1e-1)
+        assert np.abs(got_state[b] - refs[b].state).max() <= 5e-2
 
 
 @pytest.mark.parametrize("bf16_state", [False, True])
@@ -160,12 +174,10 @@ def test_gdn_long_call_on_the_matrix_cores_batch_and_state_types(nv, ctx, bf16_s
     chunk = act_np(gdn.encode_delta_gated_norm(conv, cat("a"), cat("b"), *args, state_b, cat("z"), _bits(w["norm_w"]), rows=rows))
     torch.cuda.synchronize()
     want = np.stack(seq, axis=1).reshape(batch * rows, -1)            # [batch, rows, :] like the call's rows
-    if bf16_state:      # the row-by-row calls round the state to BF16 after every row, the long call once
-        assert np.all(np.abs(chunk - want) <= np.maximum(0.15, np.abs(want) * 0.3))
-    else:
-        assert _close(chunk, want, ctx.act)
+    # (with the BF16 state the row-by-row calls round the state after every row, the long call once per call)
+    assert _close(chunk, want, ctx.act, "chunked, bf16 state" if bf16_state else "chunked, fp32 state")
     assert torch.equal(tail_a, tail_b)
-    assert (state_a.float() - state_b.float()).abs().max().item() <= (5e-2 if not bf16_state else 1e-1)
+    assert (state_a.float() - state_b.float()).abs().max().item() <= 5e-2
 
 
 @pytest.mark.parametrize("rows", [8, 37, 80])
@@ -212,7 +224,7 @@ def test_gdn_full_size_prompt_is_the_same_in_one_call_or_in_pieces(nv, ctx):
         outs.append(np.concatenate(got)); tails.append(tail); states.append(state)
     assert np.isfinite(outs[0]).all()
     for k in (1, 2):
-        assert _close(outs[k], outs[0], ctx.act), k
+        assert _close(outs[k], outs[0], ctx.act, "full size, pieces %d" % k), k
         assert torch.equal(tails[k], tails[0])
         assert (states[k] - states[0]).abs().max().item() <= 5e-2
 
@@ -249,7 +261,7 @@ def test_gdn_decode_step_in_one_launch_equals_the_two_calls(nv, ctx, cfg, bf16_s
         if not bf16_state:
             want = O.gdn_step(ref, fxs[0]["qkv"][t], fxs[0]["a"][t], fxs[0]["b"][t], fxs[0]["z"][t], w["conv_w"],
                               w["a_log"], w["dt_bias"], w["norm_w"], ctx.act)
-            assert _close(act_np(one)[0], want, ctx.act)
+            assert _close(act_np(one)[0], want, ctx.act, "one launch")
     # a shape without a fused kernel and no scratch rows
     if cfg == (2, 2, 64, 64, 2):
         with pytest.raises(nv.NvmaiError):
@@ -343,3 +355,32 @@ def test_dense_bf16_gemv(nv):
     torch.cuda.synchronize()
     ctx.close()
     c16.close()
+
+
+@pytest.mark.parametrize("tokens", [1, 16])
+def test_dense_bf16_gemv_at_the_lm_head_size(nv, tokens):
+    # the BF16 LM head of configs[4]: 248,320 x 2048, one and sixteen input rows (the launch's grid policy
+    # follows the row count and the resident blocks), every logit against a float64 product
+    say("dense bf16 gemv, LM head size", tokens)
+    ctx = nv.Context(0, 0)
+    m, n = 248320, 2048
+    gen = torch.Generator(device="cuda").manual_seed(2048 + tokens)
+    wd = torch.empty((m, n), dtype=torch.float32, device="cuda").normal_(0.0, 0.02, generator=gen).to(torch.bfloat16)
+    x = torch.empty((tokens, n), dtype=torch.float32, device="cuda").normal_(0.0, 1.0, generator=gen).to(torch.bfloat16)
+    y = nv.affine_gemv(ctx, wd.view(torch.int16), None, None, 16, x, m, n)
+    yf = nv.affine_gemv(ctx, wd.view(torch.int16), None, None, 16, x, m, n, out_f32=True)
+    torch.cuda.synchronize()
+    x64 = x.float().cpu().numpy().astype(np.float64)
+    want = np.empty((tokens, m), np.float64)
+    for r0 in range(0, m, 32768):                      # the float64 copy of the head, a slab at a time
+        want[:, r0:r0 + 32768] = x64 @ wd[r0:r0 + 32768].float().cpu().numpy().astype(np.float64).T
+    rel32 = O.rel_error(yf.cpu().numpy(), want.astype(np.float32))
+    rel16 = O.rel_error(act_np(y), want.astype(np.float32))
+    print("[measure] dense bf16 gemv 248320 x 2048, %d rows: fp32 out rel %.3e, bf16 out rel %.3e" % (tokens, rel32, rel16), flush=True)
+    assert rel32 < 2e-3 and rel16 < 1e-2
+    # and no row was skipped or written twice by the grid policy: the argmax agrees wherever the margin is clear
+    top2 = np.sort(want, axis=1)[:, -2:]
+    clear = (top2[:, 1] - top2[:, 0]) > 1e-2 * np.abs(top2[:, 1])
+    assert np.array_equal(yf.cpu().numpy().argmax(axis=1)[clear], want.argmax(axis=1)[clear])
+    torch.cuda.synchronize()
+    ctx.close()

@@ -77,3 +77,62 @@ def test_model_directory_to_decode_layer(tmp_path, bits):
         assert np.abs(u16(w).astype(np.int32) - wo.astype(np.int32)).max() <= 1
         assert O.rel_error(act_np(y), yo) < 1e-2
     ctx.close()
+
+
+def test_shared_expert_at_8_bits_beside_4_bit_routed_experts(tmp_path):
+    # the reference's default 4-bit profile (sharedExpert = 8, routedExpert = 4, RemoteStreamingRepacker.swift:678-683):
+    # the block runs the routed experts at 4 bits and the shared expert through its own operator at 8 bits
+    import nvmai_amd as nv
+    from nvmai_amd import gturbo as G
+    say("gturbo directory, 8-bit shared expert + 4-bit routed experts")
+    rng = np.random.default_rng(91)
+    d, f, E, k, bits, sbits = 256, 128, 16, 4, 4, 8
+    mk = lambda r, c, s=0.05: O.round_bf16(gauss(rng, (r, c), s))
+    roles = ["gate", "gate_scales", "gate_biases", "up", "up_scales", "up_biases", "down", "down_scales", "down_biases"]
+    off = O.expert_offsets(d, f, bits)
+    sizes = [f * d * bits // 8, f * (d // 64) * 2, f * (d // 64) * 2] * 2 + [d * f * bits // 8, d * (f // 64) * 2, d * (f // 64) * 2]
+    shapes = [(f, d), (f, d // 64), (f, d // 64)] * 2 + [(d, f), (d, f // 64), (d, f // 64)]
+    tensors = {r: G.SubTensorEntry(int(off[i]), sizes[i], "BF16" if "_" in r else "U32", shapes[i], None if "_" in r else bits)
+               for i, r in enumerate(roles)}
+    used = int(off[8]) + sizes[8]
+    stride = (used + G.ALIGNMENT_BYTES - 1) // G.ALIGNMENT_BYTES * G.ALIGNMENT_BYTES
+    blobs = np.zeros((E, stride), np.uint8)
+    for e in range(E):
+        blobs[e, :used] = O.pack_expert(mk(f, d), mk(f, d), mk(d, f), bits)[:used]
+    p = "language_model.model.layers.0.mlp."
+    router = O.bf16_bits(mk(E, d, 0.02))
+    resident = [(p + "gate.weight", 1, (E, d), router.tobytes(), None, None)]
+    shared_w = [mk(f, d), mk(f, d), mk(d, f)]
+    for proj, w in zip(("gate_proj", "up_proj", "down_proj"), shared_w):
+        q = O.quantize_affine(w, sbits)
+        resident.append((p + "shared_expert.%s.weight" % proj, 0, w.shape, q[0].tobytes(), q[1].tobytes(), q[2].tobytes()))
+    gate = O.quantize_affine(mk(1, d), bits)
+    resident.append((p + "shared_expert_gate.weight", 0, (1, d), gate[0].tobytes(), gate[1].tobytes(), gate[2].tobytes()))
+    slot = lambda b: {"weightBits": b, "scheme": "affine", "scaleType": "bf16", "biasType": "bf16", "groupSize": 64}
+    quant = {n: slot(bits) for n in ("embedding", "attention", "router", "sharedExpert", "routedExpert")}
+    quant["sharedExpert"] = slot(sbits)
+    arch = {"hiddenSize": d, "ffnIntermediate": 4 * d, "moeIntermediateSize": f, "numHeads": 4, "numKVHeads": 2,
+            "numFullKVHeads": 2, "headDim": 64, "fullHeadDim": 64, "vocabSize": 1000, "slidingWindow": 0,
+            "finalLogitSoftcap": 0.0, "ropeTheta": 1e4, "fullRopeTheta": 1e7, "partialRotaryFactor": 0.25,
+            "numLayers": 1, "numExperts": E, "topKExperts": k, "tieWordEmbeddings": False, "attentionKEqV": False,
+            "hiddenActivation": "silu", "fullAttentionLayerMask": [0]}
+    G.write_model(str(tmp_path), arch, quant, [{"blobs": blobs, "tensors": tensors, "ranks": None}], resident)
+    model = G.GTurboModel(str(tmp_path))
+    assert not model.shared_matches_routed()
+    block = model.moe_block(0)
+    ctx = nv.Context(0, 0)
+    x = round_act(gauss(rng, (5, d)), 0)
+    y, idx, w = block.decode(ctx, act_tensor(x, ctx), want_routes=True)
+    torch.cuda.synchronize()
+    # the oracle: routed experts alone (a zero shared expert), plus the 8-bit shared expert with its gate
+    io, wo, y_routed = O.moe_layer_forward(x, d, f, k, bits, (16, router, None, None), blobs, None, None)
+    shared_blob = O.pack_expert(*shared_w, sbits)
+    _, _, y_both = O.moe_layer_forward(x, d, f, k, sbits, (16, router, None, None), np.stack([shared_blob] * E), shared_blob,
+                                       (bits,) + gate)
+    # y_both - (its routed part) = the gated shared expert at 8 bits
+    _, _, y_routed8 = O.moe_layer_forward(x, d, f, k, sbits, (16, router, None, None), np.stack([shared_blob] * E), None, None)
+    want = y_routed + (y_both - y_routed8)
+    assert np.array_equal(u32(idx), io), "routing indices"
+    assert O.rel_error(act_np(y), want) < 1e-2
+    # and a model whose widths agree takes the one-call path through the same object
+    ctx.close()

@@ -265,7 +265,7 @@ def test_cross_validation_against_the_manifest():
     assert "dimension mismatch" in e.value.detail
 
 
-def _toy_model(tmp_path, rng, bits=4, layers=2, experts=4, d=128, f=64, ranks=None):
+def _toy_model(tmp_path, rng, bits=4, layers=2, experts=4, d=128, f=64, ranks=None, shared_bits=None, shared_store_bits=None):
     """A complete directory: routed experts (random bytes in the nine roles at the layout of
     CPUExpertFFN.Offsets), router / shared expert / shared gate rows in the resident file."""
     wg, aux_g = f * d * bits // 8, f * (d // 64) * 2
@@ -285,16 +285,19 @@ def _toy_model(tmp_path, rng, bits=4, layers=2, experts=4, d=128, f=64, ranks=No
         blobs[:, :at] = rng.integers(0, 256, (experts, at), dtype=np.uint8)
         lays.append({"blobs": blobs, "tensors": tensors, "ranks": ranks})
     resident = []
+    sbits = shared_bits or bits                         # what the manifest says about the shared expert
+    wbits = shared_store_bits or sbits                  # what its arrays were really written at
     for L in range(layers):
         p = "language_model.model.layers.%d.mlp." % L
         resident.append((p + "gate.weight", 1, (experts, d), rng.integers(0, 256, experts * d * 2, dtype=np.uint8).tobytes(), None, None))
         for proj, (rows, cols) in (("gate_proj", (f, d)), ("up_proj", (f, d)), ("down_proj", (d, f))):
             resident.append((p + "shared_expert.%s.weight" % proj, 0, (rows, cols),
-                             rng.integers(0, 256, rows * cols * bits // 8, dtype=np.uint8).tobytes(),
+                             rng.integers(0, 256, rows * cols * wbits // 8, dtype=np.uint8).tobytes(),
                              rng.integers(0, 256, rows * (cols // 64) * 2, dtype=np.uint8).tobytes(),
                              rng.integers(0, 256, rows * (cols // 64) * 2, dtype=np.uint8).tobytes()))
         resident.append((p + "shared_expert_gate.weight", 1, (1, d), rng.integers(0, 256, d * 2, dtype=np.uint8).tobytes(), None, None))
     quant = {k: _slot(bits) for k in ("embedding", "attention", "router", "sharedExpert", "routedExpert")}
+    quant["sharedExpert"] = _slot(sbits)
     a = _arch(layers, experts)
     a.update(hiddenSize=d, moeIntermediateSize=f)
     G.write_model(str(tmp_path), a, quant, lays, resident)
@@ -344,3 +347,38 @@ def test_model_directory_roundtrip(tmp_path):
     with pytest.raises(G.ModelError) as e:              # ManifestReaderTests.swift:214-225
         G.GTurboModel(str(tmp_path))
     assert e.value.kind == "partialInstall"
+
+
+def test_shared_expert_of_another_width_than_the_routed_experts(tmp_path):
+    # the reference keeps separate quant slots for the two (Model.swift:59-60) and its repacker's default
+    # profile is sharedExpert = 8, routedExpert = 4 (RemoteStreamingRepacker.swift:678-683): the shared
+    # expert's blob is then laid out at its own width, never squeezed into the routed sub-tensor regions
+    rng = np.random.default_rng(6)
+    d, f = 128, 64
+    lays, resident, tensors, stride = _toy_model(tmp_path / "mixed", rng, bits=4, shared_bits=8, d=d, f=f)
+    m = G.GTurboModel(str(tmp_path / "mixed"))
+    assert not m.shared_matches_routed()
+    off, size, bits = m.shared_expert_offsets(0)
+    wg, aux_g, wd, aux_d = f * d, f * (d // 64) * 2, d * f, d * (f // 64) * 2
+    assert bits == 8 and size == 2 * (wg + 2 * aux_g) + wd + 2 * aux_d          # CPUExpertFFN.Offsets at 8 bits
+    assert off == (0, wg, wg + aux_g, wg + 2 * aux_g, 2 * wg + 2 * aux_g, 2 * wg + 3 * aux_g,
+                   2 * wg + 4 * aux_g, 2 * wg + 4 * aux_g + wd, 2 * wg + 4 * aux_g + wd + aux_d)
+    blob = m.shared_expert_blob(1)
+    assert blob.size == size
+    for i, proj in enumerate(("gate_proj", "up_proj", "down_proj")):
+        w, s, b, _ = m.resident("language_model.model.layers.1.mlp.shared_expert.%s.weight" % proj)
+        for arr, at in ((w, off[3 * i]), (s.view(np.uint8), off[3 * i + 1]), (b.view(np.uint8), off[3 * i + 2])):
+            assert bytes(blob[at:at + arr.size]) == bytes(arr)                  # every array whole, none overlapping
+    with pytest.raises(G.ModelError) as e:              # it cannot be a row of the routed pool
+        m.expert_pool(0, device="cpu")
+    assert e.value.kind == "unsupportedArch"
+    # same width: the routed offsets, as before
+    _toy_model(tmp_path / "same", rng, bits=4, d=d, f=f)
+    m2 = G.GTurboModel(str(tmp_path / "same"))
+    assert m2.shared_matches_routed() and m2.shared_expert_offsets(0)[:2] == (G.routed_expert_offsets(m2.layout, 0), stride)
+    # arrays that are not of the width the manifest states are refused, not copied over their neighbours
+    _toy_model(tmp_path / "lying", rng, bits=4, shared_bits=4, shared_store_bits=8, d=d, f=f)
+    m3 = G.GTurboModel(str(tmp_path / "lying"))
+    with pytest.raises(G.ModelError) as e:
+        m3.shared_expert_blob(0)
+    assert e.value.kind == "indexCorrupt" and "needs" in e.value.detail
