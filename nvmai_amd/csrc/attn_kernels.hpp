@@ -444,8 +444,11 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
                 uint16_t hb[8];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    hb[e] = f32_to_f16(qf[g][h][e] * sc);
-                    s += f16_to_f32(hb[e]);
+                    // 4 bit: the K codes of elements 1, 3, 5, 7 are used where they lie, at bits 4..7 of a half
+                    // (16 c * 2^-24, see the operand build in the loop), so those query elements carry 1/16
+                    const bool sixteenth = BITS == 4 && (e & 1);
+                    hb[e] = f32_to_f16(qf[g][h][e] * (sixteenth ? sc * 0.0625f : sc));
+                    s += f16_to_f32(hb[e]) * (sixteenth ? 16.0f : 1.0f);
                 }
                 if (BITS == 8) {
                     // K codes unpack in natural byte order: pairs (0,1) (2,3) (4,5) (6,7)
@@ -483,7 +486,12 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
     constexpr int LPT = CODE_ROW / 16;                              // lanes (16-byte chunks) per token
     constexpr int TPI = 64 / LPT;                                   // tokens per instruction
     const uint32_t d_tok = lane / LPT, d_slot = lane % LPT;
-    const uint32_t d_chunk16 = ((d_slot ^ d_tok) & (LPT - 1)) * 16u;  // 8 bit: ^ 64 (j & 3) per instruction
+    // The 16-byte chunks of a token are XOR-swizzled so that the operand reads below touch every bank once.
+    // 8 bit (256-byte rows, sixteen chunks): chunk ^ token.  4 bit (128-byte rows: the token's lowest bit already
+    // picks the half of the 256 bytes the banks span, and only eight chunks): chunk ^ (token >> 1) -- swizzled by
+    // the token's low three bits, tokens 8 apart fell on the same banks (two-way conflicts in both operand reads).
+    const uint32_t d_chunk16 = BITS == 8 ? ((d_slot ^ d_tok) & (LPT - 1)) * 16u        // ^ 64 (j & 3) per instruction
+                                         : ((d_slot ^ (d_tok >> 1)) & (LPT - 1)) * 16u;  // ^ 64 (j & 1) per instruction
     const uint32_t m_part = (lane & 3) < 2 ? meta_sc + 4 * (lane & 3) : meta_bi + 4 * ((lane & 3) - 2);
     uint8_t* const myk = kst + wave * REGION;
     uint8_t* const myv = vst + wave * REGION;
@@ -492,7 +500,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
         const uint32_t row = (s0 + d_tok) * p.f.stride;
 #pragma unroll
         for (int j = 0; j < 32 / TPI; ++j) {
-            const uint32_t voff = row + (BITS == 8 ? (d_chunk16 ^ (64u * (j & 3))) : d_chunk16);
+            const uint32_t voff = row + (d_chunk16 ^ (64u * (j & (BITS == 8 ? 3 : 1))));
             const uint32_t soff = (uint32_t)(j * TPI) * p.f.stride + code_off;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(st + j * 1024), 16, voff, soff, 0, 0);
         }
@@ -522,6 +530,11 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
         float sv[8];                                                // scores of head i at this lane's 8 tokens
 #pragma unroll
         for (int tile = 0; tile < 2; ++tile) {
+            // the scales and biases of this lane's four tokens of the tile, requested ahead of the products: read
+            // where they are used, each read was waited for on the spot, inside a branch of its own
+            uint4 km4[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) km4[t] = *reinterpret_cast<const uint4*>(myk + OFF_META + slot_tok(tile * 4 + t) * 16);
             f4_t sacc[4];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
@@ -532,7 +545,7 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
                     const uint4 w = *reinterpret_cast<const uint4*>(myk + (tile * 16 + i) * CODE_ROW + (((4 * g + r) ^ i) & 15) * 16);
                     kw[0] = w.x; kw[1] = w.y; kw[2] = w.z; kw[3] = w.w;
                 } else {
-                    const uint2 w = *reinterpret_cast<const uint2*>(myk + (tile * 16 + i) * CODE_ROW + (((2 * g + (r >> 1)) ^ i) & 7) * 16 + (r & 1) * 8);
+                    const uint2 w = *reinterpret_cast<const uint2*>(myk + (tile * 16 + i) * CODE_ROW + (((2 * g + (r >> 1)) ^ (i >> 1)) & 7) * 16 + (r & 1) * 8);
                     kw[0] = w.x; kw[1] = w.y;
                 }
 #pragma unroll
@@ -545,9 +558,11 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
                         a.u[2] = __builtin_amdgcn_perm(w1, w1, 0x0C050C04u);
                         a.u[3] = __builtin_amdgcn_perm(w1, w1, 0x0C070C06u);
                     } else {
-                        const uint32_t w = kw[h];
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) a.u[j] = (w >> (4 * j)) & 0x000F000Fu;
+                        // pairs (j, j + 4) of the dword's nibbles; a nibble at bits 4..7 of a half reads as 16 c * 2^-24
+                        // (still a subnormal), which the query's 1/16 takes back: one shift instead of three
+                        const uint32_t w = kw[h], w8 = w >> 8;
+                        a.u[0] = w & 0x000F000Fu; a.u[1] = w & 0x00F000F0u;
+                        a.u[2] = w8 & 0x000F000Fu; a.u[3] = w8 & 0x00F000F0u;
                     }
                     sacc[g] = mfma16(a, qop[g][h], sacc[g]);
                 }
@@ -555,17 +570,25 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const int slot = tile * 4 + t;
-                const uint4 km = *reinterpret_cast<const uint4*>(myk + OFF_META + slot_tok(slot) * 16);
-                const uint32_t scw[2] = {km.x, km.y}, biw[2] = {km.z, km.w};
-                float acc_s = 0.0f, acc_b = 0.0f;
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const float sc = f16_to_f32((uint16_t)(scw[g >> 1] >> (16 * (g & 1))));
-                    const float bi = f16_to_f32((uint16_t)(biw[g >> 1] >> (16 * (g & 1))));
-                    acc_s = fmaf(sc, sacc[g][t], acc_s);
-                    acc_b = fmaf(bi, qsum[g], acc_b);
-                }
-                sv[slot] = tok_ok[slot] ? fmaf(acc_s, 16777216.0f, acc_b) * q_unscale : -INFINITY;
+                const uint4 km = km4[t];
+                // the fp16 scales and biases go into the multiply-adds as they are (mixed-precision fma reads either
+                // half of a dword): extracted and converted on their own they cost two more instructions each
+                typedef _Float16 hh2_t __attribute__((ext_vector_type(2)));
+                const hh2_t s01 = __builtin_bit_cast(hh2_t, km.x), s23 = __builtin_bit_cast(hh2_t, km.y);
+                const hh2_t b01 = __builtin_bit_cast(hh2_t, km.z), b23 = __builtin_bit_cast(hh2_t, km.w);
+                float acc_s = __builtin_fmaf((float)s01.x, sacc[0][t], 0.0f);
+                acc_s = __builtin_fmaf((float)s01.y, sacc[1][t], acc_s);
+                acc_s = __builtin_fmaf((float)s23.x, sacc[2][t], acc_s);
+                acc_s = __builtin_fmaf((float)s23.y, sacc[3][t], acc_s);
+                float acc_b = __builtin_fmaf((float)b01.x, qsum[0], 0.0f);
+                acc_b = __builtin_fmaf((float)b01.y, qsum[1], acc_b);
+                acc_b = __builtin_fmaf((float)b23.x, qsum[2], acc_b);
+                acc_b = __builtin_fmaf((float)b23.y, qsum[3], acc_b);
+                float val = fmaf(acc_s, 16777216.0f, acc_b) * q_unscale;
+#if defined(__HIP_DEVICE_COMPILE__)
+                asm("" : "+v"(val));                        // computed for every slot, masked by a select: no branch per slot
+#endif
+                sv[slot] = tok_ok[slot] ? val : -INFINITY;
             }
         }
 
@@ -595,22 +618,27 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
         uint4 vm[8];                                                // (sc.x, sc.y, bi.x, bi.y) of the 8 token slots
 #pragma unroll
         for (int t = 0; t < 8; ++t) vm[t] = *reinterpret_cast<const uint4*>(myv + OFF_META + slot_tok(t) * 16);
+        // Both factors of p * vsc are fp16 values (the cache stores fp16 scales and biases, p <= 1 is rounded to
+        // fp16 once), so two tokens take one packed multiply, and the bias correction one two-term dot product:
+        // per group four byte-permutes pick the (token 2w, token 2w + 1) pair of scales and of biases.
+        typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+        typedef float f2_t __attribute__((ext_vector_type(2)));
         H8 pop[4];
+        h2_t p2[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) p2[w] = __builtin_convertvector(f2_t{pe[2 * w], pe[2 * w + 1]}, h2_t);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             float c = corr[g] * alpha;
-            uint16_t hb[8];
+            const uint32_t sel = (g & 1) ? 0x07060302u : 0x05040100u;   // the group's half of (token 2w, token 2w + 1)
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                const uint32_t scw = g < 2 ? vm[t].x : vm[t].y, biw = g < 2 ? vm[t].z : vm[t].w;
-                const float sc = f16_to_f32((uint16_t)(scw >> (16 * (g & 1))));
-                const float bi = f16_to_f32((uint16_t)(biw >> (16 * (g & 1))));
-                hb[t] = f32_to_f16(pe[t] * sc);
-                c = fmaf(pe[t], bi, c);
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t sc2 = __builtin_amdgcn_perm(g < 2 ? vm[2 * w + 1].x : vm[2 * w + 1].y, g < 2 ? vm[2 * w].x : vm[2 * w].y, sel);
+                const uint32_t bi2 = __builtin_amdgcn_perm(g < 2 ? vm[2 * w + 1].z : vm[2 * w + 1].w, g < 2 ? vm[2 * w].z : vm[2 * w].w, sel);
+                pop[g].u[w] = __builtin_bit_cast(uint32_t, p2[w] * __builtin_bit_cast(h2_t, sc2));
+                c = __builtin_amdgcn_fdot2(p2[w], __builtin_bit_cast(h2_t, bi2), c, false);
             }
             corr[g] = c;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) pop[g].u[w] = hb[2 * w] | ((uint32_t)hb[2 * w + 1] << 16);
         }
         if (i < 16 && r == 0) bc[i] = alpha;                        // head-indexed broadcast through LDS
         __builtin_amdgcn_wave_barrier();
@@ -634,12 +662,12 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
             for (int t = 0; t < 8; ++t) {
                 const uint32_t tk = slot_tok(t);
                 if (BITS == 8) vr[t] = *reinterpret_cast<const uint32_t*>(myv + tk * CODE_ROW + (((4 * g + (i >> 2)) ^ tk) & 15) * 16 + (i & 3) * 4);
-                else vr[t] = *reinterpret_cast<const uint16_t*>(myv + tk * CODE_ROW + (((2 * g + (i >> 3)) ^ tk) & 7) * 16 + (i & 7) * 2);
+                else vr[t] = *reinterpret_cast<const uint16_t*>(myv + tk * CODE_ROW + (((2 * g + (i >> 3)) ^ (tk >> 1)) & 7) * 16 + (i & 7) * 2);
             }
             uint32_t pair4[4];                                      // 4-bit: nibbles of two tokens side by side
             if (BITS == 4) {
 #pragma unroll
-                for (int w = 0; w < 4; ++w) pair4[w] = vr[2 * w] | (vr[2 * w + 1] << 16);
+                for (int w = 0; w < 4; ++w) pair4[w] = __builtin_amdgcn_perm(vr[2 * w + 1], vr[2 * w], 0x05040100u);
             }
 #pragma unroll
             for (int n = 0; n < 4; ++n) {
@@ -651,7 +679,8 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
                         const uint32_t sel = 0x0C000C00u | (uint32_t)n | ((uint32_t)(4 + n) << 16);
                         bop.u[w] = __builtin_amdgcn_perm(vr[2 * w + 1], vr[2 * w], sel);
                     } else {
-                        bop.u[w] = (pair4[w] >> (4 * n)) & 0x000F000Fu;
+                        // dims n = 1, 3 where they lie (bits 4..7 of a half: 16 c * 2^-24, taken back when O leaves its scale)
+                        bop.u[w] = ((n & 2) ? pair4[w] >> 8 : pair4[w]) & ((n & 1) ? 0x00F000F0u : 0x000F000Fu);
                     }
                 }
                 oacc[g][n] = mfma16(pop[g], bop, oacc[g][n]);
@@ -678,8 +707,9 @@ __global__ __launch_bounds__(256, 2) void attn_partial_mfma_kernel(AttnParams p)
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int n = 0; n < 4; ++n) {                               // O leaves its 2^-24 here
-            oacc[g][n][0] = fmaf(oacc[g][n][0], 16777216.0f, cg.x); oacc[g][n][1] = fmaf(oacc[g][n][1], 16777216.0f, cg.y);
-            oacc[g][n][2] = fmaf(oacc[g][n][2], 16777216.0f, cg.z); oacc[g][n][3] = fmaf(oacc[g][n][3], 16777216.0f, cg.w);
+            const float unscale = (BITS == 4 && (n & 1)) ? 1048576.0f : 16777216.0f;   // 4 bit, odd dims: 2^24 / 16
+            oacc[g][n][0] = fmaf(oacc[g][n][0], unscale, cg.x); oacc[g][n][1] = fmaf(oacc[g][n][1], unscale, cg.y);
+            oacc[g][n][2] = fmaf(oacc[g][n][2], unscale, cg.z); oacc[g][n][3] = fmaf(oacc[g][n][3], unscale, cg.w);
         }
     }
 
