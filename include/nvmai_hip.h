@@ -262,7 +262,8 @@ int nvmai_hip_moe_decode_layer_norms(nvmai_hip_ctx* ctx, nvmai_stream stream, co
  * top-8, shared expert) returns NVMAI_ERR_SCRATCH and launches nothing.  Every call on one
  * GPU shares that GPU's array and finds the previous call's contents in it (each call writes
  * what it reads, nothing has to be cleared): calls that overlap on one GPU, from different
- * streams or contexts, race. */
+ * streams or contexts, race.  The ctx's device must be the current device (each GPU has its own
+ * copy of the array at its own address): otherwise NVMAI_ERR_INVALID_ARG. */
 int nvmai_hip_moe_decode_layer_noalloc(nvmai_hip_ctx* ctx, nvmai_stream stream,
                                        const nvmai_moe_layer* layer, const void* x, uint32_t x_stride,
                                        uint32_t n_tokens, void* y, uint32_t y_stride, uint32_t* out_idx,
@@ -682,7 +683,12 @@ int nvmai_hip_gdn_conv_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai
  * state_is_bf16 (half the bytes per token, arithmetic still fp32) -- and
  * out = rmsnorm(y) * norm_weight * silu(z) per value head.  a_proj, b_proj: [batch * rows, ab_stride]
  * activations; a_log, dt_bias: BF16 [Hv]; z, out: [batch * rows, stride] activations; norm_weight
- * BF16 [Dv].  (Dk, Dv) in {(128, 128), (64, 64), (32, 32), (64, 128), (128, 64)}. */
+ * BF16 [Dv].  (Dk, Dv) in {(128, 128), (64, 64), (32, 32), (64, 128), (128, 64)}.
+ * A call of 64 rows or more over 128 x 128 heads takes sixteen rows at a time on the matrix cores and needs
+ * 2,304 bytes of workspace per (sequence, value head, sixteen rows): under stream capture that workspace must
+ * already be there (nvmai_hip_ctx_reserve, or the same call made eagerly once), else the call returns
+ * NVMAI_ERR_SCRATCH and launches nothing -- it does not fall back to the row-by-row kernels, whose summation
+ * order (and so the last bits) would differ from the eager call's. */
 int nvmai_hip_gdn_delta_gated_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai_gdn_config* config,
                                    const void* conv_out, uint32_t conv_out_stride, const void* a_proj,
                                    const void* b_proj, uint32_t ab_stride, const uint16_t* a_log,

@@ -45,54 +45,64 @@ void launch_gated_norm_rows(const GdnDeltaParams& p, hipStream_t s) {
     gdn_gated_norm_rows_kernel<ACT><<<ngrid, 256, 0, s>>>(p.out, p.out_stride, p.z, p.z_stride, p.norm_w, p.sh);
 }
 
+// Returns 1 = launched, 0 = not a shape or alignment this form takes (the caller goes on to the row-by-row
+// kernels), or a negative status: the workspace could not be had -- in particular NVMAI_ERR_SCRATCH when it
+// would have to grow while the stream is being captured.  That is handed back to the caller instead of taking
+// the other kernels silently: their summation order differs, so a captured call would not give the bits of
+// the eager one.  Reserve sizeof(GdnChunkPrep) = 2,304 bytes * batch * value heads * ceil(rows / 16) with
+// nvmai_hip_ctx_reserve (or run the same call eagerly once) before capturing.
 template <int ACT, int DK, int DV>
-bool launch_delta_chunked(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
-    if (DK != 128 || DV != 128) return false;
+int launch_delta_chunked(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
+    if (DK != 128 || DV != 128) return 0;
     const uint32_t nchunks = (p.sh.rows + 15) / 16;
     const size_t count = (size_t)p.sh.batch * p.sh.v_heads * nchunks;
     if (!ctx || nchunks > 65535 || p.sh.batch > 65535 || (p.sh.rows + 1) / 2 > 65535 || !aligned16(p.conv_out) || p.conv_stride % 8 ||
         (!state_bf16 && !aligned16(p.state)) || (reinterpret_cast<uintptr_t>(p.state) & 7u))
-        return false;
-    if (ws_begin(ctx, (nvmai_stream)s, ws_round(count * sizeof(GdnChunkPrep))) != NVMAI_OK) return false;
+        return 0;
+    const int ws_rc = ws_begin(ctx, (nvmai_stream)s, ws_round(count * sizeof(GdnChunkPrep)));
+    if (ws_rc != NVMAI_OK) return ws_rc;
     GdnChunkPrep* prep = ws_take<GdnChunkPrep>(ctx, count);
     gdn_chunk_prep_kernel<ACT, 128><<<dim3(nchunks, p.sh.v_heads, p.sh.batch), 64, 0, s>>>(p, prep, nchunks);
     const dim3 cgrid(p.sh.v_heads, p.sh.batch, 128 / 16);
     if (state_bf16) gdn_chunk_delta_kernel<ACT, 128, 128, true><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
     else gdn_chunk_delta_kernel<ACT, 128, 128, false><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
     launch_gated_norm_rows<ACT>(p, s);
-    return true;
+    return 1;
 }
 
 template <int ACT, int DK, int DV>
-void launch_delta(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
+int launch_delta(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
     const dim3 grid(p.sh.v_heads, p.sh.batch);
-    if (p.sh.rows >= GDN_CHUNKED_FROM && launch_delta_chunked<ACT, DK, DV>(ctx, p, state_bf16, s)) return;
+    if (p.sh.rows >= GDN_CHUNKED_FROM) {
+        const int rc = launch_delta_chunked<ACT, DK, DV>(ctx, p, state_bf16, s);
+        if (rc != 0) return rc < 0 ? rc : NVMAI_OK;
+    }
     if (p.sh.rows >= GDN_ROWS_PARALLEL_FROM && (p.sh.rows + 1) / 2 <= 65535 && aligned16(p.conv_out) && p.conv_stride % 8 == 0) {
         const dim3 rgrid(p.sh.v_heads, p.sh.batch, DV / 16);      // one group of sixteen state rows per block
         if (state_bf16) gdn_delta_rows_kernel<ACT, DK, DV, true, 1><<<rgrid, 256, 0, s>>>(p);
         else gdn_delta_rows_kernel<ACT, DK, DV, false, 1><<<rgrid, 256, 0, s>>>(p);
         launch_gated_norm_rows<ACT>(p, s);
-        return;
+        return NVMAI_OK;
     }
     if (DK == 128 && DV == 128 && aligned16(p.state)) {       // the production head, state rows in 16-byte pieces
         if (state_bf16) gdn_delta_gated_kernel<ACT, DK, DV, true, DK == 128><<<grid, 256, 0, s>>>(p);
         else gdn_delta_gated_kernel<ACT, DK, DV, false, DK == 128><<<grid, 256, 0, s>>>(p);
-        return;
+        return NVMAI_OK;
     }
     if (state_bf16) gdn_delta_gated_kernel<ACT, DK, DV, true><<<grid, 256, 0, s>>>(p);
     else gdn_delta_gated_kernel<ACT, DK, DV, false><<<grid, 256, 0, s>>>(p);
+    return NVMAI_OK;
 }
 
 template <int ACT>
 int launch_delta_shape(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
     const uint32_t dk = p.sh.dk, dv = p.sh.dv;
-    if (dk == 128 && dv == 128) launch_delta<ACT, 128, 128>(ctx, p, state_bf16, s);
-    else if (dk == 64 && dv == 64) launch_delta<ACT, 64, 64>(ctx, p, state_bf16, s);
-    else if (dk == 32 && dv == 32) launch_delta<ACT, 32, 32>(ctx, p, state_bf16, s);
-    else if (dk == 64 && dv == 128) launch_delta<ACT, 64, 128>(ctx, p, state_bf16, s);
-    else if (dk == 128 && dv == 64) launch_delta<ACT, 128, 64>(ctx, p, state_bf16, s);
-    else return NVMAI_ERR_UNSUPPORTED;
-    return NVMAI_OK;
+    if (dk == 128 && dv == 128) return launch_delta<ACT, 128, 128>(ctx, p, state_bf16, s);
+    if (dk == 64 && dv == 64) return launch_delta<ACT, 64, 64>(ctx, p, state_bf16, s);
+    if (dk == 32 && dv == 32) return launch_delta<ACT, 32, 32>(ctx, p, state_bf16, s);
+    if (dk == 64 && dv == 128) return launch_delta<ACT, 64, 128>(ctx, p, state_bf16, s);
+    if (dk == 128 && dv == 64) return launch_delta<ACT, 128, 64>(ctx, p, state_bf16, s);
+    return NVMAI_ERR_UNSUPPORTED;
 }
 
 }  // namespace

@@ -1,5 +1,6 @@
 // Entry points of the decode-side MoE path: context, quantizer, affine GEMV,
 // router top-k, routed phase 1 / phase 2, shared expert, fused decode layer.
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <new>
@@ -18,20 +19,24 @@ namespace {
 constexpr size_t STATIC_SCRATCH_BYTES = (size_t)4 << 20;
 static __device__ __align__(256) __attribute__((used)) uint8_t scratch[STATIC_SCRATCH_BYTES];
 constexpr int STATIC_SCRATCH_MAX_DEVICES = 64;
-uint8_t* g_static_scratch[STATIC_SCRATCH_MAX_DEVICES];   // device address of `scratch` on each device, nullptr = not asked yet
+// Device address of `scratch` on each device, nullptr = not asked yet.  Contexts may be created from several
+// threads: the slots are atomics (every thread that fills one stores the same address, so no lock is needed).
+std::atomic<uint8_t*> g_static_scratch[STATIC_SCRATCH_MAX_DEVICES];
 
 // The device address of this device's copy of the array (the device must be current).
 int static_scratch_ptr(int device, uint8_t** out) {
     if (device < 0 || device >= STATIC_SCRATCH_MAX_DEVICES) return NVMAI_ERR_INVALID_ARG;
-    if (!g_static_scratch[device]) {
+    uint8_t* known = g_static_scratch[device].load(std::memory_order_acquire);
+    if (!known) {
         void* ptr = nullptr;
         if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
             (void)hipGetLastError();
             return NVMAI_ERR_HIP;
         }
-        g_static_scratch[device] = static_cast<uint8_t*>(ptr);
+        known = static_cast<uint8_t*>(ptr);
+        g_static_scratch[device].store(known, std::memory_order_release);
     }
-    *out = g_static_scratch[device];
+    *out = known;
     return NVMAI_OK;
 }
 
@@ -1284,6 +1289,10 @@ extern "C" int nvmai_hip_moe_decode_layer_noalloc(nvmai_hip_ctx* ctx, nvmai_stre
                                                   uint32_t* out_idx, uint16_t* out_w, uint32_t* stats) {
     if (!ctx) return NVMAI_ERR_INVALID_ARG;
     if (!ctx->static_scratch) return NVMAI_ERR_HIP;     // the symbol lookup failed at context creation
+    // every device holds its own copy of the array at its own address: the address this context keeps is
+    // only good while its device is the current one
+    int current = -1;
+    if (hipGetDevice(&current) != hipSuccess || current != ctx->device) return NVMAI_ERR_INVALID_ARG;
     return decode_layer_impl(ctx, stream, L, x, x_stride, n_tokens, y, y_stride, out_idx, out_w, stats,
                              ctx->static_scratch, STATIC_SCRATCH_BYTES);
 }

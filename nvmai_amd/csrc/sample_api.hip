@@ -102,10 +102,14 @@ extern "C" int nvmai_hip_repetition_penalty(nvmai_hip_ctx* ctx, nvmai_stream str
     if (n_ids == 0 || penalty == 1.0f) return NVMAI_OK;          // Sampler.swift:181
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((n_ids + 255) / 256);
+    const int rc = ws_begin(ctx, stream, ws_round((size_t)n_ids * 2));     // the snapshot: two bytes per history entry
+    if (rc) return rc;
+    uint16_t* snapshot = ws_take<uint16_t>(ctx, n_ids);
+    repetition_penalty_gather_kernel<<<grid, 256, 0, s>>>((const uint16_t*)logits, v, history_ids, n_ids, snapshot);
     if (ctx->act == ACT_BF16)
-        repetition_penalty_kernel<ACT_BF16><<<grid, 256, 0, s>>>((uint16_t*)logits, v, history_ids, n_ids, penalty, logit_softcap);
+        repetition_penalty_kernel<ACT_BF16><<<grid, 256, 0, s>>>((uint16_t*)logits, v, history_ids, n_ids, snapshot, penalty, logit_softcap);
     else
-        repetition_penalty_kernel<ACT_FP16><<<grid, 256, 0, s>>>((uint16_t*)logits, v, history_ids, n_ids, penalty, logit_softcap);
+        repetition_penalty_kernel<ACT_FP16><<<grid, 256, 0, s>>>((uint16_t*)logits, v, history_ids, n_ids, snapshot, penalty, logit_softcap);
     return launch_status();
 }
 

@@ -472,20 +472,30 @@ __global__ __launch_bounds__(256) void sample_generic_kernel(const uint16_t* pro
     }
 }
 
-// Sampler.applyRepetitionPenaltyInPlace (Sampler.swift:259-293) on the device: one thread per history
-// id.  The reference walks the distinct ids of its history dictionary; here a thread drops out when
-// an earlier entry of the list holds the same id, so a list with repeats gives the same result.
-// Without a softcap the new logit is one IEEE division or product, rounded to the activation type.
+// Sampler.applyRepetitionPenaltyInPlace (Sampler.swift:259-293) on the device, one thread per history
+// entry, in two launches.  The reference walks the distinct ids of its history dictionary; a list may
+// hold an id many times.  The first launch copies the logit of every entry into a snapshot; the second
+// writes the penalised value computed from the snapshot: entries with the same id write the same bits,
+// so repeats need no search for an earlier occurrence (that search was a chain of up to n dependent
+// reads in the last thread: quadratic in the history, which reaches 128K tokens).  Without a softcap
+// the new logit is one IEEE division or product, rounded to the activation type.
+__global__ __launch_bounds__(256) void repetition_penalty_gather_kernel(const uint16_t* logits, uint32_t v, const int32_t* ids,
+                                                                        uint32_t n_ids, uint16_t* snapshot) {
+    const uint32_t j = blockIdx.x * 256u + threadIdx.x;
+    if (j >= n_ids) return;
+    const int32_t id = ids[j];
+    snapshot[j] = (id < 0 || (uint32_t)id >= v) ? (uint16_t)0 : logits[id];
+}
+
 template <int ACT>
 __global__ __launch_bounds__(256) void repetition_penalty_kernel(uint16_t* logits, uint32_t v, const int32_t* ids,
-                                                                 uint32_t n_ids, float penalty, float softcap) {
+                                                                 uint32_t n_ids, const uint16_t* snapshot, float penalty,
+                                                                 float softcap) {
     const uint32_t j = blockIdx.x * 256u + threadIdx.x;
     if (j >= n_ids) return;
     const int32_t id = ids[j];
     if (id < 0 || (uint32_t)id >= v) return;
-    for (uint32_t h = 0; h < j; ++h)
-        if (ids[h] == id) return;
-    const float z = act_to_f32<ACT>(logits[id]);
+    const float z = act_to_f32<ACT>(snapshot[j]);
     float out;
     if (softcap > 0.0f) {
         const float capped = softcap * tanhf(z / softcap);

@@ -25,8 +25,9 @@ class HybridConfig:
     def __init__(self, hidden=2048, layers=40, full_every=4, num_heads=16, num_kv_heads=2, head_dim=256,
                  rotary_dim=64, rope_theta=1e7, gdn=(16, 32, 128, 128, 4), num_experts=256, top_k=8,
                  moe_intermediate=512, vocab=248320, expert_bits=4, attn_bits=4, kv_bits=8, head_bits=16,
-                 embed_bits=4, rms_eps=1e-6, logit_softcap=0.0, gdn_state_bf16=True):
+                 embed_bits=4, rms_eps=1e-6, logit_softcap=0.0, gdn_state_bf16=True, full_mask=None):
         self.hidden, self.layers, self.full_every = hidden, layers, full_every
+        self.full_mask = None if full_mask is None else [bool(v) for v in full_mask]   # per layer: full attention?
         self.num_heads, self.num_kv_heads, self.head_dim = num_heads, num_kv_heads, head_dim
         self.rotary_dim, self.rope_theta, self.gdn = rotary_dim, rope_theta, gdn
         self.num_experts, self.top_k, self.moe_intermediate, self.vocab = num_experts, top_k, moe_intermediate, vocab
@@ -35,7 +36,10 @@ class HybridConfig:
         self.rms_eps, self.logit_softcap, self.gdn_state_bf16 = rms_eps, logit_softcap, gdn_state_bf16
 
     def is_linear(self, layer):
-        """layerIsLinear: every full_every-th layer is full attention, the others gated DeltaNet."""
+        """layerIsLinear (ModelTypes.swift:288-289): by the model's layer mask when one was given, else every
+        full_every-th layer is full attention and the others gated DeltaNet."""
+        if self.full_mask is not None:
+            return not self.full_mask[layer]
         return (layer + 1) % self.full_every != 0
 
     @property
@@ -134,6 +138,109 @@ class HybridWeights:
                                           ops.rows_desc(16, w["router"]), pool[:cfg.num_experts], pool[cfg.num_experts],
                                           ops.rows_desc(8, *w["gate"]))
             self.layers.append(w)
+
+
+def _from_gturbo(cls, ctx, model, gdn=None, kv_bits=8, gdn_state_bf16=True):
+    """HybridWeights (and its HybridConfig) from an opened model directory (gturbo.GTurboModel): the resident
+    tensors bound by the reference's names (Model.swift:137-306), the matrices of a projection group stacked
+    as the rows of one matrix (one launch per group), each layer's experts in HBM with the shared expert as
+    the pool's last row.  The manifest carries no gated-DeltaNet head shape (the reference compiles it in,
+    ModelTypes.swift:162-204): value heads, value head size and conv taps are read off the tensor shapes,
+    key heads assume key head size = value head size unless gdn = (Hk, Hv, Dk, Dv, taps) says otherwise.
+    Returns (config, weights)."""
+    import numpy as np
+
+    from . import gturbo as G
+    a, q = model.manifest.arch, model.manifest.quant
+    if q is None:
+        raise G.ModelError("indexCorrupt", "manifest.quant is required by the executable runtime schema")
+    if not model.shared_matches_routed():
+        raise G.ModelError("unsupportedArch", "the decode step runs the shared expert in the routed experts' launches: a shared "
+                           "expert of another width is run per layer through gturbo.GTurboMoEBlock")
+    mask = a["fullAttentionLayerMask"]
+    if any(v == 0 for v in mask):
+        raise G.ModelError("unsupportedArch", "sliding-window layers")
+    D, layers = a["hiddenSize"], a["numLayers"]
+    dev = ctx.device
+    keep = []
+
+    def t3(name, bits):
+        """(codes, scales, biases) device tensors of an affine matrix, or (BF16 bits, None, None) of a dense one."""
+        w, s_, b_, e = model.resident(name)
+        up = lambda x, dt: torch.from_numpy(np.array(x)).to(dev).view(dt)
+        if e.dtype == 1:
+            return (up(w, torch.int16).view(e.shape[0], -1), None, None), 16, e.shape
+        rows = e.shape[0]
+        return (up(w, torch.uint8).view(rows, -1), up(s_.view(np.uint8), torch.int16).view(rows, -1),
+                up(b_.view(np.uint8), torch.int16).view(rows, -1)), bits, e.shape
+
+    def bf(name):
+        w, _, _, e = model.resident(name)
+        if e.dtype != 1:
+            raise G.ModelError("indexCorrupt", "%s must be BF16" % name)
+        return torch.from_numpy(np.array(w)).to(dev).view(torch.int16)
+
+    def stack(names, bits):
+        parts = [t3(n, bits) for n in names]
+        if any(p[1] != bits for p in parts):
+            raise G.ModelError("indexCorrupt", "%s: the matrices of one projection group differ in format" % names[0])
+        return tuple(torch.cat([p[0][j] for p in parts]).contiguous() for j in range(3)), [p[2][0] for p in parts]
+
+    first_linear = next((L for L in range(layers) if mask[L] == 2), None)
+    if gdn is None and first_linear is not None:
+        p = G.LAYER_PREFIX % first_linear
+        _, _, _, ea = model.resident(p + "linear_attn.in_proj_a.weight")
+        _, _, _, en = model.resident(p + "linear_attn.norm.weight")
+        _, _, _, eq = model.resident(p + "linear_attn.in_proj_qkv.weight")
+        _, _, _, ec = model.resident(p + "linear_attn.conv1d.weight")
+        vh, dv, qkv_rows = ea.shape[0], en.shape[0], eq.shape[0]
+        conv_count = int(np.prod([n for n in ec.shape if n]))      # the index pads shapes with zeros
+        if (qkv_rows - vh * dv) % (2 * dv) or conv_count % qkv_rows:
+            raise G.ModelError("indexCorrupt", "gated-DeltaNet tensor shapes do not give a head layout; pass gdn=")
+        gdn = ((qkv_rows - vh * dv) // (2 * dv), vh, dv, dv, conv_count // qkv_rows)
+    attn_bits, embed_bits, expert_bits = q["attention"].weightBits, q["embedding"].weightBits, q["routedExpert"].weightBits
+    self = cls.__new__(cls)
+    self.ctx = ctx
+    self.embed, _, _ = t3("language_model.model.embed_tokens.weight", embed_bits)
+    self.lm_head, head_bits, _ = t3("language_model.lm_head.weight", embed_bits)
+    self.final_norm = bf("language_model.model.norm.weight")
+    cfg = HybridConfig(hidden=D, layers=layers, num_heads=a["numHeads"], num_kv_heads=a["numFullKVHeads"],
+                       head_dim=a["fullHeadDim"], rotary_dim=int(round(a["partialRotaryFactor"] * a["fullHeadDim"])),
+                       rope_theta=a["fullRopeTheta"], gdn=gdn or (1, 1, 32, 32, 1), num_experts=a["numExperts"],
+                       top_k=a["topKExperts"], moe_intermediate=a["moeIntermediateSize"], vocab=a["vocabSize"],
+                       expert_bits=expert_bits, attn_bits=attn_bits, kv_bits=kv_bits, head_bits=head_bits,
+                       embed_bits=embed_bits, logit_softcap=a["finalLogitSoftcap"], gdn_state_bf16=gdn_state_bf16,
+                       full_mask=[v == 1 for v in mask])
+    self.cfg = cfg
+    self.layers = []
+    for L in range(layers):
+        p = G.LAYER_PREFIX % L
+        w = dict(in_norm=bf(p + "input_layernorm.weight"), post_norm=bf(p + "post_attention_layernorm.weight"))
+        if cfg.is_linear(L):
+            w["in_proj"], rows = stack([p + n for n in G.LINEAR_PROJECTIONS], attn_bits)
+            if rows != [cfg.gdn_qkv_dim, cfg.gdn_value_dim, gdn[1], gdn[1]]:
+                raise G.ModelError("indexCorrupt", "layer %d: linear_attn projection rows %s do not fit the head layout %s"
+                                   % (L, rows, gdn))
+            w["out_proj"], _, _ = t3(p + "linear_attn.out_proj.weight", attn_bits)
+            w["conv_w"] = bf(p + "linear_attn.conv1d.weight").view(cfg.gdn_qkv_dim, gdn[4])
+            w["a_log"], w["dt_bias"] = bf(p + "linear_attn.A_log"), bf(p + "linear_attn.dt_bias")
+            w["gdn_norm"] = bf(p + "linear_attn.norm.weight")
+        else:
+            w["qkv"], rows = stack([p + n for n in G.FULL_PROJECTIONS], attn_bits)
+            if rows != [2 * cfg.q_dim, cfg.kv_dim, cfg.kv_dim]:
+                raise G.ModelError("indexCorrupt", "layer %d: self_attn projection rows %s do not fit %d heads of %d"
+                                   % (L, rows, cfg.num_heads, cfg.head_dim))
+            w["o_proj"], _, _ = t3(p + "self_attn.o_proj.weight", attn_bits)
+            w["q_norm"], w["k_norm"] = bf(p + "self_attn.q_norm.weight"), bf(p + "self_attn.k_norm.weight")
+        w["pool"] = model.expert_pool(L, dev, with_shared=True)
+        w["moe"], held = model.moe_layer(L, w["pool"], dev)
+        keep.append(held)
+        self.layers.append(w)
+    self._keep = keep
+    return cfg, self
+
+
+HybridWeights.from_gturbo = classmethod(_from_gturbo)
 
 
 class HybridDecoder:

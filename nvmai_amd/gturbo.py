@@ -803,6 +803,123 @@ class GTurboMoEBlock:
         return out
 
 
+# ------------------------------------------------------------------------------------ whole-model binding
+# The resident tensors of the hybrid model by the reference's names (Model.swift:137-306; the schema
+# validateLayerTensors checks, Model.swift:760-840).  A full-attention layer keeps q_proj (gate-packed
+# [query; gate], 2 * heads * headDim rows), k_proj, v_proj; a gated-DeltaNet layer keeps in_proj_qkv,
+# in_proj_z, in_proj_a, in_proj_b: the decode step here runs each group as ONE launch, so the binder lays
+# the matrices of a group out as the rows of one matrix, in this order.
+LAYER_PREFIX = "language_model.model.layers.%d."
+FULL_PROJECTIONS = ("self_attn.q_proj.weight", "self_attn.k_proj.weight", "self_attn.v_proj.weight")
+LINEAR_PROJECTIONS = ("linear_attn.in_proj_qkv.weight", "linear_attn.in_proj_z.weight", "linear_attn.in_proj_a.weight",
+                      "linear_attn.in_proj_b.weight")
+
+
+def hybrid_tensor_names(layer, full):
+    """Every resident tensor name of one layer, in the reference's order of lookup."""
+    p = LAYER_PREFIX % layer
+    names = [p + "input_layernorm.weight", p + "post_attention_layernorm.weight", p + "mlp.gate.weight",
+             p + "mlp.shared_expert_gate.weight"] + [p + "mlp.shared_expert.%s.weight" % q for q in ("gate_proj", "up_proj", "down_proj")]
+    if full:
+        names += [p + n for n in FULL_PROJECTIONS] + [p + "self_attn.o_proj.weight", p + "self_attn.q_norm.weight",
+                                                       p + "self_attn.k_norm.weight"]
+    else:
+        names += [p + n for n in LINEAR_PROJECTIONS] + [p + "linear_attn.out_proj.weight", p + "linear_attn.conv1d.weight",
+                                                         p + "linear_attn.A_log", p + "linear_attn.dt_bias", p + "linear_attn.norm.weight"]
+    return names
+
+
+def write_hybrid_model(directory, cfg, weights, model_id="nvmai-amd-synthetic"):
+    """A decoder.HybridWeights instance (config decoder.HybridConfig) as a model directory under the reference's
+    tensor names: what the repack tool would write for this model (sources/NVMAIRepack), reduced to what the format
+    requires.  Rows of a fused projection group are split back into the reference's separate matrices."""
+    D, F, E = cfg.hidden, cfg.moe_intermediate, cfg.num_experts
+    host = lambda t: t.detach().cpu().numpy()
+    raw = lambda t: np.ascontiguousarray(host(t)).view(np.uint8).reshape(-1).tobytes()
+    resident = []
+
+    def affine(name, t3, rows, cols, r0=0, r1=None):
+        r1 = rows if r1 is None else r1
+        w, s, b = t3
+        w2, s2, b2 = w.reshape(rows, -1), s.reshape(rows, -1), b.reshape(rows, -1)
+        resident.append((name, 0, (r1 - r0, cols), raw(w2[r0:r1]), raw(s2[r0:r1]), raw(b2[r0:r1])))
+
+    def bf16(name, t, shape):
+        resident.append((name, 1, tuple(shape), raw(t), None, None))
+
+    affine("language_model.model.embed_tokens.weight", weights.embed, cfg.vocab, D)
+    if cfg.head_bits == 16:
+        bf16("language_model.lm_head.weight", weights.lm_head[0], (cfg.vocab, D))
+    else:
+        affine("language_model.lm_head.weight", weights.lm_head, cfg.vocab, D)
+    bf16("language_model.model.norm.weight", weights.final_norm, (D,))
+    off, used = _cpu_expert_offsets(D, F, cfg.expert_bits)
+    sizes = [F * D * cfg.expert_bits // 8, F * (D // 64) * 2, F * (D // 64) * 2] * 2 + \
+            [D * F * cfg.expert_bits // 8, D * (F // 64) * 2, D * (F // 64) * 2]
+    shapes = [(F, D), (F, D // 64), (F, D // 64)] * 2 + [(D, F), (D, F // 64), (D, F // 64)]
+    tensors = {r: SubTensorEntry(off[i], sizes[i], "BF16" if "_" in r else "U32", shapes[i], None if "_" in r else cfg.expert_bits)
+               for i, r in enumerate(_ROLES)}
+    stride = (used + ALIGNMENT_BYTES - 1) // ALIGNMENT_BYTES * ALIGNMENT_BYTES
+    lays = []
+    kh, vh, dk, dv, taps = cfg.gdn
+    for L, w in enumerate(weights.layers):
+        p = LAYER_PREFIX % L
+        bf16(p + "input_layernorm.weight", w["in_norm"], (D,))
+        bf16(p + "post_attention_layernorm.weight", w["post_norm"], (D,))
+        bf16(p + "mlp.gate.weight", w["router"], (E, D))
+        affine(p + "mlp.shared_expert_gate.weight", w["gate"], 1, D)
+        pool = host(w["pool"])
+        blobs = np.zeros((E, stride), np.uint8)
+        blobs[:, :used] = pool[:E, :used]
+        lays.append({"blobs": blobs, "tensors": tensors, "ranks": None})
+        shared = pool[E]
+        for i, (proj, rows, cols) in enumerate((("gate_proj", F, D), ("up_proj", F, D), ("down_proj", D, F))):
+            cut = lambda j: shared[off[3 * i + j]:off[3 * i + j] + sizes[3 * i + j]].tobytes()
+            resident.append((p + "mlp.shared_expert.%s.weight" % proj, 0, (rows, cols), cut(0), cut(1), cut(2)))
+        if cfg.is_linear(L):
+            rows_of = (cfg.gdn_qkv_dim, cfg.gdn_value_dim, vh, vh)
+            total, at = sum(rows_of), 0
+            for name, n in zip(LINEAR_PROJECTIONS, rows_of):
+                affine(p + name, w["in_proj"], total, D, at, at + n)
+                at += n
+            affine(p + "linear_attn.out_proj.weight", w["out_proj"], D, cfg.gdn_value_dim)
+            bf16(p + "linear_attn.conv1d.weight", w["conv_w"], (cfg.gdn_qkv_dim, taps))
+            bf16(p + "linear_attn.A_log", w["a_log"], (vh,))
+            bf16(p + "linear_attn.dt_bias", w["dt_bias"], (vh,))
+            bf16(p + "linear_attn.norm.weight", w["gdn_norm"], (dv,))
+        else:
+            rows_of = (2 * cfg.q_dim, cfg.kv_dim, cfg.kv_dim)
+            total, at = sum(rows_of), 0
+            for name, n in zip(FULL_PROJECTIONS, rows_of):
+                affine(p + name, w["qkv"], total, D, at, at + n)
+                at += n
+            affine(p + "self_attn.o_proj.weight", w["o_proj"], D, cfg.q_dim)
+            bf16(p + "self_attn.q_norm.weight", w["q_norm"], (cfg.head_dim,))
+            bf16(p + "self_attn.k_norm.weight", w["k_norm"], (cfg.head_dim,))
+    slot = lambda b: {"weightBits": b, "scheme": "affine", "scaleType": "bf16", "biasType": "bf16", "groupSize": 64}
+    quant = {"embedding": slot(cfg.embed_bits), "attention": slot(cfg.attn_bits), "router": slot(8),
+             "sharedExpert": slot(cfg.expert_bits), "routedExpert": slot(cfg.expert_bits)}
+    arch = {"hiddenSize": D, "ffnIntermediate": F, "moeIntermediateSize": F, "numHeads": cfg.num_heads,
+            "numKVHeads": cfg.num_kv_heads, "numFullKVHeads": cfg.num_kv_heads, "headDim": cfg.head_dim,
+            "fullHeadDim": cfg.head_dim, "vocabSize": cfg.vocab, "slidingWindow": 0,
+            "finalLogitSoftcap": float(cfg.logit_softcap), "ropeTheta": float(cfg.rope_theta),
+            "fullRopeTheta": float(cfg.rope_theta), "partialRotaryFactor": cfg.rotary_dim / cfg.head_dim,
+            "numLayers": cfg.layers, "numExperts": E, "topKExperts": cfg.top_k, "tieWordEmbeddings": False,
+            "attentionKEqV": False, "hiddenActivation": "silu",
+            "fullAttentionLayerMask": [2 if cfg.is_linear(L) else 1 for L in range(cfg.layers)]}
+    return write_model(directory, arch, quant, lays, resident, model_id=model_id)
+
+
+def _cpu_expert_offsets(d, f, bits):
+    """CPUExpertFFN.Offsets(d:f:) (CPUExpertFFN.swift:42-59): (nine offsets, blob bytes)."""
+    sizes = [f * d * bits // 8, f * (d // 64) * 2, f * (d // 64) * 2] * 2 + [d * f * bits // 8, d * (f // 64) * 2, d * (f // 64) * 2]
+    off, at = [], 0
+    for n in sizes:
+        off.append(at)
+        at += n
+    return off, at
+
+
 # ------------------------------------------------------------------------------------ writer (tests, tools)
 def write_model(directory, arch, quant, layers, resident, model_id="toy", flags=None):
     """Writes a model directory the readers above accept: `layers` = list of dicts

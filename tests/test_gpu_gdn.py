@@ -180,6 +180,45 @@ def test_gdn_long_call_on_the_matrix_cores_batch_and_state_types(nv, ctx, bf16_s
     assert (state_a.float() - state_b.float()).abs().max().item() <= 5e-2
 
 
+def test_gdn_long_call_captured_in_a_graph_equals_the_eager_call(nv):
+    # 100 rows of a 128 x 128 head take the chunked form, which carves 2,304 bytes per (sequence, head, chunk) out of
+    # the context's workspace: a fresh context reserves them, captures the call, and every replay gives the bits of
+    # the eager call (outputs, tail, state) -- a capture may not fall back to the row-by-row kernels
+    say("gdn chunked call under a graph")
+    cfg, rows = (2, 4, 128, 128, 4), 100
+    eager_ctx = nv.Context(0, 0)
+    fx = _fixture(cfg, rows, 0x6A, 0)
+    gdn_e = nv.GDN(eager_ctx, *cfg)
+    tail_e, state_e = gdn_e.new_state()
+    want = _gpu_rows(nv, eager_ctx, gdn_e, fx, tail_e, state_e, 0, rows).clone()
+    torch.cuda.synchronize()
+    ctx = nv.Context(0, 0)
+    ctx.reserve(1 << 20)                                # 4 heads x 7 chunks x 2,304 bytes, and room to spare
+    gdn = nv.GDN(ctx, *cfg)
+    tail, state = gdn.new_state()
+    ins = [act_tensor(fx[k][:rows], ctx) for k in ("qkv", "a", "b", "z")]
+    w = [_bits(fx[k]) for k in ("conv_w", "a_log", "dt_bias", "norm_w")]
+    conv = torch.empty_like(ins[0])
+    out = torch.empty((rows, gdn.value_dim), dtype=ctx.dtype, device="cuda")
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            gdn.encode_conv_norm(ins[0], tail, w[0], conv_out=conv, rows=rows)
+            gdn.encode_delta_gated_norm(conv, ins[1], ins[2], w[1], w[2], state, ins[3], w[3], out=out, rows=rows)
+    torch.cuda.synchronize()
+    for trial in range(3):
+        tail.zero_(); state.zero_(); out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), trial
+        assert torch.equal(tail, tail_e) and torch.equal(state, state_e), trial
+    ctx.close()
+    eager_ctx.close()
+
+
 @pytest.mark.parametrize("rows", [8, 37, 80])
 def test_gdn_gated_norm_in_16_byte_pieces_same_bits(nv, ctx, rows):
     # heads of 128 values take the gated output norm in 16-byte pieces, sixteen lanes per (row, head);

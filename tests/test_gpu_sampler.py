@@ -227,6 +227,33 @@ def test_sampler_sample_front_end(nv, ctx):
         nv.Sampler(ctx, v, 0.0).sample(logits, [], nv.GenerationConfig(top_k=300), 0)
 
 
+def test_repetition_penalty_long_history_with_repeats(nv, ctx):
+    # a history of 131,072 ids drawn from 5,000 distinct ones (every id about 26 times, plus ids out of range):
+    # every distinct id is penalised exactly once, whatever the number and the order of its occurrences --
+    # the oracle walks the distinct ids as the reference's dictionary does (Sampler.swift:259-293)
+    say("repetition penalty, long history", ctx.act)
+    rng = np.random.default_rng(131072)
+    v = 248320
+    base = round_act(gauss(rng, (v,), 3.0), ctx.act)
+    pool_ids = rng.choice(v, 5000, replace=False)
+    history = rng.choice(pool_ids, 131072).astype(np.int32)
+    history[::1000] = -1
+    history[500::1000] = v + 7
+    for softcap in (0.0, 30.0):
+        logits = act_tensor(base, ctx)
+        nv.ops.repetition_penalty(ctx, logits, dev(history), 1.3, softcap)
+        torch.cuda.synchronize()
+        distinct = [int(i) for i in dict.fromkeys(history.tolist()) if 0 <= i < v]
+        want = O.repetition_penalty(base, ctx.act, distinct, 1.3, softcap)
+        if softcap == 0.0:
+            assert np.array_equal(act_np(logits), want)                     # one IEEE operation per id
+        else:
+            assert np.abs(act_np(logits) - want).max() <= 2 ** -5           # tanh / atanh from two libraries
+        untouched = np.ones(v, bool)
+        untouched[distinct] = False
+        assert np.array_equal(act_np(logits)[untouched], base[untouched])
+
+
 def test_sampler_sample_reference_properties(nv, ctx):
     # The reference's own Sampler tests (tests/NVMAI/Core/Runtime/Generation/SamplerTests.swift:68-197)
     # through the C ABI, default softcap 30 as there.
