@@ -174,9 +174,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # bits, batch or tokens); other configurations report null.
 MEASURED_TRAFFIC_BYTES = {
     ("decode", 8, 32): ((181300 * 2.00 + 1229 * 1.00) * 1024, "profiles/expert_rows_fast_decode_configs1_8bit_batch32.txt"),
-    ("prefill", 4, 4096): ((279390 * 2.00 + 36142 * 1.00) * 1024, "profiles/prefill_gemm_kernel_configs2_4bit_4096tokens.txt"),
-    ("attention", 8, 8, 131072): ((565650 * 2.00 + 4383 * 1.00) * 1024, "profiles/attn_partial_mfma_kernel_configs3_8bit_128k_batch8.txt"),
-    ("attention", 4, 8, 131072): ((295900 * 2.00 + 4356 * 1.00) * 1024, "profiles/attn_partial_mfma_kernel_configs3_8bit_128k_batch8.txt"),
+    ("prefill", 4, 4096): ((246530 * 2.00 + 36144 * 1.00) * 1024, "profiles/prefill_gemm_kernel_configs2_4bit_4096tokens.txt"),
+    ("attention", 8, 8, 131072): ((557830 * 2.00 + 2176 * 1.00) * 1024, "profiles/attn_partial_mfma_kernel_configs3_8bit_128k_batch8.txt"),
+    ("attention", 4, 8, 131072): ((295590 * 2.00 + 4362 * 1.00) * 1024, "profiles/attn_partial_mfma_kernel_configs3_4bit_128k_batch8.txt"),
 }
 
 
