@@ -685,7 +685,9 @@ int nvmai_hip_gdn_conv_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, const nvmai
  * activations; a_log, dt_bias: BF16 [Hv]; z, out: [batch * rows, stride] activations; norm_weight
  * BF16 [Dv].  (Dk, Dv) in {(128, 128), (64, 64), (32, 32), (64, 128), (128, 64)}.
  * A call of 64 rows or more over 128 x 128 heads takes sixteen rows at a time on the matrix cores and needs
- * 2,304 bytes of workspace per (sequence, value head, sixteen rows): under stream capture that workspace must
+ * workspace: 2,304 bytes per (sequence, value head, sixteen rows), and in a BF16 context 8,192 bytes more per
+ * (sequence, value head, sixteen rows) plus 4,096 per (sequence, key head, sixteen rows) -- 103 MB for one
+ * sequence of 4096 rows with 32 value and 16 key heads.  Under stream capture that workspace must
  * already be there (nvmai_hip_ctx_reserve, or the same call made eagerly once), else the call returns
  * NVMAI_ERR_SCRATCH and launches nothing -- it does not fall back to the row-by-row kernels, whose summation
  * order (and so the last bits) would differ from the eager call's. */

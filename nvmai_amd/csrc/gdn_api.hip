@@ -3,6 +3,7 @@
 #include "ctx.hpp"
 #include "gdn_kernels.hpp"
 #include "gdn_chunk_kernels.hpp"
+#include "gdn_wy_kernels.hpp"
 
 using namespace nvmai;
 
@@ -27,7 +28,7 @@ GdnShape shape_of(const nvmai_gdn_config* c, uint32_t rows, uint32_t batch) {
 constexpr uint32_t GDN_ROWS_PARALLEL_FROM = 8;
 
 // From this many rows per sequence on the recurrence of a 128 x 128 head runs sixteen rows at a time on
-// the matrix cores (a launch more, and 2,304 bytes of workspace per head and chunk).
+// the matrix cores (one or two launches more, and workspace per head and chunk: launch_delta_chunked).
 constexpr uint32_t GDN_CHUNKED_FROM = 64;
 
 // The gated norm over the rows the recurrence left in out: heads of 128 values in 16-byte pieces where
@@ -49,8 +50,9 @@ void launch_gated_norm_rows(const GdnDeltaParams& p, hipStream_t s) {
 // kernels), or a negative status: the workspace could not be had -- in particular NVMAI_ERR_SCRATCH when it
 // would have to grow while the stream is being captured.  That is handed back to the caller instead of taking
 // the other kernels silently: their summation order differs, so a captured call would not give the bits of
-// the eager one.  Reserve sizeof(GdnChunkPrep) = 2,304 bytes * batch * value heads * ceil(rows / 16) with
-// nvmai_hip_ctx_reserve (or run the same call eagerly once) before capturing.
+// the eager one.  Reserve (sizeof(GdnChunkPrep) = 2,304 bytes, and with BF16 activations sizeof(GdnChunkWY) = 8,192
+// more) * batch * value heads * ceil(rows / 16), and with BF16 activations sizeof(GdnChunkKT) = 4,096 * batch * key
+// heads * ceil(rows / 16), with nvmai_hip_ctx_reserve (or run the same call eagerly once) before capturing.
 template <int ACT, int DK, int DV>
 int launch_delta_chunked(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state_bf16, hipStream_t s) {
     if (DK != 128 || DV != 128) return 0;
@@ -59,13 +61,27 @@ int launch_delta_chunked(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state
     if (!ctx || nchunks > 65535 || p.sh.batch > 65535 || (p.sh.rows + 1) / 2 > 65535 || !aligned16(p.conv_out) || p.conv_stride % 8 ||
         (!state_bf16 && !aligned16(p.state)) || (reinterpret_cast<uintptr_t>(p.state) & 7u))
         return 0;
-    const int ws_rc = ws_begin(ctx, (nvmai_stream)s, ws_round(count * sizeof(GdnChunkPrep)));
+    // BF16 activations: the chain on the 16-bit matrix instructions from operands prepared per chunk
+    // (8,192 bytes more per (sequence, value head, chunk) and 4,096 per (sequence, key head, chunk))
+    const bool wy_form = ACT == ACT_BF16;
+    const size_t count_k = (size_t)p.sh.batch * p.sh.k_heads * nchunks;
+    const size_t wy_bytes = wy_form ? ws_round(count * sizeof(GdnChunkWY)) + ws_round(count_k * sizeof(GdnChunkKT)) : 0;
+    const int ws_rc = ws_begin(ctx, (nvmai_stream)s, ws_round(count * sizeof(GdnChunkPrep)) + wy_bytes);
     if (ws_rc != NVMAI_OK) return ws_rc;
     GdnChunkPrep* prep = ws_take<GdnChunkPrep>(ctx, count);
     gdn_chunk_prep_kernel<ACT, 128><<<dim3(nchunks, p.sh.v_heads, p.sh.batch), 64, 0, s>>>(p, prep, nchunks);
     const dim3 cgrid(p.sh.v_heads, p.sh.batch, 128 / 16);
-    if (state_bf16) gdn_chunk_delta_kernel<ACT, 128, 128, true><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
-    else gdn_chunk_delta_kernel<ACT, 128, 128, false><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
+    if (wy_form) {
+        GdnChunkWY* wy = ws_take<GdnChunkWY>(ctx, count);
+        GdnChunkKT* kts = ws_take<GdnChunkKT>(ctx, count_k);
+        gdn_wy_prep_kernel<<<dim3(nchunks, p.sh.v_heads, p.sh.batch), 64, 0, s>>>(p, prep, wy, kts, nchunks);
+        if (state_bf16) gdn_wy_delta_kernel<true><<<cgrid, 64 * GDN_WY_WAVES, 0, s>>>(p, prep, wy, kts, nchunks);
+        else gdn_wy_delta_kernel<false><<<cgrid, 64 * GDN_WY_WAVES, 0, s>>>(p, prep, wy, kts, nchunks);
+    } else if (state_bf16) {
+        gdn_chunk_delta_kernel<ACT, 128, 128, true><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
+    } else {
+        gdn_chunk_delta_kernel<ACT, 128, 128, false><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
+    }
     launch_gated_norm_rows<ACT>(p, s);
     return 1;
 }

@@ -180,8 +180,30 @@ def test_gdn_long_call_on_the_matrix_cores_batch_and_state_types(nv, ctx, bf16_s
     assert (state_a.float() - state_b.float()).abs().max().item() <= 5e-2
 
 
+@pytest.mark.parametrize("rows", [64, 113])
+def test_gdn_long_call_matches_the_oracle_row_by_row(nv, ctx, rows):
+    # the chunked forms of the recurrence (fp32 matrix products with fp16 activations; split-BF16 operands and
+    # precomputed chunk operands with BF16 activations) against the oracle's row-by-row fp32 rule: outputs of
+    # every row, the conv tail and the recurrent state after the last one; 113 rows end in a ragged chunk
+    say("gdn long call vs oracle", ctx.act, rows)
+    cfg = (2, 4, 128, 128, 4)
+    fx = _fixture(cfg, rows, 0xC0 + rows, ctx.act)
+    gdn = nv.GDN(ctx, *cfg)
+    tail, state = gdn.new_state()
+    got = act_np(_gpu_rows(nv, ctx, gdn, fx, tail, state, 0, rows))
+    torch.cuda.synchronize()
+    ref = O.GdnLayerState(*cfg)
+    want = np.stack([O.gdn_step(ref, fx["qkv"][t], fx["a"][t], fx["b"][t], fx["z"][t], fx["conv_w"], fx["a_log"],
+                                fx["dt_bias"], fx["norm_w"], ctx.act) for t in range(rows)])
+    assert _close(got, want, ctx.act, "long call vs oracle, %d rows" % rows)
+    assert np.array_equal(act_np(tail[0]), ref.tail)
+    d_state = np.abs(state[0].cpu().numpy() - ref.state).max()
+    print("[measure] gdn long call state: max|d| %.3e of max|ref| %.3e" % (d_state, np.abs(ref.state).max()), flush=True)
+    assert d_state <= 1e-4 * float(np.abs(ref.state).max())      # the split operands keep sixteen bits: measured 7e-6
+
+
 def test_gdn_long_call_captured_in_a_graph_equals_the_eager_call(nv):
-    # 100 rows of a 128 x 128 head take the chunked form, which carves 2,304 bytes per (sequence, head, chunk) out of
+    # 100 rows of a 128 x 128 head take the chunked form, which carves 10,496 bytes per (sequence, head, chunk) out of
     # the context's workspace: a fresh context reserves them, captures the call, and every replay gives the bits of
     # the eager call (outputs, tail, state) -- a capture may not fall back to the row-by-row kernels
     say("gdn chunked call under a graph")
@@ -193,7 +215,7 @@ def test_gdn_long_call_captured_in_a_graph_equals_the_eager_call(nv):
     want = _gpu_rows(nv, eager_ctx, gdn_e, fx, tail_e, state_e, 0, rows).clone()
     torch.cuda.synchronize()
     ctx = nv.Context(0, 0)
-    ctx.reserve(1 << 20)                                # 4 heads x 7 chunks x 2,304 bytes, and room to spare
+    ctx.reserve(1 << 20)                                # 4 value heads x 7 chunks x 10,496 bytes + 2 key heads x 7 x 4,096, and room to spare
     gdn = nv.GDN(ctx, *cfg)
     tail, state = gdn.new_state()
     ins = [act_tensor(fx[k][:rows], ctx) for k in ("qkv", "a", "b", "z")]
