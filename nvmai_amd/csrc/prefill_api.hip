@@ -133,10 +133,11 @@ extern "C" int nvmai_hip_prefill_group_routes(nvmai_hip_ctx* ctx, nvmai_stream s
 
 namespace {
 
-// Blocks of a dense launch over `tiles` M tiles: whole units, dealt over eight XCDs.
+// Blocks of a dense launch over `tiles` M tiles: eight XCDs times the most any of them owns (M tiles dealt over
+// the XCDs from eight tiles on, column tiles otherwise; prefill_gemm_kernel).
 uint32_t gemm_grid(uint32_t tiles, const GemmParams& g) {
-    const uint32_t units = tiles * g.units_per_tile;
-    return (units + 7) / 8 * 8 * GEMM_UNIT;
+    const uint32_t per_xcd = tiles >= 8 ? (tiles + 7) / 8 * g.n_tiles_n : (g.n_tiles_n + 7) / 8 * tiles;
+    return GEMM_XCDS * per_xcd;
 }
 
 // Blocks of a grouped launch.  The work lists are dealt in serpentine order from a sorted sequence of
@@ -148,17 +149,28 @@ uint32_t grouped_grid(uint32_t max_mtiles, const GemmParams& g) {
     return GEMM_XCDS * grouped_list_max(max_mtiles) * g.n_tiles_n;
 }
 
-// dense: grid over `tiles` M tiles cut by the kernel; grouped: a block per column tile of every list position.
+// Rows per M tile of a dense product.  A launch of at most 128 blocks of 128 rows leaves half of the compute
+// units idle; tiles of 64 rows (the same kernel's four-row-tile body) double the blocks: the shared expert's
+// gate/up product over 4096 rows 46 -> 38 us.  At 256 blocks -- one per unit where two fit -- the shorter
+// tiles were measured too and do not pay (2048 x 4096 over 4096 rows: 98 -> 107 us; 2048 x 512: 22 us both ways).
+uint32_t dense_bm_for(uint32_t rows, uint32_t n_tiles_n) {
+    const uint64_t blocks = (uint64_t)((rows + GEMM_BM - 1) / GEMM_BM) * n_tiles_n;
+    return rows > 64 && blocks <= 128 ? 64u : (uint32_t)GEMM_BM;
+}
+uint32_t dense_tiles(const GemmParams& g) { return (g.dense_rows + g.dense_bm - 1) / g.dense_bm; }
+
+// dense: grid over the M tiles the kernel cuts itself; grouped: a block per column tile of every list position
+// of at most `tiles` M tiles.
 template <int ACT, int BITS, int NT>
 void launch_gemms(const GemmParams& g1, const GemmParams& g2, uint32_t tiles, nvmai_hip_ctx* ctx, hipStream_t s) {
     const bool dense = g1.dense_rows != 0;
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM1, s);
-        prefill_gemm_kernel<ACT, BITS, true, NT><<<dense ? gemm_grid(tiles, g1) : grouped_grid(tiles, g1), 256, 0, s>>>(g1);
+        prefill_gemm_kernel<ACT, BITS, true, NT><<<dense ? gemm_grid(dense_tiles(g1), g1) : grouped_grid(tiles, g1), 256, 0, s>>>(g1);
     }
     {
         ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM2, s);
-        prefill_gemm_kernel<ACT, BITS, false, NT><<<dense ? gemm_grid(tiles, g2) : grouped_grid(tiles, g2), 256, 0, s>>>(g2);
+        prefill_gemm_kernel<ACT, BITS, false, NT><<<dense ? gemm_grid(dense_tiles(g2), g2) : grouped_grid(tiles, g2), 256, 0, s>>>(g2);
     }
 }
 
@@ -181,13 +193,13 @@ int expert_ffn_dense(nvmai_hip_ctx* ctx, hipStream_t s, const uint8_t* blob, con
     g1.dense_rows = tokens;
     g1.x = x; g1.x_stride = x_stride; g1.out = act; g1.out_stride = f;
     g1.K = d; g1.N = f; g1.top_k = 1; g1.n_tiles_n = (f + 32 * nt - 1) / (32 * nt);
-    g1.units_per_tile = (g1.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
+    g1.dense_bm = dense_bm_for(tokens, g1.n_tiles_n);
     GemmParams g2 = g1;
     g2.wA = off->down_w; g2.sA = off->down_s; g2.bA = off->down_b;
     g2.wB = g2.sB = g2.bB = 0;
     g2.x = act; g2.x_stride = f; g2.out = tmp; g2.out_stride = d;
     g2.K = f; g2.N = d; g2.n_tiles_n = (d + 64 * nt - 1) / (64 * nt);
-    g2.units_per_tile = (g2.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
+    g2.dense_bm = dense_bm_for(tokens, g2.n_tiles_n);
     if (ctx->act == ACT_BF16) {
         if (bits == 4) launch_gemms<ACT_BF16, 4, 4>(g1, g2, tiles, ctx, s);
         else launch_gemms<ACT_BF16, 8, 2>(g1, g2, tiles, ctx, s);
@@ -261,14 +273,12 @@ extern "C" int nvmai_hip_prefill_grouped_moe(nvmai_hip_ctx* ctx, nvmai_stream st
     g1.x = hidden; g1.x_stride = hidden_stride;
     g1.out = act_scratch; g1.out_stride = f;
     g1.K = d; g1.N = f; g1.top_k = top_k; g1.n_tiles_n = (f + 32 * nt - 1) / (32 * nt);
-    g1.units_per_tile = (g1.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
     GemmParams g2 = g1;
     g2.wA = off->down_w; g2.sA = off->down_s; g2.bA = off->down_b;
     g2.wB = g2.sB = g2.bB = 0;
     g2.x = act_scratch; g2.x_stride = f;
     g2.out = route_partials; g2.out_stride = d;
     g2.K = f; g2.N = d; g2.n_tiles_n = (d + 64 * nt - 1) / (64 * nt);
-    g2.units_per_tile = (g2.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
     if (ctx->act == ACT_BF16) {
         if (bits == 4) launch_gemms<ACT_BF16, 4, 4>(g1, g2, max_mtiles, ctx, s);
         else launch_gemms<ACT_BF16, 8, 2>(g1, g2, max_mtiles, ctx, s);
@@ -348,14 +358,12 @@ extern "C" int nvmai_hip_prefill_grouped_moe_streamed(nvmai_hip_ctx* ctx, nvmai_
     g1.x = hidden; g1.x_stride = params->hidden_stride_elements;
     g1.out = act_scratch; g1.out_stride = f;
     g1.K = d; g1.N = f; g1.top_k = top_k; g1.n_tiles_n = (f + 32 * nt - 1) / (32 * nt);
-    g1.units_per_tile = (g1.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
     GemmParams g2 = g1;
     g2.wA = offs[6]; g2.sA = offs[7]; g2.bA = offs[8];
     g2.wB = g2.sB = g2.bB = 0;
     g2.x = act_scratch; g2.x_stride = f;
     g2.out = route_partials; g2.out_stride = d;
     g2.K = f; g2.N = d; g2.n_tiles_n = (d + 64 * nt - 1) / (64 * nt);
-    g2.units_per_tile = (g2.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
     if (ctx->act == ACT_BF16) {
         if (bits == 4) launch_gemms<ACT_BF16, 4, 4>(g1, g2, max_mtiles, ctx, s);
         else launch_gemms<ACT_BF16, 8, 2>(g1, g2, max_mtiles, ctx, s);
@@ -388,7 +396,6 @@ extern "C" int nvmai_hip_affine_qmm(nvmai_hip_ctx* ctx, nvmai_stream stream, con
     // the GEMM kernel addresses every operand array with 32-bit byte offsets
     if ((uint64_t)m * x_stride * 2 > 0xFFFFFFFFull || (uint64_t)n * k * bits / 8 > 0xFFFFFFFFull)
         return NVMAI_ERR_UNSUPPORTED;
-    const uint32_t tiles = (m + GEMM_BM - 1) / GEMM_BM;
     hipStream_t s = (hipStream_t)stream;
     ProfScope prof(ctx, NVMAI_PROF_PREFILL_GEMM2, s);
     const uint32_t nt = bits == 4 ? 4 : 2;
@@ -400,8 +407,8 @@ extern "C" int nvmai_hip_affine_qmm(nvmai_hip_ctx* ctx, nvmai_stream stream, con
     g.dense_rows = m;                           // the kernel cuts the rows into M tiles itself
     g.x = x; g.x_stride = x_stride; g.out = y; g.out_stride = y_stride;
     g.K = k; g.N = n; g.top_k = 1; g.n_tiles_n = (n + 64 * nt - 1) / (64 * nt);
-    g.units_per_tile = (g.n_tiles_n + GEMM_UNIT - 1) / GEMM_UNIT;
-    const uint32_t blocks = gemm_grid(tiles, g);
+    g.dense_bm = dense_bm_for(m, g.n_tiles_n);
+    const uint32_t blocks = gemm_grid(dense_tiles(g), g);
     if (ctx->act == ACT_BF16) { if (bits == 4) launch_qmm<ACT_BF16, 4, 4>(g, blocks, s); else launch_qmm<ACT_BF16, 8, 2>(g, blocks, s); }
     else { if (bits == 4) launch_qmm<ACT_FP16, 4, 4>(g, blocks, s); else launch_qmm<ACT_FP16, 8, 2>(g, blocks, s); }
     return launch_status();

@@ -321,6 +321,27 @@ def test_dense_qmm_every_row_tile_count(nv, ctx_bf16, bits, m, n, k):
     assert O.rel_error(act_np(y), want) <= TOL_ACT
 
 
+@pytest.mark.parametrize("bits,m", [(4, 1056), (4, 1280 + 64), (8, 1024 + 40), (4, 1024 + 96)])
+def test_projection_with_a_sliver_of_rows_at_the_end(nv, ctx, bits, m):
+    """A projection over many input rows whose matrix ends in a few rows past the last full block of the
+    matrix-core product (the concatenated input projections of a gated-DeltaNet layer end in 2 x 32 rows):
+    every column against the oracle, and the last partial block's columns on their own."""
+    say("projection with sliver", ctx.act, bits, m)
+    n, tokens = 512, 300
+    rng = np.random.default_rng(m + bits)
+    w = gauss(rng, (m, n), 0.05)
+    p, s, b = O.quantize_affine(w, bits)
+    xs = gauss(rng, (tokens, n))
+    x = O.round_bf16(xs) if ctx.act == 0 else O.f16_to_float(O.f16_bits(xs))
+    y = nv.affine_gemv(ctx, dev(p), dev(s.view(np.int16)), dev(b.view(np.int16)), bits, act_tensor(x, ctx), m, n)
+    torch.cuda.synchronize()
+    got = act_np(y)
+    want = np.stack([O.affine_gemv(p, s, b, x[t], bits) for t in range(0, tokens, 7)])
+    assert O.rel_error(got[::7], want) <= TOL_ACT
+    tail = m % (256 if bits == 4 else 128)
+    assert O.rel_error(got[::7, m - tail:], want[:, m - tail:]) <= TOL_ACT        # the sliver on its own
+
+
 def test_gemm_refuses_operands_beyond_32_bit_offsets(nv, ctx_bf16):
     say("gemm 4 GiB limits")
     q = nv.MPPPrefillInt4QMM(ctx_bf16, 4)
