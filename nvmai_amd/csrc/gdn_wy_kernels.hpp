@@ -145,7 +145,9 @@ __device__ __forceinline__ void gdn_wy_barrier() {
 
 // Waves of a block go to the four SIMDs of a compute unit in turn, and the chain should have its SIMD to itself:
 // wave 0 runs the chain, wave 1 makes the rows, waves 2, 3 and 5 are the producers, wave 4 (the chain's SIMD) only
-// keeps the barriers' count.
+// keeps the barriers' count.  (Measured and not kept: the chain shared by two waves, half of the state columns each,
+// their shares of Kt S^T exchanged through LDS at a second barrier in the middle of the iteration -- 182 against
+// 153 us for 256 chunks: the barrier costs more than half of the split, the products and the update saves.)
 constexpr int GDN_WY_WAVES = 6;
 
 template <bool STATE_BF16>
