@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--sweep", action="store_true", help="also print batch/bits sweep lines to stderr")
     ap.add_argument("--no-extra", action="store_true", help="skip the `extra` object (the other cells of the metric) "
                     "that the default invocation appends")
-    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "prefill_attention", "sampler", "greedy", "step", "prefill_step", "copy"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "prefill", "attention", "prefill_attention", "sampler", "greedy", "step", "prefill_step", "copy", "read"],
                     help="decode = configs[1] (the headline line); prefill = configs[2] grouped GEMM; "
                          "attention = configs[3] quantized-KV decode attention; prefill_attention = causal attention of --tokens queries "
                          "at the end of a --context cache; sampler = the end of configs[4]: "
@@ -777,6 +777,32 @@ def run_copy(torch, a):
             "config": {"workload": "copy: 1 GiB read + 1 GiB written per launch", "bytes_read": n, "bytes_written": n}}
 
 
+def run_read(nv, ctx, torch, a, window_mib=512):
+    """What a kernel that only reads reaches on this device: windows of 512 MiB out of 8 GiB in turn (twice the
+    memory-side cache apart, so every launch comes from HBM), one launch per step, HIP events around the timed steps."""
+    window = window_mib << 20
+    pool = torch.empty(8 << 30, dtype=torch.uint8, device="cuda")
+    pool.view(torch.int32).random_(0, 1 << 31)
+    n_win = pool.numel() // window
+    views = [pool[i * window:(i + 1) * window] for i in range(n_win)]
+    for i in range(max(a.warmup, 4)):
+        ctx.read_probe(views[i % n_win])
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    steps = max(a.steps, 16)
+    e0.record()
+    for i in range(steps):
+        ctx.read_probe(views[i % n_win])
+    e1.record()
+    torch.cuda.synchronize()
+    dt = e0.elapsed_time(e1) * 1e-3 / steps
+    gbps = window / dt / 1e9
+    return {"metric": "plain device read", "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps,
+            "warmup": max(a.warmup, 4), "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "read: %d MiB per launch, nothing else (nvmai_hip_read_probe)" % window_mib,
+                       "bytes_read": window, "frac_of_hbm_peak": round(gbps / 8000.0, 4)}}
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -796,7 +822,8 @@ def main():
                 run_sampler(nv, ctx, torch, a) if a.workload == "sampler" else
                 run_greedy(nv, ctx, torch, a) if a.workload == "greedy" else
                 run_step(nv, ctx, torch, a) if a.workload == "step" else
-                run_prefill_step(nv, ctx, torch, a) if a.workload == "prefill_step" else run_copy(torch, a))
+                run_prefill_step(nv, ctx, torch, a) if a.workload == "prefill_step" else
+                run_read(nv, ctx, torch, a) if a.workload == "read" else run_copy(torch, a))
         print(json.dumps(line), flush=True)
         return
     layers, stride = build_layers(nv, ctx, torch, a.bits, a.layers)
@@ -921,11 +948,17 @@ def run_config0(nv, ctx, torch, layers4, stride4, a):
 def extra_cells(nv, ctx, torch, a, layers8, stride8):
     """The other cells of the metric, each measured like its own --workload line but shorter and printed in
     compact form (the key names the cell; v = value, u = unit, ms = per step, kern_us / kern / frac = the
-    roofline kernel's launch time, rate and fraction of its peak).  The twelve cells of configs[3] come first as
+    roofline kernel's launch time, rate and fraction of its peak).  First what a kernel that only reads reaches on
+    this device in this run, the measuring stick for the HBM fractions; then the twelve cells of configs[3] as
     one table, the metric's own cells last: configs[0], the configs[2] prefill grouped GEMM, 4-bit decode at batch
     32, 8-bit decode at one token, configs[4] at batch 1 and 16."""
     import argparse
     out = {}
+    sub = argparse.Namespace(**vars(a))
+    sub.steps, sub.warmup = 32, 8
+    c = run_read(nv, ctx, torch, sub)
+    out["plain_read_512MiB"] = {"v": c["value"], "u": "GB/s", "frac": c["config"]["frac_of_hbm_peak"]}
+    torch.cuda.empty_cache()
     rows = []
     for bits in (8, 4):
         for context, batch in ((131072, 8), (131072, 1), (32768, 8), (32768, 1), (4096, 8), (4096, 1)):

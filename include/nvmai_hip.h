@@ -94,6 +94,12 @@ enum {
 int nvmai_hip_profile_enable(nvmai_hip_ctx* ctx, int on);
 int nvmai_hip_profile_read(nvmai_hip_ctx* ctx, int tag, double* total_ms, uint32_t* launches);
 
+/* No counterpart in the reference: a measuring stick for the roofline fractions.  Reads `bytes` (a multiple of 16,
+ * 16-byte aligned) of device memory and does nothing else -- what a kernel that only streams reaches on this
+ * device, to set beside the rate of the library's own streaming kernels in the same run.  `sink` (may be NULL) is
+ * never written in practice; it only keeps the loads alive. */
+int nvmai_hip_read_probe(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* data, uint64_t bytes, uint32_t* sink);
+
 /* CPUExpertFFN.Offsets(d:f:) (CPUExpertFFN.swift:42-59) for `bits` in {4,8}.
  * Host-only arithmetic; *stride_bytes receives the blob size. */
 int nvmai_expert_offsets_for(uint32_t d, uint32_t f, uint32_t bits,

@@ -86,6 +86,7 @@ SIGNATURES = {
     "nvmai_hip_ctx_reserve": [vp, C.c_size_t],
     "nvmai_hip_profile_enable": [vp, C.c_int],
     "nvmai_hip_profile_read": [vp, C.c_int, C.POINTER(C.c_double), C.POINTER(u32)],
+    "nvmai_hip_read_probe": [vp, vp, vp, u64, vp],
     "nvmai_expert_offsets_for": [u32, u32, u32, C.POINTER(ExpertOffsets), C.POINTER(u64)],
     "nvmai_hip_quantize_affine": [vp, vp, vp, C.c_int, u32, u32, u32, vp, vp, vp],
     "nvmai_hip_dequantize_affine": [vp, vp, vp, vp, vp, u64, u32, vp, vp],

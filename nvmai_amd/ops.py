@@ -52,6 +52,12 @@ class Context:
         check(lib.nvmai_hip_profile_read(self.handle, tag, C.byref(ms), C.byref(n)), "profile_read")
         return ms.value, n.value
 
+    def read_probe(self, data):
+        """Launch the kernel that only reads `data` (a contiguous device tensor of a multiple of 16 bytes): the
+        measuring stick for the HBM fractions of the streaming kernels."""
+        check(lib.nvmai_hip_read_probe(self.handle, _stream(), _ptr(data), data.numel() * data.element_size(), None),
+              "read_probe")
+
     def close(self):
         if self.handle:
             lib.nvmai_hip_ctx_destroy(self.handle)

@@ -175,6 +175,23 @@ def test_reference_signature_host_gemv(nv, ctx_bf16):
     assert np.isnan(bad).all()
 
 
+def test_read_probe_runs_and_checks_its_arguments(nv, ctx_bf16):
+    # the measuring stick of bench.py: reads a buffer and writes nothing; sizes with a ragged end, the empty
+    # buffer, and the refusals (misaligned start, a size that is no multiple of 16)
+    say("read probe")
+    buf = torch.full(((1 << 20) + 48,), 7, dtype=torch.uint8, device="cuda")
+    for n in (0, 16, 1008, 8192, 65536 + 16, 1 << 20, (1 << 20) + 48):
+        ctx_bf16.read_probe(buf[:n])
+    torch.cuda.synchronize()
+    assert bool((buf == 7).all())
+    with pytest.raises(nv.NvmaiError) as e:
+        ctx_bf16.read_probe(buf[8:8 + 64])
+    assert e.value.name == "alignment"
+    with pytest.raises(nv.NvmaiError) as e:
+        ctx_bf16.read_probe(buf[:40])
+    assert e.value.name == "alignment"
+
+
 def test_gemv_rejects_bad_arguments(nv, ctx_bf16):
     say("gemv-errors")
     w = torch.zeros(64 * 128, dtype=torch.uint8, device="cuda")
