@@ -25,13 +25,16 @@ class HybridConfig:
     def __init__(self, hidden=2048, layers=40, full_every=4, num_heads=16, num_kv_heads=2, head_dim=256,
                  rotary_dim=64, rope_theta=1e7, gdn=(16, 32, 128, 128, 4), num_experts=256, top_k=8,
                  moe_intermediate=512, vocab=248320, expert_bits=4, attn_bits=4, kv_bits=8, head_bits=16,
-                 embed_bits=4, rms_eps=1e-6, logit_softcap=0.0, gdn_state_bf16=True, full_mask=None):
+                 embed_bits=4, rms_eps=1e-6, logit_softcap=0.0, gdn_state_bf16=True, full_mask=None, shared_bits=None):
         self.hidden, self.layers, self.full_every = hidden, layers, full_every
         self.full_mask = None if full_mask is None else [bool(v) for v in full_mask]   # per layer: full attention?
         self.num_heads, self.num_kv_heads, self.head_dim = num_heads, num_kv_heads, head_dim
         self.rotary_dim, self.rope_theta, self.gdn = rotary_dim, rope_theta, gdn
         self.num_experts, self.top_k, self.moe_intermediate, self.vocab = num_experts, top_k, moe_intermediate, vocab
         self.expert_bits, self.attn_bits, self.kv_bits = expert_bits, attn_bits, kv_bits
+        # quant.sharedExpert beside quant.routedExpert (Model.swift:59-60): the repacker's 4-bit profile keeps the
+        # shared expert at 8 bits (RemoteStreamingRepacker.swift:678-683)
+        self.shared_bits = expert_bits if shared_bits is None else shared_bits
         self.head_bits, self.embed_bits = head_bits, embed_bits
         self.rms_eps, self.logit_softcap, self.gdn_state_bf16 = rms_eps, logit_softcap, gdn_state_bf16
 
@@ -67,7 +70,8 @@ class HybridConfig:
         mat = lambda rows, cols, bits: rows * cols * bits / 8 + (0 if bits == 16 else 2 * rows * (cols // 64) * 2)
         expert = 2 * mat(F, D, self.expert_bits) + mat(D, F, self.expert_bits)
         distinct = E * (1.0 - (1.0 - k / E) ** batch)
-        moe = (distinct + 1) * expert + E * D * 2 + mat(1, D, 8)
+        shared = 2 * mat(F, D, self.shared_bits) + mat(D, F, self.shared_bits)
+        moe = distinct * expert + shared + E * D * 2 + mat(1, D, 8)
         kh, vh, dk, dv, taps = self.gdn
         lin = mat(self.gdn_qkv_dim + self.gdn_value_dim + 2 * vh, D, self.attn_bits) + mat(D, self.gdn_value_dim, self.attn_bits) \
             + self.gdn_qkv_dim * taps * 2
@@ -121,22 +125,36 @@ class HybridWeights:
                 w["qkv"] = q(2 * cfg.q_dim + 2 * cfg.kv_dim, D, cfg.attn_bits)
                 w["q_norm"], w["k_norm"] = normw(cfg.head_dim), normw(cfg.head_dim)
                 w["o_proj"] = q(D, cfg.q_dim, cfg.attn_bits)
-            pool = torch.empty((cfg.num_experts + 1, stride), dtype=torch.uint8, device=dev)
             F = cfg.moe_intermediate
-            for (rows, n, wo, so, bo) in ((F, D, off.gate_w, off.gate_s, off.gate_b), (F, D, off.up_w, off.up_s, off.up_b),
-                                          (D, F, off.down_w, off.down_s, off.down_b)):
-                p_, s_, b_ = q((cfg.num_experts + 1) * rows, n, cfg.expert_bits)
-                wb, mb = rows * n * cfg.expert_bits // 8, rows * n // 32
-                pool[:, wo:wo + wb] = p_.view(cfg.num_experts + 1, wb)
-                pool[:, so:so + mb] = s_.view(torch.uint8).view(cfg.num_experts + 1, mb)
-                pool[:, bo:bo + mb] = b_.view(torch.uint8).view(cfg.num_experts + 1, mb)
-                del p_, s_, b_
+            mixed = cfg.shared_bits != cfg.expert_bits      # the shared expert then has a blob of its own width
+
+            def fill(pool, n_blobs, o, bits):
+                for (rows, n, wo, so, bo) in ((F, D, o.gate_w, o.gate_s, o.gate_b), (F, D, o.up_w, o.up_s, o.up_b),
+                                              (D, F, o.down_w, o.down_s, o.down_b)):
+                    p_, s_, b_ = q(n_blobs * rows, n, bits)
+                    wb, mb = rows * n * bits // 8, rows * n // 32
+                    pool[:, wo:wo + wb] = p_.view(n_blobs, wb)
+                    pool[:, so:so + mb] = s_.view(torch.uint8).view(n_blobs, mb)
+                    pool[:, bo:bo + mb] = b_.view(torch.uint8).view(n_blobs, mb)
+                    del p_, s_, b_
+
+            n_pool = cfg.num_experts + (0 if mixed else 1)
+            pool = torch.empty((n_pool, stride), dtype=torch.uint8, device=dev)
+            fill(pool, n_pool, off, cfg.expert_bits)
             w["pool"] = pool
             w["router"] = _randn(gen, (cfg.num_experts, D), std, dev).view(torch.int16)
             w["gate"] = q(1, D, 8)
-            w["moe"] = ops.moe_layer_desc(D, F, cfg.num_experts, cfg.top_k, cfg.expert_bits,
-                                          ops.rows_desc(16, w["router"]), pool[:cfg.num_experts], pool[cfg.num_experts],
-                                          ops.rows_desc(8, *w["gate"]))
+            if mixed:
+                s_off, s_stride = ops.expert_offsets(D, F, cfg.shared_bits)
+                blob = torch.empty((1, s_stride), dtype=torch.uint8, device=dev)
+                fill(blob, 1, s_off, cfg.shared_bits)
+                w["shared"] = dict(blob=blob[0], offsets=s_off, bits=cfg.shared_bits, gate=ops.rows_desc(8, *w["gate"]))
+                w["moe"] = ops.moe_layer_desc(D, F, cfg.num_experts, cfg.top_k, cfg.expert_bits,
+                                              ops.rows_desc(16, w["router"]), pool)
+            else:
+                w["moe"] = ops.moe_layer_desc(D, F, cfg.num_experts, cfg.top_k, cfg.expert_bits,
+                                              ops.rows_desc(16, w["router"]), pool[:cfg.num_experts], pool[cfg.num_experts],
+                                              ops.rows_desc(8, *w["gate"]))
             self.layers.append(w)
 
 
@@ -144,7 +162,8 @@ def _from_gturbo(cls, ctx, model, gdn=None, kv_bits=8, gdn_state_bf16=True):
     """HybridWeights (and its HybridConfig) from an opened model directory (gturbo.GTurboModel): the resident
     tensors bound by the reference's names (Model.swift:137-306), the matrices of a projection group stacked
     as the rows of one matrix (one launch per group), each layer's experts in HBM with the shared expert as
-    the pool's last row.  The manifest carries no gated-DeltaNet head shape (the reference compiles it in,
+    the pool's last row -- or, when quant.sharedExpert differs from quant.routedExpert, in a blob of its own
+    that the step runs beside the routed block.  The manifest carries no gated-DeltaNet head shape (the reference compiles it in,
     ModelTypes.swift:162-204): value heads, value head size and conv taps are read off the tensor shapes,
     key heads assume key head size = value head size unless gdn = (Hk, Hv, Dk, Dv, taps) says otherwise.
     Returns (config, weights)."""
@@ -154,9 +173,7 @@ def _from_gturbo(cls, ctx, model, gdn=None, kv_bits=8, gdn_state_bf16=True):
     a, q = model.manifest.arch, model.manifest.quant
     if q is None:
         raise G.ModelError("indexCorrupt", "manifest.quant is required by the executable runtime schema")
-    if not model.shared_matches_routed():
-        raise G.ModelError("unsupportedArch", "the decode step runs the shared expert in the routed experts' launches: a shared "
-                           "expert of another width is run per layer through gturbo.GTurboMoEBlock")
+    mixed = not model.shared_matches_routed()           # the shared expert then runs beside the routed block, at its width
     mask = a["fullAttentionLayerMask"]
     if any(v == 0 for v in mask):
         raise G.ModelError("unsupportedArch", "sliding-window layers")
@@ -210,7 +227,7 @@ def _from_gturbo(cls, ctx, model, gdn=None, kv_bits=8, gdn_state_bf16=True):
                        top_k=a["topKExperts"], moe_intermediate=a["moeIntermediateSize"], vocab=a["vocabSize"],
                        expert_bits=expert_bits, attn_bits=attn_bits, kv_bits=kv_bits, head_bits=head_bits,
                        embed_bits=embed_bits, logit_softcap=a["finalLogitSoftcap"], gdn_state_bf16=gdn_state_bf16,
-                       full_mask=[v == 1 for v in mask])
+                       full_mask=[v == 1 for v in mask], shared_bits=q["sharedExpert"].weightBits)
     self.cfg = cfg
     self.layers = []
     for L in range(layers):
@@ -232,8 +249,13 @@ def _from_gturbo(cls, ctx, model, gdn=None, kv_bits=8, gdn_state_bf16=True):
                                    % (L, rows, cfg.num_heads, cfg.head_dim))
             w["o_proj"], _, _ = t3(p + "self_attn.o_proj.weight", attn_bits)
             w["q_norm"], w["k_norm"] = bf(p + "self_attn.q_norm.weight"), bf(p + "self_attn.k_norm.weight")
-        w["pool"] = model.expert_pool(L, dev, with_shared=True)
+        w["pool"] = model.expert_pool(L, dev, with_shared=not mixed)
         w["moe"], held = model.moe_layer(L, w["pool"], dev)
+        if mixed:
+            s_off, _, _ = model.shared_expert_offsets(L)
+            blob = torch.from_numpy(model.shared_expert_blob(L)).to(dev)
+            gate = model._rows(p + "mlp.shared_expert_gate.weight", q["router"].weightBits, dev, held)
+            w["shared"] = dict(blob=blob, offsets=ops.ExpertOffsets(*[int(v) for v in s_off]), bits=cfg.shared_bits, gate=gate)
         keep.append(held)
         self.layers.append(w)
     self._keep = keep
@@ -255,6 +277,7 @@ class HybridDecoder:
         self.hidden, self.normed, self.branch = buf(batch, D), buf(batch, D), buf(batch, D)
         self.hidden_alt = buf(batch, D)            # the residual rows alternate between two buffers
         self.moe_out = buf(batch, D)
+        self.shared_out = buf(batch, D)           # a shared expert of another width than the routed ones
         kh, vh, dk, dv, taps = cfg.gdn
         self.gdn = ops.GDN(ctx, kh, vh, dk, dv, taps)
         self.lin_rows = cfg.gdn_qkv_dim + cfg.gdn_value_dim + 2 * vh
@@ -388,6 +411,20 @@ class HybridDecoder:
             # residual add + post-attention norm + MoE: the router launch does the add and the norm itself,
             # so the updated residual rows go to the second buffer (other blocks still read the first)
             nxt = self.w.layers[L + 1]["in_norm"] if L + 1 < cfg.layers else self.w.final_norm
+            if w.get("shared") is not None:
+                # a shared expert of another width (quant.sharedExpert != quant.routedExpert): the routed block on
+                # its own, the shared-expert operator at its width over the same normed rows
+                # (RealForwardRunner.swift:3866-3912), its output added to the routed sum
+                self.moe.decode_layer_prenorm(w["moe"], self.hidden, self.branch, w["post_norm"], self.hidden_alt, self.normed,
+                                              self.moe_out, eps=cfg.rms_eps)
+                self.hidden, self.hidden_alt = self.hidden_alt, self.hidden
+                sh = w["shared"]
+                ops.SharedExpertRuntime(ctx, sh["bits"]).encode(sh["blob"], sh["offsets"], self.normed, cfg.hidden,
+                                                                cfg.moe_intermediate, shared_gate=sh["gate"], y=self.shared_out)
+                self.ew.encode_residual_add(self.moe_out, self.shared_out)
+                if not fold or L + 1 == cfg.layers:
+                    ops.residual_add_rmsnorm(ctx, self.hidden, self.moe_out, nxt, out=self.normed, eps=cfg.rms_eps)
+                continue
             if not fold:
                 # five sequences or more: the residual add that closes the layer and the next norm ride in the
                 # block's combine launch (the post-attention rows in self.normed are dead by then)
@@ -496,16 +533,24 @@ class HybridDecoder:
         GEMM, rank-order reduce -- with the shared expert beside it."""
         cfg, ctx = self.cfg, self.ctx
         D, F, E, K = cfg.hidden, cfg.moe_intermediate, cfg.num_experts, cfg.top_k
+        sh = w.get("shared")                 # a shared expert of another width: beside the routed block
         if T < 64 and T * K <= 4096:
-            return self.moe.decode_layer(w["moe"], x)
+            y = self.moe.decode_layer(w["moe"], x)
+            if sh is not None:
+                self.ew.encode_residual_add(y, ops.SharedExpertRuntime(ctx, sh["bits"]).encode(
+                    sh["blob"], sh["offsets"], x, D, F, shared_gate=sh["gate"]))
+            return y
         layer = w["moe"]
         idx, wts = self.moe.encode_router(layer.router, x, E, D, K)
         routes = ops.PrefillMoEGrouping(ctx).group_routes(idx, wts, E)
         pool = w["pool"]
         partials, _ = ops.PrefillGroupedRoutedMoE(ctx, cfg.expert_bits).encode(pool[:E], layer.offsets, x, D, F, routes)
         h2 = ops.PrefillMoE(ctx).encode_reduce_token_major(partials, wts, T, K, D)
-        shared = ops.SharedExpertRuntime(ctx, cfg.expert_bits).encode(pool[E], layer.offsets, x, D, F,
-                                                                      shared_gate=layer.shared_gate)
+        if sh is not None:
+            shared = ops.SharedExpertRuntime(ctx, sh["bits"]).encode(sh["blob"], sh["offsets"], x, D, F, shared_gate=sh["gate"])
+        else:
+            shared = ops.SharedExpertRuntime(ctx, cfg.expert_bits).encode(pool[E], layer.offsets, x, D, F,
+                                                                          shared_gate=layer.shared_gate)
         return self.ew.encode_residual_add(h2, shared)
 
     def head(self):

@@ -872,9 +872,14 @@ def write_hybrid_model(directory, cfg, weights, model_id="nvmai-amd-synthetic"):
         blobs = np.zeros((E, stride), np.uint8)
         blobs[:, :used] = pool[:E, :used]
         lays.append({"blobs": blobs, "tensors": tensors, "ranks": None})
-        shared = pool[E]
+        if w.get("shared") is not None:          # a shared expert of another width than the routed ones: its own blob
+            shared, sb = host(w["shared"]["blob"]), w["shared"]["bits"]
+            s_off, _ = _cpu_expert_offsets(D, F, sb)
+            s_sizes = [F * D * sb // 8, F * (D // 64) * 2, F * (D // 64) * 2] * 2 + [D * F * sb // 8, D * (F // 64) * 2, D * (F // 64) * 2]
+        else:
+            shared, s_off, s_sizes = pool[E], off, sizes
         for i, (proj, rows, cols) in enumerate((("gate_proj", F, D), ("up_proj", F, D), ("down_proj", D, F))):
-            cut = lambda j: shared[off[3 * i + j]:off[3 * i + j] + sizes[3 * i + j]].tobytes()
+            cut = lambda j: shared[s_off[3 * i + j]:s_off[3 * i + j] + s_sizes[3 * i + j]].tobytes()
             resident.append((p + "mlp.shared_expert.%s.weight" % proj, 0, (rows, cols), cut(0), cut(1), cut(2)))
         if cfg.is_linear(L):
             rows_of = (cfg.gdn_qkv_dim, cfg.gdn_value_dim, vh, vh)
@@ -898,7 +903,7 @@ def write_hybrid_model(directory, cfg, weights, model_id="nvmai-amd-synthetic"):
             bf16(p + "self_attn.k_norm.weight", w["k_norm"], (cfg.head_dim,))
     slot = lambda b: {"weightBits": b, "scheme": "affine", "scaleType": "bf16", "biasType": "bf16", "groupSize": 64}
     quant = {"embedding": slot(cfg.embed_bits), "attention": slot(cfg.attn_bits), "router": slot(8),
-             "sharedExpert": slot(cfg.expert_bits), "routedExpert": slot(cfg.expert_bits)}
+             "sharedExpert": slot(cfg.shared_bits), "routedExpert": slot(cfg.expert_bits)}
     arch = {"hiddenSize": D, "ffnIntermediate": F, "moeIntermediateSize": F, "numHeads": cfg.num_heads,
             "numKVHeads": cfg.num_kv_heads, "numFullKVHeads": cfg.num_kv_heads, "headDim": cfg.head_dim,
             "fullHeadDim": cfg.head_dim, "vocabSize": cfg.vocab, "slidingWindow": 0,

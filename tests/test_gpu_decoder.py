@@ -39,6 +39,8 @@ class OracleModel:
         for L, lw in enumerate(w.layers):
             d = dict(in_norm=_np16(lw["in_norm"]), post_norm=_np16(lw["post_norm"]), pool=lw["pool"].cpu().numpy(),
                      router=_np16(lw["router"]), gate=q3(lw["gate"]))
+            if lw.get("shared") is not None:
+                d["shared_blob"] = lw["shared"]["blob"].cpu().numpy()
             if cfg.is_linear(L):
                 d.update(in_proj=q3(lw["in_proj"]), out_proj=q3(lw["out_proj"]), conv_w=_np16(lw["conv_w"]),
                          a_log=_np16(lw["a_log"]), dt_bias=_np16(lw["dt_bias"]), gdn_norm=_np16(lw["gdn_norm"]))
@@ -88,9 +90,20 @@ class OracleModel:
                 hidden = r(hidden + branch)
                 routed_x = r(O.rmsnorm(hidden[None], lw["post_norm"], cfg.rms_eps)[0])
                 E = cfg.num_experts
-                _, _, y = O.moe_layer_forward(routed_x[None], D, cfg.moe_intermediate, cfg.top_k, cfg.expert_bits,
-                                              (16, lw["router"].reshape(E, D), None, None), lw["pool"][:E], lw["pool"][E],
-                                              (8,) + lw["gate"])
+                router = (16, lw["router"].reshape(E, D), None, None)
+                if "shared_blob" in lw:
+                    # the routed experts alone at their width; the gated shared expert at its own: a layer whose
+                    # experts all ARE the shared blob, with and without the shared slot -- the difference is the slot
+                    F, sb = cfg.moe_intermediate, cfg.shared_bits
+                    _, _, y_routed = O.moe_layer_forward(routed_x[None], D, F, cfg.top_k, cfg.expert_bits, router, lw["pool"][:E])
+                    copies = np.stack([lw["shared_blob"]] * E)
+                    _, _, y_both = O.moe_layer_forward(routed_x[None], D, F, cfg.top_k, sb, router, copies, lw["shared_blob"],
+                                                       (8,) + lw["gate"])
+                    _, _, y_none = O.moe_layer_forward(routed_x[None], D, F, cfg.top_k, sb, router, copies)
+                    y = r(r(y_routed) + r(y_both - y_none))
+                else:
+                    _, _, y = O.moe_layer_forward(routed_x[None], D, cfg.moe_intermediate, cfg.top_k, cfg.expert_bits,
+                                                  router, lw["pool"][:E], lw["pool"][E], (8,) + lw["gate"])
                 hidden = r(hidden + r(y[0]))
                 nxt = self.layers[L + 1]["in_norm"] if L + 1 < cfg.layers else self.final_norm
                 normed = r(O.rmsnorm(hidden[None], nxt, cfg.rms_eps)[0])
@@ -179,8 +192,42 @@ def test_step_replays_from_a_captured_graph():
     ctx.close()
 
 
-@pytest.mark.parametrize("prompt,chunk", [(80, 512), (80, 48), (200, 512)], ids=["one-chunk", "two-chunks", "dense-shared"])
-def test_prefill_chunks_leave_the_state_that_decode_steps_leave(prompt, chunk):
+@pytest.mark.parametrize("batch", [2, 5], ids=["folded-norms", "five-sequences"])
+def test_toy_hybrid_model_with_a_shared_expert_of_another_width(batch):
+    # quant.sharedExpert = 8 beside quant.routedExpert = 4, the reference repacker's 4-bit profile
+    # (RemoteStreamingRepacker.swift:678-683): the step runs the routed block on its own and the shared-expert operator
+    # at its width beside it (RealForwardRunner.swift:3866-3912).  Two sequences take the path that folds a layer's
+    # closing add and the next norm into the next projection launch, five the one with explicit launches.  Every expert
+    # is selected (top_k = experts), so that no near-tie of the router can send the oracle and the GPU, whose rows
+    # differ in the last bits by then, to different experts.
+    import nvmai_amd as nv
+    from nvmai_amd.decoder import HybridConfig, HybridDecoder, HybridWeights
+    say("toy hybrid decode steps, shared expert at 8 bits", batch)
+    ctx = nv.Context(0, nv.ACT_BF16)
+    cfg = HybridConfig(hidden=256, layers=4, full_every=4, num_heads=4, num_kv_heads=2, head_dim=64, rotary_dim=16,
+                       rope_theta=1e4, gdn=(2, 4, 32, 32, 4), num_experts=4, top_k=4, moe_intermediate=128, vocab=1024,
+                       expert_bits=4, attn_bits=4, kv_bits=8, head_bits=16, gdn_state_bf16=False, shared_bits=8)
+    w = HybridWeights(ctx, cfg, seed=17, std=0.06)
+    assert all(lw["shared"]["bits"] == 8 and lw["pool"].shape[0] == cfg.num_experts for lw in w.layers)
+    dec = HybridDecoder(ctx, cfg, w, batch=batch, max_context=16)
+    ref = OracleModel(cfg, w, batch)
+    tokens = np.array([5, 900, 33, 512, 77][:batch], np.int32)
+    for position in range(3):
+        dec.tokens.copy_(torch.from_numpy(tokens).cuda())
+        seeds = [nv.sampler_seed_for(42 + b, position) for b in range(batch)]
+        nxt = dec.step(position, seeds)
+        torch.cuda.synchronize()
+        want_normed, want_logits = ref.step(tokens, position)
+        err_n, err_l = O.rel_error(act_np(dec.normed), want_normed), O.rel_error(act_np(dec.logits), want_logits)
+        print("position", position, "normed rel", err_n, "logits rel", err_l, flush=True)
+        assert err_n < 1e-2 and err_l < 1e-2
+        tokens = nxt.cpu().numpy().astype(np.int32)
+    ctx.close()
+
+
+@pytest.mark.parametrize("prompt,chunk,shared_bits", [(80, 512, None), (80, 48, None), (200, 512, None), (200, 512, 8), (80, 48, 8)],
+                         ids=["one-chunk", "two-chunks", "dense-shared", "dense-shared-8bit", "two-chunks-shared-8bit"])
+def test_prefill_chunks_leave_the_state_that_decode_steps_leave(prompt, chunk, shared_bits):
     # RealForwardRunner.prefillChunked against its own serial decode loop: the prompt through the prefill
     # kernels (dense matrix-core projections, recurrent kernels over the rows of a chunk, causal attention
     # over the quantized cache, tiled router + permutation + grouped GEMM + reduce, shared expert) and
@@ -190,11 +237,11 @@ def test_prefill_chunks_leave_the_state_that_decode_steps_leave(prompt, chunk):
     # that no near-tie of the router can send the two paths to different experts.
     import nvmai_amd as nv
     from nvmai_amd.decoder import HybridConfig, HybridDecoder, HybridWeights
-    say("prefill chunks vs decode steps", prompt, chunk)
+    say("prefill chunks vs decode steps", prompt, chunk, shared_bits)
     ctx = nv.Context(0, nv.ACT_BF16)
     cfg = HybridConfig(hidden=256, layers=4, full_every=2, num_heads=4, num_kv_heads=2, head_dim=64, rotary_dim=16,
                        rope_theta=1e4, gdn=(2, 4, 32, 32, 4), num_experts=4, top_k=4, moe_intermediate=128, vocab=1024,
-                       expert_bits=4, attn_bits=4, kv_bits=8, head_bits=16, gdn_state_bf16=False)
+                       expert_bits=4, attn_bits=4, kv_bits=8, head_bits=16, gdn_state_bf16=False, shared_bits=shared_bits)
     w = HybridWeights(ctx, cfg, seed=11, std=0.06)
     serial, chunked = HybridDecoder(ctx, cfg, w, 1, 256), HybridDecoder(ctx, cfg, w, 1, 256)
     gen = torch.Generator(device="cuda").manual_seed(prompt)

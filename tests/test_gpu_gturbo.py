@@ -138,19 +138,21 @@ def test_shared_expert_at_8_bits_beside_4_bit_routed_experts(tmp_path):
     ctx.close()
 
 
-@pytest.mark.parametrize("head_bits", [16, 4], ids=["bf16-head", "4bit-head"])
-def test_whole_hybrid_model_from_a_directory_equals_the_model_from_arrays(tmp_path, head_bits):
+@pytest.mark.parametrize("head_bits,shared_bits", [(16, None), (4, None), (16, 8)], ids=["bf16-head", "4bit-head", "shared-expert-8bit"])
+def test_whole_hybrid_model_from_a_directory_equals_the_model_from_arrays(tmp_path, head_bits, shared_bits):
     # every resident tensor bound by the reference's names (Model.swift:137-306): a toy hybrid model (gated-DeltaNet
     # and full-attention layers, MoE in each) written as a model directory, read back, and stepped beside the model
-    # it was written from -- hidden rows, logits and sampled tokens must be the same bits, token after token
+    # it was written from -- hidden rows, logits and sampled tokens must be the same bits, token after token.  The third
+    # case keeps the shared expert at 8 bits beside 4-bit routed experts (the reference repacker's 4-bit profile).
     import nvmai_amd as nv
     from nvmai_amd import gturbo as G
     from nvmai_amd.decoder import HybridConfig, HybridDecoder, HybridWeights
-    say("gturbo directory -> HybridWeights -> decode steps", head_bits)
+    say("gturbo directory -> HybridWeights -> decode steps", head_bits, shared_bits)
     ctx = nv.Context(0, nv.ACT_BF16)
     cfg = HybridConfig(hidden=256, layers=4, full_every=2, num_heads=4, num_kv_heads=2, head_dim=64, rotary_dim=16,
                        rope_theta=1e4, gdn=(2, 4, 32, 32, 4), num_experts=16, top_k=4, moe_intermediate=128, vocab=1024,
-                       expert_bits=4, attn_bits=4, kv_bits=8, head_bits=head_bits, embed_bits=4, gdn_state_bf16=True)
+                       expert_bits=4, attn_bits=4, kv_bits=8, head_bits=head_bits, embed_bits=4, gdn_state_bf16=True,
+                       shared_bits=shared_bits)
     w = HybridWeights(ctx, cfg, seed=21, std=0.06)
     torch.cuda.synchronize()
     G.write_hybrid_model(str(tmp_path), cfg, w)
@@ -160,6 +162,7 @@ def test_whole_hybrid_model_from_a_directory_equals_the_model_from_arrays(tmp_pa
             assert name in model.entries, name
     cfg2, w2 = HybridWeights.from_gturbo(ctx, model, kv_bits=8, gdn_state_bf16=True)
     assert cfg2.gdn == cfg.gdn and cfg2.head_bits == head_bits and cfg2.rotary_dim == cfg.rotary_dim
+    assert cfg2.shared_bits == cfg.shared_bits and model.shared_matches_routed() == (shared_bits is None)
     assert [cfg2.is_linear(L) for L in range(4)] == [cfg.is_linear(L) for L in range(4)]
     a, b = HybridDecoder(ctx, cfg, w, 2, 16), HybridDecoder(ctx, cfg2, w2, 2, 16)
     tokens = torch.tensor([5, 900], dtype=torch.int32, device="cuda")
