@@ -69,7 +69,6 @@ int launch_delta_chunked(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state
     const int ws_rc = ws_begin(ctx, (nvmai_stream)s, ws_round(count * sizeof(GdnChunkPrep)) + wy_bytes);
     if (ws_rc != NVMAI_OK) return ws_rc;
     GdnChunkPrep* prep = ws_take<GdnChunkPrep>(ctx, count);
-    gdn_chunk_prep_kernel<ACT, 128><<<dim3(nchunks, p.sh.v_heads, p.sh.batch), 64, 0, s>>>(p, prep, nchunks);
     const dim3 cgrid(p.sh.v_heads, p.sh.batch, 128 / 16);
     if (wy_form) {
         GdnChunkWY* wy = ws_take<GdnChunkWY>(ctx, count);
@@ -77,10 +76,10 @@ int launch_delta_chunked(nvmai_hip_ctx* ctx, const GdnDeltaParams& p, bool state
         gdn_wy_prep_kernel<<<dim3(nchunks, p.sh.v_heads, p.sh.batch), 64, 0, s>>>(p, prep, wy, kts, nchunks);
         if (state_bf16) gdn_wy_delta_kernel<true><<<cgrid, 64 * GDN_WY_WAVES, 0, s>>>(p, prep, wy, kts, nchunks);
         else gdn_wy_delta_kernel<false><<<cgrid, 64 * GDN_WY_WAVES, 0, s>>>(p, prep, wy, kts, nchunks);
-    } else if (state_bf16) {
-        gdn_chunk_delta_kernel<ACT, 128, 128, true><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
     } else {
-        gdn_chunk_delta_kernel<ACT, 128, 128, false><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
+        gdn_chunk_prep_kernel<ACT, 128><<<dim3(nchunks, p.sh.v_heads, p.sh.batch), 64, 0, s>>>(p, prep, nchunks);
+        if (state_bf16) gdn_chunk_delta_kernel<ACT, 128, 128, true><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
+        else gdn_chunk_delta_kernel<ACT, 128, 128, false><<<cgrid, 64 * GDN_CHUNK_WAVES, 0, s>>>(p, prep, nchunks);
     }
     launch_gated_norm_rows<ACT>(p, s);
     return 1;

@@ -48,12 +48,27 @@ __device__ __forceinline__ gc_f4 gc_mfma4(float a, float b, gc_f4 c) {
 }
 
 // ---- per (chunk, head, sequence): T, W and the gate vectors ----------------------------------------
-// One wave.  Lane (i16 = lane % 16, g = lane / 16).
-template <int ACT, int DK>
-__global__ __launch_bounds__(64) void gdn_chunk_prep_kernel(GdnDeltaParams p, GdnChunkPrep* prep, uint32_t nchunks) {
+// One wave.  Lane (i16 = lane % 16, g = lane / 16).  The work is a function of its own so that the kernel which
+// goes on to the split operands of gdn_wy_kernels.hpp can run it first: with KEEP it leaves the chunk's k rows
+// (dead rows zero), T and beta G in the LDS arrays of `keep` for that kernel; the caller synchronizes.
+struct GdnPrepLds {
+    float xs[16], bs[16];
+    float Ls[16][16];
+};
+template <int DK>
+struct GdnPrepKeep {
+    uint16_t ks[16][DK + 8];
+    float Ts[16][17];
+    float bG[16];
+};
+
+template <int ACT, int DK, bool KEEP>
+__device__ __forceinline__ void gdn_chunk_prep_body(const GdnDeltaParams& p, GdnChunkPrep* prep, uint32_t nchunks, GdnPrepLds& l,
+                                                    GdnPrepKeep<DK>* keep) {
     static_assert(DK % 16 == 0, "shape");
-    __shared__ float xs[16], bs[16];
-    __shared__ float Ls[16][16];
+    float (&xs)[16] = l.xs;
+    float (&bs)[16] = l.bs;
+    float (&Ls)[16][16] = l.Ls;
     const uint32_t lane = threadIdx.x, i16 = lane & 15u, g = lane >> 4;
     const uint32_t c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const GdnShape& sh = p.sh;
@@ -76,6 +91,7 @@ __global__ __launch_bounds__(64) void gdn_chunk_prep_kernel(GdnDeltaParams p, Gd
         uint2 kf = *reinterpret_cast<const uint2*>(base + (sh.k_heads + hk) * DK + 16 * st + 4 * g);
         uint2 qf = *reinterpret_cast<const uint2*>(base + hk * DK + 16 * st + 4 * g);
         if (!row_live) { kf = uint2{0u, 0u}; qf = uint2{0u, 0u}; }
+        if (KEEP) *reinterpret_cast<uint2*>(&keep->ks[i16][16 * st + 4 * g]) = kf;
         kk = gc_mfma16<ACT>(kf, kf, kk);       // kk[r] = k_{4g+r} . k_{i16}
         qk = gc_mfma16<ACT>(qf, kf, qk);       // qk[r] = q_{4g+r} . k_{i16}
     }
@@ -108,6 +124,7 @@ __global__ __launch_bounds__(64) void gdn_chunk_prep_kernel(GdnDeltaParams p, Gd
         out->bG[lane] = bs[lane] * G;
         out->beta[lane] = bs[lane];
         out->c[lane] = expf(-(X15 - Xm));
+        if (KEEP) keep->bG[lane] = bs[lane] * G;
     }
     __syncthreads();
     // column j of T by forward substitution: T[i][j] = [i == j] - sum_{m < i} L[i][m] T[m][j]
@@ -120,8 +137,15 @@ __global__ __launch_bounds__(64) void gdn_chunk_prep_kernel(GdnDeltaParams p, Gd
             for (int m = 0; m < i; ++m) acc = fmaf(-Ls[i][m], t[m], acc);
             t[i] = acc;
             out->T[i][lane] = acc;
+            if (KEEP) keep->Ts[i][lane] = acc;
         }
     }
+}
+
+template <int ACT, int DK>
+__global__ __launch_bounds__(64) void gdn_chunk_prep_kernel(GdnDeltaParams p, GdnChunkPrep* prep, uint32_t nchunks) {
+    __shared__ GdnPrepLds l;
+    gdn_chunk_prep_body<ACT, DK, false>(p, prep, nchunks, l, nullptr);
 }
 
 // ---- the chunks in sequence: one block of four waves per (head, sequence, sixteen state rows) ---------

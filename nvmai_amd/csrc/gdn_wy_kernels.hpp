@@ -70,37 +70,30 @@ __device__ __forceinline__ uint32_t gc_lo2(float a, float b) {
     return gc_rne2(a - __uint_as_float(__float_as_uint(a) & 0xFFFF0000u), b - __uint_as_float(__float_as_uint(b) & 0xFFFF0000u));
 }
 
-// ---- per (chunk, value head, sequence): Kt in two halves, and k^T once per key head ------------------
-// One wave, after gdn_chunk_prep_kernel (it reads that kernel's T and beta G).
-__global__ __launch_bounds__(64) void gdn_wy_prep_kernel(GdnDeltaParams p, const GdnChunkPrep* prep, GdnChunkWY* wy,
-                                                        GdnChunkKT* kts, uint32_t nchunks) {
+// ---- per (chunk, value head, sequence): T, W and the gate vectors, then Kt in two halves, and k^T once per key head
+// One wave: the preparation of gdn_chunk_kernels.hpp and, from what it leaves in LDS, the split operands.
+__global__ __launch_bounds__(64) void gdn_wy_prep_kernel(GdnDeltaParams p, GdnChunkPrep* prep, GdnChunkWY* wy, GdnChunkKT* kts,
+                                                        uint32_t nchunks) {
     constexpr int DK = 128;
-    __shared__ __attribute__((aligned(16))) uint16_t ks[16][DK + 8];
+    __shared__ GdnPrepLds l;
+    __shared__ __attribute__((aligned(16))) GdnPrepKeep<DK> keep;
     __shared__ __attribute__((aligned(16))) float kt[16][DK + 4];
+    gdn_chunk_prep_body<ACT_BF16, DK, true>(p, prep, nchunks, l, &keep);
+    __syncthreads();
     const uint32_t lane = threadIdx.x, i16 = lane & 15u, g = lane >> 4;
     const uint32_t c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const GdnShape& sh = p.sh;
-    const uint32_t ratio = sh.v_heads / sh.k_heads, hk = h / ratio, t0 = c * 16;
-    const GdnChunkPrep* pc = prep + ((size_t)b * sh.v_heads + h) * nchunks + c;
-    const float4 Tf = *reinterpret_cast<const float4*>(&pc->T[i16][4 * g]);
-    const float4 bG = *reinterpret_cast<const float4*>(&pc->bG[4 * g]);
-    const float Tp[4] = {Tf.x * bG.x, Tf.y * bG.y, Tf.z * bG.z, Tf.w * bG.w};
-    const bool row_live = t0 + i16 < sh.rows;
-    const uint16_t* base = p.conv_out + ((size_t)b * sh.rows + min(t0 + i16, sh.rows - 1)) * p.conv_stride + (sh.k_heads + hk) * DK;
+    const uint32_t ratio = sh.v_heads / sh.k_heads, hk = h / ratio;
+    float Tp[4];
 #pragma unroll
-    for (int st = 0; st < DK / 16; ++st) {
-        uint2 kf = *reinterpret_cast<const uint2*>(base + 16 * st + 4 * g);
-        if (!row_live) kf = uint2{0u, 0u};
-        *reinterpret_cast<uint2*>(&ks[i16][16 * st + 4 * g]) = kf;
-    }
-    __syncthreads();
+    for (int s = 0; s < 4; ++s) Tp[s] = keep.Ts[i16][4 * g + s] * keep.bG[4 * g + s];
     GdnChunkKT* ko = kts + ((size_t)b * sh.k_heads + hk) * nchunks + c;
     const bool write_kt = h % ratio == 0;
 #pragma unroll
     for (int bb = 0; bb < DK / 16; ++bb) {
         uint16_t raw[4];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) raw[s] = ks[4 * g + s][16 * bb + i16];
+        for (int s = 0; s < 4; ++s) raw[s] = keep.ks[4 * g + s][16 * bb + i16];
         gc_f4 C = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int s = 0; s < 4; ++s) C = gc_mfma4(Tp[s], bf16_to_f32(raw[s]), C);       // C[r] = Kt[4 g + r][16 bb + i16]
