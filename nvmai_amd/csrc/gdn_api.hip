@@ -136,7 +136,18 @@ extern "C" int nvmai_hip_gdn_conv_norm(nvmai_hip_ctx* ctx, nvmai_stream stream, 
     if (rows >= GDN_ROWS_PARALLEL_FROM && sh.dk <= 128 && sh.dv <= 128 && (rows + 1) / 2 <= 65535) {
         // a chunk of rows: thirty-two rows of a head segment per block, then the tail in a launch of its own
         const dim3 rgrid(2 * sh.k_heads + sh.v_heads, batch, (rows + GDN_CONV_ROWS_PER_BLOCK - 1) / GDN_CONV_ROWS_PER_BLOCK);
-        if (ctx->act == ACT_BF16)
+        const bool pieces = sh.taps == 4 && sh.dk % 8 == 0 && sh.dv % 8 == 0 && qkv_stride % 8 == 0 && conv_out_stride % 8 == 0 &&
+                            aligned16(qkv_raw) && aligned16(tail) && aligned16(conv_weight) && aligned16(conv_out);
+        if (pieces) {
+            // rows in 16-byte pieces: eight rows of a head segment per sixteen lanes
+            const dim3 pgrid(2 * sh.k_heads + sh.v_heads, batch, (rows + GDN_CONV8_ROWS_PER_BLOCK - 1) / GDN_CONV8_ROWS_PER_BLOCK);
+            if (ctx->act == ACT_BF16)
+                gdn_conv_norm_rows8_kernel<ACT_BF16><<<pgrid, 256, 0, s>>>((const uint16_t*)qkv_raw, qkv_stride, (const uint16_t*)tail,
+                                                                          conv_weight, (uint16_t*)conv_out, conv_out_stride, sh);
+            else
+                gdn_conv_norm_rows8_kernel<ACT_FP16><<<pgrid, 256, 0, s>>>((const uint16_t*)qkv_raw, qkv_stride, (const uint16_t*)tail,
+                                                                          conv_weight, (uint16_t*)conv_out, conv_out_stride, sh);
+        } else if (ctx->act == ACT_BF16)
             gdn_conv_norm_rows_kernel<ACT_BF16><<<rgrid, 256, 0, s>>>((const uint16_t*)qkv_raw, qkv_stride, (const uint16_t*)tail,
                                                                      conv_weight, (uint16_t*)conv_out, conv_out_stride, sh);
         else

@@ -346,6 +346,96 @@ __global__ __launch_bounds__(256) void gdn_conv_norm_rows_kernel(const uint16_t*
     }
 }
 
+// The same rows in 16-byte pieces, for four taps, segment lengths that are multiples of eight and rows that start at
+// 16-byte boundaries: sixteen lanes take eight consecutive rows of one segment, lane j the channels 8 j .. 8 j + 7 --
+// one load and one store per row and lane instead of eight, and a sixteenth of the wave-wide sums' instructions per
+// channel.  Same bits: the conv sum runs over the taps in the same order, and the sum of squares is the same
+// balanced tree over the channel index (neighbours first: three levels inside the lane, three across lanes 0..7 for
+// channels 0..63 and across lanes 8..15 for channels 64..127, the two halves added last).
+constexpr uint32_t GDN_CONV8_ROWS_PER_UNIT = 8, GDN_CONV8_ROWS_PER_BLOCK = 16 * GDN_CONV8_ROWS_PER_UNIT;
+
+template <int ACT>
+__global__ __launch_bounds__(256) void gdn_conv_norm_rows8_kernel(const uint16_t* qkv_raw, uint32_t qkv_stride,
+                                                                 const uint16_t* tail, const uint16_t* conv_w,
+                                                                 uint16_t* conv_out, uint32_t out_stride, GdnShape sh) {
+    constexpr uint32_t RPU = GDN_CONV8_ROWS_PER_UNIT, TAPS = 4, HIST = TAPS - 1;
+    const uint32_t seg = blockIdx.x, b = blockIdx.y;
+    const uint32_t unit = threadIdx.x >> 4, j16 = threadIdx.x & 15u;
+    const uint32_t t_first = (blockIdx.z * 16 + unit) * RPU;
+    if (t_first >= sh.rows) return;                                         // uniform per sixteen lanes; no barrier below
+    const uint32_t C = 2 * sh.k_heads * sh.dk + sh.v_heads * sh.dv;
+    const bool is_qk = seg < 2 * sh.k_heads;
+    const uint32_t seg_len = is_qk ? sh.dk : sh.dv;
+    const uint32_t base = is_qk ? seg * sh.dk : 2 * sh.k_heads * sh.dk + (seg - 2 * sh.k_heads) * sh.dv;
+    const bool live = 8u * j16 < seg_len;
+    const uint32_t ch0 = base + (live ? 8u * j16 : 0u);
+    const uint16_t* tl = tail + (size_t)b * HIST * C;
+    const uint16_t* raw = qkv_raw + (size_t)b * sh.rows * qkv_stride;
+    auto eight = [](const uint4& v, float* f) {
+        act2_to_f32<ACT>(v.x, f[0], f[1]); act2_to_f32<ACT>(v.y, f[2], f[3]);
+        act2_to_f32<ACT>(v.z, f[4], f[5]); act2_to_f32<ACT>(v.w, f[6], f[7]);
+    };
+    // every load of the run is requested before the first is used
+    uint4 wraw[4], praw[HIST], curv[RPU];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) wraw[q] = *reinterpret_cast<const uint4*>(conv_w + (size_t)ch0 * TAPS + 8 * q);
+#pragma unroll
+    for (uint32_t j = 0; j < HIST; ++j) {
+        const int src = (int)t_first - (int)HIST + (int)j;                  // row src of [old tail | rows]
+        praw[j] = *reinterpret_cast<const uint4*>(src >= 0 ? raw + (size_t)src * qkv_stride + ch0
+                                                            : tl + (size_t)((int)HIST + src) * C + ch0);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < RPU; ++k)                                      // rows past the end read the last row again
+        curv[k] = *reinterpret_cast<const uint4*>(raw + (size_t)min(t_first + k, sh.rows - 1u) * qkv_stride + ch0);
+    float wt[8][TAPS], pre[8][HIST];
+    {
+        const uint16_t* wh = reinterpret_cast<const uint16_t*>(wraw);      // [channel][tap]
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (uint32_t j = 0; j < TAPS; ++j) wt[c][j] = bf16_to_f32(wh[c * TAPS + j]);
+#pragma unroll
+        for (uint32_t j = 0; j < HIST; ++j) {
+            float f[8];
+            eight(praw[j], f);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) pre[c][j] = f[c];
+        }
+    }
+    const float scale = seg < sh.k_heads ? 1.0f / (float)sh.dk : rsqrtf((float)sh.dk);
+#pragma unroll
+    for (uint32_t k = 0; k < RPU; ++k) {
+        const uint32_t t = t_first + k;
+        if (t >= sh.rows) break;                                            // uniform per sixteen lanes
+        float cur[8], x[8];
+        uint16_t r[8];
+        eight(curv[k], cur);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            float acc = 0.0f;
+#pragma unroll
+            for (uint32_t j = 0; j < TAPS; ++j) acc = fmaf(j < HIST ? pre[c][j] : cur[c], wt[c][j], acc);
+#pragma unroll
+            for (uint32_t j = 0; j < HIST; ++j) pre[c][j] = j + 1 < HIST ? pre[c][j + 1] : cur[c];
+            r[c] = live ? f32_to_act<ACT>(gdn_silu(acc)) : (uint16_t)0;
+            x[c] = live ? act_to_f32<ACT>(r[c]) : 0.0f;
+        }
+        uint16_t* o = conv_out + ((size_t)b * sh.rows + t) * out_stride + ch0;
+        if (is_qk) {                                                        // block-uniform
+            float sq = ((x[0] * x[0] + x[1] * x[1]) + (x[2] * x[2] + x[3] * x[3])) +
+                       ((x[4] * x[4] + x[5] * x[5]) + (x[6] * x[6] + x[7] * x[7]));
+            const float total = seg_reduce_sum<16>(sq) + (0.0f + 0.0f);     // lanes 0..7, lanes 8..15, then the two halves
+            const float inv = rsqrtf(total / (float)sh.dk + GDN_RMS_EPS);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) r[c] = f32_to_act<ACT>(x[c] * inv * scale);
+        }
+        if (live)
+            *reinterpret_cast<uint4*>(o) = uint4{(uint32_t)r[0] | ((uint32_t)r[1] << 16), (uint32_t)r[2] | ((uint32_t)r[3] << 16),
+                                                 (uint32_t)r[4] | ((uint32_t)r[5] << 16), (uint32_t)r[6] | ((uint32_t)r[7] << 16)};
+    }
+}
+
 // The new tail of every sequence: the last K - 1 raw rows of [old tail | rows].  One thread per channel
 // reads its column before it writes it, so the update is in place.
 __global__ __launch_bounds__(256) void gdn_tail_update_kernel(const uint16_t* qkv_raw, uint32_t qkv_stride, uint16_t* tail,

@@ -241,6 +241,34 @@ def test_gdn_long_call_captured_in_a_graph_equals_the_eager_call(nv):
     eager_ctx.close()
 
 
+@pytest.mark.parametrize("rows", [8, 37, 133])
+def test_gdn_conv_rows_in_16_byte_pieces_same_bits(nv, ctx, rows):
+    # a chunk of rows with four taps and rows at 16-byte boundaries takes the conv + norm eight channels per
+    # lane; input rows at a stride that is not a multiple of 16 bytes take the two-channels-per-lane kernel:
+    # the same rows through both must give the same bits, the tail too (run boundaries at 8 and 128 rows)
+    say("gdn conv rows pieces", ctx.act, rows)
+    cfg, batch = (2, 4, 128, 128, 4), 2
+    fxs = [_fixture(cfg, rows, 940 + b, ctx.act) for b in range(batch)]
+    w = fxs[0]
+    gdn = nv.GDN(ctx, *cfg)
+    qkv = act_tensor(np.concatenate([fx["qkv"] for fx in fxs]), ctx)
+    outs, tails = [], []
+    for pad in (0, 4):
+        tail, _ = gdn.new_state(batch)
+        tail.copy_(torch.randn(tail.shape, generator=torch.Generator().manual_seed(7)).to(tail.dtype))
+        x = qkv
+        if pad:
+            wide = torch.zeros((qkv.shape[0], qkv.shape[1] + pad), dtype=qkv.dtype, device=qkv.device)
+            wide[:, :qkv.shape[1]] = qkv
+            x = wide[:, :qkv.shape[1]]
+            assert x.stride(0) % 8 != 0
+        outs.append(gdn.encode_conv_norm(x, tail, _bits(w["conv_w"]), rows=rows))
+        tails.append(tail)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(tails[0], tails[1])
+
+
 @pytest.mark.parametrize("rows", [8, 37, 80])
 def test_gdn_gated_norm_in_16_byte_pieces_same_bits(nv, ctx, rows):
     # heads of 128 values take the gated output norm in 16-byte pieces, sixteen lanes per (row, head);
