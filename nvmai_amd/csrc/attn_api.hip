@@ -2,6 +2,7 @@
 #include <cmath>
 
 #include "attn_kernels.hpp"
+#include "attn_prefill_kernels.hpp"
 #include "ctx.hpp"
 
 using namespace nvmai;
@@ -252,5 +253,35 @@ extern "C" int nvmai_hip_attention_prefill_causal(nvmai_hip_ctx* ctx, nvmai_stre
     p.ring = kv_ring_capacity;
     const uint32_t longest = start_position + query_count;          // keys of the last query without a window
     const uint32_t max_len = sliding_window != 0 && sliding_window < longest ? sliding_window : longest;
+    // A chunk with enough queries to give every compute unit a block of the flash-attention kernel: the key range
+    // is dequantized once into fp16 scratch and that kernel runs on it (attn_prefill_kernels.hpp) -- every key
+    // row is then read by hundreds of query blocks, and taking it apart once (2.6 ns per row) costs less than what
+    // the kernels that multiply the codes spend per (row, query block).  Fewer queries keep those kernels, which
+    // split the key range over blocks (512 queries at the end of a 32K cache: 0.64 ms against 0.98 ms on 128
+    // blocks of this form); so does a range whose scratch would pass 512 MB.
+    const uint32_t qpk = num_q_heads / num_kv_heads;
+    const uint32_t first_a = start_position + 1u;
+    const uint32_t key_lo = (sliding_window != 0u && first_a > sliding_window ? first_a - sliding_window : 0u) & ~31u;
+    const uint32_t key_hi = longest < kv_valid_count ? longest : kv_valid_count;
+    const uint64_t ntok = ((uint64_t)(key_hi - key_lo) + 31u) & ~(uint64_t)31u;
+    const uint64_t scratch = ntok * num_kv_heads * ATTN_HD * 2;
+    const bool fa_shape = head_dim == ATTN_HD && (qpk == 1 || qpk == 2 || qpk == 4 || qpk == 8 || qpk == 16);
+    const uint64_t fa_blocks = fa_shape ? ((uint64_t)query_count + 64u / qpk - 1) / (64u / qpk) * num_kv_heads : 0;
+    if (fa_shape && fa_blocks >= ATTN_FA_MIN_BLOCKS && scratch <= (1ull << 28) && aligned16(q) && q_token_stride % 8 == 0 && aligned16(out) &&
+        o_token_stride % 8 == 0) {
+        hipStream_t s = (hipStream_t)stream;
+        const int wrc = ws_begin(ctx, stream, 2 * ws_round(scratch));
+        if (wrc) return wrc;
+        uint16_t* kd = ws_take<uint16_t>(ctx, scratch / 2);
+        uint16_t* vt = ws_take<uint16_t>(ctx, scratch / 2);
+        ProfScope ps(ctx, NVMAI_PROF_ATTN_PARTIAL, s);
+        const AttnDequantParams dq{p.k, p.v, p.f, kv_ring_capacity, key_lo, key_hi, (uint32_t)ntok, num_kv_heads, kd, vt};
+        attn_prefill_dequant_kernel<<<dim3((uint32_t)(ntok / 32), num_kv_heads), 256, 0, s>>>(dq);
+        const uint32_t tpb = 4u * (16u / qpk);
+        const dim3 grid(((query_count + tpb - 1) / tpb) * num_kv_heads);
+        if (ctx->act == ACT_BF16) attn_prefill_fa_kernel<ACT_BF16><<<grid, 256, 0, s>>>(p, kd, vt, (uint32_t)ntok, key_lo);
+        else attn_prefill_fa_kernel<ACT_FP16><<<grid, 256, 0, s>>>(p, kd, vt, (uint32_t)ntok, key_lo);
+        return launch_status();
+    }
     return run_attention(ctx, stream, p, k, v, max_len, true);
 }

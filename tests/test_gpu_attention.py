@@ -274,6 +274,8 @@ def _prefill_case(nv, ctx, seed, bits, start, chunk, window, hd, nq, nkv, extra_
     k = round_act(rng.uniform(lo, hi, (kv_valid, elements)).astype(np.float32), ctx.act)
     v = round_act(rng.uniform(lo, hi, (kv_valid, elements)).astype(np.float32), ctx.act)
     q_stride, o_stride, q_off, o_off = (row + 3, row + 7, 17, 29) if pad else (row, row, 0, 0)
+    if pad == "aligned":                                            # strided and offset, every row at a 16-byte boundary
+        q_stride, o_stride, q_off, o_off = row + 8, row + 16, 24, 40
     q_buf = torch.zeros(q_off + chunk * q_stride, dtype=ctx.dtype, device="cuda")
     q_buf[q_off:].view(chunk, q_stride)[:, :row] = act_tensor(q, ctx)
     out_buf = torch.full((o_off + chunk * o_stride,), 7.0, dtype=ctx.dtype, device="cuda")
@@ -339,6 +341,30 @@ def test_prefill_attention_quantized_rows(nv, ctx, bits):
         say("prefill attention quantized", ctx.act, bits, start, chunk, window, hd, nq, nkv, extra, pad)
         _prefill_case(nv, ctx, start + chunk, bits, start, chunk, window, hd, nq, nkv, extra_kv=extra, pad=pad,
                       lo=-1.0, hi=1.0, scale=1.0 / np.sqrt(hd))
+
+
+def test_prefill_attention_long_chunks(nv):
+    # chunks whose queries give every compute unit a block (queries x q heads >= 16,384) take the two-launch form
+    # -- the key range dequantized once into fp16 scratch, then flash attention on that: every row against the
+    # oracle over the same cache rows -- quantized and fp16 rows, a chunk deep in the cache, a window, keys past
+    # the chunk, odd query counts (a last block with dead waves and dead columns), every group size, a ring,
+    # strided and offset rows at 16-byte boundaries, and rows that are not (those keep the one-launch kernels,
+    # which need no scratch: the context's workspace tells which form ran)
+    for act in (0, 1):
+        for bits, start, chunk, window, nq, nkv, extra, pad, ring in [
+                (8, 0, 258, 0, 64, 8, 0, False, 0), (4, 37, 261, 0, 64, 8, 5, False, 0), (8, 300, 257, 64, 64, 8, 0, False, 0),
+                (8, 0, 260, 0, 64, 64, 0, False, 0), (16, 5, 256, 0, 64, 16, 0, False, 0), (4, 64, 259, 0, 64, 32, 3, "aligned", 0),
+                (16, 200, 256, 64, 64, 8, 0, False, 320), (8, 0, 300, 0, 64, 4, 0, "aligned", 0), (8, 11, 270, 0, 64, 8, 0, True, 0)]:
+            if act == 1 and bits == 4:
+                continue                                            # the fp16 context repeats the 8- and 16-bit cases only
+            ctx = nv.Context(0, act)
+            say("prefill attention long chunk", act, bits, start, chunk, window, nq, nkv, extra, pad, ring)
+            _prefill_case(nv, ctx, 0xFA00 + start + chunk, bits, start, chunk, window, 256, nq, nkv, extra_kv=extra, pad=pad,
+                          ring=ring, lo=-1.0, hi=1.0, scale=1.0 / 16.0)
+            keys = min(start + chunk, window + chunk) if window else start + chunk
+            scratch = 2 * (keys // 32 * 32) * nkv * 256 * 2          # at least: K rows and V^T rows of the key range
+            assert (ctx.workspace_bytes >= scratch) == (pad is not True), ctx.workspace_bytes
+            ctx.close()
 
 
 @pytest.mark.parametrize("bits", [8, 4])
