@@ -107,10 +107,22 @@ __global__ __launch_bounds__(256) void attn_prefill_dequant_kernel(AttnDequantPa
 // [dim][4 pieces of eight tokens], piece c of dim d in slot c ^ sigma(d): both operand reads touch every bank once.
 constexpr uint32_t ATTN_FA_KTILE = 32 * ATTN_HD * 2;      // bytes
 constexpr uint32_t ATTN_FA_MIN_BLOCKS = 256;              // blocks below which the one-launch kernels are taken
-// Slot swizzle of a V^T row: bijective on (d / 2) % 4 among eight consecutive dims of one parity and on (d / 4) % 4
-// among the dims d, d + 4, d + 8, d + 12, so sixteen lanes reading piece r of sixteen consecutive dims touch every
-// 16-byte bank group of a 256-byte LDS line once, and eight of them every group of a 128-byte line.
-__device__ __forceinline__ uint32_t attn_fa_vsigma(uint32_t d) { return (((d >> 1) ^ (d >> 3)) & 1u) | (((d >> 2) & 1u) << 1); }
+// Slot swizzle of a V^T row (rows of 64 bytes, sixteen lanes reading piece r of sixteen consecutive dims): chosen by
+// measurement -- a wave's 16-byte reads at slot r ^ ((d / 2) % 4) run at the rate of a linear read (1.9 ns per
+// wave-read and compute unit with eight waves reading), unswizzled or swizzled by (d / 4) % 4 at half of it.
+__device__ __forceinline__ uint32_t attn_fa_vsigma(uint32_t d) { return (d >> 1) & 3u; }
+
+// Maximum over the four lane quarters (lanes l, l ^ 16, l ^ 32, l ^ 48) by the two row-swap instructions of this
+// target: a swap hands every lane its partner's value in one of its two results, so the maximum of the two is the
+// pairwise maximum in every lane -- vector instructions of a few cycles where a bpermute is a trip through LDS,
+// and this maximum heads the dependency chain of every tile.
+__device__ __forceinline__ float attn_fa_max_quarters(float v) {
+    typedef unsigned u2_t __attribute__((ext_vector_type(2)));
+    const u2_t a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a.x), __uint_as_float(a.y));
+    const u2_t b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(b.x), __uint_as_float(b.y));
+}
 
 template <int ACT>
 __global__ __launch_bounds__(256, 2) void attn_prefill_fa_kernel(AttnParams p, const uint16_t* kd, const uint16_t* vt, uint32_t ntok,
@@ -239,8 +251,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_fa_kernel(AttnParams p, c
         float mx = sv[0];
 #pragma unroll
         for (int s = 1; s < 8; ++s) mx = fmaxf(mx, sv[s]);
-        mx = fmaxf(mx, shfl_xor_f(mx, 16));
-        mx = fmaxf(mx, shfl_xor_f(mx, 32));
+        mx = attn_fa_max_quarters(mx);
         const float m_new = fmaxf(m_run, mx);                       // -inf while the column has seen no key yet
         const bool none = m_new == -INFINITY;
         const float alpha = none ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
