@@ -277,10 +277,19 @@ extern "C" int nvmai_hip_attention_prefill_causal(nvmai_hip_ctx* ctx, nvmai_stre
         ProfScope ps(ctx, NVMAI_PROF_ATTN_PARTIAL, s);
         const AttnDequantParams dq{p.k, p.v, p.f, kv_ring_capacity, key_lo, key_hi, (uint32_t)ntok, num_kv_heads, kd, vt};
         attn_prefill_dequant_kernel<<<dim3((uint32_t)(ntok / 32), num_kv_heads), 256, 0, s>>>(dq);
-        const uint32_t tpb = 4u * (16u / qpk);
+        // eight waves per block (twice the queries per K / V tile fetched from the L2) when that still leaves every
+        // compute unit a block, four otherwise
+        const uint32_t tpw = 16u / qpk;
+        const bool wide = ((uint64_t)query_count + 8u * tpw - 1) / (8u * tpw) * num_kv_heads >= ATTN_FA_MIN_BLOCKS;
+        const uint32_t tpb = (wide ? 8u : 4u) * tpw;
         const dim3 grid(((query_count + tpb - 1) / tpb) * num_kv_heads);
-        if (ctx->act == ACT_BF16) attn_prefill_fa_kernel<ACT_BF16><<<grid, 256, 0, s>>>(p, kd, vt, (uint32_t)ntok, key_lo);
-        else attn_prefill_fa_kernel<ACT_FP16><<<grid, 256, 0, s>>>(p, kd, vt, (uint32_t)ntok, key_lo);
+        if (wide) {
+            if (ctx->act == ACT_BF16) attn_prefill_fa_kernel<ACT_BF16, 8><<<grid, 512, 0, s>>>(p, kd, vt, (uint32_t)ntok, key_lo);
+            else attn_prefill_fa_kernel<ACT_FP16, 8><<<grid, 512, 0, s>>>(p, kd, vt, (uint32_t)ntok, key_lo);
+        } else {
+            if (ctx->act == ACT_BF16) attn_prefill_fa_kernel<ACT_BF16, 4><<<grid, 256, 0, s>>>(p, kd, vt, (uint32_t)ntok, key_lo);
+            else attn_prefill_fa_kernel<ACT_FP16, 4><<<grid, 256, 0, s>>>(p, kd, vt, (uint32_t)ntok, key_lo);
+        }
         return launch_status();
     }
     return run_attention(ctx, stream, p, k, v, max_len, true);

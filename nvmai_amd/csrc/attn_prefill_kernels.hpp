@@ -90,8 +90,8 @@ __global__ __launch_bounds__(256) void attn_prefill_dequant_kernel(AttnDequantPa
 }
 
 // ---- flash attention over the fp16 scratch -------------------------------------------------------------------
-// One block per (kv head, 4 * 16 / qpk consecutive query tokens): wave w owns sixteen score columns -- 16 / qpk
-// query tokens x the qpk heads of the group -- for the whole key range; the four waves share every 32-token
+// One block of NW waves (4 or 8) per (kv head, NW * 16 / qpk consecutive query tokens): wave w owns sixteen score columns -- 16 / qpk
+// query tokens x the qpk heads of the group -- for the whole key range; the waves share every 32-token
 // K / V tile, which reaches LDS without passing through registers (buffer_load ... lds), the next tile while
 // this one is multiplied: one barrier per tile.
 //   S[tokens, columns] = K . Q^T    A = K rows from LDS, B = q * (scale log2 e) as fp16, in registers
@@ -124,15 +124,16 @@ __device__ __forceinline__ float attn_fa_max_quarters(float v) {
     return fmaxf(__uint_as_float(b.x), __uint_as_float(b.y));
 }
 
-template <int ACT>
-__global__ __launch_bounds__(256, 2) void attn_prefill_fa_kernel(AttnParams p, const uint16_t* kd, const uint16_t* vt, uint32_t ntok,
+template <int ACT, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_fa_kernel(AttnParams p, const uint16_t* kd, const uint16_t* vt, uint32_t ntok,
                                                                  uint32_t lo0) {
     __shared__ __attribute__((aligned(16))) uint8_t k0s[ATTN_FA_KTILE];
     __shared__ __attribute__((aligned(16))) uint8_t k1s[ATTN_FA_KTILE];
     __shared__ __attribute__((aligned(16))) uint8_t v0s[ATTN_FA_KTILE];
     __shared__ __attribute__((aligned(16))) uint8_t v1s[ATTN_FA_KTILE];
-    __shared__ float bc_all[256];
-    __shared__ uint32_t rng[8];
+    constexpr int LPW = 16 / NW;                                   // load instructions per wave, tile and array
+    __shared__ float bc_all[64 * NW];
+    __shared__ uint32_t rng[2 * NW];
     // the tiles are written by load instructions only; a store that never runs keeps the optimizer from treating
     // them as never written (head_dim 0 is rejected by the entry point)
     if (p.head_dim == 0) { k0s[threadIdx.x] = 0; k1s[threadIdx.x] = 0; v0s[threadIdx.x] = 0; v1s[threadIdx.x] = 0; }
@@ -140,7 +141,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_fa_kernel(AttnParams p, c
     const int i = lane & 15, r = lane >> 4;
     float* bc = bc_all + wave * 64;
     const uint32_t qpk = p.num_q_heads / p.num_kv_heads;           // 1, 2, 4, 8 or 16
-    const uint32_t tpw = 16u / qpk, tpb = 4u * tpw;                // query tokens per wave, per block
+    const uint32_t tpw = 16u / qpk, tpb = (uint32_t)NW * tpw;                // query tokens per wave, per block
     const uint32_t n_qb = (p.batch + tpb - 1) / tpb;
     const uint32_t kvh = blockIdx.x % p.num_kv_heads;
     const uint32_t qb = n_qb - 1u - blockIdx.x / p.num_kv_heads;   // the longest key ranges start first
@@ -158,10 +159,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_fa_kernel(AttnParams p, c
     }
     wlo = __builtin_amdgcn_readfirstlane(wlo); whi = __builtin_amdgcn_readfirstlane(whi);
     ilo = __builtin_amdgcn_readfirstlane(ilo); ihi = __builtin_amdgcn_readfirstlane(ihi);
-    if (lane == 0) { rng[wave] = wlo; rng[4 + wave] = whi; }
+    if (lane == 0) { rng[wave] = wlo; rng[NW + wave] = whi; }
     __syncthreads();
-    const uint32_t blo = min(min(rng[0], rng[1]), min(rng[2], rng[3]));
-    const uint32_t bhi = max(max(rng[4], rng[5]), max(rng[6], rng[7]));
+    uint32_t blo = rng[0], bhi = rng[NW];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) { blo = min(blo, rng[w]); bhi = max(bhi, rng[NW + w]); }
     // tiles of the scratch: tile t holds the keys lo0 + 32 t .. + 32
     const uint32_t t_first = blo < bhi ? (blo - lo0) / 32u : 0u, t_end = blo < bhi ? (bhi - lo0 + 31u) / 32u : 0u;
 
@@ -183,26 +185,27 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_fa_kernel(AttnParams p, c
         }
     }
 
-    // ---- tile loads: wave w fetches tokens 8 w .. 8 w + 7 of the K tile and dims 64 w .. 64 w + 63 of the V^T tile
+    // ---- tile loads: the sixteen 1 KB pieces of the K tile (two tokens each) and of the V^T tile (sixteen dims each)
+    // are dealt over the waves
     [[maybe_unused]] const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(kd), 0, (int)((size_t)p.num_kv_heads * ntok * ATTN_HD * 2), 0x00020000);
     [[maybe_unused]] const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t*>(vt), 0, (int)((size_t)p.num_kv_heads * ntok * ATTN_HD * 2), 0x00020000);
-    uint32_t k_off[4], v_off[4];
+    uint32_t k_off[LPW], v_off[LPW];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t tok = 2u * (4u * wave + j) + ((uint32_t)lane >> 5), slot = (uint32_t)lane & 31u;
+    for (int j = 0; j < LPW; ++j) {
+        const uint32_t tok = 2u * ((uint32_t)LPW * wave + j) + ((uint32_t)lane >> 5), slot = (uint32_t)lane & 31u;
         k_off[j] = ((kvh * ntok + tok) * ATTN_HD) * 2u + ((slot ^ (tok & 15u)) * 16u);
-        const uint32_t dim = 16u * (4u * wave + j) + ((uint32_t)lane >> 2), s16 = (uint32_t)lane & 3u;
+        const uint32_t dim = 16u * ((uint32_t)LPW * wave + j) + ((uint32_t)lane >> 2), s16 = (uint32_t)lane & 3u;
         v_off[j] = ((kvh * ATTN_HD + dim) * ntok) * 2u + ((s16 ^ attn_fa_vsigma(dim)) * 16u);
     }
     auto issue_tile = [&](uint32_t t, uint8_t* ks, uint8_t* vs) {
 #if defined(__HIP_DEVICE_COMPILE__)     // the host pass rejects the 16-byte form of the load
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(krsrc, (__attribute__((address_space(3))) void*)(ks + (4 * wave + j) * 1024), 16,
+        for (int j = 0; j < LPW; ++j) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(krsrc, (__attribute__((address_space(3))) void*)(ks + (LPW * wave + j) * 1024), 16,
                                                      k_off[j], t * (32u * ATTN_HD * 2u), 0, 0);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(vrsrc, (__attribute__((address_space(3))) void*)(vs + (4 * wave + j) * 1024), 16,
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(vrsrc, (__attribute__((address_space(3))) void*)(vs + (LPW * wave + j) * 1024), 16,
                                                      v_off[j], t * 64u, 0, 0);
         }
 #endif
@@ -313,7 +316,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_fa_kernel(AttnParams p, c
     __builtin_amdgcn_wave_barrier();
     const float dd[4] = {d4.x, d4.y, d4.z, d4.w};
     __syncthreads();                                                // every wave is through with the tiles
-    uint16_t* orow = reinterpret_cast<uint16_t*>(wave < 2 ? k0s + wave * 8192 : k1s + (wave - 2) * 8192);   // [16 columns][256]
+    uint8_t* const stage = (wave >> 1) == 0 ? k0s : (wave >> 1) == 1 ? k1s : (wave >> 1) == 2 ? v0s : v1s;
+    uint16_t* orow = reinterpret_cast<uint16_t*>(stage + (wave & 1) * 8192);   // [16 columns][256]
 #pragma unroll
     for (int g = 0; g < 4; ++g)
 #pragma unroll

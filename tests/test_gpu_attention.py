@@ -354,8 +354,10 @@ def test_prefill_attention_long_chunks(nv):
         for bits, start, chunk, window, nq, nkv, extra, pad, ring in [
                 (8, 0, 258, 0, 64, 8, 0, False, 0), (4, 37, 261, 0, 64, 8, 5, False, 0), (8, 300, 257, 64, 64, 8, 0, False, 0),
                 (8, 0, 260, 0, 64, 64, 0, False, 0), (16, 5, 256, 0, 64, 16, 0, False, 0), (4, 64, 259, 0, 64, 32, 3, "aligned", 0),
-                (16, 200, 256, 64, 64, 8, 0, False, 320), (8, 0, 300, 0, 64, 4, 0, "aligned", 0), (8, 11, 270, 0, 64, 8, 0, True, 0)]:
-            if act == 1 and bits == 4:
+                (16, 200, 256, 64, 64, 8, 0, False, 320), (8, 0, 300, 0, 64, 4, 0, "aligned", 0), (8, 11, 270, 0, 64, 8, 0, True, 0),
+                # enough queries for blocks of eight waves (sixteen queries per block at this group size)
+                (8, 100, 523, 64, 64, 8, 0, False, 0), (4, 0, 513, 0, 64, 8, 0, False, 0)]:
+            if act == 1 and (bits == 4 or chunk > 512):
                 continue                                            # the fp16 context repeats the 8- and 16-bit cases only
             ctx = nv.Context(0, act)
             say("prefill attention long chunk", act, bits, start, chunk, window, nq, nkv, extra, pad, ring)
