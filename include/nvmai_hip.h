@@ -479,7 +479,13 @@ int nvmai_hip_attention_decode_ragged(nvmai_hip_ctx* ctx, nvmai_stream stream, c
  * elements.  kv_ring_capacity != 0: the row of key p is p % kv_ring_capacity (function constant
  * 76 of the reference).  Errors follow PrefillAttention.validate (PrefillAttention.swift:169-191):
  * strides below num_q_heads * head_dim, query_count == 0, or start_position + query_count >
- * kv_valid_count give NVMAI_ERR_INVALID_ARG.  scale <= 0 selects 1/sqrt(head_dim). */
+ * kv_valid_count give NVMAI_ERR_INVALID_ARG.  scale <= 0 selects 1/sqrt(head_dim).
+ * A chunk with head_dim 256, a power-of-two group size and enough queries to give every compute
+ * unit a block (query_count * num_q_heads >= 16,384), its q and out rows at 16-byte boundaries,
+ * runs in two launches: the key range is dequantized once into fp16 scratch in the context's
+ * workspace (1,024 bytes per key and kv head), then a flash-attention kernel works on that.  Size
+ * the workspace with an eager call or nvmai_hip_ctx_reserve before capturing such a call into a
+ * graph (a captured call that would have to grow it returns NVMAI_ERR_SCRATCH). */
 int nvmai_hip_attention_prefill_causal(nvmai_hip_ctx* ctx, nvmai_stream stream, const void* q,
                                        uint32_t q_token_stride, const nvmai_kv_view* k,
                                        const nvmai_kv_view* v, void* out, uint32_t o_token_stride,
