@@ -27,6 +27,9 @@ struct AttnDequantParams {
     uint16_t* vt;
 };
 
+// fp16 of x, saturating: a row whose scale and bias reach past the fp16 range (values of 1e5 and more) stays finite.
+__device__ __forceinline__ uint16_t attn_f16_sat(float x) { return f32_to_f16(fminf(fmaxf(x, -65504.0f), 65504.0f)); }
+
 __device__ __forceinline__ void attn_dequant32(const uint8_t* row, const KvFormat& f, uint32_t e0, bool live, bool vec, uint16_t* out) {
     if (!live) {
 #pragma unroll
@@ -41,17 +44,17 @@ __device__ __forceinline__ void attn_dequant32(const uint8_t* row, const KvForma
             const uint4 a = *reinterpret_cast<const uint4*>(row + e0), c = *reinterpret_cast<const uint4*>(row + e0 + 16);
             const uint32_t w[8] = {a.x, a.y, a.z, a.w, c.x, c.y, c.z, c.w};
 #pragma unroll
-            for (int e = 0; e < 32; ++e) out[e] = f32_to_f16(fmaf((float)((w[e >> 2] >> (8 * (e & 3))) & 0xFFu), s, b));
+            for (int e = 0; e < 32; ++e) out[e] = attn_f16_sat(fmaf((float)((w[e >> 2] >> (8 * (e & 3))) & 0xFFu), s, b));
         } else {
             const uint4 a = *reinterpret_cast<const uint4*>(row + e0 / 2);
             const uint32_t w[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
-            for (int e = 0; e < 32; ++e) out[e] = f32_to_f16(fmaf((float)((w[e >> 3] >> (4 * (e & 7))) & 0xFu), s, b));
+            for (int e = 0; e < 32; ++e) out[e] = attn_f16_sat(fmaf((float)((w[e >> 3] >> (4 * (e & 7))) & 0xFu), s, b));
         }
         return;
     }
 #pragma unroll
-    for (int e = 0; e < 32; ++e) out[e] = f32_to_f16(kv_load(row, f, e0 + e));
+    for (int e = 0; e < 32; ++e) out[e] = attn_f16_sat(kv_load(row, f, e0 + e));
 }
 
 __global__ __launch_bounds__(256) void attn_prefill_dequant_kernel(AttnDequantParams p) {
@@ -180,7 +183,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_fa_kern
             act2_to_f32<ACT>(raw.z, f[4], f[5]); act2_to_f32<ACT>(raw.w, f[6], f[7]);
             uint32_t w[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) w[e] = (uint32_t)f32_to_f16(f[2 * e] * qs) | ((uint32_t)f32_to_f16(f[2 * e + 1] * qs) << 16);
+            for (int e = 0; e < 4; ++e) w[e] = (uint32_t)attn_f16_sat(f[2 * e] * qs) | ((uint32_t)attn_f16_sat(f[2 * e + 1] * qs) << 16);
             qop[ks] = uint4{w[0], w[1], w[2], w[3]};
         }
     }
