@@ -109,6 +109,7 @@ __global__ __launch_bounds__(256) void attn_prefill_dequant_kernel(AttnDequantPa
 // LDS: a K tile is [token][32 chunks of 16 bytes], chunk c of token t in slot c ^ (t % 16); a V^T tile is
 // [dim][4 pieces of eight tokens], piece c of dim d in slot c ^ sigma(d): both operand reads touch every bank once.
 constexpr uint32_t ATTN_FA_KTILE = 32 * ATTN_HD * 2;      // bytes
+constexpr float ATTN_FA_LAZY = 6.0f;                        // see the softmax of attn_prefill_fa_kernel
 constexpr uint32_t ATTN_FA_MIN_BLOCKS = 256;              // blocks below which the one-launch kernels are taken
 // Slot swizzle of a V^T row (rows of 64 bytes, sixteen lanes reading piece r of sixteen consecutive dims): chosen by
 // measurement -- a wave's 16-byte reads at slot r ^ ((d / 2) % 4) run at the rate of a linear read (1.9 ns per
@@ -231,7 +232,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_fa_kern
     auto compute = [&](uint32_t t, const uint8_t* ks_, const uint8_t* vs_) {
         const uint32_t pos0 = lo0 + 32u * t;
         if (pos0 >= whi || pos0 + 32u <= wlo) return;               // wave-uniform: no key of this wave's columns
-        f4_t sacc[2] = {f4_t{0.0f, 0.0f, 0.0f, 0.0f}, f4_t{0.0f, 0.0f, 0.0f, 0.0f}};
+        // four accumulators (even and odd steps of the head dimension for each half of the tile), so that a
+        // product never waits for the one before it
+        f4_t sacc4[4] = {f4_t{0.0f, 0.0f, 0.0f, 0.0f}, f4_t{0.0f, 0.0f, 0.0f, 0.0f}, f4_t{0.0f, 0.0f, 0.0f, 0.0f}, f4_t{0.0f, 0.0f, 0.0f, 0.0f}};
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             H8 a0, a1, b;
@@ -240,9 +243,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_fa_kern
             a0.u[0] = w0.x; a0.u[1] = w0.y; a0.u[2] = w0.z; a0.u[3] = w0.w;
             a1.u[0] = w1.x; a1.u[1] = w1.y; a1.u[2] = w1.z; a1.u[3] = w1.w;
             b.u[0] = qop[ks].x; b.u[1] = qop[ks].y; b.u[2] = qop[ks].z; b.u[3] = qop[ks].w;
-            sacc[0] = mfma16(a0, b, sacc[0]);
-            sacc[1] = mfma16(a1, b, sacc[1]);
+            sacc4[2 * (ks & 1)] = mfma16(a0, b, sacc4[2 * (ks & 1)]);
+            sacc4[2 * (ks & 1) + 1] = mfma16(a1, b, sacc4[2 * (ks & 1) + 1]);
         }
+        const f4_t sacc[2] = {sacc4[0] + sacc4[2], sacc4[1] + sacc4[3]};
         float sv[8];
 #pragma unroll
         for (int s = 0; s < 8; ++s) sv[s] = sacc[s >> 2][s & 3];
@@ -258,7 +262,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_fa_kern
 #pragma unroll
         for (int s = 1; s < 8; ++s) mx = fmaxf(mx, sv[s]);
         mx = attn_fa_max_quarters(mx);
-        const float m_new = fmaxf(m_run, mx);                       // -inf while the column has seen no key yet
+        // The reference point of the column's exponentials moves only when the maximum has grown by more than
+        // ATTN_FA_LAZY (the probabilities then reach 2^ATTN_FA_LAZY at most, well inside fp16 and exact in the
+        // final quotient): after the first tiles O is hardly ever rescaled.
+        const float m_new = mx > m_run + ATTN_FA_LAZY ? mx : m_run; // -inf while the column has seen no key yet
         const bool none = m_new == -INFINITY;
         const float alpha = none ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
         float pe[8], psum = 0.0f;
