@@ -220,7 +220,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_fa_kern
     for (int g = 0; g < 4; ++g)
 #pragma unroll
         for (int n = 0; n < 4; ++n) oacc[g][n] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    float m_run = -INFINITY, d_run = 0.0f;                          // column i; d over this lane's tokens only
+    float m_run = -1e30f, d_run = 0.0f;                             // column i; d over this lane's tokens only
 
     // operand addresses inside a tile
     uint32_t ka[8];
@@ -265,12 +265,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void attn_prefill_fa_kern
         // The reference point of the column's exponentials moves only when the maximum has grown by more than
         // ATTN_FA_LAZY (the probabilities then reach 2^ATTN_FA_LAZY at most, well inside fp16 and exact in the
         // final quotient): after the first tiles O is hardly ever rescaled.
-        const float m_new = mx > m_run + ATTN_FA_LAZY ? mx : m_run; // -inf while the column has seen no key yet
-        const bool none = m_new == -INFINITY;
-        const float alpha = none ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+        // (m_run starts at a finite -1e30: a column that has seen no key yet needs no case of its own, the
+        // exponentials of its masked scores are 2^-inf = 0 and alpha is 2^0)
+        const float m_new = mx > m_run + ATTN_FA_LAZY ? mx : m_run;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         float pe[8], psum = 0.0f;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) { pe[s] = none ? 0.0f : __builtin_amdgcn_exp2f(sv[s] - m_new); psum += pe[s]; }
+        for (int s = 0; s < 8; ++s) { pe[s] = __builtin_amdgcn_exp2f(sv[s] - m_new); psum += pe[s]; }
         d_run = d_run * alpha + psum;
         m_run = m_new;
         typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
