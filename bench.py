@@ -456,8 +456,9 @@ def run_prefill_attention(nv, ctx, torch, a):
         "config": {"workload": "attention of a configs[2] prefill step: causal, %d query tokens at positions %d..%d, "
                                "16 query / 2 KV heads, head_dim 256, %d-bit KV" % (T, start, kv_valid - 1, bits),
                    "tokens_per_s": round(T / dt), "query_key_pairs": pairs},
-        "roofline": {"kernel": "attn_prefill_dequant_kernel + attn_prefill_fa_kernel (the key range dequantized once into "
-                               "fp16 scratch, then flash attention, %d queries per block)" % (4 * (16 // (HQ // HKV))),
+        "roofline": {"kernel": ("attn_prefill_dequant_kernel + attn_prefill_fa_kernel (the key range dequantized once into "
+                                "fp16 scratch, then flash attention)" if T * HQ >= 16384 else
+                                "attn_partial_mfma_kernel (causal, %d queries per block)" % (16 // (HQ // HKV))),
                      "bound": "mfma", "achieved": round(tf, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
                      "flops_per_launch": flops, "avg_launch_us": round(kern_us, 2)},
