@@ -369,6 +369,42 @@ def test_prefill_attention_long_chunks(nv):
             ctx.close()
 
 
+@pytest.mark.parametrize("bits,start,chunk,window", [(8, 777, 1500, 0), (4, 1000, 4100, 2000), (8, 0, 4096, 0), (4, 2049, 1100, 333)])
+def test_prefill_attention_two_forms_agree(nv, bits, start, chunk, window):
+    # size-independent property at sizes the scalar oracle cannot walk: the same chunk through the two-launch
+    # form (fp16 scratch + flash attention, four- and eight-wave blocks) and through the one-launch kernels that
+    # multiply the codes -- reached by giving q and out rows that do not start at 16-byte boundaries -- agree
+    # to the bar both are held to against the oracle; starts and windows that are no multiples of the 32-key
+    # tile, query counts that leave dead waves and dead columns in the last block
+    say("prefill attention two forms", bits, start, chunk, window)
+    ctx = nv.Context(0, 0)
+    gen = torch.Generator(device="cuda").manual_seed(300 + bits + chunk)
+    nq, nkv, hd = 16, 2, 256
+    kv_valid, row = start + chunk, nq * hd
+    kc, vc, _ = _long_cache(nv, ctx, gen, 1, kv_valid, nkv * hd, bits)
+    q = torch.randn((chunk, row), generator=gen, device="cuda", dtype=torch.float32).to(ctx.dtype)
+    pa = nv.PrefillAttention(ctx)
+    out_a = torch.empty_like(q)
+    pa.encode_causal(q, kc.view(), vc.view(), out_a, start, chunk, hd, nq, nkv, kv_valid, sliding_window=window)
+    assert ctx.workspace_bytes >= 2 * (min(kv_valid, window + chunk) if window else kv_valid) // 32 * 32 * nkv * hd * 2
+    other = nv.Context(0, 0)                                        # a context of its own: its workspace stays empty
+    q_buf = torch.zeros(1 + chunk * row, dtype=ctx.dtype, device="cuda")
+    q_buf[1:].view(chunk, row).copy_(q)
+    out_buf = torch.zeros(1 + chunk * row, dtype=ctx.dtype, device="cuda")
+    nv.PrefillAttention(other).encode_causal(q_buf[1:], kc.view(), vc.view(), out_buf[1:], start, chunk, hd, nq, nkv, kv_valid,
+                                             sliding_window=window)
+    torch.cuda.synchronize()
+    assert other.workspace_bytes < 1 << 20
+    a, b = act_np(out_a), act_np(out_buf[1:].view(chunk, row))
+    assert np.isfinite(a).all()
+    assert O.rel_error(a, b) < 1e-2
+    # row by row as well: no query may be off while the whole chunk looks right
+    worst = max(O.rel_error(a[t], b[t]) for t in range(0, chunk, 37))
+    assert worst < 2e-2, worst
+    ctx.close()
+    other.close()
+
+
 @pytest.mark.parametrize("bits", [8, 4])
 def test_prefill_attention_chunk_equals_decode_steps(nv, bits):
     # size-independent property at a prefill size the scalar oracle cannot walk: query t of a
