@@ -369,7 +369,18 @@ def test_prefill_attention_long_chunks(nv):
             ctx.close()
 
 
-@pytest.mark.parametrize("bits,start,chunk,window", [(8, 777, 1500, 0), (4, 1000, 4100, 2000), (8, 0, 4096, 0), (4, 2049, 1100, 333)])
+def _two_forms_cases():
+    cases = [(8, 777, 1500, 0), (4, 1000, 4100, 2000), (8, 0, 4096, 0), (4, 2049, 1100, 333)]
+    rng = np.random.default_rng(20240521)
+    for _ in range(10):                                             # seeded draws: starts, counts and windows off every grid
+        chunk = int(rng.integers(1024, 2300))
+        start = int(rng.integers(0, 3000))
+        window = int(rng.choice([0, 0, int(rng.integers(1, 64)), int(rng.integers(64, 2500))]))
+        cases.append((int(rng.choice([4, 8])), start, chunk, window))
+    return cases
+
+
+@pytest.mark.parametrize("bits,start,chunk,window", _two_forms_cases())
 def test_prefill_attention_two_forms_agree(nv, bits, start, chunk, window):
     # size-independent property at sizes the scalar oracle cannot walk: the same chunk through the two-launch
     # form (fp16 scratch + flash attention, four- and eight-wave blocks) and through the one-launch kernels that
